@@ -1,0 +1,163 @@
+"""Seeded single-layer cases shared by the fixture generator, the oracle tests and the GPU parity tests.
+
+A case is a dict of plain numpy arrays and ints: the op kind, its hyper-parameters in the reference's
+terms and its inputs. `reference_io(case)` turns it into the topology text and weight blob the
+reference reads, `oracle_eval(case)` evaluates it with the CPU restatement.
+"""
+import numpy as np
+
+from excalibur_amd import modelfile as mf
+from oracle import port
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+def conv_f32_case(seed, n, c, h, w, k, kernel, stride=1, pad=0, act=1, groups=1, bias=True, dw=False):
+    r = _rng(seed)
+    kh, kw = (kernel, kernel) if np.isscalar(kernel) else kernel
+    return dict(op="dw_f32" if dw else "conv_f32", n=n, c=c, h=h, w=w, k=k, kh=kh, kw=kw, stride=stride, pad=pad,
+                act=act, groups=groups,
+                x=r.uniform(-1, 1, (n, c, h, w)).astype(np.float32),
+                wt=r.normal(0, 0.05, (k, c // groups, kh, kw)).astype(np.float32),
+                bias=r.normal(0, 0.01, (k,)).astype(np.float32) if bias else None)
+
+
+def conv_i8_case(seed, n, c, h, w, k, kernel, stride=1, pad=0, act=1, bias=True, integer_x=False, groups=1):
+    r = _rng(seed)
+    kh, kw = (kernel, kernel) if np.isscalar(kernel) else kernel
+    if integer_x:
+        x = r.integers(-127, 128, (n, c, h, w)).astype(np.float32)
+        fs = np.float32(1.0)
+    else:
+        x = r.uniform(-3, 3, (n, c, h, w)).astype(np.float32)
+        fs = np.float32(127.0 / np.abs(x).max() * 1.1)  # a few values saturate
+    wt = r.integers(-127, 128, (k, c // groups, kh, kw)).astype(np.int8)
+    s = r.uniform(1e-4, 1e-2, (k,)).astype(np.float32)       # wanted dequant scale
+    ws = (np.float32(1.0) / (s * fs)).astype(np.float32)     # stored weight scale
+    ws[0] = np.float32(5e-7)                                  # |ws| <= 1e-6 -> scale forced to 0
+    return dict(op="conv_i8", n=n, c=c, h=h, w=w, k=k, kh=kh, kw=kw, stride=stride, pad=pad, act=act, groups=groups,
+                x=x, wt=wt, ws=ws, fs=fs,
+                bias=(r.integers(-2 ** 15, 2 ** 15, (k,)).astype(np.float32) * s).astype(np.float32) if bias else None)
+
+
+def dw_i8_case(seed, n, c, h, w, stride, pad=1, act=1):
+    r = _rng(seed)
+    ws = r.uniform(20, 200, (c,)).astype(np.float32)
+    ws[1] = np.float32(-3.0)  # negative scale -> weights become 0 (no fabs in the reference)
+    return dict(op="dw_i8", n=n, c=c, h=h, w=w, k=c, kh=3, kw=3, stride=stride, pad=pad, act=act, groups=c,
+                x=r.uniform(-1, 1, (n, c, h, w)).astype(np.float32),
+                wt=r.integers(-127, 128, (c, 1, 3, 3)).astype(np.int8), ws=ws, fs=np.float32(1.0),
+                bias=r.normal(0, 0.01, (c,)).astype(np.float32))
+
+
+def pool_case(seed, n, c, h, w, ptype, kernel=0, stride=1, pad=0, global_pool=False, pad_mode=1, count_include_pad=0):
+    r = _rng(seed)
+    return dict(op="pool", n=n, c=c, h=h, w=w, ptype=ptype, kernel=kernel, stride=stride, pad=pad,
+                global_pool=global_pool, pad_mode=pad_mode, count_include_pad=count_include_pad,
+                x=r.uniform(-1, 1, (n, c, h, w)).astype(np.float32))
+
+
+def eltwise_case(seed, shape, etype, n_inputs=2, coeffs=None):
+    r = _rng(seed)
+    return dict(op="eltwise", etype=etype, coeffs=coeffs,
+                xs=[r.uniform(-2, 2, shape).astype(np.float32) for _ in range(n_inputs)])
+
+
+def binaryop_case(seed, shape):
+    r = _rng(seed)
+    return dict(op="binaryop_add", xs=[r.uniform(-2, 2, shape).astype(np.float32) for _ in range(2)])
+
+
+def relu_case(seed, shape):
+    return dict(op="relu", x=_rng(seed).uniform(-2, 2, shape).astype(np.float32))
+
+
+def fc_case(seed, m, c, h, w, n_out, bias=True):
+    r = _rng(seed)
+    return dict(op="fc", n_out=n_out, x=r.uniform(-1, 1, (m, c, h, w)).astype(np.float32),
+                wt=r.normal(0, 0.05, (n_out, c * h * w)).astype(np.float32),
+                bias=r.normal(0, 0.01, (n_out,)).astype(np.float32) if bias else None)
+
+
+def geom_of(case):
+    return port.geom((case["n"], case["c"], case["h"], case["w"]), case["k"], case["kh"], case["kw"],
+                     case["stride"], case["pad"], case["groups"])
+
+
+def reference_io(case):
+    """-> (topology text, weight blob bytes or b'', [input arrays], output blob name)."""
+    op = case["op"]
+    if op in ("conv_f32", "dw_f32", "conv_i8", "dw_i8"):
+        typ = "ConvolutionDepthWise" if op.startswith("dw") else "Convolution"
+        line = mf.conv_line(typ, "layer", "data", "out", case["k"], (case["kh"], case["kw"]), case["stride"],
+                            case["pad"], case["bias"] is not None, case["wt"].size, case["groups"],
+                            int8=op.endswith("i8"), act=case["act"])
+        if op.endswith("i8"):
+            blob = mf.conv_blob_i8(case["wt"], case["bias"], case["ws"], case["fs"])
+        else:
+            blob = mf.conv_blob_f32(case["wt"], case["bias"])
+        return mf.topology([line]), blob, [case["x"]], "out"
+    if op == "pool":
+        line = mf.pool_line("layer", "data", "out", case["ptype"], case["kernel"], case["stride"], case["pad"],
+                            case["global_pool"], case["pad_mode"], case["count_include_pad"])
+        return mf.topology([line]), b"", [case["x"]], "out"
+    if op == "relu":
+        return mf.topology(["ReLU layer 1 1 data out"]), b"", [case["x"]], "out"
+    if op == "fc":
+        line = f"InnerProduct layer 1 1 data out 0={case['n_out']} 1={int(case['bias'] is not None)} 2={case['wt'].size}"
+        return mf.topology([line]), mf.fc_blob_f32(case["wt"], case["bias"]), [case["x"]], "out"
+    raise ValueError(op)
+
+
+def multi_input_topology(case):
+    """Eltwise / BinaryOp take several producers but the reference feeds only one pipeline input
+    (src/Excalibur/pipeline.cpp:242): the operands are channel slices of one input tensor, cut by a
+    Split_Slice layer (src/Excalibur/operation_split_slice.cpp:12-36, axis key 1=0 is the channel axis).
+    -> (topology text, the concatenated input)."""
+    n = len(case["xs"])
+    c = case["xs"][0].shape[1]
+    names = " ".join(f"x{i}" for i in range(n))
+    lines = [f"Split_Slice cut 1 {n} data {names} 0={n}," + ",".join(str(c) for _ in range(n)) + " 1=0"]
+    if case["op"] == "eltwise":
+        extra = f"0={case['etype']}"
+        if case.get("coeffs") is not None:
+            extra += " -23301=" + ",".join([str(n + 1)] + [repr(float(v)) for v in case["coeffs"]])
+        lines.append(f"Eltwise layer {n} 1 {names} out {extra}")
+    else:
+        lines.append(f"BinaryOp layer 2 1 {names} out 0=0")
+    return mf.topology(lines), np.concatenate(case["xs"], axis=1)
+
+
+def oracle_eval(case):
+    op = case["op"]
+    if op == "conv_f32":
+        return port.conv2d_f32(case["x"], case["wt"], case["bias"], case["act"], geom_of(case))
+    if op == "dw_f32":
+        return port.dwconv_f32(case["x"], case["wt"], case["bias"], case["act"], geom_of(case))
+    if op == "dw_i8":
+        wf = port.dw_dequant_weights(case["wt"], case["ws"])
+        return port.dwconv_f32(case["x"], wf, case["bias"], case["act"], geom_of(case))
+    if op == "conv_i8":
+        return port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], case["act"], geom_of(case))
+    if op == "pool":
+        return port.pool2d(case["x"], case["ptype"], case["kernel"], case["stride"], case["pad"], case["global_pool"],
+                           case["pad_mode"], case["count_include_pad"])
+    if op == "eltwise":
+        return port.eltwise(case["xs"], case["etype"], case.get("coeffs"))
+    if op == "binaryop_add":
+        return port.binaryop_add(*case["xs"])
+    if op == "relu":
+        return port.relu(case["x"])
+    if op == "fc":
+        return port.innerproduct(case["x"], case["wt"], case["bias"])
+    raise ValueError(op)
+
+
+def check_value(a, b, t):
+    """The reference's only tolerance rule (src/Julius/julius_test.cpp:12-39):
+    |a - b| <= max(t, t * max(|a|, |b|)). Returns the number of violations."""
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    return int((np.abs(a - b) > np.maximum(t, t * np.maximum(np.abs(a), np.abs(b)))).sum())

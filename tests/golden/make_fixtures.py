@@ -1,0 +1,126 @@
+"""Writes tests/golden/*.npz: inputs and outputs of single layers run through the COMPILED REFERENCE.
+
+Run in a container that has the reference sources: `make -C oracle ref && python -m tests.golden.make_fixtures`.
+Each file holds the case's arrays, its scalar parameters as a JSON string and `expected`, the bytes the
+reference's CPU path produced. Fixtures are data; they let the oracle be checked where the reference is absent.
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from tests import cases  # noqa: E402
+from tests.refrun import run_reference  # noqa: E402
+
+
+def fixture_cases():
+    c = cases
+    return {
+        # f32 convolution: Winograd path (K < 128), im2col path (K >= 128), stride 2, 1x1, 7x7 stem shape, groups
+        "conv_f32_3x3s1_wino": c.conv_f32_case(1, 1, 16, 12, 12, 24, 3, 1, 1),
+        "conv_f32_3x3s1_im2col_k136": c.conv_f32_case(2, 2, 8, 12, 12, 136, 3, 1, 1),
+        "conv_f32_3x3s2": c.conv_f32_case(3, 2, 16, 13, 13, 24, 3, 2, 1),
+        "conv_f32_7x7s2_c3": c.conv_f32_case(4, 1, 3, 32, 32, 16, 7, 2, 3),
+        "conv_f32_1x1_noact": c.conv_f32_case(5, 2, 16, 8, 8, 32, 1, 1, 0, act=0),
+        "conv_f32_relu6": c.conv_f32_case(6, 1, 8, 8, 8, 8, 3, 1, 1, act=3),
+        "conv_f32_groups2": c.conv_f32_case(7, 1, 8, 8, 8, 16, 3, 1, 1, groups=2),
+        # int8 convolution: Winograd (K < 128) and im2col (K >= 128 or not 3x3 s1) paths
+        "conv_i8_3x3s1_wino": c.conv_i8_case(10, 2, 16, 12, 12, 24, 3, 1, 1),
+        "conv_i8_3x3s1_im2col_k136": c.conv_i8_case(11, 2, 8, 12, 12, 136, 3, 1, 1),
+        "conv_i8_3x3s2": c.conv_i8_case(12, 2, 16, 16, 16, 24, 3, 2, 1),
+        "conv_i8_1x1_noact": c.conv_i8_case(13, 1, 32, 8, 8, 64, 1, 1, 0, act=0),
+        "conv_i8_integer_x_nobias": c.conv_i8_case(14, 1, 16, 8, 8, 16, 3, 1, 1, bias=False, integer_x=True),
+        "conv_i8_7x7s2_c3": c.conv_i8_case(15, 1, 3, 32, 32, 16, 7, 2, 3),
+        # depthwise
+        "dw_f32_3x3s1": c.conv_f32_case(20, 2, 8, 10, 10, 8, 3, 1, 1, groups=8, dw=True),
+        "dw_f32_3x3s2": c.conv_f32_case(21, 2, 8, 11, 11, 8, 3, 2, 1, groups=8, dw=True),
+        "dw_i8_3x3s1": c.dw_i8_case(22, 1, 8, 10, 10, 1),
+        "dw_i8_3x3s2": c.dw_i8_case(23, 1, 8, 11, 11, 2),
+        # pooling
+        "pool_max_3x3s2p1": c.pool_case(30, 2, 5, 20, 20, 0, 3, 2, 1),
+        "pool_max_5x5s1p2": c.pool_case(31, 2, 5, 20, 20, 0, 5, 1, 2),
+        "pool_avg_2x2s2": c.pool_case(32, 2, 5, 20, 20, 1, 2, 2, 0),
+        "pool_avg_3x3s2p1_ceil": c.pool_case(33, 2, 5, 19, 19, 1, 3, 2, 1, pad_mode=0),
+        "pool_avg_include_pad": c.pool_case(34, 2, 5, 19, 19, 1, 3, 2, 1, count_include_pad=1),
+        "pool_avg_global": c.pool_case(35, 2, 5, 7, 7, 1, global_pool=True),
+        "pool_max_ceil": c.pool_case(36, 1, 3, 14, 14, 0, 3, 2, 0, pad_mode=0),
+        # elementwise
+        "eltwise_sum": c.eltwise_case(40, (2, 4, 6, 6), 1),
+        "eltwise_sum3_coeffs": c.eltwise_case(41, (2, 4, 6, 7), 1, 3, [0.5, -1.25, 2.0]),
+        "eltwise_max3": c.eltwise_case(42, (2, 4, 6, 6), 2, 3),
+        "eltwise_prod3": c.eltwise_case(43, (2, 4, 6, 6), 0, 3),
+        "binaryop_add": c.binaryop_case(44, (2, 4, 6, 6)),
+        "relu": c.relu_case(45, (2, 4, 6, 7)),
+        # inner product
+        "fc_bias": c.fc_case(46, 3, 8, 4, 4, 10),
+        "fc_nobias": c.fc_case(47, 2, 16, 1, 1, 7, bias=False),
+    }
+
+
+def f16_cases():
+    c = cases
+    return {
+        "f16_conv_3x3s1": c.conv_f32_case(50, 2, 16, 10, 10, 24, 3, 1, 1),
+        "f16_conv_tail75": c.conv_f32_case(51, 1, 4, 5, 5, 3, 3, 1, 1),
+        "f16_dw_3x3s2": c.conv_f32_case(52, 1, 8, 11, 11, 8, 3, 2, 1, groups=8, dw=True),
+        "f16_pool_max": c.pool_case(53, 1, 5, 12, 12, 0, 3, 2, 1),
+    }
+
+
+def save_case(path, case, expected):
+    arrays, meta = {}, {}
+    for k, v in case.items():
+        if v is None:
+            meta[k] = None
+        elif isinstance(v, np.ndarray):
+            arrays[k] = v
+        elif isinstance(v, list) and v and isinstance(v[0], np.ndarray):
+            meta[k + "__list"] = len(v)
+            for i, a in enumerate(v):
+                arrays[f"{k}__{i}"] = a
+        elif isinstance(v, (np.floating, np.integer)):
+            arrays[k] = np.asarray(v)
+        else:
+            meta[k] = v
+    arrays["expected"] = expected
+    arrays["meta_json"] = np.frombuffer(json.dumps(meta).encode(), np.uint8)
+    np.savez_compressed(path, **arrays)
+
+
+def load_case(path):
+    z = np.load(path, allow_pickle=False)
+    meta = json.loads(bytes(z["meta_json"]).decode())
+    case = {}
+    for k, v in meta.items():
+        if k.endswith("__list"):
+            name = k[:-6]
+            case[name] = [z[f"{name}__{i}"] for i in range(v)]
+        else:
+            case[k] = v
+    for k in z.files:
+        if k in ("expected", "meta_json") or "__" in k:
+            continue
+        a = z[k]
+        case[k] = a if a.ndim else a[()]
+    return case, z["expected"]
+
+
+def main():
+    for name, case in fixture_cases().items():
+        save_case(os.path.join(HERE, name + ".npz"), case, run_reference(case))
+    for name, case in f16_cases().items():
+        case = dict(case)
+        case["x"] = case["x"].astype(np.float16).view(np.uint16)
+        save_case(os.path.join(HERE, name + ".npz"), case, run_reference(case, dtype="f16"))
+    total = sum(os.path.getsize(os.path.join(HERE, f)) for f in os.listdir(HERE) if f.endswith(".npz"))
+    print(f"wrote {len(fixture_cases()) + len(f16_cases())} fixtures, {total / 1024:.0f} KiB")
+
+
+if __name__ == "__main__":
+    main()
