@@ -1,0 +1,739 @@
+// Bandwidth-bound operators of the CNN forward path: layout / precision conversion, depthwise 3x3,
+// pooling, elementwise, inner product, and a definition-order convolution for shapes the MFMA path
+// does not take. All are one pass over their operands; arithmetic follows the reference's CPU order
+// where that order is observable in the result (depthwise columns, average-pool row-major sums,
+// saxpby rounding), so these kernels are bit-exact against it in fp32.
+#include <float.h>
+
+#include "common.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kBlock = 256;
+inline unsigned blocks_for(size_t n, int per_block = kBlock) { return (unsigned)((n + per_block - 1) / per_block); }
+
+// ---------------------------------------------------------------------------------------------
+// NCHW -> NHWC with optional quantization. One workgroup moves 64 pixels x 64 channels through LDS:
+// reads are coalesced along pixels of a channel plane, writes are 16-byte runs of channels.
+// MODE 0: f32 -> i8 (quantize), 1: f32 -> f32, 2: f32 -> f16, 3: f16 -> f16
+// ---------------------------------------------------------------------------------------------
+template <int MODE> struct Conv;
+template <> struct Conv<0> { typedef float in_t; typedef int8_t out_t; };
+template <> struct Conv<1> { typedef float in_t; typedef float out_t; };
+template <> struct Conv<2> { typedef float in_t; typedef uint16_t out_t; };
+template <> struct Conv<3> { typedef uint16_t in_t; typedef uint16_t out_t; };
+
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void nchw_to_nhwc_kernel(const typename Conv<MODE>::in_t* __restrict__ x,
+                                                              typename Conv<MODE>::out_t* __restrict__ y, int C, int HW,
+                                                              int c_stride, float fs, const float* __restrict__ fs_pc) {
+    typedef typename Conv<MODE>::out_t out_t;
+    constexpr int ES = sizeof(out_t);
+    constexpr int ROW = 64 * ES + 4;  // bytes per pixel row in LDS; ROW/4 is odd: conflict-free column writes
+    __shared__ __attribute__((aligned(16))) char tile[64 * ROW];
+    const int n = blockIdx.y, p0 = blockIdx.x * 64, tid = threadIdx.x;
+    const int px = tid & 63, csub = tid >> 6;
+    for (int c0 = 0; c0 < c_stride; c0 += 64) {
+#pragma unroll 4
+        for (int i = 0; i < 16; ++i) {
+            const int cl = i * 4 + csub, c = c0 + cl, p = p0 + px;
+            out_t v = 0;
+            if (c < C && p < HW) {
+                const auto in = x[((size_t)n * C + c) * HW + p];
+                if constexpr (MODE == 0) v = (out_t)exhip_q8(in * (fs_pc ? fs_pc[c] : fs));
+                else if constexpr (MODE == 2) v = exhip_f2h(in);
+                else v = in;
+            }
+            *reinterpret_cast<out_t*>(tile + px * ROW + cl * ES) = v;
+        }
+        __syncthreads();
+        // 64 pixels x (64*ES/16) vectors of 16 bytes
+        constexpr int VPP = 64 * ES / 16;
+        for (int v = tid; v < 64 * VPP; v += kBlock) {
+            const int pp = v / VPP, part = v % VPP;
+            const int cbase = c0 + part * (16 / ES);
+            if (p0 + pp < HW && cbase < c_stride) {
+                const int* src = reinterpret_cast<const int*>(tile + pp * ROW + part * 16);
+                out_t* dst = y + ((size_t)n * HW + p0 + pp) * c_stride + cbase;
+                if (cbase + 16 / ES <= c_stride && (c_stride * ES) % 16 == 0) {
+                    v4i o = {src[0], src[1], src[2], src[3]};
+                    *reinterpret_cast<v4i*>(dst) = o;
+                } else {
+                    const out_t* s = reinterpret_cast<const out_t*>(src);
+                    for (int e = 0; e < 16 / ES && cbase + e < c_stride; ++e) dst[e] = s[e];
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// First-layer form: C <= 4 channels packed into one 4-byte int8 pixel (one thread per pixel).
+__global__ __launch_bounds__(kBlock) void quantize_nchw_to_nhwc4_kernel(const float* __restrict__ x, int* __restrict__ y,
+                                                                        int C, int HW, float fs,
+                                                                        const float* __restrict__ fs_pc) {
+    const int n = blockIdx.y;
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= HW) return;
+    uint32_t w = 0;
+    for (int c = 0; c < C; ++c) {
+        const float v = x[((size_t)n * C + c) * HW + p] * (fs_pc ? fs_pc[c] : fs);
+        w |= (uint32_t)(exhip_q8(v) & 0xff) << (8 * c);
+    }
+    y[(size_t)n * HW + p] = (int)w;
+}
+
+// NHWC -> NCHW (graph outputs; small). MODE 0: f32->f32, 1: f16->f32, 2: f16->f16
+template <int MODE, typename Tin, typename Tout>
+__global__ __launch_bounds__(kBlock) void nhwc_to_nchw_kernel(const Tin* __restrict__ x, Tout* __restrict__ y, int C, int HW,
+                                                              int c_stride, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int p = (int)(i % HW);
+    const size_t nc = i / HW;
+    const int c = (int)(nc % C);
+    const size_t n = nc / C;
+    const Tin v = x[(n * HW + p) * c_stride + c];
+    if constexpr (MODE == 1) y[i] = exhip_h2f(v);
+    else y[i] = v;
+}
+
+__global__ __launch_bounds__(kBlock) void f32_to_f16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) y[i] = exhip_f2h(x[i]);
+}
+__global__ __launch_bounds__(kBlock) void f16_to_f32_kernel(const uint16_t* __restrict__ x, float* __restrict__ y, size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) y[i] = exhip_h2f(x[i]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Depthwise 3x3. Column order of the reference: col_j = fma(r2j,k2j, fma(r1j,k1j, fma(r0j,k0j,0)));
+// out = ((bias + col0) + col1) + col2; then the fused activation.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float dw_pixel(const float r[3][3], const float* k, float bias) {
+    float col[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < 3; ++i) s = __builtin_fmaf(r[i][j], k[i * 3 + j], s);
+        col[j] = s;
+    }
+    float sum = bias;
+    sum += col[0];
+    sum += col[1];
+    sum += col[2];
+    return sum;
+}
+
+__global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                    const float* __restrict__ bias, float* __restrict__ y,
+                                                                    int C, int H, int W, int OH, int OW, int stride, int pt,
+                                                                    int pl, int act, size_t total) {
+    const size_t gi = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (gi >= total) return;
+    const size_t nc = gi / ((size_t)OH * OW);
+    const int c = (int)(nc % C);
+    const int o = (int)(gi - nc * ((size_t)OH * OW));
+    const int oy = o / OW, ox = o - oy * OW;
+    const float* in = x + (size_t)nc * H * W;
+    float k[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) k[i] = w[c * 9 + i];
+    float r[3][3];
+#pragma unroll
+    for (int i = 0; i < 3; ++i)
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            const int iy = oy * stride - pt + i, ix = ox * stride - pl + j;
+            r[i][j] = (iy >= 0 && iy < H && ix >= 0 && ix < W) ? in[(size_t)iy * W + ix] : 0.f;
+        }
+    y[(size_t)nc * OH * OW + o] = exhip_act(dw_pixel(r, k, bias ? bias[c] : 0.f), act);
+}
+
+// NHWC half storage, 8 channels (16 bytes) per thread, f32 math in the same order.
+__global__ __launch_bounds__(kBlock) void dwconv3x3_nhwc_f16_kernel(const uint16_t* __restrict__ x, const float* __restrict__ w,
+                                                                    const float* __restrict__ bias, uint16_t* __restrict__ y,
+                                                                    int C, int H, int W, int cs, int OH, int OW, int stride,
+                                                                    int pt, int pl, int act, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 8;
+    const int g = (int)(i % groups);
+    size_t pix = i / groups;
+    const int ox = (int)(pix % OW);
+    pix /= OW;
+    const int oy = (int)(pix % OH);
+    const size_t n = pix / OH;
+    float r[8][3][3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+#pragma unroll
+        for (int b = 0; b < 3; ++b) {
+            const int iy = oy * stride - pt + a, ix = ox * stride - pl + b;
+            v4i v = {0, 0, 0, 0};
+            if (iy >= 0 && iy < H && ix >= 0 && ix < W)
+                v = *reinterpret_cast<const v4i*>(x + ((n * H + iy) * W + ix) * cs + g * 8);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                r[2 * e][a][b] = exhip_h2f((uint16_t)(v[e] & 0xffff));
+                r[2 * e + 1][a][b] = exhip_h2f((uint16_t)((uint32_t)v[e] >> 16));
+            }
+        }
+    v4i o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int c = g * 8 + e;
+        float res = 0.f;
+        if (c < C) {
+            float k[9];
+#pragma unroll
+            for (int q = 0; q < 9; ++q) k[q] = w[c * 9 + q];
+            res = exhip_act(dw_pixel(r[e], k, bias ? bias[c] : 0.f), act);
+        }
+        const uint32_t h = exhip_f2h(res);
+        if (e & 1) o[e >> 1] |= (int)(h << 16);
+        else o[e >> 1] = (int)h;
+    }
+    *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 8) = o;
+}
+
+__global__ __launch_bounds__(kBlock) void dw_dequant_kernel(const int8_t* __restrict__ w, const float* __restrict__ ws,
+                                                            float* __restrict__ wf, int k, int per_group) {
+    const int i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= k * per_group) return;
+    const float s = ws[i / per_group] <= 1e-6f ? 0.f : 1.f / ws[i / per_group];
+    wf[i] = (float)w[i] * s;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Pooling
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void pool2d_nchw_f32_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W,
+                                                                 int OH, int OW, int type, int kh, int kw, int sh, int sw,
+                                                                 int pt, int pb, int pl, int pr, int include_pad,
+                                                                 size_t total) {
+    // flat index over (plane, output pixel): global pooling then runs one plane per thread
+    const size_t gi = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (gi >= total) return;
+    const size_t nc = gi / ((size_t)OH * OW);
+    const int o = (int)(gi - nc * ((size_t)OH * OW));
+    const int ph = o / OW, pw = o - ph * OW;
+    const float* in = x + (size_t)nc * H * W;
+    int hs = ph * sh - pt, wsx = pw * sw - pl;
+    float out;
+    if (type == 0) {
+        const int he = min(hs + kh, H), we = min(wsx + kw, W);
+        hs = max(hs, 0);
+        wsx = max(wsx, 0);
+        float v = -FLT_MAX;
+        for (int a = hs; a < he; ++a)
+            for (int b = wsx; b < we; ++b) {
+                const float t = in[(size_t)a * W + b];
+                v = v < t ? t : v;
+            }
+        out = v;
+    } else {
+        int he = min(hs + kh, H + pb), we = min(wsx + kw, W + pr);
+        int pool = (he - hs) * (we - wsx);
+        hs = max(hs, 0);
+        wsx = max(wsx, 0);
+        he = min(he, H);
+        we = min(we, W);
+        float s = 0.f;
+        for (int a = hs; a < he; ++a)
+            for (int b = wsx; b < we; ++b) s += in[(size_t)a * W + b];
+        if (!include_pad) pool = (he - hs) * (we - wsx);
+        out = s / (float)pool;
+    }
+    y[(size_t)nc * OH * OW + o] = out;
+}
+
+__global__ __launch_bounds__(kBlock) void maxpool_nhwc_f32_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                                  int8_t* __restrict__ yq, float fs_out, int H, int W, int cs,
+                                                                  int OH, int OW, int kh, int kw, int sh, int sw, int pt,
+                                                                  int pl, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 4;
+    const int g = (int)(i % groups);
+    size_t pix = i / groups;
+    const int ox = (int)(pix % OW);
+    pix /= OW;
+    const int oy = (int)(pix % OH);
+    const size_t n = pix / OH;
+    const int hs = max(oy * sh - pt, 0), wsx = max(ox * sw - pl, 0);
+    const int he = min(oy * sh - pt + kh, H), we = min(ox * sw - pl + kw, W);
+    v4f m = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+    for (int a = hs; a < he; ++a)
+        for (int b = wsx; b < we; ++b) {
+            const v4f t = *reinterpret_cast<const v4f*>(x + ((n * H + a) * W + b) * cs + g * 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) m[e] = m[e] < t[e] ? t[e] : m[e];
+        }
+    const size_t o = ((n * OH + oy) * OW + ox) * cs + g * 4;
+    if (y) *reinterpret_cast<v4f*>(y + o) = m;
+    if (yq) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(m[e] * fs_out) & 0xff) << (8 * e);
+        *reinterpret_cast<int*>(yq + o) = (int)w;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void pool2d_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int H,
+                                                                 int W, int cs, int OH, int OW, int type, int kh, int kw,
+                                                                 int sh, int sw, int pt, int pb, int pl, int pr,
+                                                                 int include_pad, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 8;
+    const int g = (int)(i % groups);
+    size_t pix = i / groups;
+    const int ox = (int)(pix % OW);
+    pix /= OW;
+    const int oy = (int)(pix % OH);
+    const size_t n = pix / OH;
+    int hs = oy * sh - pt, wsx = ox * sw - pl;
+    int he = min(hs + kh, type == 0 ? H : H + pb), we = min(wsx + kw, type == 0 ? W : W + pr);
+    int pool = (he - hs) * (we - wsx);
+    hs = max(hs, 0);
+    wsx = max(wsx, 0);
+    he = min(he, H);
+    we = min(we, W);
+    if (!include_pad) pool = (he - hs) * (we - wsx);
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = type == 0 ? -FLT_MAX : 0.f;
+    for (int a = hs; a < he; ++a)
+        for (int b = wsx; b < we; ++b) {
+            const v4i v = *reinterpret_cast<const v4i*>(x + ((n * H + a) * W + b) * cs + g * 8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float t = exhip_h2f((uint16_t)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffff));
+                if (type == 0) acc[e] = acc[e] < t ? t : acc[e];
+                else acc[e] += t;
+            }
+        }
+    v4i o = {0, 0, 0, 0};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float r = type == 0 ? acc[e] : acc[e] / (float)pool;
+        o[e >> 1] |= (int)((uint32_t)exhip_f2h(r) << ((e & 1) * 16));
+    }
+    *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 8) = o;
+}
+
+// ---------------------------------------------------------------------------------------------
+// Elementwise
+// ---------------------------------------------------------------------------------------------
+struct EltArgs {
+    const float* in[8];
+    float coeff[8];
+    int n;
+};
+
+__global__ __launch_bounds__(kBlock) void eltwise_f32_kernel(EltArgs a, int type, float* __restrict__ y, size_t count, size_t body) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= count) return;
+    float r;
+    if (type == 1) {  // SUM through saxpby: body unfused, tail fused
+        r = 0.f;
+        for (int k = 0; k < a.n; ++k) {
+            const float xv = a.in[k][i];
+            if (i < body) r = xv * a.coeff[k] + r * 1.0f;
+            else r = __builtin_fmaf(a.coeff[k], xv, r * 1.0f);
+        }
+    } else if (type == 2) {
+        r = a.in[0][i] < a.in[1][i] ? a.in[1][i] : a.in[0][i];
+        for (int k = 2; k < a.n; ++k) r = r < a.in[k][i] ? a.in[k][i] : r;
+    } else {
+        r = a.in[0][i] * a.in[1][i];
+        for (int k = 2; k < a.n; ++k) r = r * a.in[k][i];
+    }
+    y[i] = r;
+}
+
+// a + b (+ ReLU), four floats per thread where the arrays allow it
+__global__ __launch_bounds__(kBlock) void add_f32_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                         float* __restrict__ y, size_t n4, size_t count, int relu) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n4) {
+        const v4f va = reinterpret_cast<const v4f*>(a)[i];
+        v4f r = va;
+        if (b) {
+            const v4f vb = reinterpret_cast<const v4f*>(b)[i];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = va[e] + vb[e];
+        }
+        if (relu) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[e] = (0.f > r[e]) ? 0.f : r[e];
+        }
+        reinterpret_cast<v4f*>(y)[i] = r;
+    } else {
+        const size_t j = n4 * 4 + (i - n4);
+        if (j < count) {
+            float r = b ? a[j] + b[j] : a[j];
+            if (relu) r = (0.f > r) ? 0.f : r;
+            y[j] = r;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void add_f16_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
+                                                         uint16_t* __restrict__ y, size_t count, int relu) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= count) return;
+    float r = exhip_h2f(a[i]);
+    if (b) r += exhip_h2f(b[i]);
+    if (relu) r = (0.f > r) ? 0.f : r;
+    y[i] = exhip_f2h(r);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Inner product: one wave per output neuron, up to 8 batch rows at a time, float4 loads along k.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void innerproduct_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                  const float* __restrict__ bias, float* __restrict__ y, int m,
+                                                                  int n_out, int k_in) {
+    const int lane = threadIdx.x & 63;
+    const int j = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+    if (j >= n_out) return;
+    const float* wr = w + (size_t)j * k_in;
+    const bool vec = (k_in % 4 == 0);
+    for (int m0 = 0; m0 < m; m0 += 8) {
+        float acc[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) acc[r] = 0.f;
+        if (vec) {
+            for (int k = lane * 4; k < k_in; k += 256) {
+                const v4f wv = *reinterpret_cast<const v4f*>(wr + k);
+#pragma unroll
+                for (int r = 0; r < 8; ++r)
+                    if (m0 + r < m) {
+                        const v4f xv = *reinterpret_cast<const v4f*>(x + (size_t)(m0 + r) * k_in + k);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) acc[r] = __builtin_fmaf(xv[e], wv[e], acc[r]);
+                    }
+            }
+        } else {
+            for (int k = lane; k < k_in; k += 64) {
+                const float wv = wr[k];
+#pragma unroll
+                for (int r = 0; r < 8; ++r)
+                    if (m0 + r < m) acc[r] = __builtin_fmaf(x[(size_t)(m0 + r) * k_in + k], wv, acc[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+            float v = acc[r];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+            if (lane == 0 && m0 + r < m) y[(size_t)(m0 + r) * n_out + j] = v + (bias ? bias[j] : 0.f);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Convolution straight from the definition on NCHW f32 (any geometry, groups). One thread per output.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void conv_direct_kernel(const float* __restrict__ x, const float* __restrict__ wf,
+                                                             const int8_t* __restrict__ wq, float fs,
+                                                             const float* __restrict__ scale, const float* __restrict__ bias,
+                                                             float* __restrict__ y, int C, int H, int W, int K, int OH, int OW,
+                                                             int kh, int kw, int sh, int sw, int pt, int pl, int groups,
+                                                             int act, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int ox = (int)(i % OW);
+    size_t t = i / OW;
+    const int oy = (int)(t % OH);
+    t /= OH;
+    const int k = (int)(t % K);
+    const size_t n = t / K;
+    const int cg = C / groups, g = k / (K / groups);
+    float accf = 0.f;
+    int acci = 0;
+    for (int c = 0; c < cg; ++c) {
+        const float* in = x + (n * C + g * cg + c) * H * W;
+        for (int a = 0; a < kh; ++a) {
+            const int iy = oy * sh - pt + a;
+            if (iy < 0 || iy >= H) continue;
+            for (int b = 0; b < kw; ++b) {
+                const int ix = ox * sw - pl + b;
+                if (ix < 0 || ix >= W) continue;
+                const size_t wi = (((size_t)k * cg + c) * kh + a) * kw + b;
+                const float xv = in[(size_t)iy * W + ix];
+                if (wq) acci += exhip_q8(xv * fs) * (int)wq[wi];
+                else accf = __builtin_fmaf(xv, wf[wi], accf);
+            }
+        }
+    }
+    float v;
+    if (wq) v = __builtin_fmaf((float)acci, scale[k], bias ? bias[k] : 0.f);
+    else v = accf + (bias ? bias[k] : 0.f);
+    y[i] = exhip_act(v, act);
+}
+
+}  // namespace
+
+// ================================ C ABI ================================
+
+#define REQ_CTX(name) EXHIP_REQUIRE(ctx, name ": NULL ctx")
+
+template <int MODE>
+static int launch_to_nhwc(exhip_ctx* ctx, const void* x, void* y, int n, int c, int h, int w, int c_stride, float fs,
+                          const float* fs_pc) {
+    EXHIP_REQUIRE(x && y, "layout conversion: NULL tensor");
+    EXHIP_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && c_stride >= c, "layout conversion: bad shape");
+    dim3 grid((h * w + 63) / 64, n);
+    hipLaunchKernelGGL(nchw_to_nhwc_kernel<MODE>, grid, dim3(kBlock), 0, ctx->stream,
+                       (const typename Conv<MODE>::in_t*)x, (typename Conv<MODE>::out_t*)y, c, h * w, c_stride, fs, fs_pc);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_quantize_nchw_f32_to_nhwc_i8(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, float fs,
+                                                  const float* fs_pc, int c_stride, int8_t* y) {
+    REQ_CTX("exhip_quantize_nchw_f32_to_nhwc_i8");
+    if (c_stride == 4 && c <= 4) {
+        EXHIP_REQUIRE(x && y && n > 0 && h > 0 && w > 0, "quantize: bad argument");
+        dim3 grid(blocks_for((size_t)h * w), n);
+        hipLaunchKernelGGL(quantize_nchw_to_nhwc4_kernel, grid, dim3(kBlock), 0, ctx->stream, x, (int*)y, c, h * w, fs, fs_pc);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
+    return launch_to_nhwc<0>(ctx, x, y, n, c, h, w, c_stride, fs, fs_pc);
+}
+extern "C" int exhip_nchw_f32_to_nhwc_f32(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, int cs, float* y) {
+    REQ_CTX("exhip_nchw_f32_to_nhwc_f32");
+    return launch_to_nhwc<1>(ctx, x, y, n, c, h, w, cs, 0.f, nullptr);
+}
+extern "C" int exhip_nchw_f32_to_nhwc_f16(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, int cs, uint16_t* y) {
+    REQ_CTX("exhip_nchw_f32_to_nhwc_f16");
+    return launch_to_nhwc<2>(ctx, x, y, n, c, h, w, cs, 0.f, nullptr);
+}
+extern "C" int exhip_nchw_f16_to_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, int n, int c, int h, int w, int cs, uint16_t* y) {
+    REQ_CTX("exhip_nchw_f16_to_nhwc_f16");
+    return launch_to_nhwc<3>(ctx, x, y, n, c, h, w, cs, 0.f, nullptr);
+}
+
+template <int MODE, typename Tin, typename Tout>
+static int launch_to_nchw(exhip_ctx* ctx, const Tin* x, Tout* y, int n, int c, int h, int w, int cs) {
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 0 && w > 0 && cs >= c, "layout conversion: bad argument");
+    const size_t total = (size_t)n * c * h * w;
+    hipLaunchKernelGGL((nhwc_to_nchw_kernel<MODE, Tin, Tout>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c,
+                       h * w, cs, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+extern "C" int exhip_nhwc_f32_to_nchw_f32(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, int cs, float* y) {
+    REQ_CTX("exhip_nhwc_f32_to_nchw_f32");
+    return launch_to_nchw<0>(ctx, x, y, n, c, h, w, cs);
+}
+extern "C" int exhip_nhwc_f16_to_nchw_f32(exhip_ctx* ctx, const uint16_t* x, int n, int c, int h, int w, int cs, float* y) {
+    REQ_CTX("exhip_nhwc_f16_to_nchw_f32");
+    return launch_to_nchw<1>(ctx, x, y, n, c, h, w, cs);
+}
+extern "C" int exhip_nhwc_f16_to_nchw_f16(exhip_ctx* ctx, const uint16_t* x, int n, int c, int h, int w, int cs, uint16_t* y) {
+    REQ_CTX("exhip_nhwc_f16_to_nchw_f16");
+    return launch_to_nchw<2>(ctx, x, y, n, c, h, w, cs);
+}
+
+extern "C" int exhip_f32_to_f16(exhip_ctx* ctx, const float* x, uint16_t* y, size_t count) {
+    REQ_CTX("exhip_f32_to_f16");
+    EXHIP_REQUIRE((x && y) || !count, "exhip_f32_to_f16: NULL tensor");
+    if (!count) return 0;
+    hipLaunchKernelGGL(f32_to_f16_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, x, y, count);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+extern "C" int exhip_f16_to_f32(exhip_ctx* ctx, const uint16_t* x, float* y, size_t count) {
+    REQ_CTX("exhip_f16_to_f32");
+    EXHIP_REQUIRE((x && y) || !count, "exhip_f16_to_f32: NULL tensor");
+    if (!count) return 0;
+    hipLaunchKernelGGL(f16_to_f32_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, x, y, count);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+static int dw_out(int h, int w, int stride, int pt, int pb, int pl, int pr, int* oh, int* ow) {
+    EXHIP_REQUIRE(stride == 1 || stride == 2, "dwconv3x3: stride %d not supported", stride);
+    EXHIP_REQUIRE(h + pt + pb >= 3 && w + pl + pr >= 3, "dwconv3x3: input smaller than the kernel");
+    *oh = (h + pt + pb - 3) / stride + 1;
+    *ow = (w + pl + pr - 3) / stride + 1;
+    return 0;
+}
+
+extern "C" int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const float* w9, const float* bias, float* y, int n,
+                                        int c, int h, int w, int stride, int pt, int pb, int pl, int pr, int act) {
+    REQ_CTX("exhip_dwconv3x3_nchw_f32");
+    EXHIP_REQUIRE(x && w9 && y && n > 0 && c > 0, "exhip_dwconv3x3_nchw_f32: bad argument");
+    int oh, ow;
+    int rc = dw_out(h, w, stride, pt, pb, pl, pr, &oh, &ow);
+    if (rc) return rc;
+    const size_t total = (size_t)n * c * oh * ow;
+    hipLaunchKernelGGL(dwconv3x3_nchw_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, w9, bias, y, c, h, w,
+                       oh, ow, stride, pt, pl, act, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const float* bias, uint16_t* y,
+                                        int n, int c, int h, int w, int cs, int stride, int pt, int pb, int pl, int pr,
+                                        int act) {
+    REQ_CTX("exhip_dwconv3x3_nhwc_f16");
+    EXHIP_REQUIRE(x && w9 && y && n > 0 && c > 0 && cs >= c && cs % 8 == 0, "exhip_dwconv3x3_nhwc_f16: bad argument (c_stride %% 8)");
+    int oh, ow;
+    int rc = dw_out(h, w, stride, pt, pb, pl, pr, &oh, &ow);
+    if (rc) return rc;
+    const size_t total = (size_t)n * oh * ow * (cs / 8);
+    hipLaunchKernelGGL(dwconv3x3_nhwc_f16_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, w9, bias, y, c, h, w,
+                       cs, oh, ow, stride, pt, pl, act, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_dw_dequant_weights(exhip_ctx* ctx, const int8_t* w, const float* ws, float* wf, int k, int per_group) {
+    REQ_CTX("exhip_dw_dequant_weights");
+    EXHIP_REQUIRE(w && ws && wf && k > 0 && per_group > 0, "exhip_dw_dequant_weights: bad argument");
+    hipLaunchKernelGGL(dw_dequant_kernel, dim3(blocks_for((size_t)k * per_group)), dim3(kBlock), 0, ctx->stream, w, ws, wf, k,
+                       per_group);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_pool_out_hw(int h, int w, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr, int pad_mode,
+                                 int* oh, int* ow) {
+    EXHIP_REQUIRE(oh && ow && sh > 0 && sw > 0, "exhip_pool_out_hw: bad argument");
+    EXHIP_REQUIRE(pad_mode == 0 || pad_mode == 1, "exhip_pool_out_hw: pad_mode %d", pad_mode);
+    // float quotient then ceil / floor, as src/Excalibur/operation_pooling.cpp:103-121
+    const float qh = (float)(h + pt + pb - kh) / sh, qw = (float)(w + pl + pr - kw) / sw;
+    *oh = (int)(pad_mode == 0 ? ceilf(qh) : floorf(qh)) + 1;
+    *ow = (int)(pad_mode == 0 ? ceilf(qw) : floorf(qw)) + 1;
+    return 0;
+}
+
+extern "C" int exhip_pool2d_nchw_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w, int oh, int ow,
+                                     int type, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr,
+                                     int include_pad) {
+    REQ_CTX("exhip_pool2d_nchw_f32");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && oh > 0 && ow > 0 && kh > 0 && kw > 0, "exhip_pool2d_nchw_f32: bad argument");
+    EXHIP_REQUIRE(type == 0 || type == 1, "exhip_pool2d_nchw_f32: unknown pooling type %d", type);
+    const size_t total = (size_t)n * c * oh * ow;
+    hipLaunchKernelGGL(pool2d_nchw_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, oh, ow, type,
+                       kh, kw, sh, sw, pt, pb, pl, pr, include_pad, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_maxpool2d_nhwc_f32(exhip_ctx* ctx, const float* x, float* y, int8_t* y_i8, float fs_out, int n, int c,
+                                        int h, int w, int cs, int oh, int ow, int kh, int kw, int sh, int sw, int pt, int pl) {
+    REQ_CTX("exhip_maxpool2d_nhwc_f32");
+    EXHIP_REQUIRE(x && (y || y_i8) && n > 0 && c > 0 && cs >= c && cs % 4 == 0, "exhip_maxpool2d_nhwc_f32: bad argument");
+    const size_t total = (size_t)n * oh * ow * (cs / 4);
+    hipLaunchKernelGGL(maxpool_nhwc_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, y_i8, fs_out, h, w,
+                       cs, oh, ow, kh, kw, sh, sw, pt, pl, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_pool2d_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int cs,
+                                     int oh, int ow, int type, int kh, int kw, int sh, int sw, int pt, int pb, int pl,
+                                     int pr, int include_pad) {
+    REQ_CTX("exhip_pool2d_nhwc_f16");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && cs >= c && cs % 8 == 0, "exhip_pool2d_nhwc_f16: bad argument");
+    EXHIP_REQUIRE(type == 0 || type == 1, "exhip_pool2d_nhwc_f16: unknown pooling type %d", type);
+    const size_t total = (size_t)n * oh * ow * (cs / 8);
+    hipLaunchKernelGGL(pool2d_nhwc_f16_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, cs, oh, ow,
+                       type, kh, kw, sh, sw, pt, pb, pl, pr, include_pad, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_eltwise_f32(exhip_ctx* ctx, const float* const* inputs, int n_inputs, const float* coeffs, int type,
+                                 float* y, size_t count) {
+    REQ_CTX("exhip_eltwise_f32");
+    EXHIP_REQUIRE(inputs && y, "exhip_eltwise_f32: NULL tensor");
+    EXHIP_REQUIRE(n_inputs >= 2 && n_inputs <= 8, "exhip_eltwise_f32: %d inputs (2..8 supported)", n_inputs);
+    EXHIP_REQUIRE(type >= 0 && type <= 2, "exhip_eltwise_f32: unknown elementwise operation %d", type);
+    if (!count) return 0;
+    EltArgs a;
+    a.n = n_inputs;
+    for (int i = 0; i < n_inputs; ++i) {
+        EXHIP_REQUIRE(inputs[i], "exhip_eltwise_f32: input %d is NULL", i);
+        a.in[i] = inputs[i];
+        a.coeff[i] = coeffs ? coeffs[i] : 1.0f;
+    }
+    hipLaunchKernelGGL(eltwise_f32_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, a, type, y, count,
+                       count - count % 8);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+static int launch_add_f32(exhip_ctx* ctx, const float* a, const float* b, float* y, size_t count, int relu) {
+    if (!count) return 0;
+    const bool aligned = ((uintptr_t)a % 16 == 0) && ((uintptr_t)y % 16 == 0) && (!b || (uintptr_t)b % 16 == 0);
+    const size_t n4 = aligned ? count / 4 : 0;
+    const size_t threads = n4 + (count - n4 * 4);
+    hipLaunchKernelGGL(add_f32_kernel, dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, a, b, y, n4, count, relu);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_add_f32(exhip_ctx* ctx, const float* a, const float* b, float* y, size_t count, int relu) {
+    REQ_CTX("exhip_add_f32");
+    EXHIP_REQUIRE((a && b && y) || !count, "exhip_add_f32: NULL tensor");
+    return launch_add_f32(ctx, a, b, y, count, relu);
+}
+extern "C" int exhip_relu_f32(exhip_ctx* ctx, const float* x, float* y, size_t count) {
+    REQ_CTX("exhip_relu_f32");
+    EXHIP_REQUIRE((x && y) || !count, "exhip_relu_f32: NULL tensor");
+    return launch_add_f32(ctx, x, nullptr, y, count, 1);
+}
+extern "C" int exhip_add_f16(exhip_ctx* ctx, const uint16_t* a, const uint16_t* b, uint16_t* y, size_t count, int relu) {
+    REQ_CTX("exhip_add_f16");
+    EXHIP_REQUIRE((a && b && y) || !count, "exhip_add_f16: NULL tensor");
+    if (!count) return 0;
+    hipLaunchKernelGGL(add_f16_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, a, b, y, count, relu);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+extern "C" int exhip_relu_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, size_t count) {
+    REQ_CTX("exhip_relu_f16");
+    EXHIP_REQUIRE((x && y) || !count, "exhip_relu_f16: NULL tensor");
+    if (!count) return 0;
+    hipLaunchKernelGGL(add_f16_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, x, (const uint16_t*)nullptr, y, count, 1);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_innerproduct_f32(exhip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, int m,
+                                      int n_out, int k_in) {
+    REQ_CTX("exhip_innerproduct_f32");
+    EXHIP_REQUIRE(x && w && y && m > 0 && n_out > 0 && k_in > 0, "exhip_innerproduct_f32: bad argument");
+    hipLaunchKernelGGL(innerproduct_f32_kernel, dim3((n_out + 3) / 4), dim3(kBlock), 0, ctx->stream, x, w, bias, y, m, n_out, k_in);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_conv2d_direct_nchw(exhip_ctx* ctx, const exhip_conv_desc* d, int groups, const float* x, const float* wf,
+                                        const int8_t* wq, float fs, const float* scale, const float* bias, float* y) {
+    REQ_CTX("exhip_conv2d_direct_nchw");
+    EXHIP_REQUIRE(d && x && y && (wf || wq), "exhip_conv2d_direct_nchw: NULL argument");
+    EXHIP_REQUIRE(!wq || scale, "exhip_conv2d_direct_nchw: int8 weights need scales");
+    EXHIP_REQUIRE(groups > 0 && d->c % groups == 0 && d->k % groups == 0, "exhip_conv2d_direct_nchw: channels not divisible by groups");
+    EXHIP_REQUIRE(d->sh > 0 && d->sw > 0 && d->kh > 0 && d->kw > 0, "exhip_conv2d_direct_nchw: bad kernel/stride");
+    const int oh = (d->h + d->pt + d->pb - d->kh) / d->sh + 1, ow = (d->w + d->pl + d->pr - d->kw) / d->sw + 1;
+    EXHIP_REQUIRE(oh > 0 && ow > 0, "exhip_conv2d_direct_nchw: empty output");
+    const size_t total = (size_t)d->n * d->k * oh * ow;
+    hipLaunchKernelGGL(conv_direct_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, wf, wq, fs, scale, bias, y,
+                       d->c, d->h, d->w, d->k, oh, ow, d->kh, d->kw, d->sh, d->sw, d->pt, d->pl, groups, d->act, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}

@@ -1,0 +1,57 @@
+// Shared declarations of the exhip library (HIP for gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/exhip.h"
+
+struct exhip_ctx {
+    int device;
+    hipStream_t stream;
+};
+
+void exhip_set_error(const char* fmt, ...);
+
+#define EXHIP_CHECK(expr)                                                                          \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess) {                                                                    \
+            exhip_set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return (int)e_;                                                                        \
+        }                                                                                          \
+    } while (0)
+
+#define EXHIP_REQUIRE(cond, ...)          \
+    do {                                  \
+        if (!(cond)) {                    \
+            exhip_set_error(__VA_ARGS__); \
+            return EXHIP_ERR_ARG;         \
+        }                                 \
+    } while (0)
+
+// Kernel launch check: launch errors are reported at once, execution errors at the next sync.
+#define EXHIP_LAUNCH_CHECK() EXHIP_CHECK(hipGetLastError())
+
+// ---- device helpers shared by the kernels ----
+// float32_to_int8 of the reference (src/Primitives/simd_types.cpp:140-152): add +-0.5, saturate, truncate.
+__device__ __forceinline__ int exhip_q8(float v) {
+    float t = v >= 0.f ? v + 0.5f : v - 0.5f;
+    t = t > 127.f ? 127.f : t;
+    t = t < -128.f ? -128.f : t;
+    return (int)t;  // v_cvt_i32_f32 truncates toward zero
+}
+
+// suffix_activation_cpu_f32 of the reference (src/Excalibur/operation_general_conv.cpp:127-272).
+__device__ __forceinline__ float exhip_act(float v, int act) {
+    switch (act) {
+    case 1: return (0.f > v) ? 0.f : v;
+    case 3: { float d = (0.f > v) ? 0.f : v; return d <= 6.f ? d : 0.f; }
+    case 4: return (float)(1.0 / (1.0 + exp(-(double)v)));
+    case 5: return (float)((double)v * tanh(log(1.0 + exp((double)v))));
+    default: return v;
+    }
+}
+
+__device__ __forceinline__ float exhip_h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t exhip_f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }

@@ -1,0 +1,678 @@
+// Dense convolution as an implicit GEMM on the gfx950 matrix cores.
+//
+// GEMM view: rows = output channels (the packed weights are the MFMA A operand), columns = output
+// pixels (activations are the B operand), reduction = filter taps x input channels. One workgroup of
+// 4 waves owns TM output channels x TN pixels of one image, where the pixels form a PH x PW patch so
+// that the input halo is staged once in LDS and reused by every tap. The reduction walks "stages":
+// (input-channel chunk, group of filter rows). Per stage the workgroup holds the weight slice for that
+// chunk/rows in LDS, already in MFMA fragment order (the host packs it so), and per channel chunk the
+// halo tile. The next stage's global loads are issued before the current stage's MFMAs and written to
+// LDS afterwards.
+//
+// One k-step is 32 bytes of reduction per pixel: 32 int8 / 16 half / 8 float input channels of one
+// tap ("generic" form), or, for first layers with <= 4 channels, one whole filter row of up to 8 (int8)
+// or 4 (half) neighbouring pixels ("packed-row" form), which keeps the 7x7x3 stem from being padded
+// out to 32 channels.
+//
+// MFMA 32x32 accumulator layout (verified on hardware): lane l, register i holds row
+// 8*(i/4) + 4*(l/32) + i%4, column l%32. The host permutes the weight rows of each 32-channel tile so
+// that a lane's 16 registers are 16 consecutive output channels of one pixel: NHWC stores are then
+// 16-byte (int8) or 64-byte (f32) vectors.
+#include <string.h>
+
+#include <vector>
+
+#include "common.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxActVec = 10;   // 16-byte activation vectors staged per thread and channel chunk
+constexpr int kMaxWVec = 6;      // 16-byte weight vectors staged per thread and stage
+constexpr int kMaxPackedPix = 8; // pixels staged per thread in packed-row form
+
+struct ConvParams {
+    const char* x;
+    const char* wp;
+    const float* scale;
+    const float* bias;
+    const void* residual;
+    void* y_q;       // i8: int8 NHWC ; f16: half NHWC ; f32: unused
+    void* y_nhwc;    // f32 NHWC (i8 and f32 kernels)
+    void* y_nchw;    // f32 NCHW
+    void* y_nchw_h;  // half NCHW (f16 kernel)
+    int32_t* acc_nchw;
+    int N, H, W, K, OH, OW;
+    int KH, KWe, KS;          // filter rows, k-step groups per row (KW, or 1 packed), k-steps per chunk
+    int S;                    // stride seen inside the staged tile
+    int tile_step;            // input pixels between staged tile pixels (2 for 1x1 stride 2)
+    int PT, PL;
+    int cstride_b;            // bytes per input pixel
+    int kstride;              // output channel stride (elements)
+    int PH, PW, IH, IW;       // output patch and staged tile size in pixels
+    int lds_pix_b, lds_row_b; // LDS bytes per tile pixel / row
+    int lds_act_b;            // LDS bytes of the activation tile (weights follow)
+    int n_chunks, chunk_b;
+    int RS, n_rg;             // filter rows per stage, stages per chunk
+    int tiles_x, tiles_y, ktiles;
+    int act, post_relu;
+    float fs_out;
+    int b_align;              // alignment of B fragment reads in packed-row form (4, 8 or 16)
+};
+
+template <int DT> struct Acc { typedef v16i type; };
+template <> struct Acc<EXHIP_F16> { typedef v16f type; };
+template <> struct Acc<EXHIP_F32> { typedef v16f type; };
+
+template <int DT>
+__device__ __forceinline__ void mma(typename Acc<DT>::type& acc, const v4i& a, const v4i& b) {
+    if constexpr (DT == EXHIP_I8) {
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc, 0, 0, 0);
+    } else if constexpr (DT == EXHIP_F16) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), acc, 0, 0, 0);
+    } else {
+        const v4f af = __builtin_bit_cast(v4f, a), bf = __builtin_bit_cast(v4f, b);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[e], bf[e], acc, 0, 0, 0);
+    }
+}
+
+__device__ __forceinline__ v4i lds_read16(const char* p) { return *reinterpret_cast<const v4i*>(p); }
+
+__device__ __forceinline__ v4i lds_read16_unaligned(const char* p, int align) {
+    v4i r;
+    if (align >= 8) {
+        const v2i lo = *reinterpret_cast<const v2i*>(p), hi = *reinterpret_cast<const v2i*>(p + 8);
+        r[0] = lo[0]; r[1] = lo[1]; r[2] = hi[0]; r[3] = hi[1];
+    } else {
+        const int* q = reinterpret_cast<const int*>(p);
+        r[0] = q[0]; r[1] = q[1]; r[2] = q[2]; r[3] = q[3];
+    }
+    return r;
+}
+
+template <int DT, int MT, int NT, int WM, int WN, bool PACKED>
+__global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p) {
+    static_assert(WM * WN == 4, "four waves per workgroup");
+    constexpr int TM = 32 * MT * WM;
+    typedef typename Acc<DT>::type acc_t;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    char* lds_a = smem;
+    char* lds_w = smem + p.lds_act_b;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD one contiguous run of tiles so
+    // that the channel tiles of a patch and its spatial neighbours share that XCD's L2.
+    int bid = blockIdx.x;
+    {
+        const int per = gridDim.x >> 3;
+        if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+    }
+    const int kt = bid % p.ktiles;
+    int t = bid / p.ktiles;
+    const int tx = t % p.tiles_x;
+    t /= p.tiles_x;
+    const int ty = t % p.tiles_y;
+    const int n = t / p.tiles_y;
+    const int oy0 = ty * p.PH, ox0 = tx * p.PW;
+    const int iy0 = oy0 * p.S * p.tile_step - p.PT, ix0 = ox0 * p.S * p.tile_step - p.PL;
+    const char* ximg = p.x + (size_t)n * p.H * p.W * p.cstride_b;
+
+    // ---- staging plan (same for every chunk) ----
+    int a_goff[PACKED ? kMaxPackedPix : kMaxActVec];
+    int a_loff[PACKED ? kMaxPackedPix : kMaxActVec];
+    if constexpr (!PACKED) {
+        const int vp = p.chunk_b >> 4;
+        const int nvec = p.IH * p.IW * vp;
+#pragma unroll
+        for (int i = 0; i < kMaxActVec; ++i) {
+            const int v = tid + kThreads * i;
+            a_goff[i] = -1;
+            a_loff[i] = -1;
+            if (v < nvec) {
+                const int pix = v / vp, part = v - pix * vp;
+                const int iy = pix / p.IW, ix = pix - iy * p.IW;
+                const int gy = iy0 + iy * p.tile_step, gx = ix0 + ix * p.tile_step;
+                a_loff[i] = iy * p.lds_row_b + ix * p.lds_pix_b + part * 16;
+                if (gy >= 0 && gy < p.H && gx >= 0 && gx < p.W) a_goff[i] = (gy * p.W + gx) * p.cstride_b + part * 16;
+            }
+        }
+    } else {
+        const int npix = p.IH * p.IW;
+#pragma unroll
+        for (int i = 0; i < kMaxPackedPix; ++i) {
+            const int v = tid + kThreads * i;
+            a_goff[i] = -1;
+            a_loff[i] = -1;
+            if (v < npix) {
+                const int iy = v / p.IW, ix = v - iy * p.IW;
+                const int gy = iy0 + iy, gx = ix0 + ix;
+                a_loff[i] = iy * p.lds_row_b + ix * p.lds_pix_b;
+                if (gy >= 0 && gy < p.H && gx >= 0 && gx < p.W) a_goff[i] = (gy * p.W + gx) * p.cstride_b;
+            }
+        }
+    }
+
+    // per-lane B fragment offsets inside the tile and the lane's pixels
+    int boff[NT];
+    int pvalid = 0;
+    int ppy[NT], ppx[NT];
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+        int pp = (wn * NT + j) * 32 + (lane & 31);
+        const bool ok = pp < p.PH * p.PW;
+        pp = ok ? pp : 0;
+        const int py = pp / p.PW, px = pp - py * p.PW;
+        ppy[j] = py;
+        ppx[j] = px;
+        if (ok && oy0 + py < p.OH && ox0 + px < p.OW) pvalid |= 1 << j;
+        boff[j] = py * p.S * p.lds_row_b + px * p.S * p.lds_pix_b + (lane >> 5) * 16;
+    }
+    const int aoff = wm * MT * 1024 + lane * 16;
+
+    acc_t acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;  // packed weight bytes of one filter row
+    const int n_stages = p.n_chunks * p.n_rg;
+    const char* wkt = p.wp + (size_t)kt * p.n_chunks * p.KH * row_w_b;
+
+    v4i a_reg[PACKED ? 1 : kMaxActVec];
+    v2i a_reg_p[PACKED ? kMaxPackedPix : 1];
+    v4i w_reg[kMaxWVec];
+
+    auto load_act = [&](int cc) {
+        if constexpr (!PACKED) {
+#pragma unroll
+            for (int i = 0; i < kMaxActVec; ++i) {
+                v4i v = {0, 0, 0, 0};
+                if (a_goff[i] >= 0) v = *reinterpret_cast<const v4i*>(ximg + a_goff[i] + cc * p.chunk_b);
+                a_reg[i] = v;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < kMaxPackedPix; ++i) {
+                v2i v = {0, 0};
+                if (a_goff[i] >= 0) {
+                    if (p.cstride_b == 4) v[0] = *reinterpret_cast<const int*>(ximg + a_goff[i]);
+                    else v = *reinterpret_cast<const v2i*>(ximg + a_goff[i]);
+                }
+                a_reg_p[i] = v;
+            }
+        }
+    };
+    auto store_act = [&]() {
+        if constexpr (!PACKED) {
+#pragma unroll
+            for (int i = 0; i < kMaxActVec; ++i)
+                if (a_loff[i] >= 0) *reinterpret_cast<v4i*>(lds_a + a_loff[i]) = a_reg[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kMaxPackedPix; ++i)
+                if (a_loff[i] >= 0) {
+                    if (p.cstride_b == 4) *reinterpret_cast<int*>(lds_a + a_loff[i]) = a_reg_p[i][0];
+                    else *reinterpret_cast<v2i*>(lds_a + a_loff[i]) = a_reg_p[i];
+                }
+        }
+    };
+    auto stage_rows = [&](int rg) { const int r0 = rg * p.RS; return (p.KH - r0 < p.RS ? p.KH - r0 : p.RS); };
+    auto load_w = [&](int cc, int rg) {
+        const char* src = wkt + ((size_t)cc * p.KH + rg * p.RS) * row_w_b;
+        const int nvec = (stage_rows(rg) * row_w_b) >> 4;
+#pragma unroll
+        for (int i = 0; i < kMaxWVec; ++i) {
+            const int v = tid + kThreads * i;
+            if (v < nvec) w_reg[i] = *reinterpret_cast<const v4i*>(src + (size_t)v * 16);
+        }
+    };
+    auto store_w = [&](int rg) {
+        const int nvec = (stage_rows(rg) * row_w_b) >> 4;
+#pragma unroll
+        for (int i = 0; i < kMaxWVec; ++i) {
+            const int v = tid + kThreads * i;
+            if (v < nvec) *reinterpret_cast<v4i*>(lds_w + v * 16) = w_reg[i];
+        }
+    };
+
+    load_act(0);
+    load_w(0, 0);
+    store_act();
+    store_w(0);
+    __syncthreads();
+
+    for (int st = 0; st < n_stages; ++st) {
+        const int cc = st / p.n_rg, rg = st - cc * p.n_rg;
+        const bool more = st + 1 < n_stages;
+        const bool next_chunk = rg + 1 == p.n_rg;
+        if (more) {
+            if (next_chunk) {
+                load_act(cc + 1);
+                load_w(cc + 1, 0);
+            } else {
+                load_w(cc, rg + 1);
+            }
+        }
+        // ---- MFMA over this stage ----
+        const int rows = stage_rows(rg);
+        const char* wl = lds_w + aoff;
+        for (int rr = 0; rr < rows; ++rr) {
+            const char* arow = lds_a + (rg * p.RS + rr) * p.lds_row_b;
+            for (int q = 0; q < p.KWe; ++q) {
+                const char* apix = arow + q * p.lds_pix_b;
+                for (int j = 0; j < p.KS; ++j) {
+                    v4i af[MT], bf[NT];
+#pragma unroll
+                    for (int m = 0; m < MT; ++m) af[m] = lds_read16(wl + m * 1024);
+#pragma unroll
+                    for (int nn = 0; nn < NT; ++nn) {
+                        if constexpr (PACKED) bf[nn] = lds_read16_unaligned(apix + boff[nn], p.b_align);
+                        else bf[nn] = lds_read16(apix + boff[nn] + j * 32);
+                    }
+#pragma unroll
+                    for (int m = 0; m < MT; ++m)
+#pragma unroll
+                        for (int nn = 0; nn < NT; ++nn) mma<DT>(acc[m][nn], af[m], bf[nn]);
+                    wl += (TM / 32) * 1024;
+                }
+            }
+        }
+        __syncthreads();
+        if (more) {
+            if (next_chunk) {
+                store_act();
+                store_w(0);
+            } else {
+                store_w(rg + 1);
+            }
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue ----
+    const size_t img_px = (size_t)p.OH * p.OW;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int ch0 = kt * TM + (wm * MT + m) * 32 + (lane >> 5) * 16;
+        if (ch0 >= p.kstride && ch0 >= p.K) continue;
+        float sc[16], bi[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const int ch = ch0 + e;
+            sc[e] = (DT == EXHIP_I8 && ch < p.K) ? p.scale[ch] : 0.f;
+            bi[e] = (p.bias && ch < p.K) ? p.bias[ch] : 0.f;
+        }
+#pragma unroll
+        for (int nn = 0; nn < NT; ++nn) {
+            if (!((pvalid >> nn) & 1)) continue;
+            const int oy = oy0 + ppy[nn], ox = ox0 + ppx[nn];
+            const size_t pix = (size_t)n * img_px + (size_t)oy * p.OW + ox;
+            float v[16];
+            if constexpr (DT == EXHIP_I8) {
+                if (p.acc_nchw) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        if (ch0 + e < p.K) p.acc_nchw[((size_t)n * p.K + ch0 + e) * img_px + (size_t)oy * p.OW + ox] = acc[m][nn][e];
+                }
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e], sc[e], bi[e]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = acc[m][nn][e] + bi[e];
+            }
+            if (p.act) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = exhip_act(v[e], p.act);
+            }
+            if (p.residual) {
+                if constexpr (DT == EXHIP_F16) {
+                    const uint16_t* r = reinterpret_cast<const uint16_t*>(p.residual) + pix * p.kstride + ch0;
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        if (ch0 + e < p.K) v[e] += exhip_h2f(r[e]);
+                } else {
+                    const float* r = reinterpret_cast<const float*>(p.residual) + pix * p.kstride + ch0;
+                    if (ch0 + 16 <= p.kstride) {
+#pragma unroll
+                        for (int e4 = 0; e4 < 4; ++e4) {
+                            const v4f rv = *reinterpret_cast<const v4f*>(r + e4 * 4);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e4 * 4 + e] += rv[e];
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            if (ch0 + e < p.K) v[e] += r[e];
+                    }
+                }
+            }
+            if (p.post_relu) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = (0.f > v[e]) ? 0.f : v[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
+            if (p.y_nchw) {
+                float* y = reinterpret_cast<float*>(p.y_nchw);
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    if (ch0 + e < p.K) y[((size_t)n * p.K + ch0 + e) * img_px + (size_t)oy * p.OW + ox] = v[e];
+            }
+            if constexpr (DT == EXHIP_F16) {
+                if (p.y_nchw_h) {
+                    uint16_t* y = reinterpret_cast<uint16_t*>(p.y_nchw_h);
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        if (ch0 + e < p.K) y[((size_t)n * p.K + ch0 + e) * img_px + (size_t)oy * p.OW + ox] = exhip_f2h(v[e]);
+                }
+                if (p.y_q && ch0 + 16 <= p.kstride) {
+                    v4i o[2];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const uint32_t lo = exhip_f2h(v[2 * e]), hi = exhip_f2h(v[2 * e + 1]);
+                        o[e >> 2][e & 3] = (int)(lo | (hi << 16));
+                    }
+                    v4i* y = reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.y_q) + pix * p.kstride + ch0);
+                    y[0] = o[0];
+                    y[1] = o[1];
+                }
+            } else {
+                if (p.y_nhwc) {
+                    float* y = reinterpret_cast<float*>(p.y_nhwc) + pix * p.kstride + ch0;
+                    if (ch0 + 16 <= p.kstride) {
+#pragma unroll
+                        for (int e4 = 0; e4 < 4; ++e4) {
+                            v4f o = {v[e4 * 4], v[e4 * 4 + 1], v[e4 * 4 + 2], v[e4 * 4 + 3]};
+                            *reinterpret_cast<v4f*>(y + e4 * 4) = o;
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            if (ch0 + e < p.kstride) y[e] = v[e];
+                    }
+                }
+                if constexpr (DT == EXHIP_I8) {
+                    if (p.y_q && ch0 + 16 <= p.kstride) {
+                        v4i o;
+#pragma unroll
+                        for (int e4 = 0; e4 < 4; ++e4) {
+                            uint32_t w = 0;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(v[e4 * 4 + e] * p.fs_out) & 0xff) << (8 * e);
+                            o[e4] = (int)w;
+                        }
+                        *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(p.y_q) + pix * p.kstride + ch0) = o;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---- host side: configuration search, packing, launch ----
+
+inline int esize_of(int dt) { return dt == EXHIP_I8 ? 1 : dt == EXHIP_F16 ? 2 : 4; }
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+struct Plan {
+    bool packed;
+    int variant;  // 0: TM 64, TN 256 ; 1: TM 128, TN 256 ; 2: TM 128, TN 128
+    int TM, TN;
+    int KWe, KS, chunk_b, n_chunks, RS, n_rg;
+    int S, tile_step, PH, PW, IH, IW, lds_pix_b, lds_row_b, lds_act_b, lds_w_b, b_align;
+    int tiles_x, tiles_y, ktiles;
+    int OH, OW;
+};
+
+int validate(const exhip_conv_desc* d, int dt) {
+    EXHIP_REQUIRE(d, "conv: NULL descriptor");
+    EXHIP_REQUIRE(d->n > 0 && d->c > 0 && d->h > 0 && d->w > 0 && d->k > 0, "conv: empty shape");
+    EXHIP_REQUIRE(d->kh > 0 && d->kw > 0 && d->sh > 0 && d->sw > 0, "conv: bad kernel/stride");
+    EXHIP_REQUIRE(d->sh == d->sw, "conv: MFMA path needs equal strides (got %dx%d)", d->sh, d->sw);
+    EXHIP_REQUIRE(d->pt >= 0 && d->pb >= 0 && d->pl >= 0 && d->pr >= 0, "conv: negative padding");
+    EXHIP_REQUIRE(d->h + d->pt + d->pb >= d->kh && d->w + d->pl + d->pr >= d->kw, "conv: kernel larger than padded input");
+    EXHIP_REQUIRE(d->c_stride >= d->c, "conv: c_stride %d < c %d", d->c_stride, d->c);
+    const int es = esize_of(dt), cb = d->c_stride * es;
+    const bool packed_ok = (cb == 4 && dt == EXHIP_I8 && d->kw <= 8) || (cb == 8 && dt == EXHIP_F16 && d->kw <= 4);
+    EXHIP_REQUIRE(cb % 32 == 0 || packed_ok, "conv: input pixel is %d bytes; need a multiple of 32 (or the packed first-layer form)", cb);
+    return 0;
+}
+
+// Picks the tile variant, patch shape and staging split for a layer. Maximises the share of issued
+// MFMA work that is useful, subject to the per-thread staging limits and the LDS size.
+int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
+    int rc = validate(d, dt);
+    if (rc) return rc;
+    Plan best;
+    double best_score = -1e30;
+    bool found = false;
+    const int es = esize_of(dt), cb = d->c_stride * es;
+    const int OH = (d->h + d->pt + d->pb - d->kh) / d->sh + 1, OW = (d->w + d->pl + d->pr - d->kw) / d->sw + 1;
+    const bool packed = cb < 32;
+    for (int vc = 0; vc < 6; ++vc) {
+        const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
+        if (packed && chunk_opt == 64) continue;
+        if (!packed && cb % chunk_opt != 0) continue;
+        const int TM = variant == 0 ? 64 : 128, TN = variant == 2 ? 128 : 256;
+        const int ktiles = ceil_div(d->k, TM);
+        Plan p;
+        p.packed = packed;
+        p.variant = variant;
+        p.TM = TM;
+        p.TN = TN;
+        p.OH = OH;
+        p.OW = OW;
+        p.ktiles = ktiles;
+        if (packed) {
+            p.KWe = 1; p.KS = 1; p.chunk_b = 32; p.n_chunks = 1;
+        } else {
+            p.KWe = d->kw;
+            p.chunk_b = chunk_opt;
+            p.KS = p.chunk_b / 32;
+            p.n_chunks = cb / p.chunk_b;
+        }
+        p.tile_step = (d->kh == 1 && d->kw == 1) ? d->sh : 1;
+        p.S = d->sh / p.tile_step;
+        const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;
+        p.RS = (kMaxWVec * kThreads * 16) / row_w_b;
+        if (p.RS < 1) continue;  // one filter row does not fit the staging registers
+        if (p.RS > d->kh) p.RS = d->kh;
+        p.n_rg = ceil_div(d->kh, p.RS);
+        p.lds_w_b = p.RS * row_w_b;
+        for (int PW = 1; PW <= TN && PW <= OW; ++PW) {
+            int PH = TN / PW;
+            if (PH > OH) PH = OH;
+            if (PH < 1) continue;
+            p.PH = PH;
+            p.PW = PW;
+            p.IH = (PH - 1) * p.S + d->kh;
+            if (packed) {
+                const int slots = 32 / cb;
+                p.IW = (PW - 1) * p.S + slots;
+                p.lds_pix_b = cb;
+                p.lds_row_b = (p.IW * cb + 15) / 16 * 16;
+                const int step = p.S * cb;
+                p.b_align = step % 16 == 0 ? 16 : step % 8 == 0 ? 8 : 4;
+                if (p.IH * p.IW > kMaxPackedPix * kThreads) continue;
+            } else {
+                p.IW = (PW - 1) * p.S + d->kw;
+                p.lds_pix_b = p.chunk_b + 16;
+                p.lds_row_b = p.IW * p.lds_pix_b;
+                p.b_align = 16;
+                if (p.IH * p.IW * (p.chunk_b / 16) > kMaxActVec * kThreads) continue;
+            }
+            p.lds_act_b = (p.IH * p.lds_row_b + 63) / 64 * 64;
+            if (p.lds_act_b + p.lds_w_b > 150 * 1024) continue;
+            p.tiles_y = ceil_div(OH, PH);
+            p.tiles_x = ceil_div(OW, PW);
+            const double useful = (double)OH * OW * d->k;
+            const double issued = (double)p.tiles_y * p.tiles_x * TN * ktiles * TM;
+            // prefer square-ish patches (less halo) at equal utilisation
+            const double halo = (double)p.IH * p.IW / ((double)PH * PW * p.S * p.S);
+            // small preferences: wide channel tiles re-stage the input less often, 64-byte chunks halve
+            // the number of stages, the 128-pixel variant has the least reuse per staged byte
+            const double score = useful / issued - 0.01 * halo + (TM == 128 ? 0.005 : 0.0) -
+                                 (chunk_opt == 32 ? 0.004 : 0.0) - (variant == 2 ? 0.02 : 0.0);
+            if (!found || score > best_score) {
+                best_score = score;
+                best = p;
+                found = true;
+            }
+        }
+    }
+    if (!found) {
+        exhip_set_error("conv: no tile configuration fits (kernel %dx%d, pixel bytes %d)", d->kh, d->kw, cb);
+        return EXHIP_ERR_UNSUPPORTED;
+    }
+    *out = best;
+    return 0;
+}
+
+template <int DT, bool PACKED>
+int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid, size_t lds) {
+    if (pl.variant == 0) {
+        auto k = conv_igemm_kernel<DT, 2, 2, 1, 4, PACKED>;
+        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), lds, ctx->stream, p);
+    } else if (pl.variant == 1) {
+        auto k = conv_igemm_kernel<DT, 4, 2, 1, 4, PACKED>;
+        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), lds, ctx->stream, p);
+    } else {
+        auto k = conv_igemm_kernel<DT, 2, 2, 2, 2, PACKED>;
+        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), lds, ctx->stream, p);
+    }
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+template <int DT>
+int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p) {
+    EXHIP_REQUIRE(ctx, "conv: NULL ctx");
+    Plan pl;
+    int rc = make_plan(d, DT, &pl);
+    if (rc) return rc;
+    EXHIP_REQUIRE(p.x && p.wp, "conv: NULL input or weights");
+    EXHIP_REQUIRE(d->k_stride >= d->k || (!p.y_q && !p.y_nhwc && !p.residual), "conv: k_stride %d < k %d", d->k_stride, d->k);
+    EXHIP_REQUIRE(!(p.y_q) || d->k_stride % 16 == 0, "conv: NHWC int8/half output needs k_stride %% 16 == 0");
+    p.N = d->n; p.H = d->h; p.W = d->w; p.K = d->k; p.OH = pl.OH; p.OW = pl.OW;
+    p.KH = d->kh; p.KWe = pl.KWe; p.KS = pl.KS; p.S = pl.S; p.tile_step = pl.tile_step;
+    p.PT = d->pt; p.PL = d->pl;
+    p.cstride_b = d->c_stride * esize_of(DT);
+    p.kstride = d->k_stride;
+    p.PH = pl.PH; p.PW = pl.PW; p.IH = pl.IH; p.IW = pl.IW;
+    p.lds_pix_b = pl.lds_pix_b; p.lds_row_b = pl.lds_row_b; p.lds_act_b = pl.lds_act_b;
+    p.n_chunks = pl.n_chunks; p.chunk_b = pl.chunk_b; p.RS = pl.RS; p.n_rg = pl.n_rg;
+    p.tiles_x = pl.tiles_x; p.tiles_y = pl.tiles_y; p.ktiles = pl.ktiles;
+    p.act = d->act; p.post_relu = d->post_relu; p.fs_out = d->fs_out; p.b_align = pl.b_align;
+    const long long grid = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
+    EXHIP_REQUIRE(grid > 0 && grid < (1ll << 31), "conv: grid too large");
+    // a lane reads 16 bytes at its fragment offset: keep the last read inside the allocation
+    const size_t lds = (size_t)pl.lds_act_b + pl.lds_w_b + 64;
+    if (pl.packed) return launch_variant<DT, true>(ctx, pl, p, (int)grid, lds);
+    return launch_variant<DT, false>(ctx, pl, p, (int)grid, lds);
+}
+
+template <typename T>
+void pack_weights_t(const exhip_conv_desc* d, int dt, const Plan& pl, const T* w, char* out) {
+    const int es = esize_of(dt), cb = d->c_stride * es;
+    const int mts = pl.TM / 32;
+    const int C = d->c, K = d->k, KH = d->kh, KW = d->kw;
+    size_t o = 0;
+    for (int kt = 0; kt < pl.ktiles; ++kt)
+        for (int cc = 0; cc < pl.n_chunks; ++cc)
+            for (int r = 0; r < KH; ++r)
+                for (int q = 0; q < pl.KWe; ++q)
+                    for (int j = 0; j < pl.KS; ++j)
+                        for (int mt = 0; mt < mts; ++mt)
+                            for (int lane = 0; lane < 64; ++lane) {
+                                const int rr = lane % 32, h = lane / 32;
+                                const int chan = ((rr / 4) % 2) * 16 + (rr / 8) * 4 + (rr % 4);
+                                const int k = kt * pl.TM + mt * 32 + chan;
+                                for (int e = 0; e < 16 / es; ++e, o += es) {
+                                    T val = 0;
+                                    if (pl.packed) {
+                                        const int byte = h * 16 + e * es;
+                                        const int slot = byte / cb, c = (byte % cb) / es;
+                                        if (k < K && slot < KW && c < C) val = w[(((size_t)k * C + c) * KH + r) * KW + slot];
+                                    } else {
+                                        const int c = (cc * pl.chunk_b + j * 32 + h * 16) / es + e;
+                                        if (k < K && c < C) val = w[(((size_t)k * C + c) * KH + r) * KW + q];
+                                    }
+                                    memcpy(out + o, &val, es);
+                                }
+                            }
+}
+
+}  // namespace
+
+extern "C" int exhip_conv_out_hw(const exhip_conv_desc* d, int* oh, int* ow) {
+    EXHIP_REQUIRE(d && oh && ow, "exhip_conv_out_hw: NULL argument");
+    EXHIP_REQUIRE(d->sh > 0 && d->sw > 0, "exhip_conv_out_hw: bad stride");
+    *oh = (d->h + d->pt + d->pb - d->kh) / d->sh + 1;
+    *ow = (d->w + d->pl + d->pr - d->kw) / d->sw + 1;
+    return 0;
+}
+
+extern "C" size_t exhip_conv_packed_bytes(const exhip_conv_desc* d, int dtype) {
+    Plan pl;
+    if (dtype < 0 || dtype > 2 || make_plan(d, dtype, &pl)) return 0;
+    return (size_t)pl.ktiles * pl.n_chunks * d->kh * pl.KWe * pl.KS * (pl.TM / 32) * 1024;
+}
+
+extern "C" int exhip_conv_pack_weights(const exhip_conv_desc* d, int dtype, const void* w, void* packed) {
+    EXHIP_REQUIRE(w && packed, "exhip_conv_pack_weights: NULL argument");
+    EXHIP_REQUIRE(dtype >= 0 && dtype <= 2, "exhip_conv_pack_weights: bad dtype %d", dtype);
+    Plan pl;
+    int rc = make_plan(d, dtype, &pl);
+    if (rc) return rc;
+    if (dtype == EXHIP_I8) pack_weights_t<int8_t>(d, dtype, pl, (const int8_t*)w, (char*)packed);
+    else if (dtype == EXHIP_F16) pack_weights_t<uint16_t>(d, dtype, pl, (const uint16_t*)w, (char*)packed);
+    else pack_weights_t<float>(d, dtype, pl, (const float*)w, (char*)packed);
+    return 0;
+}
+
+extern "C" int exhip_conv2d_i8(exhip_ctx* ctx, const exhip_conv_desc* d, const int8_t* x, const void* wp,
+                               const float* scale, const float* bias, const float* residual, int8_t* y_i8,
+                               float* y_f32_nhwc, float* y_f32_nchw, int32_t* acc_nchw) {
+    EXHIP_REQUIRE(scale, "exhip_conv2d_i8: NULL scale");
+    EXHIP_REQUIRE(y_i8 || y_f32_nhwc || y_f32_nchw || acc_nchw, "exhip_conv2d_i8: no output requested");
+    ConvParams p = {};
+    p.x = (const char*)x; p.wp = (const char*)wp; p.scale = scale; p.bias = bias; p.residual = residual;
+    p.y_q = y_i8; p.y_nhwc = y_f32_nhwc; p.y_nchw = y_f32_nchw; p.acc_nchw = acc_nchw;
+    return run_conv<EXHIP_I8>(ctx, d, p);
+}
+
+extern "C" int exhip_conv2d_f16(exhip_ctx* ctx, const exhip_conv_desc* d, const uint16_t* x, const void* wp,
+                                const float* bias, const uint16_t* residual, uint16_t* y_f16_nhwc,
+                                uint16_t* y_f16_nchw, float* y_f32_nchw) {
+    EXHIP_REQUIRE(y_f16_nhwc || y_f16_nchw || y_f32_nchw, "exhip_conv2d_f16: no output requested");
+    ConvParams p = {};
+    p.x = (const char*)x; p.wp = (const char*)wp; p.bias = bias; p.residual = residual;
+    p.y_q = y_f16_nhwc; p.y_nchw_h = y_f16_nchw; p.y_nchw = y_f32_nchw;
+    return run_conv<EXHIP_F16>(ctx, d, p);
+}
+
+extern "C" int exhip_conv2d_f32(exhip_ctx* ctx, const exhip_conv_desc* d, const float* x, const void* wp,
+                                const float* bias, const float* residual, float* y_f32_nhwc, float* y_f32_nchw) {
+    EXHIP_REQUIRE(y_f32_nhwc || y_f32_nchw, "exhip_conv2d_f32: no output requested");
+    ConvParams p = {};
+    p.x = (const char*)x; p.wp = (const char*)wp; p.bias = bias; p.residual = residual;
+    p.y_nhwc = y_f32_nhwc; p.y_nchw = y_f32_nchw;
+    return run_conv<EXHIP_F32>(ctx, d, p);
+}

@@ -1,0 +1,133 @@
+// exhip runtime: context, memory, events. Everything runs on one stream per context.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+static thread_local char g_err[512] = "";
+
+void exhip_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+extern "C" const char* exhip_last_error(void) { return g_err; }
+
+extern "C" int exhip_init(int device, exhip_ctx** out) {
+    EXHIP_REQUIRE(out != nullptr, "exhip_init: ctx is NULL");
+    int count = 0;
+    EXHIP_CHECK(hipGetDeviceCount(&count));
+    EXHIP_REQUIRE(device >= 0 && device < count, "exhip_init: device %d out of range (have %d)", device, count);
+    EXHIP_CHECK(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    EXHIP_CHECK(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        exhip_set_error("exhip_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+        return EXHIP_ERR_UNSUPPORTED;
+    }
+    exhip_ctx* c = new exhip_ctx();
+    c->device = device;
+    hipError_t e = hipStreamCreate(&c->stream);  // default priority
+    if (e != hipSuccess) {
+        delete c;
+        exhip_set_error("hipStreamCreate failed: %s", hipGetErrorString(e));
+        return (int)e;
+    }
+    *out = c;
+    return 0;
+}
+
+extern "C" int exhip_destroy(exhip_ctx* ctx) {
+    if (!ctx) return 0;
+    hipStreamSynchronize(ctx->stream);
+    hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return 0;
+}
+
+extern "C" int exhip_malloc(exhip_ctx* ctx, size_t bytes, void** dptr) {
+    EXHIP_REQUIRE(ctx && dptr, "exhip_malloc: NULL argument");
+    EXHIP_CHECK(hipMalloc(dptr, bytes ? bytes : 1));
+    return 0;
+}
+
+extern "C" int exhip_free(exhip_ctx* ctx, void* dptr) {
+    EXHIP_REQUIRE(ctx, "exhip_free: NULL ctx");
+    if (dptr) {
+        EXHIP_CHECK(hipStreamSynchronize(ctx->stream));
+        EXHIP_CHECK(hipFree(dptr));
+    }
+    return 0;
+}
+
+extern "C" int exhip_memset(exhip_ctx* ctx, void* dptr, int value, size_t bytes) {
+    EXHIP_REQUIRE(ctx && (dptr || !bytes), "exhip_memset: NULL argument");
+    if (bytes) EXHIP_CHECK(hipMemsetAsync(dptr, value, bytes, ctx->stream));
+    return 0;
+}
+
+extern "C" int exhip_memcpy_h2d(exhip_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    EXHIP_REQUIRE(ctx && ((dst && src) || !bytes), "exhip_memcpy_h2d: NULL argument");
+    if (bytes) {
+        EXHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+        EXHIP_CHECK(hipStreamSynchronize(ctx->stream));  // src may be pageable and reused by the caller
+    }
+    return 0;
+}
+
+extern "C" int exhip_memcpy_d2h(exhip_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    EXHIP_REQUIRE(ctx && ((dst && src) || !bytes), "exhip_memcpy_d2h: NULL argument");
+    if (bytes) {
+        EXHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+        EXHIP_CHECK(hipStreamSynchronize(ctx->stream));
+    }
+    return 0;
+}
+
+extern "C" int exhip_memcpy_d2d(exhip_ctx* ctx, void* dst, const void* src, size_t bytes) {
+    EXHIP_REQUIRE(ctx && ((dst && src) || !bytes), "exhip_memcpy_d2d: NULL argument");
+    if (bytes) EXHIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return 0;
+}
+
+extern "C" int exhip_sync(exhip_ctx* ctx) {
+    EXHIP_REQUIRE(ctx, "exhip_sync: NULL ctx");
+    EXHIP_CHECK(hipStreamSynchronize(ctx->stream));
+    return 0;
+}
+
+extern "C" int exhip_device_name(exhip_ctx* ctx, char* buf, size_t len) {
+    EXHIP_REQUIRE(ctx && buf && len, "exhip_device_name: NULL argument");
+    hipDeviceProp_t prop;
+    EXHIP_CHECK(hipGetDeviceProperties(&prop, ctx->device));
+    snprintf(buf, len, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return 0;
+}
+
+extern "C" int exhip_event_create(void** ev) {
+    EXHIP_REQUIRE(ev, "exhip_event_create: NULL argument");
+    hipEvent_t e;
+    EXHIP_CHECK(hipEventCreate(&e));
+    *ev = (void*)e;
+    return 0;
+}
+
+extern "C" int exhip_event_destroy(void* ev) {
+    if (ev) EXHIP_CHECK(hipEventDestroy((hipEvent_t)ev));
+    return 0;
+}
+
+extern "C" int exhip_event_record(exhip_ctx* ctx, void* ev) {
+    EXHIP_REQUIRE(ctx && ev, "exhip_event_record: NULL argument");
+    EXHIP_CHECK(hipEventRecord((hipEvent_t)ev, ctx->stream));
+    return 0;
+}
+
+extern "C" int exhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms) {
+    EXHIP_REQUIRE(ev_start && ev_stop && ms, "exhip_event_elapsed_ms: NULL argument");
+    EXHIP_CHECK(hipEventSynchronize((hipEvent_t)ev_stop));
+    EXHIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)ev_start, (hipEvent_t)ev_stop));
+    return 0;
+}

@@ -1,0 +1,318 @@
+"""ctypes binding of the exhip C ABI (include/exhip.h) with numpy at the host boundary.
+
+This is the Python face of the product library: it loads excalibur_amd/lib/libexhip.so and fails
+loudly if that library or a gfx950 device is missing. There is no CPU fallback.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libexhip.so")
+
+I8, F16, F32 = 0, 1, 2
+_NP = {I8: np.int8, F16: np.uint16, F32: np.float32}
+
+
+class ExhipError(RuntimeError):
+    pass
+
+
+class ConvDesc(ctypes.Structure):
+    _fields_ = [(k, ctypes.c_int) for k in
+                ("n", "c", "h", "w", "k", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr", "act", "c_stride", "k_stride",
+                 "post_relu")] + [("fs_out", ctypes.c_float)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ExhipError(f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                             "or `make -C excalibur_amd/csrc`")
+        L = ctypes.CDLL(LIB_PATH)
+        L.exhip_last_error.restype = ctypes.c_char_p
+        L.exhip_conv_packed_bytes.restype = ctypes.c_size_t
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise ExhipError(f"exhip error {rc}: {lib().exhip_last_error().decode()}")
+
+
+def pad_to(v, m):
+    return (v + m - 1) // m * m
+
+
+class DevArray:
+    """A device allocation with a logical numpy shape/dtype."""
+
+    def __init__(self, ctx, shape, dtype):
+        self.ctx = ctx
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = ctypes.c_void_p()
+        _check(lib().exhip_malloc(ctx.h, ctypes.c_size_t(self.nbytes), ctypes.byref(p)))
+        self.ptr = p
+
+    @property
+    def size(self):
+        return self.nbytes // self.dtype.itemsize
+
+    def upload(self, a):
+        a = np.ascontiguousarray(a, self.dtype)
+        assert a.nbytes == self.nbytes, (a.shape, self.shape)
+        _check(lib().exhip_memcpy_h2d(self.ctx.h, self.ptr, a.ctypes.data_as(ctypes.c_void_p), ctypes.c_size_t(self.nbytes)))
+        return self
+
+    def download(self):
+        out = np.empty(self.shape, self.dtype)
+        _check(lib().exhip_memcpy_d2h(self.ctx.h, out.ctypes.data_as(ctypes.c_void_p), self.ptr, ctypes.c_size_t(self.nbytes)))
+        return out
+
+    def zero(self):
+        _check(lib().exhip_memset(self.ctx.h, self.ptr, 0, ctypes.c_size_t(self.nbytes)))
+        return self
+
+    def free(self):
+        if self.ptr:
+            _check(lib().exhip_free(self.ctx.h, self.ptr))
+            self.ptr = None
+
+
+class Event:
+    def __init__(self):
+        self.h = ctypes.c_void_p()
+        _check(lib().exhip_event_create(ctypes.byref(self.h)))
+
+    def record(self, ctx):
+        _check(lib().exhip_event_record(ctx.h, self.h))
+
+    def elapsed_ms(self, stop):
+        ms = ctypes.c_float()
+        _check(lib().exhip_event_elapsed_ms(self.h, stop.h, ctypes.byref(ms)))
+        return ms.value
+
+
+def _ptr(a):
+    return a.ptr if a is not None else None
+
+
+class Ctx:
+    def __init__(self, device=0):
+        self.h = ctypes.c_void_p()
+        _check(lib().exhip_init(int(device), ctypes.byref(self.h)))
+
+    def close(self):
+        if self.h:
+            lib().exhip_destroy(self.h)
+            self.h = None
+
+    def device_name(self):
+        buf = ctypes.create_string_buffer(256)
+        _check(lib().exhip_device_name(self.h, buf, ctypes.c_size_t(256)))
+        return buf.value.decode()
+
+    def sync(self):
+        _check(lib().exhip_sync(self.h))
+
+    def empty(self, shape, dtype):
+        return DevArray(self, shape, dtype)
+
+    def array(self, a, dtype=None):
+        a = np.ascontiguousarray(a, dtype if dtype is not None else a.dtype)
+        return DevArray(self, a.shape, a.dtype).upload(a)
+
+    # ---- layout / precision ----
+    def quantize_nchw_to_nhwc_i8(self, x, fs, c_stride, fs_per_channel=None):
+        n, c, h, w = x.shape
+        y = self.empty((n, h, w, c_stride), np.int8)
+        _check(lib().exhip_quantize_nchw_f32_to_nhwc_i8(self.h, x.ptr, n, c, h, w, ctypes.c_float(float(fs)),
+                                                       _ptr(fs_per_channel), c_stride, y.ptr))
+        return y
+
+    def nchw_to_nhwc(self, x, c_stride, out="f32"):
+        n, c, h, w = x.shape
+        if x.dtype == np.float32 and out == "f32":
+            y = self.empty((n, h, w, c_stride), np.float32)
+            _check(lib().exhip_nchw_f32_to_nhwc_f32(self.h, x.ptr, n, c, h, w, c_stride, y.ptr))
+        elif x.dtype == np.float32 and out == "f16":
+            y = self.empty((n, h, w, c_stride), np.uint16)
+            _check(lib().exhip_nchw_f32_to_nhwc_f16(self.h, x.ptr, n, c, h, w, c_stride, y.ptr))
+        else:
+            y = self.empty((n, h, w, c_stride), np.uint16)
+            _check(lib().exhip_nchw_f16_to_nhwc_f16(self.h, x.ptr, n, c, h, w, c_stride, y.ptr))
+        return y
+
+    def nhwc_to_nchw(self, x, c, out="f32"):
+        n, h, w, cs = x.shape
+        if x.dtype == np.float32:
+            y = self.empty((n, c, h, w), np.float32)
+            _check(lib().exhip_nhwc_f32_to_nchw_f32(self.h, x.ptr, n, c, h, w, cs, y.ptr))
+        elif out == "f32":
+            y = self.empty((n, c, h, w), np.float32)
+            _check(lib().exhip_nhwc_f16_to_nchw_f32(self.h, x.ptr, n, c, h, w, cs, y.ptr))
+        else:
+            y = self.empty((n, c, h, w), np.uint16)
+            _check(lib().exhip_nhwc_f16_to_nchw_f16(self.h, x.ptr, n, c, h, w, cs, y.ptr))
+        return y
+
+    def f32_to_f16(self, x):
+        y = self.empty(x.shape, np.uint16)
+        _check(lib().exhip_f32_to_f16(self.h, x.ptr, y.ptr, ctypes.c_size_t(x.size)))
+        return y
+
+    def f16_to_f32(self, x):
+        y = self.empty(x.shape, np.float32)
+        _check(lib().exhip_f16_to_f32(self.h, x.ptr, y.ptr, ctypes.c_size_t(x.size)))
+        return y
+
+    # ---- convolution ----
+    @staticmethod
+    def conv_desc(n, c, h, w, k, kernel, stride=1, pad=0, act=0, c_stride=None, k_stride=None, post_relu=0, fs_out=0.0):
+        kh, kw = (kernel, kernel) if np.isscalar(kernel) else kernel
+        sh, sw = (stride, stride) if np.isscalar(stride) else stride
+        pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+        return ConvDesc(n, c, h, w, k, kh, kw, sh, sw, pt, pb, pl, pr, act, c_stride if c_stride else c,
+                        k_stride if k_stride else k, post_relu, fs_out)
+
+    @staticmethod
+    def conv_out_hw(d):
+        oh, ow = ctypes.c_int(), ctypes.c_int()
+        _check(lib().exhip_conv_out_hw(ctypes.byref(d), ctypes.byref(oh), ctypes.byref(ow)))
+        return oh.value, ow.value
+
+    def pack_conv_weights(self, d, dtype, w_oihw):
+        nbytes = lib().exhip_conv_packed_bytes(ctypes.byref(d), dtype)
+        if nbytes == 0:
+            raise ExhipError(f"exhip_conv_packed_bytes: {lib().exhip_last_error().decode()}")
+        w = np.ascontiguousarray(w_oihw, _NP[dtype])
+        packed = np.empty(nbytes, np.uint8)
+        _check(lib().exhip_conv_pack_weights(ctypes.byref(d), dtype, w.ctypes.data_as(ctypes.c_void_p),
+                                             packed.ctypes.data_as(ctypes.c_void_p)))
+        return self.array(packed)
+
+    def conv2d_i8(self, d, x, wp, scale, bias=None, residual=None, y_i8=None, y_f32_nhwc=None, y_f32_nchw=None, acc=None):
+        _check(lib().exhip_conv2d_i8(self.h, ctypes.byref(d), x.ptr, wp.ptr, scale.ptr, _ptr(bias), _ptr(residual),
+                                     _ptr(y_i8), _ptr(y_f32_nhwc), _ptr(y_f32_nchw), _ptr(acc)))
+
+    def conv2d_f16(self, d, x, wp, bias=None, residual=None, y_f16_nhwc=None, y_f16_nchw=None, y_f32_nchw=None):
+        _check(lib().exhip_conv2d_f16(self.h, ctypes.byref(d), x.ptr, wp.ptr, _ptr(bias), _ptr(residual), _ptr(y_f16_nhwc),
+                                      _ptr(y_f16_nchw), _ptr(y_f32_nchw)))
+
+    def conv2d_f32(self, d, x, wp, bias=None, residual=None, y_f32_nhwc=None, y_f32_nchw=None):
+        _check(lib().exhip_conv2d_f32(self.h, ctypes.byref(d), x.ptr, wp.ptr, _ptr(bias), _ptr(residual), _ptr(y_f32_nhwc),
+                                      _ptr(y_f32_nchw)))
+
+    def conv2d_direct(self, d, groups, x, y, w_f32=None, w_i8=None, fs=1.0, scale=None, bias=None):
+        _check(lib().exhip_conv2d_direct_nchw(self.h, ctypes.byref(d), groups, x.ptr, _ptr(w_f32), _ptr(w_i8),
+                                              ctypes.c_float(float(fs)), _ptr(scale), _ptr(bias), y.ptr))
+
+    # ---- bandwidth-bound operators ----
+    def dwconv3x3_nchw_f32(self, x, w9, bias, stride, pad, act):
+        n, c, h, w = x.shape
+        pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+        oh, ow = (h + pt + pb - 3) // stride + 1, (w + pl + pr - 3) // stride + 1
+        y = self.empty((n, c, oh, ow), np.float32)
+        _check(lib().exhip_dwconv3x3_nchw_f32(self.h, x.ptr, w9.ptr, _ptr(bias), y.ptr, n, c, h, w, stride, pt, pb, pl, pr, act))
+        return y
+
+    def dwconv3x3_nhwc_f16(self, x, c, w9, bias, stride, pad, act):
+        n, h, w, cs = x.shape
+        pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+        oh, ow = (h + pt + pb - 3) // stride + 1, (w + pl + pr - 3) // stride + 1
+        y = self.empty((n, oh, ow, cs), np.uint16)
+        _check(lib().exhip_dwconv3x3_nhwc_f16(self.h, x.ptr, w9.ptr, _ptr(bias), y.ptr, n, c, h, w, cs, stride, pt, pb, pl, pr,
+                                              act))
+        return y
+
+    def dw_dequant_weights(self, w_i8, ws):
+        k = w_i8.shape[0]
+        wf = self.empty(w_i8.shape, np.float32)
+        _check(lib().exhip_dw_dequant_weights(self.h, w_i8.ptr, ws.ptr, wf.ptr, k, w_i8.size // k))
+        return wf
+
+    @staticmethod
+    def pool_out_hw(h, w, kh, kw, sh, sw, pt, pb, pl, pr, pad_mode):
+        oh, ow = ctypes.c_int(), ctypes.c_int()
+        _check(lib().exhip_pool_out_hw(h, w, kh, kw, sh, sw, pt, pb, pl, pr, pad_mode, ctypes.byref(oh), ctypes.byref(ow)))
+        return oh.value, ow.value
+
+    @staticmethod
+    def _pool_args(h, w, kernel, stride, pad, global_pool, pad_mode):
+        kh, kw = (kernel, kernel) if np.isscalar(kernel) else kernel
+        sh, sw = (stride, stride) if np.isscalar(stride) else stride
+        pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+        if global_pool:  # src/Excalibur/operation_pooling.cpp:90-100
+            kh, kw, sh, sw, pt, pb, pl, pr = h, w, 1, 1, 0, 0, 0, 0
+        oh, ow = Ctx.pool_out_hw(h, w, kh, kw, sh, sw, pt, pb, pl, pr, pad_mode)
+        return kh, kw, sh, sw, pt, pb, pl, pr, oh, ow
+
+    def pool2d_nchw_f32(self, x, ptype, kernel=0, stride=1, pad=0, global_pool=False, pad_mode=1, count_include_pad=0):
+        n, c, h, w = x.shape
+        kh, kw, sh, sw, pt, pb, pl, pr, oh, ow = self._pool_args(h, w, kernel, stride, pad, global_pool, pad_mode)
+        y = self.empty((n, c, oh, ow), np.float32)
+        _check(lib().exhip_pool2d_nchw_f32(self.h, x.ptr, y.ptr, n, c, h, w, oh, ow, ptype, kh, kw, sh, sw, pt, pb, pl, pr,
+                                           count_include_pad))
+        return y
+
+    def maxpool2d_nhwc_f32(self, x, c, kernel, stride, pad, fs_out=None, want_f32=True):
+        n, h, w, cs = x.shape
+        kh, kw, sh, sw, pt, pb, pl, pr, oh, ow = self._pool_args(h, w, kernel, stride, pad, False, 1)
+        y = self.empty((n, oh, ow, cs), np.float32) if want_f32 else None
+        yq = self.empty((n, oh, ow, cs), np.int8) if fs_out is not None else None
+        _check(lib().exhip_maxpool2d_nhwc_f32(self.h, x.ptr, _ptr(y), _ptr(yq), ctypes.c_float(float(fs_out or 0.0)), n, c, h,
+                                              w, cs, oh, ow, kh, kw, sh, sw, pt, pl))
+        return y, yq
+
+    def pool2d_nhwc_f16(self, x, c, ptype, kernel=0, stride=1, pad=0, global_pool=False, pad_mode=1, count_include_pad=0):
+        n, h, w, cs = x.shape
+        kh, kw, sh, sw, pt, pb, pl, pr, oh, ow = self._pool_args(h, w, kernel, stride, pad, global_pool, pad_mode)
+        y = self.empty((n, oh, ow, cs), np.uint16)
+        _check(lib().exhip_pool2d_nhwc_f16(self.h, x.ptr, y.ptr, n, c, h, w, cs, oh, ow, ptype, kh, kw, sh, sw, pt, pb, pl, pr,
+                                           count_include_pad))
+        return y
+
+    def eltwise_f32(self, inputs, etype, coeffs=None):
+        ptrs = (ctypes.c_void_p * len(inputs))(*[a.ptr.value for a in inputs])
+        co = None
+        if coeffs is not None:
+            co = (ctypes.c_float * len(inputs))(*[float(v) for v in coeffs])
+        y = self.empty(inputs[0].shape, np.float32)
+        _check(lib().exhip_eltwise_f32(self.h, ptrs, len(inputs), co, etype, y.ptr, ctypes.c_size_t(y.size)))
+        return y
+
+    def add_f32(self, a, b, relu=False):
+        y = self.empty(a.shape, np.float32)
+        _check(lib().exhip_add_f32(self.h, a.ptr, b.ptr, y.ptr, ctypes.c_size_t(y.size), int(relu)))
+        return y
+
+    def relu_f32(self, x):
+        y = self.empty(x.shape, np.float32)
+        _check(lib().exhip_relu_f32(self.h, x.ptr, y.ptr, ctypes.c_size_t(y.size)))
+        return y
+
+    def add_f16(self, a, b, relu=False):
+        y = self.empty(a.shape, np.uint16)
+        _check(lib().exhip_add_f16(self.h, a.ptr, b.ptr, y.ptr, ctypes.c_size_t(y.size), int(relu)))
+        return y
+
+    def relu_f16(self, x):
+        y = self.empty(x.shape, np.uint16)
+        _check(lib().exhip_relu_f16(self.h, x.ptr, y.ptr, ctypes.c_size_t(y.size)))
+        return y
+
+    def innerproduct_f32(self, x, w, bias=None):
+        m = x.shape[0]
+        k_in = x.size // m
+        n_out = w.size // k_in
+        y = self.empty((m, n_out, 1, 1), np.float32)
+        _check(lib().exhip_innerproduct_f32(self.h, x.ptr, w.ptr, _ptr(bias), y.ptr, m, n_out, k_in))
+        return y

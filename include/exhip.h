@@ -1,0 +1,177 @@
+/* exhip: C ABI of the MI355X (gfx950) backend for Excalibur's CNN forward hot path.
+ *
+ * Plain pointers and sizes only. Every function returns 0 on success and a non-zero code on
+ * failure (a hipError_t, or EXHIP_ERR_* for argument errors); nothing throws. exhip_last_error()
+ * returns a text for the last failure on the calling thread. Device pointers are raw HIP device
+ * addresses; the library never owns or frees caller memory.
+ *
+ * The reference (zhousheng-zser/Excalibur) has no C interface for its operators: each entry below
+ * states the C++ member function whose device-side work it replaces (paths relative to the reference
+ * tree). The C++ operator classes of this repository (excalibur_amd/host) override the reference's
+ * forward_gpu_{f32,f16,i8} virtuals (include/Excalibur/operation.hpp:172-183,268-276,359-370) and call
+ * only these functions.
+ *
+ * Tensor layouts
+ *   NCHW f32 / f16 : the reference's boundary layout (include/Primitives/tensor.hpp:124-134), dense.
+ *   NHWC i8/f16/f32: internal, channel-fastest with a channel stride `c_stride` >= C elements (pad
+ *                    channels hold zeros). Convolution inputs need c_stride * sizeof(elem) to be a
+ *                    multiple of 32 bytes, or exactly 4 bytes (i8, C <= 4) / 8 bytes (f16, C <= 4)
+ *                    for the packed first-layer form.
+ */
+#ifndef EXHIP_H_
+#define EXHIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EXHIP_ERR_ARG 10001        /* invalid argument / unsupported geometry */
+#define EXHIP_ERR_UNSUPPORTED 10002
+
+typedef struct exhip_ctx exhip_ctx; /* one device + one stream; not thread-safe, like a reference pipeline */
+
+/* ---- runtime: replaces syncedmem's cudaMalloc/cudaMemcpy use, src/Primitives/syncedmem.cpp:176-276 ---- */
+int exhip_init(int device, exhip_ctx** ctx);
+int exhip_destroy(exhip_ctx* ctx);
+int exhip_malloc(exhip_ctx* ctx, size_t bytes, void** dptr);
+int exhip_free(exhip_ctx* ctx, void* dptr);
+int exhip_memset(exhip_ctx* ctx, void* dptr, int value, size_t bytes);
+int exhip_memcpy_h2d(exhip_ctx* ctx, void* dst, const void* src, size_t bytes);
+int exhip_memcpy_d2h(exhip_ctx* ctx, void* dst, const void* src, size_t bytes);
+int exhip_memcpy_d2d(exhip_ctx* ctx, void* dst, const void* src, size_t bytes);
+int exhip_sync(exhip_ctx* ctx);
+const char* exhip_last_error(void);
+int exhip_device_name(exhip_ctx* ctx, char* buf, size_t len);
+
+/* HIP events on the context's stream, for timing kernels where they are launched
+ * (the reference times with a host clock, include/Primitives/profiler.hpp:186-226). */
+int exhip_event_create(void** ev);
+int exhip_event_destroy(void* ev);
+int exhip_event_record(exhip_ctx* ctx, void* ev);
+int exhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms); /* synchronises on ev_stop */
+
+/* ---- layout / precision conversion at the boundary ---- */
+/* quantize_float32_to_int8 (src/Excalibur/operation_general_conv.cpp:584-720) fused with NCHW->NHWC:
+ * y[n,h,w,c] = sat8(trunc(x[n,c,h,w]*fs +- 0.5)); fs per tensor (fs_per_channel == NULL) or a device
+ * array of C per-input-channel scales. Pad channels c in [C, c_stride) are written as 0. */
+int exhip_quantize_nchw_f32_to_nhwc_i8(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, float fs,
+                                       const float* fs_per_channel, int c_stride, int8_t* y);
+/* NCHW f32 -> NHWC f32 / f16 (round to nearest even) with zero pad channels; NCHW f16 -> NHWC f16. */
+int exhip_nchw_f32_to_nhwc_f32(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, int c_stride, float* y);
+int exhip_nchw_f32_to_nhwc_f16(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, int c_stride, uint16_t* y);
+int exhip_nchw_f16_to_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, int n, int c, int h, int w, int c_stride, uint16_t* y);
+/* NHWC -> NCHW f32 (drops pad channels). */
+int exhip_nhwc_f32_to_nchw_f32(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, int c_stride, float* y);
+int exhip_nhwc_f16_to_nchw_f32(exhip_ctx* ctx, const uint16_t* x, int n, int c, int h, int w, int c_stride, float* y);
+int exhip_nhwc_f16_to_nchw_f16(exhip_ctx* ctx, const uint16_t* x, int n, int c, int h, int w, int c_stride, uint16_t* y);
+/* float2half / half2float on flat arrays (src/Primitives/simd_types.cpp:198-252); round to nearest even. */
+int exhip_f32_to_f16(exhip_ctx* ctx, const float* x, uint16_t* y, size_t count);
+int exhip_f16_to_f32(exhip_ctx* ctx, const uint16_t* x, float* y, size_t count);
+
+/* ---- dense convolution as an implicit GEMM on MFMA ---- */
+enum { EXHIP_I8 = 0, EXHIP_F16 = 1, EXHIP_F32 = 2 };
+/* activation codes of the reference's key 9 (src/Excalibur/operation_general_conv.cpp:127-272):
+ * 0 none, 1 ReLU, 3 "ReLU6" that zeroes values above 6, 4 sigmoid, 5 mish. */
+
+typedef struct exhip_conv_desc {
+    int n, c, h, w;             /* logical input shape */
+    int k;                      /* output channels */
+    int kh, kw, sh, sw;         /* kernel and stride (dilation 1 only, as the reference's AVX paths) */
+    int pt, pb, pl, pr;         /* zero padding top/bottom/left/right */
+    int act;                    /* fused activation applied to conv + bias */
+    int c_stride;               /* channel stride of the NHWC input, in elements */
+    int k_stride;               /* channel stride of the NHWC outputs, in elements (>= k) */
+    int post_relu;              /* ReLU applied after the residual add (0/1) */
+    float fs_out;               /* scale of the optional int8 output: q = sat8(trunc(v*fs_out +- 0.5)) */
+} exhip_conv_desc;
+
+/* Output spatial size, (H + pt + pb - kh)/sh + 1 (src/Excalibur/operation_convolution.cpp:270-271). */
+int exhip_conv_out_hw(const exhip_conv_desc* d, int* oh, int* ow);
+
+/* Weight pre-packing, the counterpart of the reference's load-time weight transforms
+ * (conv3x3s1_winograd23_tr_kernel*, forward_im2col*_tr_kernel, src/Excalibur/operation_convolution.cpp:90-97,136-143).
+ * Runs on the host: w is OIHW (int8 / IEEE half bits / float per dtype), `packed` a host buffer of
+ * exhip_conv_packed_bytes() bytes that the caller then uploads. */
+size_t exhip_conv_packed_bytes(const exhip_conv_desc* d, int dtype);
+int exhip_conv_pack_weights(const exhip_conv_desc* d, int dtype, const void* w_oihw, void* packed);
+
+/* operation_convolution::forward_cpu_i8 after quantization (src/Excalibur/operation_convolution.cpp:373-408):
+ * acc = int8 x int8 -> int32 convolution; v = fmaf((float)acc, scale[k], bias[k]) (bias NULL = 0);
+ * v = act(v); if residual: v += residual[n,oh,ow,k] (NHWC f32, stride k_stride); if post_relu: v = max(0, v).
+ * Any non-NULL output is written: y_i8 NHWC (requantized with fs_out, pad channels zeroed),
+ * y_f32_nhwc, y_f32_nchw (the reference's boundary layout), acc_nchw (raw int32 accumulators).
+ * `scale` is the per-output-channel dequantization scale the host computes exactly as the reference,
+ * fabs(ws) <= 1e-6 ? 0 : 1.0f/(ws*fs) (:400-403). */
+int exhip_conv2d_i8(exhip_ctx* ctx, const exhip_conv_desc* d, const int8_t* x_nhwc, const void* w_packed,
+                    const float* scale, const float* bias, const float* residual_nhwc, int8_t* y_i8_nhwc,
+                    float* y_f32_nhwc, float* y_f32_nchw, int32_t* acc_nchw);
+
+/* operation_convolution::forward_cpu_f32 (src/Excalibur/operation_convolution.cpp:251-329) with fp16
+ * storage and f32 accumulation (include/Excalibur/operation.hpp:234-260 describes the fp16 layer):
+ * x NHWC f16; outputs NHWC f16 and/or NCHW f16 and/or NCHW f32; residual NHWC f16. */
+int exhip_conv2d_f16(exhip_ctx* ctx, const exhip_conv_desc* d, const uint16_t* x_nhwc, const void* w_packed,
+                     const float* bias, const uint16_t* residual_nhwc, uint16_t* y_f16_nhwc, uint16_t* y_f16_nchw,
+                     float* y_f32_nchw);
+
+/* operation_convolution::forward_cpu_f32 in fp32 (f32 MFMA): x NHWC f32; outputs NHWC and/or NCHW f32. */
+int exhip_conv2d_f32(exhip_ctx* ctx, const exhip_conv_desc* d, const float* x_nhwc, const void* w_packed,
+                     const float* bias, const float* residual_nhwc, float* y_f32_nhwc, float* y_f32_nchw);
+
+/* Any geometry incl. groups, straight from the definition on NCHW f32 (slow; used for shapes the
+ * MFMA path does not take). int8 mode when w_i8 != NULL: quantizes x with fs on the fly and applies
+ * fmaf(acc, scale[k], bias[k]); otherwise f32 weights. */
+int exhip_conv2d_direct_nchw(exhip_ctx* ctx, const exhip_conv_desc* d, int groups, const float* x, const float* w_f32,
+                             const int8_t* w_i8, float fs, const float* scale, const float* bias, float* y);
+
+/* ---- bandwidth-bound operators ---- */
+/* operation_convolutiondepthwise::forward_cpu_f32, 3x3 stride 1/2 (src/Excalibur/operation_convolutiondepthwise.cpp:321-626):
+ * per pixel three vertical fused multiply-adds per kernel column, then bias + col0 + col1 + col2; act fused.
+ * NCHW f32 (boundary layout) and NHWC f16 (between fp16 layers; f32 math, result rounded to half). */
+int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const float* w9, const float* bias, float* y, int n,
+                             int c, int h, int w, int stride, int pt, int pb, int pl, int pr, int act);
+int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const float* bias, uint16_t* y,
+                             int n, int c, int h, int w, int c_stride, int stride, int pt, int pb, int pl, int pr,
+                             int act);
+/* operation_convolutiondepthwise::dequantize_int8 (:195-222): wf = w_i8 * (ws <= 1e-6 ? 0 : 1/ws). */
+int exhip_dw_dequant_weights(exhip_ctx* ctx, const int8_t* w, const float* ws, float* wf, int k, int per_group);
+
+/* operation_pooling::forward_cpu_f32 (src/Excalibur/operation_pooling.cpp:80-208). type 0 max, 1 average.
+ * Output size is computed by the caller with exhip_pool_out_hw (pad_mode 0 ceil, 1 floor). */
+int exhip_pool_out_hw(int h, int w, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr, int pad_mode,
+                      int* oh, int* ow);
+int exhip_pool2d_nchw_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w, int oh, int ow,
+                          int type, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr,
+                          int count_include_pad);
+/* NHWC variants used between fused layers. The int8 one exists because max commutes with the
+ * (monotone) quantizer; the f32 one can also emit the requantized int8 copy (y_i8 may be NULL). */
+int exhip_maxpool2d_nhwc_f32(exhip_ctx* ctx, const float* x, float* y, int8_t* y_i8, float fs_out, int n, int c,
+                             int h, int w, int c_stride, int oh, int ow, int kh, int kw, int sh, int sw, int pt,
+                             int pl);
+int exhip_pool2d_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int c_stride,
+                          int oh, int ow, int type, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr,
+                          int count_include_pad);
+
+/* operation_eltwise::forward_cpu_f32 (src/Excalibur/operation_eltwise.cpp:43-94): type 0 PROD, 1 SUM
+ * (coeffs host array or NULL = ones), 2 MAX over n_inputs same-shape device arrays (inputs: host array
+ * of device pointers). SUM follows the reference's saxpby rounding (body unfused, last count%8 fused). */
+int exhip_eltwise_f32(exhip_ctx* ctx, const float* const* inputs, int n_inputs, const float* coeffs, int type,
+                      float* y, size_t count);
+/* operation_binaryop equal-shape ADD (src/Excalibur/operation_binaryop.cpp:75-84) with optional fused ReLU
+ * (operation_relu, src/Excalibur/operation_relu.cpp:31-81) and optional requantized NHWC/flat int8 copy. */
+int exhip_add_f32(exhip_ctx* ctx, const float* a, const float* b, float* y, size_t count, int relu);
+int exhip_relu_f32(exhip_ctx* ctx, const float* x, float* y, size_t count);
+int exhip_add_f16(exhip_ctx* ctx, const uint16_t* a, const uint16_t* b, uint16_t* y, size_t count, int relu);
+int exhip_relu_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, size_t count);
+
+/* operation_innerproduct::forward_cpu_f32 (src/Excalibur/operation_innerproduct.cpp:176-224):
+ * y[m,n] = sum_k x[m,k]*w[n,k] + bias[n]; x [m][k_in], w [n_out][k_in] row-major f32. */
+int exhip_innerproduct_f32(exhip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, int m,
+                           int n_out, int k_in);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EXHIP_H_ */

@@ -98,6 +98,18 @@ def dequant_scales(ws, fs, k):
     return np.array([dequant_scale(ws[i], fs[i]) for i in range(k)], np.float32)
 
 
+def dequant(acc, ws, fs, bias):
+    """fmaf((float)acc, scale_k, bias_k) over an NCHW int32 accumulator tensor."""
+    acc = np.ascontiguousarray(acc, np.int32)
+    n, k, h, w = acc.shape
+    ws = _f32(np.atleast_1d(ws))
+    fs = _f32(np.atleast_1d(fs))
+    bias = _f32(bias)
+    y = np.empty(acc.shape, np.float32)
+    lib().exo_dequant_i32_f32(_p(acc), _p(y), n, k, h * w, _p(ws), ws.size, _p(fs), fs.size, _p(bias))
+    return y
+
+
 def conv2d_i8(x, w, bias, ws, fs, act, g, want_acc=False):
     x = _f32(x)
     w = np.ascontiguousarray(w, np.int8)

@@ -1,0 +1,282 @@
+"""GPU parity tests: every operator of the hot path through the exhip C ABI against
+(1) the golden fixtures written by the compiled reference, (2) the CPU restatement on larger seeded
+shapes, (3) size-independent properties at the BASELINE sizes.
+
+Bars: int32 accumulators, dequantized outputs of the int8 path, requantized int8 outputs, depthwise,
+pooling and elementwise results bit-exact (== on floats, so +0.0 equals -0.0); fp32 convolution and
+inner product within 1e-4 and fp16 within 2e-3 under the reference's check_value rule
+(|a-b| <= max(t, t*max(|a|,|b|)), src/Julius/julius_test.cpp:12-39).
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from oracle import port
+from tests import cases, gpueval
+from tests.golden.make_fixtures import load_case
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")))
+TOLERANT = ("conv_f32", "fc_")
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    from excalibur_amd import hip
+    c = hip.Ctx(0)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("name", [n for n in NAMES if not n.startswith("f16_")])
+def test_golden_fixture(ctx, name):
+    case, expected = load_case(os.path.join(GOLDEN, name + ".npz"))
+    got = gpueval.gpu_eval(ctx, case)
+    assert got.shape == expected.shape
+    if name.startswith(TOLERANT):
+        assert cases.check_value(got, expected, 1e-4) == 0
+    else:
+        assert np.array_equal(got, expected)
+
+
+@pytest.mark.parametrize("name", ["f16_conv_3x3s1", "f16_conv_tail75"])
+def test_golden_fixture_fp16_conv(ctx, name):
+    case, expected = load_case(os.path.join(GOLDEN, name + ".npz"))
+    got = gpueval.conv_f16(ctx, case, case["x"])
+    assert cases.check_value(got.view(np.float16).astype(np.float32), expected.view(np.float16).astype(np.float32), 2e-3) == 0
+
+
+I8_SHAPES = [
+    # seed, n, c, h, w, k, kernel, stride, pad
+    (200, 2, 128, 80, 80, 128, 3, 1, 1),    # cfg2 3x3 (two of the eight images)
+    (201, 2, 128, 80, 80, 256, 1, 1, 0),    # cfg2 1x1
+    (202, 1, 64, 160, 160, 64, 3, 1, 1),    # ResNet-18 stage 1
+    (203, 2, 64, 160, 160, 128, 3, 2, 1),   # stage 2 entry, stride 2
+    (204, 2, 64, 160, 160, 128, 1, 2, 0),   # 1x1 stride-2 downsample
+    (205, 1, 3, 256, 256, 64, 7, 2, 3),     # stem shape (packed first-layer form)
+    (206, 3, 512, 20, 20, 512, 3, 1, 1),    # stage 4: patch wider than the image rows
+    (207, 2, 48, 33, 31, 72, 3, 1, 1),      # channels not a multiple of 32, odd sizes
+    (208, 1, 128, 40, 40, 255, 1, 1, 0),    # YOLO head: K = 255
+    (209, 2, 32, 17, 17, 40, 5, 1, 2),      # 5x5
+    (210, 1, 16, 30, 30, 24, 7, 2, 3),      # 7x7 with 16 channels (generic form)
+    (211, 2, 96, 24, 24, 160, 3, 2, (0, 1, 0, 1)),  # asymmetric padding
+]
+
+
+@pytest.mark.parametrize("args", I8_SHAPES, ids=[f"s{a[0]}" for a in I8_SHAPES])
+def test_conv_i8_acc_and_output_bit_exact(ctx, args):
+    case = cases.conv_i8_case(*args)
+    g = cases.geom_of(case)
+    want_y, want_acc = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], case["act"], g, want_acc=True)
+    got = gpueval.conv_i8(ctx, case)
+    # quantized input in NHWC equals the reference's quantizer
+    q = port.quantize(case["x"], case["fs"])
+    assert np.array_equal(got["xq"][..., :case["c"]], q.transpose(0, 2, 3, 1))
+    assert not got["xq"][..., case["c"]:].any()
+    assert np.array_equal(got["acc"], want_acc)
+    assert np.array_equal(got["nchw"], want_y)
+
+
+def test_conv_i8_fused_residual_relu_requant(ctx):
+    """conv(act 0) -> + shortcut -> ReLU -> next layer's quantizer, in one epilogue."""
+    case = cases.conv_i8_case(220, 2, 64, 40, 40, 64, 3, 1, 1, act=0)
+    r = np.random.default_rng(221)
+    res_nchw = r.uniform(-4, 4, (2, 64, 40, 40)).astype(np.float32)
+    fs_out = np.float32(17.3)
+    y = cases.oracle_eval(case)
+    z = port.relu(port.binaryop_add(y, res_nchw))
+    want_q = port.quantize(z, fs_out)
+    got = gpueval.conv_i8(ctx, case, fs_out=fs_out, residual=np.ascontiguousarray(res_nchw.transpose(0, 2, 3, 1)),
+                          post_relu=1, want=("nchw", "nhwc"))
+    assert np.array_equal(got["nchw"], z)
+    assert np.array_equal(got["nhwc"], z.transpose(0, 2, 3, 1))
+    assert np.array_equal(got["i8"], want_q.transpose(0, 2, 3, 1))
+
+
+def test_conv_i8_requant_pad_channels_are_zero(ctx):
+    case = cases.conv_i8_case(222, 1, 32, 12, 12, 40, 3, 1, 1)
+    fs_out = np.float32(9.0)
+    got = gpueval.conv_i8(ctx, case, fs_out=fs_out, want=("nchw",))
+    want_q = port.quantize(cases.oracle_eval(case), fs_out).transpose(0, 2, 3, 1)
+    assert got["i8"].shape[-1] == 64
+    assert np.array_equal(got["i8"][..., :40], want_q)
+    assert not got["i8"][..., 40:].any()
+
+
+F32_SHAPES = [
+    (230, 1, 64, 56, 56, 64, 3, 1, 1),      # cfg1
+    (231, 1, 64, 56, 56, 128, 3, 1, 1),
+    (232, 2, 24, 31, 29, 40, 3, 2, 1),
+    (233, 1, 3, 64, 64, 32, 7, 2, 3),
+    (234, 2, 128, 14, 14, 256, 1, 1, 0),
+]
+
+
+@pytest.mark.parametrize("args", F32_SHAPES, ids=[f"s{a[0]}" for a in F32_SHAPES])
+def test_conv_f32_within_1e4(ctx, args):
+    case = cases.conv_f32_case(*args)
+    assert cases.check_value(gpueval.conv_f32(ctx, case), cases.oracle_eval(case), 1e-4) == 0
+
+
+F16_SHAPES = [
+    (240, 2, 32, 56, 56, 64, 1, 1, 0),      # MobileNet pointwise
+    (241, 1, 3, 112, 112, 32, 3, 2, 1),     # MobileNet stem (packed first-layer form)
+    (242, 2, 64, 28, 28, 128, 3, 1, 1),
+    (243, 1, 128, 40, 40, 255, 1, 1, 0),
+]
+
+
+@pytest.mark.parametrize("args", F16_SHAPES, ids=[f"s{a[0]}" for a in F16_SHAPES])
+def test_conv_f16_within_2e3(ctx, args):
+    case = cases.conv_f32_case(*args)
+    x16 = case["x"].astype(np.float16).view(np.uint16)
+    want = port.float2half(cases.oracle_eval(dict(case, x=port.half2float(x16))))
+    got = gpueval.conv_f16(ctx, case, x16)
+    assert cases.check_value(got.view(np.float16).astype(np.float32), want.view(np.float16).astype(np.float32), 2e-3) == 0
+
+
+@pytest.mark.parametrize("groups", [2, 4])
+def test_grouped_conv_definition_kernel(ctx, groups):
+    case = cases.conv_f32_case(250 + groups, 2, 16, 13, 13, 24 if groups == 2 else 16, 3, 1, 1, groups=groups)
+    assert cases.check_value(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case), 1e-4) == 0
+    ci = cases.conv_i8_case(260 + groups, 1, 16, 12, 12, 16, 3, 2, 1, groups=groups)
+    assert np.array_equal(gpueval.gpu_eval(ctx, ci), cases.oracle_eval(ci))
+
+
+@pytest.mark.parametrize("stride,h,w", [(1, 56, 56), (2, 57, 55), (1, 7, 9), (2, 112, 112)])
+def test_depthwise_bit_exact(ctx, stride, h, w):
+    case = cases.conv_f32_case(270 + h, 2, 32, h, w, 32, 3, stride, 1, groups=32, dw=True)
+    assert np.array_equal(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case))
+    ci = cases.dw_i8_case(280 + h, 1, 16, h, w, stride)
+    assert np.array_equal(gpueval.gpu_eval(ctx, ci), cases.oracle_eval(ci))
+
+
+def test_depthwise_nhwc_f16(ctx):
+    from excalibur_amd import hip
+    case = cases.conv_f32_case(290, 2, 40, 28, 30, 40, 3, 2, 1, groups=40, dw=True)
+    x16 = case["x"].astype(np.float16).view(np.uint16)
+    want = port.float2half(cases.oracle_eval(dict(case, x=port.half2float(x16))))
+    x = ctx.nchw_to_nhwc(ctx.array(x16), hip.pad_to(40, 16), "f16")
+    y = ctx.dwconv3x3_nhwc_f16(x, 40, ctx.array(case["wt"]), ctx.array(case["bias"]), 2, 1, case["act"])
+    got = ctx.nhwc_to_nchw(y, 40, "f16").download()
+    assert cases.check_value(got.view(np.float16).astype(np.float32), want.view(np.float16).astype(np.float32), 2e-3) == 0
+
+
+POOLS = [
+    dict(ptype=0, kernel=3, stride=2, pad=1), dict(ptype=0, kernel=5, stride=1, pad=2),
+    dict(ptype=0, kernel=9, stride=1, pad=4), dict(ptype=0, kernel=13, stride=1, pad=6),
+    dict(ptype=1, kernel=2, stride=2, pad=0), dict(ptype=1, kernel=2, stride=2, pad=(0, 1, 0, 1)),
+    dict(ptype=1, kernel=3, stride=2, pad=1, pad_mode=0), dict(ptype=1, kernel=3, stride=2, pad=1, count_include_pad=1),
+    dict(ptype=1, global_pool=True), dict(ptype=0, global_pool=True),
+]
+
+
+@pytest.mark.parametrize("kw", POOLS, ids=[str(i) for i in range(len(POOLS))])
+def test_pool_bit_exact(ctx, kw):
+    case = cases.pool_case(300, 2, 6, 41, 38, **kw)
+    assert np.array_equal(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case))
+
+
+def test_maxpool_nhwc_with_requant_commutes(ctx):
+    """NHWC f32 max pooling that also emits the next layer's int8 input: max commutes with the quantizer."""
+    r = np.random.default_rng(310)
+    x = r.uniform(-3, 3, (2, 64, 30, 34)).astype(np.float32)
+    fs = np.float32(40.0)
+    want = port.pool2d(x, port.POOL_MAX, 3, 2, 1)
+    xd = ctx.nchw_to_nhwc(ctx.array(x), 64, "f32")
+    y, yq = ctx.maxpool2d_nhwc_f32(xd, 64, 3, 2, 1, fs_out=fs)
+    assert np.array_equal(y.download(), want.transpose(0, 2, 3, 1))
+    assert np.array_equal(yq.download(), port.quantize(want, fs).transpose(0, 2, 3, 1))
+
+
+def test_pool_nhwc_f16(ctx):
+    r = np.random.default_rng(311)
+    x16 = r.uniform(-3, 3, (2, 24, 14, 14)).astype(np.float16)
+    xd = ctx.nchw_to_nhwc(ctx.array(x16.view(np.uint16)), 24, "f16")
+    got = ctx.nhwc_to_nchw(ctx.pool2d_nhwc_f16(xd, 24, 1, global_pool=True), 24, "f32").download()
+    want = port.pool2d(x16.astype(np.float32), port.POOL_AVE, global_pool=True)
+    assert cases.check_value(got, want, 2e-3) == 0
+    got = ctx.nhwc_to_nchw(ctx.pool2d_nhwc_f16(xd, 24, 0, 3, 2, 1), 24, "f32").download()
+    assert np.array_equal(got, port.pool2d(x16.astype(np.float32), port.POOL_MAX, 3, 2, 1))
+
+
+@pytest.mark.parametrize("etype,n,coeffs", [(1, 2, None), (1, 3, [0.5, -1.25, 2.0]), (2, 3, None), (0, 3, None)])
+def test_eltwise_bit_exact(ctx, etype, n, coeffs):
+    case = cases.eltwise_case(320 + etype, (2, 16, 21, 23), etype, n, coeffs)
+    assert np.array_equal(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case))
+
+
+def test_add_relu_and_empty_and_ragged(ctx):
+    from excalibur_amd import hip
+    for shape in [(1, 1, 1, 1), (1, 3, 5, 7), (2, 64, 40, 40)]:
+        case = cases.binaryop_case(330, shape)
+        a, b = (ctx.array(v) for v in case["xs"])
+        assert np.array_equal(ctx.add_f32(a, b).download(), port.binaryop_add(*case["xs"]))
+        assert np.array_equal(ctx.add_f32(a, b, relu=True).download(), port.relu(port.binaryop_add(*case["xs"])))
+        assert np.array_equal(ctx.relu_f32(a).download(), port.relu(case["xs"][0]))
+    # empty tensors are a no-op, not an error
+    e = ctx.empty((0,), np.float32)
+    assert hip.lib().exhip_add_f32(ctx.h, e.ptr, e.ptr, e.ptr, 0, 0) == 0
+
+
+def test_innerproduct_within_1e4(ctx):
+    for args in [(340, 4, 512, 1, 1, 1000), (341, 32, 64, 7, 7, 100), (342, 3, 5, 3, 3, 7)]:
+        case = cases.fc_case(*args)
+        assert cases.check_value(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case), 1e-4) == 0
+
+
+def test_error_paths_return_codes_not_crashes(ctx):
+    from excalibur_amd import hip
+    d = ctx.conv_desc(1, 20, 8, 8, 8, 3, 1, 1, c_stride=20)  # 20-byte pixels: not a multiple of 32
+    assert hip.lib().exhip_conv_packed_bytes(__import__("ctypes").byref(d), hip.I8) == 0
+    assert b"multiple of 32" in hip.lib().exhip_last_error()
+    with pytest.raises(hip.ExhipError):
+        ctx.eltwise_f32([ctx.array(np.zeros(4, np.float32))], 1)  # fewer than two inputs
+    assert hip.lib().exhip_pool2d_nchw_f32(ctx.h, None, None, 1, 1, 4, 4, 2, 2, 0, 2, 2, 2, 2, 0, 0, 0, 0, 0) == 10001
+
+
+def _sampled_acc(case, q_nchw, samples, rng):
+    """Brute-force int32 accumulators at random output positions (numpy, a few thousand dot products)."""
+    n, c, h, w = q_nchw.shape
+    k, kh, kw, s = case["k"], case["kh"], case["kw"], case["stride"]
+    pt, pb, pl, pr = (case["pad"],) * 4 if np.isscalar(case["pad"]) else case["pad"]
+    oh, ow = (h + pt + pb - kh) // s + 1, (w + pl + pr - kw) // s + 1
+    qp = np.zeros((n, c, h + pt + pb, w + pl + pr), np.int32)
+    qp[:, :, pt:pt + h, pl:pl + w] = q_nchw
+    wt = case["wt"].astype(np.int32)
+    idx = [(rng.integers(n), rng.integers(k), rng.integers(oh), rng.integers(ow)) for _ in range(samples)]
+    idx += [(0, 0, 0, 0), (n - 1, k - 1, oh - 1, ow - 1), (n - 1, 0, 0, ow - 1), (0, k - 1, oh - 1, 0)]
+    vals = [int((qp[a, :, y * s:y * s + kh, x * s:x * s + kw] * wt[b]).sum()) for a, b, y, x in idx]
+    return idx, vals
+
+
+FULL = [
+    ("cfg2_3x3", (400, 8, 128, 80, 80, 128, 3, 1, 1)),
+    ("cfg2_1x1_k256", (401, 8, 128, 80, 80, 256, 1, 1, 0)),
+    ("resnet_stage1_n8", (402, 8, 64, 160, 160, 64, 3, 1, 1)),
+    ("resnet_stem_n4", (403, 4, 3, 640, 640, 64, 7, 2, 3)),
+]
+
+
+@pytest.mark.parametrize("name,args", FULL, ids=[f[0] for f in FULL])
+def test_full_size_sampled_and_linear(ctx, name, args):
+    """At BASELINE sizes: (a) sampled accumulators against brute force, (b) linearity in the weights:
+    acc(w1) + acc(w2) == acc(w1 + w2), (c) the dequantized output recomputed from the GPU's own
+    accumulators with the closed form fmaf(acc, s, b) + ReLU."""
+    case = cases.conv_i8_case(*args, integer_x=True)
+    rng = np.random.default_rng(args[0])
+    got = gpueval.conv_i8(ctx, case)
+    q = case["x"].astype(np.int32)
+    idx, vals = _sampled_acc(case, q, 1500, rng)
+    assert [int(got["acc"][i]) for i in idx] == vals
+    w1 = (case["wt"].astype(np.int32) // 2).astype(np.int8)
+    w2 = (case["wt"].astype(np.int32) - w1).astype(np.int8)
+    a1 = gpueval.conv_i8(ctx, dict(case, wt=w1), want=("acc",))["acc"]
+    a2 = gpueval.conv_i8(ctx, dict(case, wt=w2), want=("acc",))["acc"]
+    assert np.array_equal(a1 + a2, got["acc"])
+    want = port.dequant(got["acc"], case["ws"], case["fs"], case["bias"])
+    assert np.array_equal(got["nchw"], port.relu(want))
