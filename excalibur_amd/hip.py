@@ -95,6 +95,11 @@ class Event:
     def record(self, ctx):
         _check(lib().exhip_event_record(ctx.h, self.h))
 
+    def destroy(self):
+        if self.h:
+            _check(lib().exhip_event_destroy(self.h))
+            self.h = None
+
     def elapsed_ms(self, stop):
         ms = ctypes.c_float()
         _check(lib().exhip_event_elapsed_ms(self.h, stop.h, ctypes.byref(ms)))

@@ -1,0 +1,27 @@
+"""The ResNet-18-shaped int8 network description: the oracle chain against the compiled reference running the
+generated .phai/.racy through its own loader (marker `ref`), plus closed-form checks of the builder."""
+import numpy as np
+import pytest
+
+from excalibur_amd.resnet18 import ResNet18Int8
+from tests import netref
+
+
+def test_algorithmic_work_matches_the_survey_figure():
+    net = ResNet18Int8(seed=3, calib_hw=32)
+    # 14.80 GMAC per 640x640 image: stem 0.963 + stage1 4x0.944 + three stages of (0.472 + 0.052 + 3x0.944)
+    assert abs(net.gmac_per_image(640, 640) - 14.805) < 0.01
+    assert len(net.convs) == 20 and len(net.blocks) == 8
+    assert all(c.fs > 0 for c in net.convs)
+
+
+@pytest.mark.ref
+def test_oracle_chain_equals_compiled_reference():
+    net = ResNet18Int8(seed=5, calib_hw=32)
+    x = np.random.default_rng(6).uniform(-1, 1, (2, 3, 64, 64)).astype(np.float32)
+    want, blobs = netref.oracle_forward(net, x)
+    got = netref.reference_forward(net, x, extra=["pool1", "l2b1_out"])
+    assert np.array_equal(got["pool1"], blobs["pool1"])
+    assert np.array_equal(got["l2b1_out"], blobs["l2b1_out"])
+    assert np.array_equal(got[net.output], want)
+    assert want.shape == (2, 512, 2, 2) and np.count_nonzero(want) > want.size // 4
