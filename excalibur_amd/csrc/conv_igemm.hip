@@ -33,10 +33,10 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kMaxActVec = 10;   // 16-byte activation vectors staged per thread and channel chunk
-constexpr int kMaxWVec = 6;      // 16-byte weight vectors staged per thread and stage
-constexpr int kMaxPackedPix = 8; // pixels staged per thread in packed-row form
+constexpr int kMaxActVec = 10;   // 16-byte activation vectors staged per thread and channel chunk (256-thread groups)
+constexpr int kMaxWVec = 9;      // 16-byte weight vectors staged per thread and stage (256-thread groups)
+constexpr int kMaxPackedPix = 8; // pixels staged per thread in packed-row form (256-thread groups)
+constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format: out-of-range reads return 0
 
 struct ConvParams {
     const char* x;
@@ -58,13 +58,16 @@ struct ConvParams {
     int kstride;              // output channel stride (elements)
     int PH, PW, IH, IW;       // output patch and staged tile size in pixels
     int lds_pix_b, lds_row_b; // LDS bytes per tile pixel / row
-    int lds_act_b;            // LDS bytes of the activation tile (weights follow)
+    int lds_act_b;            // LDS bytes of one activation tile buffer
+    int lds_w_b;              // LDS bytes of one weight stage buffer
+    int act_bufs, w_bufs;     // 1, or 2 when consecutive chunks / stages alternate buffers
     int n_chunks, chunk_b;
     int RS, n_rg;             // filter rows per stage, stages per chunk
     int tiles_x, tiles_y, ktiles;
     int act, post_relu;
     float fs_out;
     int b_align;              // alignment of B fragment reads in packed-row form (4, 8 or 16)
+    unsigned img_bytes;       // bytes of one input image (buffer range for the bounds-checked loads)
 };
 
 template <int DT> struct Acc { typedef v16i type; };
@@ -98,14 +101,28 @@ __device__ __forceinline__ v4i lds_read16_unaligned(const char* p, int align) {
     return r;
 }
 
+// sigmoid / mish evaluate double-precision transcendentals: kept out of line so the common epilogue stays small
+__device__ __noinline__ float slow_activation(float v, int act) { return exhip_act(v, act); }
+
+__device__ __forceinline__ float fast_activation(float v, int act) {
+    if (act == 1) return (0.f > v) ? 0.f : v;
+    if (act == 3) { const float d = (0.f > v) ? 0.f : v; return d <= 6.f ? d : 0.f; }
+    return v;
+}
+
 template <int DT, int MT, int NT, int WM, int WN, bool PACKED>
-__global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p) {
-    static_assert(WM * WN == 4, "four waves per workgroup");
+__global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvParams p) {
+    constexpr int THREADS = 64 * WM * WN;
     constexpr int TM = 32 * MT * WM;
+    // staging limits scale with the group size so that a 512-thread group needs half the registers
+    constexpr int NAV = PACKED ? 1 : kMaxActVec * 256 / THREADS;
+    constexpr int NPP = PACKED ? kMaxPackedPix * 256 / THREADS : 1;
+    constexpr int NWV = kMaxWVec * 256 / THREADS;
     typedef typename Acc<DT>::type acc_t;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    char* lds_a = smem;
-    char* lds_w = smem + p.lds_act_b;
+    // [activation buffers][weight buffers]
+    char* const lds_a0 = smem;
+    char* const lds_w0 = smem + p.act_bufs * p.lds_act_b;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
@@ -125,40 +142,40 @@ __global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p
     const int n = t / p.tiles_y;
     const int oy0 = ty * p.PH, ox0 = tx * p.PW;
     const int iy0 = oy0 * p.S * p.tile_step - p.PT, ix0 = ox0 * p.S * p.tile_step - p.PL;
-    const char* ximg = p.x + (size_t)n * p.H * p.W * p.cstride_b;
+
+    // Bounds-checked buffer views: any offset at or past the range reads as zero, which is how halo
+    // pixels outside the image and threads beyond the staged vector count are handled without branches.
+    // The range check covers the per-lane offset only, so chunk and stage offsets go into the view's base.
+    const char* const ximg = p.x + (size_t)n * p.img_bytes;
 
     // ---- staging plan (same for every chunk) ----
-    int a_goff[PACKED ? kMaxPackedPix : kMaxActVec];
-    int a_loff[PACKED ? kMaxPackedPix : kMaxActVec];
+    int a_goff[PACKED ? NPP : NAV];
+    int a_loff[PACKED ? NPP : NAV];
     if constexpr (!PACKED) {
         const int vp = p.chunk_b >> 4;
         const int nvec = p.IH * p.IW * vp;
 #pragma unroll
-        for (int i = 0; i < kMaxActVec; ++i) {
-            const int v = tid + kThreads * i;
-            a_goff[i] = -1;
-            a_loff[i] = -1;
-            if (v < nvec) {
-                const int pix = v / vp, part = v - pix * vp;
-                const int iy = pix / p.IW, ix = pix - iy * p.IW;
-                const int gy = iy0 + iy * p.tile_step, gx = ix0 + ix * p.tile_step;
-                a_loff[i] = iy * p.lds_row_b + ix * p.lds_pix_b + part * 16;
-                if (gy >= 0 && gy < p.H && gx >= 0 && gx < p.W) a_goff[i] = (gy * p.W + gx) * p.cstride_b + part * 16;
-            }
+        for (int i = 0; i < NAV; ++i) {
+            const int v = tid + THREADS * i;
+            const int pix = v / vp, part = v - pix * vp;
+            const int iy = pix / p.IW, ix = pix - iy * p.IW;
+            const int gy = iy0 + iy * p.tile_step, gx = ix0 + ix * p.tile_step;
+            const bool in_tile = v < nvec;
+            const bool in_img = in_tile && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
+            a_loff[i] = in_tile ? iy * p.lds_row_b + ix * p.lds_pix_b + part * 16 : -1;
+            a_goff[i] = in_img ? (gy * p.W + gx) * p.cstride_b + part * 16 : (int)p.img_bytes;
         }
     } else {
         const int npix = p.IH * p.IW;
 #pragma unroll
-        for (int i = 0; i < kMaxPackedPix; ++i) {
-            const int v = tid + kThreads * i;
-            a_goff[i] = -1;
-            a_loff[i] = -1;
-            if (v < npix) {
-                const int iy = v / p.IW, ix = v - iy * p.IW;
-                const int gy = iy0 + iy, gx = ix0 + ix;
-                a_loff[i] = iy * p.lds_row_b + ix * p.lds_pix_b;
-                if (gy >= 0 && gy < p.H && gx >= 0 && gx < p.W) a_goff[i] = (gy * p.W + gx) * p.cstride_b;
-            }
+        for (int i = 0; i < NPP; ++i) {
+            const int v = tid + THREADS * i;
+            const int iy = v / p.IW, ix = v - iy * p.IW;
+            const int gy = iy0 + iy, gx = ix0 + ix;
+            const bool in_tile = v < npix;
+            const bool in_img = in_tile && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
+            a_loff[i] = in_tile ? iy * p.lds_row_b + ix * p.lds_pix_b : -1;
+            a_goff[i] = in_img ? (gy * p.W + gx) * p.cstride_b : (int)p.img_bytes;
         }
     }
 
@@ -189,69 +206,61 @@ __global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p
 
     const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;  // packed weight bytes of one filter row
     const int n_stages = p.n_chunks * p.n_rg;
-    const char* wkt = p.wp + (size_t)kt * p.n_chunks * p.KH * row_w_b;
+    const char* const wkt = p.wp + (size_t)kt * p.n_chunks * p.KH * row_w_b;
 
-    v4i a_reg[PACKED ? 1 : kMaxActVec];
-    v2i a_reg_p[PACKED ? kMaxPackedPix : 1];
-    v4i w_reg[kMaxWVec];
+    v4i a_reg[NAV];
+    int a_reg_p[NPP][2];
+    v4i w_reg[NWV];
 
     auto load_act = [&](int cc) {
+        const int soff = PACKED ? 0 : cc * p.chunk_b;
+        const __amdgpu_buffer_rsrc_t xr =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ximg + soff), 0, (int)(p.img_bytes - soff), kRsrcWord3);
         if constexpr (!PACKED) {
 #pragma unroll
-            for (int i = 0; i < kMaxActVec; ++i) {
-                v4i v = {0, 0, 0, 0};
-                if (a_goff[i] >= 0) v = *reinterpret_cast<const v4i*>(ximg + a_goff[i] + cc * p.chunk_b);
-                a_reg[i] = v;
-            }
+            for (int i = 0; i < NAV; ++i) a_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, a_goff[i], 0, 0);
         } else {
 #pragma unroll
-            for (int i = 0; i < kMaxPackedPix; ++i) {
-                v2i v = {0, 0};
-                if (a_goff[i] >= 0) {
-                    if (p.cstride_b == 4) v[0] = *reinterpret_cast<const int*>(ximg + a_goff[i]);
-                    else v = *reinterpret_cast<const v2i*>(ximg + a_goff[i]);
-                }
-                a_reg_p[i] = v;
+            for (int i = 0; i < NPP; ++i) {
+                a_reg_p[i][0] = __builtin_amdgcn_raw_buffer_load_b32(xr, a_goff[i], 0, 0);
+                a_reg_p[i][1] = p.cstride_b == 8 ? __builtin_amdgcn_raw_buffer_load_b32(xr, a_goff[i] + 4, 0, 0) : 0;
             }
         }
     };
-    auto store_act = [&]() {
+    auto store_act = [&](char* dst) {
         if constexpr (!PACKED) {
 #pragma unroll
-            for (int i = 0; i < kMaxActVec; ++i)
-                if (a_loff[i] >= 0) *reinterpret_cast<v4i*>(lds_a + a_loff[i]) = a_reg[i];
+            for (int i = 0; i < NAV; ++i)
+                if (a_loff[i] >= 0) *reinterpret_cast<v4i*>(dst + a_loff[i]) = a_reg[i];
         } else {
 #pragma unroll
-            for (int i = 0; i < kMaxPackedPix; ++i)
+            for (int i = 0; i < NPP; ++i)
                 if (a_loff[i] >= 0) {
-                    if (p.cstride_b == 4) *reinterpret_cast<int*>(lds_a + a_loff[i]) = a_reg_p[i][0];
-                    else *reinterpret_cast<v2i*>(lds_a + a_loff[i]) = a_reg_p[i];
+                    *reinterpret_cast<int*>(dst + a_loff[i]) = a_reg_p[i][0];
+                    if (p.cstride_b == 8) *reinterpret_cast<int*>(dst + a_loff[i] + 4) = a_reg_p[i][1];
                 }
         }
     };
     auto stage_rows = [&](int rg) { const int r0 = rg * p.RS; return (p.KH - r0 < p.RS ? p.KH - r0 : p.RS); };
     auto load_w = [&](int cc, int rg) {
-        const char* src = wkt + ((size_t)cc * p.KH + rg * p.RS) * row_w_b;
-        const int nvec = (stage_rows(rg) * row_w_b) >> 4;
+        // a view of exactly this stage's slice: lanes past its end read zeros
+        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<char*>(wkt + (size_t)(cc * p.KH + rg * p.RS) * row_w_b), 0, stage_rows(rg) * row_w_b, kRsrcWord3);
 #pragma unroll
-        for (int i = 0; i < kMaxWVec; ++i) {
-            const int v = tid + kThreads * i;
-            if (v < nvec) w_reg[i] = *reinterpret_cast<const v4i*>(src + (size_t)v * 16);
-        }
+        for (int i = 0; i < NWV; ++i) w_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (tid + THREADS * i) * 16, 0, 0);
     };
-    auto store_w = [&](int rg) {
-        const int nvec = (stage_rows(rg) * row_w_b) >> 4;
+    auto store_w = [&](char* dst) {
 #pragma unroll
-        for (int i = 0; i < kMaxWVec; ++i) {
-            const int v = tid + kThreads * i;
-            if (v < nvec) *reinterpret_cast<v4i*>(lds_w + v * 16) = w_reg[i];
+        for (int i = 0; i < NWV; ++i) {
+            const int v = (tid + THREADS * i) * 16;
+            if (v < p.lds_w_b) *reinterpret_cast<v4i*>(dst + v) = w_reg[i];
         }
     };
 
     load_act(0);
     load_w(0, 0);
-    store_act();
-    store_w(0);
+    store_act(lds_a0);
+    store_w(lds_w0);
     __syncthreads();
 
     for (int st = 0; st < n_stages; ++st) {
@@ -266,38 +275,59 @@ __global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p
                 load_w(cc, rg + 1);
             }
         }
-        // ---- MFMA over this stage ----
-        const int rows = stage_rows(rg);
-        const char* wl = lds_w + aoff;
-        for (int rr = 0; rr < rows; ++rr) {
-            const char* arow = lds_a + (rg * p.RS + rr) * p.lds_row_b;
-            for (int q = 0; q < p.KWe; ++q) {
-                const char* apix = arow + q * p.lds_pix_b;
-                for (int j = 0; j < p.KS; ++j) {
-                    v4i af[MT], bf[NT];
+        // ---- MFMA over this stage: k-steps in (row, tap, channel) order, fragments fetched one step ahead ----
+        const int nk = stage_rows(rg) * p.KWe * p.KS;
+        const char* wl = lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff;
+        const char* al = lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b;
+        int q = 0, j = 0;          // tap column and channel k-step of the fragments being fetched
+        int koff = 0;              // their byte offset inside the activation tile
+        v4i af[2][MT], bf[2][NT];
+        auto fetch = [&](int buf) {
 #pragma unroll
-                    for (int m = 0; m < MT; ++m) af[m] = lds_read16(wl + m * 1024);
+            for (int m = 0; m < MT; ++m) af[buf][m] = lds_read16(wl + m * 1024);
 #pragma unroll
-                    for (int nn = 0; nn < NT; ++nn) {
-                        if constexpr (PACKED) bf[nn] = lds_read16_unaligned(apix + boff[nn], p.b_align);
-                        else bf[nn] = lds_read16(apix + boff[nn] + j * 32);
-                    }
-#pragma unroll
-                    for (int m = 0; m < MT; ++m)
-#pragma unroll
-                        for (int nn = 0; nn < NT; ++nn) mma<DT>(acc[m][nn], af[m], bf[nn]);
-                    wl += (TM / 32) * 1024;
+            for (int nn = 0; nn < NT; ++nn) {
+                if constexpr (PACKED) bf[buf][nn] = lds_read16_unaligned(al + koff + boff[nn], p.b_align);
+                else bf[buf][nn] = lds_read16(al + koff + boff[nn]);
+            }
+            wl += (TM / 32) * 1024;
+            // advance (j, q, row) and the tile offset
+            if (++j == p.KS) {
+                j = 0;
+                koff += p.lds_pix_b - (p.KS - 1) * 32;
+                if (++q == p.KWe) {
+                    q = 0;
+                    koff += p.lds_row_b - p.KWe * p.lds_pix_b;
                 }
-            }
-        }
-        __syncthreads();
-        if (more) {
-            if (next_chunk) {
-                store_act();
-                store_w(0);
             } else {
-                store_w(rg + 1);
+                koff += 32;
             }
+        };
+        auto compute = [&](int buf) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int nn = 0; nn < NT; ++nn) mma<DT>(acc[m][nn], af[buf][m], bf[buf][nn]);
+        };
+        fetch(0);
+        int it = 0;
+        for (; it + 2 <= nk - 1; it += 2) {
+            fetch(1);
+            compute(0);
+            fetch(0);
+            compute(1);
+        }
+        // 1 or 2 k-steps left; buffer 0 holds step `it`
+        if (it + 1 < nk) {
+            fetch(1);
+            compute(0);
+            compute(1);
+        } else {
+            compute(0);
+        }
+        if (more) {
+            if (next_chunk) store_act(lds_a0 + ((cc + 1) & (p.act_bufs - 1)) * p.lds_act_b);
+            store_w(lds_w0 + ((st + 1) & (p.w_bufs - 1)) * p.lds_w_b);
         }
         __syncthreads();
     }
@@ -309,11 +339,25 @@ __global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p
         const int ch0 = kt * TM + (wm * MT + m) * 32 + (lane >> 5) * 16;
         if (ch0 >= p.kstride && ch0 >= p.K) continue;
         float sc[16], bi[16];
+        if (ch0 + 16 <= p.K) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const int ch = ch0 + e;
-            sc[e] = (DT == EXHIP_I8 && ch < p.K) ? p.scale[ch] : 0.f;
-            bi[e] = (p.bias && ch < p.K) ? p.bias[ch] : 0.f;
+            for (int e4 = 0; e4 < 4; ++e4) {
+                v4f s4 = {0.f, 0.f, 0.f, 0.f}, b4 = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (DT == EXHIP_I8) s4 = *reinterpret_cast<const v4f*>(p.scale + ch0 + e4 * 4);
+                if (p.bias) b4 = *reinterpret_cast<const v4f*>(p.bias + ch0 + e4 * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sc[e4 * 4 + e] = s4[e];
+                    bi[e4 * 4 + e] = b4[e];
+                }
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int ch = ch0 + e;
+                sc[e] = (DT == EXHIP_I8 && ch < p.K) ? p.scale[ch] : 0.f;
+                bi[e] = (p.bias && ch < p.K) ? p.bias[ch] : 0.f;
+            }
         }
 #pragma unroll
         for (int nn = 0; nn < NT; ++nn) {
@@ -333,9 +377,12 @@ __global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p
 #pragma unroll
                 for (int e = 0; e < 16; ++e) v[e] = acc[m][nn][e] + bi[e];
             }
-            if (p.act) {
+            if (p.act >= 4) {
+#pragma unroll 1
+                for (int e = 0; e < 16; ++e) v[e] = slow_activation(v[e], p.act);
+            } else if (p.act) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) v[e] = exhip_act(v[e], p.act);
+                for (int e = 0; e < 16; ++e) v[e] = fast_activation(v[e], p.act);
             }
             if (p.residual) {
                 if constexpr (DT == EXHIP_F16) {
@@ -428,14 +475,27 @@ __global__ __launch_bounds__(kThreads) void conv_igemm_kernel(const ConvParams p
 inline int esize_of(int dt) { return dt == EXHIP_I8 ? 1 : dt == EXHIP_F16 ? 2 : 4; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Tile variants: output channels x pixels per workgroup, and its wave grid. Every wave owns a 64 x 64
+// accumulator tile (MT = NT = 2): 128 bytes of LDS reads per MFMA-cycle per CU at full rate, within
+// what the LDS delivers, at 64 accumulator registers so that two waves fit per SIMD.
+struct Variant { int TM, TN, threads; };
+const Variant kVariants[] = {
+    {64, 256, 256},   // 0: waves 1 x 4
+    {128, 256, 512},  // 1: waves 2 x 4
+    {128, 128, 256},  // 2: waves 2 x 2
+};
+constexpr int kNumVariants = 3;
+
 struct Plan {
     bool packed;
-    int variant;  // 0: TM 64, TN 256 ; 1: TM 128, TN 256 ; 2: TM 128, TN 128
-    int TM, TN;
+    int variant;
+    int TM, TN, threads;
     int KWe, KS, chunk_b, n_chunks, RS, n_rg;
     int S, tile_step, PH, PW, IH, IW, lds_pix_b, lds_row_b, lds_act_b, lds_w_b, b_align;
+    int act_bufs, w_bufs;
     int tiles_x, tiles_y, ktiles;
     int OH, OW;
+    size_t lds_bytes() const { return (size_t)act_bufs * lds_act_b + (size_t)w_bufs * lds_w_b; }
 };
 
 int validate(const exhip_conv_desc* d, int dt) {
@@ -449,6 +509,7 @@ int validate(const exhip_conv_desc* d, int dt) {
     const int es = esize_of(dt), cb = d->c_stride * es;
     const bool packed_ok = (cb == 4 && dt == EXHIP_I8 && d->kw <= 8) || (cb == 8 && dt == EXHIP_F16 && d->kw <= 4);
     EXHIP_REQUIRE(cb % 32 == 0 || packed_ok, "conv: input pixel is %d bytes; need a multiple of 32 (or the packed first-layer form)", cb);
+    EXHIP_REQUIRE((long long)d->h * d->w * cb < (1ll << 31), "conv: one input image exceeds 2 GiB");
     return 0;
 }
 
@@ -463,17 +524,18 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
     const int es = esize_of(dt), cb = d->c_stride * es;
     const int OH = (d->h + d->pt + d->pb - d->kh) / d->sh + 1, OW = (d->w + d->pl + d->pr - d->kw) / d->sw + 1;
     const bool packed = cb < 32;
-    for (int vc = 0; vc < 6; ++vc) {
+    for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
         if (packed && chunk_opt == 64) continue;
         if (!packed && cb % chunk_opt != 0) continue;
-        const int TM = variant == 0 ? 64 : 128, TN = variant == 2 ? 128 : 256;
+        const int TM = kVariants[variant].TM, TN = kVariants[variant].TN;
         const int ktiles = ceil_div(d->k, TM);
         Plan p;
         p.packed = packed;
         p.variant = variant;
         p.TM = TM;
         p.TN = TN;
+        p.threads = kVariants[variant].threads;
         p.OH = OH;
         p.OW = OW;
         p.ktiles = ktiles;
@@ -488,11 +550,15 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
         p.tile_step = (d->kh == 1 && d->kw == 1) ? d->sh : 1;
         p.S = d->sh / p.tile_step;
         const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;
-        p.RS = (kMaxWVec * kThreads * 16) / row_w_b;
-        if (p.RS < 1) continue;  // one filter row does not fit the staging registers
+        // bytes one group's staging registers hold: whole 16-byte vectors per thread
+        const int w_budget = (kMaxWVec * 256 / p.threads) * p.threads * 16;
+        p.RS = w_budget / row_w_b;
+        if (p.RS < 1) continue;                  // one filter row does not fit
         if (p.RS > d->kh) p.RS = d->kh;
         p.n_rg = ceil_div(d->kh, p.RS);
         p.lds_w_b = p.RS * row_w_b;
+        p.act_bufs = p.n_chunks > 1 ? 2 : 1;
+        p.w_bufs = p.n_chunks * p.n_rg > 1 ? 2 : 1;
         for (int PW = 1; PW <= TN && PW <= OW; ++PW) {
             int PH = TN / PW;
             if (PH > OH) PH = OH;
@@ -507,16 +573,17 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
                 p.lds_row_b = (p.IW * cb + 15) / 16 * 16;
                 const int step = p.S * cb;
                 p.b_align = step % 16 == 0 ? 16 : step % 8 == 0 ? 8 : 4;
-                if (p.IH * p.IW > kMaxPackedPix * kThreads) continue;
+                if (p.IH * p.IW > kMaxPackedPix * 256) continue;
             } else {
                 p.IW = (PW - 1) * p.S + d->kw;
                 p.lds_pix_b = p.chunk_b + 16;
                 p.lds_row_b = p.IW * p.lds_pix_b;
                 p.b_align = 16;
-                if (p.IH * p.IW * (p.chunk_b / 16) > kMaxActVec * kThreads) continue;
+                if (p.IH * p.IW * (p.chunk_b / 16) > kMaxActVec * 256) continue;
             }
-            p.lds_act_b = (p.IH * p.lds_row_b + 63) / 64 * 64;
-            if (p.lds_act_b + p.lds_w_b > 150 * 1024) continue;
+            // the tile plus the 16 bytes a lane may read past its last row's last pixel
+            p.lds_act_b = (p.IH * p.lds_row_b + 16 + 63) / 64 * 64;
+            if (p.lds_bytes() > 156 * 1024) continue;
             p.tiles_y = ceil_div(OH, PH);
             p.tiles_x = ceil_div(OW, PW);
             const double useful = (double)OH * OW * d->k;
@@ -542,23 +609,25 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
     return 0;
 }
 
-template <int DT, bool PACKED>
-int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid, size_t lds) {
-    if (pl.variant == 0) {
-        auto k = conv_igemm_kernel<DT, 2, 2, 1, 4, PACKED>;
-        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), lds, ctx->stream, p);
-    } else if (pl.variant == 1) {
-        auto k = conv_igemm_kernel<DT, 4, 2, 1, 4, PACKED>;
-        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), lds, ctx->stream, p);
-    } else {
-        auto k = conv_igemm_kernel<DT, 2, 2, 2, 2, PACKED>;
-        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        hipLaunchKernelGGL(k, dim3(grid), dim3(kThreads), lds, ctx->stream, p);
+template <typename K>
+int launch_kernel(exhip_ctx* ctx, K kernel, bool* attr_set, const Plan& pl, const ConvParams& p, int grid) {
+    if (!*attr_set) {  // raise the dynamic LDS limit once per kernel
+        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        *attr_set = true;
     }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(pl.threads), pl.lds_bytes(), ctx->stream, p);
     EXHIP_LAUNCH_CHECK();
     return 0;
+}
+
+template <int DT, bool PACKED>
+int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
+    static bool attr[kNumVariants] = {false, false, false};
+    switch (pl.variant) {
+    case 0: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 1, 4, PACKED>, &attr[0], pl, p, grid);
+    case 1: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 4, PACKED>, &attr[1], pl, p, grid);
+    default: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 2, PACKED>, &attr[2], pl, p, grid);
+    }
 }
 
 template <int DT>
@@ -570,22 +639,25 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p) {
     EXHIP_REQUIRE(p.x && p.wp, "conv: NULL input or weights");
     EXHIP_REQUIRE(d->k_stride >= d->k || (!p.y_q && !p.y_nhwc && !p.residual), "conv: k_stride %d < k %d", d->k_stride, d->k);
     EXHIP_REQUIRE(!(p.y_q) || d->k_stride % 16 == 0, "conv: NHWC int8/half output needs k_stride %% 16 == 0");
+    EXHIP_REQUIRE((!p.scale || (uintptr_t)p.scale % 16 == 0) && (!p.bias || (uintptr_t)p.bias % 16 == 0),
+                  "conv: scale and bias arrays must be 16-byte aligned");
+    EXHIP_REQUIRE((uintptr_t)p.x % 16 == 0 && (uintptr_t)p.wp % 16 == 0, "conv: input and weights must be 16-byte aligned");
     p.N = d->n; p.H = d->h; p.W = d->w; p.K = d->k; p.OH = pl.OH; p.OW = pl.OW;
     p.KH = d->kh; p.KWe = pl.KWe; p.KS = pl.KS; p.S = pl.S; p.tile_step = pl.tile_step;
     p.PT = d->pt; p.PL = d->pl;
     p.cstride_b = d->c_stride * esize_of(DT);
     p.kstride = d->k_stride;
     p.PH = pl.PH; p.PW = pl.PW; p.IH = pl.IH; p.IW = pl.IW;
-    p.lds_pix_b = pl.lds_pix_b; p.lds_row_b = pl.lds_row_b; p.lds_act_b = pl.lds_act_b;
+    p.lds_pix_b = pl.lds_pix_b; p.lds_row_b = pl.lds_row_b; p.lds_act_b = pl.lds_act_b; p.lds_w_b = pl.lds_w_b;
+    p.act_bufs = pl.act_bufs; p.w_bufs = pl.w_bufs;
     p.n_chunks = pl.n_chunks; p.chunk_b = pl.chunk_b; p.RS = pl.RS; p.n_rg = pl.n_rg;
     p.tiles_x = pl.tiles_x; p.tiles_y = pl.tiles_y; p.ktiles = pl.ktiles;
     p.act = d->act; p.post_relu = d->post_relu; p.fs_out = d->fs_out; p.b_align = pl.b_align;
+    p.img_bytes = (unsigned)((size_t)d->h * d->w * p.cstride_b);
     const long long grid = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
     EXHIP_REQUIRE(grid > 0 && grid < (1ll << 31), "conv: grid too large");
-    // a lane reads 16 bytes at its fragment offset: keep the last read inside the allocation
-    const size_t lds = (size_t)pl.lds_act_b + pl.lds_w_b + 64;
-    if (pl.packed) return launch_variant<DT, true>(ctx, pl, p, (int)grid, lds);
-    return launch_variant<DT, false>(ctx, pl, p, (int)grid, lds);
+    if (pl.packed) return launch_variant<DT, true>(ctx, pl, p, (int)grid);
+    return launch_variant<DT, false>(ctx, pl, p, (int)grid);
 }
 
 template <typename T>
