@@ -18,6 +18,7 @@
 // 8*(i/4) + 4*(l/32) + i%4, column l%32. The host permutes the weight rows of each 32-channel tile so
 // that a lane's 16 registers are 16 consecutive output channels of one pixel: NHWC stores are then
 // 16-byte (int8) or 64-byte (f32) vectors.
+#include <stdlib.h>
 #include <string.h>
 
 #include <vector>
@@ -37,6 +38,13 @@ constexpr int kMaxActVec = 10;   // 16-byte activation vectors staged per thread
 constexpr int kMaxWVec = 9;      // 16-byte weight vectors staged per thread and stage (256-thread groups)
 constexpr int kMaxPackedPix = 8; // pixels staged per thread in packed-row form (256-thread groups)
 constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format: out-of-range reads return 0
+// per-wave LDS of the epilogue: a 32 x 64 float tile, a 32 x 64 int8 tile (rows padded by 16 bytes so that
+// 16-byte accesses one row apart fall into different banks) and 32 pixel indices
+constexpr int kEpiRowF = 64 * 4 + 16;
+constexpr int kEpiRowQ = 64 + 16;
+constexpr int kEpiWaveBytes = 32 * kEpiRowF + 32 * kEpiRowQ + 128;
+constexpr int kSbBytes = 1024;  // LDS kept for per-channel scale and bias of the group's (at most 128) channels
+constexpr unsigned kEpiInvalid = 0x3FFFFF00u;  // element offset whose byte offsets (x1, x4) lie past any accepted tensor
 
 struct ConvParams {
     const char* x;
@@ -49,6 +57,7 @@ struct ConvParams {
     void* y_nchw;    // f32 NCHW
     void* y_nchw_h;  // half NCHW (f16 kernel)
     int32_t* acc_nchw;
+    long long* dbg;  // optional phase timestamps (development aid), NULL in normal use
     int N, H, W, K, OH, OW;
     int KH, KWe, KS;          // filter rows, k-step groups per row (KW, or 1 packed), k-steps per chunk
     int S;                    // stride seen inside the staged tile
@@ -68,6 +77,8 @@ struct ConvParams {
     float fs_out;
     int b_align;              // alignment of B fragment reads in packed-row form (4, 8 or 16)
     unsigned img_bytes;       // bytes of one input image (buffer range for the bounds-checked loads)
+    unsigned magic_iw, magic_pw; // ceil(2^32 / IW), ceil(2^32 / PW): exact quotients by one multiply-high for operands < 2^16
+    int vp_shift;             // log2 of the 16-byte vectors per staged pixel
 };
 
 template <int DT> struct Acc { typedef v16i type; };
@@ -87,6 +98,9 @@ __device__ __forceinline__ void mma(typename Acc<DT>::type& acc, const v4i& a, c
     }
 }
 
+// n / d for n < 2^16 with magic = ceil(2^32 / d): one multiply-high instead of an emulated division
+__device__ __forceinline__ int fast_div(int n, unsigned magic) { return (int)__umulhi((unsigned)n, magic); }
+
 __device__ __forceinline__ v4i lds_read16(const char* p) { return *reinterpret_cast<const v4i*>(p); }
 
 __device__ __forceinline__ v4i lds_read16_unaligned(const char* p, int align) {
@@ -101,6 +115,15 @@ __device__ __forceinline__ v4i lds_read16_unaligned(const char* p, int align) {
     return r;
 }
 
+// Orders a wave's LDS writes before its later LDS reads of other lanes' data. One wave runs in lockstep and
+// the LDS serves a wave's accesses in issue order, so all that is needed is that the compiler keeps the
+// order and that outstanding LDS operations have completed. A memory fence is deliberately not used: it would
+// also wait for every outstanding global store, one full memory round trip per call.
+__device__ __forceinline__ void wave_sync() {
+    __asm__ volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_wave_barrier();
+}
+
 // sigmoid / mish evaluate double-precision transcendentals: kept out of line so the common epilogue stays small
 __device__ __noinline__ float slow_activation(float v, int act) { return exhip_act(v, act); }
 
@@ -110,8 +133,8 @@ __device__ __forceinline__ float fast_activation(float v, int act) {
     return v;
 }
 
-template <int DT, int MT, int NT, int WM, int WN, bool PACKED>
-__global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvParams p) {
+template <int DT, int MT, int NT, int WM, int WN, bool PACKED, int EPI>
+__global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvParams p) {
     constexpr int THREADS = 64 * WM * WN;
     constexpr int TM = 32 * MT * WM;
     // staging limits scale with the group size so that a 512-thread group needs half the registers
@@ -120,12 +143,17 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvPara
     constexpr int NWV = kMaxWVec * 256 / THREADS;
     typedef typename Acc<DT>::type acc_t;
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    // [activation buffers][weight buffers]
-    char* const lds_a0 = smem;
-    char* const lds_w0 = smem + p.act_bufs * p.lds_act_b;
+    // [scale, bias of this group's channels: 2 x 128 floats][activation buffers][weight buffers]
+    float* const lds_sb = reinterpret_cast<float*>(smem);
+    char* const lds_a0 = smem + kSbBytes;
+    char* const lds_w0 = lds_a0 + p.act_bufs * p.lds_act_b;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
+    auto stamp = [&](int k) {
+        if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * (THREADS / 64) + wave) * 16 + k] = wall_clock64();
+    };
+    stamp(0);
 
     // Workgroup ids are dealt round-robin to the 8 XCDs; give each XCD one contiguous run of tiles so
     // that the channel tiles of a patch and its spatial neighbours share that XCD's L2.
@@ -152,13 +180,12 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvPara
     int a_goff[PACKED ? NPP : NAV];
     int a_loff[PACKED ? NPP : NAV];
     if constexpr (!PACKED) {
-        const int vp = p.chunk_b >> 4;
-        const int nvec = p.IH * p.IW * vp;
+        const int nvec = (p.IH * p.IW) << p.vp_shift;
 #pragma unroll
         for (int i = 0; i < NAV; ++i) {
             const int v = tid + THREADS * i;
-            const int pix = v / vp, part = v - pix * vp;
-            const int iy = pix / p.IW, ix = pix - iy * p.IW;
+            const int pix = v >> p.vp_shift, part = v - (pix << p.vp_shift);
+            const int iy = fast_div(pix, p.magic_iw), ix = pix - iy * p.IW;
             const int gy = iy0 + iy * p.tile_step, gx = ix0 + ix * p.tile_step;
             const bool in_tile = v < nvec;
             const bool in_img = in_tile && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
@@ -170,7 +197,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvPara
 #pragma unroll
         for (int i = 0; i < NPP; ++i) {
             const int v = tid + THREADS * i;
-            const int iy = v / p.IW, ix = v - iy * p.IW;
+            const int iy = fast_div(v, p.magic_iw), ix = v - iy * p.IW;
             const int gy = iy0 + iy, gx = ix0 + ix;
             const bool in_tile = v < npix;
             const bool in_img = in_tile && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
@@ -188,7 +215,7 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvPara
         int pp = (wn * NT + j) * 32 + (lane & 31);
         const bool ok = pp < p.PH * p.PW;
         pp = ok ? pp : 0;
-        const int py = pp / p.PW, px = pp - py * p.PW;
+        const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
         ppy[j] = py;
         ppx[j] = px;
         if (ok && oy0 + py < p.OH && ox0 + px < p.OW) pvalid |= 1 << j;
@@ -208,9 +235,12 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvPara
     const int n_stages = p.n_chunks * p.n_rg;
     const char* const wkt = p.wp + (size_t)kt * p.n_chunks * p.KH * row_w_b;
 
+    // Staging registers. Weights of stage st travel in set (st & 1); with DEEP the set of stage st + 2 is
+    // requested at the start of stage st, so every load has one whole stage to land before it is needed.
+    constexpr bool DEEP = THREADS == 512;
     v4i a_reg[NAV];
     int a_reg_p[NPP][2];
-    v4i w_reg[NWV];
+    v4i w_set0[NWV], w_set1[DEEP ? NWV : 1];
 
     auto load_act = [&](int cc) {
         const int soff = PACKED ? 0 : cc * p.chunk_b;
@@ -242,38 +272,48 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvPara
         }
     };
     auto stage_rows = [&](int rg) { const int r0 = rg * p.RS; return (p.KH - r0 < p.RS ? p.KH - r0 : p.RS); };
-    auto load_w = [&](int cc, int rg) {
+    auto load_w = [&](int cc, int rg, auto& regs) {
         // a view of exactly this stage's slice: lanes past its end read zeros
         const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<char*>(wkt + (size_t)(cc * p.KH + rg * p.RS) * row_w_b), 0, stage_rows(rg) * row_w_b, kRsrcWord3);
 #pragma unroll
-        for (int i = 0; i < NWV; ++i) w_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (tid + THREADS * i) * 16, 0, 0);
+        for (int i = 0; i < NWV; ++i) regs[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (tid + THREADS * i) * 16, 0, 0);
     };
-    auto store_w = [&](char* dst) {
+    auto store_w = [&](char* dst, auto& regs) {
 #pragma unroll
         for (int i = 0; i < NWV; ++i) {
             const int v = (tid + THREADS * i) * 16;
-            if (v < p.lds_w_b) *reinterpret_cast<v4i*>(dst + v) = w_reg[i];
+            if (v < p.lds_w_b) *reinterpret_cast<v4i*>(dst + v) = regs[i];
         }
     };
 
-    load_act(0);
-    load_w(0, 0);
-    store_act(lds_a0);
-    store_w(lds_w0);
-    __syncthreads();
-
-    for (int st = 0; st < n_stages; ++st) {
-        const int cc = st / p.n_rg, rg = st - cc * p.n_rg;
+    // One stage: request what later stages need, run the MFMAs of this one from LDS, then publish the next
+    // stage's operands into the other LDS buffers. `mine` is the register set this stage's weights came in
+    // (free again), `next` the set holding stage st + 1.
+    // (chunk, row group) of the stage `by` stages after (cc, rg), without dividing
+    auto stage_after = [&](int cc, int rg, int by, int& cc_out, int& rg_out) {
+        for (int i = 0; i < by; ++i)
+            if (++rg == p.n_rg) { rg = 0; ++cc; }
+        cc_out = cc;
+        rg_out = rg;
+    };
+    auto run_stage = [&](int st, int cc, int rg, auto& mine, auto& next) {
         const bool more = st + 1 < n_stages;
         const bool next_chunk = rg + 1 == p.n_rg;
-        if (more) {
-            if (next_chunk) {
-                load_act(cc + 1);
-                load_w(cc + 1, 0);
-            } else {
-                load_w(cc, rg + 1);
+        if constexpr (DEEP) {
+            if (st + 2 < n_stages) {
+                int c2, r2;
+                stage_after(cc, rg, 2, c2, r2);
+                load_w(c2, r2, mine);
             }
+            if (rg == 0 && cc + 1 < p.n_chunks) load_act(cc + 1);
+        } else {
+            if (more) {
+                int c1, r1;
+                stage_after(cc, rg, 1, c1, r1);
+                load_w(c1, r1, next);
+            }
+            if (more && next_chunk) load_act(cc + 1);
         }
         // ---- MFMA over this stage: k-steps in (row, tap, channel) order, fragments fetched one step ahead ----
         const int nk = stage_rows(rg) * p.KWe * p.KS;
@@ -327,147 +367,272 @@ __global__ __launch_bounds__(64 * WM * WN) void conv_igemm_kernel(const ConvPara
         }
         if (more) {
             if (next_chunk) store_act(lds_a0 + ((cc + 1) & (p.act_bufs - 1)) * p.lds_act_b);
-            store_w(lds_w0 + ((st + 1) & (p.w_bufs - 1)) * p.lds_w_b);
+            store_w(lds_w0 + ((st + 1) & (p.w_bufs - 1)) * p.lds_w_b, next);
         }
         __syncthreads();
-    }
+    };
 
-    // ---- epilogue ----
-    const size_t img_px = (size_t)p.OH * p.OW;
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        const int ch0 = kt * TM + (wm * MT + m) * 32 + (lane >> 5) * 16;
-        if (ch0 >= p.kstride && ch0 >= p.K) continue;
-        float sc[16], bi[16];
-        if (ch0 + 16 <= p.K) {
-#pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-                v4f s4 = {0.f, 0.f, 0.f, 0.f}, b4 = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (DT == EXHIP_I8) s4 = *reinterpret_cast<const v4f*>(p.scale + ch0 + e4 * 4);
-                if (p.bias) b4 = *reinterpret_cast<const v4f*>(p.bias + ch0 + e4 * 4);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    sc[e4 * 4 + e] = s4[e];
-                    bi[e4 * 4 + e] = b4[e];
+    stamp(1);
+    if constexpr (EPI == 1) {
+        // per-channel scale and bias of this group's channels, fetched now so that the epilogue finds them in LDS
+        if (tid < 2 * TM) {
+            const int c = tid < TM ? tid : tid - TM;
+            const int ch = kt * TM + c;
+            float v = 0.f;
+            if (ch < p.K) v = tid < TM ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
+            lds_sb[(tid < TM ? 0 : 128) + c] = v;
+        }
+    }
+    load_act(0);
+    load_w(0, 0, w_set0);
+    if constexpr (DEEP) {
+        if (n_stages > 1) {
+            int c1, r1;
+            stage_after(0, 0, 1, c1, r1);
+            load_w(c1, r1, w_set1);
+        }
+    }
+    stamp(2);
+    store_act(lds_a0);
+    store_w(lds_w0, w_set0);
+    stamp(3);
+    __syncthreads();
+    stamp(4);
+
+    {
+        int cc = 0, rg = 0;
+        if constexpr (DEEP) {
+            for (int st = 0; st < n_stages; st += 2) {
+                run_stage(st, cc, rg, w_set0, w_set1);
+                stage_after(cc, rg, 1, cc, rg);
+                if (st + 1 < n_stages) {
+                    run_stage(st + 1, cc, rg, w_set1, w_set0);
+                    stage_after(cc, rg, 1, cc, rg);
                 }
             }
         } else {
+            for (int st = 0; st < n_stages; ++st) {
+                run_stage(st, cc, rg, w_set0, w_set0);
+                stage_after(cc, rg, 1, cc, rg);
+            }
+        }
+    }
+
+    stamp(5);
+    // ---- epilogue ----
+    // A lane holds, per accumulator tile, 16 consecutive output channels of one pixel.
+    const int img_px = p.OH * p.OW;
+    if constexpr (EPI == 1) {
+        // Fused int8 form (K a multiple of 64, channel stride == K): optional f32 NHWC shortcut input, optional
+        // f32 NHWC and int8 NHWC outputs. A lane's own NHWC vectors lie a whole pixel apart from its neighbours',
+        // so the three tensors go through a per-wave LDS tile of 32 pixels x 64 channels: lanes exchange rows
+        // there and global memory sees 256 / 64 contiguous bytes per pixel. All global accesses are
+        // bounds-checked buffer operations: a pixel outside the image gets an offset past the range, its
+        // loads return 0 and its stores are dropped, so no lane-divergent branch is needed.
+        char* const epi = smem + kSbBytes + wave * kEpiWaveBytes;  // the staging buffers are free: the loop ended with a barrier
+        char* const tile_f = epi;                       // [32 px][64 ch f32 + 16 B]
+        char* const tile_q = epi + 32 * kEpiRowF;       // [32 px][64 ch i8 + 16 B]
+        unsigned* const table = reinterpret_cast<unsigned*>(epi + 32 * kEpiRowF + 32 * kEpiRowQ);  // element offset per tile pixel
+        const int chb = kt * TM + wm * 64;              // first channel of this wave's 64-channel slab
+        const int px_l = lane & 31, hh = lane >> 5;
+        const bool has_res = p.residual != nullptr, has_f = p.y_nhwc != nullptr, has_q = p.y_q != nullptr;
+        const unsigned bytes_q = (unsigned)p.N * (unsigned)img_px * (unsigned)p.K;
+        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(p.y_q, 0, (int)bytes_q, kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_nhwc, 0, (int)(bytes_q * 4u), kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rr =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.residual), 0, (int)(bytes_q * 4u), kRsrcWord3);
+        const int nt_run = chb < p.K ? NT : 0;  // a wave whose slab lies past the last channel has nothing to write
+#pragma unroll
+        for (int nn = 0; nn < NT; ++nn) {
+            if (nn >= nt_run) break;
+            const bool valid = (pvalid >> nn) & 1;
+            const unsigned pix = (unsigned)n * img_px + (oy0 + ppy[nn]) * p.OW + ox0 + ppx[nn];
+            if (lane < 32) table[lane] = valid ? pix * (unsigned)p.K + chb : kEpiInvalid;
+            wave_sync();
+            if (has_res) {
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    const int idx = it * 64 + lane, tp = idx >> 4, part = idx & 15;
+                    const v4i rv = __builtin_amdgcn_raw_buffer_load_b128(rr, (int)((table[tp] + part * 4) * 4u), 0, 0);
+                    *reinterpret_cast<v4i*>(tile_f + tp * kEpiRowF + part * 16) = rv;
+                }
+                wave_sync();
+            }
+            if (nn == 0) stamp(6);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int ch0 = chb + m * 32 + hh * 16;
+                char* const tf = tile_f + px_l * kEpiRowF + (m * 32 + hh * 16) * 4;
+                v4i q4;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const v4f s4 = *reinterpret_cast<const v4f*>(lds_sb + (ch0 - kt * TM) + e4 * 4);
+                    const v4f b4 = *reinterpret_cast<const v4f*>(lds_sb + 128 + (ch0 - kt * TM) + e4 * 4);
+                    v4f v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e], b4[e]);
+                    if (p.act == 1) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
+                    }
+                    if (has_res) {
+                        const v4f rv = *reinterpret_cast<const v4f*>(tf + e4 * 16);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += rv[e];
+                    }
+                    if (p.post_relu) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
+                    }
+                    if (has_f) *reinterpret_cast<v4f*>(tf + e4 * 16) = v;
+                    // float32_to_int8(v * fs): product rounded first, then +-0.5, saturate, truncate
+                    int b[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float t = v[e] * p.fs_out;
+                        b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
+                    }
+                    q4[e4] = (b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24);
+                }
+                if (has_q) *reinterpret_cast<v4i*>(tile_q + px_l * kEpiRowQ + m * 32 + hh * 16) = q4;
+            }
+            wave_sync();
+            if (nn == 0) stamp(7);
+            if (has_f) {
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    const int idx = it * 64 + lane, tp = idx >> 4, part = idx & 15;
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const v4i*>(tile_f + tp * kEpiRowF + part * 16), rf,
+                                                           (int)((table[tp] + part * 4) * 4u), 0, 0);
+                }
+            }
+            if (has_q) {
+#pragma unroll
+                for (int it = 0; it < 2; ++it) {
+                    const int idx = it * 64 + lane, tp = idx >> 2, part = idx & 3;
+                    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const v4i*>(tile_q + tp * kEpiRowQ + part * 16), rq,
+                                                           (int)(table[tp] + part * 16), 0, 0);
+                }
+            }
+            wave_sync();  // the tiles and the table are rewritten by the next column block
+        }
+    } else {
+        // General form: every output kind, ragged channel counts, direct per-lane accesses.
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const int ch0 = kt * TM + (wm * MT + m) * 32 + (lane >> 5) * 16;
+            if (ch0 >= p.kstride && ch0 >= p.K) continue;
+            float sc[16], bi[16];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int ch = ch0 + e;
                 sc[e] = (DT == EXHIP_I8 && ch < p.K) ? p.scale[ch] : 0.f;
                 bi[e] = (p.bias && ch < p.K) ? p.bias[ch] : 0.f;
             }
-        }
 #pragma unroll
-        for (int nn = 0; nn < NT; ++nn) {
-            if (!((pvalid >> nn) & 1)) continue;
-            const int oy = oy0 + ppy[nn], ox = ox0 + ppx[nn];
-            const size_t pix = (size_t)n * img_px + (size_t)oy * p.OW + ox;
-            float v[16];
-            if constexpr (DT == EXHIP_I8) {
-                if (p.acc_nchw) {
+            for (int nn = 0; nn < NT; ++nn) {
+                if (!((pvalid >> nn) & 1)) continue;
+                const int oy = oy0 + ppy[nn], ox = ox0 + ppx[nn];
+                const size_t pix = (size_t)n * img_px + (size_t)oy * p.OW + ox;
+                const size_t nchw0 = ((size_t)n * p.K + ch0) * img_px + (size_t)oy * p.OW + ox;
+                float v[16];
+                if constexpr (DT == EXHIP_I8) {
+                    if (p.acc_nchw) {
 #pragma unroll
-                    for (int e = 0; e < 16; ++e)
-                        if (ch0 + e < p.K) p.acc_nchw[((size_t)n * p.K + ch0 + e) * img_px + (size_t)oy * p.OW + ox] = acc[m][nn][e];
-                }
+                        for (int e = 0; e < 16; ++e)
+                            if (ch0 + e < p.K) p.acc_nchw[nchw0 + (size_t)e * img_px] = acc[m][nn][e];
+                    }
 #pragma unroll
-                for (int e = 0; e < 16; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e], sc[e], bi[e]);
-            } else {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) v[e] = acc[m][nn][e] + bi[e];
-            }
-            if (p.act >= 4) {
-#pragma unroll 1
-                for (int e = 0; e < 16; ++e) v[e] = slow_activation(v[e], p.act);
-            } else if (p.act) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) v[e] = fast_activation(v[e], p.act);
-            }
-            if (p.residual) {
-                if constexpr (DT == EXHIP_F16) {
-                    const uint16_t* r = reinterpret_cast<const uint16_t*>(p.residual) + pix * p.kstride + ch0;
-#pragma unroll
-                    for (int e = 0; e < 16; ++e)
-                        if (ch0 + e < p.K) v[e] += exhip_h2f(r[e]);
+                    for (int e = 0; e < 16; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e], sc[e], bi[e]);
                 } else {
-                    const float* r = reinterpret_cast<const float*>(p.residual) + pix * p.kstride + ch0;
-                    if (ch0 + 16 <= p.kstride) {
 #pragma unroll
-                        for (int e4 = 0; e4 < 4; ++e4) {
-                            const v4f rv = *reinterpret_cast<const v4f*>(r + e4 * 4);
+                    for (int e = 0; e < 16; ++e) v[e] = acc[m][nn][e] + bi[e];
+                }
+                if (p.act >= 4) {
+#pragma unroll 1
+                    for (int e = 0; e < 16; ++e) v[e] = slow_activation(v[e], p.act);
+                } else if (p.act) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) v[e4 * 4 + e] += rv[e];
-                        }
+                    for (int e = 0; e < 16; ++e) v[e] = fast_activation(v[e], p.act);
+                }
+                if (p.residual) {
+                    if constexpr (DT == EXHIP_F16) {
+                        const uint16_t* r = reinterpret_cast<const uint16_t*>(p.residual) + pix * p.kstride + ch0;
+#pragma unroll
+                        for (int e = 0; e < 16; ++e)
+                            if (ch0 + e < p.K) v[e] += exhip_h2f(r[e]);
                     } else {
+                        const float* r = reinterpret_cast<const float*>(p.residual) + pix * p.kstride + ch0;
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
                             if (ch0 + e < p.K) v[e] += r[e];
                     }
                 }
-            }
-            if (p.post_relu) {
+                if (p.post_relu) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) v[e] = (0.f > v[e]) ? 0.f : v[e];
-            }
-#pragma unroll
-            for (int e = 0; e < 16; ++e)
-                if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
-            if (p.y_nchw) {
-                float* y = reinterpret_cast<float*>(p.y_nchw);
+                    for (int e = 0; e < 16; ++e) v[e] = (0.f > v[e]) ? 0.f : v[e];
+                }
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
-                    if (ch0 + e < p.K) y[((size_t)n * p.K + ch0 + e) * img_px + (size_t)oy * p.OW + ox] = v[e];
-            }
-            if constexpr (DT == EXHIP_F16) {
-                if (p.y_nchw_h) {
-                    uint16_t* y = reinterpret_cast<uint16_t*>(p.y_nchw_h);
+                    if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
+                if (p.y_nchw) {
+                    float* y = reinterpret_cast<float*>(p.y_nchw) + nchw0;
 #pragma unroll
                     for (int e = 0; e < 16; ++e)
-                        if (ch0 + e < p.K) y[((size_t)n * p.K + ch0 + e) * img_px + (size_t)oy * p.OW + ox] = exhip_f2h(v[e]);
+                        if (ch0 + e < p.K) y[(size_t)e * img_px] = v[e];
                 }
-                if (p.y_q && ch0 + 16 <= p.kstride) {
-                    v4i o[2];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const uint32_t lo = exhip_f2h(v[2 * e]), hi = exhip_f2h(v[2 * e + 1]);
-                        o[e >> 2][e & 3] = (int)(lo | (hi << 16));
-                    }
-                    v4i* y = reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.y_q) + pix * p.kstride + ch0);
-                    y[0] = o[0];
-                    y[1] = o[1];
-                }
-            } else {
-                if (p.y_nhwc) {
-                    float* y = reinterpret_cast<float*>(p.y_nhwc) + pix * p.kstride + ch0;
-                    if (ch0 + 16 <= p.kstride) {
-#pragma unroll
-                        for (int e4 = 0; e4 < 4; ++e4) {
-                            v4f o = {v[e4 * 4], v[e4 * 4 + 1], v[e4 * 4 + 2], v[e4 * 4 + 3]};
-                            *reinterpret_cast<v4f*>(y + e4 * 4) = o;
-                        }
-                    } else {
+                const bool vec_ok = ch0 + 16 <= p.kstride;
+                if constexpr (DT == EXHIP_F16) {
+                    if (p.y_nchw_h) {
+                        uint16_t* y = reinterpret_cast<uint16_t*>(p.y_nchw_h) + nchw0;
 #pragma unroll
                         for (int e = 0; e < 16; ++e)
-                            if (ch0 + e < p.kstride) y[e] = v[e];
+                            if (ch0 + e < p.K) y[(size_t)e * img_px] = exhip_f2h(v[e]);
                     }
-                }
-                if constexpr (DT == EXHIP_I8) {
-                    if (p.y_q && ch0 + 16 <= p.kstride) {
-                        v4i o;
+                    if (p.y_q && vec_ok) {
+                        v4i o[2];
 #pragma unroll
-                        for (int e4 = 0; e4 < 4; ++e4) {
-                            uint32_t w = 0;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(v[e4 * 4 + e] * p.fs_out) & 0xff) << (8 * e);
-                            o[e4] = (int)w;
+                        for (int e = 0; e < 8; ++e) {
+                            const uint32_t lo = exhip_f2h(v[2 * e]), hi = exhip_f2h(v[2 * e + 1]);
+                            o[e >> 2][e & 3] = (int)(lo | (hi << 16));
                         }
-                        *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(p.y_q) + pix * p.kstride + ch0) = o;
+                        v4i* y = reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.y_q) + pix * p.kstride + ch0);
+                        y[0] = o[0];
+                        y[1] = o[1];
+                    }
+                } else {
+                    if (p.y_nhwc) {
+                        float* y = reinterpret_cast<float*>(p.y_nhwc) + pix * p.kstride + ch0;
+                        if (vec_ok) {
+#pragma unroll
+                            for (int e4 = 0; e4 < 4; ++e4) {
+                                const v4f o = {v[e4 * 4], v[e4 * 4 + 1], v[e4 * 4 + 2], v[e4 * 4 + 3]};
+                                *reinterpret_cast<v4f*>(y + e4 * 4) = o;
+                            }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 16; ++e)
+                                if (ch0 + e < p.kstride) y[e] = v[e];
+                        }
+                    }
+                    if constexpr (DT == EXHIP_I8) {
+                        if (p.y_q && vec_ok) {
+                            v4i o;
+#pragma unroll
+                            for (int e4 = 0; e4 < 4; ++e4) {
+                                uint32_t w = 0;
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(v[e4 * 4 + e] * p.fs_out) & 0xff) << (8 * e);
+                                o[e4] = (int)w;
+                            }
+                            *reinterpret_cast<v4i*>(reinterpret_cast<int8_t*>(p.y_q) + pix * p.kstride + ch0) = o;
+                        }
                     }
                 }
             }
         }
     }
+    stamp(8);
 }
 
 // ---- host side: configuration search, packing, launch ----
@@ -495,7 +660,11 @@ struct Plan {
     int act_bufs, w_bufs;
     int tiles_x, tiles_y, ktiles;
     int OH, OW;
-    size_t lds_bytes() const { return (size_t)act_bufs * lds_act_b + (size_t)w_bufs * lds_w_b; }
+    size_t lds_bytes() const {  // staging buffers, reused by the epilogue's per-wave tiles
+        const size_t staging = (size_t)act_bufs * lds_act_b + (size_t)w_bufs * lds_w_b;
+        const size_t epilogue = (size_t)(threads / 64) * kEpiWaveBytes;
+        return kSbBytes + (staging > epilogue ? staging : epilogue);
+    }
 };
 
 int validate(const exhip_conv_desc* d, int dt) {
@@ -524,8 +693,10 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
     const int es = esize_of(dt), cb = d->c_stride * es;
     const int OH = (d->h + d->pt + d->pb - d->kh) / d->sh + 1, OW = (d->w + d->pl + d->pr - d->kw) / d->sw + 1;
     const bool packed = cb < 32;
+    static const int force_variant = getenv("EXHIP_FORCE_VARIANT") ? atoi(getenv("EXHIP_FORCE_VARIANT")) : -1;
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
+        if (force_variant >= 0 && variant != force_variant) continue;
         if (packed && chunk_opt == 64) continue;
         if (!packed && cb % chunk_opt != 0) continue;
         const int TM = kVariants[variant].TM, TN = kVariants[variant].TN;
@@ -583,7 +754,7 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
             }
             // the tile plus the 16 bytes a lane may read past its last row's last pixel
             p.lds_act_b = (p.IH * p.lds_row_b + 16 + 63) / 64 * 64;
-            if (p.lds_bytes() > 156 * 1024) continue;
+            if (p.lds_bytes() > 158 * 1024) continue;
             p.tiles_y = ceil_div(OH, PH);
             p.tiles_x = ceil_div(OW, PW);
             const double useful = (double)OH * OW * d->k;
@@ -620,13 +791,13 @@ int launch_kernel(exhip_ctx* ctx, K kernel, bool* attr_set, const Plan& pl, cons
     return 0;
 }
 
-template <int DT, bool PACKED>
+template <int DT, bool PACKED, int EPI>
 int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
     static bool attr[kNumVariants] = {false, false, false};
     switch (pl.variant) {
-    case 0: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 1, 4, PACKED>, &attr[0], pl, p, grid);
-    case 1: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 4, PACKED>, &attr[1], pl, p, grid);
-    default: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 2, PACKED>, &attr[2], pl, p, grid);
+    case 0: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 1, 4, PACKED, EPI>, &attr[0], pl, p, grid);
+    case 1: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 4, PACKED, EPI>, &attr[1], pl, p, grid);
+    default: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 2, PACKED, EPI>, &attr[2], pl, p, grid);
     }
 }
 
@@ -653,11 +824,26 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p) {
     p.n_chunks = pl.n_chunks; p.chunk_b = pl.chunk_b; p.RS = pl.RS; p.n_rg = pl.n_rg;
     p.tiles_x = pl.tiles_x; p.tiles_y = pl.tiles_y; p.ktiles = pl.ktiles;
     p.act = d->act; p.post_relu = d->post_relu; p.fs_out = d->fs_out; p.b_align = pl.b_align;
+    p.dbg = getenv("EXHIP_DEBUG_STAMPS") ? (long long*)strtoull(getenv("EXHIP_DEBUG_STAMPS"), nullptr, 0) : nullptr;
     p.img_bytes = (unsigned)((size_t)d->h * d->w * p.cstride_b);
+    p.magic_iw = (unsigned)(((1ull << 32) + pl.IW - 1) / pl.IW);
+    p.magic_pw = (unsigned)(((1ull << 32) + pl.PW - 1) / pl.PW);
+    p.vp_shift = pl.chunk_b == 64 ? 2 : 1;
+    EXHIP_REQUIRE((long long)d->n * pl.OH * pl.OW < (1ll << 31), "conv: more than 2^31 output pixels");
     const long long grid = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
     EXHIP_REQUIRE(grid > 0 && grid < (1ll << 31), "conv: grid too large");
-    if (pl.packed) return launch_variant<DT, true>(ctx, pl, p, (int)grid);
-    return launch_variant<DT, false>(ctx, pl, p, (int)grid);
+    if constexpr (DT == EXHIP_I8) {
+        // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
+        const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
+        const bool fused = !p.y_nchw && !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
+                           out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
+        if (fused) {
+            if (pl.packed) return launch_variant<DT, true, 1>(ctx, pl, p, (int)grid);
+            return launch_variant<DT, false, 1>(ctx, pl, p, (int)grid);
+        }
+    }
+    if (pl.packed) return launch_variant<DT, true, 0>(ctx, pl, p, (int)grid);
+    return launch_variant<DT, false, 0>(ctx, pl, p, (int)grid);
 }
 
 template <typename T>
