@@ -75,26 +75,43 @@ def main():
               "is part of it (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
 
+    import tempfile
+
     from excalibur_amd import hip
+    from excalibur_amd import pipeline as xp
     from excalibur_amd.resnet18 import FusedRunner, ResNet18Int8
 
     ctx = hip.Ctx(0)
     net = ResNet18Int8(seed=1234, calib_hw=64)
     n, hw = args.batch, args.hw
-    run = FusedRunner(ctx, net, n, hw, hw)
     x = np.random.default_rng(99).uniform(-1, 1, (n, 3, hw, hw)).astype(np.float32)
-    run.set_input(x)
 
+    # The timed path: the generated .phai / .racy loaded through the host-side pipeline<float>(lines, model, device 0),
+    # which runs the int8 chain as one fused plan over the exhip C ABI. The input blob is uploaded before timing.
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        model_path = f.name
+    net.write_model(model_path)
+    pipe = xp.Pipeline(net.topology(), model_path, 0, "f32", fusion=True)
+    os.unlink(model_path)
+    pipe.set_input(x)
     for _ in range(args.warmup):
-        run.forward()
-    ctx.sync()
+        pipe.run()
+    pipe.sync()
+    assert pipe.fused, "the int8 ResNet-18 topology did not take the fused plan"
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        run.forward()
-    ctx.sync()
+        pipe.run()
+    pipe.sync()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     images_per_s = n * args.steps / elapsed
+
+    # The same launches issued one by one from Python, for per-kernel event timing.
+    run = FusedRunner(ctx, net, n, hw, hw)
+    run.set_input(x)
+    for _ in range(2):
+        run.forward()
+    ctx.sync()
 
     # per-launch durations (HIP events on the library's stream) for the roofline of the dominant kernel
     reps = max(3, min(args.steps, 10))
@@ -130,6 +147,7 @@ def main():
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(net, hw)
     print(json.dumps(line))
+    pipe.close()
     ctx.close()
 
 

@@ -1,0 +1,51 @@
+// The reference's public entry point (include/Excalibur/pipeline.hpp:17-47): a pipeline is built from a
+// `.phai` topology (file or lines) and a `.racy` model file (or dummy weights), and forward() returns the
+// output blobs by name. device >= 0 selects this MI355X backend; device < 0 is fatal here (no CPU path).
+#pragma once
+#include <memory>
+#include <string>
+#include <string_view>
+#include <unordered_map>
+#include <vector>
+
+#include "../Primitives/tensor.hpp"
+
+namespace glasssix {
+namespace excalibur {
+
+template <typename Dtype>
+class pipeline {
+public:
+    class impl;
+    using blob_map = std::unordered_map<std::string, std::shared_ptr<memory::tensor<Dtype>>>;
+
+    explicit pipeline(std::string_view param_file, std::string_view model_file, int device = -1);
+    explicit pipeline(std::string_view param_file, int device = -1);
+    explicit pipeline(const std::vector<std::string>& hardcode_params, std::string_view model_file, int device = -1);
+    ~pipeline();
+
+    blob_map forward(const std::shared_ptr<memory::tensor<Dtype>>& input_tensor);
+    blob_map forward_cpu(const std::shared_ptr<memory::tensor<Dtype>>& input_tensor);
+    blob_map forward_gpu(const std::shared_ptr<memory::tensor<Dtype>>& input_tensor);
+    std::shared_ptr<memory::tensor<Dtype>> get_featmap(std::string_view featmap_name);
+
+    void enable_profiler();   // per-layer HIP-event timings printed after each forward
+    void disable_profiler();
+
+    // Backend switch without a counterpart in the reference: run int8 convolution chains with fused
+    // epilogues and int8 NHWC tensors between layers (default on). Intermediate blobs are then not
+    // materialised as float tensors; get_featmap() returns pipeline outputs only.
+    void set_fusion(bool on);
+    bool fused() const;
+    double last_forward_ms() const;
+
+    static std::string version();
+
+private:
+    impl* impl_;
+    pipeline(const pipeline&) = delete;
+    pipeline& operator=(const pipeline&) = delete;
+};
+
+}  // namespace excalibur
+}  // namespace glasssix

@@ -1,0 +1,108 @@
+// C ABI over pipeline<float> / pipeline<unsigned short> (include/excalibur_capi.h).
+#include "../../../include/excalibur_capi.h"
+
+#include <cstring>
+#include <sstream>
+
+#include "../include/Excalibur/operation_reflector.hpp"
+#include "../include/Excalibur/pipeline.hpp"
+
+using glasssix::excalibur::pipeline;
+using glasssix::memory::tensor;
+
+struct exc_pipeline {
+    int dtype = 0, device = 0;
+    std::unique_ptr<pipeline<float>> f32;
+    std::unique_ptr<pipeline<unsigned short>> f16;
+    std::shared_ptr<tensor<float>> in32;
+    std::shared_ptr<tensor<unsigned short>> in16;
+    pipeline<float>::blob_map out32;
+    pipeline<unsigned short>::blob_map out16;
+};
+
+namespace {
+std::vector<std::string> split_lines(const char* text) {
+    std::vector<std::string> lines;
+    std::istringstream in{std::string(text)};
+    std::string line;
+    while (std::getline(in, line)) lines.push_back(line);
+    return lines;
+}
+
+template <typename T>
+void set_input(std::shared_ptr<tensor<T>>& slot, int device, const void* data, const int* shape) {
+    const std::vector<int> s{shape[0], shape[1], shape[2], shape[3]};
+    if (!slot || slot->data_shape() != s) slot = std::make_shared<tensor<T>>(s, device, glasssix::memory::NCHW);
+    std::memcpy(slot->mutable_cpu_data(), data, sizeof(T) * static_cast<size_t>(slot->count()));
+    slot->gpu_data();  // upload now, so that timed runs start with the input resident in HBM
+}
+
+template <typename T, typename P, typename M>
+long get_blob(P& pipe, M& outs, const char* name, void* out, long capacity, int* shape) {
+    std::shared_ptr<tensor<T>> t;
+    auto it = outs.find(name);
+    t = it != outs.end() ? it->second : pipe.get_featmap(name);
+    if (!t) return -1;
+    const std::vector<int> s = t->data_shape();
+    for (int i = 0; i < 4; ++i) shape[i] = s[i];
+    const long n = t->count();
+    if (out && n <= capacity) std::memcpy(out, t->cpu_data(), sizeof(T) * static_cast<size_t>(n));
+    return n;
+}
+}  // namespace
+
+extern "C" exc_pipeline* exc_pipeline_create(const char* topology, const char* model_path, int device, int dtype) {
+    auto* p = new exc_pipeline();
+    p->dtype = dtype;
+    p->device = device;
+    const std::vector<std::string> lines = split_lines(topology);
+    const std::string model(model_path ? model_path : "");
+    if (dtype == 0) p->f32.reset(new pipeline<float>(lines, model, device));
+    else p->f16.reset(new pipeline<unsigned short>(lines, model, device));
+    return p;
+}
+
+extern "C" void exc_pipeline_destroy(exc_pipeline* p) { delete p; }
+
+extern "C" void exc_pipeline_set_fusion(exc_pipeline* p, int on) {
+    if (p->f32) p->f32->set_fusion(on != 0);
+}
+
+extern "C" int exc_pipeline_last_fused(exc_pipeline* p) { return p->f32 ? p->f32->fused() : 0; }
+
+extern "C" int exc_pipeline_set_input(exc_pipeline* p, const void* input, const int shape[4]) {
+    if (p->dtype == 0) set_input(p->in32, p->device, input, shape);
+    else set_input(p->in16, p->device, input, shape);
+    return 0;
+}
+
+extern "C" int exc_pipeline_run(exc_pipeline* p) {
+    if (p->dtype == 0) p->out32 = p->f32->forward(p->in32);
+    else p->out16 = p->f16->forward(p->in16);
+    return 0;
+}
+
+extern "C" int exc_pipeline_sync(exc_pipeline* p) { return exhip_sync(glasssix::memory::device_context(p->device)); }
+
+extern "C" int exc_pipeline_forward(exc_pipeline* p, const void* input, const int shape[4]) {
+    exc_pipeline_set_input(p, input, shape);
+    exc_pipeline_run(p);
+    return exc_pipeline_sync(p);
+}
+
+extern "C" long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, long capacity, int shape[4]) {
+    if (p->dtype == 0) return get_blob<float>(*p->f32, p->out32, name, out, capacity, shape);
+    return get_blob<unsigned short>(*p->f16, p->out16, name, out, capacity, shape);
+}
+
+extern "C" size_t exc_registered_operations(int dtype, char* buf, size_t len) {
+    std::string all;
+    const std::vector<std::string> names = dtype == 0 ? glasssix::excalibur::operation_reflector<float>::instance().registered()
+                                                      : glasssix::excalibur::operation_reflector<unsigned short>::instance().registered();
+    for (const std::string& n : names) all += n + "\n";
+    if (buf && len) {
+        std::strncpy(buf, all.c_str(), len - 1);
+        buf[len - 1] = 0;
+    }
+    return all.size() + 1;
+}

@@ -1,0 +1,166 @@
+// syncedmem / tensor / device contexts (the reference's src/Primitives/{syncedmem,tensor}.cpp roles).
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+
+#include "../include/Primitives/tensor.hpp"
+
+namespace glasssix {
+namespace memory {
+
+namespace {
+std::mutex g_mu;
+std::map<int, exhip_ctx*> g_ctx;
+std::map<std::pair<int, size_t>, std::vector<void*>> g_free;  // (device, rounded bytes) -> idle blocks
+
+size_t round_block(size_t bytes) {
+    size_t b = 256;
+    while (b < bytes) b <<= 1;
+    // above 1 MiB round to 1/8 of the power of two instead, to bound the slack
+    if (b > (1u << 20)) {
+        const size_t step = b >> 4;
+        b = (bytes + step - 1) / step * step;
+    }
+    return b;
+}
+}  // namespace
+
+exhip_ctx* device_context(int device) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_ctx.find(device);
+    if (it != g_ctx.end()) return it->second;
+    exhip_ctx* ctx = nullptr;
+    int rc = exhip_init(device, &ctx);
+    if (rc != 0) LOG(FATAL) << "cannot open HIP device " << device << ": " << exhip_last_error();
+    g_ctx[device] = ctx;
+    return ctx;
+}
+
+void* device_alloc(int device, size_t bytes) {
+    exhip_ctx* ctx = device_context(device);
+    const size_t rb = round_block(bytes);
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        auto& pool = g_free[{device, rb}];
+        if (!pool.empty()) {
+            void* p = pool.back();
+            pool.pop_back();
+            return p;
+        }
+    }
+    void* p = nullptr;
+    EXHIP_FATAL(exhip_malloc(ctx, rb, &p));
+    return p;
+}
+
+void device_release(int device, void* ptr, size_t bytes) {
+    if (!ptr) return;
+    std::lock_guard<std::mutex> lock(g_mu);
+    g_free[{device, round_block(bytes)}].push_back(ptr);
+}
+
+template <typename Dtype>
+syncedmem<Dtype>::syncedmem(size_t size, int device) : size_(size), device_(device) {}
+
+template <typename Dtype>
+syncedmem<Dtype>::~syncedmem() {
+    if (cpu_ptr_) std::free(cpu_ptr_);
+    if (gpu_ptr_) {
+        // kernels reading this buffer may still be queued: recycle only after the stream has drained
+        exhip_sync(device_context(device_));
+        device_release(device_, gpu_ptr_, size_ * sizeof(Dtype));
+    }
+}
+
+template <typename Dtype>
+void syncedmem<Dtype>::to_cpu() {
+    const size_t bytes = size_ * sizeof(Dtype);
+    switch (head_) {
+    case UNINITIALIZED:
+        cpu_ptr_ = static_cast<Dtype*>(std::aligned_alloc(64, (bytes + 63) / 64 * 64 + 64));
+        std::memset(cpu_ptr_, 0, bytes);
+        head_ = HEAD_AT_CPU;
+        break;
+    case HEAD_AT_GPU:
+        if (!cpu_ptr_) cpu_ptr_ = static_cast<Dtype*>(std::aligned_alloc(64, (bytes + 63) / 64 * 64 + 64));
+        EXHIP_FATAL(exhip_memcpy_d2h(device_context(device_), cpu_ptr_, gpu_ptr_, bytes));  // synchronises the stream
+        head_ = SYNCED;
+        break;
+    default: break;
+    }
+}
+
+template <typename Dtype>
+void syncedmem<Dtype>::to_gpu() {
+    if (device_ < 0) LOG(FATAL) << "gpu_data() on a tensor created without a device";
+    const size_t bytes = size_ * sizeof(Dtype);
+    exhip_ctx* ctx = device_context(device_);
+    switch (head_) {
+    case UNINITIALIZED:
+        gpu_ptr_ = static_cast<Dtype*>(device_alloc(device_, bytes));
+        EXHIP_FATAL(exhip_memset(ctx, gpu_ptr_, 0, bytes));
+        head_ = HEAD_AT_GPU;
+        break;
+    case HEAD_AT_CPU:
+        if (!gpu_ptr_) gpu_ptr_ = static_cast<Dtype*>(device_alloc(device_, bytes));
+        EXHIP_FATAL(exhip_memcpy_h2d(ctx, gpu_ptr_, cpu_ptr_, bytes));
+        head_ = SYNCED;
+        break;
+    default: break;
+    }
+}
+
+template <typename Dtype>
+const Dtype* syncedmem<Dtype>::cpu_data() { to_cpu(); return cpu_ptr_; }
+template <typename Dtype>
+const Dtype* syncedmem<Dtype>::gpu_data() { to_gpu(); return gpu_ptr_; }
+template <typename Dtype>
+Dtype* syncedmem<Dtype>::mutable_cpu_data() { to_cpu(); head_ = HEAD_AT_CPU; return cpu_ptr_; }
+template <typename Dtype>
+Dtype* syncedmem<Dtype>::mutable_gpu_data() { to_gpu(); head_ = HEAD_AT_GPU; return gpu_ptr_; }
+
+template <typename Dtype>
+void tensor<Dtype>::init(const std::vector<int>& shape, int device) {
+    shape_ = shape;
+    device_ = device;
+    data_ = std::make_shared<syncedmem<Dtype>>(static_cast<size_t>(count()), device);
+}
+template <typename Dtype>
+tensor<Dtype>::tensor(orderType order, pool_allocator<Dtype>*) : order_(order) { init({0, 0, 0, 0}, -1); }
+template <typename Dtype>
+tensor<Dtype>::tensor(const int w, int device, orderType order, pool_allocator<Dtype>*) : order_(order) {
+    init(order == NCHW ? std::vector<int>{1, 1, 1, w} : std::vector<int>{1, 1, w, 1}, device);
+}
+template <typename Dtype>
+tensor<Dtype>::tensor(const int h, const int w, int device, orderType order, pool_allocator<Dtype>*) : order_(order) {
+    init(order == NCHW ? std::vector<int>{1, 1, h, w} : std::vector<int>{1, h, w, 1}, device);
+}
+template <typename Dtype>
+tensor<Dtype>::tensor(const int c, const int h, const int w, int device, orderType order, pool_allocator<Dtype>*) : order_(order) {
+    init(order == NCHW ? std::vector<int>{1, c, h, w} : std::vector<int>{1, h, w, c}, device);
+}
+template <typename Dtype>
+tensor<Dtype>::tensor(const std::vector<int>& shape, int device, orderType order, pool_allocator<Dtype>*) : order_(order) {
+    std::vector<int> s = shape;
+    while (s.size() < 4) s.insert(s.begin(), 1);
+    init(s, device);
+}
+template <typename Dtype>
+void tensor<Dtype>::copy_from(const void* data, size_t size) {
+    CHECK_LE(size, static_cast<size_t>(count()) * sizeof(Dtype));
+    std::memcpy(mutable_cpu_data(), data, size);
+}
+
+#define INSTANTIATE_MEMORY(T) \
+    template class syncedmem<T>; \
+    template class tensor<T>;
+INSTANTIATE_MEMORY(float)
+INSTANTIATE_MEMORY(double)
+INSTANTIATE_MEMORY(int)
+INSTANTIATE_MEMORY(signed char)
+INSTANTIATE_MEMORY(unsigned char)
+INSTANTIATE_MEMORY(unsigned short)
+
+}  // namespace memory
+}  // namespace glasssix

@@ -1,0 +1,813 @@
+// Operator implementations: parameter parsing and weight loading as the reference does them, computation
+// through the exhip C ABI on the operator's device. Tensors at this interface are the reference's dense NCHW
+// blobs; the kernels' NHWC / int8 forms are produced and consumed inside each forward call.
+#include "../include/Excalibur/operators.hpp"
+
+#include <cmath>
+#include <cstring>
+#include <random>
+
+#include "../include/Excalibur/operation_reflector.hpp"
+
+namespace glasssix {
+namespace excalibur {
+
+using memory::tensor;
+
+std::vector<std::string> split_string(const std::string& s, const std::string& c) {
+    std::vector<std::string> out;
+    size_t from = 0, at;
+    while ((at = s.find(c, from)) != std::string::npos) {
+        out.push_back(s.substr(from, at - from));
+        from = at + c.size();
+    }
+    if (from != s.length()) out.push_back(s.substr(from));
+    return out;
+}
+
+std::vector<layer_attr> parse_attrs(const std::string& specific_params) {
+    std::vector<layer_attr> attrs;
+    for (const std::string& tok : split_string(specific_params, " ")) {
+        if (tok.empty()) continue;
+        const size_t eq = tok.find('=');
+        attrs.push_back({tok.substr(0, eq), eq == std::string::npos ? std::string() : tok.substr(eq + 1)});
+    }
+    return attrs;
+}
+
+template <typename Dtype>
+operation<Dtype>::operation(const operation_param& param) : params_(param) {
+    if (sizeof(Dtype) == 2) params_.set_float16(true);  // pipeline<unsigned short> is the fp16 pipeline (operation.cpp:13-16)
+}
+
+template <>
+void operation<float>::forward_cpu(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    if (params_.int8_quantization_) forward_cpu_i8(bottoms, tops);
+    else forward_cpu_f32(bottoms, tops);
+}
+template <>
+void operation<float>::forward_gpu(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    if (params_.int8_quantization_) forward_gpu_i8(bottoms, tops);
+    else forward_gpu_f32(bottoms, tops);
+}
+template <>
+void operation<unsigned short>::forward_cpu(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    forward_cpu_f16(bottoms, tops);
+}
+template <>
+void operation<unsigned short>::forward_gpu(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    forward_gpu_f16(bottoms, tops);
+}
+template class operation<float>;
+template class operation<unsigned short>;
+
+namespace {
+
+inline int pad_to(int v, int m) { return (v + m - 1) / m * m; }
+
+template <typename T>
+std::shared_ptr<tensor<T>> new_tensor(std::vector<int> shape, int device) {
+    return std::make_shared<tensor<T>>(shape, device, memory::NCHW, nullptr);
+}
+
+// 1 x 1 x 1 x n vector blob (the reference's tensor(w, device, order, allocator) constructor)
+template <typename T>
+std::shared_ptr<tensor<T>> vec_tensor(int n, int device) {
+    return std::make_shared<tensor<T>>(n, device, memory::NCHW, nullptr);
+}
+
+// float -> IEEE half bits, round to nearest even
+unsigned short half_bits_rne(float f) {
+    unsigned int u;
+    std::memcpy(&u, &f, 4);
+    const unsigned int sign = (u >> 16) & 0x8000u;
+    unsigned int a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return static_cast<unsigned short>(sign | 0x7E00u);
+    if (a >= 0x47800000u) return static_cast<unsigned short>(sign | 0x7C00u);
+    if (a < 0x38800000u) {
+        if (a < 0x33000000u) return static_cast<unsigned short>(sign);
+        const int e = static_cast<int>(a >> 23);
+        const unsigned int m = (a & 0x7FFFFFu) | 0x800000u;
+        const int shift = 126 - e;
+        unsigned int r = m >> shift;
+        const unsigned int rem = m & ((1u << shift) - 1), halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (r & 1))) ++r;
+        return static_cast<unsigned short>(sign | r);
+    }
+    unsigned int r = (a - 0x38000000u) >> 13;
+    const unsigned int rem = a & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (r & 1))) ++r;
+    return static_cast<unsigned short>(sign | r);
+}
+
+// input channel stride (elements) the MFMA convolution wants for a dtype / kernel width
+int conv_in_stride(int c, int dtype, int kw) {
+    const int es = dtype == EXHIP_I8 ? 1 : dtype == EXHIP_F16 ? 2 : 4;
+    if (c <= 4 && ((dtype == EXHIP_I8 && kw <= 8) || (dtype == EXHIP_F16 && kw <= 4))) return 4;
+    return pad_to(c * es, 32) / es;
+}
+
+void require_nchw(memory::orderType o) {
+    if (o != memory::NCHW) LOG(FATAL) << "this backend takes NCHW blobs at the operator interface";
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------ convolution parameters
+template <typename Dtype>
+operation_general_conv<Dtype>::operation_general_conv(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        const int v = a.as_int();
+        switch (key) {
+        case 0: output_channel_ = v; break;
+        case 1: kernel_size_w_ = kernel_size_h_ = v; break;
+        case 2: dilation_w_ = dilation_h_ = v; break;
+        case 3: stride_w_ = stride_h_ = v; break;
+        case 4: pad_left_ = pad_right_ = pad_top_ = pad_bottom_ = v; break;
+        case 5: bias_term_ = v != 0; break;
+        case 6: weight_data_size_ = v; break;
+        case 7: group_ = v; break;
+        case 8:
+            int8_scale_term_ = v != 0;
+            this->params_.set_int8_quantization(int8_scale_term_);
+            break;
+        case 9: activation_type_ = v; break;
+        case 10: NOT_IMPLEMENTED; break;
+        case 11: kernel_size_h_ = v; break;
+        case 12: dilation_h_ = v; break;
+        case 13: stride_h_ = v; break;
+        case 14: pad_top_ = v; break;
+        case 15: pad_right_ = v; break;
+        case 16: pad_bottom_ = v; break;
+        case 17: impl_type_ = v; break;
+        case 18: output_pad_right_ = output_pad_bottom_ = v; break;
+        case 19: output_pad_bottom_ = v; break;
+        case 20: output_dim_h_ = output_dim_w_ = v; break;
+        case 21: output_dim_w_ = v; break;
+        case -23330: break;
+        default: LOG(FATAL) << "Un-supported Convolution Attribution " << a.key;
+        }
+    }
+    CHECK_GT(group_, 0);
+    CHECK_EQ(output_channel_ % group_, 0);
+}
+
+// ------------------------------------------------------------------ convolution
+template <typename Dtype>
+operation_convolution<Dtype>::operation_convolution(const operation_param& param) : operation_general_conv<Dtype>(param) {}
+
+template <typename Dtype>
+operation_convolution<Dtype>::~operation_convolution() {
+    for (auto& kv : packed_) memory::device_release(this->params_.device_, kv.second.ptr, kv.second.bytes);
+}
+
+// Weight blob, src/Excalibur/operation_convolution.cpp:71-152: int32 tag; tag 0: float W (OIHW) then float bias[K];
+// tag 871224: int8 W padded to a multiple of 4 bytes, float bias[K], float ws[K], float fs[1]. In the int8 case the
+// bias sits in weights_f32_[1] behind a one-element placeholder (:121-126).
+template <typename Dtype>
+int operation_convolution<Dtype>::init_weights(FILE* fp) {
+    const int dev = this->params_.device_;
+    int tag = 0;
+    if (fread(&tag, 1, sizeof(int), fp) != sizeof(int)) LOG(FATAL) << "model file ended inside layer " << this->params_.name_;
+    int mem = 0;
+    const int k = this->output_channel_;
+    auto read_into = [&](void* dst, size_t bytes) {
+        if (fread(dst, 1, bytes, fp) != bytes) LOG(FATAL) << "model file ended inside layer " << this->params_.name_;
+        mem += static_cast<int>(bytes);
+    };
+    if (tag == 0) {
+        this->weights_f32_.push_back(vec_tensor<float>(this->weight_data_size_, dev));
+        read_into(this->weights_f32_[0]->mutable_cpu_data(), sizeof(float) * this->weight_data_size_);
+        if (this->bias_term_) {
+            this->weights_f32_.push_back(vec_tensor<float>(k, dev));
+            read_into(this->weights_f32_[1]->mutable_cpu_data(), sizeof(float) * k);
+        }
+    } else if (tag == 871224) {
+        const int aligned = (this->weight_data_size_ + 3) & ~3;
+        this->weights_i8_.push_back(vec_tensor<signed char>(aligned, dev));
+        read_into(this->weights_i8_[0]->mutable_cpu_data(), aligned);
+        if (this->bias_term_) {
+            this->weights_f32_.push_back(vec_tensor<float>(1, dev));
+            this->weights_f32_.push_back(vec_tensor<float>(k, dev));
+            read_into(this->weights_f32_[1]->mutable_cpu_data(), sizeof(float) * k);
+        }
+        this->weights_scaletable_i8_ = vec_tensor<float>(k, dev);
+        read_into(this->weights_scaletable_i8_->mutable_cpu_data(), sizeof(float) * k);
+        this->featmap_scaletable_i8_ = vec_tensor<float>(1, dev);
+        read_into(this->featmap_scaletable_i8_->mutable_cpu_data(), sizeof(float));
+    } else {
+        NOT_IMPLEMENTED;
+    }
+    return mem;
+}
+
+// Dummy weights, src/Excalibur/operation_convolution.cpp:155-248: a default-seeded std::default_random_engine
+// drawn in this order: weights, bias, (int8: weight scales, feature-map scale).
+template <typename Dtype>
+int operation_convolution<Dtype>::init_weights() {
+    const int dev = this->params_.device_;
+    std::default_random_engine e;
+    std::normal_distribution<float> n(0, 0.3);
+    std::uniform_int_distribution<int> u(-128, 127);
+    const int k = this->output_channel_;
+    int mem = 0;
+    if (!this->params_.int8_quantization_) {
+        this->weights_f32_.push_back(vec_tensor<float>(this->weight_data_size_, dev));
+        float* w = this->weights_f32_[0]->mutable_cpu_data();
+        for (int i = 0; i < this->weight_data_size_; ++i) w[i] = n(e);
+        mem += this->weight_data_size_ * sizeof(float);
+        if (this->bias_term_) {
+            this->weights_f32_.push_back(vec_tensor<float>(k, dev));
+            float* b = this->weights_f32_[1]->mutable_cpu_data();
+            for (int i = 0; i < k; ++i) b[i] = n(e);
+            mem += k * sizeof(float);
+        }
+    } else {
+        const int aligned = (this->weight_data_size_ + 3) & ~3;
+        this->weights_i8_.push_back(vec_tensor<signed char>(aligned, dev));
+        signed char* w = this->weights_i8_[0]->mutable_cpu_data();
+        for (int i = 0; i < aligned; ++i) w[i] = static_cast<signed char>(u(e));
+        mem += aligned;
+        if (this->bias_term_) {
+            this->weights_f32_.push_back(vec_tensor<float>(1, dev));
+            this->weights_f32_.push_back(vec_tensor<float>(k, dev));
+            float* b = this->weights_f32_[1]->mutable_cpu_data();
+            for (int i = 0; i < k; ++i) b[i] = n(e);
+            mem += k * sizeof(float);
+        }
+        this->weights_scaletable_i8_ = vec_tensor<float>(k, dev);
+        float* ws = this->weights_scaletable_i8_->mutable_cpu_data();
+        for (int i = 0; i < k; ++i) ws[i] = n(e);
+        this->featmap_scaletable_i8_ = vec_tensor<float>(1, dev);
+        this->featmap_scaletable_i8_->mutable_cpu_data()[0] = n(e);
+        mem += (k + 1) * sizeof(float);
+    }
+    return mem;
+}
+
+template <typename Dtype>
+float operation_convolution<Dtype>::featmap_scale() const {
+    CHECK(this->featmap_scaletable_i8_ != nullptr) << "layer " << this->params_.name_ << " has no int8 scales";
+    return this->featmap_scaletable_i8_->cpu_data()[0];
+}
+
+template <typename Dtype>
+std::vector<float> operation_convolution<Dtype>::dequantize_scales() const {
+    const int k = this->output_channel_;
+    const float fs = featmap_scale();
+    const float* ws = this->weights_scaletable_i8_->cpu_data();
+    const int n_ws = this->weights_scaletable_i8_->count();
+    std::vector<float> s(k);
+    for (int q = 0; q < k; ++q) {
+        const float w = n_ws == 1 ? ws[0] : ws[q];
+        volatile float prod = w * fs;  // float product, then float division
+        s[q] = (std::fabs(w) <= 1e-6) ? 0.f : (1.0f / prod);
+    }
+    return s;
+}
+
+template <typename Dtype>
+const float* operation_convolution<Dtype>::bias_gpu() {
+    if (!this->bias_term_) return nullptr;
+    return this->weights_f32_[1]->gpu_data();
+}
+
+template <typename Dtype>
+const float* operation_convolution<Dtype>::scale_gpu() {
+    if (!scale_dev_) {
+        const std::vector<float> s = dequantize_scales();
+        scale_dev_ = vec_tensor<float>(static_cast<int>(s.size()), this->params_.device_);
+        std::memcpy(scale_dev_->mutable_cpu_data(), s.data(), s.size() * sizeof(float));
+    }
+    return scale_dev_->gpu_data();
+}
+
+template <typename Dtype>
+exhip_conv_desc operation_convolution<Dtype>::describe(int n, int h, int w, int c_stride, int k_stride) const {
+    exhip_conv_desc d;
+    std::memset(&d, 0, sizeof(d));
+    d.n = n; d.c = this->input_channels(); d.h = h; d.w = w; d.k = this->output_channel_;
+    d.kh = this->kernel_size_h_; d.kw = this->kernel_size_w_; d.sh = this->stride_h_; d.sw = this->stride_w_;
+    d.pt = this->pad_top_; d.pb = this->pad_bottom_; d.pl = this->pad_left_; d.pr = this->pad_right_;
+    d.act = this->activation_type_; d.c_stride = c_stride; d.k_stride = k_stride;
+    return d;
+}
+
+template <typename Dtype>
+const void* operation_convolution<Dtype>::packed_weights(int dtype, const exhip_conv_desc& d) {
+    const std::vector<int> key{dtype, d.n, d.h, d.w, d.c_stride};
+    auto it = packed_.find(key);
+    if (it != packed_.end()) return it->second.ptr;
+    const size_t bytes = exhip_conv_packed_bytes(&d, dtype);
+    if (bytes == 0) LOG(FATAL) << "layer " << this->params_.name_ << ": " << exhip_last_error();
+    std::vector<char> host(bytes);
+    std::vector<unsigned short> half_w;
+    const void* src = nullptr;
+    if (dtype == EXHIP_I8) {
+        src = this->weights_i8_[0]->cpu_data();
+    } else if (dtype == EXHIP_F32) {
+        src = this->weights_f32_[0]->cpu_data();
+    } else {
+        // fp16 MFMA operands: float weights rounded to nearest-even half once, here
+        const float* w = this->weights_f32_[0]->cpu_data();
+        half_w.resize(this->weight_data_size_);
+        for (int i = 0; i < this->weight_data_size_; ++i) half_w[i] = half_bits_rne(w[i]);
+        src = half_w.data();
+    }
+    EXHIP_FATAL(exhip_conv_pack_weights(&d, dtype, src, host.data()));
+    void* dev = memory::device_alloc(this->params_.device_, bytes);
+    EXHIP_FATAL(exhip_memcpy_h2d(this->ctx(), dev, host.data(), bytes));
+    packed_[key] = {dev, bytes};
+    return dev;
+}
+
+template <typename Dtype>
+bool operation_convolution<Dtype>::mfma_path_ok() const {
+    if (this->dilation_h_ != 1 || this->dilation_w_ != 1)
+        LOG(FATAL) << "layer " << this->params_.name_ << ": dilation is ignored by the reference's x86 path and not supported here";
+    return this->group_ == 1 && this->stride_h_ == this->stride_w_;
+}
+
+template <typename Dtype>
+void operation_convolution<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    require_nchw(bottoms[0]->order());
+    const int dev = this->params_.device_;
+    const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
+    CHECK_EQ(c, this->input_channels());
+    exhip_conv_desc d = describe(n, h, w, c, this->output_channel_);
+    int oh, ow;
+    EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
+    tops[0] = new_tensor<float>({n, this->output_channel_, oh, ow}, dev);
+    if (!mfma_path_ok()) {
+        EXHIP_FATAL(exhip_conv2d_direct_nchw(this->ctx(), &d, this->group_, bottoms[0]->gpu_data(), this->weights_f32_[0]->gpu_data(),
+                                             nullptr, 1.f, nullptr, bias_gpu(), tops[0]->mutable_gpu_data()));
+        return;
+    }
+    d.c_stride = conv_in_stride(c, EXHIP_F32, d.kw);
+    auto x = new_tensor<float>({n, h, w, d.c_stride}, dev);
+    EXHIP_FATAL(exhip_nchw_f32_to_nhwc_f32(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, d.c_stride, x->mutable_gpu_data()));
+    EXHIP_FATAL(exhip_conv2d_f32(this->ctx(), &d, x->gpu_data(), packed_weights(EXHIP_F32, d), bias_gpu(), nullptr, nullptr,
+                                 tops[0]->mutable_gpu_data()));
+}
+
+template <typename Dtype>
+void operation_convolution<Dtype>::forward_gpu_i8(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    require_nchw(bottoms[0]->order());
+    const int dev = this->params_.device_;
+    const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
+    CHECK_EQ(c, this->input_channels());
+    CHECK_EQ(this->featmap_scaletable_i8_->count(), 1) << "per-channel feature-map scales are not supported";
+    exhip_conv_desc d = describe(n, h, w, c, this->output_channel_);
+    int oh, ow;
+    EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
+    tops[0] = new_tensor<float>({n, this->output_channel_, oh, ow}, dev);
+    if (!mfma_path_ok()) {
+        EXHIP_FATAL(exhip_conv2d_direct_nchw(this->ctx(), &d, this->group_, bottoms[0]->gpu_data(), nullptr,
+                                             this->weights_i8_[0]->gpu_data(), featmap_scale(), scale_gpu(), bias_gpu(),
+                                             tops[0]->mutable_gpu_data()));
+        return;
+    }
+    d.c_stride = conv_in_stride(c, EXHIP_I8, d.kw);
+    auto q = new_tensor<signed char>({n, h, w, d.c_stride}, dev);
+    EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, featmap_scale(), nullptr,
+                                                   d.c_stride, reinterpret_cast<int8_t*>(q->mutable_gpu_data())));
+    EXHIP_FATAL(exhip_conv2d_i8(this->ctx(), &d, reinterpret_cast<const int8_t*>(q->gpu_data()), packed_weights(EXHIP_I8, d),
+                                scale_gpu(), bias_gpu(), nullptr, nullptr, nullptr, tops[0]->mutable_gpu_data(), nullptr));
+}
+
+template <typename Dtype>
+void operation_convolution<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    require_nchw(bottoms[0]->order());
+    const int dev = this->params_.device_;
+    const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
+    CHECK_EQ(c, this->input_channels());
+    exhip_conv_desc d = describe(n, h, w, c, this->output_channel_);
+    int oh, ow;
+    EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
+    tops[0] = new_tensor<unsigned short>({n, this->output_channel_, oh, ow}, dev);
+    if (!mfma_path_ok()) {
+        // definition-order kernel in float on converted tensors, result rounded to half
+        auto xf = new_tensor<float>({n, c, h, w}, dev);
+        auto yf = new_tensor<float>({n, this->output_channel_, oh, ow}, dev);
+        EXHIP_FATAL(exhip_f16_to_f32(this->ctx(), bottoms[0]->gpu_data(), xf->mutable_gpu_data(), xf->count()));
+        EXHIP_FATAL(exhip_conv2d_direct_nchw(this->ctx(), &d, this->group_, xf->gpu_data(), this->weights_f32_[0]->gpu_data(), nullptr,
+                                             1.f, nullptr, bias_gpu(), yf->mutable_gpu_data()));
+        EXHIP_FATAL(exhip_f32_to_f16(this->ctx(), yf->gpu_data(), tops[0]->mutable_gpu_data(), yf->count()));
+        return;
+    }
+    d.c_stride = conv_in_stride(c, EXHIP_F16, d.kw);
+    auto x = new_tensor<unsigned short>({n, h, w, d.c_stride}, dev);
+    EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, d.c_stride, x->mutable_gpu_data()));
+    EXHIP_FATAL(exhip_conv2d_f16(this->ctx(), &d, x->gpu_data(), packed_weights(EXHIP_F16, d), bias_gpu(), nullptr, nullptr,
+                                 tops[0]->mutable_gpu_data(), nullptr));
+}
+
+// ------------------------------------------------------------------ depthwise convolution
+template <typename Dtype>
+bool operation_convolutiondepthwise<Dtype>::fast3x3() const {
+    return this->kernel_size_h_ == 3 && this->kernel_size_w_ == 3 && this->stride_h_ == this->stride_w_ &&
+           (this->stride_h_ == 1 || this->stride_h_ == 2);
+}
+
+template <typename Dtype>
+void operation_convolutiondepthwise<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    CHECK_EQ(this->output_channel_, this->group_);
+    CHECK_EQ(bottoms[0]->channels(), this->output_channel_);
+    if (!fast3x3()) {  // the reference falls back to the grouped dense convolution (operation_convolutiondepthwise.cpp:118)
+        operation_convolution<Dtype>::forward_gpu_f32(bottoms, tops);
+        return;
+    }
+    require_nchw(bottoms[0]->order());
+    const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
+    const int oh = (h + this->pad_top_ + this->pad_bottom_ - 3) / this->stride_h_ + 1;
+    const int ow = (w + this->pad_left_ + this->pad_right_ - 3) / this->stride_w_ + 1;
+    tops[0] = new_tensor<float>({n, c, oh, ow}, this->params_.device_);
+    EXHIP_FATAL(exhip_dwconv3x3_nchw_f32(this->ctx(), bottoms[0]->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
+                                         tops[0]->mutable_gpu_data(), n, c, h, w, this->stride_h_, this->pad_top_, this->pad_bottom_,
+                                         this->pad_left_, this->pad_right_, this->activation_type_));
+}
+
+// Weight-only quantization: the int8 weights are dequantized once and the float path runs
+// (src/Excalibur/operation_convolutiondepthwise.cpp:184-222).
+template <typename Dtype>
+void operation_convolutiondepthwise<Dtype>::forward_gpu_i8(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    if (this->int8_scale_term_) {
+        const int aligned = (this->weight_data_size_ + 3) & ~3;
+        auto wf = vec_tensor<float>(aligned, this->params_.device_);
+        EXHIP_FATAL(exhip_dw_dequant_weights(this->ctx(), reinterpret_cast<const int8_t*>(this->weights_i8_[0]->gpu_data()),
+                                             this->weights_scaletable_i8_->gpu_data(), wf->mutable_gpu_data(), this->output_channel_,
+                                             aligned / this->group_));
+        if (this->weights_f32_.empty()) this->weights_f32_.push_back(wf);
+        else this->weights_f32_[0] = wf;
+        this->int8_scale_term_ = false;
+    }
+    forward_gpu_f32(bottoms, tops);
+}
+
+template <typename Dtype>
+void operation_convolutiondepthwise<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms,
+                                                            tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    CHECK_EQ(this->output_channel_, this->group_);
+    if (!fast3x3()) {
+        operation_convolution<Dtype>::forward_gpu_f16(bottoms, tops);
+        return;
+    }
+    require_nchw(bottoms[0]->order());
+    const int dev = this->params_.device_;
+    const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
+    const int oh = (h + this->pad_top_ + this->pad_bottom_ - 3) / this->stride_h_ + 1;
+    const int ow = (w + this->pad_left_ + this->pad_right_ - 3) / this->stride_w_ + 1;
+    const int cs = pad_to(c, 8);
+    auto x = new_tensor<unsigned short>({n, h, w, cs}, dev);
+    auto y = new_tensor<unsigned short>({n, oh, ow, cs}, dev);
+    tops[0] = new_tensor<unsigned short>({n, c, oh, ow}, dev);
+    EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, cs, x->mutable_gpu_data()));
+    EXHIP_FATAL(exhip_dwconv3x3_nhwc_f16(this->ctx(), x->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
+                                         y->mutable_gpu_data(), n, c, h, w, cs, this->stride_h_, this->pad_top_, this->pad_bottom_,
+                                         this->pad_left_, this->pad_right_, this->activation_type_));
+    EXHIP_FATAL(exhip_nhwc_f16_to_nchw_f16(this->ctx(), y->gpu_data(), n, c, oh, ow, cs, tops[0]->mutable_gpu_data()));
+}
+
+// ------------------------------------------------------------------ pooling
+template <typename Dtype>
+operation_pooling<Dtype>::operation_pooling(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int v = a.as_int();
+        switch (std::atoi(a.key.c_str())) {
+        case 0: type_ = v; break;
+        case 1: kernel_size_w_ = kernel_size_h_ = v; break;
+        case 2: stride_w_ = stride_h_ = v; break;
+        case 3: pad_left_ = pad_right_ = pad_top_ = pad_bottom_ = v; break;
+        case 4: global_pooling_ = v != 0; break;
+        case 5: pad_mode_ = v; break;
+        case 6: avgpool_count_include_pad_ = v; break;
+        case 11: kernel_size_h_ = v; break;
+        case 12: stride_h_ = v; break;
+        case 13: pad_top_ = v; break;
+        case 14: pad_right_ = v; break;
+        case 15: pad_bottom_ = v; break;
+        case -23330: break;
+        default: LOG(FATAL) << "Un-supported Pooling Attribution " << a.key;
+        }
+    }
+}
+
+template <typename Dtype>
+void operation_pooling<Dtype>::geometry(int h, int w, int* kh, int* kw, int* sh, int* sw, int* pt, int* pb, int* pl, int* pr,
+                                        int* oh, int* ow) const {
+    *kh = kernel_size_h_; *kw = kernel_size_w_; *sh = stride_h_; *sw = stride_w_;
+    *pt = pad_top_; *pb = pad_bottom_; *pl = pad_left_; *pr = pad_right_;
+    if (global_pooling_) {  // src/Excalibur/operation_pooling.cpp:90-100
+        *kh = h; *kw = w; *sh = *sw = 1; *pt = *pb = *pl = *pr = 0;
+    }
+    if (type_ != 0 && type_ != 1) LOG(FATAL) << "Unknown pooling method.";
+    if (pad_mode_ != 0 && pad_mode_ != 1) NOT_IMPLEMENTED;
+    EXHIP_FATAL(exhip_pool_out_hw(h, w, *kh, *kw, *sh, *sw, *pt, *pb, *pl, *pr, pad_mode_, oh, ow));
+}
+
+template <typename Dtype>
+void operation_pooling<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        require_nchw(bottoms[i]->order());
+        const int n = bottoms[i]->num(), c = bottoms[i]->channels(), h = bottoms[i]->height(), w = bottoms[i]->width();
+        int kh, kw, sh, sw, pt, pb, pl, pr, oh, ow;
+        geometry(h, w, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &oh, &ow);
+        tops[i] = new_tensor<float>({n, c, oh, ow}, this->params_.device_);
+        EXHIP_FATAL(exhip_pool2d_nchw_f32(this->ctx(), bottoms[i]->gpu_data(), tops[i]->mutable_gpu_data(), n, c, h, w, oh, ow, type_,
+                                          kh, kw, sh, sw, pt, pb, pl, pr, avgpool_count_include_pad_));
+    }
+}
+
+template <typename Dtype>
+void operation_pooling<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    const int dev = this->params_.device_;
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        require_nchw(bottoms[i]->order());
+        const int n = bottoms[i]->num(), c = bottoms[i]->channels(), h = bottoms[i]->height(), w = bottoms[i]->width();
+        int kh, kw, sh, sw, pt, pb, pl, pr, oh, ow;
+        geometry(h, w, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &oh, &ow);
+        const int cs = pad_to(c, 8);
+        auto x = new_tensor<unsigned short>({n, h, w, cs}, dev);
+        auto y = new_tensor<unsigned short>({n, oh, ow, cs}, dev);
+        tops[i] = new_tensor<unsigned short>({n, c, oh, ow}, dev);
+        EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), bottoms[i]->gpu_data(), n, c, h, w, cs, x->mutable_gpu_data()));
+        EXHIP_FATAL(exhip_pool2d_nhwc_f16(this->ctx(), x->gpu_data(), y->mutable_gpu_data(), n, c, h, w, cs, oh, ow, type_, kh, kw, sh,
+                                          sw, pt, pb, pl, pr, avgpool_count_include_pad_));
+        EXHIP_FATAL(exhip_nhwc_f16_to_nchw_f16(this->ctx(), y->gpu_data(), n, c, oh, ow, cs, tops[i]->mutable_gpu_data()));
+    }
+}
+
+// ------------------------------------------------------------------ eltwise / binaryop / relu / split
+template <typename Dtype>
+operation_eltwise<Dtype>::operation_eltwise(const operation_param& param) : operation<Dtype>(param) {
+    coeffs_.assign(param.input_count_, 1.0f);
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) {
+            type_ = a.as_int();
+        } else if (key == -23301) {
+            // "n,c0,c1,...": the reference reads entries 1 .. n-1 into coeffs_[0 .. n-2] (operation_eltwise.cpp:26-33)
+            const std::vector<std::string> parts = split_string(a.value, ",");
+            CHECK_EQ(type_, static_cast<int>(SUM));
+            const int cnt = parts.empty() ? 0 : std::atoi(parts[0].c_str());
+            for (int j = 1; j < cnt && j < static_cast<int>(parts.size()) && j - 1 < static_cast<int>(coeffs_.size()); ++j)
+                coeffs_[j - 1] = static_cast<float>(std::atof(parts[j].c_str()));
+        } else if (key != -23330) {
+            LOG(FATAL) << "Un-supported Eltwise Attribution " << a.key;
+        }
+    }
+}
+
+template <typename Dtype>
+void operation_eltwise<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_GE(bottoms.size(), 2);
+    CHECK_EQ(tops.size(), 1);
+    for (size_t i = 1; i < bottoms.size(); ++i) CHECK(bottoms[i]->data_shape() == bottoms[0]->data_shape());
+    if (type_ < 0 || type_ > 2) LOG(FATAL) << "Unknown elementwise operation.";
+    tops[0] = std::make_shared<tensor<float>>(bottoms[0]->data_shape(), this->params_.device_, bottoms[0]->order());
+    std::vector<const float*> in;
+    for (auto& b : bottoms) in.push_back(b->gpu_data());
+    EXHIP_FATAL(exhip_eltwise_f32(this->ctx(), in.data(), static_cast<int>(in.size()), coeffs_.data(), type_,
+                                  tops[0]->mutable_gpu_data(), tops[0]->count()));
+}
+
+template <typename Dtype>
+void operation_eltwise<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    // fp16 layer = float operator on half-rounded inputs, result rounded to half
+    CHECK_GE(bottoms.size(), 2);
+    CHECK_EQ(tops.size(), 1);
+    const int dev = this->params_.device_;
+    tensor_list<float> f(bottoms.size());
+    std::vector<const float*> in;
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        CHECK(bottoms[i]->data_shape() == bottoms[0]->data_shape());
+        f[i] = std::make_shared<tensor<float>>(bottoms[i]->data_shape(), dev, bottoms[i]->order());
+        EXHIP_FATAL(exhip_f16_to_f32(this->ctx(), bottoms[i]->gpu_data(), f[i]->mutable_gpu_data(), f[i]->count()));
+        in.push_back(f[i]->gpu_data());
+    }
+    auto y = std::make_shared<tensor<float>>(bottoms[0]->data_shape(), dev, bottoms[0]->order());
+    EXHIP_FATAL(exhip_eltwise_f32(this->ctx(), in.data(), static_cast<int>(in.size()), coeffs_.data(), type_, y->mutable_gpu_data(),
+                                  y->count()));
+    tops[0] = std::make_shared<tensor<unsigned short>>(bottoms[0]->data_shape(), dev, bottoms[0]->order());
+    EXHIP_FATAL(exhip_f32_to_f16(this->ctx(), y->gpu_data(), tops[0]->mutable_gpu_data(), y->count()));
+}
+
+template <typename Dtype>
+operation_binaryop<Dtype>::operation_binaryop(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        switch (std::atoi(a.key.c_str())) {
+        case 0: op_type_ = a.as_int(); break;
+        case 1: with_scalar_ = a.as_int(); break;
+        case 2: coef_ = a.as_float(); break;
+        default: LOG(FATAL) << "Un-supported BinaryOp Attribution " << a.key;
+        }
+    }
+}
+
+template <typename Dtype>
+void operation_binaryop<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_GE(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    if (op_type_ != 0 || with_scalar_ || bottoms.size() != 2 || bottoms[0]->data_shape() != bottoms[1]->data_shape())
+        LOG(FATAL) << "layer " << this->params_.name_ << ": this backend implements BinaryOp as equal-shape ADD only (the residual add)";
+    tops[0] = std::make_shared<tensor<float>>(bottoms[0]->data_shape(), this->params_.device_, bottoms[0]->order());
+    EXHIP_FATAL(exhip_add_f32(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
+}
+
+template <typename Dtype>
+void operation_binaryop<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(tops.size(), 1);
+    if (op_type_ != 0 || with_scalar_ || bottoms.size() != 2 || bottoms[0]->data_shape() != bottoms[1]->data_shape())
+        LOG(FATAL) << "layer " << this->params_.name_ << ": this backend implements BinaryOp as equal-shape ADD only (the residual add)";
+    tops[0] = std::make_shared<tensor<unsigned short>>(bottoms[0]->data_shape(), this->params_.device_, bottoms[0]->order());
+    EXHIP_FATAL(exhip_add_f16(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
+}
+
+template <typename Dtype>
+operation_relu<Dtype>::operation_relu(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) slope_ = a.as_float();
+        else if (key != -23330) LOG(FATAL) << "Un-supported ReLU Attribution " << a.key;
+    }
+    this->params_.inplace_ = true;
+}
+
+template <typename Dtype>
+void operation_relu<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        tops[i] = std::make_shared<tensor<float>>(bottoms[i]->data_shape(), this->params_.device_, bottoms[i]->order());
+        EXHIP_FATAL(exhip_relu_f32(this->ctx(), bottoms[i]->gpu_data(), tops[i]->mutable_gpu_data(), tops[i]->count()));
+    }
+}
+
+template <typename Dtype>
+void operation_relu<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        tops[i] = std::make_shared<tensor<unsigned short>>(bottoms[i]->data_shape(), this->params_.device_, bottoms[i]->order());
+        EXHIP_FATAL(exhip_relu_f16(this->ctx(), bottoms[i]->gpu_data(), tops[i]->mutable_gpu_data(), tops[i]->count()));
+    }
+}
+
+// Split hands the same blob to every consumer (src/Excalibur/operation_split.cpp:14-23).
+template <typename Dtype>
+void operation_split<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    for (auto& t : tops) t = bottoms[0];
+}
+template <typename Dtype>
+void operation_split<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    for (auto& t : tops) t = bottoms[0];
+}
+
+// ------------------------------------------------------------------ inner product
+template <typename Dtype>
+operation_innerproduct<Dtype>::operation_innerproduct(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int v = a.as_int();
+        switch (std::atoi(a.key.c_str())) {
+        case 0: num_output_ = v; break;
+        case 1: bias_term_ = v != 0; break;
+        case 2: weight_data_size_ = v; break;
+        case 8:
+            int8_scale_term_ = v != 0;
+            this->params_.set_int8_quantization(int8_scale_term_);
+            break;
+        case 9: activation_type_ = v; break;
+        case 10: NOT_IMPLEMENTED; break;
+        case -23330: break;
+        default: LOG(FATAL) << "Un-supported InnerProduct Attribution " << a.key;
+        }
+    }
+}
+
+// src/Excalibur/operation_innerproduct.cpp:77-120: like the convolution blob, with a single weight scale.
+template <typename Dtype>
+int operation_innerproduct<Dtype>::init_weights(FILE* fp) {
+    const int dev = this->params_.device_;
+    int tag = 0, mem = 0;
+    if (fread(&tag, 1, sizeof(int), fp) != sizeof(int)) LOG(FATAL) << "model file ended inside layer " << this->params_.name_;
+    auto read_into = [&](void* dst, size_t bytes) {
+        if (fread(dst, 1, bytes, fp) != bytes) LOG(FATAL) << "model file ended inside layer " << this->params_.name_;
+        mem += static_cast<int>(bytes);
+    };
+    if (tag == 0) {
+        this->weights_f32_.push_back(vec_tensor<float>(weight_data_size_, dev));
+        read_into(this->weights_f32_[0]->mutable_cpu_data(), sizeof(float) * weight_data_size_);
+        if (bias_term_) {
+            this->weights_f32_.push_back(vec_tensor<float>(num_output_, dev));
+            read_into(this->weights_f32_[1]->mutable_cpu_data(), sizeof(float) * num_output_);
+        }
+    } else if (tag == 871224) {
+        const int aligned = (weight_data_size_ + 3) & ~3;
+        this->weights_i8_.push_back(vec_tensor<signed char>(aligned, dev));
+        read_into(this->weights_i8_[0]->mutable_cpu_data(), aligned);
+        if (bias_term_) {
+            this->weights_f32_.push_back(vec_tensor<float>(1, dev));
+            this->weights_f32_.push_back(vec_tensor<float>(num_output_, dev));
+            read_into(this->weights_f32_[1]->mutable_cpu_data(), sizeof(float) * num_output_);
+        }
+        this->weights_scaletable_i8_ = vec_tensor<float>(1, dev);
+        read_into(this->weights_scaletable_i8_->mutable_cpu_data(), sizeof(float));
+        this->featmap_scaletable_i8_ = vec_tensor<float>(1, dev);
+        read_into(this->featmap_scaletable_i8_->mutable_cpu_data(), sizeof(float));
+    } else {
+        NOT_IMPLEMENTED;
+    }
+    return mem;
+}
+
+template <typename Dtype>
+int operation_innerproduct<Dtype>::init_weights() {
+    std::default_random_engine e;
+    std::normal_distribution<float> n(0, 0.3);
+    const int dev = this->params_.device_;
+    this->weights_f32_.push_back(vec_tensor<float>(weight_data_size_, dev));
+    float* w = this->weights_f32_[0]->mutable_cpu_data();
+    for (int i = 0; i < weight_data_size_; ++i) w[i] = n(e);
+    int mem = weight_data_size_ * sizeof(float);
+    if (bias_term_) {
+        this->weights_f32_.push_back(vec_tensor<float>(num_output_, dev));
+        float* b = this->weights_f32_[1]->mutable_cpu_data();
+        for (int i = 0; i < num_output_; ++i) b[i] = n(e);
+        mem += num_output_ * sizeof(float);
+    }
+    return mem;
+}
+
+// Y[m,n] = sum_k X[m,k] W[n,k] (+ b[n]); when exactly two of (C,H,W) differ from 1 the reference treats the H rows
+// of each image as a batch of W-long vectors and adds no bias (src/Excalibur/operation_innerproduct.cpp:197-212).
+template <typename Dtype>
+void operation_innerproduct<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    require_nchw(bottoms[0]->order());
+    if (this->weights_f32_.empty()) NOT_IMPLEMENTED << " (int8 InnerProduct has no CPU counterpart in the reference)";
+    const int dev = this->params_.device_;
+    const int m = bottoms[0]->num(), n = num_output_, c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
+    const float* bias = bias_term_ ? this->weights_f32_[1]->gpu_data() : nullptr;
+    const int dims = (w == 1 ? 0 : 1) + (h == 1 ? 0 : 1) + (c == 1 ? 0 : 1);
+    if (dims == 2) {
+        tops[0] = new_tensor<float>({m, 1, h, n}, dev);
+        for (int i = 0; i < m; ++i)
+            EXHIP_FATAL(exhip_innerproduct_f32(this->ctx(), bottoms[0]->gpu_data() + bottoms[0]->offset(i), this->weights_f32_[0]->gpu_data(),
+                                               nullptr, tops[0]->mutable_gpu_data() + tops[0]->offset(i), h, n, w));
+        return;
+    }
+    const int k = bottoms[0]->count(1, 4);
+    CHECK_EQ(k * n, weight_data_size_);
+    tops[0] = new_tensor<float>({m, n, 1, 1}, dev);
+    EXHIP_FATAL(exhip_innerproduct_f32(this->ctx(), bottoms[0]->gpu_data(), this->weights_f32_[0]->gpu_data(), bias,
+                                       tops[0]->mutable_gpu_data(), m, n, k));
+}
+
+template <typename Dtype>
+void operation_innerproduct<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const int dev = this->params_.device_;
+    tensor_list<float> fb(1), ft(1);
+    fb[0] = std::make_shared<tensor<float>>(bottoms[0]->data_shape(), dev, bottoms[0]->order());
+    EXHIP_FATAL(exhip_f16_to_f32(this->ctx(), bottoms[0]->gpu_data(), fb[0]->mutable_gpu_data(), fb[0]->count()));
+    forward_gpu_f32(fb, ft);
+    tops[0] = std::make_shared<tensor<unsigned short>>(ft[0]->data_shape(), dev, ft[0]->order());
+    EXHIP_FATAL(exhip_f32_to_f16(this->ctx(), ft[0]->gpu_data(), tops[0]->mutable_gpu_data(), ft[0]->count()));
+}
+
+INSTANCE_CLASS(operation_general_conv);
+INSTANCE_CLASS(operation_convolution);
+INSTANCE_CLASS(operation_convolutiondepthwise);
+INSTANCE_CLASS(operation_pooling);
+INSTANCE_CLASS(operation_eltwise);
+INSTANCE_CLASS(operation_binaryop);
+INSTANCE_CLASS(operation_relu);
+INSTANCE_CLASS(operation_split);
+INSTANCE_CLASS(operation_innerproduct);
+
+REGISTE(operation_convolution);
+REGISTE(operation_convolutiondepthwise);
+REGISTE(operation_pooling);
+REGISTE(operation_eltwise);
+REGISTE(operation_binaryop);
+REGISTE(operation_relu);
+REGISTE(operation_split);
+REGISTE(operation_innerproduct);
+
+}  // namespace excalibur
+}  // namespace glasssix

@@ -1,0 +1,480 @@
+// pipeline: `.phai` topology parsing, operator creation through the registry, `.racy` weight loading and the two
+// executors of this backend. Parsing and bookkeeping follow the reference (src/Excalibur/pipeline.cpp:35-194,
+// 218-232, 406-451): line 0 is the magic and optional name, line 1 is ignored, every further line is
+// "<Type> <name> <n_in> <n_out> <inputs...> <outputs...> <key=value...>"; a layer with n_in == 0 gets the input
+// "<name>_input"; blobs nobody produces are pipeline inputs (the first one is fed), blobs nobody consumes are
+// outputs; layers run in file order.
+//
+// Executors:
+//  * per-layer: every operator's forward_gpu on float (or half) NCHW blobs, exactly the reference's contract;
+//  * fused (pipeline<float>, int8 networks made of Convolution / max Pooling / Split / BinaryOp add / ReLU):
+//    int8 NHWC tensors between layers, each convolution's epilogue doing dequantization + bias + activation
+//    (+ shortcut add + ReLU) and writing what its consumers read. Same values as the per-layer executor.
+#include "../include/Excalibur/pipeline.hpp"
+
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <functional>
+#include <map>
+#include <set>
+
+#include "../include/Excalibur/operation_reflector.hpp"
+#include "../include/Excalibur/operators.hpp"
+
+namespace glasssix {
+namespace excalibur {
+
+using memory::tensor;
+
+namespace {
+inline int pad_to(int v, int m) { return (v + m - 1) / m * m; }
+
+struct dev_buffer {  // device allocation owned by a fused plan
+    int device = -1;
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    dev_buffer() {}
+    dev_buffer(int dev, size_t n) : device(dev), ptr(memory::device_alloc(dev, n)), bytes(n) {}
+    dev_buffer(dev_buffer&& o) noexcept : device(o.device), ptr(o.ptr), bytes(o.bytes) { o.ptr = nullptr; }
+    dev_buffer& operator=(dev_buffer&& o) noexcept {
+        release();
+        device = o.device; ptr = o.ptr; bytes = o.bytes; o.ptr = nullptr;
+        return *this;
+    }
+    ~dev_buffer() { release(); }
+    void release() {
+        if (ptr) memory::device_release(device, ptr, bytes);
+        ptr = nullptr;
+    }
+    dev_buffer(const dev_buffer&) = delete;
+    dev_buffer& operator=(const dev_buffer&) = delete;
+};
+}  // namespace
+
+template <typename Dtype>
+class pipeline<Dtype>::impl {
+public:
+    using tensor_ptr = std::shared_ptr<tensor<Dtype>>;
+
+    impl(const std::vector<std::string>& lines, std::string_view model_file, int device) : device_(device) {
+        if (device >= 0) memory::device_context(device);  // opens the device, fatal if it is not an MI355X
+        if (lines.empty()) LOG(FATAL) << "Incorrect param file.";
+        const std::vector<std::string> head = split_string(lines[0], " ");
+        if (head.empty() || (head[0] != "glsv1" && head[0] != "7767517")) LOG(FATAL) << "Incorrect param file version.";
+        if (head.size() > 1) name_ = head[1];
+        for (size_t i = 2; i < lines.size(); ++i) {
+            std::vector<std::string> tok;
+            for (const std::string& t : split_string(lines[i], " "))
+                if (!t.empty() && t != "\r") tok.push_back(t);
+            if (tok.empty()) continue;
+            if (tok.size() < 4) LOG(FATAL) << "Incorrect layer line: " << lines[i];
+            operation_param p;
+            p.type_ = tok[0];
+            p.name_ = tok[1];
+            p.device_ = device_;
+            p.input_count_ = std::atoi(tok[2].c_str());
+            p.output_count_ = std::atoi(tok[3].c_str());
+            const size_t n_in = static_cast<size_t>(std::max(p.input_count_, 0)), n_out = static_cast<size_t>(std::max(p.output_count_, 0));
+            if (tok.size() < 4 + n_in + n_out) LOG(FATAL) << "Incorrect layer line: " << lines[i];
+            for (size_t j = 0; j < n_out; ++j) p.output_featmaps_.push_back(tok[4 + n_in + j]);
+            for (size_t j = 4 + n_in + n_out; j < tok.size(); ++j) p.specific_params_ += tok[j] + " ";
+            if (p.input_count_ <= 0) {
+                p.input_count_ = 1;
+                p.input_featmaps_ = {p.name_ + "_input"};
+            } else {
+                for (size_t j = 0; j < n_in; ++j) p.input_featmaps_.push_back(tok[4 + j]);
+            }
+            op_params_.push_back(p);
+        }
+        for (const operation_param& p : op_params_) operations_.push_back(operation_reflector<Dtype>::instance().create_object(p));
+
+        if (model_file.empty()) {
+            LOG(WARNING) << "THIS PIPELINE IS LOADED WITH DUMMY DATA.";
+            for (auto& op : operations_) weights_mem_cost_ += op->init_weights();
+        } else {
+            const std::string path(model_file);
+            FILE* fp = std::fopen(path.c_str(), "rb");
+            if (!fp) LOG(FATAL) << "Cannot open " << path;
+            for (auto& op : operations_) weights_mem_cost_ += op->init_weights(fp);
+            CHECK_EQ(std::fclose(fp), 0) << "Cannot close " << path;
+        }
+
+        // blob table, producers, consumers
+        std::map<std::string, int> produced_by;
+        for (size_t i = 0; i < op_params_.size(); ++i)
+            for (const std::string& o : op_params_[i].output_featmaps_) produced_by[o] = static_cast<int>(i);
+        std::set<std::string> consumed;
+        auto blob_id = [&](const std::string& name) {
+            auto it = blob_index_.find(name);
+            if (it != blob_index_.end()) return it->second;
+            const int id = static_cast<int>(blob_index_.size());
+            blob_index_[name] = id;
+            blob_names_.push_back(name);
+            return id;
+        };
+        for (size_t i = 0; i < op_params_.size(); ++i) {
+            std::vector<int> in, out;
+            for (const std::string& b : op_params_[i].input_featmaps_) {
+                in.push_back(blob_id(b));
+                consumed.insert(b);
+                if (!produced_by.count(b) && std::find(input_names_.begin(), input_names_.end(), b) == input_names_.end())
+                    input_names_.push_back(b);
+            }
+            for (const std::string& b : op_params_[i].output_featmaps_) out.push_back(blob_id(b));
+            op_inputs_.push_back(in);
+            op_outputs_.push_back(out);
+        }
+        for (size_t i = 0; i < op_params_.size(); ++i)
+            for (const std::string& b : op_params_[i].output_featmaps_)
+                if (!consumed.count(b)) output_names_.push_back(b);
+        if (input_names_.empty()) LOG(FATAL) << "the topology has no input blob";
+        featmaps_.resize(blob_names_.size());
+    }
+
+    blob_map forward(const tensor_ptr& input) {
+        if (device_ >= 0) return forward_gpu(input);
+        return forward_cpu(input);
+    }
+
+    blob_map forward_cpu(const tensor_ptr&) {
+        NO_CPU;
+        return {};
+    }
+
+    blob_map forward_gpu(const tensor_ptr& input) {
+        if (device_ < 0) LOG(FATAL) << "forward_gpu on a pipeline created with device < 0";
+        const auto t0 = std::chrono::steady_clock::now();
+        blob_map results;
+        if (!try_fused(input, &results)) results = forward_layers(input);
+        if (profile_) {
+            exhip_sync(memory::device_context(device_));
+            last_ms_ = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            LOG(INFO) << name_ << ": forward " << last_ms_ << " ms (" << (last_fused_ ? "fused int8 plan" : "per-layer") << ")";
+        }
+        return results;
+    }
+
+    tensor_ptr get_featmap(std::string_view name) {
+        auto it = blob_index_.find(std::string(name));
+        if (it == blob_index_.end()) return nullptr;
+        return featmaps_[it->second];
+    }
+
+    bool profile_ = false;
+    bool fusion_ = true;
+    bool last_fused_ = false;
+    double last_ms_ = 0;
+
+private:
+    // ---------------------------------------------------------------- per-layer executor
+    blob_map forward_layers(const tensor_ptr& input) {
+        last_fused_ = false;
+        featmaps_[blob_index_[input_names_[0]]] = input;
+        for (size_t i = 0; i < operations_.size(); ++i) {
+            std::vector<tensor_ptr> in, out(op_outputs_[i].size());
+            for (int b : op_inputs_[i]) {
+                if (!featmaps_[b]) LOG(FATAL) << "layer " << op_params_[i].name_ << " reads blob " << blob_names_[b] << " before it is produced";
+                in.push_back(featmaps_[b]);
+            }
+            operations_[i]->forward_gpu(in, out);
+            for (size_t j = 0; j < out.size(); ++j) featmaps_[op_outputs_[i][j]] = out[j];
+        }
+        blob_map results;
+        for (const std::string& o : output_names_) results[o] = featmaps_[blob_index_[o]];
+        return results;
+    }
+
+    // ---------------------------------------------------------------- fused int8 executor
+    bool try_fused(const tensor_ptr& input, blob_map* results);
+    struct fused_plan;
+    std::shared_ptr<fused_plan> plan_;
+    bool fused_unsupported_ = false;
+
+    std::string name_ = "Unknown Pipeleine Name";
+    int device_ = -1;
+    std::vector<operation_param> op_params_;
+    std::vector<std::shared_ptr<operation<Dtype>>> operations_;
+    std::map<std::string, int> blob_index_;
+    std::vector<std::string> blob_names_;
+    std::vector<std::vector<int>> op_inputs_, op_outputs_;
+    std::vector<std::string> input_names_, output_names_;
+    std::vector<tensor_ptr> featmaps_;
+    int weights_mem_cost_ = 0;
+};
+
+// The plan: device buffers per value and the launches in execution order.
+template <typename Dtype>
+struct pipeline<Dtype>::impl::fused_plan {
+    std::vector<int> in_shape;
+    std::vector<dev_buffer> buffers;
+    std::vector<std::function<void()>> launches;
+    std::vector<std::pair<std::string, std::shared_ptr<tensor<float>>>> outputs;
+    const float** input_slot = nullptr;
+    const float* input_ptr = nullptr;
+};
+
+template <>
+bool pipeline<unsigned short>::impl::try_fused(const tensor_ptr&, blob_map*) { return false; }
+
+template <>
+bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results) {
+    if (!fusion_ || fused_unsupported_) return false;
+    const std::vector<int> shape = input->data_shape();
+    if (!plan_ || plan_->in_shape != shape) {
+        // ---- classify layers; anything outside the fusable set selects the per-layer executor ----
+        using conv_t = operation_convolution<float>;
+        const int n_ops = static_cast<int>(operations_.size());
+        auto give_up = [&]() { fused_unsupported_ = true; plan_.reset(); return false; };
+        if (input->order() != memory::NCHW) return give_up();
+        std::vector<int> alias(blob_names_.size());
+        for (size_t b = 0; b < alias.size(); ++b) alias[b] = static_cast<int>(b);
+        std::vector<char> kind(n_ops, 0);  // c conv, p max pool, s split, a add, r relu
+        for (int i = 0; i < n_ops; ++i) {
+            operation<float>* op = operations_[i].get();
+            if (dynamic_cast<operation_convolutiondepthwise<float>*>(op)) return give_up();
+            if (auto* c = dynamic_cast<conv_t*>(op)) {
+                if (!c->param().int8_quantization_ || c->group_ != 1 || c->stride_h_ != c->stride_w_ || c->dilation_h_ != 1 ||
+                    c->dilation_w_ != 1 || c->activation_type_ > 1 || c->weights_i8().empty())
+                    return give_up();
+                kind[i] = 'c';
+            } else if (auto* p = dynamic_cast<operation_pooling<float>*>(op)) {
+                if (p->type_ != 0 || p->global_pooling_) return give_up();
+                kind[i] = 'p';
+            } else if (dynamic_cast<operation_split<float>*>(op)) {
+                kind[i] = 's';
+                for (int o : op_outputs_[i]) alias[o] = alias[op_inputs_[i][0]];
+            } else if (auto* b = dynamic_cast<operation_binaryop<float>*>(op)) {
+                if (b->op_type_ != 0 || b->with_scalar_ || op_inputs_[i].size() != 2) return give_up();
+                kind[i] = 'a';
+            } else if (dynamic_cast<operation_relu<float>*>(op)) {
+                kind[i] = 'r';
+            } else {
+                return give_up();
+            }
+        }
+        auto root = [&](int b) { return alias[b]; };
+        // consumers of every value (through Split aliases)
+        std::vector<std::vector<int>> consumers(blob_names_.size());
+        for (int i = 0; i < n_ops; ++i)
+            if (kind[i] != 's')
+                for (int b : op_inputs_[i]) consumers[root(b)].push_back(i);
+        std::vector<char> is_output(blob_names_.size(), 0);
+        for (const std::string& o : output_names_) is_output[root(blob_index_[o])] = 1;
+
+        // ---- group layers into nodes: conv [+ add] [+ relu], max pool ----
+        struct node {
+            char kind;            // 'c' or 'p'
+            int op;               // conv / pool layer
+            int at;               // position in file order at which the node runs
+            int in_value, res_value = -1, out_value;
+            bool post_relu = false;
+        };
+        std::vector<node> nodes;
+        std::vector<char> absorbed(n_ops, 0);
+        for (int i = 0; i < n_ops; ++i) {
+            if (kind[i] == 'p') {
+                nodes.push_back({'p', i, i, root(op_inputs_[i][0]), -1, root(op_outputs_[i][0]), false});
+            } else if (kind[i] == 'c') {
+                node nd{'c', i, i, root(op_inputs_[i][0]), -1, root(op_outputs_[i][0]), false};
+                auto sole = [&](int v, char want) -> int {  // the single consumer of v if it is a layer of kind `want`
+                    if (is_output[v] || consumers[v].size() != 1) return -1;
+                    const int c = consumers[v][0];
+                    return (kind[c] == want && !absorbed[c]) ? c : -1;
+                };
+                int a = sole(nd.out_value, 'a');
+                if (a >= 0) {
+                    const int x = root(op_inputs_[a][0]), y = root(op_inputs_[a][1]);
+                    nd.res_value = (x == nd.out_value) ? y : x;
+                    if (nd.res_value == nd.out_value) return give_up();
+                    absorbed[a] = 1;
+                    nd.at = a;
+                    nd.out_value = root(op_outputs_[a][0]);
+                }
+                int r = sole(nd.out_value, 'r');
+                if (r >= 0) {
+                    absorbed[r] = 1;
+                    nd.at = r;
+                    nd.post_relu = true;
+                    nd.out_value = root(op_outputs_[r][0]);
+                }
+                nodes.push_back(nd);
+            }
+        }
+        for (int i = 0; i < n_ops; ++i)
+            if ((kind[i] == 'a' || kind[i] == 'r') && !absorbed[i]) return give_up();  // free-standing elementwise layers
+        std::stable_sort(nodes.begin(), nodes.end(), [](const node& a, const node& b) { return a.at < b.at; });
+
+        // ---- what each value must exist as ----
+        struct value_info {
+            bool need_f32 = false, need_i8 = false;
+            float fs = 0.f;
+            int n = 0, c = 0, h = 0, w = 0, cs = 0;
+            void *f32 = nullptr, *i8 = nullptr;
+            std::shared_ptr<tensor<float>> nchw;  // pipeline outputs
+        };
+        std::vector<value_info> vals(blob_names_.size());
+        const int in_value = root(blob_index_[input_names_[0]]);
+        for (const node& nd : nodes) {
+            if (nd.kind == 'c') {
+                auto* c = static_cast<conv_t*>(operations_[nd.op].get());
+                value_info& v = vals[nd.in_value];
+                const float fs = c->featmap_scale();
+                if (v.need_i8 && v.fs != fs) return give_up();  // one int8 copy per tensor
+                v.need_i8 = true;
+                v.fs = fs;
+                if (nd.res_value >= 0) vals[nd.res_value].need_f32 = true;
+            } else {
+                vals[nd.in_value].need_f32 = true;
+            }
+        }
+        if (vals[in_value].need_f32) return give_up();  // the network input is read by int8 convolutions only
+
+        // ---- shapes, buffers, launches ----
+        auto plan = std::make_shared<fused_plan>();
+        plan->in_shape = shape;
+        exhip_ctx* ctx = memory::device_context(device_);
+        const int dev = device_;
+        auto alloc = [&](size_t bytes) {
+            plan->buffers.emplace_back(dev, bytes);
+            return plan->buffers.back().ptr;
+        };
+        {
+            value_info& v = vals[in_value];
+            v.n = shape[0]; v.c = shape[1]; v.h = shape[2]; v.w = shape[3];
+            int kw_first = 0;
+            for (const node& nd : nodes)
+                if (nd.kind == 'c' && nd.in_value == in_value) kw_first = std::max(kw_first, static_cast<conv_t*>(operations_[nd.op].get())->kernel_size_w_);
+            v.cs = (v.c <= 4 && kw_first <= 8) ? 4 : pad_to(v.c, 32);
+            v.i8 = alloc(static_cast<size_t>(v.n) * v.h * v.w * v.cs);
+            int8_t* q = static_cast<int8_t*>(v.i8);
+            const value_info vi = v;
+            fused_plan* pl = plan.get();
+            plan->launches.push_back([=]() {
+                EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(ctx, pl->input_ptr, vi.n, vi.c, vi.h, vi.w, vi.fs, nullptr, vi.cs, q));
+            });
+        }
+        for (const node& nd : nodes) {
+            const value_info in = vals[nd.in_value];
+            value_info& out = vals[nd.out_value];
+            if (in.n == 0) return give_up();  // produced by something outside the plan
+            if (nd.kind == 'c') {
+                auto* c = static_cast<conv_t*>(operations_[nd.op].get());
+                if (in.c != c->input_channels() || !in.i8) return give_up();
+                const int ks = pad_to(c->output_channel_, 32);
+                exhip_conv_desc d = c->describe(in.n, in.h, in.w, in.cs, ks);
+                d.post_relu = nd.post_relu ? 1 : 0;
+                d.fs_out = out.need_i8 ? out.fs : 0.f;
+                int oh, ow;
+                EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
+                out.n = in.n; out.c = c->output_channel_; out.h = oh; out.w = ow; out.cs = ks;
+                const size_t elems = static_cast<size_t>(out.n) * oh * ow * ks;
+                if (out.need_i8) out.i8 = alloc(elems);
+                if (out.need_f32) out.f32 = alloc(elems * sizeof(float));
+                float* nchw = nullptr;
+                if (is_output[nd.out_value]) {
+                    out.nchw = std::make_shared<tensor<float>>(std::vector<int>{out.n, out.c, oh, ow}, dev);
+                    nchw = out.nchw->mutable_gpu_data();
+                }
+                const float* res = nullptr;
+                if (nd.res_value >= 0) {
+                    const value_info& r = vals[nd.res_value];
+                    if (!r.f32 || r.n != out.n || r.h != oh || r.w != ow || r.cs != ks) return give_up();
+                    res = static_cast<const float*>(r.f32);
+                }
+                const void* wp = c->packed_weights(EXHIP_I8, d);
+                const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
+                const int8_t* x = static_cast<const int8_t*>(in.i8);
+                int8_t* yq = static_cast<int8_t*>(out.i8);
+                float* yf = static_cast<float*>(out.f32);
+                if (!yq && !yf && !nchw) yf = static_cast<float*>(out.f32 = alloc(elems * sizeof(float)));  // dead value: still computed
+                plan->launches.push_back([=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, res, yq, yf, nchw, nullptr)); });
+            } else {
+                auto* p = static_cast<operation_pooling<float>*>(operations_[nd.op].get());
+                if (!in.f32) return give_up();
+                int kh, kw, sh, sw, pt, pb, pl, pr, oh, ow;
+                p->geometry(in.h, in.w, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &oh, &ow);
+                out.n = in.n; out.c = in.c; out.h = oh; out.w = ow; out.cs = in.cs;
+                const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
+                if (out.need_i8) out.i8 = alloc(elems);
+                if (out.need_f32 || is_output[nd.out_value] || !out.need_i8) out.f32 = alloc(elems * sizeof(float));
+                const float* x = static_cast<const float*>(in.f32);
+                float* yf = static_cast<float*>(out.f32);
+                int8_t* yq = static_cast<int8_t*>(out.i8);
+                const value_info o = out;
+                plan->launches.push_back([=]() {
+                    EXHIP_FATAL(exhip_maxpool2d_nhwc_f32(ctx, x, yf, yq, o.fs, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl));
+                });
+                if (is_output[nd.out_value]) {
+                    out.nchw = std::make_shared<tensor<float>>(std::vector<int>{out.n, out.c, oh, ow}, dev);
+                    float* nchw = out.nchw->mutable_gpu_data();
+                    plan->launches.push_back([=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, yf, o.n, o.c, oh, ow, o.cs, nchw)); });
+                }
+            }
+        }
+        for (const std::string& o : output_names_) {
+            const value_info& v = vals[root(blob_index_[o])];
+            if (!v.nchw) return give_up();
+            plan->outputs.push_back({o, v.nchw});
+        }
+        plan_ = plan;
+    }
+    plan_->input_ptr = input->gpu_data();
+    for (auto& launch : plan_->launches) launch();
+    last_fused_ = true;
+    for (auto& kv : plan_->outputs) {
+        kv.second->mutable_gpu_data();  // the kernels just wrote it: the device copy is the newest
+        (*results)[kv.first] = kv.second;
+        featmaps_[blob_index_[kv.first]] = kv.second;
+    }
+    return true;
+}
+
+// ---------------------------------------------------------------- public wrappers
+namespace {
+std::vector<std::string> read_lines(std::string_view path) {
+    std::vector<std::string> lines;
+    std::ifstream in{std::string(path)};
+    std::string line;
+    while (in.is_open() && std::getline(in, line)) lines.push_back(line);
+    return lines;
+}
+}  // namespace
+
+template <typename Dtype>
+pipeline<Dtype>::pipeline(std::string_view param_file, std::string_view model_file, int device)
+    : impl_(new impl(read_lines(param_file), model_file, device)) {}
+template <typename Dtype>
+pipeline<Dtype>::pipeline(std::string_view param_file, int device) : impl_(new impl(read_lines(param_file), std::string_view(), device)) {}
+template <typename Dtype>
+pipeline<Dtype>::pipeline(const std::vector<std::string>& hardcode_params, std::string_view model_file, int device)
+    : impl_(new impl(hardcode_params, model_file, device)) {}
+template <typename Dtype>
+pipeline<Dtype>::~pipeline() { delete impl_; }
+template <typename Dtype>
+typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward(const std::shared_ptr<memory::tensor<Dtype>>& t) { return impl_->forward(t); }
+template <typename Dtype>
+typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward_cpu(const std::shared_ptr<memory::tensor<Dtype>>& t) { return impl_->forward_cpu(t); }
+template <typename Dtype>
+typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward_gpu(const std::shared_ptr<memory::tensor<Dtype>>& t) { return impl_->forward_gpu(t); }
+template <typename Dtype>
+std::shared_ptr<memory::tensor<Dtype>> pipeline<Dtype>::get_featmap(std::string_view name) { return impl_->get_featmap(name); }
+template <typename Dtype>
+void pipeline<Dtype>::enable_profiler() { impl_->profile_ = true; }
+template <typename Dtype>
+void pipeline<Dtype>::disable_profiler() { impl_->profile_ = false; }
+template <typename Dtype>
+void pipeline<Dtype>::set_fusion(bool on) { impl_->fusion_ = on; }
+template <typename Dtype>
+bool pipeline<Dtype>::fused() const { return impl_->last_fused_; }
+template <typename Dtype>
+double pipeline<Dtype>::last_forward_ms() const { return impl_->last_ms_; }
+template <typename Dtype>
+std::string pipeline<Dtype>::version() { return "1.0.0"; }
+
+template class pipeline<float>;
+template class pipeline<unsigned short>;
+
+}  // namespace excalibur
+}  // namespace glasssix

@@ -1,0 +1,90 @@
+"""ctypes binding of the host-side pipeline (include/excalibur_capi.h): Excalibur's `pipeline<Dtype>` API on the MI355X
+backend. Loads excalibur_amd/host/lib/libexcalibur_hip.so and fails loudly if it is missing."""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "host", "lib", "libexcalibur_hip.so")
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is not built; run `make -C excalibur_amd/csrc && make -C excalibur_amd/host`")
+        from . import hip
+        hip.lib()  # libexhip.so first: the host library links against it
+        L = ctypes.CDLL(LIB_PATH)
+        L.exc_pipeline_create.restype = ctypes.c_void_p
+        L.exc_pipeline_create.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
+        L.exc_pipeline_destroy.argtypes = [ctypes.c_void_p]
+        L.exc_pipeline_set_fusion.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        L.exc_pipeline_last_fused.argtypes = [ctypes.c_void_p]
+        L.exc_pipeline_set_input.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
+        L.exc_pipeline_run.argtypes = [ctypes.c_void_p]
+        L.exc_pipeline_sync.argtypes = [ctypes.c_void_p]
+        L.exc_pipeline_forward.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
+        L.exc_pipeline_get.restype = ctypes.c_long
+        L.exc_pipeline_get.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_long,
+                                       ctypes.POINTER(ctypes.c_int)]
+        L.exc_registered_operations.restype = ctypes.c_size_t
+        L.exc_registered_operations.argtypes = [ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
+        _lib = L
+    return _lib
+
+
+def registered_operations(dtype="f32"):
+    buf = ctypes.create_string_buffer(4096)
+    lib().exc_registered_operations(0 if dtype == "f32" else 1, buf, 4096)
+    return buf.value.decode().split()
+
+
+class Pipeline:
+    """pipeline<float> (dtype 'f32') or pipeline<unsigned short> (dtype 'f16') on HIP device `device`."""
+
+    def __init__(self, topology, model_path="", device=0, dtype="f32", fusion=True):
+        self.dtype = np.float32 if dtype == "f32" else np.uint16
+        self.h = lib().exc_pipeline_create(topology.encode(), (model_path or "").encode(), device, 0 if dtype == "f32" else 1)
+        lib().exc_pipeline_set_fusion(self.h, int(fusion))
+
+    def close(self):
+        if self.h:
+            lib().exc_pipeline_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
+
+    def set_input(self, x):
+        x = np.ascontiguousarray(x, self.dtype)
+        assert x.ndim == 4
+        lib().exc_pipeline_set_input(self.h, x.ctypes.data, (ctypes.c_int * 4)(*x.shape))
+
+    def run(self):
+        lib().exc_pipeline_run(self.h)
+
+    def sync(self):
+        rc = lib().exc_pipeline_sync(self.h)
+        if rc:
+            raise RuntimeError(f"exhip_sync failed ({rc})")
+
+    def forward(self, x):
+        self.set_input(x)
+        self.run()
+        self.sync()
+
+    @property
+    def fused(self):
+        return bool(lib().exc_pipeline_last_fused(self.h))
+
+    def get(self, name):
+        shape = (ctypes.c_int * 4)()
+        n = lib().exc_pipeline_get(self.h, name.encode(), None, 0, shape)
+        if n < 0:
+            raise KeyError(name)
+        out = np.empty(tuple(shape), self.dtype)
+        lib().exc_pipeline_get(self.h, name.encode(), out.ctypes.data, out.size, shape)
+        return out

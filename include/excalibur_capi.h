@@ -1,0 +1,38 @@
+/* C ABI over the host-side pipeline of this backend, for callers without a C++ toolchain (the Python tests and
+ * bench.py bind it with ctypes). It wraps glasssix::excalibur::pipeline<Dtype>, whose C++ interface is the
+ * reference's own (include/Excalibur/pipeline.hpp:17-47): construct from topology lines and a model file with a
+ * device ordinal, forward() one NCHW input, read output blobs by name.
+ * Failures inside the pipeline follow the reference's policy: a message on stderr and std::terminate(). */
+#ifndef EXCALIBUR_CAPI_H_
+#define EXCALIBUR_CAPI_H_
+#include <stddef.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct exc_pipeline exc_pipeline;
+
+/* topology: the `.phai` text ('\n' separated); model_path: a `.racy` file or "" for dummy weights;
+ * device: HIP ordinal (>= 0); dtype: 0 = pipeline<float>, 1 = pipeline<unsigned short> (fp16 storage). */
+exc_pipeline* exc_pipeline_create(const char* topology, const char* model_path, int device, int dtype);
+void exc_pipeline_destroy(exc_pipeline* p);
+/* 1 (default): int8 convolution chains run as one fused plan; 0: every layer through forward_gpu on NCHW blobs. */
+void exc_pipeline_set_fusion(exc_pipeline* p, int on);
+int exc_pipeline_last_fused(exc_pipeline* p);
+/* Copies a host NCHW tensor into the pipeline's input blob and uploads it to the device. */
+int exc_pipeline_set_input(exc_pipeline* p, const void* input, const int shape[4]);
+/* pipeline::forward on the resident input; kernels are queued, not awaited. */
+int exc_pipeline_run(exc_pipeline* p);
+int exc_pipeline_sync(exc_pipeline* p);
+/* set_input + run + sync */
+int exc_pipeline_forward(exc_pipeline* p, const void* input, const int shape[4]);
+/* Copies output blob (or, with fusion off, any feature map) `name` to `out` if it fits in `capacity` elements;
+ * returns its element count (-1 if unknown) and its shape. */
+long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, long capacity, int shape[4]);
+/* Newline-separated list of registered operator class names for a dtype. Returns the length needed. */
+size_t exc_registered_operations(int dtype, char* buf, size_t len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,135 @@
+"""The host-side mirror of the reference's operator / pipeline API on the GPU: single layers and whole topologies
+loaded from `.phai` text + `.racy` blobs through pipeline<Dtype>(lines, model_file, device = 0), against the golden
+fixtures of the compiled reference and the CPU restatement."""
+import glob
+import os
+import tempfile
+
+import numpy as np
+import pytest
+
+from excalibur_amd import pipeline as xp
+from excalibur_amd.resnet18 import ResNet18Int8
+from oracle import port
+from tests import cases, netref
+from tests.golden.make_fixtures import load_case
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")))
+TOLERANT = ("conv_f32", "fc_")
+
+
+def run_case(case, dtype="f32"):
+    if case["op"] in ("eltwise", "binaryop_add"):
+        topo, x = cases.multi_input_topology(case)
+        blob = b""
+    else:
+        topo, blob, xs, _ = cases.reference_io(case)
+        x = xs[0]
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        f.write(blob if blob else b"\0\0\0\0")
+        path = f.name
+    try:
+        p = xp.Pipeline(topo, path, 0, dtype)
+        p.forward(x)
+        out = p.get("out")
+        p.close()
+        return out
+    finally:
+        os.unlink(path)
+
+
+# the host layer registers Split_Slice only as far as the hot path needs it: multi-input cases use it to cut operands
+MULTI = ("eltwise", "binaryop")
+
+
+@pytest.mark.parametrize("name", [n for n in NAMES if not n.startswith("f16_") and not n.startswith(MULTI)])
+def test_single_layer_topologies_match_reference_fixtures(name):
+    case, expected = load_case(os.path.join(GOLDEN, name + ".npz"))
+    got = run_case(case)
+    assert got.shape == expected.shape
+    if name.startswith(TOLERANT):
+        assert cases.check_value(got, expected, 1e-4) == 0
+    else:
+        assert np.array_equal(got, expected)
+
+
+@pytest.mark.parametrize("name", [n for n in NAMES if n.startswith("f16_")])
+def test_fp16_pipeline_matches_reference_fixtures(name):
+    case, expected = load_case(os.path.join(GOLDEN, name + ".npz"))
+    got = run_case(case, "f16")
+    assert got.shape == expected.shape
+    assert cases.check_value(got.view(np.float16).astype(np.float32), expected.view(np.float16).astype(np.float32), 2e-3) == 0
+
+
+@pytest.mark.parametrize("fusion", [False, True])
+def test_resnet18_topology_through_the_pipeline(fusion):
+    net = ResNet18Int8(seed=21, calib_hw=32)
+    x = np.random.default_rng(22).uniform(-1, 1, (2, 3, 96, 96)).astype(np.float32)
+    want, blobs = netref.oracle_forward(net, x)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        net.write_model(path)
+        p = xp.Pipeline(net.topology(), path, 0, "f32", fusion=fusion)
+        p.forward(x)
+        assert p.fused == fusion
+        got = p.get(net.output)
+        assert np.array_equal(got, want)
+        if not fusion:  # every intermediate blob exists as a float NCHW tensor, as in the reference
+            assert np.array_equal(p.get("pool1"), blobs["pool1"])
+            assert np.array_equal(p.get("l3b1_out"), blobs["l3b1_out"])
+        # a second input of another shape rebuilds the plan
+        x2 = np.random.default_rng(23).uniform(-1, 1, (1, 3, 64, 64)).astype(np.float32)
+        p.forward(x2)
+        assert np.array_equal(p.get(net.output), netref.oracle_forward(net, x2)[0])
+        p.close()
+    finally:
+        os.unlink(path)
+
+
+def test_mixed_topology_falls_back_to_per_layer():
+    """conv(int8) -> global average pool -> inner product: not a fusable chain; runs layer by layer."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(31)
+    c = cases.conv_i8_case(32, 2, 16, 12, 12, 32, 3, 1, 1)
+    wfc = r.normal(0, 0.1, (10, 32)).astype(np.float32)
+    bfc = r.normal(0, 0.1, (10,)).astype(np.float32)
+    lines = [mf.conv_line("Convolution", "c", "data", "a", 32, 3, 1, 1, True, c["wt"].size, 1, int8=True, act=1),
+             mf.pool_line("gap", "a", "b", 1, global_pool=True),
+             f"InnerProduct fc 1 1 b out 0=10 1=1 2={wfc.size}"]
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        f.write(mf.conv_blob_i8(c["wt"], c["bias"], c["ws"], c["fs"]) + mf.fc_blob_f32(wfc, bfc))
+        path = f.name
+    try:
+        p = xp.Pipeline(mf.topology(lines), path, 0)
+        p.forward(c["x"])
+        assert not p.fused
+        a = cases.oracle_eval(c)
+        b = port.pool2d(a, port.POOL_AVE, global_pool=True)
+        want = port.innerproduct(b, wfc, bfc)
+        assert np.array_equal(p.get("a"), a)
+        assert cases.check_value(p.get("out"), want, 1e-4) == 0
+        p.close()
+    finally:
+        os.unlink(path)
+
+
+@pytest.mark.parametrize("layer,evaluate", [
+    ("Eltwise e 2 1 ra b out 0=1", lambda a, b: port.eltwise([a, b], port.ELT_SUM)),
+    ("Eltwise e 2 1 ra b out 0=1 -23301=3,0.5,-1.25", lambda a, b: port.eltwise([a, b], port.ELT_SUM, [0.5, -1.25])),
+    ("Eltwise e 2 1 ra b out 0=2", lambda a, b: port.eltwise([a, b], port.ELT_MAX)),
+    ("Eltwise e 2 1 ra b out 0=0", lambda a, b: port.eltwise([a, b], port.ELT_PROD)),
+    ("BinaryOp e 2 1 ra b out 0=0", lambda a, b: port.binaryop_add(a, b)),
+])
+def test_two_input_layers_through_split_aliasing(layer, evaluate):
+    """Split hands one blob to two consumers (aliasing, as in the reference); the operands are relu(x) and x."""
+    from excalibur_amd import modelfile as mf
+    x = np.random.default_rng(41).uniform(-2, 2, (2, 5, 9, 11)).astype(np.float32)
+    lines = ["Split s 1 2 data a b", "ReLU r 1 1 a ra", layer]
+    p = xp.Pipeline(mf.topology(lines), "", 0)
+    p.forward(x)
+    assert np.array_equal(p.get("out"), evaluate(port.relu(x), x))
+    p.close()
