@@ -79,6 +79,7 @@ struct ConvParams {
     unsigned img_bytes;       // bytes of one input image (buffer range for the bounds-checked loads)
     unsigned magic_iw, magic_pw; // ceil(2^32 / IW), ceil(2^32 / PW): exact quotients by one multiply-high for operands < 2^16
     int vp_shift;             // log2 of the 16-byte vectors per staged pixel
+    int prefetch_res;         // fused epilogue: touch the shortcut tensor before the MFMA loop (short reductions only)
 };
 
 template <int DT> struct Acc { typedef v16i type; };
@@ -373,7 +374,26 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
     };
 
     stamp(1);
+    int prefetched[2] = {0, 0};
     if constexpr (EPI == 1) {
+        // Touch this group's part of the float32 shortcut tensor now (one dword per 128-byte line): the lines travel
+        // from HBM into L2 while the MFMA loop runs, so the epilogue's reads do not start cold. The two values are
+        // only "used" at the end of the kernel, which keeps the loads in flight without waiting for them here.
+        if (p.prefetch_res) {
+            constexpr int lines_px = (TM * 4) >> 7;                    // 128-byte lines per pixel of this group's slab
+            const int total = p.PH * p.PW * lines_px;                  // <= 2 * THREADS for every variant
+            const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<void*>(p.residual), 0, (int)((unsigned)p.N * (unsigned)(p.OH * p.OW) * (unsigned)p.K * 4u), kRsrcWord3);
+#pragma unroll
+            for (int r = 0; r < 2; ++r) {
+                const int i = tid + r * THREADS;
+                const int pp = i / lines_px, ln = i - pp * lines_px;
+                const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
+                const bool ok = i < total && oy0 + py < p.OH && ox0 + px < p.OW && kt * TM * 4 + ln * 128 < p.K * 4;
+                const unsigned off = ((unsigned)(n * p.OH + oy0 + py) * p.OW + ox0 + px) * (unsigned)p.K * 4u + kt * TM * 4 + ln * 128;
+                prefetched[r] = __builtin_amdgcn_raw_buffer_load_b32(rr, ok ? (int)off : (int)0xFFFFFF00u, 0, 0);
+            }
+        }
         // per-channel scale and bias of this group's channels, fetched now so that the epilogue finds them in LDS
         if (tid < 2 * TM) {
             const int c = tid < TM ? tid : tid - TM;
@@ -632,6 +652,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
             }
         }
     }
+    __asm__ volatile("" ::"v"(prefetched[0]), "v"(prefetched[1]));
     stamp(8);
 }
 
@@ -837,6 +858,8 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p) {
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = !p.y_nchw && !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
                            out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
+        // worth it only when the MFMA loop is too short to hide the shortcut's first-touch latency by itself
+        p.prefetch_res = fused && p.residual && (long long)d->c_stride * d->kh * d->kw < 1024;
         if (fused) {
             if (pl.packed) return launch_variant<DT, true, 1>(ctx, pl, p, (int)grid);
             return launch_variant<DT, false, 1>(ctx, pl, p, (int)grid);
