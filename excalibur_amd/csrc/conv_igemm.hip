@@ -21,6 +21,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <type_traits>
 #include <vector>
 
 #include "common.h"
@@ -78,8 +79,12 @@ struct ConvParams {
     int b_align;              // alignment of B fragment reads in packed-row form (4, 8 or 16)
     unsigned img_bytes;       // bytes of one input image (buffer range for the bounds-checked loads)
     unsigned magic_iw, magic_pw; // ceil(2^32 / IW), ceil(2^32 / PW): exact quotients by one multiply-high for operands < 2^16
+    unsigned magic_mpw;          // ceil(2^32 / MPW)
     int vp_shift;             // log2 of the 16-byte vectors per staged pixel
     int prefetch_res;         // fused epilogue: touch the shortcut tensor before the MFMA loop (short reductions only)
+    int tile_dy, tile_dx;     // output pixels between the origins of neighbouring patches (PH, PW unless pooled)
+    int tile_oy, tile_ox;     // the first patch starts this many pixels before output pixel 0 (pooled form: the pool's padding)
+    int MPH, MPW, POH, POW;   // pooled form: pooled pixels per patch and pooled image size
 };
 
 template <int DT> struct Acc { typedef v16i type; };
@@ -134,7 +139,9 @@ __device__ __forceinline__ float fast_activation(float v, int act) {
     return v;
 }
 
-template <int DT, int MT, int NT, int WM, int WN, bool PACKED, int EPI>
+// KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
+// turns every LDS fragment address of a row into an immediate offset; KWE == 0 keeps them as run-time values.
+template <int DT, int MT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
 __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvParams p) {
     constexpr int THREADS = 64 * WM * WN;
     constexpr int TM = 32 * MT * WM;
@@ -169,7 +176,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
     t /= p.tiles_x;
     const int ty = t % p.tiles_y;
     const int n = t / p.tiles_y;
-    const int oy0 = ty * p.PH, ox0 = tx * p.PW;
+    const int oy0 = ty * p.tile_dy - p.tile_oy, ox0 = tx * p.tile_dx - p.tile_ox;
     const int iy0 = oy0 * p.S * p.tile_step - p.PT, ix0 = ox0 * p.S * p.tile_step - p.PL;
 
     // Bounds-checked buffer views: any offset at or past the range reads as zero, which is how halo
@@ -219,7 +226,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
         ppy[j] = py;
         ppx[j] = px;
-        if (ok && oy0 + py < p.OH && ox0 + px < p.OW) pvalid |= 1 << j;
+        if (ok && (unsigned)(oy0 + py) < (unsigned)p.OH && (unsigned)(ox0 + px) < (unsigned)p.OW) pvalid |= 1 << j;
         boff[j] = py * p.S * p.lds_row_b + px * p.S * p.lds_pix_b + (lane >> 5) * 16;
     }
     const int aoff = wm * MT * 1024 + lane * 16;
@@ -317,54 +324,102 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
             if (more && next_chunk) load_act(cc + 1);
         }
         // ---- MFMA over this stage: k-steps in (row, tap, channel) order, fragments fetched one step ahead ----
-        const int nk = stage_rows(rg) * p.KWe * p.KS;
         const char* wl = lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff;
         const char* al = lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b;
-        int q = 0, j = 0;          // tap column and channel k-step of the fragments being fetched
-        int koff = 0;              // their byte offset inside the activation tile
         v4i af[2][MT], bf[2][NT];
-        auto fetch = [&](int buf) {
-#pragma unroll
-            for (int m = 0; m < MT; ++m) af[buf][m] = lds_read16(wl + m * 1024);
-#pragma unroll
-            for (int nn = 0; nn < NT; ++nn) {
-                if constexpr (PACKED) bf[buf][nn] = lds_read16_unaligned(al + koff + boff[nn], p.b_align);
-                else bf[buf][nn] = lds_read16(al + koff + boff[nn]);
-            }
-            wl += (TM / 32) * 1024;
-            // advance (j, q, row) and the tile offset
-            if (++j == p.KS) {
-                j = 0;
-                koff += p.lds_pix_b - (p.KS - 1) * 32;
-                if (++q == p.KWe) {
-                    q = 0;
-                    koff += p.lds_row_b - p.KWe * p.lds_pix_b;
-                }
-            } else {
-                koff += 32;
-            }
-        };
         auto compute = [&](int buf) {
 #pragma unroll
             for (int m = 0; m < MT; ++m)
 #pragma unroll
                 for (int nn = 0; nn < NT; ++nn) mma<DT>(acc[m][nn], af[buf][m], bf[buf][nn]);
         };
-        fetch(0);
-        int it = 0;
-        for (; it + 2 <= nk - 1; it += 2) {
-            fetch(1);
-            compute(0);
-            fetch(0);
-            compute(1);
-        }
-        // 1 or 2 k-steps left; buffer 0 holds step `it`
-        if (it + 1 < nk) {
-            fetch(1);
-            compute(0);
-            compute(1);
+        if constexpr (KWE > 0) {
+            constexpr int NS = KWE * KSC;             // k-steps per filter row
+            constexpr int STEPB = (TM / 32) * 1024;   // weight bytes per k-step
+            constexpr int PIXB = PACKED ? 0 : KSC * 32 + 16;
+            const int nrows = stage_rows(rg);
+            const char* ar[NT];
+#pragma unroll
+            for (int nn = 0; nn < NT; ++nn) ar[nn] = al + boff[nn];
+            auto fetch_at = [&](int buf, const char* wrow, const char* const (&arow)[NT], int s_) {
+                const int q_ = s_ / KSC, j_ = s_ % KSC;
+#pragma unroll
+                for (int m = 0; m < MT; ++m) af[buf][m] = lds_read16(wrow + s_ * STEPB + m * 1024);
+#pragma unroll
+                for (int nn = 0; nn < NT; ++nn) {
+                    if constexpr (PACKED) bf[buf][nn] = lds_read16_unaligned(arow[nn], p.b_align);
+                    else bf[buf][nn] = lds_read16(arow[nn] + q_ * PIXB + j_ * 32);
+                }
+            };
+            // One filter row, entered with k-step 0 already in buffer P0; leaves the next row's k-step 0 in
+            // buffer (P0 + NS) & 1 when there is a next row.
+            auto row = [&](auto p0, bool has_next) {
+                constexpr int P0 = decltype(p0)::value;
+                const char* nr[NT];
+#pragma unroll
+                for (int nn = 0; nn < NT; ++nn) nr[nn] = ar[nn] + p.lds_row_b;
+#pragma unroll
+                for (int s_ = 0; s_ < NS; ++s_) {
+                    if (s_ + 1 < NS) fetch_at((P0 + s_ + 1) & 1, wl, ar, s_ + 1);
+                    else if (has_next) fetch_at((P0 + s_ + 1) & 1, wl + NS * STEPB, nr, 0);
+                    compute((P0 + s_) & 1);
+                }
+                wl += NS * STEPB;
+#pragma unroll
+                for (int nn = 0; nn < NT; ++nn) ar[nn] = nr[nn];
+            };
+            fetch_at(0, wl, ar, 0);
+            if constexpr (NS % 2 == 0) {
+                for (int r = 0; r < nrows; ++r) row(std::integral_constant<int, 0>{}, r + 1 < nrows);
+            } else {
+                int r = 0;
+                for (; r + 1 < nrows; r += 2) {
+                    row(std::integral_constant<int, 0>{}, true);
+                    row(std::integral_constant<int, 1>{}, r + 2 < nrows);
+                }
+                if (r < nrows) row(std::integral_constant<int, 0>{}, false);
+            }
         } else {
-            compute(0);
+            const int nk = stage_rows(rg) * p.KWe * p.KS;
+            int q = 0, j = 0;          // tap column and channel k-step of the fragments being fetched
+            int koff = 0;              // their byte offset inside the activation tile
+            auto fetch = [&](int buf) {
+#pragma unroll
+                for (int m = 0; m < MT; ++m) af[buf][m] = lds_read16(wl + m * 1024);
+#pragma unroll
+                for (int nn = 0; nn < NT; ++nn) {
+                    if constexpr (PACKED) bf[buf][nn] = lds_read16_unaligned(al + koff + boff[nn], p.b_align);
+                    else bf[buf][nn] = lds_read16(al + koff + boff[nn]);
+                }
+                wl += (TM / 32) * 1024;
+                // advance (j, q, row) and the tile offset
+                if (++j == p.KS) {
+                    j = 0;
+                    koff += p.lds_pix_b - (p.KS - 1) * 32;
+                    if (++q == p.KWe) {
+                        q = 0;
+                        koff += p.lds_row_b - p.KWe * p.lds_pix_b;
+                    }
+                } else {
+                    koff += 32;
+                }
+            };
+            fetch(0);
+            int it = 0;
+            for (; it + 2 <= nk - 1; it += 2) {
+                fetch(1);
+                compute(0);
+                fetch(0);
+                compute(1);
+            }
+            // 1 or 2 k-steps left; buffer 0 holds step `it`
+            if (it + 1 < nk) {
+                fetch(1);
+                compute(0);
+                compute(1);
+            } else {
+                compute(0);
+            }
         }
         if (more) {
             if (next_chunk) store_act(lds_a0 + ((cc + 1) & (p.act_bufs - 1)) * p.lds_act_b);
@@ -394,6 +449,8 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                 prefetched[r] = __builtin_amdgcn_raw_buffer_load_b32(rr, ok ? (int)off : (int)0xFFFFFF00u, 0, 0);
             }
         }
+    }
+    if constexpr (EPI >= 1) {
         // per-channel scale and bias of this group's channels, fetched now so that the epilogue finds them in LDS
         if (tid < 2 * TM) {
             const int c = tid < TM ? tid : tid - TM;
@@ -535,6 +592,77 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                 }
             }
             wave_sync();  // the tiles and the table are rewritten by the next column block
+        }
+    } else if constexpr (EPI == 2) {
+        // Convolution followed by a 3x3 stride-2 max pool (int8 path, TM == 64): the patch is (2 MPH + 1) x (2 MPW + 1)
+        // convolution pixels, written as float32 into one LDS tile [pixel][64 channels]; pixels outside the
+        // convolution's output hold -inf, which is how the pool's own padding drops out of the maximum. After a
+        // barrier the MPH x MPW pooled pixels are formed from the tile and leave as NHWC float32 and / or int8.
+        static_assert(TM == 64, "pooled epilogue: one 64-channel slab per group");
+        char* const pool = smem + kSbBytes;
+        const int px_l = lane & 31, hh = lane >> 5;
+        const int npatch = p.PH * p.PW;
+        const float ninf = -__builtin_inff();
+#pragma unroll
+        for (int nn = 0; nn < NT; ++nn) {
+            const int pp = (wn * NT + nn) * 32 + px_l;
+            const bool valid = (pvalid >> nn) & 1;
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                const int c0 = m * 32 + hh * 16;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const v4f s4 = *reinterpret_cast<const v4f*>(lds_sb + c0 + e4 * 4);
+                    const v4f b4 = *reinterpret_cast<const v4f*>(lds_sb + 128 + c0 + e4 * 4);
+                    v4f v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e], b4[e]);
+                        if (p.act == 1) v[e] = __builtin_fmaxf(v[e], 0.f);
+                        v[e] = valid ? v[e] : ninf;
+                    }
+                    if (pp < npatch) *reinterpret_cast<v4f*>(pool + pp * kEpiRowF + (c0 + e4 * 4) * 4) = v;
+                }
+            }
+        }
+        __syncthreads();
+        stamp(6);
+        const unsigned out_px = (unsigned)p.N * (unsigned)(p.POH * p.POW);
+        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(p.y_q, 0, (int)(out_px * (unsigned)p.K), kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_nhwc, 0, (int)(out_px * (unsigned)p.K * 4u), kRsrcWord3);
+        const bool has_f = p.y_nhwc != nullptr, has_q = p.y_q != nullptr;
+        const int items = p.MPH * p.MPW * 16;  // 4-channel vectors of the pooled patch
+        for (int i = tid; i < items; i += THREADS) {
+            const int pq = i >> 4, part = i & 15;
+            const int pyy = fast_div(pq, p.magic_mpw), pxx = pq - pyy * p.MPW;
+            const int gy = ty * p.MPH + pyy, gx = tx * p.MPW + pxx;
+            const char* w0 = pool + ((2 * pyy) * p.PW + 2 * pxx) * kEpiRowF + part * 16;
+            v4f best = *reinterpret_cast<const v4f*>(w0);
+#pragma unroll
+            for (int dr = 0; dr < 3; ++dr)
+#pragma unroll
+                for (int dc = 0; dc < 3; ++dc) {
+                    if (dr == 0 && dc == 0) continue;
+                    const v4f t = *reinterpret_cast<const v4f*>(w0 + (dr * p.PW + dc) * kEpiRowF);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) best[e] = __builtin_fmaxf(best[e], t[e]);
+                }
+            const bool ok = gy < p.POH && gx < p.POW;
+            const unsigned elem = ((unsigned)(n * p.POH + gy) * (unsigned)p.POW + gx) * (unsigned)p.K + kt * TM + part * 4;
+            const unsigned off = ok ? elem : kEpiInvalid;
+            if (has_f) {
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, best), rf, (int)(off * 4u), 0, 0);
+            }
+            if (has_q) {
+                int b[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float t = best[e] * p.fs_out;
+                    b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
+                }
+                __builtin_amdgcn_raw_buffer_store_b32((b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24),
+                                                      rq, (int)off, 0, 0);
+            }
         }
     } else {
         // General form: every output kind, ragged channel counts, direct per-lane accesses.
@@ -681,12 +809,16 @@ struct Plan {
     int act_bufs, w_bufs;
     int tiles_x, tiles_y, ktiles;
     int OH, OW;
-    size_t lds_bytes() const {  // staging buffers, reused by the epilogue's per-wave tiles
+    int MPH, MPW;  // pooled form: pooled pixels per patch (0 otherwise); the patch is then (2 MPH + 1) x (2 MPW + 1)
+    size_t lds_bytes() const {  // staging buffers, reused by the epilogue's tiles
         const size_t staging = (size_t)act_bufs * lds_act_b + (size_t)w_bufs * lds_w_b;
-        const size_t epilogue = (size_t)(threads / 64) * kEpiWaveBytes;
+        const size_t epilogue = MPH ? (size_t)PH * PW * kEpiRowF : (size_t)(threads / 64) * kEpiWaveBytes;
         return kSbBytes + (staging > epilogue ? staging : epilogue);
     }
 };
+
+// A 3x3 stride-2 max pool fused behind the convolution: its top / left padding and its output size.
+struct PoolSpec { int pt, pl, oh, ow; };
 
 int validate(const exhip_conv_desc* d, int dt) {
     EXHIP_REQUIRE(d, "conv: NULL descriptor");
@@ -705,7 +837,7 @@ int validate(const exhip_conv_desc* d, int dt) {
 
 // Picks the tile variant, patch shape and staging split for a layer. Maximises the share of issued
 // MFMA work that is useful, subject to the per-thread staging limits and the LDS size.
-int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
+int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool = nullptr) {
     int rc = validate(d, dt);
     if (rc) return rc;
     Plan best;
@@ -718,6 +850,7 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
         if (force_variant >= 0 && variant != force_variant) continue;
+        if (pool && variant != 0) continue;  // the pooled epilogue holds one 64-channel slab per group
         if (packed && chunk_opt == 64) continue;
         if (!packed && cb % chunk_opt != 0) continue;
         const int TM = kVariants[variant].TM, TN = kVariants[variant].TN;
@@ -751,10 +884,9 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
         p.lds_w_b = p.RS * row_w_b;
         p.act_bufs = p.n_chunks > 1 ? 2 : 1;
         p.w_bufs = p.n_chunks * p.n_rg > 1 ? 2 : 1;
-        for (int PW = 1; PW <= TN && PW <= OW; ++PW) {
-            int PH = TN / PW;
-            if (PH > OH) PH = OH;
-            if (PH < 1) continue;
+        p.MPH = p.MPW = 0;
+        // fills the patch-dependent fields; false when the patch exceeds a staging or LDS limit
+        auto shape_patch = [&](int PH, int PW) {
             p.PH = PH;
             p.PW = PW;
             p.IH = (PH - 1) * p.S + d->kh;
@@ -765,32 +897,57 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out) {
                 p.lds_row_b = (p.IW * cb + 15) / 16 * 16;
                 const int step = p.S * cb;
                 p.b_align = step % 16 == 0 ? 16 : step % 8 == 0 ? 8 : 4;
-                if (p.IH * p.IW > kMaxPackedPix * 256) continue;
+                if (p.IH * p.IW > kMaxPackedPix * 256) return false;
             } else {
                 p.IW = (PW - 1) * p.S + d->kw;
                 p.lds_pix_b = p.chunk_b + 16;
                 p.lds_row_b = p.IW * p.lds_pix_b;
                 p.b_align = 16;
-                if (p.IH * p.IW * (p.chunk_b / 16) > kMaxActVec * 256) continue;
+                if (p.IH * p.IW * (p.chunk_b / 16) > kMaxActVec * 256) return false;
             }
             // the tile plus the 16 bytes a lane may read past its last row's last pixel
             p.lds_act_b = (p.IH * p.lds_row_b + 16 + 63) / 64 * 64;
-            if (p.lds_bytes() > 158 * 1024) continue;
+            return p.lds_bytes() <= 158 * 1024;
+        };
+        // small preferences: wide channel tiles re-stage the input less often, 64-byte chunks halve
+        // the number of stages, the 128-pixel variant has the least reuse per staged byte
+        const double prefs = (TM == 128 ? 0.005 : 0.0) - (chunk_opt == 32 ? 0.004 : 0.0) - (variant == 2 ? 0.02 : 0.0);
+        auto consider = [&](double score) {
+            if (!found || score > best_score) {
+                best_score = score;
+                best = p;
+                found = true;
+            }
+        };
+        if (pool) {
+            for (int MPW = 1; 2 * MPW + 1 <= TN / 3 && MPW <= pool->ow; ++MPW) {
+                int MPH = (TN / (2 * MPW + 1) - 1) / 2;
+                if (MPH > pool->oh) MPH = pool->oh;
+                if (MPH < 1) continue;
+                p.MPH = MPH;
+                p.MPW = MPW;
+                if (!shape_patch(2 * MPH + 1, 2 * MPW + 1)) continue;
+                p.tiles_y = ceil_div(pool->oh, MPH);
+                p.tiles_x = ceil_div(pool->ow, MPW);
+                // four convolution pixels per pooled pixel are the useful part of a patch
+                const double useful = 4.0 * pool->oh * pool->ow;
+                const double issued = (double)p.tiles_y * p.tiles_x * TN;
+                consider(useful / issued + prefs);
+            }
+            continue;
+        }
+        for (int PW = 1; PW <= TN && PW <= OW; ++PW) {
+            int PH = TN / PW;
+            if (PH > OH) PH = OH;
+            if (PH < 1) continue;
+            if (!shape_patch(PH, PW)) continue;
             p.tiles_y = ceil_div(OH, PH);
             p.tiles_x = ceil_div(OW, PW);
             const double useful = (double)OH * OW * d->k;
             const double issued = (double)p.tiles_y * p.tiles_x * TN * ktiles * TM;
             // prefer square-ish patches (less halo) at equal utilisation
             const double halo = (double)p.IH * p.IW / ((double)PH * PW * p.S * p.S);
-            // small preferences: wide channel tiles re-stage the input less often, 64-byte chunks halve
-            // the number of stages, the 128-pixel variant has the least reuse per staged byte
-            const double score = useful / issued - 0.01 * halo + (TM == 128 ? 0.005 : 0.0) -
-                                 (chunk_opt == 32 ? 0.004 : 0.0) - (variant == 2 ? 0.02 : 0.0);
-            if (!found || score > best_score) {
-                best_score = score;
-                best = p;
-                found = true;
-            }
+            consider(useful / issued - 0.01 * halo + prefs);
         }
     }
     if (!found) {
@@ -812,21 +969,40 @@ int launch_kernel(exhip_ctx* ctx, K kernel, bool* attr_set, const Plan& pl, cons
     return 0;
 }
 
+template <int DT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
+int launch_inst(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
+    static bool attr = false;
+    return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, WM, WN, PACKED, EPI, KWE, KSC>, &attr, pl, p, grid);
+}
+
+// The row shapes with compile-time fragment addresses: 3 taps x 64-byte chunks (3x3 layers), 1 tap x 64-byte
+// chunks (1x1 layers), and the packed first-layer form (one 32-byte k-step per filter row). Anything else
+// runs the run-time form.
+template <int DT, int WM, int WN, bool PACKED, int EPI>
+int launch_shape(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
+    if constexpr (PACKED) {
+        return launch_inst<DT, WM, WN, true, EPI, 1, 1>(ctx, pl, p, grid);
+    } else {
+        if (pl.KWe == 3 && pl.KS == 2) return launch_inst<DT, WM, WN, false, EPI, 3, 2>(ctx, pl, p, grid);
+        if (pl.KWe == 1 && pl.KS == 2) return launch_inst<DT, WM, WN, false, EPI, 1, 2>(ctx, pl, p, grid);
+        return launch_inst<DT, WM, WN, false, EPI, 0, 0>(ctx, pl, p, grid);
+    }
+}
+
 template <int DT, bool PACKED, int EPI>
 int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
-    static bool attr[kNumVariants] = {false, false, false};
     switch (pl.variant) {
-    case 0: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 1, 4, PACKED, EPI>, &attr[0], pl, p, grid);
-    case 1: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 4, PACKED, EPI>, &attr[1], pl, p, grid);
-    default: return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, 2, 2, PACKED, EPI>, &attr[2], pl, p, grid);
+    case 0: return launch_shape<DT, 1, 4, PACKED, EPI>(ctx, pl, p, grid);
+    case 1: return launch_shape<DT, 2, 4, PACKED, EPI>(ctx, pl, p, grid);
+    default: return launch_shape<DT, 2, 2, PACKED, EPI>(ctx, pl, p, grid);
     }
 }
 
 template <int DT>
-int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p) {
+int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolSpec* pool = nullptr) {
     EXHIP_REQUIRE(ctx, "conv: NULL ctx");
     Plan pl;
-    int rc = make_plan(d, DT, &pl);
+    int rc = make_plan(d, DT, &pl, pool);
     if (rc) return rc;
     EXHIP_REQUIRE(p.x && p.wp, "conv: NULL input or weights");
     EXHIP_REQUIRE(d->k_stride >= d->k || (!p.y_q && !p.y_nhwc && !p.residual), "conv: k_stride %d < k %d", d->k_stride, d->k);
@@ -850,10 +1026,22 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p) {
     p.magic_iw = (unsigned)(((1ull << 32) + pl.IW - 1) / pl.IW);
     p.magic_pw = (unsigned)(((1ull << 32) + pl.PW - 1) / pl.PW);
     p.vp_shift = pl.chunk_b == 64 ? 2 : 1;
+    p.tile_dy = pl.PH; p.tile_dx = pl.PW;
+    if (pool) {
+        p.MPH = pl.MPH; p.MPW = pl.MPW; p.POH = pool->oh; p.POW = pool->ow;
+        p.tile_dy = 2 * pl.MPH; p.tile_dx = 2 * pl.MPW; p.tile_oy = pool->pt; p.tile_ox = pool->pl;
+        p.magic_mpw = (unsigned)(((1ull << 32) + pl.MPW - 1) / pl.MPW);
+    }
     EXHIP_REQUIRE((long long)d->n * pl.OH * pl.OW < (1ll << 31), "conv: more than 2^31 output pixels");
     const long long grid = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
     EXHIP_REQUIRE(grid > 0 && grid < (1ll << 31), "conv: grid too large");
     if constexpr (DT == EXHIP_I8) {
+        if (pool) {
+            const long long out_elems = (long long)d->n * pool->oh * pool->ow * d->k;
+            EXHIP_REQUIRE(out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid, "conv+pool: output tensor too large");
+            if (pl.packed) return launch_shape<DT, 1, 4, true, 2>(ctx, pl, p, (int)grid);
+            return launch_shape<DT, 1, 4, false, 2>(ctx, pl, p, (int)grid);
+        }
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = !p.y_nchw && !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
@@ -937,6 +1125,42 @@ extern "C" int exhip_conv2d_i8(exhip_ctx* ctx, const exhip_conv_desc* d, const i
     p.x = (const char*)x; p.wp = (const char*)wp; p.scale = scale; p.bias = bias; p.residual = residual;
     p.y_q = y_i8; p.y_nhwc = y_f32_nhwc; p.y_nchw = y_f32_nchw; p.acc_nchw = acc_nchw;
     return run_conv<EXHIP_I8>(ctx, d, p);
+}
+
+extern "C" int exhip_conv2d_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_desc* d, int pool_pt, int pool_pl, int pool_oh,
+                                            int pool_ow, const int8_t* x, const void* wp, const float* scale,
+                                            const float* bias, int8_t* y_i8, float* y_f32_nhwc) {
+    EXHIP_REQUIRE(d && scale, "exhip_conv2d_i8_maxpool3x3s2: NULL descriptor or scale");
+    EXHIP_REQUIRE(y_i8 || y_f32_nhwc, "exhip_conv2d_i8_maxpool3x3s2: no output requested");
+    EXHIP_REQUIRE(d->k % 64 == 0 && d->k_stride == d->k, "conv+pool: needs k %% 64 == 0 and k_stride == k (k %d, k_stride %d)", d->k, d->k_stride);
+    EXHIP_REQUIRE(d->act <= 1 && !d->post_relu, "conv+pool: activation must be none or ReLU");
+    int oh = 0, ow = 0;
+    int rc = exhip_conv_out_hw(d, &oh, &ow);
+    if (rc) return rc;
+    // every pooled window must hold at least one convolution pixel, as the reference's pooling guarantees
+    EXHIP_REQUIRE(pool_pt >= 0 && pool_pt <= 1 && pool_pl >= 0 && pool_pl <= 1, "conv+pool: pool padding must be 0 or 1");
+    EXHIP_REQUIRE(pool_oh > 0 && pool_ow > 0 && 2 * (pool_oh - 1) - pool_pt < oh && 2 * (pool_ow - 1) - pool_pl < ow,
+                  "conv+pool: pooled size %dx%d does not fit a %dx%d convolution output", pool_oh, pool_ow, oh, ow);
+    // same packed weights as exhip_conv2d_i8: the unpooled plan must use 64-channel slabs too
+    Plan plain;
+    rc = make_plan(d, EXHIP_I8, &plain);
+    if (rc) return rc;
+    if (plain.TM != 64) {
+        exhip_set_error("conv+pool: this layer's weights are packed for %d-channel slabs", plain.TM);
+        return EXHIP_ERR_UNSUPPORTED;
+    }
+    const PoolSpec pool = {pool_pt, pool_pl, pool_oh, pool_ow};
+    Plan pooled;
+    rc = make_plan(d, EXHIP_I8, &pooled, &pool);
+    if (rc) return rc;
+    if (pooled.chunk_b != plain.chunk_b || pooled.n_chunks != plain.n_chunks || pooled.KWe != plain.KWe || pooled.KS != plain.KS) {
+        exhip_set_error("conv+pool: the pooled tiling needs a different weight packing than exhip_conv_pack_weights produced");
+        return EXHIP_ERR_UNSUPPORTED;
+    }
+    ConvParams p = {};
+    p.x = (const char*)x; p.wp = (const char*)wp; p.scale = scale; p.bias = bias;
+    p.y_q = y_i8; p.y_nhwc = y_f32_nhwc;
+    return run_conv<EXHIP_I8>(ctx, d, p, &pool);
 }
 
 extern "C" int exhip_conv2d_f16(exhip_ctx* ctx, const exhip_conv_desc* d, const uint16_t* x, const void* wp,

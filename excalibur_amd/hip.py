@@ -208,6 +208,10 @@ class Ctx:
         _check(lib().exhip_conv2d_i8(self.h, ctypes.byref(d), x.ptr, wp.ptr, scale.ptr, _ptr(bias), _ptr(residual),
                                      _ptr(y_i8), _ptr(y_f32_nhwc), _ptr(y_f32_nchw), _ptr(acc)))
 
+    def conv2d_i8_maxpool3x3s2(self, d, pool_pad, pool_oh, pool_ow, x, wp, scale, bias=None, y_i8=None, y_f32_nhwc=None):
+        _check(lib().exhip_conv2d_i8_maxpool3x3s2(self.h, ctypes.byref(d), pool_pad, pool_pad, pool_oh, pool_ow, x.ptr, wp.ptr,
+                                                  scale.ptr, _ptr(bias), _ptr(y_i8), _ptr(y_f32_nhwc)))
+
     def conv2d_f16(self, d, x, wp, bias=None, residual=None, y_f16_nhwc=None, y_f16_nchw=None, y_f32_nchw=None):
         _check(lib().exhip_conv2d_f16(self.h, ctypes.byref(d), x.ptr, wp.ptr, _ptr(bias), _ptr(residual), _ptr(y_f16_nhwc),
                                       _ptr(y_f16_nchw), _ptr(y_f32_nchw)))

@@ -136,9 +136,10 @@ class FusedRunner:
     float32_to_int8(x * fs) of the very float the CPU path would have produced.
     """
 
-    def __init__(self, ctx, net, n, h, w, profile=False):
+    def __init__(self, ctx, net, n, h, w, profile=False, fuse_pool=True):
         from . import hip
         self.ctx, self.net, self.n, self.h, self.w = ctx, net, n, h, w
+        self.fuse_pool = fuse_pool  # stem convolution and max pool as one launch
         self.hip = hip
         self.steps = []       # (label, kind, callable)
         self.conv_gop = {}    # label -> algorithmic GOP per launch
@@ -165,6 +166,25 @@ class FusedRunner:
         self.steps.append((layer.name, "conv", lambda: ctx.conv2d_i8(d, x_i8, wp, scale_d, bias_d, residual, y_i8, y_f32,
                                                                       y_nchw, None)))
         return y_i8, y_f32, y_nchw, oh, ow, ks
+
+    def _conv_maxpool(self, layer, x_i8, hin, win, cs_in, fs_out):
+        """Convolution and the 3x3 stride-2 pad-1 max pool behind it as one launch: pooled f32 and int8 NHWC."""
+        ctx, hip = self.ctx, self.hip
+        d = ctx.conv_desc(self.n, layer.c, hin, win, layer.k, layer.kernel, layer.stride, layer.pad, layer.act, cs_in, layer.k,
+                          0, float(fs_out))
+        oh, ow = ctx.conv_out_hw(d)
+        ph, pw = (oh + 2 - 3) // 2 + 1, (ow + 2 - 3) // 2 + 1
+        wp = ctx.pack_conv_weights(d, hip.I8, layer.w_i8)
+        ws, fs = layer.ws, layer.fs
+        with np.errstate(divide="ignore"):
+            scale = np.where(np.abs(ws.astype(np.float64)) <= 1e-6, np.float32(0),
+                             np.float32(1.0) / (ws * fs).astype(np.float32)).astype(np.float32)
+        scale_d, bias_d = ctx.array(scale), ctx.array(layer.bias)
+        y = ctx.empty((self.n, ph, pw, layer.k), np.float32)
+        yq = ctx.empty((self.n, ph, pw, layer.k), np.int8)
+        self.conv_gop[layer.name] = 2.0 * self.n * oh * ow * layer.k * layer.c * layer.kernel * layer.kernel / 1e9
+        self.steps.append((layer.name, "conv", lambda: ctx.conv2d_i8_maxpool3x3s2(d, 1, ph, pw, x_i8, wp, scale_d, bias_d, yq, y)))
+        return y, yq, ph, pw, layer.k
 
     def _quantize_input(self, x, q, fs):
         import ctypes
@@ -196,8 +216,11 @@ class FusedRunner:
         self.x = ctx.empty((n, 3, self.h, self.w), np.float32)
         self.q0 = ctx.empty((n, self.h, self.w, 4), np.int8)
         self._quantize_input(self.x, self.q0, net.stem.fs)
-        _, stem_f32, _, oh, ow, ks = self._conv(net.stem, self.q0, self.h, self.w, 4, None, 0, None, True, False)
-        pool_f32, pool_i8, ph, pw = self._maxpool(stem_f32, 64, oh, ow, ks, net.blocks[0][0].fs)
+        if self.fuse_pool:
+            pool_f32, pool_i8, ph, pw, ks = self._conv_maxpool(net.stem, self.q0, self.h, self.w, 4, net.blocks[0][0].fs)
+        else:
+            _, stem_f32, _, oh, ow, ks = self._conv(net.stem, self.q0, self.h, self.w, 4, None, 0, None, True, False)
+            pool_f32, pool_i8, ph, pw = self._maxpool(stem_f32, 64, oh, ow, ks, net.blocks[0][0].fs)
         cur_i8, cur_f32, hh, ww, cs = pool_i8, pool_f32, ph, pw, ks
         nb = len(net.blocks)
         for bi, (c1, c2, ds) in enumerate(net.blocks):

@@ -109,6 +109,18 @@ int exhip_conv2d_i8(exhip_ctx* ctx, const exhip_conv_desc* d, const int8_t* x_nh
                     const float* scale, const float* bias, const float* residual_nhwc, int8_t* y_i8_nhwc,
                     float* y_f32_nhwc, float* y_f32_nchw, int32_t* acc_nchw);
 
+/* exhip_conv2d_i8 followed by operation_pooling::forward_cpu_f32's MAX pooling
+ * (src/Excalibur/operation_pooling.cpp:80-190) with a 3x3 window and stride 2, in one kernel: the
+ * convolution's own output never reaches memory. pool_pt / pool_pl (0 or 1) are the pool's top / left
+ * padding, pool_oh x pool_ow its output size (exhip_pool_out_hw); windows are clipped to the convolution's
+ * output exactly as the reference clips them. Outputs (either may be NULL): pooled NHWC int8 requantized
+ * with d->fs_out, pooled NHWC float32. Needs d->k % 64 == 0, k_stride == k, act 0 or 1; returns
+ * EXHIP_ERR_UNSUPPORTED when the layer's packed weights use a tiling the pooled kernel cannot share (the
+ * caller then runs exhip_conv2d_i8 and exhip_maxpool2d_nhwc_f32). w_packed is exhip_conv_pack_weights' output. */
+int exhip_conv2d_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_desc* d, int pool_pt, int pool_pl, int pool_oh,
+                                 int pool_ow, const int8_t* x_nhwc, const void* w_packed, const float* scale,
+                                 const float* bias, int8_t* y_i8_nhwc, float* y_f32_nhwc);
+
 /* operation_convolution::forward_cpu_f32 (src/Excalibur/operation_convolution.cpp:251-329) with fp16
  * storage and f32 accumulation (include/Excalibur/operation.hpp:234-260 describes the fp16 layer):
  * x NHWC f16; outputs NHWC f16 and/or NCHW f16 and/or NCHW f32; residual NHWC f16. */

@@ -107,6 +107,43 @@ def test_conv_i8_requant_pad_channels_are_zero(ctx):
     assert not got["i8"][..., 40:].any()
 
 
+CONV_POOL_SHAPES = [
+    # seed, n, c, h, w, k, kernel, stride, pad, pool pad, pool pad_mode
+    (240, 2, 3, 150, 134, 64, 7, 2, 3, 1, 1),   # stem + pool, sizes that leave ragged pooled tiles
+    (241, 1, 3, 64, 64, 64, 7, 2, 3, 0, 0),     # no pool padding, the reference's "full" output size (clipped windows)
+    (242, 2, 32, 37, 41, 64, 3, 1, 1, 1, 1),    # generic (unpacked) convolution in front of the pool
+    (243, 1, 64, 9, 11, 64, 3, 1, 1, 1, 1),     # image smaller than one pooled tile
+]
+
+
+@pytest.mark.parametrize("args", CONV_POOL_SHAPES, ids=[f"s{a[0]}" for a in CONV_POOL_SHAPES])
+def test_conv_i8_maxpool_one_launch_bit_exact(ctx, args):
+    """Convolution (+ReLU) and the 3x3 stride-2 max pool behind it in one kernel == oracle conv then oracle pool."""
+    seed, n, c, h, w, k, kernel, stride, pad, ppad, pad_mode = args
+    case = cases.conv_i8_case(seed, n, c, h, w, k, kernel, stride, pad, act=1)
+    fs_out = np.float32(23.5)
+    y = cases.oracle_eval(case)
+    want = port.pool2d(y, port.POOL_MAX, 3, 2, ppad, pad_mode=pad_mode)
+    poh, pow_ = want.shape[2:]
+    cs = gpueval.in_stride(c, gpueval.hip.I8, kernel)
+    d = ctx.conv_desc(n, c, h, w, k, kernel, stride, pad, 1, cs, k, 0, float(fs_out))
+    xq = ctx.quantize_nchw_to_nhwc_i8(ctx.array(case["x"]), case["fs"], cs)
+    wp = ctx.pack_conv_weights(d, gpueval.hip.I8, case["wt"])
+    scale = ctx.array(gpueval.dequant_scales(case["ws"], case["fs"], k))
+    bias = ctx.array(case["bias"])
+    yf = ctx.empty((n, poh, pow_, k), np.float32)
+    yq = ctx.empty((n, poh, pow_, k), np.int8)
+    ctx.conv2d_i8_maxpool3x3s2(d, ppad, poh, pow_, xq, wp, scale, bias, yq, yf)
+    ctx.sync()
+    assert np.array_equal(yf.download(), want.transpose(0, 2, 3, 1))
+    assert np.array_equal(yq.download(), port.quantize(want, fs_out).transpose(0, 2, 3, 1))
+    # the int8 copy alone
+    yq2 = ctx.empty((n, poh, pow_, k), np.int8)
+    ctx.conv2d_i8_maxpool3x3s2(d, ppad, poh, pow_, xq, wp, scale, bias, yq2, None)
+    ctx.sync()
+    assert np.array_equal(yq2.download(), yq.download())
+
+
 F32_SHAPES = [
     (230, 1, 64, 56, 56, 64, 3, 1, 1),      # cfg1
     (231, 1, 64, 56, 56, 128, 3, 1, 1),
