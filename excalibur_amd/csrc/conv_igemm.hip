@@ -35,7 +35,7 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 namespace {
 
-constexpr int kMaxActVec = 10;   // 16-byte activation vectors staged per thread and channel chunk (256-thread groups)
+constexpr int kMaxActVec = 12;   // loads per thread for one activation tile of one channel chunk (256-thread groups)
 constexpr int kMaxWVec = 9;      // 16-byte weight vectors staged per thread and stage (256-thread groups)
 constexpr int kMaxPackedPix = 8; // pixels staged per thread in packed-row form (256-thread groups)
 constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format: out-of-range reads return 0
@@ -81,6 +81,9 @@ struct ConvParams {
     unsigned magic_iw, magic_pw; // ceil(2^32 / IW), ceil(2^32 / PW): exact quotients by one multiply-high for operands < 2^16
     unsigned magic_mpw;          // ceil(2^32 / MPW)
     int vp_shift;             // log2 of the 16-byte vectors per staged pixel
+    int SL;                   // non-packed: 16-byte LDS slots per staged pixel (chunk / 16 + 1 padding slot)
+    unsigned magic_sl;        // ceil(2^32 / SL)
+    int nal, nwl;             // non-packed: asynchronous loads per thread for one activation tile / one weight stage
     int prefetch_res;         // fused epilogue: touch the shortcut tensor before the MFMA loop (short reductions only)
     int tile_dy, tile_dx;     // output pixels between the origins of neighbouring patches (PH, PW unless pooled)
     int tile_oy, tile_ox;     // the first patch starts this many pixels before output pixel 0 (pooled form: the pool's padding)
@@ -139,6 +142,33 @@ __device__ __forceinline__ float fast_activation(float v, int act) {
     return v;
 }
 
+// One 16-byte element per lane from a bounds-checked buffer view straight into LDS: lane l's data lands at
+// lds_base + 16 * l (lds_base wave-uniform, in M0). Completion is counted by vmcnt like any other load.
+__device__ __forceinline__ void async_load16(__amdgpu_buffer_rsrc_t rsrc, int voff, unsigned lds_base) {
+    __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                     ::"s"(lds_base), "v"(voff), "s"(rsrc)
+                     : "memory", "m0");
+}
+
+// Waits until at most `keep` of this wave's loads are in flight. The instruction takes an immediate, so a
+// wave-uniform value picks the largest supported immediate that does not exceed it.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_imm() { __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+__device__ __forceinline__ void wait_vmcnt(int keep) {
+    if (keep >= 16) wait_vmcnt_imm<16>();
+    else if (keep >= 12) wait_vmcnt_imm<12>();
+    else if (keep >= 10) wait_vmcnt_imm<10>();
+    else if (keep >= 8) wait_vmcnt_imm<8>();
+    else if (keep == 7) wait_vmcnt_imm<7>();
+    else if (keep == 6) wait_vmcnt_imm<6>();
+    else if (keep == 5) wait_vmcnt_imm<5>();
+    else if (keep == 4) wait_vmcnt_imm<4>();
+    else if (keep == 3) wait_vmcnt_imm<3>();
+    else if (keep == 2) wait_vmcnt_imm<2>();
+    else if (keep == 1) wait_vmcnt_imm<1>();
+    else wait_vmcnt_imm<0>();
+}
+
 // KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
 // turns every LDS fragment address of a row into an immediate offset; KWE == 0 keeps them as run-time values.
 template <int DT, int MT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
@@ -146,7 +176,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
     constexpr int THREADS = 64 * WM * WN;
     constexpr int TM = 32 * MT * WM;
     // staging limits scale with the group size so that a 512-thread group needs half the registers
-    constexpr int NAV = PACKED ? 1 : kMaxActVec * 256 / THREADS;
+    constexpr int NAV = PACKED ? 1 : kMaxActVec * 256 / THREADS;  // asynchronous loads per thread and activation tile
     constexpr int NPP = PACKED ? kMaxPackedPix * 256 / THREADS : 1;
     constexpr int NWV = kMaxWVec * 256 / THREADS;
     typedef typename Acc<DT>::type acc_t;
@@ -156,7 +186,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
     char* const lds_a0 = smem + kSbBytes;
     char* const lds_w0 = lds_a0 + p.act_bufs * p.lds_act_b;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // wave-uniform values are pinned to scalar registers: a buffer resource built from a value the compiler keeps
+    // in vector registers costs a serialising loop around every access
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     auto stamp = [&](int k) {
         if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * (THREADS / 64) + wave) * 16 + k] = wall_clock64();
@@ -170,12 +202,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         const int per = gridDim.x >> 3;
         if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
     }
-    const int kt = bid % p.ktiles;
+    const int kt = __builtin_amdgcn_readfirstlane(bid % p.ktiles);
     int t = bid / p.ktiles;
-    const int tx = t % p.tiles_x;
+    const int tx = __builtin_amdgcn_readfirstlane(t % p.tiles_x);
     t /= p.tiles_x;
-    const int ty = t % p.tiles_y;
-    const int n = t / p.tiles_y;
+    const int ty = __builtin_amdgcn_readfirstlane(t % p.tiles_y);
+    const int n = __builtin_amdgcn_readfirstlane(t / p.tiles_y);
     const int oy0 = ty * p.tile_dy - p.tile_oy, ox0 = tx * p.tile_dx - p.tile_ox;
     const int iy0 = oy0 * p.S * p.tile_step - p.PT, ix0 = ox0 * p.S * p.tile_step - p.PL;
 
@@ -185,19 +217,25 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
     const char* const ximg = p.x + (size_t)n * p.img_bytes;
 
     // ---- staging plan (same for every chunk) ----
+    // Non-packed form: operands travel from global memory straight into LDS (buffer loads with the LDS
+    // modifier), no staging registers and no LDS store instructions. One such load moves 64 lanes x 16 bytes
+    // to 1 KiB of consecutive LDS, so the LDS image of a tile is cut into 16-byte slots and slot v is fetched by
+    // thread v % THREADS in its (v / THREADS)-th load. A pixel owns SL = chunk / 16 + 1 slots: its channel
+    // chunk and one padding slot (the padding keeps the fragment reads of neighbouring pixels on different
+    // banks); padding slots, halo pixels outside the image and slots past the tile get an offset beyond the
+    // view's range and so are filled with zeros.
+    // Packed form (first layer): 4- or 8-byte pixels through registers, as dword loads and LDS stores.
     int a_goff[PACKED ? NPP : NAV];
-    int a_loff[PACKED ? NPP : NAV];
+    int a_loff[PACKED ? NPP : 1];
     if constexpr (!PACKED) {
-        const int nvec = (p.IH * p.IW) << p.vp_shift;
+        const int npix = p.IH * p.IW;
 #pragma unroll
         for (int i = 0; i < NAV; ++i) {
             const int v = tid + THREADS * i;
-            const int pix = v >> p.vp_shift, part = v - (pix << p.vp_shift);
+            const int pix = fast_div(v, p.magic_sl), part = v - pix * p.SL;
             const int iy = fast_div(pix, p.magic_iw), ix = pix - iy * p.IW;
             const int gy = iy0 + iy * p.tile_step, gx = ix0 + ix * p.tile_step;
-            const bool in_tile = v < nvec;
-            const bool in_img = in_tile && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
-            a_loff[i] = in_tile ? iy * p.lds_row_b + ix * p.lds_pix_b + part * 16 : -1;
+            const bool in_img = pix < npix && part < p.SL - 1 && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
             a_goff[i] = in_img ? (gy * p.W + gx) * p.cstride_b + part * 16 : (int)p.img_bytes;
         }
     } else {
@@ -242,62 +280,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
     const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;  // packed weight bytes of one filter row
     const int n_stages = p.n_chunks * p.n_rg;
     const char* const wkt = p.wp + (size_t)kt * p.n_chunks * p.KH * row_w_b;
-
-    // Staging registers. Weights of stage st travel in set (st & 1); with DEEP the set of stage st + 2 is
-    // requested at the start of stage st, so every load has one whole stage to land before it is needed.
-    constexpr bool DEEP = THREADS == 512;
-    v4i a_reg[NAV];
-    int a_reg_p[NPP][2];
-    v4i w_set0[NWV], w_set1[DEEP ? NWV : 1];
-
-    auto load_act = [&](int cc) {
-        const int soff = PACKED ? 0 : cc * p.chunk_b;
-        const __amdgpu_buffer_rsrc_t xr =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ximg + soff), 0, (int)(p.img_bytes - soff), kRsrcWord3);
-        if constexpr (!PACKED) {
-#pragma unroll
-            for (int i = 0; i < NAV; ++i) a_reg[i] = __builtin_amdgcn_raw_buffer_load_b128(xr, a_goff[i], 0, 0);
-        } else {
-#pragma unroll
-            for (int i = 0; i < NPP; ++i) {
-                a_reg_p[i][0] = __builtin_amdgcn_raw_buffer_load_b32(xr, a_goff[i], 0, 0);
-                a_reg_p[i][1] = p.cstride_b == 8 ? __builtin_amdgcn_raw_buffer_load_b32(xr, a_goff[i] + 4, 0, 0) : 0;
-            }
-        }
-    };
-    auto store_act = [&](char* dst) {
-        if constexpr (!PACKED) {
-#pragma unroll
-            for (int i = 0; i < NAV; ++i)
-                if (a_loff[i] >= 0) *reinterpret_cast<v4i*>(dst + a_loff[i]) = a_reg[i];
-        } else {
-#pragma unroll
-            for (int i = 0; i < NPP; ++i)
-                if (a_loff[i] >= 0) {
-                    *reinterpret_cast<int*>(dst + a_loff[i]) = a_reg_p[i][0];
-                    if (p.cstride_b == 8) *reinterpret_cast<int*>(dst + a_loff[i] + 4) = a_reg_p[i][1];
-                }
-        }
-    };
     auto stage_rows = [&](int rg) { const int r0 = rg * p.RS; return (p.KH - r0 < p.RS ? p.KH - r0 : p.RS); };
-    auto load_w = [&](int cc, int rg, auto& regs) {
-        // a view of exactly this stage's slice: lanes past its end read zeros
-        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<char*>(wkt + (size_t)(cc * p.KH + rg * p.RS) * row_w_b), 0, stage_rows(rg) * row_w_b, kRsrcWord3);
-#pragma unroll
-        for (int i = 0; i < NWV; ++i) regs[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (tid + THREADS * i) * 16, 0, 0);
-    };
-    auto store_w = [&](char* dst, auto& regs) {
-#pragma unroll
-        for (int i = 0; i < NWV; ++i) {
-            const int v = (tid + THREADS * i) * 16;
-            if (v < p.lds_w_b) *reinterpret_cast<v4i*>(dst + v) = regs[i];
-        }
-    };
-
-    // One stage: request what later stages need, run the MFMAs of this one from LDS, then publish the next
-    // stage's operands into the other LDS buffers. `mine` is the register set this stage's weights came in
-    // (free again), `next` the set holding stage st + 1.
     // (chunk, row group) of the stage `by` stages after (cc, rg), without dividing
     auto stage_after = [&](int cc, int rg, int by, int& cc_out, int& rg_out) {
         for (int i = 0; i < by; ++i)
@@ -305,27 +288,10 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         cc_out = cc;
         rg_out = rg;
     };
-    auto run_stage = [&](int st, int cc, int rg, auto& mine, auto& next) {
-        const bool more = st + 1 < n_stages;
-        const bool next_chunk = rg + 1 == p.n_rg;
-        if constexpr (DEEP) {
-            if (st + 2 < n_stages) {
-                int c2, r2;
-                stage_after(cc, rg, 2, c2, r2);
-                load_w(c2, r2, mine);
-            }
-            if (rg == 0 && cc + 1 < p.n_chunks) load_act(cc + 1);
-        } else {
-            if (more) {
-                int c1, r1;
-                stage_after(cc, rg, 1, c1, r1);
-                load_w(c1, r1, next);
-            }
-            if (more && next_chunk) load_act(cc + 1);
-        }
-        // ---- MFMA over this stage: k-steps in (row, tap, channel) order, fragments fetched one step ahead ----
-        const char* wl = lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff;
-        const char* al = lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b;
+
+    // ---- the MFMAs of one stage: k-steps in (row, tap, channel) order, fragments fetched one step ahead ----
+    // wl: this wave's first weight fragment of the stage; al: the stage's first filter row in the activation tile
+    auto mfma_stage = [&](const char* wl, const char* al, int rg) {
         v4i af[2][MT], bf[2][NT];
         auto compute = [&](int buf) {
 #pragma unroll
@@ -421,11 +387,6 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                 compute(0);
             }
         }
-        if (more) {
-            if (next_chunk) store_act(lds_a0 + ((cc + 1) & (p.act_bufs - 1)) * p.lds_act_b);
-            store_w(lds_w0 + ((st + 1) & (p.w_bufs - 1)) * p.lds_w_b, next);
-        }
-        __syncthreads();
     };
 
     stamp(1);
@@ -460,23 +421,149 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
             lds_sb[(tid < TM ? 0 : 128) + c] = v;
         }
     }
-    load_act(0);
-    load_w(0, 0, w_set0);
-    if constexpr (DEEP) {
+
+    if constexpr (!PACKED) {
+        // ---- asynchronous pipeline ----
+        // Weights of stage st + 2 and the activation tile of the next chunk are requested while stage st runs;
+        // weights rotate through up to three LDS buffers, activation tiles through two. The loads are inline
+        // assembly the compiler does not track, so the waits are explicit: three wave-uniform counters hold how
+        // many loads this wave has issued after the last load of (a) the next stage's weights, (b) the weights
+        // after those, (c) the next chunk's tile; the wait before the stage-end barrier lets exactly that many
+        // stay in flight. Every wave issues the same number of loads per request (slots past the end of a tile
+        // or slice read zeros), which keeps the counters uniform across the group.
+        const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+        const unsigned wave_slot = (unsigned)wave * 1024u;
+        const int nal = p.nal, nwl = p.nwl;
+        int after_near = 0, after_far = 0, after_act = 0;
+        auto issue_act = [&](int cc, int buf) {
+            const int soff = cc * p.chunk_b;
+            const __amdgpu_buffer_rsrc_t xr =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ximg + soff), 0, (int)(p.img_bytes - soff), kRsrcWord3);
+            const unsigned dst = lds_base + kSbBytes + buf * p.lds_act_b + wave_slot;
+#pragma unroll
+            for (int i = 0; i < NAV; ++i)
+                if (i < nal) async_load16(xr, a_goff[i], dst + i * (THREADS * 16));
+            after_near += nal; after_far += nal; after_act = 0;
+        };
+        auto issue_w = [&](int cc, int rg, int buf) {
+            // a view of exactly this stage's slice: lanes past its end read zeros
+            const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<char*>(wkt + (size_t)(cc * p.KH + rg * p.RS) * row_w_b), 0, stage_rows(rg) * row_w_b, kRsrcWord3);
+            const unsigned dst = lds_base + kSbBytes + p.act_bufs * p.lds_act_b + buf * p.lds_w_b + wave_slot;
+            for (int i = 0; i < nwl; ++i) async_load16(wr, (tid + THREADS * i) * 16, dst + i * (THREADS * 16));
+            after_near += nwl; after_act += nwl; after_far = 0;
+        };
+        issue_act(0, 0);
+        issue_w(0, 0, 0);
         if (n_stages > 1) {
             int c1, r1;
             stage_after(0, 0, 1, c1, r1);
-            load_w(c1, r1, w_set1);
+            issue_w(c1, r1, 1);
         }
-    }
-    stamp(2);
-    store_act(lds_a0);
-    store_w(lds_w0, w_set0);
-    stamp(3);
-    __syncthreads();
-    stamp(4);
-
-    {
+        stamp(2);
+        wait_vmcnt(n_stages > 1 ? nwl : 0);
+        stamp(3);
+        __syncthreads();
+        stamp(4);
+        after_near = 0;
+        int cc = 0, rg = 0, wb = 0;
+        for (int st = 0; st < n_stages; ++st) {
+            const bool more = st + 1 < n_stages;
+            const bool next_chunk = rg + 1 == p.n_rg;
+            const bool want_a = rg == 0 && cc + 1 < p.n_chunks;
+            // the request needed sooner goes first, so that the wait below can leave the other in flight
+            if (want_a && next_chunk) issue_act(cc + 1, (cc + 1) & 1);
+            if (st + 2 < n_stages) {
+                int c2, r2;
+                stage_after(cc, rg, 2, c2, r2);
+                int b2 = wb + 2;
+                if (b2 >= p.w_bufs) b2 -= p.w_bufs;
+                issue_w(c2, r2, b2);
+            }
+            if (want_a && !next_chunk) issue_act(cc + 1, (cc + 1) & 1);
+            mfma_stage(lds_w0 + wb * p.lds_w_b + aoff, lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b, rg);
+            if (more) {
+                int keep = after_near;
+                if (next_chunk && after_act < keep) keep = after_act;
+                wait_vmcnt(keep);
+            }
+            __syncthreads();
+            after_near = after_far;
+            if (++wb == p.w_bufs) wb = 0;
+            stage_after(cc, rg, 1, cc, rg);
+        }
+    } else {
+        // ---- register-staged pipeline (packed first-layer form) ----
+        // Weights of stage st travel in set (st & 1); with DEEP the set of stage st + 2 is requested at the start
+        // of stage st, so every load has one whole stage to land before it is needed.
+        constexpr bool DEEP = THREADS == 512;
+        int a_reg_p[NPP][2];
+        v4i w_set0[NWV], w_set1[DEEP ? NWV : 1];
+        auto load_act = [&]() {
+            const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ximg), 0, (int)p.img_bytes, kRsrcWord3);
+#pragma unroll
+            for (int i = 0; i < NPP; ++i) {
+                a_reg_p[i][0] = __builtin_amdgcn_raw_buffer_load_b32(xr, a_goff[i], 0, 0);
+                a_reg_p[i][1] = p.cstride_b == 8 ? __builtin_amdgcn_raw_buffer_load_b32(xr, a_goff[i] + 4, 0, 0) : 0;
+            }
+        };
+        auto store_act = [&](char* dst) {
+#pragma unroll
+            for (int i = 0; i < NPP; ++i)
+                if (a_loff[i] >= 0) {
+                    *reinterpret_cast<int*>(dst + a_loff[i]) = a_reg_p[i][0];
+                    if (p.cstride_b == 8) *reinterpret_cast<int*>(dst + a_loff[i] + 4) = a_reg_p[i][1];
+                }
+        };
+        auto load_w = [&](int cc, int rg, auto& regs, bool valid) {
+            // a view of exactly this stage's slice: lanes past its end read zeros; an invalid request gets a
+            // zero-length view, so that every stage issues the same number of loads
+            const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<char*>(wkt + (size_t)(cc * p.KH + rg * p.RS) * row_w_b), 0, valid ? stage_rows(rg) * row_w_b : 0, kRsrcWord3);
+#pragma unroll
+            for (int i = 0; i < NWV; ++i) regs[i] = __builtin_amdgcn_raw_buffer_load_b128(wr, (tid + THREADS * i) * 16, 0, 0);
+        };
+        auto store_w = [&](char* dst, auto& regs) {
+#pragma unroll
+            for (int i = 0; i < NWV; ++i) {
+                const int v = (tid + THREADS * i) * 16;
+                if (v < p.lds_w_b) *reinterpret_cast<v4i*>(dst + v) = regs[i];
+            }
+        };
+        // One stage: request what later stages need, run the MFMAs of this one from LDS, then publish the next
+        // stage's weights into the other LDS buffer. `mine` is the register set this stage's weights came in
+        // (free again), `next` the set holding stage st + 1. The packed form has one channel chunk, so the
+        // activation tile is staged once, before the first stage.
+        auto run_stage = [&](int st, int cc, int rg, auto& mine, auto& next) {
+            const bool more = st + 1 < n_stages;
+            if constexpr (DEEP) {
+                int c2, r2;
+                stage_after(cc, rg, 2, c2, r2);
+                load_w(c2, r2, mine, st + 2 < n_stages);
+            } else {
+                if (more) {
+                    int c1, r1;
+                    stage_after(cc, rg, 1, c1, r1);
+                    load_w(c1, r1, next, true);
+                }
+            }
+            mfma_stage(lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff, lds_a0 + rg * p.RS * p.lds_row_b, rg);
+            if (more) store_w(lds_w0 + ((st + 1) & (p.w_bufs - 1)) * p.lds_w_b, next);
+            __syncthreads();
+        };
+        load_act();
+        load_w(0, 0, w_set0, true);
+        if constexpr (DEEP) {
+            int c1, r1;
+            stage_after(0, 0, 1, c1, r1);
+            load_w(c1, r1, w_set1, n_stages > 1);
+        }
+        stamp(2);
+        store_act(lds_a0);
+        store_w(lds_w0, w_set0);
+        stamp(3);
+        __syncthreads();
+        stamp(4);
         int cc = 0, rg = 0;
         if constexpr (DEEP) {
             for (int st = 0; st < n_stages; st += 2) {
@@ -527,11 +614,18 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
             if (lane < 32) table[lane] = valid ? pix * (unsigned)p.K + chb : kEpiInvalid;
             wave_sync();
             if (has_res) {
+                // offsets first, then all loads, then all LDS writes: the table lives in the same LDS as the tile,
+                // and reading it between the writes would serialise load, wait and write
+                unsigned goff[8];
+#pragma unroll
+                for (int it = 0; it < 8; ++it) goff[it] = (table[(it * 64 + lane) >> 4] + (lane & 15) * 4) * 4u;
+                v4i rv[8];
+#pragma unroll
+                for (int it = 0; it < 8; ++it) rv[it] = __builtin_amdgcn_raw_buffer_load_b128(rr, (int)goff[it], 0, 0);
 #pragma unroll
                 for (int it = 0; it < 8; ++it) {
                     const int idx = it * 64 + lane, tp = idx >> 4, part = idx & 15;
-                    const v4i rv = __builtin_amdgcn_raw_buffer_load_b128(rr, (int)((table[tp] + part * 4) * 4u), 0, 0);
-                    *reinterpret_cast<v4i*>(tile_f + tp * kEpiRowF + part * 16) = rv;
+                    *reinterpret_cast<v4i*>(tile_f + tp * kEpiRowF + part * 16) = rv[it];
                 }
                 wave_sync();
             }
@@ -807,6 +901,7 @@ struct Plan {
     int KWe, KS, chunk_b, n_chunks, RS, n_rg;
     int S, tile_step, PH, PW, IH, IW, lds_pix_b, lds_row_b, lds_act_b, lds_w_b, b_align;
     int act_bufs, w_bufs;
+    int SL, nal, nwl;
     int tiles_x, tiles_y, ktiles;
     int OH, OW;
     int MPH, MPW;  // pooled form: pooled pixels per patch (0 otherwise); the patch is then (2 MPH + 1) x (2 MPW + 1)
@@ -875,15 +970,30 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
         p.tile_step = (d->kh == 1 && d->kw == 1) ? d->sh : 1;
         p.S = d->sh / p.tile_step;
         const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;
-        // bytes one group's staging registers hold: whole 16-byte vectors per thread
-        const int w_budget = (kMaxWVec * 256 / p.threads) * p.threads * 16;
-        p.RS = w_budget / row_w_b;
-        if (p.RS < 1) continue;                  // one filter row does not fit
-        if (p.RS > d->kh) p.RS = d->kh;
-        p.n_rg = ceil_div(d->kh, p.RS);
-        p.lds_w_b = p.RS * row_w_b;
-        p.act_bufs = p.n_chunks > 1 ? 2 : 1;
-        p.w_bufs = p.n_chunks * p.n_rg > 1 ? 2 : 1;
+        const int group_b = p.threads * 16;  // bytes one load per thread moves
+        p.nal = p.nwl = 0;
+        p.SL = p.chunk_b / 16 + 1;
+        if (packed) {
+            // register-staged weights: whole 16-byte vectors per thread
+            const int w_budget = (kMaxWVec * 256 / p.threads) * group_b;
+            p.RS = w_budget / row_w_b;
+            if (p.RS < 1) continue;                  // one filter row does not fit
+            if (p.RS > d->kh) p.RS = d->kh;
+            p.n_rg = ceil_div(d->kh, p.RS);
+            p.lds_w_b = p.RS * row_w_b;
+            p.act_bufs = 1;
+            p.w_bufs = p.n_rg > 1 ? 2 : 1;
+        }
+        // Non-packed form: filter rows per stage. A stage should hold at least six k-steps (less leaves the
+        // barrier and the load requests a large share of the stage); among such splits the finest one is
+        // tried first, because it lets the MFMA loop start on less data and needs the least LDS.
+        int rs_order[16], n_rs = 0;
+        if (!packed) {
+            for (int rs = 1; rs <= d->kh && n_rs < 16; ++rs)
+                if (d->kh % rs == 0 && rs * p.KWe * p.KS >= 6) rs_order[n_rs++] = rs;
+            for (int rs = d->kh; rs >= 1 && n_rs < 16; --rs)
+                if (d->kh % rs == 0 && rs * p.KWe * p.KS < 6) rs_order[n_rs++] = rs;
+        }
         p.MPH = p.MPW = 0;
         // fills the patch-dependent fields; false when the patch exceeds a staging or LDS limit
         auto shape_patch = [&](int PH, int PW) {
@@ -903,7 +1013,22 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
                 p.lds_pix_b = p.chunk_b + 16;
                 p.lds_row_b = p.IW * p.lds_pix_b;
                 p.b_align = 16;
-                if (p.IH * p.IW * (p.chunk_b / 16) > kMaxActVec * 256) return false;
+                // the tile image plus the 16 bytes a lane may read past its last pixel, in whole load groups
+                p.lds_act_b = (p.IH * p.lds_row_b + 16 + group_b - 1) / group_b * group_b;
+                p.nal = p.lds_act_b / group_b;
+                if (p.nal > kMaxActVec * 256 / p.threads) return false;
+                if (p.lds_act_b / 16 >= (1 << 16)) return false;  // slot numbers are divided by multiply-high
+                p.act_bufs = p.n_chunks > 1 ? 2 : 1;
+                for (int i = 0; i < n_rs; ++i) {
+                    p.RS = rs_order[i];
+                    p.n_rg = d->kh / p.RS;
+                    p.lds_w_b = (p.RS * row_w_b + group_b - 1) / group_b * group_b;
+                    p.nwl = p.lds_w_b / group_b;
+                    const int n_stages = p.n_chunks * p.n_rg;
+                    p.w_bufs = n_stages < 3 ? n_stages : 3;
+                    if (p.lds_bytes() <= 158 * 1024) return true;
+                }
+                return false;
             }
             // the tile plus the 16 bytes a lane may read past its last row's last pixel
             p.lds_act_b = (p.IH * p.lds_row_b + 16 + 63) / 64 * 64;
@@ -1026,6 +1151,8 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.magic_iw = (unsigned)(((1ull << 32) + pl.IW - 1) / pl.IW);
     p.magic_pw = (unsigned)(((1ull << 32) + pl.PW - 1) / pl.PW);
     p.vp_shift = pl.chunk_b == 64 ? 2 : 1;
+    p.SL = pl.SL; p.nal = pl.nal; p.nwl = pl.nwl;
+    p.magic_sl = (unsigned)(((1ull << 32) + pl.SL - 1) / pl.SL);
     p.tile_dy = pl.PH; p.tile_dx = pl.PW;
     if (pool) {
         p.MPH = pl.MPH; p.MPW = pl.MPW; p.POH = pool->oh; p.POW = pool->ow;
