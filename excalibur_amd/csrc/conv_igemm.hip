@@ -44,6 +44,7 @@ constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format:
 constexpr int kEpiRowF = 64 * 4 + 16;
 constexpr int kEpiRowQ = 64 + 16;
 constexpr int kEpiWaveBytes = 32 * kEpiRowF + 32 * kEpiRowQ + 128;
+constexpr size_t kLdsLimit = 158 * 1024;  // dynamic LDS one group may use
 constexpr int kSbBytes = 1024;  // LDS kept for per-channel scale and bias of the group's (at most 128) channels
 constexpr unsigned kEpiInvalid = 0x3FFFFF00u;  // element offset whose byte offsets (x1, x4) lie past any accepted tensor
 
@@ -83,7 +84,10 @@ struct ConvParams {
     int vp_shift;             // log2 of the 16-byte vectors per staged pixel
     int SL;                   // non-packed: 16-byte LDS slots per staged pixel (chunk / 16 + 1 padding slot)
     unsigned magic_sl;        // ceil(2^32 / SL)
-    int nal, nwl;             // non-packed: asynchronous loads per thread for one activation tile / one weight stage
+    int act_need_b;           // non-packed: bytes of one activation tile image in LDS (whole 16-byte slots)
+    int epi_f;                // fused epilogue: the per-wave LDS tiles include the float32 one
+    int epi_mode;             // which epilogue the launched kernel has (0 general, 1 fused, 2 pooled)
+    int q_nonneg;             // fused epilogue: values reaching the quantizer are >= 0 (ReLU last, fs_out > 0)
     int prefetch_res;         // fused epilogue: touch the shortcut tensor before the MFMA loop (short reductions only)
     int tile_dy, tile_dx;     // output pixels between the origins of neighbouring patches (PH, PW unless pooled)
     int tile_oy, tile_ox;     // the first patch starts this many pixels before output pixel 0 (pooled form: the pool's padding)
@@ -231,6 +235,8 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         const int npix = p.IH * p.IW;
 #pragma unroll
         for (int i = 0; i < NAV; ++i) {
+            a_goff[i] = (int)p.img_bytes;
+            if (i * (THREADS * 16) + wave * 1024 >= p.act_need_b) continue;  // wave-uniform: this wave issues no i-th load
             const int v = tid + THREADS * i;
             const int pix = fast_div(v, p.magic_sl), part = v - pix * p.SL;
             const int iy = fast_div(pix, p.magic_iw), ix = pix - iy * p.IW;
@@ -433,8 +439,14 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         // or slice read zeros), which keeps the counters uniform across the group.
         const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
         const unsigned wave_slot = (unsigned)wave * 1024u;
-        const int nal = p.nal, nwl = p.nwl;
-        int after_near = 0, after_far = 0, after_act = 0;
+        // loads this wave issues per activation tile / weight stage: its 1 KiB pieces that start inside the data
+        auto pieces = [&](int need_b) {
+            const int left = need_b - wave * 1024;
+            return left <= 0 ? 0 : (left + THREADS * 16 - 1) / (THREADS * 16);
+        };
+        const int nal = pieces(p.act_need_b), nwl = pieces(p.RS * row_w_b);
+        const int dist = p.w_bufs - 1;  // weights are requested this many stages ahead (when there are that many)
+        int after_w[2] = {0, 0}, after_act = 0;  // loads issued after those of W(st + 1), W(st + 2), the next tile
         auto issue_act = [&](int cc, int buf) {
             const int soff = cc * p.chunk_b;
             const __amdgpu_buffer_rsrc_t xr =
@@ -443,52 +455,52 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
 #pragma unroll
             for (int i = 0; i < NAV; ++i)
                 if (i < nal) async_load16(xr, a_goff[i], dst + i * (THREADS * 16));
-            after_near += nal; after_far += nal; after_act = 0;
+            after_w[0] += nal; after_w[1] += nal; after_act = 0;
         };
-        auto issue_w = [&](int cc, int rg, int buf) {
+        auto issue_w = [&](int cc, int rg, int buf, int slot) {
             // a view of exactly this stage's slice: lanes past its end read zeros
             const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
                 const_cast<char*>(wkt + (size_t)(cc * p.KH + rg * p.RS) * row_w_b), 0, stage_rows(rg) * row_w_b, kRsrcWord3);
             const unsigned dst = lds_base + kSbBytes + p.act_bufs * p.lds_act_b + buf * p.lds_w_b + wave_slot;
             for (int i = 0; i < nwl; ++i) async_load16(wr, (tid + THREADS * i) * 16, dst + i * (THREADS * 16));
-            after_near += nwl; after_act += nwl; after_far = 0;
+            after_w[0] += nwl; after_w[1] += nwl; after_act += nwl;
+            after_w[slot] = 0;
         };
         issue_act(0, 0);
-        issue_w(0, 0, 0);
-        if (n_stages > 1) {
+        issue_w(0, 0, 0, 0);
+        if (dist == 2) {
             int c1, r1;
             stage_after(0, 0, 1, c1, r1);
-            issue_w(c1, r1, 1);
+            issue_w(c1, r1, 1, 0);
         }
         stamp(2);
-        wait_vmcnt(n_stages > 1 ? nwl : 0);
+        wait_vmcnt(dist == 2 ? nwl : 0);
         stamp(3);
         __syncthreads();
         stamp(4);
-        after_near = 0;
         int cc = 0, rg = 0, wb = 0;
         for (int st = 0; st < n_stages; ++st) {
             const bool more = st + 1 < n_stages;
             const bool next_chunk = rg + 1 == p.n_rg;
             const bool want_a = rg == 0 && cc + 1 < p.n_chunks;
             // the request needed sooner goes first, so that the wait below can leave the other in flight
-            if (want_a && next_chunk) issue_act(cc + 1, (cc + 1) & 1);
-            if (st + 2 < n_stages) {
+            if (want_a && next_chunk && dist == 2) issue_act(cc + 1, (cc + 1) & 1);
+            if (dist > 0 && st + dist < n_stages) {
                 int c2, r2;
-                stage_after(cc, rg, 2, c2, r2);
-                int b2 = wb + 2;
+                stage_after(cc, rg, dist, c2, r2);
+                int b2 = wb + dist;
                 if (b2 >= p.w_bufs) b2 -= p.w_bufs;
-                issue_w(c2, r2, b2);
+                issue_w(c2, r2, b2, dist - 1);
             }
-            if (want_a && !next_chunk) issue_act(cc + 1, (cc + 1) & 1);
+            if (want_a && !(next_chunk && dist == 2)) issue_act(cc + 1, (cc + 1) & 1);
             mfma_stage(lds_w0 + wb * p.lds_w_b + aoff, lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b, rg);
             if (more) {
-                int keep = after_near;
+                int keep = after_w[0];
                 if (next_chunk && after_act < keep) keep = after_act;
                 wait_vmcnt(keep);
             }
             __syncthreads();
-            after_near = after_far;
+            after_w[0] = after_w[1];
             if (++wb == p.w_bufs) wb = 0;
             stage_after(cc, rg, 1, cc, rg);
         }
@@ -593,10 +605,13 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         // there and global memory sees 256 / 64 contiguous bytes per pixel. All global accesses are
         // bounds-checked buffer operations: a pixel outside the image gets an offset past the range, its
         // loads return 0 and its stores are dropped, so no lane-divergent branch is needed.
-        char* const epi = smem + kSbBytes + wave * kEpiWaveBytes;  // the staging buffers are free: the loop ended with a barrier
+        // the staging buffers are free: the loop ended with a barrier. The float32 tile exists only when a
+        // float32 tensor is read or written (the launch sizes the LDS accordingly).
+        const int tile_f_b = p.epi_f ? 32 * kEpiRowF : 0;
+        char* const epi = smem + kSbBytes + wave * (tile_f_b + 32 * kEpiRowQ + 128);
         char* const tile_f = epi;                       // [32 px][64 ch f32 + 16 B]
-        char* const tile_q = epi + 32 * kEpiRowF;       // [32 px][64 ch i8 + 16 B]
-        unsigned* const table = reinterpret_cast<unsigned*>(epi + 32 * kEpiRowF + 32 * kEpiRowQ);  // element offset per tile pixel
+        char* const tile_q = epi + tile_f_b;            // [32 px][64 ch i8 + 16 B]
+        unsigned* const table = reinterpret_cast<unsigned*>(epi + tile_f_b + 32 * kEpiRowQ);  // element offset per tile pixel
         const int chb = kt * TM + wm * 64;              // first channel of this wave's 64-channel slab
         const int px_l = lane & 31, hh = lane >> 5;
         const bool has_res = p.residual != nullptr, has_f = p.y_nhwc != nullptr, has_q = p.y_q != nullptr;
@@ -656,14 +671,21 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                         for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
                     }
                     if (has_f) *reinterpret_cast<v4f*>(tf + e4 * 16) = v;
-                    // float32_to_int8(v * fs): product rounded first, then +-0.5, saturate, truncate
+                    // float32_to_int8(v * fs): product rounded first, then +-0.5, saturate, truncate. After a
+                    // final ReLU every product is >= 0: the sign select and the lower clamp fall away.
                     int b[4];
+                    if (p.q_nonneg) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float t = v[e] * p.fs_out;
-                        b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
+                        for (int e = 0; e < 4; ++e) b[e] = (int)__builtin_fminf(v[e] * p.fs_out + 0.5f, 127.f);
+                        q4[e4] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float t = v[e] * p.fs_out;
+                            b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
+                        }
+                        q4[e4] = (b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24);
                     }
-                    q4[e4] = (b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24);
                 }
                 if (has_q) *reinterpret_cast<v4i*>(tile_q + px_l * kEpiRowQ + m * 32 + hh * 16) = q4;
             }
@@ -901,15 +923,20 @@ struct Plan {
     int KWe, KS, chunk_b, n_chunks, RS, n_rg;
     int S, tile_step, PH, PW, IH, IW, lds_pix_b, lds_row_b, lds_act_b, lds_w_b, b_align;
     int act_bufs, w_bufs;
-    int SL, nal, nwl;
+    int SL, act_need_b;
     int tiles_x, tiles_y, ktiles;
     int OH, OW;
     int MPH, MPW;  // pooled form: pooled pixels per patch (0 otherwise); the patch is then (2 MPH + 1) x (2 MPW + 1)
-    size_t lds_bytes() const {  // staging buffers, reused by the epilogue's tiles
-        const size_t staging = (size_t)act_bufs * lds_act_b + (size_t)w_bufs * lds_w_b;
-        const size_t epilogue = MPH ? (size_t)PH * PW * kEpiRowF : (size_t)(threads / 64) * kEpiWaveBytes;
-        return kSbBytes + (staging > epilogue ? staging : epilogue);
+    size_t staging_bytes() const { return (size_t)act_bufs * lds_act_b + (size_t)w_bufs * lds_w_b; }
+    // What the launch asks for: the staging buffers, reused by the epilogue's tiles. epi_wave_b: bytes of LDS
+    // each wave's epilogue uses.
+    size_t launch_lds_bytes(int epi_wave_b) const {
+        const size_t epilogue = MPH ? (size_t)PH * PW * kEpiRowF : (size_t)(threads / 64) * epi_wave_b;
+        return kSbBytes + (staging_bytes() > epilogue ? staging_bytes() : epilogue);
     }
+    // What planning assumes: the largest epilogue, so that the plan (and with it the weight packing) does
+    // not depend on which outputs a call asks for.
+    size_t lds_bytes() const { return launch_lds_bytes(kEpiWaveBytes); }
 };
 
 // A 3x3 stride-2 max pool fused behind the convolution: its top / left padding and its output size.
@@ -971,7 +998,7 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
         p.S = d->sh / p.tile_step;
         const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;
         const int group_b = p.threads * 16;  // bytes one load per thread moves
-        p.nal = p.nwl = 0;
+        p.act_need_b = 0;
         p.SL = p.chunk_b / 16 + 1;
         if (packed) {
             // register-staged weights: whole 16-byte vectors per thread
@@ -1013,26 +1040,34 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
                 p.lds_pix_b = p.chunk_b + 16;
                 p.lds_row_b = p.IW * p.lds_pix_b;
                 p.b_align = 16;
-                // the tile image plus the 16 bytes a lane may read past its last pixel, in whole load groups
-                p.lds_act_b = (p.IH * p.lds_row_b + 16 + group_b - 1) / group_b * group_b;
-                p.nal = p.lds_act_b / group_b;
-                if (p.nal > kMaxActVec * 256 / p.threads) return false;
+                // the tile image plus the 16 bytes a lane may read past its last pixel, in whole 1 KiB pieces (one
+                // wave-wide load each)
+                p.act_need_b = p.IH * p.lds_row_b + 16;
+                p.lds_act_b = (p.act_need_b + 1023) / 1024 * 1024;
+                if ((p.act_need_b + group_b - 1) / group_b > kMaxActVec * 256 / p.threads) return false;
                 if (p.lds_act_b / 16 >= (1 << 16)) return false;  // slot numbers are divided by multiply-high
                 p.act_bufs = p.n_chunks > 1 ? 2 : 1;
                 for (int i = 0; i < n_rs; ++i) {
                     p.RS = rs_order[i];
                     p.n_rg = d->kh / p.RS;
-                    p.lds_w_b = (p.RS * row_w_b + group_b - 1) / group_b * group_b;
-                    p.nwl = p.lds_w_b / group_b;
+                    p.lds_w_b = p.RS * row_w_b;
                     const int n_stages = p.n_chunks * p.n_rg;
+                    // three weight buffers (requests two stages ahead) unless two let one more group share the CU
                     p.w_bufs = n_stages < 3 ? n_stages : 3;
-                    if (p.lds_bytes() <= 158 * 1024) return true;
+                    if (p.w_bufs == 3) {
+                        const size_t with3 = p.lds_bytes();
+                        p.w_bufs = 2;
+                        const size_t with2 = p.lds_bytes();
+                        const bool fits3 = with3 <= kLdsLimit;
+                        if (fits3 && kLdsLimit / with2 <= kLdsLimit / with3) p.w_bufs = 3;
+                    }
+                    if (p.lds_bytes() <= kLdsLimit) return true;
                 }
                 return false;
             }
             // the tile plus the 16 bytes a lane may read past its last row's last pixel
             p.lds_act_b = (p.IH * p.lds_row_b + 16 + 63) / 64 * 64;
-            return p.lds_bytes() <= 158 * 1024;
+            return p.lds_bytes() <= kLdsLimit;
         };
         // small preferences: wide channel tiles re-stage the input less often, 64-byte chunks halve
         // the number of stages, the 128-pixel variant has the least reuse per staged byte
@@ -1085,11 +1120,14 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
 
 template <typename K>
 int launch_kernel(exhip_ctx* ctx, K kernel, bool* attr_set, const Plan& pl, const ConvParams& p, int grid) {
+    // per-wave epilogue LDS: none in the general form, the int8 tile and offset table in the fused form, plus
+    // the float32 tile when a float32 tensor is read or written
+    const int epi_wave_b = p.epi_mode == 0 ? 0 : (p.epi_f ? kEpiWaveBytes : 32 * kEpiRowQ + 128);
     if (!*attr_set) {  // raise the dynamic LDS limit once per kernel
         EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         *attr_set = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(pl.threads), pl.lds_bytes(), ctx->stream, p);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(pl.threads), pl.launch_lds_bytes(epi_wave_b), ctx->stream, p);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -1151,7 +1189,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.magic_iw = (unsigned)(((1ull << 32) + pl.IW - 1) / pl.IW);
     p.magic_pw = (unsigned)(((1ull << 32) + pl.PW - 1) / pl.PW);
     p.vp_shift = pl.chunk_b == 64 ? 2 : 1;
-    p.SL = pl.SL; p.nal = pl.nal; p.nwl = pl.nwl;
+    p.SL = pl.SL; p.act_need_b = pl.act_need_b;
     p.magic_sl = (unsigned)(((1ull << 32) + pl.SL - 1) / pl.SL);
     p.tile_dy = pl.PH; p.tile_dx = pl.PW;
     if (pool) {
@@ -1166,6 +1204,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         if (pool) {
             const long long out_elems = (long long)d->n * pool->oh * pool->ow * d->k;
             EXHIP_REQUIRE(out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid, "conv+pool: output tensor too large");
+            p.epi_mode = 2;
             if (pl.packed) return launch_shape<DT, 1, 4, true, 2>(ctx, pl, p, (int)grid);
             return launch_shape<DT, 1, 4, false, 2>(ctx, pl, p, (int)grid);
         }
@@ -1176,6 +1215,9 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         // worth it only when the MFMA loop is too short to hide the shortcut's first-touch latency by itself
         p.prefetch_res = fused && p.residual && (long long)d->c_stride * d->kh * d->kw < 1024;
         if (fused) {
+            p.epi_mode = 1;
+            p.epi_f = p.residual || p.y_nhwc;
+            p.q_nonneg = d->fs_out > 0.f && (d->post_relu || (d->act == 1 && !p.residual));
             if (pl.packed) return launch_variant<DT, true, 1>(ctx, pl, p, (int)grid);
             return launch_variant<DT, false, 1>(ctx, pl, p, (int)grid);
         }
