@@ -270,11 +270,13 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
             int at;               // position in file order at which the node runs
             int in_value, res_value = -1, out_value;
             bool post_relu = false;
+            int pool_op = -1;     // conv node: the max pooling layer that reads its output and nothing else does
         };
         std::vector<node> nodes;
         std::vector<char> absorbed(n_ops, 0);
         for (int i = 0; i < n_ops; ++i) {
             if (kind[i] == 'p') {
+                if (absorbed[i]) continue;
                 nodes.push_back({'p', i, i, root(op_inputs_[i][0]), -1, root(op_outputs_[i][0]), false});
             } else if (kind[i] == 'c') {
                 node nd{'c', i, i, root(op_inputs_[i][0]), -1, root(op_outputs_[i][0]), false};
@@ -298,6 +300,15 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                     nd.at = r;
                     nd.post_relu = true;
                     nd.out_value = root(op_outputs_[r][0]);
+                }
+                if (a < 0 && r < 0) {
+                    const int pl = sole(nd.out_value, 'p');
+                    if (pl >= 0) {
+                        absorbed[pl] = 1;
+                        nd.at = pl;
+                        nd.pool_op = pl;
+                        nd.out_value = root(op_outputs_[pl][0]);
+                    }
                 }
                 nodes.push_back(nd);
             }
@@ -370,10 +381,11 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                 EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
                 out.n = in.n; out.c = c->output_channel_; out.h = oh; out.w = ow; out.cs = ks;
                 const size_t elems = static_cast<size_t>(out.n) * oh * ow * ks;
-                if (out.need_i8) out.i8 = alloc(elems);
-                if (out.need_f32) out.f32 = alloc(elems * sizeof(float));
+                const bool pooled_node = nd.pool_op >= 0;  // its output tensors have the pooled size: allocated below
+                if (out.need_i8 && !pooled_node) out.i8 = alloc(elems);
+                if (out.need_f32 && !pooled_node) out.f32 = alloc(elems * sizeof(float));
                 float* nchw = nullptr;
-                if (is_output[nd.out_value]) {
+                if (is_output[nd.out_value] && !pooled_node) {
                     out.nchw = std::make_shared<tensor<float>>(std::vector<int>{out.n, out.c, oh, ow}, dev);
                     nchw = out.nchw->mutable_gpu_data();
                 }
@@ -386,6 +398,47 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                 const void* wp = c->packed_weights(EXHIP_I8, d);
                 const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
                 const int8_t* x = static_cast<const int8_t*>(in.i8);
+                if (nd.pool_op >= 0) {
+                    // convolution + max pooling: one kernel when the pool is 3x3 stride 2 and the layer's tiling
+                    // allows it, else the two kernels with a float32 tensor between them
+                    auto* p = static_cast<operation_pooling<float>*>(operations_[nd.pool_op].get());
+                    int kh, kw, sh, sw, pt, pb, pl, pr, ph, pw;
+                    p->geometry(oh, ow, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &ph, &pw);
+                    out.h = ph; out.w = pw;
+                    const size_t pooled = static_cast<size_t>(out.n) * ph * pw * ks;
+                    const bool out_is_result = is_output[nd.out_value];
+                    if (out.need_i8) out.i8 = alloc(pooled);
+                    if (out.need_f32 || out_is_result || !out.need_i8) out.f32 = alloc(pooled * sizeof(float));
+                    int8_t* yq = static_cast<int8_t*>(out.i8);
+                    float* yf = static_cast<float*>(out.f32);
+                    const value_info o = out;
+                    bool one_kernel = kh == 3 && kw == 3 && sh == 2 && sw == 2 && pt <= 1 && pl <= 1 && ks == c->output_channel_ &&
+                                      c->output_channel_ % 64 == 0;
+                    if (one_kernel) {
+                        d.fs_out = o.fs;
+                        const int rc = exhip_conv2d_i8_maxpool3x3s2(ctx, &d, pt, pl, ph, pw, x, wp, scale, bias, yq, yf);  // trial launch
+                        if (rc == EXHIP_ERR_UNSUPPORTED) one_kernel = false;
+                        else EXHIP_FATAL(rc);
+                    }
+                    if (one_kernel) {
+                        plan->launches.push_back(
+                            [=]() { EXHIP_FATAL(exhip_conv2d_i8_maxpool3x3s2(ctx, &d, pt, pl, ph, pw, x, wp, scale, bias, yq, yf)); });
+                    } else {
+                        d.fs_out = 0.f;
+                        float* mid = static_cast<float*>(alloc(static_cast<size_t>(out.n) * oh * ow * ks * sizeof(float)));
+                        const int n = in.n, ch = c->output_channel_;
+                        plan->launches.push_back([=]() {
+                            EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, nullptr, nullptr, mid, nullptr, nullptr));
+                            EXHIP_FATAL(exhip_maxpool2d_nhwc_f32(ctx, mid, yf, yq, o.fs, n, ch, oh, ow, ks, ph, pw, kh, kw, sh, sw, pt, pl));
+                        });
+                    }
+                    if (out_is_result) {
+                        out.nchw = std::make_shared<tensor<float>>(std::vector<int>{out.n, out.c, ph, pw}, dev);
+                        float* nchw = out.nchw->mutable_gpu_data();
+                        plan->launches.push_back([=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, yf, o.n, o.c, ph, pw, o.cs, nchw)); });
+                    }
+                    continue;
+                }
                 int8_t* yq = static_cast<int8_t*>(out.i8);
                 float* yf = static_cast<float*>(out.f32);
                 if (!yq && !yf && !nchw) yf = static_cast<float*>(out.f32 = alloc(elems * sizeof(float)));  // dead value: still computed

@@ -117,6 +117,37 @@ def test_mixed_topology_falls_back_to_per_layer():
         os.unlink(path)
 
 
+@pytest.mark.parametrize("k,pool", [(64, (3, 2, 1)), (32, (3, 2, 1)), (64, (2, 2, 0))],
+                         ids=["one-kernel", "k32-two-kernels", "pool2x2-two-kernels"])
+def test_fused_plan_conv_then_maxpool_as_network_output(k, pool):
+    """conv(int8, ReLU) -> max pool -> conv(int8): the pool joins the convolution's node; its output is also fetched."""
+    from excalibur_amd import modelfile as mf
+    c1 = cases.conv_i8_case(41, 2, 32, 21, 23, k, 3, 1, 1)
+    a = cases.oracle_eval(c1)
+    pk, ps, pp = pool
+    b = port.pool2d(a, port.POOL_MAX, pk, ps, pp)
+    c2 = cases.conv_i8_case(42, 2, k, b.shape[2], b.shape[3], 64, 3, 1, 1)
+    c2["x"] = b
+    c2["fs"] = np.float32(127.0 / np.abs(b).max())
+    want = cases.oracle_eval(c2)
+    lines = [mf.conv_line("Convolution", "c1", "data", "a", k, 3, 1, 1, True, c1["wt"].size, 1, int8=True, act=1),
+             mf.pool_line("p", "a", "b", 0, pk, ps, pp),
+             "Split s 1 2 b b0 b1",
+             mf.conv_line("Convolution", "c2", "b0", "out", 64, 3, 1, 1, True, c2["wt"].size, 1, int8=True, act=1)]
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        f.write(mf.conv_blob_i8(c1["wt"], c1["bias"], c1["ws"], c1["fs"]) + mf.conv_blob_i8(c2["wt"], c2["bias"], c2["ws"], c2["fs"]))
+        path = f.name
+    try:
+        p = xp.Pipeline(mf.topology(lines), path, 0)
+        p.forward(c1["x"])
+        assert p.fused
+        assert np.array_equal(p.get("out"), want)
+        assert np.array_equal(p.get("b1"), b)
+        p.close()
+    finally:
+        os.unlink(path)
+
+
 @pytest.mark.parametrize("layer,evaluate", [
     ("Eltwise e 2 1 ra b out 0=1", lambda a, b: port.eltwise([a, b], port.ELT_SUM)),
     ("Eltwise e 2 1 ra b out 0=1 -23301=3,0.5,-1.25", lambda a, b: port.eltwise([a, b], port.ELT_SUM, [0.5, -1.25])),
