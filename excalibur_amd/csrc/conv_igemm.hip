@@ -43,6 +43,7 @@ constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer, 32-bit data format:
 // 16-byte accesses one row apart fall into different banks) and 32 pixel indices
 constexpr int kEpiRowF = 64 * 4 + 16;
 constexpr int kEpiRowQ = 64 + 16;
+constexpr int kPoolRowB = 32 * 4 + 16;  // pooled epilogue: one tile pixel, 32 float32 channels + padding
 constexpr int kEpiWaveBytes = 32 * kEpiRowF + 32 * kEpiRowQ + 128;
 constexpr size_t kLdsLimit = 158 * 1024;  // dynamic LDS one group may use
 constexpr int kSbBytes = 1024;  // LDS kept for per-channel scale and bias of the group's (at most 128) channels
@@ -621,6 +622,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         const __amdgpu_buffer_rsrc_t rr =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.residual), 0, (int)(bytes_q * 4u), kRsrcWord3);
         const int nt_run = chb < p.K ? NT : 0;  // a wave whose slab lies past the last channel has nothing to write
+        const float act_floor = p.act == 1 ? 0.f : -__builtin_inff(), post_floor = p.post_relu ? 0.f : -__builtin_inff();
 #pragma unroll
         for (int nn = 0; nn < NT; ++nn) {
             if (nn >= nt_run) break;
@@ -657,19 +659,16 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                     v4f v;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e], b4[e]);
-                    if (p.act == 1) {
+                    // ReLU as a maximum with 0, no ReLU as a maximum with -inf: one instruction either way
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
-                    }
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], act_floor);
                     if (has_res) {
                         const v4f rv = *reinterpret_cast<const v4f*>(tf + e4 * 16);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] += rv[e];
                     }
-                    if (p.post_relu) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
-                    }
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], post_floor);
                     if (has_f) *reinterpret_cast<v4f*>(tf + e4 * 16) = v;
                     // float32_to_int8(v * fs): product rounded first, then +-0.5, saturate, truncate. After a
                     // final ReLU every product is >= 0: the sign select and the lower clamp fall away.
@@ -711,20 +710,31 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         }
     } else if constexpr (EPI == 2) {
         // Convolution followed by a 3x3 stride-2 max pool (int8 path, TM == 64): the patch is (2 MPH + 1) x (2 MPW + 1)
-        // convolution pixels, written as float32 into one LDS tile [pixel][64 channels]; pixels outside the
+        // convolution pixels, written as float32 into an LDS tile [pixel][32 channels]; pixels outside the
         // convolution's output hold -inf, which is how the pool's own padding drops out of the maximum. After a
         // barrier the MPH x MPW pooled pixels are formed from the tile and leave as NHWC float32 and / or int8.
         static_assert(TM == 64, "pooled epilogue: one 64-channel slab per group");
+        // One pass per 32-channel block (an accumulator tile row): half the LDS of a 64-channel tile, which lets
+        // more groups share a CU.
         char* const pool = smem + kSbBytes;
         const int px_l = lane & 31, hh = lane >> 5;
         const int npatch = p.PH * p.PW;
         const float ninf = -__builtin_inff();
+        const unsigned out_px = (unsigned)p.N * (unsigned)(p.POH * p.POW);
+        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(p.y_q, 0, (int)(out_px * (unsigned)p.K), kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_nhwc, 0, (int)(out_px * (unsigned)p.K * 4u), kRsrcWord3);
+        const bool has_f = p.y_nhwc != nullptr, has_q = p.y_q != nullptr;
+        const int items = p.MPH * p.MPW * 8;  // 4-channel vectors of the pooled patch, per 32-channel block
 #pragma unroll
-        for (int nn = 0; nn < NT; ++nn) {
-            const int pp = (wn * NT + nn) * 32 + px_l;
-            const bool valid = (pvalid >> nn) & 1;
+        for (int m = 0; m < MT; ++m) {
+            if (m > 0) __syncthreads();  // the previous block's tile has been read
 #pragma unroll
-            for (int m = 0; m < MT; ++m) {
+            for (int nn = 0; nn < NT; ++nn) {
+                const int pp = (wn * NT + nn) * 32 + px_l;
+                // median(v, lo, hi): a valid pixel gets max(v, 0) with ReLU (lo = 0, hi = +inf) or v without
+                // (lo = -inf); a pixel outside the convolution's output gets -inf (lo = hi = -inf)
+                const bool valid = (pvalid >> nn) & 1;
+                const float hi = valid ? __builtin_inff() : ninf, lo = (valid && p.act == 1) ? 0.f : ninf;
                 const int c0 = m * 32 + hh * 16;
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
@@ -732,52 +742,48 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                     const v4f b4 = *reinterpret_cast<const v4f*>(lds_sb + 128 + c0 + e4 * 4);
                     v4f v;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e], b4[e]);
-                        if (p.act == 1) v[e] = __builtin_fmaxf(v[e], 0.f);
-                        v[e] = valid ? v[e] : ninf;
+                    for (int e = 0; e < 4; ++e)
+                        v[e] = __builtin_amdgcn_fmed3f(__builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e], b4[e]), lo, hi);
+                    if (pp < npatch) *reinterpret_cast<v4f*>(pool + pp * kPoolRowB + (hh * 16 + e4 * 4) * 4) = v;
+                }
+            }
+            __syncthreads();
+            if (m == 0) stamp(6);
+            for (int i = tid; i < items; i += THREADS) {
+                const int pq = i >> 3, part = i & 7;
+                const int pyy = fast_div(pq, p.magic_mpw), pxx = pq - pyy * p.MPW;
+                const int gy = ty * p.MPH + pyy, gx = tx * p.MPW + pxx;
+                const char* w0 = pool + ((2 * pyy) * p.PW + 2 * pxx) * kPoolRowB + part * 16;
+                v4f best = *reinterpret_cast<const v4f*>(w0);
+#pragma unroll
+                for (int dr = 0; dr < 3; ++dr)
+#pragma unroll
+                    for (int dc = 0; dc < 3; ++dc) {
+                        if (dr == 0 && dc == 0) continue;
+                        const v4f t = *reinterpret_cast<const v4f*>(w0 + (dr * p.PW + dc) * kPoolRowB);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) best[e] = __builtin_fmaxf(best[e], t[e]);
                     }
-                    if (pp < npatch) *reinterpret_cast<v4f*>(pool + pp * kEpiRowF + (c0 + e4 * 4) * 4) = v;
+                const bool ok = gy < p.POH && gx < p.POW;
+                const unsigned elem = ((unsigned)(n * p.POH + gy) * (unsigned)p.POW + gx) * (unsigned)p.K + kt * TM + m * 32 + part * 4;
+                const unsigned off = ok ? elem : kEpiInvalid;
+                if (has_f) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, best), rf, (int)(off * 4u), 0, 0);
+                if (has_q) {
+                    int b[4], packed;
+                    if (p.q_nonneg) {  // after ReLU every maximum is >= 0
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) b[e] = (int)__builtin_fminf(best[e] * p.fs_out + 0.5f, 127.f);
+                        packed = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float t = best[e] * p.fs_out;
+                            b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
+                        }
+                        packed = (b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24);
+                    }
+                    __builtin_amdgcn_raw_buffer_store_b32(packed, rq, (int)off, 0, 0);
                 }
-            }
-        }
-        __syncthreads();
-        stamp(6);
-        const unsigned out_px = (unsigned)p.N * (unsigned)(p.POH * p.POW);
-        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(p.y_q, 0, (int)(out_px * (unsigned)p.K), kRsrcWord3);
-        const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_nhwc, 0, (int)(out_px * (unsigned)p.K * 4u), kRsrcWord3);
-        const bool has_f = p.y_nhwc != nullptr, has_q = p.y_q != nullptr;
-        const int items = p.MPH * p.MPW * 16;  // 4-channel vectors of the pooled patch
-        for (int i = tid; i < items; i += THREADS) {
-            const int pq = i >> 4, part = i & 15;
-            const int pyy = fast_div(pq, p.magic_mpw), pxx = pq - pyy * p.MPW;
-            const int gy = ty * p.MPH + pyy, gx = tx * p.MPW + pxx;
-            const char* w0 = pool + ((2 * pyy) * p.PW + 2 * pxx) * kEpiRowF + part * 16;
-            v4f best = *reinterpret_cast<const v4f*>(w0);
-#pragma unroll
-            for (int dr = 0; dr < 3; ++dr)
-#pragma unroll
-                for (int dc = 0; dc < 3; ++dc) {
-                    if (dr == 0 && dc == 0) continue;
-                    const v4f t = *reinterpret_cast<const v4f*>(w0 + (dr * p.PW + dc) * kEpiRowF);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) best[e] = __builtin_fmaxf(best[e], t[e]);
-                }
-            const bool ok = gy < p.POH && gx < p.POW;
-            const unsigned elem = ((unsigned)(n * p.POH + gy) * (unsigned)p.POW + gx) * (unsigned)p.K + kt * TM + part * 4;
-            const unsigned off = ok ? elem : kEpiInvalid;
-            if (has_f) {
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, best), rf, (int)(off * 4u), 0, 0);
-            }
-            if (has_q) {
-                int b[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float t = best[e] * p.fs_out;
-                    b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
-                }
-                __builtin_amdgcn_raw_buffer_store_b32((b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24),
-                                                      rq, (int)off, 0, 0);
             }
         }
     } else {
@@ -931,7 +937,7 @@ struct Plan {
     // What the launch asks for: the staging buffers, reused by the epilogue's tiles. epi_wave_b: bytes of LDS
     // each wave's epilogue uses.
     size_t launch_lds_bytes(int epi_wave_b) const {
-        const size_t epilogue = MPH ? (size_t)PH * PW * kEpiRowF : (size_t)(threads / 64) * epi_wave_b;
+        const size_t epilogue = MPH ? (size_t)PH * PW * kPoolRowB : (size_t)(threads / 64) * epi_wave_b;
         return kSbBytes + (staging_bytes() > epilogue ? staging_bytes() : epilogue);
     }
     // What planning assumes: the largest epilogue, so that the plan (and with it the weight packing) does
@@ -1205,6 +1211,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             const long long out_elems = (long long)d->n * pool->oh * pool->ow * d->k;
             EXHIP_REQUIRE(out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid, "conv+pool: output tensor too large");
             p.epi_mode = 2;
+            p.q_nonneg = d->fs_out > 0.f && d->act == 1;
             if (pl.packed) return launch_shape<DT, 1, 4, true, 2>(ctx, pl, p, (int)grid);
             return launch_shape<DT, 1, 4, false, 2>(ctx, pl, p, (int)grid);
         }
