@@ -86,6 +86,26 @@ __global__ __launch_bounds__(kBlock) void quantize_nchw_to_nhwc4_kernel(const fl
     y[(size_t)n * HW + p] = (int)w;
 }
 
+// The same with four pixels per thread: 16-byte loads from each channel plane and one 16-byte store
+// (HW a multiple of 4, 16-byte aligned tensors).
+__global__ __launch_bounds__(kBlock) void quantize_nchw_to_nhwc4_x4_kernel(const float* __restrict__ x, int4* __restrict__ y,
+                                                                           int C, int HW4, float fs,
+                                                                           const float* __restrict__ fs_pc) {
+    const int n = blockIdx.y;
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= HW4) return;
+    uint32_t w[4] = {0, 0, 0, 0};
+    for (int c = 0; c < C; ++c) {
+        const float s = fs_pc ? fs_pc[c] : fs;
+        const float4 v = reinterpret_cast<const float4*>(x + ((size_t)n * C + c) * HW4 * 4)[p];
+        w[0] |= (uint32_t)(exhip_q8(v.x * s) & 0xff) << (8 * c);
+        w[1] |= (uint32_t)(exhip_q8(v.y * s) & 0xff) << (8 * c);
+        w[2] |= (uint32_t)(exhip_q8(v.z * s) & 0xff) << (8 * c);
+        w[3] |= (uint32_t)(exhip_q8(v.w * s) & 0xff) << (8 * c);
+    }
+    y[(size_t)n * HW4 + p] = make_int4((int)w[0], (int)w[1], (int)w[2], (int)w[3]);
+}
+
 // NHWC -> NCHW (graph outputs; small). MODE 0: f32->f32, 1: f16->f32, 2: f16->f16
 template <int MODE, typename Tin, typename Tout>
 __global__ __launch_bounds__(kBlock) void nhwc_to_nchw_kernel(const Tin* __restrict__ x, Tout* __restrict__ y, int C, int HW,
@@ -503,6 +523,12 @@ extern "C" int exhip_quantize_nchw_f32_to_nhwc_i8(exhip_ctx* ctx, const float* x
     REQ_CTX("exhip_quantize_nchw_f32_to_nhwc_i8");
     if (c_stride == 4 && c <= 4) {
         EXHIP_REQUIRE(x && y && n > 0 && h > 0 && w > 0, "quantize: bad argument");
+        if ((h * w) % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) {
+            dim3 grid4(blocks_for((size_t)h * w / 4), n);
+            hipLaunchKernelGGL(quantize_nchw_to_nhwc4_x4_kernel, grid4, dim3(kBlock), 0, ctx->stream, x, (int4*)y, c, h * w / 4, fs, fs_pc);
+            EXHIP_LAUNCH_CHECK();
+            return 0;
+        }
         dim3 grid(blocks_for((size_t)h * w), n);
         hipLaunchKernelGGL(quantize_nchw_to_nhwc4_kernel, grid, dim3(kBlock), 0, ctx->stream, x, (int*)y, c, h * w, fs, fs_pc);
         EXHIP_LAUNCH_CHECK();

@@ -150,9 +150,11 @@ __device__ __forceinline__ float fast_activation(float v, int act) {
 // One 16-byte element per lane from a bounds-checked buffer view straight into LDS: lane l's data lands at
 // lds_base + 16 * l (lds_base wave-uniform, in M0). Completion is counted by vmcnt like any other load.
 __device__ __forceinline__ void async_load16(__amdgpu_buffer_rsrc_t rsrc, int voff, unsigned lds_base) {
+    // no "memory" clobber: the LDS region written is not read before a later wait + barrier (which are
+    // compiler barriers), and volatile keeps this ordered against them and against other loads of this kind
     __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
                      ::"s"(lds_base), "v"(voff), "s"(rsrc)
-                     : "memory", "m0");
+                     : "m0");
 }
 
 // Waits until at most `keep` of this wave's loads are in flight. The instruction takes an immediate, so a
@@ -177,7 +179,7 @@ __device__ __forceinline__ void wait_vmcnt(int keep) {
 // KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
 // turns every LDS fragment address of a row into an immediate offset; KWE == 0 keeps them as run-time values.
 template <int DT, int MT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
-__global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvParams p) {
+__global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igemm_kernel(const ConvParams p) {
     constexpr int THREADS = 64 * WM * WN;
     constexpr int TM = 32 * MT * WM;
     // staging limits scale with the group size so that a 512-thread group needs half the registers
@@ -298,8 +300,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
 
     // ---- the MFMAs of one stage: k-steps in (row, tap, channel) order, fragments fetched one step ahead ----
     // wl: this wave's first weight fragment of the stage; al: the stage's first filter row in the activation tile
-    auto mfma_stage = [&](const char* wl, const char* al, int rg) {
-        v4i af[2][MT], bf[2][NT];
+    auto mfma_stage = [&](const char* wl, const char* al, int rg, auto&& after_first_row) {
+        constexpr int NFB = 2;  // fragment buffers: the fetch of k-step s + 1 runs under the MFMAs of k-step s
+        v4i af[NFB][MT], bf[NFB][NT];
         auto compute = [&](int buf) {
 #pragma unroll
             for (int m = 0; m < MT; ++m)
@@ -324,33 +327,40 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                     else bf[buf][nn] = lds_read16(arow[nn] + q_ * PIXB + j_ * 32);
                 }
             };
-            // One filter row, entered with k-step 0 already in buffer P0; leaves the next row's k-step 0 in
-            // buffer (P0 + NS) & 1 when there is a next row.
-            auto row = [&](auto p0, bool has_next) {
-                constexpr int P0 = decltype(p0)::value;
-                const char* nr[NT];
+            {
+                // One filter row, entered with k-step 0 already in buffer P0; leaves the next row's k-step 0 in
+                // buffer (P0 + NS) & 1 when there is a next row. The callback runs once, between the first row
+                // and the rest.
+                auto row = [&](auto p0, bool has_next) {
+                    constexpr int P0 = decltype(p0)::value;
+                    const char* nr[NT];
 #pragma unroll
-                for (int nn = 0; nn < NT; ++nn) nr[nn] = ar[nn] + p.lds_row_b;
+                    for (int nn = 0; nn < NT; ++nn) nr[nn] = ar[nn] + p.lds_row_b;
 #pragma unroll
-                for (int s_ = 0; s_ < NS; ++s_) {
-                    if (s_ + 1 < NS) fetch_at((P0 + s_ + 1) & 1, wl, ar, s_ + 1);
-                    else if (has_next) fetch_at((P0 + s_ + 1) & 1, wl + NS * STEPB, nr, 0);
-                    compute((P0 + s_) & 1);
+                    for (int s_ = 0; s_ < NS; ++s_) {
+                        if (s_ + 1 < NS) fetch_at((P0 + s_ + 1) & 1, wl, ar, s_ + 1);
+                        else if (has_next) fetch_at((P0 + s_ + 1) & 1, wl + NS * STEPB, nr, 0);
+                        compute((P0 + s_) & 1);
+                    }
+                    wl += NS * STEPB;
+#pragma unroll
+                    for (int nn = 0; nn < NT; ++nn) ar[nn] = nr[nn];
+                };
+                fetch_at(0, wl, ar, 0);
+                if constexpr (NS % 2 == 0) {
+                    row(std::integral_constant<int, 0>{}, nrows > 1);
+                    after_first_row();
+                    for (int r = 1; r < nrows; ++r) row(std::integral_constant<int, 0>{}, r + 1 < nrows);
+                } else {
+                    row(std::integral_constant<int, 0>{}, nrows > 1);
+                    after_first_row();
+                    int r = 1;
+                    for (; r + 1 < nrows; r += 2) {
+                        row(std::integral_constant<int, 1>{}, true);
+                        row(std::integral_constant<int, 0>{}, r + 2 < nrows);
+                    }
+                    if (r < nrows) row(std::integral_constant<int, 1>{}, false);
                 }
-                wl += NS * STEPB;
-#pragma unroll
-                for (int nn = 0; nn < NT; ++nn) ar[nn] = nr[nn];
-            };
-            fetch_at(0, wl, ar, 0);
-            if constexpr (NS % 2 == 0) {
-                for (int r = 0; r < nrows; ++r) row(std::integral_constant<int, 0>{}, r + 1 < nrows);
-            } else {
-                int r = 0;
-                for (; r + 1 < nrows; r += 2) {
-                    row(std::integral_constant<int, 0>{}, true);
-                    row(std::integral_constant<int, 1>{}, r + 2 < nrows);
-                }
-                if (r < nrows) row(std::integral_constant<int, 0>{}, false);
             }
         } else {
             const int nk = stage_rows(rg) * p.KWe * p.KS;
@@ -378,6 +388,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                 }
             };
             fetch(0);
+            after_first_row();
             int it = 0;
             for (; it + 2 <= nk - 1; it += 2) {
                 fetch(1);
@@ -397,18 +408,21 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
     };
 
     stamp(1);
-    int prefetched[2] = {0, 0};
+    constexpr int NPF = (EPI == 1) ? (32 * NT * WN * ((TM * 4) >> 7)) / THREADS : 1;  // shortcut lines touched per thread
+    int prefetched[NPF];
+#pragma unroll
+    for (int r = 0; r < NPF; ++r) prefetched[r] = 0;
     if constexpr (EPI == 1) {
         // Touch this group's part of the float32 shortcut tensor now (one dword per 128-byte line): the lines travel
         // from HBM into L2 while the MFMA loop runs, so the epilogue's reads do not start cold. The two values are
         // only "used" at the end of the kernel, which keeps the loads in flight without waiting for them here.
         if (p.prefetch_res) {
             constexpr int lines_px = (TM * 4) >> 7;                    // 128-byte lines per pixel of this group's slab
-            const int total = p.PH * p.PW * lines_px;                  // <= 2 * THREADS for every variant
+            const int total = p.PH * p.PW * lines_px;                  // <= NPF * THREADS
             const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
                 const_cast<void*>(p.residual), 0, (int)((unsigned)p.N * (unsigned)(p.OH * p.OW) * (unsigned)p.K * 4u), kRsrcWord3);
 #pragma unroll
-            for (int r = 0; r < 2; ++r) {
+            for (int r = 0; r < NPF; ++r) {
                 const int i = tid + r * THREADS;
                 const int pp = i / lines_px, ln = i - pp * lines_px;
                 const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
@@ -484,23 +498,39 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
             const bool more = st + 1 < n_stages;
             const bool next_chunk = rg + 1 == p.n_rg;
             const bool want_a = rg == 0 && cc + 1 < p.n_chunks;
-            // the request needed sooner goes first, so that the wait below can leave the other in flight
-            if (want_a && next_chunk && dist == 2) issue_act(cc + 1, (cc + 1) & 1);
-            if (dist > 0 && st + dist < n_stages) {
-                int c2, r2;
-                stage_after(cc, rg, dist, c2, r2);
-                int b2 = wb + dist;
-                if (b2 >= p.w_bufs) b2 -= p.w_bufs;
-                issue_w(c2, r2, b2, dist - 1);
-            }
-            if (want_a && !(next_chunk && dist == 2)) issue_act(cc + 1, (cc + 1) & 1);
-            mfma_stage(lds_w0 + wb * p.lds_w_b + aoff, lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b, rg);
+            // The requests go out after the stage's first filter row has been issued: their issue cost then
+            // overlaps with MFMAs already in the pipe instead of standing in front of them. The request needed
+            // sooner goes first, so that the wait below can leave the other in flight.
+            auto requests = [&]() {
+                if (want_a && next_chunk && dist == 2) issue_act(cc + 1, (cc + 1) & 1);
+                if (dist > 0 && st + dist < n_stages) {
+                    int c2, r2;
+                    stage_after(cc, rg, dist, c2, r2);
+                    int b2 = wb + dist;
+                    if (b2 >= p.w_bufs) b2 -= p.w_bufs;
+                    issue_w(c2, r2, b2, dist - 1);
+                }
+                if (want_a && !(next_chunk && dist == 2)) issue_act(cc + 1, (cc + 1) & 1);
+            };
+            long long t0 = 0, t1 = 0, t2 = 0;
+            if (p.dbg) t0 = wall_clock64();
+            mfma_stage(lds_w0 + wb * p.lds_w_b + aoff, lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b, rg,
+                       requests);
+            if (p.dbg) t1 = wall_clock64();
             if (more) {
                 int keep = after_w[0];
                 if (next_chunk && after_act < keep) keep = after_act;
                 wait_vmcnt(keep);
             }
+            if (p.dbg) t2 = wall_clock64();
             __syncthreads();
+            if (p.dbg && lane == 0) {
+                const long long t3 = wall_clock64();
+                long long* d = p.dbg + ((size_t)blockIdx.x * (THREADS / 64) + wave) * 16;
+                d[9] += t1 - t0;
+                d[10] += t2 - t1;
+                d[11] += t3 - t2;
+            }
             after_w[0] = after_w[1];
             if (++wb == p.w_bufs) wb = 0;
             stage_after(cc, rg, 1, cc, rg);
@@ -560,7 +590,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
                     load_w(c1, r1, next, true);
                 }
             }
-            mfma_stage(lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff, lds_a0 + rg * p.RS * p.lds_row_b, rg);
+            mfma_stage(lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff, lds_a0 + rg * p.RS * p.lds_row_b, rg, []() {});
             if (more) store_w(lds_w0 + ((st + 1) & (p.w_bufs - 1)) * p.lds_w_b, next);
             __syncthreads();
         };
@@ -621,6 +651,8 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
         const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_nhwc, 0, (int)(bytes_q * 4u), kRsrcWord3);
         const __amdgpu_buffer_rsrc_t rr =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p.residual), 0, (int)(bytes_q * 4u), kRsrcWord3);
+        const bool has_nchw = p.y_nchw != nullptr;
+        const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc(p.y_nchw, 0, (int)(bytes_q * 4u), kRsrcWord3);
         const int nt_run = chb < p.K ? NT : 0;  // a wave whose slab lies past the last channel has nothing to write
         const float act_floor = p.act == 1 ? 0.f : -__builtin_inff(), post_floor = p.post_relu ? 0.f : -__builtin_inff();
 #pragma unroll
@@ -629,6 +661,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
             const bool valid = (pvalid >> nn) & 1;
             const unsigned pix = (unsigned)n * img_px + (oy0 + ppy[nn]) * p.OW + ox0 + ppx[nn];
             if (lane < 32) table[lane] = valid ? pix * (unsigned)p.K + chb : kEpiInvalid;
+            const unsigned nchw0 = ((unsigned)n * (unsigned)p.K + chb) * (unsigned)img_px + (oy0 + ppy[nn]) * p.OW + ox0 + ppx[nn];
             wave_sync();
             if (has_res) {
                 // offsets first, then all loads, then all LDS writes: the table lives in the same LDS as the tile,
@@ -670,6 +703,16 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], post_floor);
                     if (has_f) *reinterpret_cast<v4f*>(tf + e4 * 16) = v;
+                    if (has_nchw) {
+                        // the reference's boundary layout, straight from the registers: lanes run along pixels, so
+                        // each store writes runs of consecutive floats of one channel plane
+                        const v4i vi = __builtin_bit_cast(v4i, v);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const unsigned off = (nchw0 + (unsigned)((m * 32 + hh * 16 + e4 * 4 + e) * img_px)) * 4u;
+                            __builtin_amdgcn_raw_buffer_store_b32(vi[e], rn, valid ? (int)off : (int)0xFFFFFF00u, 0, 0);
+                        }
+                    }
                     // float32_to_int8(v * fs): product rounded first, then +-0.5, saturate, truncate. After a
                     // final ReLU every product is >= 0: the sign select and the lower clamp fall away.
                     int b[4];
@@ -902,7 +945,8 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void conv_igemm_kernel(const ConvP
             }
         }
     }
-    __asm__ volatile("" ::"v"(prefetched[0]), "v"(prefetched[1]));
+#pragma unroll
+    for (int r = 0; r < NPF; ++r) __asm__ volatile("" ::"v"(prefetched[r]));
     stamp(8);
 }
 
@@ -975,9 +1019,12 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
     const int OH = (d->h + d->pt + d->pb - d->kh) / d->sh + 1, OW = (d->w + d->pl + d->pr - d->kw) / d->sw + 1;
     const bool packed = cb < 32;
     static const int force_variant = getenv("EXHIP_FORCE_VARIANT") ? atoi(getenv("EXHIP_FORCE_VARIANT")) : -1;
+    static const int force_chunk = getenv("EXHIP_FORCE_CHUNK") ? atoi(getenv("EXHIP_FORCE_CHUNK")) : 0;
+    static const int force_rs = getenv("EXHIP_FORCE_RS") ? atoi(getenv("EXHIP_FORCE_RS")) : 0;
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
         if (force_variant >= 0 && variant != force_variant) continue;
+        if (force_chunk > 0 && !packed && chunk_opt != force_chunk) continue;
         if (pool && variant != 0) continue;  // the pooled epilogue holds one 64-channel slab per group
         if (packed && chunk_opt == 64) continue;
         if (!packed && cb % chunk_opt != 0) continue;
@@ -1055,6 +1102,7 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
                 p.act_bufs = p.n_chunks > 1 ? 2 : 1;
                 for (int i = 0; i < n_rs; ++i) {
                     p.RS = rs_order[i];
+                    if (force_rs > 0 && d->kh % force_rs == 0 && p.RS != force_rs) continue;
                     p.n_rg = d->kh / p.RS;
                     p.lds_w_b = p.RS * row_w_b;
                     const int n_stages = p.n_chunks * p.n_rg;
@@ -1121,6 +1169,11 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
         return EXHIP_ERR_UNSUPPORTED;
     }
     *out = best;
+    static const bool show = getenv("EXHIP_DEBUG_PLAN") != nullptr;  // development aid: one line per planned layer
+    if (show)
+        fprintf(stderr, "plan %dx%dx%dx%d k%d %dx%d s%d%s: variant %d chunk %d RS %d patch %dx%d tile %dx%d act %d B x%d w %d B x%d lds %zu\n", d->n,
+                d->c, d->h, d->w, d->k, d->kh, d->kw, d->sh, pool ? " +pool" : "", best.variant, best.chunk_b, best.RS, best.PH, best.PW,
+                best.IH, best.IW, best.lds_act_b, best.act_bufs, best.lds_w_b, best.w_bufs, best.lds_bytes());
     return 0;
 }
 
@@ -1138,32 +1191,32 @@ int launch_kernel(exhip_ctx* ctx, K kernel, bool* attr_set, const Plan& pl, cons
     return 0;
 }
 
-template <int DT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
+template <int DT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
 int launch_inst(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
     static bool attr = false;
-    return launch_kernel(ctx, conv_igemm_kernel<DT, 2, 2, WM, WN, PACKED, EPI, KWE, KSC>, &attr, pl, p, grid);
+    return launch_kernel(ctx, conv_igemm_kernel<DT, 2, NT, WM, WN, PACKED, EPI, KWE, KSC>, &attr, pl, p, grid);
 }
 
 // The row shapes with compile-time fragment addresses: 3 taps x 64-byte chunks (3x3 layers), 1 tap x 64-byte
 // chunks (1x1 layers), and the packed first-layer form (one 32-byte k-step per filter row). Anything else
 // runs the run-time form.
-template <int DT, int WM, int WN, bool PACKED, int EPI>
+template <int DT, int NT, int WM, int WN, bool PACKED, int EPI>
 int launch_shape(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
     if constexpr (PACKED) {
-        return launch_inst<DT, WM, WN, true, EPI, 1, 1>(ctx, pl, p, grid);
+        return launch_inst<DT, NT, WM, WN, true, EPI, 1, 1>(ctx, pl, p, grid);
     } else {
-        if (pl.KWe == 3 && pl.KS == 2) return launch_inst<DT, WM, WN, false, EPI, 3, 2>(ctx, pl, p, grid);
-        if (pl.KWe == 1 && pl.KS == 2) return launch_inst<DT, WM, WN, false, EPI, 1, 2>(ctx, pl, p, grid);
-        return launch_inst<DT, WM, WN, false, EPI, 0, 0>(ctx, pl, p, grid);
+        if (pl.KWe == 3 && pl.KS == 2) return launch_inst<DT, NT, WM, WN, false, EPI, 3, 2>(ctx, pl, p, grid);
+        if (pl.KWe == 1 && pl.KS == 2) return launch_inst<DT, NT, WM, WN, false, EPI, 1, 2>(ctx, pl, p, grid);
+        return launch_inst<DT, NT, WM, WN, false, EPI, 0, 0>(ctx, pl, p, grid);
     }
 }
 
 template <int DT, bool PACKED, int EPI>
 int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
     switch (pl.variant) {
-    case 0: return launch_shape<DT, 1, 4, PACKED, EPI>(ctx, pl, p, grid);
-    case 1: return launch_shape<DT, 2, 4, PACKED, EPI>(ctx, pl, p, grid);
-    default: return launch_shape<DT, 2, 2, PACKED, EPI>(ctx, pl, p, grid);
+    case 0: return launch_shape<DT, 2, 1, 4, PACKED, EPI>(ctx, pl, p, grid);
+    case 1: return launch_shape<DT, 2, 2, 4, PACKED, EPI>(ctx, pl, p, grid);
+    default: return launch_shape<DT, 2, 2, 2, PACKED, EPI>(ctx, pl, p, grid);
     }
 }
 
@@ -1212,12 +1265,12 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             EXHIP_REQUIRE(out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid, "conv+pool: output tensor too large");
             p.epi_mode = 2;
             p.q_nonneg = d->fs_out > 0.f && d->act == 1;
-            if (pl.packed) return launch_shape<DT, 1, 4, true, 2>(ctx, pl, p, (int)grid);
-            return launch_shape<DT, 1, 4, false, 2>(ctx, pl, p, (int)grid);
+            if (pl.packed) return launch_shape<DT, 2, 1, 4, true, 2>(ctx, pl, p, (int)grid);
+            return launch_shape<DT, 2, 1, 4, false, 2>(ctx, pl, p, (int)grid);
         }
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
-        const bool fused = !p.y_nchw && !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
+        const bool fused = !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
                            out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
         // worth it only when the MFMA loop is too short to hide the shortcut's first-touch latency by itself
         p.prefetch_res = fused && p.residual && (long long)d->c_stride * d->kh * d->kw < 1024;

@@ -144,6 +144,17 @@ def test_conv_i8_maxpool_one_launch_bit_exact(ctx, args):
     assert np.array_equal(yq2.download(), yq.download())
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 5, 7), (2, 3, 8, 10), (1, 1, 4, 4), (1, 4, 3, 3)], ids=str)
+def test_first_layer_quantizer_packs_four_channel_pixels(ctx, shape):
+    """float NCHW -> int8 NHWC with 4-byte pixels, through both the one-pixel and the four-pixel kernel."""
+    x = np.random.default_rng(250).uniform(-2, 2, shape).astype(np.float32)
+    fs = np.float32(77.7)
+    got = ctx.quantize_nchw_to_nhwc_i8(ctx.array(x), fs, 4).download()
+    want = port.quantize(x, fs).transpose(0, 2, 3, 1)
+    assert np.array_equal(got[..., :shape[1]], want)
+    assert not got[..., shape[1]:].any()
+
+
 F32_SHAPES = [
     (230, 1, 64, 56, 56, 64, 3, 1, 1),      # cfg1
     (231, 1, 64, 56, 56, 128, 3, 1, 1),
