@@ -1123,9 +1123,10 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
             p.lds_act_b = (p.IH * p.lds_row_b + 16 + 63) / 64 * 64;
             return p.lds_bytes() <= kLdsLimit;
         };
-        // small preferences: wide channel tiles re-stage the input less often, 64-byte chunks halve
-        // the number of stages, the 128-pixel variant has the least reuse per staged byte
-        const double prefs = (TM == 128 ? 0.005 : 0.0) - (chunk_opt == 32 ? 0.004 : 0.0) - (variant == 2 ? 0.02 : 0.0);
+        // small preferences: 64-byte chunks halve the number of stages; two independent 256-thread groups per
+        // CU overlap each other's barriers and load waits, which one 512-thread group cannot; the 128-pixel
+        // variant has the least reuse per staged byte
+        const double prefs = -(chunk_opt == 32 ? 0.004 : 0.0) - (variant == 1 ? 0.002 : 0.0) - (variant == 2 ? 0.02 : 0.0);
         auto consider = [&](double score) {
             if (!found || score > best_score) {
                 best_score = score;
