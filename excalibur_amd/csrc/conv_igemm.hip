@@ -655,6 +655,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
         const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc(p.y_nchw, 0, (int)(bytes_q * 4u), kRsrcWord3);
         const int nt_run = chb < p.K ? NT : 0;  // a wave whose slab lies past the last channel has nothing to write
         const float act_floor = p.act == 1 ? 0.f : -__builtin_inff(), post_floor = p.post_relu ? 0.f : -__builtin_inff();
+        const bool q_only = p.q_nonneg && has_q && !has_res && !has_f && !has_nchw;
 #pragma unroll
         for (int nn = 0; nn < NT; ++nn) {
             if (nn >= nt_run) break;
@@ -685,6 +686,25 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
                 const int ch0 = chb + m * 32 + hh * 16;
                 char* const tf = tile_f + px_l * kEpiRowF + (m * 32 + hh * 16) * 4;
                 v4i q4;
+                if (q_only) {
+                    // int8 output only, ReLU last: q = trunc(max(v, 0) * fs + 0.5) capped at 127. With fs > 0 the
+                    // maximum commutes with the product, and max(t, 0) + 0.5 == max(t + 0.5, 0.5) in float
+                    // arithmetic (the sum is monotone in t), so one median does ReLU and saturation.
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const v4f s4 = *reinterpret_cast<const v4f*>(lds_sb + (ch0 - kt * TM) + e4 * 4);
+                        const v4f b4 = *reinterpret_cast<const v4f*>(lds_sb + 128 + (ch0 - kt * TM) + e4 * 4);
+                        int b[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float v = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e], b4[e]);
+                            b[e] = (int)__builtin_amdgcn_fmed3f(v * p.fs_out + 0.5f, 0.5f, 127.f);
+                        }
+                        q4[e4] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                    }
+                    *reinterpret_cast<v4i*>(tile_q + px_l * kEpiRowQ + m * 32 + hh * 16) = q4;
+                    continue;
+                }
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
                     const v4f s4 = *reinterpret_cast<const v4f*>(lds_sb + (ch0 - kt * TM) + e4 * 4);
