@@ -89,7 +89,6 @@ struct ConvParams {
     int epi_f;                // fused epilogue: the per-wave LDS tiles include the float32 one
     int epi_mode;             // which epilogue the launched kernel has (0 general, 1 fused, 2 pooled)
     int q_nonneg;             // fused epilogue: values reaching the quantizer are >= 0 (ReLU last, fs_out > 0)
-    int prefetch_res;         // fused epilogue: touch the shortcut tensor before the MFMA loop (short reductions only)
     int tile_dy, tile_dx;     // output pixels between the origins of neighbouring patches (PH, PW unless pooled)
     int tile_oy, tile_ox;     // the first patch starts this many pixels before output pixel 0 (pooled form: the pool's padding)
     int MPH, MPW, POH, POW;   // pooled form: pooled pixels per patch and pooled image size
@@ -408,30 +407,6 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
     };
 
     stamp(1);
-    constexpr int NPF = (EPI == 1) ? (32 * NT * WN * ((TM * 4) >> 7)) / THREADS : 1;  // shortcut lines touched per thread
-    int prefetched[NPF];
-#pragma unroll
-    for (int r = 0; r < NPF; ++r) prefetched[r] = 0;
-    if constexpr (EPI == 1) {
-        // Touch this group's part of the float32 shortcut tensor now (one dword per 128-byte line): the lines travel
-        // from HBM into L2 while the MFMA loop runs, so the epilogue's reads do not start cold. The two values are
-        // only "used" at the end of the kernel, which keeps the loads in flight without waiting for them here.
-        if (p.prefetch_res) {
-            constexpr int lines_px = (TM * 4) >> 7;                    // 128-byte lines per pixel of this group's slab
-            const int total = p.PH * p.PW * lines_px;                  // <= NPF * THREADS
-            const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<void*>(p.residual), 0, (int)((unsigned)p.N * (unsigned)(p.OH * p.OW) * (unsigned)p.K * 4u), kRsrcWord3);
-#pragma unroll
-            for (int r = 0; r < NPF; ++r) {
-                const int i = tid + r * THREADS;
-                const int pp = i / lines_px, ln = i - pp * lines_px;
-                const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
-                const bool ok = i < total && oy0 + py < p.OH && ox0 + px < p.OW && kt * TM * 4 + ln * 128 < p.K * 4;
-                const unsigned off = ((unsigned)(n * p.OH + oy0 + py) * p.OW + ox0 + px) * (unsigned)p.K * 4u + kt * TM * 4 + ln * 128;
-                prefetched[r] = __builtin_amdgcn_raw_buffer_load_b32(rr, ok ? (int)off : (int)0xFFFFFF00u, 0, 0);
-            }
-        }
-    }
     if constexpr (EPI >= 1) {
         // per-channel scale and bias of this group's channels, fetched now so that the epilogue finds them in LDS
         if (tid < 2 * TM) {
@@ -965,8 +940,6 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
             }
         }
     }
-#pragma unroll
-    for (int r = 0; r < NPF; ++r) __asm__ volatile("" ::"v"(prefetched[r]));
     stamp(8);
 }
 
@@ -1293,8 +1266,6 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
                            out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
-        // worth it only when the MFMA loop is too short to hide the shortcut's first-touch latency by itself
-        p.prefetch_res = fused && p.residual && (long long)d->c_stride * d->kh * d->kw < 1024;
         if (fused) {
             p.epi_mode = 1;
             p.epi_f = p.residual || p.y_nhwc;

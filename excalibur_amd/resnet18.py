@@ -233,7 +233,9 @@ class FusedRunner:
                 _, short, _, _, _, _ = self._conv(ds, cur_i8, hh, ww, cs, None, 0, None, True, False)
             else:
                 short = cur_f32
-            o_i8, o_f32, o_nchw, oh, ow, ks = self._conv(c2, a_i8, oh, ow, ks, short, 1, nxt_fs, not last, last)
+            # the float32 copy is the next block's shortcut: not needed when that block has a downsample convolution
+            want_f32 = not last and net.blocks[bi + 1][2] is None
+            o_i8, o_f32, o_nchw, oh, ow, ks = self._conv(c2, a_i8, oh, ow, ks, short, 1, nxt_fs, want_f32, last)
             cur_i8, cur_f32, hh, ww, cs = o_i8, o_f32, oh, ow, ks
             if last:
                 self.out = o_nchw
@@ -246,17 +248,18 @@ class FusedRunner:
             fn()
 
     def forward_timed(self):
-        """One forward with a HIP event pair around every launch; returns {label: ms}."""
-        evs = []
-        for label, kind, fn in self.steps:
-            e0, e1 = self.hip.Event(), self.hip.Event()
-            e0.record(self.ctx)
+        """One forward with a HIP event pair around every launch; returns [(label, kind, ms)].
+
+        The events exist before the first launch and are recorded through the bare library entry point, so
+        that the host stays ahead of the GPU and the intervals hold the kernels, not host-side gaps.
+        """
+        import ctypes
+        if not hasattr(self, "_events"):
+            self._events = [(self.hip.Event(), self.hip.Event()) for _ in self.steps]
+        record, ctx_h = self.hip.lib().exhip_event_record, self.ctx.h
+        for (label, kind, fn), (e0, e1) in zip(self.steps, self._events):
+            record(ctx_h, e0.h)
             fn()
-            e1.record(self.ctx)
-            evs.append((label, kind, e0, e1))
+            record(ctx_h, e1.h)
         self.ctx.sync()
-        out = [(label, kind, e0.elapsed_ms(e1)) for label, kind, e0, e1 in evs]
-        for _, _, e0, e1 in evs:
-            e0.destroy()
-            e1.destroy()
-        return out
+        return [(label, kind, e0.elapsed_ms(e1)) for (label, kind, fn), (e0, e1) in zip(self.steps, self._events)]
