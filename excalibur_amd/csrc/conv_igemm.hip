@@ -161,18 +161,25 @@ __device__ __forceinline__ void async_load16(__amdgpu_buffer_rsrc_t rsrc, int vo
 template <int N>
 __device__ __forceinline__ void wait_vmcnt_imm() { __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 __device__ __forceinline__ void wait_vmcnt(int keep) {
-    if (keep >= 16) wait_vmcnt_imm<16>();
-    else if (keep >= 12) wait_vmcnt_imm<12>();
-    else if (keep >= 10) wait_vmcnt_imm<10>();
-    else if (keep >= 8) wait_vmcnt_imm<8>();
-    else if (keep == 7) wait_vmcnt_imm<7>();
-    else if (keep == 6) wait_vmcnt_imm<6>();
-    else if (keep == 5) wait_vmcnt_imm<5>();
-    else if (keep == 4) wait_vmcnt_imm<4>();
-    else if (keep == 3) wait_vmcnt_imm<3>();
-    else if (keep == 2) wait_vmcnt_imm<2>();
-    else if (keep == 1) wait_vmcnt_imm<1>();
-    else wait_vmcnt_imm<0>();
+    switch (keep < 16 ? keep : 16) {  // a balanced compare tree: four branches deep
+    case 0: wait_vmcnt_imm<0>(); break;
+    case 1: wait_vmcnt_imm<1>(); break;
+    case 2: wait_vmcnt_imm<2>(); break;
+    case 3: wait_vmcnt_imm<3>(); break;
+    case 4: wait_vmcnt_imm<4>(); break;
+    case 5: wait_vmcnt_imm<5>(); break;
+    case 6: wait_vmcnt_imm<6>(); break;
+    case 7: wait_vmcnt_imm<7>(); break;
+    case 8: wait_vmcnt_imm<8>(); break;
+    case 9: wait_vmcnt_imm<9>(); break;
+    case 10: wait_vmcnt_imm<10>(); break;
+    case 11: wait_vmcnt_imm<11>(); break;
+    case 12: wait_vmcnt_imm<12>(); break;
+    case 13: wait_vmcnt_imm<13>(); break;
+    case 14: wait_vmcnt_imm<14>(); break;
+    case 15: wait_vmcnt_imm<15>(); break;
+    default: wait_vmcnt_imm<16>(); break;
+    }
 }
 
 // KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
@@ -298,8 +305,9 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
     };
 
     // ---- the MFMAs of one stage: k-steps in (row, tap, channel) order, fragments fetched one step ahead ----
-    // wl: this wave's first weight fragment of the stage; al: the stage's first filter row in the activation tile
-    auto mfma_stage = [&](const char* wl, const char* al, int rg, auto&& after_first_row) {
+    // wl: this wave's first weight fragment of the stage; al: the stage's first filter row in the activation tile;
+    // nrows: filter rows in the stage
+    auto mfma_stage = [&](const char* wl, const char* al, int nrows, auto&& after_first_row) {
         constexpr int NFB = 2;  // fragment buffers: the fetch of k-step s + 1 runs under the MFMAs of k-step s
         v4i af[NFB][MT], bf[NFB][NT];
         auto compute = [&](int buf) {
@@ -312,7 +320,6 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
             constexpr int NS = KWE * KSC;             // k-steps per filter row
             constexpr int STEPB = (TM / 32) * 1024;   // weight bytes per k-step
             constexpr int PIXB = PACKED ? 0 : KSC * 32 + 16;
-            const int nrows = stage_rows(rg);
             const char* ar[NT];
 #pragma unroll
             for (int nn = 0; nn < NT; ++nn) ar[nn] = al + boff[nn];
@@ -362,7 +369,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
                 }
             }
         } else {
-            const int nk = stage_rows(rg) * p.KWe * p.KS;
+            const int nk = nrows * p.KWe * p.KS;
             int q = 0, j = 0;          // tap column and channel k-step of the fragments being fetched
             int koff = 0;              // their byte offset inside the activation tile
             auto fetch = [&](int buf) {
@@ -420,83 +427,92 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
 
     if constexpr (!PACKED) {
         // ---- asynchronous pipeline ----
-        // Weights of stage st + 2 and the activation tile of the next chunk are requested while stage st runs;
-        // weights rotate through up to three LDS buffers, activation tiles through two. The loads are inline
-        // assembly the compiler does not track, so the waits are explicit: three wave-uniform counters hold how
+        // Weights of the stage `dist` stages ahead and the activation tile of the next chunk are requested while a
+        // stage runs; weights rotate through up to three LDS buffers, activation tiles through two. The loads are
+        // inline assembly the compiler does not track, so the waits are explicit: wave-uniform counters hold how
         // many loads this wave has issued after the last load of (a) the next stage's weights, (b) the weights
         // after those, (c) the next chunk's tile; the wait before the stage-end barrier lets exactly that many
-        // stay in flight. Every wave issues the same number of loads per request (slots past the end of a tile
-        // or slice read zeros), which keeps the counters uniform across the group.
+        // stay in flight. A wave issues one load per 1 KiB piece of a tile or slice that starts inside the data.
+        // All per-stage addresses are running values advanced by additions: a stage is short (24 MFMAs per wave
+        // in a 3x3 layer), so scalar bookkeeping counts.
         const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
         const unsigned wave_slot = (unsigned)wave * 1024u;
-        // loads this wave issues per activation tile / weight stage: its 1 KiB pieces that start inside the data
         auto pieces = [&](int need_b) {
             const int left = need_b - wave * 1024;
             return left <= 0 ? 0 : (left + THREADS * 16 - 1) / (THREADS * 16);
         };
-        const int nal = pieces(p.act_need_b), nwl = pieces(p.RS * row_w_b);
-        const int dist = p.w_bufs - 1;  // weights are requested this many stages ahead (when there are that many)
-        int after_w[2] = {0, 0}, after_act = 0;  // loads issued after those of W(st + 1), W(st + 2), the next tile
-        auto issue_act = [&](int cc, int buf) {
-            const int soff = cc * p.chunk_b;
-            const __amdgpu_buffer_rsrc_t xr =
-                __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ximg + soff), 0, (int)(p.img_bytes - soff), kRsrcWord3);
-            const unsigned dst = lds_base + kSbBytes + buf * p.lds_act_b + wave_slot;
+        const int w_stage_b = p.RS * row_w_b;  // one stage's weight slice, in memory and in LDS (RS divides KH)
+        const int nal = pieces(p.act_need_b), nwl = pieces(w_stage_b);
+        const int dist = p.w_bufs - 1;
+        int after_w[2] = {0, 0}, after_act = 0;
+
+        const char* w_src = wkt;                   // slice of the next stage to request (stages lie in request order)
+        int w_req_left = n_stages;                 // stages not requested yet
+        const unsigned w_lds0 = lds_base + kSbBytes + p.act_bufs * p.lds_act_b + wave_slot;
+        const unsigned w_lds_end = w_lds0 + p.w_bufs * p.lds_w_b;
+        unsigned w_dst = w_lds0;                   // where that slice goes
+        auto request_w = [&](int slot) {
+            if (w_req_left > 0) {
+                // a view of exactly the slice: lanes past its end read zeros
+                const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(w_src), 0, w_stage_b, kRsrcWord3);
+                for (int i = 0; i < nwl; ++i) async_load16(wr, (tid + THREADS * i) * 16, w_dst + i * (THREADS * 16));
+                after_w[0] += nwl; after_w[1] += nwl; after_act += nwl;
+                after_w[slot] = 0;
+                --w_req_left;
+                w_src += w_stage_b;
+                w_dst += p.lds_w_b;
+                if (w_dst == w_lds_end) w_dst = w_lds0;
+            }
+        };
+        const char* a_src = ximg;                  // channel chunk of the next tile to request
+        int a_range = (int)p.img_bytes;
+        int a_req_left = p.n_chunks;
+        unsigned a_dst = lds_base + kSbBytes + wave_slot;
+        const unsigned a_flip = p.act_bufs > 1 ? (unsigned)p.lds_act_b : 0u;  // the two tile buffers alternate
+        bool a_odd = false;
+        auto request_a = [&]() {
+            const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a_src), 0, a_range, kRsrcWord3);
 #pragma unroll
             for (int i = 0; i < NAV; ++i)
-                if (i < nal) async_load16(xr, a_goff[i], dst + i * (THREADS * 16));
+                if (i < nal) async_load16(xr, a_goff[i], a_dst + i * (THREADS * 16));
             after_w[0] += nal; after_w[1] += nal; after_act = 0;
+            --a_req_left;
+            a_src += p.chunk_b;
+            a_range -= p.chunk_b;
+            a_dst = a_odd ? a_dst - a_flip : a_dst + a_flip;
+            a_odd = !a_odd;
         };
-        auto issue_w = [&](int cc, int rg, int buf, int slot) {
-            // a view of exactly this stage's slice: lanes past its end read zeros
-            const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<char*>(wkt + (size_t)(cc * p.KH + rg * p.RS) * row_w_b), 0, stage_rows(rg) * row_w_b, kRsrcWord3);
-            const unsigned dst = lds_base + kSbBytes + p.act_bufs * p.lds_act_b + buf * p.lds_w_b + wave_slot;
-            for (int i = 0; i < nwl; ++i) async_load16(wr, (tid + THREADS * i) * 16, dst + i * (THREADS * 16));
-            after_w[0] += nwl; after_w[1] += nwl; after_act += nwl;
-            after_w[slot] = 0;
-        };
-        issue_act(0, 0);
-        issue_w(0, 0, 0, 0);
-        if (dist == 2) {
-            int c1, r1;
-            stage_after(0, 0, 1, c1, r1);
-            issue_w(c1, r1, 1, 0);
-        }
+        request_a();
+        request_w(0);
+        if (dist == 2) request_w(0);
         stamp(2);
         wait_vmcnt(dist == 2 ? nwl : 0);
         stamp(3);
         __syncthreads();
         stamp(4);
-        int cc = 0, rg = 0, wb = 0;
+        const char* w_cur = lds_w0 + aoff;         // this wave's fragments in the current stage's buffer
+        const char* const w_cur_end = w_cur + p.w_bufs * p.lds_w_b;
+        const char* a_cur = lds_a0;                // current tile, first filter row of the current stage
+        const int a_stage_b = p.RS * p.lds_row_b;
+        bool cur_odd = false;
+        int rg = 0;
         for (int st = 0; st < n_stages; ++st) {
             const bool more = st + 1 < n_stages;
             const bool next_chunk = rg + 1 == p.n_rg;
-            const bool want_a = rg == 0 && cc + 1 < p.n_chunks;
+            const bool want_a = rg == 0 && a_req_left > 0;
             // The requests go out after the stage's first filter row has been issued: their issue cost then
             // overlaps with MFMAs already in the pipe instead of standing in front of them. The request needed
             // sooner goes first, so that the wait below can leave the other in flight.
             auto requests = [&]() {
-                if (want_a && next_chunk && dist == 2) issue_act(cc + 1, (cc + 1) & 1);
-                if (dist > 0 && st + dist < n_stages) {
-                    int c2, r2;
-                    stage_after(cc, rg, dist, c2, r2);
-                    int b2 = wb + dist;
-                    if (b2 >= p.w_bufs) b2 -= p.w_bufs;
-                    issue_w(c2, r2, b2, dist - 1);
-                }
-                if (want_a && !(next_chunk && dist == 2)) issue_act(cc + 1, (cc + 1) & 1);
+                if (want_a && next_chunk && dist == 2) request_a();
+                if (dist > 0) request_w(dist - 1);
+                if (want_a && !(next_chunk && dist == 2)) request_a();
             };
             long long t0 = 0, t1 = 0, t2 = 0;
             if (p.dbg) t0 = wall_clock64();
-            mfma_stage(lds_w0 + wb * p.lds_w_b + aoff, lds_a0 + (cc & (p.act_bufs - 1)) * p.lds_act_b + rg * p.RS * p.lds_row_b, rg,
-                       requests);
+            mfma_stage(w_cur, a_cur, p.RS, requests);
             if (p.dbg) t1 = wall_clock64();
-            if (more) {
-                int keep = after_w[0];
-                if (next_chunk && after_act < keep) keep = after_act;
-                wait_vmcnt(keep);
-            }
+            if (more) wait_vmcnt(next_chunk && after_act < after_w[0] ? after_act : after_w[0]);
             if (p.dbg) t2 = wall_clock64();
             __syncthreads();
             if (p.dbg && lane == 0) {
@@ -507,8 +523,16 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
                 d[11] += t3 - t2;
             }
             after_w[0] = after_w[1];
-            if (++wb == p.w_bufs) wb = 0;
-            stage_after(cc, rg, 1, cc, rg);
+            w_cur += p.lds_w_b;
+            if (w_cur == w_cur_end) w_cur = lds_w0 + aoff;
+            if (next_chunk) {
+                rg = 0;
+                a_cur = lds_a0 + (cur_odd ? 0 : a_flip);
+                cur_odd = !cur_odd;
+            } else {
+                ++rg;
+                a_cur += a_stage_b;
+            }
         }
     } else {
         // ---- register-staged pipeline (packed first-layer form) ----
@@ -565,7 +589,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
                     load_w(c1, r1, next, true);
                 }
             }
-            mfma_stage(lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff, lds_a0 + rg * p.RS * p.lds_row_b, rg, []() {});
+            mfma_stage(lds_w0 + (st & (p.w_bufs - 1)) * p.lds_w_b + aoff, lds_a0 + rg * p.RS * p.lds_row_b, stage_rows(rg), []() {});
             if (more) store_w(lds_w0 + ((st + 1) & (p.w_bufs - 1)) * p.lds_w_b, next);
             __syncthreads();
         };
