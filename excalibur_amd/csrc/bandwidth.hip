@@ -378,6 +378,103 @@ __global__ __launch_bounds__(kBlock) void eltwise_f32_kernel(EltArgs a, int type
     y[i] = r;
 }
 
+// ---- activation / glue layers ----
+// One value of an elementwise activation. OP 0 HardSwish, 1 LeakyReLU, 2 sigmoid, 3 HardSigmoid; the multiply-adds
+// are fused where the CPU path's are (vector fmadd, and scalar expressions contracted by its compiler flags).
+template <int OP>
+__device__ __forceinline__ float unary_value(float x, float alpha, float beta) {
+    if constexpr (OP == 0) {
+        float t = __builtin_fmaf(x, alpha, beta);
+        t = t > 0.f ? t : 0.f;
+        t = t < 1.f ? t : 1.f;
+        return t * x;
+    } else if constexpr (OP == 1) {
+        return x < 0.f ? alpha * x : x;
+    } else if constexpr (OP == 2) {
+        return (float)(1. / (1. + exp(-(double)x)));
+    } else {
+        float t = __builtin_fmaf(alpha, x, beta);
+        t = 1.f < t ? 1.f : t;
+        return 0.f < t ? t : 0.f;
+    }
+}
+
+template <int OP>
+__global__ __launch_bounds__(kBlock) void unary_f32_kernel(const float* __restrict__ x, float* __restrict__ y, size_t n4,
+                                                           size_t count, float alpha, float beta) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n4) {
+        const v4f v = reinterpret_cast<const v4f*>(x)[i];
+        v4f r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = unary_value<OP>(v[e], alpha, beta);
+        reinterpret_cast<v4f*>(y)[i] = r;
+    } else {
+        const size_t j = n4 * 4 + (i - n4);
+        if (j < count) y[j] = unary_value<OP>(x[j], alpha, beta);
+    }
+}
+
+// Per-channel layers on NCHW. OP 0 PReLU (p0 = slope, one per channel or one shared), 1 BatchNorm as
+// fma(p1[c], x, p0[c]) with the load-time a / b, 2 Input (x - p0[c]) * p1[c]. One block row per (image, channel) plane.
+template <int OP>
+__global__ __launch_bounds__(kBlock) void channelwise_f32_kernel(const float* __restrict__ x, float* __restrict__ y, int C,
+                                                                 int HW, const float* __restrict__ p0,
+                                                                 const float* __restrict__ p1, int shared) {
+    const int plane = blockIdx.y;
+    const int c = plane % C;
+    const float a = p0[shared ? 0 : c];
+    const float b = p1 ? p1[c] : 0.f;
+    const size_t base = (size_t)plane * HW;
+    for (int j = blockIdx.x * kBlock + threadIdx.x; j < HW; j += gridDim.x * kBlock) {
+        const float v = x[base + j];
+        float r;
+        if constexpr (OP == 0) r = v >= 0.f ? v : a * v;
+        else if constexpr (OP == 1) r = __builtin_fmaf(b, v, a);
+        else r = (v - a) * b;
+        y[base + j] = r;
+    }
+}
+
+// Copies one input's channel block of every image into its place in the concatenated tensor.
+__global__ __launch_bounds__(kBlock) void concat_block_kernel(const float* __restrict__ x, float* __restrict__ y, size_t block,
+                                                              size_t out_image, size_t out_offset) {
+    const size_t img = blockIdx.y;
+    for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < block; j += (size_t)gridDim.x * kBlock)
+        y[img * out_image + out_offset + j] = x[img * block + j];
+}
+
+// Nearest-neighbour resize: in = min((int)(out * scale), size - 1), scale = size / (float)out_size.
+__global__ __launch_bounds__(kBlock) void interp_nearest_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W,
+                                                                int OH, int OW, float hs, float ws, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int ox = (int)(i % OW);
+    const size_t t = i / OW;
+    const int oy = (int)(t % OH);
+    const size_t plane = t / OH;
+    int iy = (int)(oy * hs), ix = (int)(ox * ws);
+    iy = iy > H - 1 ? H - 1 : iy;
+    ix = ix > W - 1 ? W - 1 : ix;
+    y[i] = x[(plane * H + iy) * W + ix];
+}
+
+// Space to depth of the YOLOv5 stem: out[n][g*C + c][i][j] = in[n][c][2i + g % 2][2j + g / 2], g < 4.
+__global__ __launch_bounds__(kBlock) void focus_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int H, int W,
+                                                       size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int OH = H / 2, OW = W / 2;
+    const int ox = (int)(i % OW);
+    size_t t = i / OW;
+    const int oy = (int)(t % OH);
+    t /= OH;
+    const int p = (int)(t % (4 * C));
+    const size_t n = t / (4 * C);
+    const int g = p / C, c = p % C;
+    y[i] = x[((n * C + c) * H + 2 * oy + g % 2) * W + 2 * ox + g / 2];
+}
+
 // a + b (+ ReLU), four floats per thread where the arrays allow it
 __global__ __launch_bounds__(kBlock) void add_f32_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                          float* __restrict__ y, size_t n4, size_t count, int relu) {
@@ -760,6 +857,89 @@ extern "C" int exhip_conv2d_direct_nchw(exhip_ctx* ctx, const exhip_conv_desc* d
     const size_t total = (size_t)d->n * d->k * oh * ow;
     hipLaunchKernelGGL(conv_direct_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, wf, wq, fs, scale, bias, y,
                        d->c, d->h, d->w, d->k, oh, ow, d->kh, d->kw, d->sh, d->sw, d->pt, d->pl, groups, d->act, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+// ---- activation / glue layers ----
+template <int OP>
+static int launch_unary(exhip_ctx* ctx, const float* x, float* y, size_t count, float alpha, float beta) {
+    if (!count) return 0;
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0);
+    const size_t n4 = aligned ? count / 4 : 0;
+    const size_t threads = n4 + (count - n4 * 4);
+    hipLaunchKernelGGL((unary_f32_kernel<OP>), dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, x, y, n4, count, alpha, beta);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_unary_f32(exhip_ctx* ctx, int op, const float* x, float* y, size_t count, float alpha, float beta) {
+    REQ_CTX("exhip_unary_f32");
+    EXHIP_REQUIRE((x && y) || !count, "exhip_unary_f32: NULL tensor");
+    switch (op) {
+    case EXHIP_UNARY_HARDSWISH: return launch_unary<0>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_LEAKYRELU: return launch_unary<1>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_SIGMOID: return launch_unary<2>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_HARDSIGMOID: return launch_unary<3>(ctx, x, y, count, alpha, beta);
+    default: exhip_set_error("exhip_unary_f32: unknown op %d", op); return EXHIP_ERR_ARG;
+    }
+}
+
+extern "C" int exhip_channelwise_f32(exhip_ctx* ctx, int op, const float* x, float* y, int n, int c, int hw, const float* p0,
+                                     const float* p1, int shared) {
+    REQ_CTX("exhip_channelwise_f32");
+    EXHIP_REQUIRE(x && y && p0 && n > 0 && c > 0 && hw > 0, "exhip_channelwise_f32: bad argument");
+    EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || p1, "exhip_channelwise_f32: this op needs two parameter arrays");
+    EXHIP_REQUIRE((long long)n * c <= 65535, "exhip_channelwise_f32: more than 65535 (image, channel) planes");
+    unsigned bx = blocks_for((size_t)hw);
+    if (bx > 64) bx = 64;
+    const dim3 grid(bx, (unsigned)(n * c));
+    switch (op) {
+    case EXHIP_CHANNEL_PRELU: hipLaunchKernelGGL((channelwise_f32_kernel<0>), grid, dim3(kBlock), 0, ctx->stream, x, y, c, hw, p0, p1, shared); break;
+    case EXHIP_CHANNEL_BATCHNORM: hipLaunchKernelGGL((channelwise_f32_kernel<1>), grid, dim3(kBlock), 0, ctx->stream, x, y, c, hw, p0, p1, 0); break;
+    case EXHIP_CHANNEL_INPUT: hipLaunchKernelGGL((channelwise_f32_kernel<2>), grid, dim3(kBlock), 0, ctx->stream, x, y, c, hw, p0, p1, 0); break;
+    default: exhip_set_error("exhip_channelwise_f32: unknown op %d", op); return EXHIP_ERR_ARG;
+    }
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_concat_channels_f32(exhip_ctx* ctx, const float* const* inputs, const int* channels, int n_inputs, int n,
+                                         int hw, float* y) {
+    REQ_CTX("exhip_concat_channels_f32");
+    EXHIP_REQUIRE(inputs && channels && y && n_inputs > 0 && n > 0 && hw > 0 && n <= 65535, "exhip_concat_channels_f32: bad argument");
+    size_t total_c = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        EXHIP_REQUIRE(inputs[i] && channels[i] > 0, "exhip_concat_channels_f32: bad input %d", i);
+        total_c += channels[i];
+    }
+    size_t off = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        const size_t block = (size_t)channels[i] * hw;
+        unsigned bx = blocks_for(block);
+        if (bx > 1024) bx = 1024;
+        hipLaunchKernelGGL(concat_block_kernel, dim3(bx, (unsigned)n), dim3(kBlock), 0, ctx->stream, inputs[i], y, block, total_c * hw, off);
+        EXHIP_LAUNCH_CHECK();
+        off += block;
+    }
+    return 0;
+}
+
+extern "C" int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w, int oh, int ow) {
+    REQ_CTX("exhip_interp_nearest_f32");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 0 && w > 0 && oh > 0 && ow > 0, "exhip_interp_nearest_f32: bad argument");
+    const size_t total = (size_t)n * c * oh * ow;
+    hipLaunchKernelGGL(interp_nearest_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, oh, ow, h / (float)oh,
+                       w / (float)ow, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w) {
+    REQ_CTX("exhip_focus_f32");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 1 && w > 1, "exhip_focus_f32: bad argument");
+    const size_t total = (size_t)n * 4 * c * (h / 2) * (w / 2);
+    hipLaunchKernelGGL(focus_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

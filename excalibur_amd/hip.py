@@ -308,6 +308,42 @@ class Ctx:
         _check(lib().exhip_relu_f32(self.h, x.ptr, y.ptr, ctypes.c_size_t(y.size)))
         return y
 
+    # ---- activation / glue layers ----
+    UNARY = {"hardswish": 0, "leakyrelu": 1, "sigmoid": 2, "hardsigmoid": 3}
+    CHANNEL = {"prelu": 0, "batchnorm": 1, "input": 2}
+
+    def unary_f32(self, op, x, alpha=0.0, beta=0.0):
+        y = self.empty(x.shape, np.float32)
+        _check(lib().exhip_unary_f32(self.h, self.UNARY[op], x.ptr, y.ptr, ctypes.c_size_t(y.size), ctypes.c_float(float(alpha)),
+                                     ctypes.c_float(float(beta))))
+        return y
+
+    def channelwise_f32(self, op, x, p0, p1=None, shared=False):
+        n, c, h, w = x.shape
+        y = self.empty(x.shape, np.float32)
+        _check(lib().exhip_channelwise_f32(self.h, self.CHANNEL[op], x.ptr, y.ptr, n, c, h * w, p0.ptr, _ptr(p1), int(shared)))
+        return y
+
+    def concat_channels_f32(self, inputs):
+        n, _, h, w = inputs[0].shape
+        ptrs = (ctypes.c_void_p * len(inputs))(*[a.ptr.value for a in inputs])
+        ch = (ctypes.c_int * len(inputs))(*[a.shape[1] for a in inputs])
+        y = self.empty((n, sum(a.shape[1] for a in inputs), h, w), np.float32)
+        _check(lib().exhip_concat_channels_f32(self.h, ptrs, ch, len(inputs), n, h * w, y.ptr))
+        return y
+
+    def interp_nearest_f32(self, x, oh, ow):
+        n, c, h, w = x.shape
+        y = self.empty((n, c, oh, ow), np.float32)
+        _check(lib().exhip_interp_nearest_f32(self.h, x.ptr, y.ptr, n, c, h, w, oh, ow))
+        return y
+
+    def focus_f32(self, x):
+        n, c, h, w = x.shape
+        y = self.empty((n, 4 * c, h // 2, w // 2), np.float32)
+        _check(lib().exhip_focus_f32(self.h, x.ptr, y.ptr, n, c, h, w))
+        return y
+
     def add_f16(self, a, b, relu=False):
         y = self.empty(a.shape, np.uint16)
         _check(lib().exhip_add_f16(self.h, a.ptr, b.ptr, y.ptr, ctypes.c_size_t(y.size), int(relu)))

@@ -81,7 +81,9 @@ protected:
     virtual void forward_cpu_f16(const tensor_list<unsigned short>&, tensor_list<unsigned short>&) { NO_CPU; }
     virtual void forward_cpu_i8(const tensor_list<float>&, tensor_list<float>&) { NO_CPU; }
     virtual void forward_gpu_f32(const tensor_list<float>&, tensor_list<float>&) { NOT_IMPLEMENTED; }
-    virtual void forward_gpu_f16(const tensor_list<unsigned short>&, tensor_list<unsigned short>&) { NOT_IMPLEMENTED; }
+    // Default fp16 layer: the float32 operator on converted data, as the reference's CPU wrapper does
+    // (include/Excalibur/operation.hpp:204-266): half -> float, forward_gpu_f32, float -> half.
+    virtual void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops);
     virtual void forward_gpu_i8(const tensor_list<float>&, tensor_list<float>&) {
         NOT_IMPLEMENTED << " This function should be overrided in derived class";
     }

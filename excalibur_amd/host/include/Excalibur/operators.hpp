@@ -181,5 +181,137 @@ protected:
     void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 
+// ---- activation / glue layers of the shipped topologies (float32 kernels; fp16 pipelines take the base class's
+// convert-and-call wrapper) ----
+
+// HardSwish, LeakyRelu, Sigmoid, HardSigmoid: one elementwise kernel with two parameters.
+// src/Excalibur/operation_hardswish.cpp:10-63, operation_leakyrelu.cpp:12-58, operation_sigmoid.cpp:10-33,
+// operation_hardsigmoid.cpp:10-46 (keys 0 = alpha, 1 = beta).
+template <typename Dtype>
+class operation_unary : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    operation_unary(const operation_param& param, int op, float alpha, float beta, int n_keys);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int op_;
+    float alpha_, beta_;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+template <typename Dtype>
+struct operation_hardswish : operation_unary<Dtype> {
+    explicit operation_hardswish(const operation_param& p) : operation_unary<Dtype>(p, EXHIP_UNARY_HARDSWISH, 0.f, 0.f, 2) {}
+};
+template <typename Dtype>
+struct operation_leakyrelu : operation_unary<Dtype> {
+    explicit operation_leakyrelu(const operation_param& p) : operation_unary<Dtype>(p, EXHIP_UNARY_LEAKYRELU, 0.f, 0.f, 1) {}
+};
+template <typename Dtype>
+struct operation_sigmoid : operation_unary<Dtype> {
+    explicit operation_sigmoid(const operation_param& p) : operation_unary<Dtype>(p, EXHIP_UNARY_SIGMOID, 0.f, 0.f, 0) {}
+};
+template <typename Dtype>
+struct operation_hardsigmoid : operation_unary<Dtype> {
+    explicit operation_hardsigmoid(const operation_param& p) : operation_unary<Dtype>(p, EXHIP_UNARY_HARDSIGMOID, 0.2f, 0.5f, 2) {}
+};
+
+// src/Excalibur/operation_prelu.cpp:9-124: key 0 = number of slopes (1 = shared), blob = the slopes.
+template <typename Dtype>
+class operation_prelu : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_prelu(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int init_weights() override;
+    int init_weights(FILE* fp) override;
+    int num_slope_ = 0;
+    bool share_channel_ = false;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_batchnorm.cpp:10-156: keys 0 = channels, 1 = eps; blob = slope, mean, var, bias;
+// a = bias - slope*mean/sqrt(var + eps), b = slope/sqrt(var + eps) at load time, y = b*x + a.
+template <typename Dtype>
+class operation_batchnorm : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_batchnorm(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int init_weights() override;
+    int init_weights(FILE* fp) override;
+    int channels_ = 0;
+    float eps_ = 0.f;
+    std::shared_ptr<memory::tensor<float>> a_, b_;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void fold();
+};
+
+// src/Excalibur/operation_input.cpp:10-151: keys 0/1/2 = w/h/c, 3 = means, 4 = scales; (x - mean[c]) * scale[c].
+template <typename Dtype>
+class operation_input : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_input(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int w_ = 0, h_ = 0, c_ = 0;
+    std::vector<float> means_, vars_;
+    std::shared_ptr<memory::tensor<float>> means_dev_, vars_dev_;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_concat.cpp:10-103: key 0 = axis - 2 (the files carry -1 for the channel axis).
+template <typename Dtype>
+class operation_concat : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_concat(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int axis_ = 0;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_interp.cpp:185-268: keys 0 = type (1 nearest), 1 -> width scale, 2 -> height scale,
+// 3 / 4 = output width / height, 6 = align corners. Nearest without align-corners is the form on the path.
+template <typename Dtype>
+class operation_interp : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_interp(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int resize_type_ = 0, output_width_ = 0, output_height_ = 0, align_corner_ = 0;
+    float width_scale_ = 1.f, height_scale_ = 1.f;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_yolov5focus.cpp:12-50.
+template <typename Dtype>
+class operation_yolov5focus : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_yolov5focus(const operation_param& param) : operation<Dtype>(param) {}
+    const char* type() const override { return this->params_.type_.c_str(); }
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
 }  // namespace excalibur
 }  // namespace glasssix

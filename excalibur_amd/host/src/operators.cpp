@@ -790,6 +790,273 @@ void operation_innerproduct<Dtype>::forward_gpu_f16(const tensor_list<unsigned s
     EXHIP_FATAL(exhip_f32_to_f16(this->ctx(), ft[0]->gpu_data(), tops[0]->mutable_gpu_data(), ft[0]->count()));
 }
 
+// ------------------------------------------------------------------ default fp16 layer
+template <typename Dtype>
+void operation<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    tensor_list<float> in32, out32(tops.size());
+    for (const auto& b : bottoms) {
+        auto f = std::make_shared<tensor<float>>(b->data_shape(), params_.device_, b->order());
+        EXHIP_FATAL(exhip_f16_to_f32(ctx(), b->gpu_data(), f->mutable_gpu_data(), f->count()));
+        in32.push_back(f);
+    }
+    forward_gpu_f32(in32, out32);
+    for (size_t i = 0; i < tops.size(); ++i) {
+        tops[i] = std::make_shared<tensor<unsigned short>>(out32[i]->data_shape(), params_.device_, out32[i]->order());
+        EXHIP_FATAL(exhip_f32_to_f16(ctx(), out32[i]->gpu_data(), tops[i]->mutable_gpu_data(), tops[i]->count()));
+    }
+}
+template void operation<float>::forward_gpu_f16(const tensor_list<unsigned short>&, tensor_list<unsigned short>&);
+template void operation<unsigned short>::forward_gpu_f16(const tensor_list<unsigned short>&, tensor_list<unsigned short>&);
+
+// ------------------------------------------------------------------ activation / glue layers
+template <typename Dtype>
+operation_unary<Dtype>::operation_unary(const operation_param& param, int op, float alpha, float beta, int n_keys)
+    : operation<Dtype>(param), op_(op), alpha_(alpha), beta_(beta) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0 && n_keys >= 1) alpha_ = a.as_float();
+        else if (key == 1 && n_keys >= 2) beta_ = a.as_float();
+        else if (key != -23330) LOG(FATAL) << "Un-supported " << param.type_ << " Attribution " << a.key;
+    }
+}
+
+template <typename Dtype>
+void operation_unary<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        tops[i] = std::make_shared<tensor<float>>(bottoms[i]->data_shape(), this->params_.device_, bottoms[i]->order());
+        EXHIP_FATAL(exhip_unary_f32(this->ctx(), op_, bottoms[i]->gpu_data(), tops[i]->mutable_gpu_data(), tops[i]->count(), alpha_, beta_));
+    }
+}
+
+template <typename Dtype>
+operation_prelu<Dtype>::operation_prelu(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) {
+            num_slope_ = a.as_int();
+            CHECK_GE(num_slope_, 1);
+            share_channel_ = num_slope_ == 1;
+        } else if (key != -23330) {
+            LOG(FATAL) << "Un-supported PReLU Attribution " << a.key;
+        }
+    }
+    this->params_.inplace_ = true;
+}
+
+template <typename Dtype>
+int operation_prelu<Dtype>::init_weights(FILE* fp) {
+    this->weights_f32_.push_back(vec_tensor<float>(num_slope_, this->params_.device_));
+    if (std::fread(this->weights_f32_[0]->mutable_cpu_data(), sizeof(float), num_slope_, fp) != static_cast<size_t>(num_slope_))
+        LOG(FATAL) << "PReLU: model file too short";
+    return num_slope_ * static_cast<int>(sizeof(float));
+}
+
+template <typename Dtype>
+int operation_prelu<Dtype>::init_weights() {
+    this->weights_f32_.push_back(vec_tensor<float>(num_slope_, this->params_.device_));
+    float* s = this->weights_f32_[0]->mutable_cpu_data();
+    for (int i = 0; i < num_slope_; ++i) s[i] = 0.25f;  // dummy weights
+    return num_slope_ * static_cast<int>(sizeof(float));
+}
+
+template <typename Dtype>
+void operation_prelu<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        const auto& b = bottoms[i];
+        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+        if (!share_channel_) CHECK_EQ(b->channels(), num_slope_);
+        tops[i] = std::make_shared<tensor<float>>(b->data_shape(), this->params_.device_, b->order());
+        EXHIP_FATAL(exhip_channelwise_f32(this->ctx(), EXHIP_CHANNEL_PRELU, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(), b->channels(),
+                                          b->height() * b->width(), this->weights_f32_[0]->gpu_data(), nullptr, share_channel_ ? 1 : 0));
+    }
+}
+
+template <typename Dtype>
+operation_batchnorm<Dtype>::operation_batchnorm(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) channels_ = a.as_int();
+        else if (key == 1) eps_ = static_cast<float>(std::atof(a.value.c_str()));
+        else LOG(FATAL) << "Un-supported Batchnorm Attribution " << a.key;
+    }
+    this->params_.inplace_ = true;
+}
+
+// a = bias - slope*mean/sqrt(var + eps), b = slope/sqrt(var + eps) in float, the root taken in double
+// (src/Excalibur/operation_batchnorm.cpp:52-64)
+template <typename Dtype>
+void operation_batchnorm<Dtype>::fold() {
+    const float *slope = this->weights_f32_[0]->cpu_data(), *mean = this->weights_f32_[1]->cpu_data(),
+                *var = this->weights_f32_[2]->cpu_data(), *bias = this->weights_f32_[3]->cpu_data();
+    a_ = vec_tensor<float>(channels_, this->params_.device_);
+    b_ = vec_tensor<float>(channels_, this->params_.device_);
+    float *a = a_->mutable_cpu_data(), *b = b_->mutable_cpu_data();
+    for (int i = 0; i < channels_; ++i) {
+        volatile float sum = var[i] + eps_;
+        const float sqrt_var = static_cast<float>(std::sqrt(static_cast<double>(sum)));
+        volatile float prod = slope[i] * mean[i];
+        volatile float quot = prod / sqrt_var;
+        a[i] = bias[i] - quot;
+        b[i] = slope[i] / sqrt_var;
+    }
+}
+
+template <typename Dtype>
+int operation_batchnorm<Dtype>::init_weights(FILE* fp) {
+    for (int k = 0; k < 4; ++k) {
+        this->weights_f32_.push_back(vec_tensor<float>(channels_, this->params_.device_));
+        if (std::fread(this->weights_f32_[k]->mutable_cpu_data(), sizeof(float), channels_, fp) != static_cast<size_t>(channels_))
+            LOG(FATAL) << "BatchNorm: model file too short";
+    }
+    fold();
+    return channels_ * static_cast<int>(sizeof(float)) * 4;
+}
+
+template <typename Dtype>
+int operation_batchnorm<Dtype>::init_weights() {
+    const float init[4] = {1.f, 0.f, 1.f, 0.f};  // dummy weights: identity
+    for (int k = 0; k < 4; ++k) {
+        this->weights_f32_.push_back(vec_tensor<float>(channels_, this->params_.device_));
+        float* p = this->weights_f32_[k]->mutable_cpu_data();
+        for (int i = 0; i < channels_; ++i) p[i] = init[k];
+    }
+    fold();
+    return channels_ * static_cast<int>(sizeof(float)) * 4;
+}
+
+template <typename Dtype>
+void operation_batchnorm<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        const auto& b = bottoms[i];
+        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+        CHECK_EQ(b->channels(), channels_);
+        tops[i] = std::make_shared<tensor<float>>(b->data_shape(), this->params_.device_, b->order());
+        EXHIP_FATAL(exhip_channelwise_f32(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(),
+                                          b->channels(), b->height() * b->width(), a_->gpu_data(), b_->gpu_data(), 0));
+    }
+}
+
+template <typename Dtype>
+operation_input<Dtype>::operation_input(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) w_ = a.as_int();
+        else if (key == 1) h_ = a.as_int();
+        else if (key == 2) c_ = a.as_int();
+        else if (key == 3) {
+            for (const std::string& v : split_string(a.value, ",")) means_.push_back(static_cast<float>(std::atof(v.c_str())));
+        } else if (key == 4) {
+            for (const std::string& v : split_string(a.value, ",")) vars_.push_back(static_cast<float>(std::atof(v.c_str())));
+            if (c_ != 1 && c_ != static_cast<int>(vars_.size())) {  // one scale given for several channels (:42-48)
+                if (!vars_.empty()) vars_.resize(1);
+                for (int i = 1; i < c_; ++i) vars_.push_back(vars_[0]);
+            }
+        } else if (key != -23330) {
+            LOG(FATAL) << "Un-supported Input Attribution " << a.key;
+        }
+    }
+}
+
+template <typename Dtype>
+void operation_input<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        const auto& b = bottoms[i];
+        const int ch = b->channels();
+        if (ch != 1 && ch != 3) LOG(FATAL) << "Un-supprted channel num: " << ch;
+        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+        CHECK_EQ(static_cast<size_t>(ch), means_.size());
+        CHECK_GE(vars_.size(), static_cast<size_t>(ch));
+        if (!means_dev_) {
+            means_dev_ = vec_tensor<float>(ch, this->params_.device_);
+            vars_dev_ = vec_tensor<float>(ch, this->params_.device_);
+            for (int c = 0; c < ch; ++c) {
+                means_dev_->mutable_cpu_data()[c] = means_[c];
+                vars_dev_->mutable_cpu_data()[c] = vars_[c];
+            }
+        }
+        tops[i] = std::make_shared<tensor<float>>(b->data_shape(), this->params_.device_, b->order());
+        EXHIP_FATAL(exhip_channelwise_f32(this->ctx(), EXHIP_CHANNEL_INPUT, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(), ch,
+                                          b->height() * b->width(), means_dev_->gpu_data(), vars_dev_->gpu_data(), 0));
+    }
+}
+
+template <typename Dtype>
+operation_concat<Dtype>::operation_concat(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) axis_ = static_cast<int>(std::atof(a.value.c_str()));
+        else if (key != -23330) LOG(FATAL) << "Un-supported Concat Attribution " << a.key;
+    }
+}
+
+template <typename Dtype>
+void operation_concat<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_GE(bottoms.size(), 2);
+    CHECK_EQ(tops.size(), 1);
+    const int concat_axis = axis_ + 2;  // the files store the axis shifted (src/Excalibur/operation_concat.cpp:36-40)
+    if (concat_axis != 1 || bottoms[0]->order() != memory::NCHW) NOT_IMPLEMENTED << " Concat along axis " << concat_axis;
+    std::vector<const float*> ptrs;
+    std::vector<int> channels;
+    int total = 0;
+    for (const auto& b : bottoms) {
+        CHECK_EQ(b->num(), bottoms[0]->num());
+        CHECK_EQ(b->height(), bottoms[0]->height());
+        CHECK_EQ(b->width(), bottoms[0]->width());
+        ptrs.push_back(b->gpu_data());
+        channels.push_back(b->channels());
+        total += b->channels();
+    }
+    const auto& b0 = bottoms[0];
+    tops[0] = new_tensor<float>({b0->num(), total, b0->height(), b0->width()}, this->params_.device_);
+    EXHIP_FATAL(exhip_concat_channels_f32(this->ctx(), ptrs.data(), channels.data(), static_cast<int>(ptrs.size()), b0->num(),
+                                          b0->height() * b0->width(), tops[0]->mutable_gpu_data()));
+}
+
+template <typename Dtype>
+operation_interp<Dtype>::operation_interp(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        switch (std::atoi(a.key.c_str())) {
+        case 0: resize_type_ = a.as_int(); break;
+        case 1: width_scale_ = a.as_float(); break;   // sic: key 1 feeds the width scale (operation_interp.cpp:196-201)
+        case 2: height_scale_ = a.as_float(); break;
+        case 3: output_width_ = a.as_int(); break;
+        case 4: output_height_ = a.as_int(); break;
+        case 6: align_corner_ = a.as_int(); break;
+        default: LOG(FATAL) << "Un-supported Interp Attribution " << a.key;
+        }
+    }
+}
+
+template <typename Dtype>
+void operation_interp<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const auto& b = bottoms[0];
+    if (resize_type_ != 1 || align_corner_ != 0 || b->order() != memory::NCHW) NOT_IMPLEMENTED << " Interp type " << resize_type_;
+    int oh = output_height_, ow = output_width_;
+    if (oh == 0 || ow == 0) {
+        oh = static_cast<int>(b->height() * height_scale_);
+        ow = static_cast<int>(b->width() * width_scale_);
+    }
+    tops[0] = new_tensor<float>({b->num(), b->channels(), oh, ow}, this->params_.device_);
+    EXHIP_FATAL(exhip_interp_nearest_f32(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num(), b->channels(), b->height(),
+                                         b->width(), oh, ow));
+}
+
+template <typename Dtype>
+void operation_yolov5focus<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const auto& b = bottoms[0];
+    if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+    tops[0] = new_tensor<float>({b->num(), b->channels() * 4, b->height() / 2, b->width() / 2}, this->params_.device_);
+    EXHIP_FATAL(exhip_focus_f32(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num(), b->channels(), b->height(), b->width()));
+}
+
 INSTANCE_CLASS(operation_general_conv);
 INSTANCE_CLASS(operation_convolution);
 INSTANCE_CLASS(operation_convolutiondepthwise);
@@ -799,6 +1066,17 @@ INSTANCE_CLASS(operation_binaryop);
 INSTANCE_CLASS(operation_relu);
 INSTANCE_CLASS(operation_split);
 INSTANCE_CLASS(operation_innerproduct);
+INSTANCE_CLASS(operation_unary);
+INSTANCE_CLASS(operation_hardswish);
+INSTANCE_CLASS(operation_leakyrelu);
+INSTANCE_CLASS(operation_sigmoid);
+INSTANCE_CLASS(operation_hardsigmoid);
+INSTANCE_CLASS(operation_prelu);
+INSTANCE_CLASS(operation_batchnorm);
+INSTANCE_CLASS(operation_input);
+INSTANCE_CLASS(operation_concat);
+INSTANCE_CLASS(operation_interp);
+INSTANCE_CLASS(operation_yolov5focus);
 
 REGISTE(operation_convolution);
 REGISTE(operation_convolutiondepthwise);
@@ -808,6 +1086,16 @@ REGISTE(operation_binaryop);
 REGISTE(operation_relu);
 REGISTE(operation_split);
 REGISTE(operation_innerproduct);
+REGISTE(operation_hardswish);
+REGISTE(operation_leakyrelu);
+REGISTE(operation_sigmoid);
+REGISTE(operation_hardsigmoid);
+REGISTE(operation_prelu);
+REGISTE(operation_batchnorm);
+REGISTE(operation_input);
+REGISTE(operation_concat);
+REGISTE(operation_interp);
+REGISTE(operation_yolov5focus);
 
 }  // namespace excalibur
 }  // namespace glasssix

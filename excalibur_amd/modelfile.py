@@ -57,6 +57,12 @@ def conv_blob_i8(w, bias, ws, fs):
 fc_blob_f32 = conv_blob_f32
 
 
+def floats_blob(*arrays):
+    """Untagged float arrays one after the other: PReLU slopes (src/Excalibur/operation_prelu.cpp:36-41), BatchNorm
+    slope / mean / var / bias (src/Excalibur/operation_batchnorm.cpp:33-50)."""
+    return b"".join(np.ascontiguousarray(a, np.float32).tobytes() for a in arrays)
+
+
 def write_model(path, blobs):
     with open(path, "wb") as f:
         for b in blobs:

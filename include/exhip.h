@@ -178,6 +178,32 @@ int exhip_relu_f32(exhip_ctx* ctx, const float* x, float* y, size_t count);
 int exhip_add_f16(exhip_ctx* ctx, const uint16_t* a, const uint16_t* b, uint16_t* y, size_t count, int relu);
 int exhip_relu_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, size_t count);
 
+/* Elementwise activations of the shipped topologies. HardSwish x * clamp(alpha*x + beta, 0, 1)
+ * (src/Excalibur/operation_hardswish.cpp:32-63), LeakyReLU (operation_leakyrelu.cpp:31-58), sigmoid evaluated in double
+ * (operation_sigmoid.cpp:17-33), HardSigmoid clamp(alpha*x + beta, 0, 1) (operation_hardsigmoid.cpp:33-46). */
+#define EXHIP_UNARY_HARDSWISH 0
+#define EXHIP_UNARY_LEAKYRELU 1
+#define EXHIP_UNARY_SIGMOID 2
+#define EXHIP_UNARY_HARDSIGMOID 3
+int exhip_unary_f32(exhip_ctx* ctx, int op, const float* x, float* y, size_t count, float alpha, float beta);
+/* Per-channel layers on NCHW float tensors: PReLU, p0 = slope[c] or one shared slope (operation_prelu.cpp:57-124);
+ * BatchNorm as fma(p1[c], x, p0[c]) with a = p0, b = p1 computed at load time (operation_batchnorm.cpp:52-64,122-156);
+ * Input (x - p0[c]) * p1[c] (operation_input.cpp:61-151). p0 / p1: device arrays of c floats. */
+#define EXHIP_CHANNEL_PRELU 0
+#define EXHIP_CHANNEL_BATCHNORM 1
+#define EXHIP_CHANNEL_INPUT 2
+int exhip_channelwise_f32(exhip_ctx* ctx, int op, const float* x, float* y, int n, int c, int hw, const float* p0,
+                          const float* p1, int shared);
+/* operation_concat::forward_cpu_f32 along the channel axis (operation_concat.cpp:31-103): inputs is a host array of
+ * device pointers to NCHW tensors [n][channels[i]][hw]. */
+int exhip_concat_channels_f32(exhip_ctx* ctx, const float* const* inputs, const int* channels, int n_inputs, int n, int hw,
+                              float* y);
+/* operation_interp::forward_cpu_f32, nearest branch (operation_interp.cpp:247-268). */
+int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w, int oh, int ow);
+/* operation_yolov5focus::forward_cpu_f32 (operation_yolov5focus.cpp:17-50), for every image of the batch
+ * (the reference fills image 0 only). y: [n][4c][h/2][w/2]. */
+int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w);
+
 /* operation_innerproduct::forward_cpu_f32 (src/Excalibur/operation_innerproduct.cpp:176-224):
  * y[m,n] = sum_k x[m,k]*w[n,k] + bias[n]; x [m][k_in], w [n_out][k_in] row-major f32. */
 int exhip_innerproduct_f32(exhip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, int m,

@@ -406,3 +406,121 @@ void exo_float2half(const float* x, uint16_t* y, int length) {
 void exo_half2float(const uint16_t* x, float* y, int length) {
     for (int i = 0; i < length; ++i) y[i] = exo_float16_to_float32(x[i]);
 }
+
+/* ---- activation / glue layers of the shipped topologies ---- */
+
+/* operation_hardswish::forward_cpu_f32, src/Excalibur/operation_hardswish.cpp:32-63: y = x * clamp(alpha*x + beta, 0, 1).
+ * The vector body fuses alpha*x + beta (_mm256_fmadd_ps, :45); the scalar tail's alpha*x + beta (:59) is contracted to an
+ * FMA by the reference's compiler flags as well. */
+void exo_hardswish_f32(const float* x, float* y, long count, float alpha, float beta) {
+    for (long i = 0; i < count; ++i) {
+        float t = fmaf(x[i], alpha, beta);
+        t = t > 0.f ? t : 0.f;
+        t = t < 1.f ? t : 1.f;
+        y[i] = t * x[i];
+    }
+}
+
+/* operation_leakyrelu::forward_cpu_f32, src/Excalibur/operation_leakyrelu.cpp:31-58: body max(0,x) + min(0,x)*alpha,
+ * tail x < 0 ? alpha*x : x: the same values (the sign of a zero result aside). */
+void exo_leakyrelu_f32(const float* x, float* y, long count, float alpha) {
+    for (long i = 0; i < count; ++i) y[i] = x[i] < 0.f ? alpha * x[i] : x[i];
+}
+
+/* operation_sigmoid::forward_cpu_f32, src/Excalibur/operation_sigmoid.cpp:17-33: 1. / (1. + exp(-x)) in double. */
+void exo_sigmoid_f32(const float* x, float* y, long count) {
+    for (long i = 0; i < count; ++i) y[i] = (float)(1. / (1. + exp(-(double)x[i])));
+}
+
+/* operation_hardsigmoid::forward_cpu_f32, src/Excalibur/operation_hardsigmoid.cpp:33-46:
+ * max(0, min(1, alpha*x + beta)), the sum contracted to an FMA by the reference's compiler flags. */
+void exo_hardsigmoid_f32(const float* x, float* y, long count, float alpha, float beta) {
+    for (long i = 0; i < count; ++i) {
+        float t = fmaf(alpha, x[i], beta);
+        t = 1.f < t ? 1.f : t;
+        y[i] = 0.f < t ? t : 0.f;
+    }
+}
+
+/* operation_prelu::forward_cpu_f32, src/Excalibur/operation_prelu.cpp:57-124 (NCHW): slope per channel, or one shared
+ * slope when 0=1 (:19-22); body max(0,x) + slope*min(0,x), tail x >= 0 ? x : slope*x. */
+void exo_prelu_f32(const float* x, float* y, int n, int c, int hw, const float* slope, int shared) {
+    for (int i = 0; i < n * c; ++i) {
+        const float s = slope[shared ? 0 : i % c];
+        for (int j = 0; j < hw; ++j) {
+            const float v = x[(size_t)i * hw + j];
+            y[(size_t)i * hw + j] = v >= 0.f ? v : s * v;
+        }
+    }
+}
+
+/* operation_batchnorm, src/Excalibur/operation_batchnorm.cpp:33-66 (load time) and :122-156 (forward):
+ * sqrt_var = (float)sqrt(var + eps); a = bias - slope*mean/sqrt_var; b = slope/sqrt_var; y = b*x + a, which the
+ * reference's flags contract to an FMA. a and b are returned for the caller that wants them (ab may be NULL). */
+void exo_batchnorm_f32(const float* x, float* y, int n, int c, int hw, const float* slope, const float* mean,
+                       const float* var, const float* bias, float eps, float* ab) {
+    for (int ch = 0; ch < c; ++ch) {
+        const float sqrt_var = (float)sqrt((double)(var[ch] + eps));
+        const float a = bias[ch] - slope[ch] * mean[ch] / sqrt_var;
+        const float b = slope[ch] / sqrt_var;
+        if (ab) { ab[ch] = a; ab[c + ch] = b; }
+        for (int i = 0; i < n; ++i)
+            for (int j = 0; j < hw; ++j) {
+                const size_t o = ((size_t)i * c + ch) * hw + j;
+                y[o] = fmaf(b, x[o], a);
+            }
+    }
+}
+
+/* operation_input::forward_cpu_f32, src/Excalibur/operation_input.cpp:61-151 (NCHW): (x - mean[c]) * var[c];
+ * only 1- and 3-channel tensors are accepted (:78,126,143-146). */
+void exo_input_f32(const float* x, float* y, int n, int c, int hw, const float* mean, const float* scale) {
+    if (c != 1 && c != 3) abort();
+    for (int i = 0; i < n * c; ++i)
+        for (int j = 0; j < hw; ++j) y[(size_t)i * hw + j] = (x[(size_t)i * hw + j] - mean[i % c]) * scale[i % c];
+}
+
+/* operation_concat::forward_cpu_f32, channel axis (file key 0=-1 -> axis 1), NCHW,
+ * src/Excalibur/operation_concat.cpp:31-103: per image, the inputs' channel blocks one after the other. */
+void exo_concat_channels_f32(const float* const* xs, const int* channels, int n_inputs, int n, int hw, float* y) {
+    int total = 0;
+    for (int i = 0; i < n_inputs; ++i) total += channels[i];
+    for (int img = 0; img < n; ++img) {
+        size_t off = 0;
+        for (int i = 0; i < n_inputs; ++i) {
+            const size_t cnt = (size_t)channels[i] * hw;
+            memcpy(y + (size_t)img * total * hw + off, xs[i] + (size_t)img * cnt, cnt * sizeof(float));
+            off += cnt;
+        }
+    }
+}
+
+/* operation_interp::forward_cpu_f32, nearest branch (0=1, align_corner 0), src/Excalibur/operation_interp.cpp:247-268:
+ * in_y = min((int)(y * hs), h - 1) with hs = h / (float)oh, likewise for x; oh = (int)(h * height_scale) (:232-233). */
+void exo_interp_nearest_f32(const float* x, float* y, int n, int c, int h, int w, int oh, int ow) {
+    const float hs = h / (float)oh, ws = w / (float)ow;
+    for (int i = 0; i < n * c; ++i)
+        for (int oy = 0; oy < oh; ++oy) {
+            int iy = (int)(oy * hs);
+            if (iy > h - 1) iy = h - 1;
+            for (int ox = 0; ox < ow; ++ox) {
+                int ix = (int)(ox * ws);
+                if (ix > w - 1) ix = w - 1;
+                y[((size_t)i * oh + oy) * ow + ox] = x[((size_t)i * h + iy) * w + ix];
+            }
+        }
+}
+
+/* operation_yolov5focus::forward_cpu_f32, src/Excalibur/operation_yolov5focus.cpp:17-50: space to depth,
+ * out[p][i][j] = in[p % C][2i + (p / C) % 2][2j + (p / C) / 2], p < 4C. The reference fills image 0 only
+ * (offset(0, ...), :36-37); this restatement does every image the same way. */
+void exo_focus_f32(const float* x, float* y, int n, int c, int h, int w) {
+    const int oh = h / 2, ow = w / 2;
+    for (int img = 0; img < n; ++img)
+        for (int p = 0; p < 4 * c; ++p) {
+            const int g = p / c, ch = p % c, dy = g % 2, dx = g / 2;
+            for (int i = 0; i < oh; ++i)
+                for (int j = 0; j < ow; ++j)
+                    y[(((size_t)img * 4 * c + p) * oh + i) * ow + j] = x[(((size_t)img * c + ch) * h + 2 * i + dy) * w + 2 * j + dx];
+        }
+}

@@ -75,6 +75,18 @@ float exo_float16_to_float32(uint16_t v);
 void exo_float2half(const float* x, uint16_t* y, int length);
 void exo_half2float(const uint16_t* x, float* y, int length);
 
+void exo_hardswish_f32(const float* x, float* y, long count, float alpha, float beta);
+void exo_leakyrelu_f32(const float* x, float* y, long count, float alpha);
+void exo_sigmoid_f32(const float* x, float* y, long count);
+void exo_hardsigmoid_f32(const float* x, float* y, long count, float alpha, float beta);
+void exo_prelu_f32(const float* x, float* y, int n, int c, int hw, const float* slope, int shared);
+void exo_batchnorm_f32(const float* x, float* y, int n, int c, int hw, const float* slope, const float* mean,
+                       const float* var, const float* bias, float eps, float* ab);
+void exo_input_f32(const float* x, float* y, int n, int c, int hw, const float* mean, const float* scale);
+void exo_concat_channels_f32(const float* const* xs, const int* channels, int n_inputs, int n, int hw, float* y);
+void exo_interp_nearest_f32(const float* x, float* y, int n, int c, int h, int w, int oh, int ow);
+void exo_focus_f32(const float* x, float* y, int n, int c, int h, int w);
+
 #ifdef __cplusplus
 }
 #endif

@@ -221,3 +221,79 @@ def half2float(x):
     y = np.empty(x.shape, np.float32)
     lib().exo_half2float(_p(x), _p(y), x.size)
     return y
+
+
+# ---- activation / glue layers ----
+def _unary(fn, x, *scalars):
+    x = _f32(x)
+    y = np.empty(x.shape, np.float32)
+    fn(_p(x), _p(y), ctypes.c_long(y.size), *[ctypes.c_float(float(s)) for s in scalars])
+    return y
+
+
+def hardswish(x, alpha=1.0 / 6.0, beta=0.5):
+    return _unary(lib().exo_hardswish_f32, x, alpha, beta)
+
+
+def leakyrelu(x, alpha):
+    return _unary(lib().exo_leakyrelu_f32, x, alpha)
+
+
+def sigmoid(x):
+    return _unary(lib().exo_sigmoid_f32, x)
+
+
+def hardsigmoid(x, alpha=0.2, beta=0.5):
+    return _unary(lib().exo_hardsigmoid_f32, x, alpha, beta)
+
+
+def prelu(x, slope):
+    x, slope = _f32(x), _f32(slope)
+    n, c, h, w = x.shape
+    y = np.empty(x.shape, np.float32)
+    lib().exo_prelu_f32(_p(x), _p(y), n, c, h * w, _p(slope), int(slope.size == 1))
+    return y
+
+
+def batchnorm(x, slope, mean, var, bias, eps=0.0):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    y = np.empty(x.shape, np.float32)
+    lib().exo_batchnorm_f32(_p(x), _p(y), n, c, h * w, _p(_f32(slope)), _p(_f32(mean)), _p(_f32(var)), _p(_f32(bias)),
+                            ctypes.c_float(float(eps)), None)
+    return y
+
+
+def input_layer(x, mean, scale):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    y = np.empty(x.shape, np.float32)
+    lib().exo_input_f32(_p(x), _p(y), n, c, h * w, _p(_f32(mean)), _p(_f32(scale)))
+    return y
+
+
+def concat_channels(xs):
+    arrs = [_f32(a) for a in xs]
+    n, _, h, w = arrs[0].shape
+    ptrs = (ctypes.c_void_p * len(arrs))(*[a.ctypes.data for a in arrs])
+    ch = (ctypes.c_int * len(arrs))(*[a.shape[1] for a in arrs])
+    y = np.empty((n, sum(a.shape[1] for a in arrs), h, w), np.float32)
+    lib().exo_concat_channels_f32(ptrs, ch, len(arrs), n, h * w, _p(y))
+    return y
+
+
+def interp_nearest(x, height_scale, width_scale):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    oh, ow = int(np.float32(h) * np.float32(height_scale)), int(np.float32(w) * np.float32(width_scale))
+    y = np.empty((n, c, oh, ow), np.float32)
+    lib().exo_interp_nearest_f32(_p(x), _p(y), n, c, h, w, oh, ow)
+    return y
+
+
+def focus(x):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    y = np.empty((n, 4 * c, h // 2, w // 2), np.float32)
+    lib().exo_focus_f32(_p(x), _p(y), n, c, h, w)
+    return y

@@ -81,6 +81,34 @@ def fc_case(seed, m, c, h, w, n_out, bias=True):
                 bias=r.normal(0, 0.01, (n_out,)).astype(np.float32) if bias else None)
 
 
+def unary_case(seed, kind, shape, **params):
+    """kind: hardswish / leakyrelu / sigmoid / hardsigmoid / focus / interp (params: the layer's keys)."""
+    return dict(op=kind, x=_rng(seed).uniform(-4, 4, shape).astype(np.float32), **params)
+
+
+def prelu_case(seed, shape, shared=False):
+    r = _rng(seed)
+    return dict(op="prelu", x=r.uniform(-2, 2, shape).astype(np.float32),
+                slope=np.abs(r.normal(0, 0.3, (1 if shared else shape[1],))).astype(np.float32))
+
+
+def batchnorm_case(seed, shape, eps=1e-5):
+    r = _rng(seed)
+    c = shape[1]
+    return dict(op="batchnorm", x=r.uniform(-2, 2, shape).astype(np.float32), eps=eps,
+                slope=r.uniform(0.5, 1.5, (c,)).astype(np.float32), mean=r.normal(0, 0.5, (c,)).astype(np.float32),
+                var=r.uniform(0.2, 2.0, (c,)).astype(np.float32), bias=r.normal(0, 0.3, (c,)).astype(np.float32))
+
+
+def input_case(seed, shape, means, scales):
+    return dict(op="input", x=_rng(seed).uniform(0, 255, shape).astype(np.float32), means=list(means), scales=list(scales))
+
+
+def concat_case(seed, n, channels, h, w):
+    r = _rng(seed)
+    return dict(op="concat", xs=[r.uniform(-2, 2, (n, c, h, w)).astype(np.float32) for c in channels])
+
+
 def geom_of(case):
     return port.geom((case["n"], case["c"], case["h"], case["w"]), case["k"], case["kh"], case["kw"],
                      case["stride"], case["pad"], case["groups"])
@@ -108,6 +136,29 @@ def reference_io(case):
     if op == "fc":
         line = f"InnerProduct layer 1 1 data out 0={case['n_out']} 1={int(case['bias'] is not None)} 2={case['wt'].size}"
         return mf.topology([line]), mf.fc_blob_f32(case["wt"], case["bias"]), [case["x"]], "out"
+    if op == "hardswish":
+        return mf.topology([f"HardSwish layer 1 1 data out 0={case['alpha']!r} 1={case['beta']!r}"]), b"", [case["x"]], "out"
+    if op == "leakyrelu":
+        return mf.topology([f"LeakyRelu layer 1 1 data out 0={case['alpha']!r}"]), b"", [case["x"]], "out"
+    if op == "sigmoid":
+        return mf.topology(["Sigmoid layer 1 1 data out"]), b"", [case["x"]], "out"
+    if op == "hardsigmoid":
+        return mf.topology([f"HardSigmoid layer 1 1 data out 0={case['alpha']!r} 1={case['beta']!r}"]), b"", [case["x"]], "out"
+    if op == "focus":
+        return mf.topology(["Yolov5focus layer 1 1 data out"]), b"", [case["x"]], "out"
+    if op == "interp":
+        # key 1 is read into the width scale and key 2 into the height scale (src/Excalibur/operation_interp.cpp:196-201)
+        return mf.topology([f"Interp layer 1 1 data out 0=1 1={case['width_scale']!r} 2={case['height_scale']!r}"]), b"", [case["x"]], "out"
+    if op == "prelu":
+        return mf.topology([f"PReLU layer 1 1 data out 0={case['slope'].size}"]), mf.floats_blob(case["slope"]), [case["x"]], "out"
+    if op == "batchnorm":
+        line = f"BatchNorm layer 1 1 data out 0={case['x'].shape[1]} 1={case['eps']!r}"
+        return mf.topology([line]), mf.floats_blob(case["slope"], case["mean"], case["var"], case["bias"]), [case["x"]], "out"
+    if op == "input":
+        c_, h_, w_ = case["x"].shape[1:]
+        line = (f"Input layer 1 1 data out 0={w_} 1={h_} 2={c_} 3=" + ",".join(repr(float(v)) for v in case["means"]) +
+                " 4=" + ",".join(repr(float(v)) for v in case["scales"]))
+        return mf.topology([line]), b"", [case["x"]], "out"
     raise ValueError(op)
 
 
@@ -117,10 +168,11 @@ def multi_input_topology(case):
     Split_Slice layer (src/Excalibur/operation_split_slice.cpp:12-36, axis key 1=0 is the channel axis).
     -> (topology text, the concatenated input)."""
     n = len(case["xs"])
-    c = case["xs"][0].shape[1]
     names = " ".join(f"x{i}" for i in range(n))
-    lines = [f"Split_Slice cut 1 {n} data {names} 0={n}," + ",".join(str(c) for _ in range(n)) + " 1=0"]
-    if case["op"] == "eltwise":
+    lines = [f"Split_Slice cut 1 {n} data {names} 0={n}," + ",".join(str(a.shape[1]) for a in case["xs"]) + " 1=0"]
+    if case["op"] == "concat":
+        lines.append(f"Concat layer {n} 1 {names} out 0=-1")
+    elif case["op"] == "eltwise":
         extra = f"0={case['etype']}"
         if case.get("coeffs") is not None:
             extra += " -23301=" + ",".join([str(n + 1)] + [repr(float(v)) for v in case["coeffs"]])
@@ -152,6 +204,26 @@ def oracle_eval(case):
         return port.relu(case["x"])
     if op == "fc":
         return port.innerproduct(case["x"], case["wt"], case["bias"])
+    if op == "hardswish":
+        return port.hardswish(case["x"], case["alpha"], case["beta"])
+    if op == "leakyrelu":
+        return port.leakyrelu(case["x"], case["alpha"])
+    if op == "sigmoid":
+        return port.sigmoid(case["x"])
+    if op == "hardsigmoid":
+        return port.hardsigmoid(case["x"], case["alpha"], case["beta"])
+    if op == "focus":
+        return port.focus(case["x"])
+    if op == "interp":
+        return port.interp_nearest(case["x"], case["height_scale"], case["width_scale"])
+    if op == "prelu":
+        return port.prelu(case["x"], case["slope"])
+    if op == "batchnorm":
+        return port.batchnorm(case["x"], case["slope"], case["mean"], case["var"], case["bias"], case["eps"])
+    if op == "input":
+        return port.input_layer(case["x"], case["means"], case["scales"])
+    if op == "concat":
+        return port.concat_channels(case["xs"])
     raise ValueError(op)
 
 

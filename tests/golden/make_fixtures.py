@@ -60,6 +60,21 @@ def fixture_cases():
         # inner product
         "fc_bias": c.fc_case(46, 3, 8, 4, 4, 10),
         "fc_nobias": c.fc_case(47, 2, 16, 1, 1, 7, bias=False),
+        # activation / glue layers (element counts with and without a vector tail)
+        "hardswish": c.unary_case(60, "hardswish", (2, 3, 5, 7), alpha=1.0 / 6.0, beta=0.5),
+        "hardswish_ab": c.unary_case(61, "hardswish", (1, 4, 4, 4), alpha=0.25, beta=0.375),
+        "leakyrelu": c.unary_case(62, "leakyrelu", (2, 3, 5, 7), alpha=0.1),
+        "sigmoid": c.unary_case(63, "sigmoid", (2, 3, 5, 7)),
+        "hardsigmoid": c.unary_case(64, "hardsigmoid", (2, 3, 5, 7), alpha=0.2, beta=0.5),
+        "prelu_per_channel": c.prelu_case(65, (2, 6, 5, 7)),
+        "prelu_shared": c.prelu_case(66, (2, 6, 4, 4), shared=True),
+        "batchnorm": c.batchnorm_case(67, (2, 6, 5, 7)),
+        "input_3ch": c.input_case(68, (2, 3, 9, 11), (127.5, 120.0, 110.25), (0.0078125, 0.0125, 0.017)),
+        "input_1ch": c.input_case(69, (2, 1, 9, 11), (127.5,), (0.0078125,)),
+        "concat_channels": c.concat_case(70, 2, (3, 5, 2), 5, 7),
+        "interp_nearest_x2": c.unary_case(71, "interp", (2, 3, 5, 7), height_scale=2.0, width_scale=2.0),
+        "interp_nearest_frac": c.unary_case(72, "interp", (1, 2, 6, 5), height_scale=1.5, width_scale=2.5),
+        "focus": c.unary_case(73, "focus", (1, 3, 8, 10)),
     }
 
 

@@ -106,6 +106,31 @@ def gpu_eval(ctx, case):
     if op == "fc":
         return ctx.innerproduct_f32(ctx.array(case["x"]), ctx.array(case["wt"]),
                                     ctx.array(case["bias"]) if case["bias"] is not None else None).download()
+    if op in ("hardswish", "hardsigmoid"):
+        return ctx.unary_f32(op, ctx.array(case["x"]), case["alpha"], case["beta"]).download()
+    if op == "leakyrelu":
+        return ctx.unary_f32(op, ctx.array(case["x"]), case["alpha"]).download()
+    if op == "sigmoid":
+        return ctx.unary_f32(op, ctx.array(case["x"])).download()
+    if op == "prelu":
+        return ctx.channelwise_f32("prelu", ctx.array(case["x"]), ctx.array(case["slope"]), shared=case["slope"].size == 1).download()
+    if op == "batchnorm":
+        # a and b as the layer computes them when it loads (src/Excalibur/operation_batchnorm.cpp:52-64)
+        sqrt_var = np.sqrt((case["var"] + np.float32(case["eps"])).astype(np.float64)).astype(np.float32)
+        a = (case["bias"] - case["slope"] * case["mean"] / sqrt_var).astype(np.float32)
+        b = (case["slope"] / sqrt_var).astype(np.float32)
+        return ctx.channelwise_f32("batchnorm", ctx.array(case["x"]), ctx.array(a), ctx.array(b)).download()
+    if op == "input":
+        return ctx.channelwise_f32("input", ctx.array(case["x"]), ctx.array(np.asarray(case["means"], np.float32)),
+                                   ctx.array(np.asarray(case["scales"], np.float32))).download()
+    if op == "concat":
+        return ctx.concat_channels_f32([ctx.array(a) for a in case["xs"]]).download()
+    if op == "interp":
+        h, w = case["x"].shape[2:]
+        oh, ow = int(np.float32(h) * np.float32(case["height_scale"])), int(np.float32(w) * np.float32(case["width_scale"]))
+        return ctx.interp_nearest_f32(ctx.array(case["x"]), oh, ow).download()
+    if op == "focus":
+        return ctx.focus_f32(ctx.array(case["x"])).download()
     raise ValueError(op)
 
 

@@ -11,7 +11,7 @@ from tests import cases
 
 def run_reference(case, dtype="f32"):
     op = case["op"]
-    if op in ("eltwise", "binaryop_add"):
+    if op in ("eltwise", "binaryop_add", "concat"):
         topo, x = cases.multi_input_topology(case)
         return ref.run(topo, "", x, ["out"], dtype)["out"]
     topo, blob, xs, out = cases.reference_io(case)

@@ -42,7 +42,7 @@ def run_case(case, dtype="f32"):
 
 
 # the host layer registers Split_Slice only as far as the hot path needs it: multi-input cases use it to cut operands
-MULTI = ("eltwise", "binaryop")
+MULTI = ("eltwise", "binaryop", "concat")
 
 
 @pytest.mark.parametrize("name", [n for n in NAMES if not n.startswith("f16_") and not n.startswith(MULTI)])
@@ -154,6 +154,7 @@ def test_fused_plan_conv_then_maxpool_as_network_output(k, pool):
     ("Eltwise e 2 1 ra b out 0=2", lambda a, b: port.eltwise([a, b], port.ELT_MAX)),
     ("Eltwise e 2 1 ra b out 0=0", lambda a, b: port.eltwise([a, b], port.ELT_PROD)),
     ("BinaryOp e 2 1 ra b out 0=0", lambda a, b: port.binaryop_add(a, b)),
+    ("Concat e 2 1 ra b out 0=-1", lambda a, b: port.concat_channels([a, b])),
 ])
 def test_two_input_layers_through_split_aliasing(layer, evaluate):
     """Split hands one blob to two consumers (aliasing, as in the reference); the operands are relu(x) and x."""
@@ -164,3 +165,35 @@ def test_two_input_layers_through_split_aliasing(layer, evaluate):
     p.forward(x)
     assert np.array_equal(p.get("out"), evaluate(port.relu(x), x))
     p.close()
+
+
+def test_input_layer_without_bottoms_normalises_the_pipeline_input():
+    """`Input name 0 1 blob ...` (no bottoms): the pipeline input is `<name>_input`, the layer subtracts the means and
+    scales (one scale repeated over the channels), then a float convolution with PReLU behind it: fp32 and fp16."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(51)
+    x = r.uniform(0, 255, (2, 3, 12, 14)).astype(np.float32)
+    c = cases.conv_f32_case(52, 2, 3, 12, 14, 8, 3, 1, 1, act=0)
+    slope = np.abs(r.normal(0, 0.3, (8,))).astype(np.float32)
+    lines = ["Input data 0 1 data 0=14 1=12 2=3 3=123.0,117.0,104.0 4=0.0078125",
+             mf.conv_line("Convolution", "c", "data", "a", 8, 3, 1, 1, True, c["wt"].size, 1, act=0),
+             "PReLU p 1 1 a out 0=8"]
+    xin = port.input_layer(x, [123.0, 117.0, 104.0], [0.0078125] * 3)
+    c["x"] = xin
+    want = port.prelu(cases.oracle_eval(c), slope)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        f.write(mf.conv_blob_f32(c["wt"], c["bias"]) + mf.floats_blob(slope))
+        path = f.name
+    try:
+        p = xp.Pipeline(mf.topology(lines), path, 0)
+        p.forward(x)
+        assert np.array_equal(p.get("data"), xin)
+        assert cases.check_value(p.get("out"), want, 1e-4) == 0
+        p.close()
+        p16 = xp.Pipeline(mf.topology(lines), path, 0, "f16")
+        p16.forward(x.astype(np.float16).view(np.uint16))
+        got = p16.get("out").view(np.float16).astype(np.float32)
+        assert cases.check_value(got, want, 2e-2) == 0  # two half roundings of values up to 255 in front of the convolution
+        p16.close()
+    finally:
+        os.unlink(path)
