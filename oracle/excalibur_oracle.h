@@ -18,6 +18,10 @@
  *   exo_pool2d_f32, exo_eltwise_f32,
  *   exo_binaryop_add_f32, exo_relu_f32     reference fixtures (bit-exact)
  *   exo_float2half / exo_half2float        exhaustive round trip over all 65536 halfs + reference fixtures
+ *   exo_hardswish / leakyrelu / sigmoid /
+ *   hardsigmoid / prelu / batchnorm / input /
+ *   concat_channels / interp_nearest       reference fixtures (bit-exact), element counts with and without a vector tail
+ *   exo_focus_f32                          reference fixture (bit-exact) for one image; further images by the same formula
  * No function here is "parity unpinned".
  */
 #ifndef EXCALIBUR_ORACLE_H_

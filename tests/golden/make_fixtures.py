@@ -19,6 +19,9 @@ from tests import cases  # noqa: E402
 from tests.refrun import run_reference  # noqa: E402
 
 
+NETWORKS = ("net_mobilefacenet_f32",)  # whole-topology fixtures: not single-layer cases
+
+
 def fixture_cases():
     c = cases
     return {
@@ -133,6 +136,18 @@ def main():
         case = dict(case)
         case["x"] = case["x"].astype(np.float16).view(np.uint16)
         save_case(os.path.join(HERE, name + ".npz"), case, run_reference(case, dtype="f16"))
+    # one multi-layer float topology (generated by excalibur_amd.mobilenet from a seed): input and the reference's output
+    from excalibur_amd.mobilenet import MobileFaceNetF32
+    from oracle import ref
+    import tempfile
+    net = MobileFaceNetF32()
+    x = np.random.default_rng(8).uniform(0, 255, (2, 3, net.hw, net.hw)).astype(np.float32)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    net.write_model(path)
+    out = ref.run(net.topology(), path, x, [net.output])[net.output]
+    os.unlink(path)
+    np.savez_compressed(os.path.join(HERE, "net_mobilefacenet_f32.npz"), input_seed=np.asarray(8), expected=out)
     total = sum(os.path.getsize(os.path.join(HERE, f)) for f in os.listdir(HERE) if f.endswith(".npz"))
     print(f"wrote {len(fixture_cases()) + len(f16_cases())} fixtures, {total / 1024:.0f} KiB")
 

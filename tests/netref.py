@@ -50,3 +50,30 @@ def reference_forward(net, x, extra=()):
     finally:
         os.unlink(path)
     return outs
+
+
+def oracle_forward_mobilenet(net, x):
+    """The float MobileFaceNet-shaped network (excalibur_amd.mobilenet) op by op through the oracle restatement."""
+    blobs = {"data_input": np.ascontiguousarray(x, np.float32)}
+    for op in net.ops:
+        kind = op[0]
+        if kind == "input":
+            blobs["data"] = port.input_layer(blobs["data_input"], net.means, [net.scale] * 3)
+        elif kind in ("conv", "dw"):
+            _, bottom, top, w, b, kernel, stride, pad, groups = op
+            xin = blobs[bottom]
+            g = port.geom(xin.shape, w.shape[0], kernel, kernel, stride, pad, groups)
+            fn = port.dwconv_f32 if kind == "dw" else port.conv2d_f32
+            blobs[top] = fn(xin, w, b, 0, g)
+        elif kind == "prelu":
+            blobs[op[2]] = port.prelu(blobs[op[1]], op[3])
+        elif kind == "split":
+            for t in op[2]:
+                blobs[t] = blobs[op[1]]
+        elif kind == "sum":
+            blobs[op[2]] = port.eltwise([blobs[n] for n in op[1]], port.ELT_SUM)
+        elif kind == "gap":
+            blobs[op[2]] = port.pool2d(blobs[op[1]], port.POOL_AVE, global_pool=True)
+        elif kind == "fc":
+            blobs[op[2]] = port.innerproduct(blobs[op[1]], op[3], op[4])
+    return blobs[net.output], blobs

@@ -17,7 +17,7 @@ from tests.golden.make_fixtures import load_case
 pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
-NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")))
+NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(f).startswith("net_"))
 TOLERANT = ("conv_f32", "fc_")
 
 
@@ -194,6 +194,36 @@ def test_input_layer_without_bottoms_normalises_the_pipeline_input():
         p16.forward(x.astype(np.float16).view(np.uint16))
         got = p16.get("out").view(np.float16).astype(np.float32)
         assert cases.check_value(got, want, 2e-2) == 0  # two half roundings of values up to 255 in front of the convolution
+        p16.close()
+    finally:
+        os.unlink(path)
+
+
+def test_mobilefacenet_shaped_float_topology_matches_the_reference_fixture():
+    """Input -> conv/PReLU -> depthwise/pointwise bottlenecks with Eltwise residuals -> global average -> InnerProduct,
+    loaded from generated `.phai` + `.racy`: float32 against the compiled reference's output, float16 alongside."""
+    from excalibur_amd.mobilenet import MobileFaceNetF32
+    net = MobileFaceNetF32()
+    z = np.load(os.path.join(GOLDEN, "net_mobilefacenet_f32.npz"))
+    x = np.random.default_rng(int(z["input_seed"])).uniform(0, 255, (2, 3, net.hw, net.hw)).astype(np.float32)
+    expected = z["expected"]
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        net.write_model(path)
+        p = xp.Pipeline(net.topology(), path, 0)
+        p.forward(x)
+        got = p.get(net.output)
+        assert not p.fused
+        assert got.shape == expected.shape
+        assert cases.check_value(got, expected, 1e-4) == 0
+        want, blobs = netref.oracle_forward_mobilenet(net, x)
+        assert cases.check_value(p.get("b1_out"), blobs["b1_out"], 1e-4) == 0  # an intermediate blob by name
+        p.close()
+        p16 = xp.Pipeline(net.topology(), path, 0, "f16")
+        p16.forward(x.astype(np.float16).view(np.uint16))
+        got16 = p16.get(net.output).view(np.float16).astype(np.float32)
+        assert cases.check_value(got16, expected, 3e-2) == 0  # every layer rounds to half: error grows with depth
         p16.close()
     finally:
         os.unlink(path)

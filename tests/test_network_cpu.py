@@ -1,10 +1,12 @@
 """The ResNet-18-shaped int8 network description: the oracle chain against the compiled reference running the
 generated .phai/.racy through its own loader (marker `ref`), plus closed-form checks of the builder."""
+import os
+
 import numpy as np
 import pytest
 
 from excalibur_amd.resnet18 import ResNet18Int8
-from tests import netref
+from tests import cases, netref
 
 
 def test_algorithmic_work_matches_the_survey_figure():
@@ -25,3 +27,25 @@ def test_oracle_chain_equals_compiled_reference():
     assert np.array_equal(got["l2b1_out"], blobs["l2b1_out"])
     assert np.array_equal(got[net.output], want)
     assert want.shape == (2, 512, 2, 2) and np.count_nonzero(want) > want.size // 4
+
+
+@pytest.mark.ref
+def test_mobilefacenet_shaped_topology_oracle_equals_compiled_reference():
+    """The float multi-layer topology of excalibur_amd.mobilenet: the op-by-op oracle evaluation against the compiled
+    reference running the generated `.phai` / `.racy`, and against the committed fixture."""
+    import tempfile
+    from excalibur_amd.mobilenet import MobileFaceNetF32
+    from oracle import ref
+    net = MobileFaceNetF32()
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "net_mobilefacenet_f32.npz"))
+    x = np.random.default_rng(int(z["input_seed"])).uniform(0, 255, (2, 3, net.hw, net.hw)).astype(np.float32)
+    want, _ = netref.oracle_forward_mobilenet(net, x)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        net.write_model(path)
+        got = ref.run(net.topology(), path, x, [net.output])[net.output]
+    finally:
+        os.unlink(path)
+    assert np.array_equal(got, z["expected"])
+    assert cases.check_value(got.reshape(want.shape), want, 1e-4) == 0
