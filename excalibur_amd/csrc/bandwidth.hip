@@ -475,6 +475,40 @@ __global__ __launch_bounds__(kBlock) void focus_kernel(const float* __restrict__
     y[i] = x[((n * C + c) * H + 2 * oy + g % 2) * W + 2 * ox + g / 2];
 }
 
+// Transposed convolution by gathering (NCHW float32, group 1, dilation 1): output (k, oy, ox) sums, over the taps
+// (r, q) whose input pixel ((oy + pt - r) / sh, (ox + pl - q) / sw) exists, the products over the input channels.
+// Weights [C][K][kh][kw]. One thread per output element; the layers that use it are small upsampling heads.
+__global__ __launch_bounds__(kBlock) void deconv2d_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                              const float* __restrict__ bias, float* __restrict__ y, int C, int H,
+                                                              int W, int K, int KH, int KW, int SH, int SW, int PT, int PL, int OH,
+                                                              int OW, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int ox = (int)(i % OW);
+    size_t t = i / OW;
+    const int oy = (int)(t % OH);
+    t /= OH;
+    const int k = (int)(t % K);
+    const size_t n = t / K;
+    float acc = 0.f;
+    for (int r = 0; r < KH; ++r) {
+        const int ty = oy + PT - r;
+        if (ty < 0 || ty % SH) continue;
+        const int iy = ty / SH;
+        if (iy >= H) continue;
+        for (int q = 0; q < KW; ++q) {
+            const int tx = ox + PL - q;
+            if (tx < 0 || tx % SW) continue;
+            const int ix = tx / SW;
+            if (ix >= W) continue;
+            const float* xp = x + ((n * C) * H + iy) * W + ix;
+            const float* wp = w + ((size_t)k * KH + r) * KW + q;
+            for (int c = 0; c < C; ++c) acc = __builtin_fmaf(xp[(size_t)c * H * W], wp[(size_t)c * K * KH * KW], acc);
+        }
+    }
+    y[i] = bias ? acc + bias[k] : acc;
+}
+
 // a + b (+ ReLU), four floats per thread where the arrays allow it
 __global__ __launch_bounds__(kBlock) void add_f32_kernel(const float* __restrict__ a, const float* __restrict__ b,
                                                          float* __restrict__ y, size_t n4, size_t count, int relu) {
@@ -940,6 +974,20 @@ extern "C" int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, 
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 1 && w > 1, "exhip_focus_f32: bad argument");
     const size_t total = (size_t)n * 4 * c * (h / 2) * (w / 2);
     hipLaunchKernelGGL(focus_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_deconv2d_f32(exhip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, int n, int c, int h,
+                                  int wd, int k, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr) {
+    REQ_CTX("exhip_deconv2d_f32");
+    EXHIP_REQUIRE(x && w && y && n > 0 && c > 0 && h > 0 && wd > 0 && k > 0 && kh > 0 && kw > 0 && sh > 0 && sw > 0,
+                  "exhip_deconv2d_f32: bad argument");
+    const int oh = (h - 1) * sh + kh - (pt + pb), ow = (wd - 1) * sw + kw - (pl + pr);
+    EXHIP_REQUIRE(oh > 0 && ow > 0 && pt >= 0 && pl >= 0, "exhip_deconv2d_f32: empty output (%d x %d)", oh, ow);
+    const size_t total = (size_t)n * k * oh * ow;
+    hipLaunchKernelGGL(deconv2d_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, w, bias, y, c, h, wd, k, kh, kw, sh,
+                       sw, pt, pl, oh, ow, total);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -344,6 +344,15 @@ class Ctx:
         _check(lib().exhip_focus_f32(self.h, x.ptr, y.ptr, n, c, h, w))
         return y
 
+    def deconv2d_f32(self, x, w, bias, stride, pad):
+        n, c, h, wd = x.shape
+        _, k, kh, kw = w.shape
+        sh, sw = (stride, stride) if np.isscalar(stride) else stride
+        pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+        y = self.empty((n, k, (h - 1) * sh + kh - pt - pb, (wd - 1) * sw + kw - pl - pr), np.float32)
+        _check(lib().exhip_deconv2d_f32(self.h, x.ptr, w.ptr, _ptr(bias), y.ptr, n, c, h, wd, k, kh, kw, sh, sw, pt, pb, pl, pr))
+        return y
+
     def add_f16(self, a, b, relu=False):
         y = self.empty(a.shape, np.uint16)
         _check(lib().exhip_add_f16(self.h, a.ptr, b.ptr, y.ptr, ctypes.c_size_t(y.size), int(relu)))

@@ -313,5 +313,19 @@ protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
 };
 
+// src/Excalibur/operation_deconvolution.cpp:11-171: the convolution's keys; float32 weights [C][K][kh][kw]; group 1.
+template <typename Dtype>
+class operation_deconvolution : public operation_general_conv<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_deconvolution(const operation_param& param) : operation_general_conv<Dtype>(param) {}
+    int init_weights() override;
+    int init_weights(FILE* fp) override;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
 }  // namespace excalibur
 }  // namespace glasssix

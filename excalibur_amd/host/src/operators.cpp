@@ -1057,6 +1057,59 @@ void operation_yolov5focus<Dtype>::forward_gpu_f32(const tensor_list<float>& bot
     EXHIP_FATAL(exhip_focus_f32(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num(), b->channels(), b->height(), b->width()));
 }
 
+template <typename Dtype>
+int operation_deconvolution<Dtype>::init_weights(FILE* fp) {
+    int tag = 0;
+    if (std::fread(&tag, sizeof(int), 1, fp) != 1) LOG(FATAL) << "Deconvolution: model file too short";
+    if (tag != 0) NOT_IMPLEMENTED << " quantized Deconvolution";
+    int mem = 0;
+    this->weights_f32_.push_back(vec_tensor<float>(this->weight_data_size_, this->params_.device_));
+    if (std::fread(this->weights_f32_[0]->mutable_cpu_data(), sizeof(float), this->weight_data_size_, fp) !=
+        static_cast<size_t>(this->weight_data_size_))
+        LOG(FATAL) << "Deconvolution: model file too short";
+    mem += this->weight_data_size_ * static_cast<int>(sizeof(float));
+    if (this->bias_term_) {
+        this->weights_f32_.push_back(vec_tensor<float>(this->output_channel_, this->params_.device_));
+        if (std::fread(this->weights_f32_[1]->mutable_cpu_data(), sizeof(float), this->output_channel_, fp) !=
+            static_cast<size_t>(this->output_channel_))
+            LOG(FATAL) << "Deconvolution: model file too short";
+        mem += this->output_channel_ * static_cast<int>(sizeof(float));
+    }
+    return mem;
+}
+
+template <typename Dtype>
+int operation_deconvolution<Dtype>::init_weights() {
+    if (this->params_.int8_quantization_) NOT_IMPLEMENTED;
+    this->weights_f32_.push_back(vec_tensor<float>(this->weight_data_size_, this->params_.device_));
+    float* w = this->weights_f32_[0]->mutable_cpu_data();
+    for (int i = 0; i < this->weight_data_size_; ++i) w[i] = 0.01f * static_cast<float>((i % 7) - 3);  // dummy weights
+    int mem = this->weight_data_size_ * static_cast<int>(sizeof(float));
+    if (this->bias_term_) {
+        this->weights_f32_.push_back(vec_tensor<float>(this->output_channel_, this->params_.device_));
+        mem += this->output_channel_ * static_cast<int>(sizeof(float));
+    }
+    return mem;
+}
+
+template <typename Dtype>
+void operation_deconvolution<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const auto& b = bottoms[0];
+    if (b->order() != memory::NCHW || this->group_ != 1 || this->dilation_h_ != 1 || this->dilation_w_ != 1)
+        NOT_IMPLEMENTED << " Deconvolution with groups, dilation or NHWC input";
+    const int c = b->channels();
+    CHECK_EQ(c * this->output_channel_ * this->kernel_size_h_ * this->kernel_size_w_, this->weight_data_size_);
+    const int oh = (b->height() - 1) * this->stride_h_ + this->kernel_size_h_ - (this->pad_top_ + this->pad_bottom_);
+    const int ow = (b->width() - 1) * this->stride_w_ + this->kernel_size_w_ - (this->pad_left_ + this->pad_right_);
+    tops[0] = new_tensor<float>({b->num(), this->output_channel_, oh, ow}, this->params_.device_);
+    EXHIP_FATAL(exhip_deconv2d_f32(this->ctx(), b->gpu_data(), this->weights_f32_[0]->gpu_data(),
+                                   this->bias_term_ ? this->weights_f32_[1]->gpu_data() : nullptr, tops[0]->mutable_gpu_data(), b->num(), c,
+                                   b->height(), b->width(), this->output_channel_, this->kernel_size_h_, this->kernel_size_w_, this->stride_h_,
+                                   this->stride_w_, this->pad_top_, this->pad_bottom_, this->pad_left_, this->pad_right_));
+}
+
 INSTANCE_CLASS(operation_general_conv);
 INSTANCE_CLASS(operation_convolution);
 INSTANCE_CLASS(operation_convolutiondepthwise);
@@ -1077,6 +1130,7 @@ INSTANCE_CLASS(operation_input);
 INSTANCE_CLASS(operation_concat);
 INSTANCE_CLASS(operation_interp);
 INSTANCE_CLASS(operation_yolov5focus);
+INSTANCE_CLASS(operation_deconvolution);
 
 REGISTE(operation_convolution);
 REGISTE(operation_convolutiondepthwise);
@@ -1096,6 +1150,7 @@ REGISTE(operation_input);
 REGISTE(operation_concat);
 REGISTE(operation_interp);
 REGISTE(operation_yolov5focus);
+REGISTE(operation_deconvolution);
 
 }  // namespace excalibur
 }  // namespace glasssix

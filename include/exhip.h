@@ -204,6 +204,11 @@ int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y, int n, in
  * (the reference fills image 0 only). y: [n][4c][h/2][w/2]. */
 int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w);
 
+/* operation_deconvolution::forward_cpu_f32 (src/Excalibur/operation_deconvolution.cpp:80-171), group 1, dilation 1:
+ * x NCHW, w [c][k][kh][kw], y [n][k][(h-1)*sh + kh - pt - pb][(w-1)*sw + kw - pl - pr] = scatter of W^T x (+ bias). */
+int exhip_deconv2d_f32(exhip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, int n, int c, int h, int wd,
+                       int k, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr);
+
 /* operation_innerproduct::forward_cpu_f32 (src/Excalibur/operation_innerproduct.cpp:176-224):
  * y[m,n] = sum_k x[m,k]*w[n,k] + bias[n]; x [m][k_in], w [n_out][k_in] row-major f32. */
 int exhip_innerproduct_f32(exhip_ctx* ctx, const float* x, const float* w, const float* bias, float* y, int m,

@@ -524,3 +524,35 @@ void exo_focus_f32(const float* x, float* y, int n, int c, int h, int w) {
                     y[(((size_t)img * 4 * c + p) * oh + i) * ow + j] = x[(((size_t)img * c + ch) * h + 2 * i + dy) * w + 2 * j + dx];
         }
 }
+
+/* operation_deconvolution::forward_cpu_f32, src/Excalibur/operation_deconvolution.cpp:80-171 (group 1, dilation 1):
+ * col = W^T x per image (W stored [C][K][kh][kw]), col2im scatters col[k][r][s][i][j] to
+ * y[k][i*sh - pt + r][j*sw - pl + s], then the bias is added; OH = (H-1)*sh + kh - (pt+pb). The reference sums
+ * in float in its GEMM's order; this restatement sums each output in double and rounds once (compared at 1e-4). */
+void exo_deconv2d_f32(const float* x, const float* w, const float* bias, float* y, int n, int c, int h, int wd, int k, int kh,
+                      int kw, int sh, int sw, int pt, int pb, int pl, int pr) {
+    const int oh = (h - 1) * sh + kh - (pt + pb), ow = (wd - 1) * sw + kw - (pl + pr);
+    for (int img = 0; img < n; ++img)
+        for (int ko = 0; ko < k; ++ko)
+            for (int oy = 0; oy < oh; ++oy)
+                for (int ox = 0; ox < ow; ++ox) {
+                    double s = 0.0;
+                    for (int r = 0; r < kh; ++r) {
+                        const int ty = oy + pt - r;
+                        if (ty < 0 || ty % sh) continue;
+                        const int iy = ty / sh;
+                        if (iy >= h) continue;
+                        for (int q = 0; q < kw; ++q) {
+                            const int tx = ox + pl - q;
+                            if (tx < 0 || tx % sw) continue;
+                            const int ix = tx / sw;
+                            if (ix >= wd) continue;
+                            for (int ci = 0; ci < c; ++ci)
+                                s += (double)x[(((size_t)img * c + ci) * h + iy) * wd + ix] *
+                                     (double)w[(((size_t)ci * k + ko) * kh + r) * kw + q];
+                        }
+                    }
+                    if (bias) s += (double)bias[ko];
+                    y[(((size_t)img * k + ko) * oh + oy) * ow + ox] = (float)s;
+                }
+}

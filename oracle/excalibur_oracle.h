@@ -21,6 +21,7 @@
  *   exo_hardswish / leakyrelu / sigmoid /
  *   hardsigmoid / prelu / batchnorm / input /
  *   concat_channels / interp_nearest       reference fixtures (bit-exact), element counts with and without a vector tail
+ *   exo_deconv2d_f32                       float64 evaluation of the definition, reference fixtures at 1e-4
  *   exo_focus_f32                          reference fixture (bit-exact) for one image; further images by the same formula
  * No function here is "parity unpinned".
  */
@@ -90,6 +91,9 @@ void exo_input_f32(const float* x, float* y, int n, int c, int hw, const float* 
 void exo_concat_channels_f32(const float* const* xs, const int* channels, int n_inputs, int n, int hw, float* y);
 void exo_interp_nearest_f32(const float* x, float* y, int n, int c, int h, int w, int oh, int ow);
 void exo_focus_f32(const float* x, float* y, int n, int c, int h, int w);
+
+void exo_deconv2d_f32(const float* x, const float* w, const float* bias, float* y, int n, int c, int h, int wd, int k, int kh,
+                      int kw, int sh, int sw, int pt, int pb, int pl, int pr);
 
 #ifdef __cplusplus
 }

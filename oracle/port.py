@@ -297,3 +297,16 @@ def focus(x):
     y = np.empty((n, 4 * c, h // 2, w // 2), np.float32)
     lib().exo_focus_f32(_p(x), _p(y), n, c, h, w)
     return y
+
+
+def deconv2d_f32(x, w, bias, stride, pad):
+    """w: [C_in][K_out][kh][kw]; pad: one value or (top, bottom, left, right)."""
+    x, w = _f32(x), _f32(w)
+    n, c, h, wd = x.shape
+    _, k, kh, kw = w.shape
+    sh, sw = (stride, stride) if np.isscalar(stride) else stride
+    pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+    y = np.empty((n, k, (h - 1) * sh + kh - pt - pb, (wd - 1) * sw + kw - pl - pr), np.float32)
+    lib().exo_deconv2d_f32(_p(x), _p(w), _p(_f32(bias)) if bias is not None else None, _p(y), n, c, h, wd, k, kh, kw, sh, sw, pt,
+                           pb, pl, pr)
+    return y

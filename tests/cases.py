@@ -109,6 +109,13 @@ def concat_case(seed, n, channels, h, w):
     return dict(op="concat", xs=[r.uniform(-2, 2, (n, c, h, w)).astype(np.float32) for c in channels])
 
 
+def deconv_case(seed, n, c, h, w, k, kernel, stride, pad=0, bias=True):
+    r = _rng(seed)
+    return dict(op="deconv", k=k, kernel=kernel, stride=stride, pad=pad, x=r.uniform(-1, 1, (n, c, h, w)).astype(np.float32),
+                wt=r.normal(0, 0.1, (c, k, kernel, kernel)).astype(np.float32),
+                bias=r.normal(0, 0.1, (k,)).astype(np.float32) if bias else None)
+
+
 def geom_of(case):
     return port.geom((case["n"], case["c"], case["h"], case["w"]), case["k"], case["kh"], case["kw"],
                      case["stride"], case["pad"], case["groups"])
@@ -136,6 +143,10 @@ def reference_io(case):
     if op == "fc":
         line = f"InnerProduct layer 1 1 data out 0={case['n_out']} 1={int(case['bias'] is not None)} 2={case['wt'].size}"
         return mf.topology([line]), mf.fc_blob_f32(case["wt"], case["bias"]), [case["x"]], "out"
+    if op == "deconv":
+        line = mf.conv_line("Deconvolution", "layer", "data", "out", case["k"], case["kernel"], case["stride"], case["pad"],
+                            case["bias"] is not None, case["wt"].size, 1)
+        return mf.topology([line]), mf.conv_blob_f32(case["wt"], case["bias"]), [case["x"]], "out"
     if op == "hardswish":
         return mf.topology([f"HardSwish layer 1 1 data out 0={case['alpha']!r} 1={case['beta']!r}"]), b"", [case["x"]], "out"
     if op == "leakyrelu":
@@ -204,6 +215,8 @@ def oracle_eval(case):
         return port.relu(case["x"])
     if op == "fc":
         return port.innerproduct(case["x"], case["wt"], case["bias"])
+    if op == "deconv":
+        return port.deconv2d_f32(case["x"], case["wt"], case["bias"], case["stride"], case["pad"])
     if op == "hardswish":
         return port.hardswish(case["x"], case["alpha"], case["beta"])
     if op == "leakyrelu":

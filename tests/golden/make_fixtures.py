@@ -78,6 +78,10 @@ def fixture_cases():
         "interp_nearest_x2": c.unary_case(71, "interp", (2, 3, 5, 7), height_scale=2.0, width_scale=2.0),
         "interp_nearest_frac": c.unary_case(72, "interp", (1, 2, 6, 5), height_scale=1.5, width_scale=2.5),
         "focus": c.unary_case(73, "focus", (1, 3, 8, 10)),
+        # transposed convolution (the detection head's 2x2 stride-2 upsampling, and overlapping taps with padding)
+        "deconv_2x2s2": c.deconv_case(74, 2, 6, 5, 7, 4, 2, 2),
+        "deconv_4x4s2p1": c.deconv_case(75, 1, 5, 6, 6, 3, 4, 2, 1),
+        "deconv_3x3s1p1_nobias": c.deconv_case(76, 1, 4, 7, 5, 6, 3, 1, 1, bias=False),
     }
 
 

@@ -106,6 +106,9 @@ def gpu_eval(ctx, case):
     if op == "fc":
         return ctx.innerproduct_f32(ctx.array(case["x"]), ctx.array(case["wt"]),
                                     ctx.array(case["bias"]) if case["bias"] is not None else None).download()
+    if op == "deconv":
+        return ctx.deconv2d_f32(ctx.array(case["x"]), ctx.array(case["wt"]), ctx.array(case["bias"]) if case["bias"] is not None else None,
+                                case["stride"], case["pad"]).download()
     if op in ("hardswish", "hardsigmoid"):
         return ctx.unary_f32(op, ctx.array(case["x"]), case["alpha"], case["beta"]).download()
     if op == "leakyrelu":
