@@ -8,6 +8,8 @@
 #include "common.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 namespace {
@@ -222,6 +224,121 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nhwc_f16_kernel(const uint16
     *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 8) = o;
 }
 
+// Strip form of the same layer for stride 1 and 2 and the activations that need no transcendental: a thread owns
+// 4 channels (8 bytes) of a strip of PX output pixels and walks a band of output rows, keeping the three input
+// rows it needs as stored (two halves to a register), so every input value is fetched once per band and the 36
+// weights once per thread. The next step's rows are requested before the current outputs are computed. Loads and
+// stores go through buffer descriptors over the whole tensors: a tap outside the image, or an output pixel beyond
+// the row's end, gets an offset beyond the descriptor's range and reads as zero / is dropped. The kernel is bound
+// by vector ALU issue as much as by memory, hence the template on the activation and the masked, packed stores.
+// Arithmetic order per output is that of dw_pixel.
+template <int STRIDE, int PX, int ACT>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_nhwc_f16_strip_kernel(const uint16_t* __restrict__ x,
+                                                                          const float* __restrict__ w,
+                                                                          const float* __restrict__ bias,
+                                                                          uint16_t* __restrict__ y, int C, int H, int W,
+                                                                          int cs, int OH, int OW, int pt, int pl,
+                                                                          int band_rows, int bands, int strips,
+                                                                          unsigned x_bytes, unsigned y_bytes, size_t total) {
+    constexpr int NC = (PX - 1) * STRIDE + 3, KEEP = 3 - STRIDE;
+    // out-of-range markers: a tensor is at most 2^30 bytes, so a valid row offset plus the column marker, the row
+    // marker plus anything, and both markers together all land beyond the descriptor's range without wrapping
+    constexpr unsigned kRowOutside = 0x80000000u, kColOutside = 0x40000000u;
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 4;
+    const int g = (int)(i % groups);
+    size_t t = i / groups;
+    const int xs = (int)(t % strips);
+    t /= strips;
+    const int band = (int)(t % bands);
+    const int n = (int)(t / bands);
+    const int c0 = g * 4;
+    float k[4][9], b[4];
+    if (c0 + 4 <= C) {  // 36 consecutive floats, 16-byte aligned
+        v4f kv[9];
+#pragma unroll
+        for (int q = 0; q < 9; ++q) kv[q] = reinterpret_cast<const v4f*>(w + c0 * 9)[q];
+#pragma unroll
+        for (int q = 0; q < 36; ++q) k[q / 9][q % 9] = kv[q / 4][q % 4];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int c = min(c0 + e, C - 1);
+#pragma unroll
+            for (int q = 0; q < 9; ++q) k[e][q] = w[c * 9 + q];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b[e] = bias ? bias[min(c0 + e, C - 1)] : 0.f;
+    // channels of the padding are stored as zero halves
+    const int keep_lo = (c0 < C ? 0xffff : 0) | (c0 + 1 < C ? 0xffff0000 : 0);
+    const int keep_hi = (c0 + 2 < C ? 0xffff : 0) | (c0 + 3 < C ? 0xffff0000 : 0);
+    const int oy0 = band * band_rows, oy1 = min(OH, oy0 + band_rows);
+    const int ox0 = xs * PX, ix0 = ox0 * STRIDE - pl;
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(x), 0, (int)x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
+    const int row_b = W * cs * 2, orow_b = OW * cs * 2;
+    const int img_off = n * H * row_b + c0 * 2;
+    unsigned col_off[NC], ocol_off[PX];  // byte offsets within a row, or the marker
+#pragma unroll
+    for (int cidx = 0; cidx < NC; ++cidx) {
+        const int ix = ix0 + cidx;
+        col_off[cidx] = ix >= 0 && ix < W ? (unsigned)(ix * cs * 2) : kColOutside;
+    }
+#pragma unroll
+    for (int px = 0; px < PX; ++px) ocol_off[px] = ox0 + px < OW ? (unsigned)((ox0 + px) * cs * 2) : kColOutside;
+    v4h r[3][NC], nxt[STRIDE][NC];
+    auto fetch = [&](int iy, v4h (&dst)[NC]) {
+        const unsigned row_off = iy >= 0 && iy < H ? (unsigned)(img_off + iy * row_b) : kRowOutside;
+#pragma unroll
+        for (int cidx = 0; cidx < NC; ++cidx)
+            dst[cidx] = __builtin_bit_cast(v4h, __builtin_amdgcn_raw_buffer_load_b64(xr, (int)(row_off + col_off[cidx]), 0, 0));
+    };
+    // rows that the first step keeps from "the step before" go where the shift below expects them
+#pragma unroll
+    for (int a = 0; a < KEEP; ++a) fetch(oy0 * STRIDE - pt + a, r[STRIDE + a]);
+#pragma unroll
+    for (int a = 0; a < STRIDE; ++a) fetch(oy0 * STRIDE - pt + KEEP + a, nxt[a]);
+    unsigned orow_off = (unsigned)((n * OH + oy0) * orow_b + c0 * 2);
+    for (int oy = oy0; oy < oy1; ++oy, orow_off += orow_b) {
+#pragma unroll
+        for (int cidx = 0; cidx < NC; ++cidx) {
+#pragma unroll
+            for (int a = 0; a < KEEP; ++a) r[a][cidx] = r[a + STRIDE][cidx];
+#pragma unroll
+            for (int a = 0; a < STRIDE; ++a) r[KEEP + a][cidx] = nxt[a][cidx];
+        }
+        if (oy + 1 < oy1) {
+#pragma unroll
+            for (int a = 0; a < STRIDE; ++a) fetch((oy + 1) * STRIDE - pt + KEEP + a, nxt[a]);
+        }
+#pragma unroll
+        for (int px = 0; px < PX; ++px) {
+            v4f res;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float sum = b[e];
+#pragma unroll
+                for (int j = 0; j < 3; ++j) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int a = 0; a < 3; ++a) s = __builtin_fmaf((float)r[a][px * STRIDE + j][e], k[e][a * 3 + j], s);
+                    sum += s;
+                }
+                // activations 0 (none), 1 (ReLU), 3 (ReLU6 as the reference writes it)
+                if (ACT != 0) sum = (0.f > sum) ? 0.f : sum;
+                if (ACT == 3) sum = sum <= 6.f ? sum : 0.f;
+                res[e] = sum;
+            }
+            v2i o = __builtin_bit_cast(v2i, __builtin_convertvector(res, v4h));
+            o[0] &= keep_lo;
+            o[1] &= keep_hi;
+            __builtin_amdgcn_raw_buffer_store_b64(o, yr, (int)(orow_off + ocol_off[px]), 0, 0);
+        }
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void dw_dequant_kernel(const int8_t* __restrict__ w, const float* __restrict__ ws,
                                                             float* __restrict__ wf, int k, int per_group) {
     const int i = blockIdx.x * kBlock + threadIdx.x;
@@ -271,6 +388,87 @@ __global__ __launch_bounds__(kBlock) void pool2d_nchw_f32_kernel(const float* __
         out = s / (float)pool;
     }
     y[(size_t)nc * OH * OW + o] = out;
+}
+
+// Stride-2 pooling with a 2x2 or 3x3 window over planes whose rows are a multiple of four floats long: a thread
+// makes four neighbouring outputs of one row from two aligned 16-byte loads per input row (plus one halo float to
+// the left for left padding 1, or to the right for a 3-wide window without left padding), so a wave reads whole
+// rows contiguously. Window clipping, the divisor and the row-major summation order are those of the general kernel.
+template <int K, int TYPE>
+__global__ __launch_bounds__(kBlock) void pool_s2_nchw_f32_strip_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                                        int H, int W, int OH, int OW, int pt, int pb, int pl,
+                                                                        int pr, int include_pad, int strips, size_t total) {
+    const size_t gi = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (gi >= total) return;
+    const int t = (int)(gi % strips);
+    const size_t rest = gi / strips;
+    const int ph = (int)(rest % OH);
+    const size_t nc = rest / OH;
+    const float* in = x + nc * H * W;
+    const int c0 = 8 * t;  // first column of the aligned chunk; v[i] below holds column c0 - 1 + i
+    const float fill = TYPE == 0 ? -FLT_MAX : 0.f;
+    float v[K][10];
+    const int hs0 = ph * 2 - pt;
+#pragma unroll
+    for (int a = 0; a < K; ++a) {
+        const int iy = hs0 + a;
+        const bool row_ok = iy >= 0 && iy < H;
+        const float* row = in + (size_t)iy * W;
+        v4f lo = {fill, fill, fill, fill}, hi = lo;
+        if (row_ok && c0 < W) lo = *reinterpret_cast<const v4f*>(row + c0);
+        if (row_ok && c0 + 4 < W) hi = *reinterpret_cast<const v4f*>(row + c0 + 4);
+        v[a][0] = pl == 1 && row_ok && c0 >= 1 && c0 - 1 < W ? row[c0 - 1] : fill;
+        v[a][9] = K == 3 && pl == 0 && row_ok && c0 + 8 < W ? row[c0 + 8] : fill;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            v[a][1 + e] = lo[e];
+            v[a][5 + e] = hi[e];
+        }
+    }
+    v4f out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int first = 2 * j - pl + 1;  // index into v[] of the window's first column
+        float res;
+        if (TYPE == 0) {
+            res = -FLT_MAX;
+#pragma unroll
+            for (int a = 0; a < K; ++a)
+#pragma unroll
+                for (int b = 0; b < K; ++b) {
+                    const float tap = v[a][first + b];
+                    res = res < tap ? tap : res;
+                }
+        } else {
+            const int pw = 4 * t + j;
+            int hs = hs0, wsx = pw * 2 - pl;
+            int he = min(hs + K, H + pb), we = min(wsx + K, W + pr);
+            int pool = (he - hs) * (we - wsx);
+            hs = max(hs, 0);
+            wsx = max(wsx, 0);
+            he = min(he, H);
+            we = min(we, W);
+            if (!include_pad) pool = (he - hs) * (we - wsx);
+            res = 0.f;
+#pragma unroll
+            for (int a = 0; a < K; ++a)
+#pragma unroll
+                for (int b = 0; b < K; ++b) {
+                    const int iy = hs0 + a, ix = pw * 2 - pl + b;
+                    if (iy >= hs && iy < he && ix >= wsx && ix < we) res += v[a][first + b];
+                }
+            res = res / (float)pool;
+        }
+        out[j] = res;
+    }
+    float* dst = y + (nc * OH + ph) * OW + 4 * t;
+    if ((OW & 3) == 0) {
+        *reinterpret_cast<v4f*>(dst) = out;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (4 * t + j < OW) dst[j] = out[j];
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void maxpool_nhwc_f32_kernel(const float* __restrict__ x, float* __restrict__ y,
@@ -749,6 +947,38 @@ extern "C" int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const
     int oh, ow;
     int rc = dw_out(h, w, stride, pt, pb, pl, pr, &oh, &ow);
     if (rc) return rc;
+    const size_t x_bytes = (size_t)n * h * w * cs * 2, y_bytes = (size_t)n * oh * ow * cs * 2;
+    const size_t desc_limit = (size_t)1 << 30;
+    if ((stride == 1 || stride == 2) && (act == 0 || act == 1 || act == 3) && x_bytes <= desc_limit && y_bytes <= desc_limit) {
+        // bands of output rows: about fourteen rows each (the per-thread set-up is worth several rows of work),
+        // shorter where that would leave fewer than four waves for every compute unit
+        const int px = stride == 1 ? 4 : 3;
+        const int strips = (ow + px - 1) / px;
+        const size_t per_band = (size_t)n * strips * (cs / 4);
+        static const int env_rows = getenv("EXHIP_DW_BAND_ROWS") ? atoi(getenv("EXHIP_DW_BAND_ROWS")) : 0;
+        const size_t want = (size_t)256 * 4 * 64;
+        int bands = (int)std::min<size_t>((size_t)oh, std::max<size_t>((oh + 13) / 14, (want + per_band - 1) / per_band));
+        int band_rows = (oh + bands - 1) / bands;
+        if (env_rows > 0) band_rows = std::min(env_rows, oh);
+        bands = (oh + band_rows - 1) / band_rows;
+        const size_t total = per_band * bands;
+#define EXHIP_DW_STRIP(S, P, A)                                                                                          \
+    hipLaunchKernelGGL((dwconv3x3_nhwc_f16_strip_kernel<S, P, A>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, \
+                       x, w9, bias, y, c, h, w, cs, oh, ow, pt, pl, band_rows, bands, strips, (unsigned)x_bytes,        \
+                       (unsigned)y_bytes, total)
+        if (stride == 1) {
+            if (act == 0) EXHIP_DW_STRIP(1, 4, 0);
+            else if (act == 1) EXHIP_DW_STRIP(1, 4, 1);
+            else EXHIP_DW_STRIP(1, 4, 3);
+        } else {
+            if (act == 0) EXHIP_DW_STRIP(2, 3, 0);
+            else if (act == 1) EXHIP_DW_STRIP(2, 3, 1);
+            else EXHIP_DW_STRIP(2, 3, 3);
+        }
+#undef EXHIP_DW_STRIP
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t total = (size_t)n * oh * ow * (cs / 8);
     hipLaunchKernelGGL(dwconv3x3_nhwc_f16_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, w9, bias, y, c, h, w,
                        cs, oh, ow, stride, pt, pl, act, total);
@@ -782,6 +1012,22 @@ extern "C" int exhip_pool2d_nchw_f32(exhip_ctx* ctx, const float* x, float* y, i
     REQ_CTX("exhip_pool2d_nchw_f32");
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && oh > 0 && ow > 0 && kh > 0 && kw > 0, "exhip_pool2d_nchw_f32: bad argument");
     EXHIP_REQUIRE(type == 0 || type == 1, "exhip_pool2d_nchw_f32: unknown pooling type %d", type);
+    const bool strip_window = kh == kw && (kh == 2 || kh == 3) && sh == 2 && sw == 2 && pl >= 0 && pl <= 1 && pt >= 0 &&
+                              w % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    if (strip_window) {
+        const int strips = (ow + 3) / 4;
+        const size_t threads = (size_t)n * c * oh * strips;
+#define EXHIP_POOL_STRIP(K, T)                                                                                              \
+    hipLaunchKernelGGL((pool_s2_nchw_f32_strip_kernel<K, T>), dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, x, y, \
+                       h, w, oh, ow, pt, pb, pl, pr, include_pad, strips, threads)
+        if (kh == 2 && type == 0) EXHIP_POOL_STRIP(2, 0);
+        else if (kh == 2) EXHIP_POOL_STRIP(2, 1);
+        else if (type == 0) EXHIP_POOL_STRIP(3, 0);
+        else EXHIP_POOL_STRIP(3, 1);
+#undef EXHIP_POOL_STRIP
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t total = (size_t)n * c * oh * ow;
     hipLaunchKernelGGL(pool2d_nchw_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, oh, ow, type,
                        kh, kw, sh, sw, pt, pb, pl, pr, include_pad, total);

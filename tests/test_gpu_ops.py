@@ -203,15 +203,23 @@ def test_depthwise_bit_exact(ctx, stride, h, w):
     assert np.array_equal(gpueval.gpu_eval(ctx, ci), cases.oracle_eval(ci))
 
 
-def test_depthwise_nhwc_f16(ctx):
+@pytest.mark.parametrize("stride,c,h,w,act", [(2, 40, 28, 30, 1), (1, 40, 28, 30, 1), (1, 128, 56, 56, 0), (2, 64, 57, 55, 3),
+                                             (1, 8, 7, 9, 1), (2, 24, 6, 5, 1), (1, 40, 19, 23, 4)])
+def test_depthwise_nhwc_f16(ctx, stride, c, h, w, act):
+    """Half storage, float arithmetic in the reference's order: the halves must be the float results rounded to nearest.
+    Strides 1 and 2 with the plain activations take the strip kernel (ragged strips, bands and channel padding are
+    all in these shapes); activation 4 takes the one-pixel-per-thread kernel."""
     from excalibur_amd import hip
-    case = cases.conv_f32_case(290, 2, 40, 28, 30, 40, 3, 2, 1, groups=40, dw=True)
+    case = cases.conv_f32_case(290 + h, 2, c, h, w, c, 3, stride, 1, act=act, groups=c, dw=True)
     x16 = case["x"].astype(np.float16).view(np.uint16)
-    want = port.float2half(cases.oracle_eval(dict(case, x=port.half2float(x16))))
-    x = ctx.nchw_to_nhwc(ctx.array(x16), hip.pad_to(40, 16), "f16")
-    y = ctx.dwconv3x3_nhwc_f16(x, 40, ctx.array(case["wt"]), ctx.array(case["bias"]), 2, 1, case["act"])
-    got = ctx.nhwc_to_nchw(y, 40, "f16").download()
+    want32 = cases.oracle_eval(dict(case, x=port.half2float(x16)))
+    want = port.float2half(want32)
+    x = ctx.nchw_to_nhwc(ctx.array(x16), hip.pad_to(c, 16), "f16")
+    y = ctx.dwconv3x3_nhwc_f16(x, c, ctx.array(case["wt"]), ctx.array(case["bias"]), stride, 1, case["act"])
+    got = ctx.nhwc_to_nchw(y, c, "f16").download()
     assert cases.check_value(got.view(np.float16).astype(np.float32), want.view(np.float16).astype(np.float32), 2e-3) == 0
+    if act != 4:  # same float results, rounded to nearest even by the hardware conversion
+        assert np.array_equal(got, want32.astype(np.float16).view(np.uint16))
 
 
 POOLS = [
@@ -226,6 +234,24 @@ POOLS = [
 @pytest.mark.parametrize("kw", POOLS, ids=[str(i) for i in range(len(POOLS))])
 def test_pool_bit_exact(ctx, kw):
     case = cases.pool_case(300, 2, 6, 41, 38, **kw)
+    assert np.array_equal(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case))
+
+
+S2_POOLS = [
+    dict(ptype=0, kernel=3, stride=2, pad=1), dict(ptype=0, kernel=3, stride=2, pad=0), dict(ptype=0, kernel=3, stride=2, pad=0, pad_mode=0),
+    dict(ptype=0, kernel=2, stride=2, pad=0), dict(ptype=0, kernel=2, stride=2, pad=(0, 1, 0, 1)), dict(ptype=0, kernel=2, stride=2, pad=1),
+    dict(ptype=1, kernel=2, stride=2, pad=0), dict(ptype=1, kernel=2, stride=2, pad=(0, 1, 0, 1)),
+    dict(ptype=1, kernel=3, stride=2, pad=1, pad_mode=0), dict(ptype=1, kernel=3, stride=2, pad=1, count_include_pad=1),
+    dict(ptype=1, kernel=3, stride=2, pad=0, pad_mode=0), dict(ptype=1, kernel=3, stride=2, pad=(2, 1, 1, 0)),
+]
+
+
+@pytest.mark.parametrize("hw", [(41, 40), (40, 36), (17, 8), (6, 4), (9, 64)], ids=lambda v: "%dx%d" % v)
+@pytest.mark.parametrize("kw", S2_POOLS, ids=[str(i) for i in range(len(S2_POOLS))])
+def test_pool_stride2_rows_of_four_bit_exact(ctx, kw, hw):
+    """Rows a multiple of four floats long take the four-outputs-per-thread kernel: same results as the oracle for
+    both halo sides, ceil and floor output sizes, clipped windows and both average divisors."""
+    case = cases.pool_case(305 + hw[0], 2, 5, hw[0], hw[1], **kw)
     assert np.array_equal(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case))
 
 
