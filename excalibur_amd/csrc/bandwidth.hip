@@ -177,6 +177,103 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_kernel(const float*
     y[(size_t)nc * OH * OW + o] = exhip_act(dw_pixel(r, k, bias ? bias[c] : 0.f), act);
 }
 
+// Strip form of the NCHW float kernel for stride 1 and 2, rows a multiple of four floats long, left padding 0 or 1
+// and the activations that need no transcendental: a thread makes four neighbouring outputs of a row and walks a
+// band of output rows with the three input rows it needs in registers. A row arrives as one (stride 1) or two
+// (stride 2) aligned 16-byte loads plus the halo floats the padding asks for, through a buffer descriptor whose
+// range check turns taps outside the image into zeros. slot i of a row holds column c0 - 1 + i.
+template <int STRIDE, int ACT>
+__global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_strip_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                                          const float* __restrict__ bias, float* __restrict__ y,
+                                                                          int C, int H, int W, int OH, int OW, int pt, int pl,
+                                                                          int band_rows, int bands, int strips, unsigned x_bytes,
+                                                                          unsigned y_bytes, size_t total) {
+    constexpr int CH = STRIDE == 1 ? 1 : 2;  // aligned 16-byte chunks per row
+    constexpr int NI = 4 * CH + 3, KEEP = 3 - STRIDE;
+    constexpr unsigned kRowOutside = 0x80000000u, kColOutside = 0x40000000u;  // tensors are at most 2^30 bytes
+    const size_t gi = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (gi >= total) return;
+    const int t = (int)(gi % strips);
+    size_t rest = gi / strips;
+    const int band = (int)(rest % bands);
+    const int nc = (int)(rest / bands);
+    const int c = nc % C;
+    float k[9];
+#pragma unroll
+    for (int q = 0; q < 9; ++q) k[q] = w[c * 9 + q];
+    const float b = bias ? bias[c] : 0.f;
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x), 0, (int)x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
+    const int c0 = 4 * CH * t;
+    unsigned chunk_off[CH], halo_off[3];  // halo slots: 0, NI - 2, NI - 1
+#pragma unroll
+    for (int q = 0; q < CH; ++q) chunk_off[q] = c0 + 4 * q < W ? (unsigned)((c0 + 4 * q) * 4) : kColOutside;
+    {
+        const int cols[3] = {c0 - 1, c0 + 4 * CH, c0 + 4 * CH + 1};
+        const bool used[3] = {pl == 1, STRIDE == 1 || pl == 0, STRIDE == 1 && pl == 0};
+#pragma unroll
+        for (int q = 0; q < 3; ++q) halo_off[q] = used[q] && cols[q] >= 0 && cols[q] < W ? (unsigned)(cols[q] * 4) : kColOutside;
+    }
+    const int plane_off = nc * H * W * 4;
+    float r[3][NI], nxt[STRIDE][NI];
+    auto fetch = [&](int iy, float (&dst)[NI]) {
+        const unsigned row_off = iy >= 0 && iy < H ? (unsigned)(plane_off + iy * W * 4) : kRowOutside;
+#pragma unroll
+        for (int q = 0; q < CH; ++q) {
+            const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(xr, (int)(row_off + chunk_off[q]), 0, 0));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[1 + 4 * q + e] = v[e];
+        }
+        dst[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[0]), 0, 0));
+        dst[NI - 2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[1]), 0, 0));
+        dst[NI - 1] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[2]), 0, 0));
+    };
+    const int oy0 = band * band_rows, oy1 = min(OH, oy0 + band_rows);
+#pragma unroll
+    for (int a = 0; a < KEEP; ++a) fetch(oy0 * STRIDE - pt + a, r[STRIDE + a]);
+#pragma unroll
+    for (int a = 0; a < STRIDE; ++a) fetch(oy0 * STRIDE - pt + KEEP + a, nxt[a]);
+    unsigned out_off = (unsigned)(((nc * OH + oy0) * OW + 4 * t) * 4);
+    const bool whole = (OW & 3) == 0;
+    for (int oy = oy0; oy < oy1; ++oy, out_off += OW * 4) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+#pragma unroll
+            for (int a = 0; a < KEEP; ++a) r[a][i] = r[a + STRIDE][i];
+#pragma unroll
+            for (int a = 0; a < STRIDE; ++a) r[KEEP + a][i] = nxt[a][i];
+        }
+        if (oy + 1 < oy1) {
+#pragma unroll
+            for (int a = 0; a < STRIDE; ++a) fetch((oy + 1) * STRIDE - pt + KEEP + a, nxt[a]);
+        }
+        v4f out;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float sum = b;
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                float col = 0.f;
+#pragma unroll
+                for (int a = 0; a < 3; ++a) col = __builtin_fmaf(pl == 1 ? r[a][j * STRIDE + q] : r[a][j * STRIDE + q + 1], k[a * 3 + q], col);
+                sum += col;
+            }
+            if (ACT != 0) sum = (0.f > sum) ? 0.f : sum;
+            if (ACT == 3) sum = sum <= 6.f ? sum : 0.f;
+            out[j] = sum;
+        }
+        const v4i bits = __builtin_bit_cast(v4i, out);  // cast the whole vector: a cast of one element picks element 0
+        if (whole) {
+            __builtin_amdgcn_raw_buffer_store_b128(bits, yr, (int)out_off, 0, 0);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                __builtin_amdgcn_raw_buffer_store_b32(bits[j], yr,
+                                                      (int)(4 * t + j < OW ? out_off + 4 * j : kRowOutside), 0, 0);
+        }
+    }
+}
+
 // NHWC half storage, 8 channels (16 bytes) per thread, f32 math in the same order.
 __global__ __launch_bounds__(kBlock) void dwconv3x3_nhwc_f16_kernel(const uint16_t* __restrict__ x, const float* __restrict__ w,
                                                                     const float* __restrict__ bias, uint16_t* __restrict__ y,
@@ -932,6 +1029,37 @@ extern "C" int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const fl
     int oh, ow;
     int rc = dw_out(h, w, stride, pt, pb, pl, pr, &oh, &ow);
     if (rc) return rc;
+    const size_t x_bytes = (size_t)n * c * h * w * 4, y_bytes = (size_t)n * c * oh * ow * 4;
+    const size_t desc_limit = (size_t)1 << 30;
+    if ((stride == 1 || stride == 2) && (act == 0 || act == 1 || act == 3) && (pl == 0 || pl == 1) && w % 4 == 0 &&
+        (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 && x_bytes <= desc_limit &&
+        y_bytes <= desc_limit) {
+        const int strips = (ow + 3) / 4;
+        const size_t per_band = (size_t)n * c * strips;
+        const size_t want = (size_t)256 * 8 * 64;
+        int bands = (int)std::min<size_t>((size_t)oh, std::max<size_t>((oh + 15) / 16, (want + per_band - 1) / per_band));
+        static const int env_rows = getenv("EXHIP_DW_BAND_ROWS") ? atoi(getenv("EXHIP_DW_BAND_ROWS")) : 0;
+        int band_rows = (oh + bands - 1) / bands;
+        if (env_rows > 0) band_rows = std::min(env_rows, oh);
+        bands = (oh + band_rows - 1) / band_rows;
+        const size_t total = per_band * bands;
+#define EXHIP_DW_STRIP(S, A)                                                                                              \
+    hipLaunchKernelGGL((dwconv3x3_nchw_f32_strip_kernel<S, A>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, \
+                       w9, bias, y, c, h, w, oh, ow, pt, pl, band_rows, bands, strips, (unsigned)x_bytes, (unsigned)y_bytes, \
+                       total)
+        if (stride == 1) {
+            if (act == 0) EXHIP_DW_STRIP(1, 0);
+            else if (act == 1) EXHIP_DW_STRIP(1, 1);
+            else EXHIP_DW_STRIP(1, 3);
+        } else {
+            if (act == 0) EXHIP_DW_STRIP(2, 0);
+            else if (act == 1) EXHIP_DW_STRIP(2, 1);
+            else EXHIP_DW_STRIP(2, 3);
+        }
+#undef EXHIP_DW_STRIP
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t total = (size_t)n * c * oh * ow;
     hipLaunchKernelGGL(dwconv3x3_nchw_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, w9, bias, y, c, h, w,
                        oh, ow, stride, pt, pl, act, total);

@@ -203,6 +203,15 @@ def test_depthwise_bit_exact(ctx, stride, h, w):
     assert np.array_equal(gpueval.gpu_eval(ctx, ci), cases.oracle_eval(ci))
 
 
+@pytest.mark.parametrize("stride,h,w,pad,act", [(1, 23, 36, 1, 1), (2, 41, 36, 1, 0), (1, 12, 8, 0, 3), (2, 13, 44, 0, 1),
+                                               (1, 5, 4, 1, 1), (2, 6, 4, 1, 1), (1, 40, 40, 1, 4)])
+def test_depthwise_rows_of_four_bit_exact(ctx, stride, h, w, pad, act):
+    """Rows a multiple of four floats long take the four-outputs-per-thread kernel (activation 4 does not): halos on
+    both sides, ragged output rows, several bands."""
+    case = cases.conv_f32_case(275 + h, 3, 24, h, w, 24, 3, stride, pad, act=act, groups=24, dw=True)
+    assert np.array_equal(gpueval.gpu_eval(ctx, case), cases.oracle_eval(case))
+
+
 @pytest.mark.parametrize("stride,c,h,w,act", [(2, 40, 28, 30, 1), (1, 40, 28, 30, 1), (1, 128, 56, 56, 0), (2, 64, 57, 55, 3),
                                              (1, 8, 7, 9, 1), (2, 24, 6, 5, 1), (1, 40, 19, 23, 4)])
 def test_depthwise_nhwc_f16(ctx, stride, c, h, w, act):
