@@ -10,6 +10,8 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v8f __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 namespace {
@@ -123,13 +125,75 @@ __global__ __launch_bounds__(kBlock) void nhwc_to_nchw_kernel(const Tin* __restr
     else y[i] = v;
 }
 
-__global__ __launch_bounds__(kBlock) void f32_to_f16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, size_t n) {
-    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i < n) y[i] = exhip_f2h(x[i]);
+// Precision conversion, eight values per thread over the 16-byte aligned body and one per thread over the rest.
+// The same through LDS for tensors of some size: a workgroup moves 64 pixels x 64 channels; 16-byte reads along the
+// channels of a pixel, stores of 64 consecutive pixels of a channel plane.
+template <int MODE, typename Tin, typename Tout>
+__global__ __launch_bounds__(kBlock) void nhwc_to_nchw_tiled_kernel(const Tin* __restrict__ x, Tout* __restrict__ y, int C, int HW,
+                                                                    int c_stride) {
+    constexpr int VE = 16 / sizeof(Tin);  // elements per 16-byte read
+    constexpr int VPP = 64 / VE;          // reads per pixel of the tile
+    constexpr int PITCH = 65;             // words per channel row in LDS: odd, so pixel columns spread over the banks
+    __shared__ Tout tile[64 * PITCH];
+    const int n = blockIdx.y, p0 = blockIdx.x * 64, tid = threadIdx.x;
+    for (int c0 = 0; c0 < C; c0 += 64) {
+        for (int v = tid; v < 64 * VPP; v += kBlock) {
+            const int pp = v / VPP, part = v % VPP;
+            const int cb = c0 + part * VE;
+            if (p0 + pp < HW && cb < c_stride) {
+                const v4i raw = *reinterpret_cast<const v4i*>(x + ((size_t)n * HW + p0 + pp) * c_stride + cb);
+                if constexpr (sizeof(Tin) == 4) {
+                    const v4f f = __builtin_bit_cast(v4f, raw);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) tile[(part * VE + e) * PITCH + pp] = (Tout)f[e];
+                } else {
+                    const v8h hv = __builtin_bit_cast(v8h, raw);
+                    const v4i words = raw;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if constexpr (MODE == 1) tile[(part * VE + e) * PITCH + pp] = (float)hv[e];
+                        else tile[(part * VE + e) * PITCH + pp] = (Tout)(((uint32_t)words[e >> 1] >> ((e & 1) * 16)) & 0xffff);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const int px = tid & 63, csub = tid >> 6;
+#pragma unroll 4
+        for (int i = 0; i < 16; ++i) {
+            const int cl = i * 4 + csub, c = c0 + cl;
+            if (c < C && p0 + px < HW) y[((size_t)n * C + c) * HW + p0 + px] = tile[cl * PITCH + px];
+        }
+        __syncthreads();
+    }
 }
-__global__ __launch_bounds__(kBlock) void f16_to_f32_kernel(const uint16_t* __restrict__ x, float* __restrict__ y, size_t n) {
+
+__global__ __launch_bounds__(kBlock) void f32_to_f16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, size_t n8,
+                                                            size_t n) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i < n) y[i] = exhip_h2f(x[i]);
+    if (i < n8) {
+        const v4f a = reinterpret_cast<const v4f*>(x)[2 * i], b = reinterpret_cast<const v4f*>(x)[2 * i + 1];
+        const v2i lo = __builtin_bit_cast(v2i, __builtin_convertvector(a, v4h)), hi = __builtin_bit_cast(v2i, __builtin_convertvector(b, v4h));
+        const v4i o = {lo[0], lo[1], hi[0], hi[1]};
+        reinterpret_cast<v4i*>(y)[i] = o;
+    } else {
+        const size_t j = n8 * 8 + (i - n8);
+        if (j < n) y[j] = exhip_f2h(x[j]);
+    }
+}
+__global__ __launch_bounds__(kBlock) void f16_to_f32_kernel(const uint16_t* __restrict__ x, float* __restrict__ y, size_t n8,
+                                                            size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n8) {
+        const v8h v = __builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(x)[i]);
+        const v8f f = __builtin_convertvector(v, v8f);
+        const v4f a = {f[0], f[1], f[2], f[3]}, b = {f[4], f[5], f[6], f[7]};
+        reinterpret_cast<v4f*>(y)[2 * i] = a;
+        reinterpret_cast<v4f*>(y)[2 * i + 1] = b;
+    } else {
+        const size_t j = n8 * 8 + (i - n8);
+        if (j < n) y[j] = exhip_h2f(x[j]);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -673,6 +737,44 @@ __global__ __launch_bounds__(kBlock) void eltwise_f32_kernel(EltArgs a, int type
     y[i] = r;
 }
 
+// Four floats per thread over the unfused body (a multiple of eight floats), the fused tail one per thread
+template <int TYPE>
+__global__ __launch_bounds__(kBlock) void eltwise_f32_v4_kernel(EltArgs a, float* __restrict__ y, size_t count, size_t body) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t n4 = body / 4;
+    if (i < n4) {
+        v4f r;
+        if (TYPE == 1) {
+            r = (v4f){0.f, 0.f, 0.f, 0.f};
+            for (int k = 0; k < a.n; ++k) {
+                const v4f xv = reinterpret_cast<const v4f*>(a.in[k])[i];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[e] = xv[e] * a.coeff[k] + r[e] * 1.0f;
+            }
+        } else {
+            r = reinterpret_cast<const v4f*>(a.in[0])[i];
+            for (int k = 1; k < a.n; ++k) {
+                const v4f xv = reinterpret_cast<const v4f*>(a.in[k])[i];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[e] = TYPE == 2 ? (r[e] < xv[e] ? xv[e] : r[e]) : r[e] * xv[e];
+            }
+        }
+        reinterpret_cast<v4f*>(y)[i] = r;
+        return;
+    }
+    const size_t j = body + (i - n4);
+    if (j >= count) return;
+    float r;
+    if (TYPE == 1) {
+        r = 0.f;
+        for (int k = 0; k < a.n; ++k) r = __builtin_fmaf(a.coeff[k], a.in[k][j], r * 1.0f);
+    } else {
+        r = a.in[0][j];
+        for (int k = 1; k < a.n; ++k) r = TYPE == 2 ? (r < a.in[k][j] ? a.in[k][j] : r) : r * a.in[k][j];
+    }
+    y[j] = r;
+}
+
 // ---- activation / glue layers ----
 // One value of an elementwise activation. OP 0 HardSwish, 1 LeakyReLU, 2 sigmoid, 3 HardSigmoid; the multiply-adds
 // are fused where the CPU path's are (vector fmadd, and scalar expressions contracted by its compiler flags).
@@ -731,12 +833,43 @@ __global__ __launch_bounds__(kBlock) void channelwise_f32_kernel(const float* __
     }
 }
 
+// The same, four floats per thread, for planes a multiple of four floats long
+template <int OP>
+__global__ __launch_bounds__(kBlock) void channelwise_f32_v4_kernel(const float* __restrict__ x, float* __restrict__ y, int C,
+                                                                    int HW4, const float* __restrict__ p0,
+                                                                    const float* __restrict__ p1, int shared) {
+    const int plane = blockIdx.y;
+    const int c = plane % C;
+    const float a = p0[shared ? 0 : c];
+    const float b = p1 ? p1[c] : 0.f;
+    const v4f* src = reinterpret_cast<const v4f*>(x) + (size_t)plane * HW4;
+    v4f* dst = reinterpret_cast<v4f*>(y) + (size_t)plane * HW4;
+    for (int j = blockIdx.x * kBlock + threadIdx.x; j < HW4; j += gridDim.x * kBlock) {
+        const v4f v = src[j];
+        v4f r;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (OP == 0) r[e] = v[e] >= 0.f ? v[e] : a * v[e];
+            else if constexpr (OP == 1) r[e] = __builtin_fmaf(b, v[e], a);
+            else r[e] = (v[e] - a) * b;
+        }
+        dst[j] = r;
+    }
+}
+
 // Copies one input's channel block of every image into its place in the concatenated tensor.
 __global__ __launch_bounds__(kBlock) void concat_block_kernel(const float* __restrict__ x, float* __restrict__ y, size_t block,
                                                               size_t out_image, size_t out_offset) {
     const size_t img = blockIdx.y;
     for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < block; j += (size_t)gridDim.x * kBlock)
         y[img * out_image + out_offset + j] = x[img * block + j];
+}
+
+__global__ __launch_bounds__(kBlock) void concat_block_v4_kernel(const v4f* __restrict__ x, v4f* __restrict__ y, size_t block4,
+                                                                 size_t out_image4, size_t out_offset4) {
+    const size_t img = blockIdx.y;
+    for (size_t j = (size_t)blockIdx.x * kBlock + threadIdx.x; j < block4; j += (size_t)gridDim.x * kBlock)
+        y[img * out_image4 + out_offset4 + j] = x[img * block4 + j];
 }
 
 // Nearest-neighbour resize: in = min((int)(out * scale), size - 1), scale = size / (float)out_size.
@@ -768,6 +901,50 @@ __global__ __launch_bounds__(kBlock) void focus_kernel(const float* __restrict__
     const size_t n = t / (4 * C);
     const int g = p / C, c = p % C;
     y[i] = x[((n * C + c) * H + 2 * oy + g % 2) * W + 2 * ox + g / 2];
+}
+
+// Four neighbouring outputs of a row per thread (output rows a multiple of four long): one 16-byte store
+__global__ __launch_bounds__(kBlock) void interp_nearest_x4_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W,
+                                                                   int OH, int OW4, float hs, float ws, size_t total4) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total4) return;
+    const int q = (int)(i % OW4);
+    const size_t t = i / OW4;
+    const int oy = (int)(t % OH);
+    const size_t plane = t / OH;
+    int iy = (int)(oy * hs);
+    iy = iy > H - 1 ? H - 1 : iy;
+    const float* row = x + (plane * H + iy) * W;
+    v4f o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        int ix = (int)((4 * q + e) * ws);
+        ix = ix > W - 1 ? W - 1 : ix;
+        o[e] = row[ix];
+    }
+    reinterpret_cast<v4f*>(y)[i] = o;
+}
+
+// Eight neighbouring inputs of a row per thread (rows a multiple of eight long): the even columns go to one output
+// plane and the odd ones to another, 16 bytes each
+__global__ __launch_bounds__(kBlock) void focus_x8_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int H, int W,
+                                                          size_t total8) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total8) return;
+    const int W8 = W / 8, OH = H / 2, OW = W / 2;
+    const int q = (int)(i % W8);
+    size_t t = i / W8;
+    const int iy = (int)(t % (2 * OH));
+    t /= 2 * OH;
+    const int c = (int)(t % C);
+    const size_t n = t / C;
+    const v4f* src = reinterpret_cast<const v4f*>(x + ((n * C + c) * H + iy) * W + 8 * q);
+    const v4f a = src[0], b = src[1];
+    const v4f even = {a[0], a[2], b[0], b[2]}, odd = {a[1], a[3], b[1], b[3]};
+    const int g = iy & 1;  // g % 2 selects the row parity, g / 2 the column parity
+    float* dst = y + ((n * 4 * C + c) * OH + iy / 2) * OW + 4 * q;
+    *reinterpret_cast<v4f*>(dst + (size_t)g * C * OH * OW) = even;
+    *reinterpret_cast<v4f*>(dst + (size_t)(g + 2) * C * OH * OW) = odd;
 }
 
 // Transposed convolution by gathering (NCHW float32, group 1, dilation 1): output (k, oy, ox) sums, over the taps
@@ -831,14 +1008,26 @@ __global__ __launch_bounds__(kBlock) void add_f32_kernel(const float* __restrict
     }
 }
 
+// The same on half storage (float sum, rounded once), eight values per thread over the aligned body
 __global__ __launch_bounds__(kBlock) void add_f16_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
-                                                         uint16_t* __restrict__ y, size_t count, int relu) {
+                                                         uint16_t* __restrict__ y, size_t n8, size_t count, int relu) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= count) return;
-    float r = exhip_h2f(a[i]);
-    if (b) r += exhip_h2f(b[i]);
-    if (relu) r = (0.f > r) ? 0.f : r;
-    y[i] = exhip_f2h(r);
+    if (i < n8) {
+        v8f r = __builtin_convertvector(__builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(a)[i]), v8f);
+        if (b) r += __builtin_convertvector(__builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(b)[i]), v8f);
+        if (relu) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) r[e] = (0.f > r[e]) ? 0.f : r[e];
+        }
+        reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(r, v8h));
+    } else {
+        const size_t j = n8 * 8 + (i - n8);
+        if (j >= count) return;
+        float r = exhip_h2f(a[j]);
+        if (b) r += exhip_h2f(b[j]);
+        if (relu) r = (0.f > r) ? 0.f : r;
+        y[j] = exhip_f2h(r);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -975,9 +1164,17 @@ extern "C" int exhip_nchw_f16_to_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, int
     return launch_to_nhwc<3>(ctx, x, y, n, c, h, w, cs, 0.f, nullptr);
 }
 
+template <typename T> static size_t c_stride_bytes(int cs) { return (size_t)cs * sizeof(T); }
+
 template <int MODE, typename Tin, typename Tout>
 static int launch_to_nchw(exhip_ctx* ctx, const Tin* x, Tout* y, int n, int c, int h, int w, int cs) {
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 0 && w > 0 && cs >= c, "layout conversion: bad argument");
+    if ((size_t)c_stride_bytes<Tin>(cs) % 16 == 0 && (uintptr_t)x % 16 == 0 && (size_t)h * w >= 64 && n <= 65535) {
+        hipLaunchKernelGGL((nhwc_to_nchw_tiled_kernel<MODE, Tin, Tout>), dim3((h * w + 63) / 64, n), dim3(kBlock), 0, ctx->stream,
+                           x, y, c, h * w, cs);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t total = (size_t)n * c * h * w;
     hipLaunchKernelGGL((nhwc_to_nchw_kernel<MODE, Tin, Tout>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c,
                        h * w, cs, total);
@@ -1001,7 +1198,8 @@ extern "C" int exhip_f32_to_f16(exhip_ctx* ctx, const float* x, uint16_t* y, siz
     REQ_CTX("exhip_f32_to_f16");
     EXHIP_REQUIRE((x && y) || !count, "exhip_f32_to_f16: NULL tensor");
     if (!count) return 0;
-    hipLaunchKernelGGL(f32_to_f16_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, x, y, count);
+    const size_t n8 = ((uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) ? count / 8 : 0;
+    hipLaunchKernelGGL(f32_to_f16_kernel, dim3(blocks_for(n8 + (count - n8 * 8))), dim3(kBlock), 0, ctx->stream, x, y, n8, count);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -1009,7 +1207,8 @@ extern "C" int exhip_f16_to_f32(exhip_ctx* ctx, const uint16_t* x, float* y, siz
     REQ_CTX("exhip_f16_to_f32");
     EXHIP_REQUIRE((x && y) || !count, "exhip_f16_to_f32: NULL tensor");
     if (!count) return 0;
-    hipLaunchKernelGGL(f16_to_f32_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, x, y, count);
+    const size_t n8 = ((uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) ? count / 8 : 0;
+    hipLaunchKernelGGL(f16_to_f32_kernel, dim3(blocks_for(n8 + (count - n8 * 8))), dim3(kBlock), 0, ctx->stream, x, y, n8, count);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -1201,6 +1400,17 @@ extern "C" int exhip_eltwise_f32(exhip_ctx* ctx, const float* const* inputs, int
         a.in[i] = inputs[i];
         a.coeff[i] = coeffs ? coeffs[i] : 1.0f;
     }
+    bool aligned = (uintptr_t)y % 16 == 0;
+    for (int i = 0; i < n_inputs; ++i) aligned = aligned && (uintptr_t)inputs[i] % 16 == 0;
+    if (aligned) {
+        const size_t body = count - count % 8;
+        const dim3 grid(blocks_for(body / 4 + count % 8));
+        if (type == 0) hipLaunchKernelGGL((eltwise_f32_v4_kernel<0>), grid, dim3(kBlock), 0, ctx->stream, a, y, count, body);
+        else if (type == 1) hipLaunchKernelGGL((eltwise_f32_v4_kernel<1>), grid, dim3(kBlock), 0, ctx->stream, a, y, count, body);
+        else hipLaunchKernelGGL((eltwise_f32_v4_kernel<2>), grid, dim3(kBlock), 0, ctx->stream, a, y, count, body);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     hipLaunchKernelGGL(eltwise_f32_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, a, type, y, count,
                        count - count % 8);
     EXHIP_LAUNCH_CHECK();
@@ -1231,7 +1441,8 @@ extern "C" int exhip_add_f16(exhip_ctx* ctx, const uint16_t* a, const uint16_t* 
     REQ_CTX("exhip_add_f16");
     EXHIP_REQUIRE((a && b && y) || !count, "exhip_add_f16: NULL tensor");
     if (!count) return 0;
-    hipLaunchKernelGGL(add_f16_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, a, b, y, count, relu);
+    const size_t n8 = ((uintptr_t)a % 16 == 0 && (uintptr_t)b % 16 == 0 && (uintptr_t)y % 16 == 0) ? count / 8 : 0;
+    hipLaunchKernelGGL(add_f16_kernel, dim3(blocks_for(n8 + (count - n8 * 8))), dim3(kBlock), 0, ctx->stream, a, b, y, n8, count, relu);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -1239,7 +1450,8 @@ extern "C" int exhip_relu_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, si
     REQ_CTX("exhip_relu_f16");
     EXHIP_REQUIRE((x && y) || !count, "exhip_relu_f16: NULL tensor");
     if (!count) return 0;
-    hipLaunchKernelGGL(add_f16_kernel, dim3(blocks_for(count)), dim3(kBlock), 0, ctx->stream, x, (const uint16_t*)nullptr, y, count, 1);
+    const size_t n8 = ((uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) ? count / 8 : 0;
+    hipLaunchKernelGGL(add_f16_kernel, dim3(blocks_for(n8 + (count - n8 * 8))), dim3(kBlock), 0, ctx->stream, x, (const uint16_t*)nullptr, y, n8, count, 1);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -1299,6 +1511,19 @@ extern "C" int exhip_channelwise_f32(exhip_ctx* ctx, int op, const float* x, flo
     EXHIP_REQUIRE(x && y && p0 && n > 0 && c > 0 && hw > 0, "exhip_channelwise_f32: bad argument");
     EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || p1, "exhip_channelwise_f32: this op needs two parameter arrays");
     EXHIP_REQUIRE((long long)n * c <= 65535, "exhip_channelwise_f32: more than 65535 (image, channel) planes");
+    if (hw % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) {
+        unsigned bx4 = blocks_for((size_t)hw / 4);
+        if (bx4 > 64) bx4 = 64;
+        const dim3 grid4(bx4, (unsigned)(n * c));
+        switch (op) {
+        case EXHIP_CHANNEL_PRELU: hipLaunchKernelGGL((channelwise_f32_v4_kernel<0>), grid4, dim3(kBlock), 0, ctx->stream, x, y, c, hw / 4, p0, p1, shared); break;
+        case EXHIP_CHANNEL_BATCHNORM: hipLaunchKernelGGL((channelwise_f32_v4_kernel<1>), grid4, dim3(kBlock), 0, ctx->stream, x, y, c, hw / 4, p0, p1, 0); break;
+        case EXHIP_CHANNEL_INPUT: hipLaunchKernelGGL((channelwise_f32_v4_kernel<2>), grid4, dim3(kBlock), 0, ctx->stream, x, y, c, hw / 4, p0, p1, 0); break;
+        default: exhip_set_error("exhip_channelwise_f32: unknown op %d", op); return EXHIP_ERR_ARG;
+        }
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     unsigned bx = blocks_for((size_t)hw);
     if (bx > 64) bx = 64;
     const dim3 grid(bx, (unsigned)(n * c));
@@ -1324,6 +1549,15 @@ extern "C" int exhip_concat_channels_f32(exhip_ctx* ctx, const float* const* inp
     size_t off = 0;
     for (int i = 0; i < n_inputs; ++i) {
         const size_t block = (size_t)channels[i] * hw;
+        if (block % 4 == 0 && off % 4 == 0 && (total_c * hw) % 4 == 0 && (uintptr_t)inputs[i] % 16 == 0 && (uintptr_t)y % 16 == 0) {
+            unsigned bx4 = blocks_for(block / 4);
+            if (bx4 > 1024) bx4 = 1024;
+            hipLaunchKernelGGL(concat_block_v4_kernel, dim3(bx4, (unsigned)n), dim3(kBlock), 0, ctx->stream,
+                               reinterpret_cast<const v4f*>(inputs[i]), reinterpret_cast<v4f*>(y), block / 4, total_c * hw / 4, off / 4);
+            EXHIP_LAUNCH_CHECK();
+            off += block;
+            continue;
+        }
         unsigned bx = blocks_for(block);
         if (bx > 1024) bx = 1024;
         hipLaunchKernelGGL(concat_block_kernel, dim3(bx, (unsigned)n), dim3(kBlock), 0, ctx->stream, inputs[i], y, block, total_c * hw, off);
@@ -1336,6 +1570,13 @@ extern "C" int exhip_concat_channels_f32(exhip_ctx* ctx, const float* const* inp
 extern "C" int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w, int oh, int ow) {
     REQ_CTX("exhip_interp_nearest_f32");
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 0 && w > 0 && oh > 0 && ow > 0, "exhip_interp_nearest_f32: bad argument");
+    if (ow % 4 == 0 && (uintptr_t)y % 16 == 0) {
+        const size_t total4 = (size_t)n * c * oh * (ow / 4);
+        hipLaunchKernelGGL(interp_nearest_x4_kernel, dim3(blocks_for(total4)), dim3(kBlock), 0, ctx->stream, x, y, h, w, oh, ow / 4,
+                           h / (float)oh, w / (float)ow, total4);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t total = (size_t)n * c * oh * ow;
     hipLaunchKernelGGL(interp_nearest_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, oh, ow, h / (float)oh,
                        w / (float)ow, total);
@@ -1346,6 +1587,12 @@ extern "C" int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y
 extern "C" int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w) {
     REQ_CTX("exhip_focus_f32");
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 1 && w > 1, "exhip_focus_f32: bad argument");
+    if (w % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) {
+        const size_t total8 = (size_t)n * c * (h / 2 * 2) * (w / 8);
+        hipLaunchKernelGGL(focus_x8_kernel, dim3(blocks_for(total8)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total8);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t total = (size_t)n * 4 * c * (h / 2) * (w / 2);
     hipLaunchKernelGGL(focus_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total);
     EXHIP_LAUNCH_CHECK();
