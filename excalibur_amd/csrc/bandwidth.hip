@@ -33,7 +33,8 @@ template <> struct Conv<3> { typedef uint16_t in_t; typedef uint16_t out_t; };
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void nchw_to_nhwc_kernel(const typename Conv<MODE>::in_t* __restrict__ x,
                                                               typename Conv<MODE>::out_t* __restrict__ y, int C, int HW,
-                                                              int c_stride, float fs, const float* __restrict__ fs_pc) {
+                                                              int c_stride, float fs, const float* __restrict__ fs_pc,
+                                                              int quads) {
     typedef typename Conv<MODE>::out_t out_t;
     constexpr int ES = sizeof(out_t);
     constexpr int ROW = 64 * ES + 4;  // bytes per pixel row in LDS; ROW/4 is odd: conflict-free column writes
@@ -41,6 +42,38 @@ __global__ __launch_bounds__(kBlock) void nchw_to_nhwc_kernel(const typename Con
     const int n = blockIdx.y, p0 = blockIdx.x * 64, tid = threadIdx.x;
     const int px = tid & 63, csub = tid >> 6;
     for (int c0 = 0; c0 < c_stride; c0 += 64) {
+        if (quads) {
+            // four pixels of one channel per load: 16 pixel quads x 16 channels per pass
+            const int quad = tid & 15, crow = tid >> 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int cl = i * 16 + crow, c = c0 + cl, p = p0 + 4 * quad;
+                typename Conv<MODE>::in_t in[4] = {0, 0, 0, 0};
+                const bool live = c < C && p < HW;
+                if (live) {
+                    const auto* src = x + ((size_t)n * C + c) * HW + p;
+                    if constexpr (sizeof(in[0]) == 4) {
+                        const v4f v = *reinterpret_cast<const v4f*>(src);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) in[e] = v[e];
+                    } else {
+                        const v2i v = *reinterpret_cast<const v2i*>(src);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) in[e] = (uint16_t)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffff);
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    out_t v = 0;
+                    if (live) {
+                        if constexpr (MODE == 0) v = (out_t)exhip_q8(in[e] * (fs_pc ? fs_pc[c] : fs));
+                        else if constexpr (MODE == 2) v = exhip_f2h(in[e]);
+                        else v = in[e];
+                    }
+                    *reinterpret_cast<out_t*>(tile + (4 * quad + e) * ROW + cl * ES) = v;
+                }
+            }
+        } else
 #pragma unroll 4
         for (int i = 0; i < 16; ++i) {
             const int cl = i * 4 + csub, c = c0 + cl, p = p0 + px;
@@ -664,6 +697,42 @@ __global__ __launch_bounds__(kBlock) void maxpool_nhwc_f32_kernel(const float* _
     }
 }
 
+// Max pooling with a small fixed window on half storage: the maximum of halves is exact, so the taps are compared
+// as packed halves, all window loads in flight at once. Taps outside the image count as -inf (the clipped window of
+// the general kernel); an all-padding window cannot occur for the output sizes the layer computes.
+template <int K, int S>
+__global__ __launch_bounds__(kBlock) void maxpool_nhwc_f16_window_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                                         int H, int W, int cs, int OH, int OW, int pt, int pl,
+                                                                         size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 8;
+    const int g = (int)(i % groups);
+    size_t pix = i / groups;
+    const int ox = (int)(pix % OW);
+    pix /= OW;
+    const int oy = (int)(pix % OH);
+    const size_t n = pix / OH;
+    const _Float16 ninf = -__builtin_inff16();
+    const v8h lowest = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+    v8h tap[K][K];
+#pragma unroll
+    for (int a = 0; a < K; ++a)
+#pragma unroll
+        for (int b = 0; b < K; ++b) {
+            const int iy = oy * S - pt + a, ix = ox * S - pl + b;
+            tap[a][b] = lowest;
+            if (iy >= 0 && iy < H && ix >= 0 && ix < W)
+                tap[a][b] = __builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(x + ((n * H + iy) * W + ix) * cs + g * 8));
+        }
+    v8h best = lowest;
+#pragma unroll
+    for (int a = 0; a < K; ++a)
+#pragma unroll
+        for (int b = 0; b < K; ++b) best = __builtin_elementwise_max(best, tap[a][b]);
+    *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 8) = __builtin_bit_cast(v4i, best);
+}
+
 __global__ __launch_bounds__(kBlock) void pool2d_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int H,
                                                                  int W, int cs, int OH, int OW, int type, int kh, int kw,
                                                                  int sh, int sw, int pt, int pb, int pl, int pr,
@@ -1128,7 +1197,8 @@ static int launch_to_nhwc(exhip_ctx* ctx, const void* x, void* y, int n, int c, 
     EXHIP_REQUIRE(n > 0 && c > 0 && h > 0 && w > 0 && c_stride >= c, "layout conversion: bad shape");
     dim3 grid((h * w + 63) / 64, n);
     hipLaunchKernelGGL(nchw_to_nhwc_kernel<MODE>, grid, dim3(kBlock), 0, ctx->stream,
-                       (const typename Conv<MODE>::in_t*)x, (typename Conv<MODE>::out_t*)y, c, h * w, c_stride, fs, fs_pc);
+                       (const typename Conv<MODE>::in_t*)x, (typename Conv<MODE>::out_t*)y, c, h * w, c_stride, fs, fs_pc,
+                       (h * w) % 4 == 0 && (uintptr_t)x % 16 == 0 ? 1 : 0);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -1380,6 +1450,17 @@ extern "C" int exhip_pool2d_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && cs >= c && cs % 8 == 0, "exhip_pool2d_nhwc_f16: bad argument");
     EXHIP_REQUIRE(type == 0 || type == 1, "exhip_pool2d_nhwc_f16: unknown pooling type %d", type);
     const size_t total = (size_t)n * oh * ow * (cs / 8);
+    if (type == 0 && kh == kw && sh == sw && sh == 2 && (kh == 2 || kh == 3) && pt >= 0 && pl >= 0 && pt < kh && pl < kw &&
+        (oh - 1) * 2 - pt < h && (ow - 1) * 2 - pl < w) {
+        if (kh == 3)
+            hipLaunchKernelGGL((maxpool_nhwc_f16_window_kernel<3, 2>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h,
+                               w, cs, oh, ow, pt, pl, total);
+        else
+            hipLaunchKernelGGL((maxpool_nhwc_f16_window_kernel<2, 2>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h,
+                               w, cs, oh, ow, pt, pl, total);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     hipLaunchKernelGGL(pool2d_nhwc_f16_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, cs, oh, ow,
                        type, kh, kw, sh, sw, pt, pb, pl, pr, include_pad, total);
     EXHIP_LAUNCH_CHECK();
