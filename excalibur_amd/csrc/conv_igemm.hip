@@ -1143,7 +1143,11 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
         // small preferences: 64-byte chunks halve the number of stages; two independent 256-thread groups per
         // CU overlap each other's barriers and load waits, which one 512-thread group cannot; the 128-pixel
         // variant has the least reuse per staged byte
-        const double prefs = -(chunk_opt == 32 ? 0.004 : 0.0) - (variant == 1 ? 0.002 : 0.0) - (variant == 2 ? 0.02 : 0.0);
+        // A strided window stages four input pixels per output pixel: there the 512-thread variant with 32-byte
+        // chunks does best (twice the outputs per staged tile, and the tile still leaves room for the weights).
+        const bool strided_window = !packed && dt == EXHIP_I8 && p.S == 2 && d->kh > 1;  // measured on int8 layers
+        const double prefs = -(chunk_opt == 32 ? 0.004 : 0.0) - (variant == 1 ? 0.002 : 0.0) - (variant == 2 ? 0.02 : 0.0) +
+                             (strided_window && variant == 1 && chunk_opt == 32 ? 0.3 : 0.0);
         auto consider = [&](double score) {
             if (!found || score > best_score) {
                 best_score = score;
