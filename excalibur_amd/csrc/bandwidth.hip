@@ -845,7 +845,7 @@ __global__ __launch_bounds__(kBlock) void eltwise_f32_v4_kernel(EltArgs a, float
 }
 
 // ---- activation / glue layers ----
-// One value of an elementwise activation. OP 0 HardSwish, 1 LeakyReLU, 2 sigmoid, 3 HardSigmoid; the multiply-adds
+// One value of an elementwise activation. OP 0 HardSwish, 1 LeakyReLU, 2 sigmoid, 3 HardSigmoid, 4 Clip; the multiply-adds
 // are fused where the CPU path's are (vector fmadd, and scalar expressions contracted by its compiler flags).
 template <int OP>
 __device__ __forceinline__ float unary_value(float x, float alpha, float beta) {
@@ -858,10 +858,13 @@ __device__ __forceinline__ float unary_value(float x, float alpha, float beta) {
         return x < 0.f ? alpha * x : x;
     } else if constexpr (OP == 2) {
         return (float)(1. / (1. + exp(-(double)x)));
-    } else {
+    } else if constexpr (OP == 3) {
         float t = __builtin_fmaf(alpha, x, beta);
         t = 1.f < t ? 1.f : t;
         return 0.f < t ? t : 0.f;
+    } else {
+        const float t = beta < x ? beta : x;  // clip to [alpha, beta]
+        return alpha < t ? t : alpha;
     }
 }
 
@@ -1014,6 +1017,48 @@ __global__ __launch_bounds__(kBlock) void focus_x8_kernel(const float* __restric
     float* dst = y + ((n * 4 * C + c) * OH + iy / 2) * OW + 4 * q;
     *reinterpret_cast<v4f*>(dst + (size_t)g * C * OH * OW) = even;
     *reinterpret_cast<v4f*>(dst + (size_t)(g + 2) * C * OH * OW) = odd;
+}
+
+// Softmax over the channels of every (image, position) of an NCHW tensor: a thread owns one position and walks the
+// channels three times (maximum, exponentials and their sum, quotient); neighbouring threads read neighbouring
+// positions, so every access is coalesced.
+__global__ __launch_bounds__(kBlock) void softmax_channels_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW,
+                                                                  size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const size_t img = i / HW;
+    const int k = (int)(i - img * HW);
+    const float* in = x + img * C * HW + k;
+    float* out = y + img * C * HW + k;
+    float m = in[0];
+    for (int j = 1; j < C; ++j) {
+        const float v = in[(size_t)j * HW];
+        m = m < v ? v : m;
+    }
+    float sum = 0.f;
+    for (int j = 0; j < C; ++j) {
+        const float e = expf(in[(size_t)j * HW] - m);
+        out[(size_t)j * HW] = e;
+        sum += e;
+    }
+    for (int j = 0; j < C; ++j) out[(size_t)j * HW] = out[(size_t)j * HW] / sum;
+}
+
+// Rows and columns of every plane change places, through a 32 x 32 LDS tile so that both sides are coalesced.
+__global__ __launch_bounds__(kBlock) void transpose_hw_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W) {
+    __shared__ float tile[32][33];
+    const size_t plane = blockIdx.z;
+    const int x0 = blockIdx.x * 32, y0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    const float* in = x + plane * H * W;
+    float* out = y + plane * H * W;
+#pragma unroll
+    for (int r = ty; r < 32; r += 8)
+        if (y0 + r < H && x0 + tx < W) tile[r][tx] = in[(size_t)(y0 + r) * W + x0 + tx];
+    __syncthreads();
+#pragma unroll
+    for (int r = ty; r < 32; r += 8)
+        if (x0 + r < W && y0 + tx < H) out[(size_t)(x0 + r) * H + y0 + tx] = tile[tx][r];
 }
 
 // Transposed convolution by gathering (NCHW float32, group 1, dilation 1): output (k, oy, ox) sums, over the taps
@@ -1582,6 +1627,7 @@ extern "C" int exhip_unary_f32(exhip_ctx* ctx, int op, const float* x, float* y,
     case EXHIP_UNARY_LEAKYRELU: return launch_unary<1>(ctx, x, y, count, alpha, beta);
     case EXHIP_UNARY_SIGMOID: return launch_unary<2>(ctx, x, y, count, alpha, beta);
     case EXHIP_UNARY_HARDSIGMOID: return launch_unary<3>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_CLIP: return launch_unary<4>(ctx, x, y, count, alpha, beta);
     default: exhip_set_error("exhip_unary_f32: unknown op %d", op); return EXHIP_ERR_ARG;
     }
 }
@@ -1676,6 +1722,24 @@ extern "C" int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, 
     }
     const size_t total = (size_t)n * 4 * c * (h / 2) * (w / 2);
     hipLaunchKernelGGL(focus_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_softmax_channels_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int hw) {
+    REQ_CTX("exhip_softmax_channels_f32");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && hw > 0, "exhip_softmax_channels_f32: bad argument");
+    const size_t total = (size_t)n * hw;
+    hipLaunchKernelGGL(softmax_channels_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, hw, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_transpose_hw_f32(exhip_ctx* ctx, const float* x, float* y, int planes, int h, int w) {
+    REQ_CTX("exhip_transpose_hw_f32");
+    EXHIP_REQUIRE(x && y && planes > 0 && h > 0 && w > 0, "exhip_transpose_hw_f32: bad argument");
+    EXHIP_REQUIRE(planes <= 65535 && (h + 31) / 32 <= 65535, "exhip_transpose_hw_f32: more than 65535 planes or row tiles");
+    hipLaunchKernelGGL(transpose_hw_kernel, dim3((w + 31) / 32, (h + 31) / 32, planes), dim3(kBlock), 0, ctx->stream, x, y, h, w);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

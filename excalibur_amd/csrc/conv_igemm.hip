@@ -85,6 +85,8 @@ struct ConvParams {
     int vp_shift;             // log2 of the 16-byte vectors per staged pixel
     int SL;                   // non-packed: 16-byte LDS slots per staged pixel (chunk / 16 + 1 padding slot)
     unsigned magic_sl;        // ceil(2^32 / SL)
+    int adv_part, adv_pix;    // THREADS % SL, THREADS / SL: how (part, pixel) of a thread's slot advance per load
+    int adv_iy, adv_ix;       // adv_pix / IW, adv_pix % IW: how the pixel's (row, column) advance
     int act_need_b;           // non-packed: bytes of one activation tile image in LDS (whole 16-byte slots)
     int epi_f;                // fused epilogue: the per-wave LDS tiles include the float32 one
     int epi_mode;             // which epilogue the launched kernel has (0 general, 1 fused, 2 pooled)
@@ -241,17 +243,30 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
     int a_goff[PACKED ? NPP : NAV];
     int a_loff[PACKED ? NPP : 1];
     if constexpr (!PACKED) {
-        const int npix = p.IH * p.IW;
+        // Slot tid + THREADS * i of the tile: its (pixel, part) and the pixel's (row, column) advance from one i to
+        // the next by constants, so only the first needs divisions; all tests are evaluated without branches (a
+        // branch per test costs more than the arithmetic it skips, and so do the re-fetches of the parameters a
+        // branchy form makes).
+        const int H = p.H, W = p.W, IW = p.IW, SL = p.SL, step = p.tile_step, cs_b = p.cstride_b, oob = (int)p.img_bytes;
+        const int d_part = p.adv_part, d_pix = p.adv_pix, d_iy = p.adv_iy, d_ix = p.adv_ix;
+        const int npix = p.IH * IW;
+        int pix = fast_div(tid, p.magic_sl), part = tid - pix * SL;
+        int iy = fast_div(pix, p.magic_iw), ix = pix - iy * IW;
 #pragma unroll
         for (int i = 0; i < NAV; ++i) {
-            a_goff[i] = (int)p.img_bytes;
-            if (i * (THREADS * 16) + wave * 1024 >= p.act_need_b) continue;  // wave-uniform: this wave issues no i-th load
-            const int v = tid + THREADS * i;
-            const int pix = fast_div(v, p.magic_sl), part = v - pix * p.SL;
-            const int iy = fast_div(pix, p.magic_iw), ix = pix - iy * p.IW;
-            const int gy = iy0 + iy * p.tile_step, gx = ix0 + ix * p.tile_step;
-            const bool in_img = pix < npix && part < p.SL - 1 && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
-            a_goff[i] = in_img ? (gy * p.W + gx) * p.cstride_b + part * 16 : (int)p.img_bytes;
+            const int gy = iy0 + iy * step, gx = ix0 + ix * step;
+            const bool in_img = (pix < npix) & (part < SL - 1) & ((unsigned)gy < (unsigned)H) & ((unsigned)gx < (unsigned)W);
+            const int off = (gy * W + gx) * cs_b + part * 16;
+            a_goff[i] = in_img ? off : oob;
+            part += d_part;
+            const int carry = part >= SL ? 1 : 0;
+            part -= carry ? SL : 0;
+            pix += d_pix + carry;
+            ix += d_ix + carry;
+            iy += d_iy;
+            const int wrap = ix >= IW ? 1 : 0;
+            ix -= wrap ? IW : 0;
+            iy += wrap;
         }
     } else {
         const int npix = p.IH * p.IW;
@@ -1272,6 +1287,8 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.vp_shift = pl.chunk_b == 64 ? 2 : 1;
     p.SL = pl.SL; p.act_need_b = pl.act_need_b;
     p.magic_sl = (unsigned)(((1ull << 32) + pl.SL - 1) / pl.SL);
+    p.adv_part = pl.threads % pl.SL; p.adv_pix = pl.threads / pl.SL;
+    p.adv_iy = p.adv_pix / pl.IW; p.adv_ix = p.adv_pix % pl.IW;
     p.tile_dy = pl.PH; p.tile_dx = pl.PW;
     if (pool) {
         p.MPH = pl.MPH; p.MPW = pl.MPW; p.POH = pool->oh; p.POW = pool->ow;

@@ -309,7 +309,7 @@ class Ctx:
         return y
 
     # ---- activation / glue layers ----
-    UNARY = {"hardswish": 0, "leakyrelu": 1, "sigmoid": 2, "hardsigmoid": 3}
+    UNARY = {"hardswish": 0, "leakyrelu": 1, "sigmoid": 2, "hardsigmoid": 3, "clip": 4}
     CHANNEL = {"prelu": 0, "batchnorm": 1, "input": 2}
 
     def unary_f32(self, op, x, alpha=0.0, beta=0.0):
@@ -342,6 +342,18 @@ class Ctx:
         n, c, h, w = x.shape
         y = self.empty((n, 4 * c, h // 2, w // 2), np.float32)
         _check(lib().exhip_focus_f32(self.h, x.ptr, y.ptr, n, c, h, w))
+        return y
+
+    def softmax_channels_f32(self, x):
+        n, c = x.shape[:2]
+        y = self.empty(x.shape, np.float32)
+        _check(lib().exhip_softmax_channels_f32(self.h, x.ptr, y.ptr, n, c, int(np.prod(x.shape[2:], dtype=np.int64))))
+        return y
+
+    def transpose_hw_f32(self, x):
+        n, c, h, w = x.shape
+        y = self.empty((n, c, w, h), np.float32)
+        _check(lib().exhip_transpose_hw_f32(self.h, x.ptr, y.ptr, n * c, h, w))
         return y
 
     def deconv2d_f32(self, x, w, bias, stride, pad):

@@ -3,6 +3,7 @@
 // operation_convolutiondepthwise, operation_pooling, operation_eltwise, operation_binaryop, operation_relu,
 // operation_innerproduct, operation_split. Each overrides the forward_gpu_* virtuals and calls the exhip C ABI.
 #pragma once
+#include <cfloat>
 #include <map>
 
 #include "operation.hpp"
@@ -217,6 +218,12 @@ struct operation_hardsigmoid : operation_unary<Dtype> {
     explicit operation_hardsigmoid(const operation_param& p) : operation_unary<Dtype>(p, EXHIP_UNARY_HARDSIGMOID, 0.2f, 0.5f, 2) {}
 };
 
+// src/Excalibur/operation_clip.cpp:11-58: keys 0 = lower bound, 1 = upper bound.
+template <typename Dtype>
+struct operation_clip : operation_unary<Dtype> {
+    explicit operation_clip(const operation_param& p) : operation_unary<Dtype>(p, EXHIP_UNARY_CLIP, -FLT_MAX, FLT_MAX, 2) {}
+};
+
 // src/Excalibur/operation_prelu.cpp:9-124: key 0 = number of slopes (1 = shared), blob = the slopes.
 template <typename Dtype>
 class operation_prelu : public operation<Dtype> {
@@ -308,6 +315,65 @@ public:
     using tensor_list = typename operation<Dtype>::template tensor_list<T>;
     explicit operation_yolov5focus(const operation_param& param) : operation<Dtype>(param) {}
     const char* type() const override { return this->params_.type_.c_str(); }
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_reshape.cpp:8-131: keys 0 / 1 / 2 = new width / height / channels (-233 when absent: that
+// dimension is then derived from the element count, in the order channels, height, width), 3 = permute (unused). The
+// bottom tensor's shape is changed in place and the top is the same tensor.
+template <typename Dtype>
+class operation_reshape : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_reshape(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int n_ = 0, c_ = -233, h_ = -233, w_ = -233, permute_ = 0;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_flatten.cpp:11-113: key 0 = axis (default 1); a copy with shape [n][1][h'][w'].
+template <typename Dtype>
+class operation_flatten : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_flatten(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int axis_ = 1;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_softmax.cpp:10-96: key 0 = axis (read, not used: the sum always runs over the channels).
+template <typename Dtype>
+class operation_softmax : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_softmax(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    int axis_ = 0;
+
+protected:
+    void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+};
+
+// src/Excalibur/operation_transpose.cpp:9-70: key 0 = order of (h, w, c) as "a,b,c". (0,1,2) passes the tensor on,
+// (1,0,2) swaps rows and columns of every plane; the reference's other orders index past their planes and are refused.
+template <typename Dtype>
+class operation_transpose : public operation<Dtype> {
+public:
+    template <typename T>
+    using tensor_list = typename operation<Dtype>::template tensor_list<T>;
+    explicit operation_transpose(const operation_param& param);
+    const char* type() const override { return this->params_.type_.c_str(); }
+    std::vector<int> perms_{0, 1, 2};
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;

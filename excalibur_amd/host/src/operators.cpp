@@ -1058,6 +1058,130 @@ void operation_yolov5focus<Dtype>::forward_gpu_f32(const tensor_list<float>& bot
 }
 
 template <typename Dtype>
+operation_reshape<Dtype>::operation_reshape(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) w_ = a.as_int();
+        else if (key == 1) h_ = a.as_int();
+        else if (key == 2) c_ = a.as_int();
+        else if (key == 3) permute_ = a.as_int();
+        else if (key != -23330) LOG(FATAL) << "Un-supported Reshape Attribution " << a.key;
+    }
+    this->params_.inplace_ = true;
+}
+
+template <typename Dtype>
+void operation_reshape<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    if (bottoms[0]->order() != memory::NCHW) NOT_IMPLEMENTED;
+    std::vector<int> shape = bottoms[0]->data_shape();
+    const int count = static_cast<int>(bottoms[0]->count());
+    if (n_ > 0) shape[0] = n_;
+    if (c_ > 0) shape[1] = c_;
+    if (h_ > 0) shape[2] = h_;
+    if (w_ > 0) shape[3] = w_;
+    // absent or negative dimensions follow from the element count, each from the values the earlier steps left
+    auto derive = [&](int axis) {
+        int others = 1;
+        for (int i = 0; i < 4; ++i)
+            if (i != axis) others *= shape[i];
+        CHECK_EQ(count % others, 0);
+        shape[axis] = count / others;
+    };
+    if (n_ < 0) derive(0);
+    if (c_ < 0) derive(1);
+    if (h_ < 0) derive(2);
+    if (w_ < 0) derive(3);
+    CHECK_EQ(shape[0] * shape[1] * shape[2] * shape[3], count);
+    bottoms[0]->reshape(shape);
+    tops[0] = bottoms[0];
+}
+
+template <typename Dtype>
+operation_flatten<Dtype>::operation_flatten(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) axis_ = a.as_int();
+        else if (key != -23330) LOG(FATAL) << "Un-supported flatten Attribution " << a.key;
+    }
+}
+
+template <typename Dtype>
+void operation_flatten<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const auto& b = bottoms[0];
+    const int bw = b->width(), bh = b->height(), bc = b->channels();
+    int w = 0, h = 0;
+    if (axis_ == 0) { w = 1; h = bw * bh * bc; }
+    else if (axis_ == 1) { w = bw; h = bh * bc; }
+    else if (axis_ == 2) { w = bw * bh; h = bc; }
+    else { w = bw * bh * bc; h = 1; }  // the reference's last test is an assignment: every other axis lands here
+    tops[0] = new_tensor<float>({b->num(), 1, h, w}, this->params_.device_);
+    EXHIP_FATAL(exhip_memcpy_d2d(this->ctx(), tops[0]->mutable_gpu_data(), b->gpu_data(), b->count() * sizeof(float)));
+}
+
+template <typename Dtype>
+operation_softmax<Dtype>::operation_softmax(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) axis_ = a.as_int();
+        else if (key != 1 && key != -23330) LOG(FATAL) << "Un-supported Softmax Attribution " << a.key;
+    }
+}
+
+template <typename Dtype>
+void operation_softmax<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        const auto& b = bottoms[i];
+        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+        tops[i] = std::make_shared<tensor<float>>(b->data_shape(), this->params_.device_, b->order());
+        EXHIP_FATAL(exhip_softmax_channels_f32(this->ctx(), b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(), b->channels(),
+                                               b->height() * b->width()));
+    }
+}
+
+template <typename Dtype>
+operation_transpose<Dtype>::operation_transpose(const operation_param& param) : operation<Dtype>(param) {
+    for (const layer_attr& a : parse_attrs(param.specific_params_)) {
+        const int key = std::atoi(a.key.c_str());
+        if (key == 0) {
+            perms_.clear();
+            size_t pos = 0;
+            while (pos <= a.value.size()) {
+                const size_t comma = a.value.find(',', pos);
+                const std::string item = a.value.substr(pos, comma == std::string::npos ? std::string::npos : comma - pos);
+                if (!item.empty()) perms_.push_back(std::atoi(item.c_str()));
+                if (comma == std::string::npos) break;
+                pos = comma + 1;
+            }
+            CHECK_EQ(perms_.size(), 3);
+        } else if (key != -23330) {
+            LOG(FATAL) << "Un-supported Transpose Attribution " << a.key;
+        }
+    }
+}
+
+template <typename Dtype>
+void operation_transpose<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const auto& b = bottoms[0];
+    if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+    if (perms_[0] == 0 && perms_[1] == 1 && perms_[2] == 2) {
+        tops[0] = bottoms[0];
+    } else if (perms_[0] == 1 && perms_[1] == 0 && perms_[2] == 2) {
+        tops[0] = new_tensor<float>({b->num(), b->channels(), b->width(), b->height()}, this->params_.device_);
+        EXHIP_FATAL(exhip_transpose_hw_f32(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num() * b->channels(),
+                                           b->height(), b->width()));
+    } else {
+        NOT_IMPLEMENTED << " Transpose order " << perms_[0] << "," << perms_[1] << "," << perms_[2];
+    }
+}
+
+template <typename Dtype>
 int operation_deconvolution<Dtype>::init_weights(FILE* fp) {
     int tag = 0;
     if (std::fread(&tag, sizeof(int), 1, fp) != 1) LOG(FATAL) << "Deconvolution: model file too short";
@@ -1131,6 +1255,11 @@ INSTANCE_CLASS(operation_concat);
 INSTANCE_CLASS(operation_interp);
 INSTANCE_CLASS(operation_yolov5focus);
 INSTANCE_CLASS(operation_deconvolution);
+INSTANCE_CLASS(operation_clip);
+INSTANCE_CLASS(operation_reshape);
+INSTANCE_CLASS(operation_flatten);
+INSTANCE_CLASS(operation_softmax);
+INSTANCE_CLASS(operation_transpose);
 
 REGISTE(operation_convolution);
 REGISTE(operation_convolutiondepthwise);
@@ -1151,6 +1280,11 @@ REGISTE(operation_concat);
 REGISTE(operation_interp);
 REGISTE(operation_yolov5focus);
 REGISTE(operation_deconvolution);
+REGISTE(operation_clip);
+REGISTE(operation_reshape);
+REGISTE(operation_flatten);
+REGISTE(operation_softmax);
+REGISTE(operation_transpose);
 
 }  // namespace excalibur
 }  // namespace glasssix

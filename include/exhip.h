@@ -185,6 +185,7 @@ int exhip_relu_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, size_t count)
 #define EXHIP_UNARY_LEAKYRELU 1
 #define EXHIP_UNARY_SIGMOID 2
 #define EXHIP_UNARY_HARDSIGMOID 3
+#define EXHIP_UNARY_CLIP 4 /* max(alpha, min(beta, x)), src/Excalibur/operation_clip.cpp:32-58 */
 int exhip_unary_f32(exhip_ctx* ctx, int op, const float* x, float* y, size_t count, float alpha, float beta);
 /* Per-channel layers on NCHW float tensors: PReLU, p0 = slope[c] or one shared slope (operation_prelu.cpp:57-124);
  * BatchNorm as fma(p1[c], x, p0[c]) with a = p0, b = p1 computed at load time (operation_batchnorm.cpp:52-64,122-156);
@@ -203,6 +204,13 @@ int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y, int n, in
 /* operation_yolov5focus::forward_cpu_f32 (operation_yolov5focus.cpp:17-50), for every image of the batch
  * (the reference fills image 0 only). y: [n][4c][h/2][w/2]. */
 int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w);
+
+/* operation_softmax::forward_cpu_f32, NCHW branch (src/Excalibur/operation_softmax.cpp:36-96): softmax over the channels of
+ * every (image, position); x, y [n][c][hw]. */
+int exhip_softmax_channels_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int hw);
+/* operation_transpose::forward_cpu_f32, order (1, 0, 2) (src/Excalibur/operation_transpose.cpp:51-70): rows and columns of
+ * each of `planes` planes change places, y[p][i][j] = x[p][j][i]; x [planes][h][w], y [planes][w][h]. */
+int exhip_transpose_hw_f32(exhip_ctx* ctx, const float* x, float* y, int planes, int h, int w);
 
 /* operation_deconvolution::forward_cpu_f32 (src/Excalibur/operation_deconvolution.cpp:80-171), group 1, dilation 1:
  * x NCHW, w [c][k][kh][kw], y [n][k][(h-1)*sh + kh - pt - pb][(w-1)*sw + kw - pl - pr] = scatter of W^T x (+ bias). */

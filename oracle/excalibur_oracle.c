@@ -556,3 +556,40 @@ void exo_deconv2d_f32(const float* x, const float* w, const float* bias, float* 
                     y[(((size_t)img * k + ko) * oh + oy) * ow + ox] = (float)s;
                 }
 }
+
+/* operation_clip::forward_cpu_f32, src/Excalibur/operation_clip.cpp:32-58: max(lo, min(hi, x)) (vector body and scalar
+ * tail agree for lo <= hi). */
+void exo_clip_f32(const float* x, float* y, long count, float lo, float hi) {
+    for (long i = 0; i < count; ++i) {
+        const float t = hi < x[i] ? hi : x[i];
+        y[i] = lo < t ? t : lo;
+    }
+}
+
+/* operation_softmax::forward_cpu_f32, NCHW branch, src/Excalibur/operation_softmax.cpp:36-96: over the channels of each
+ * (image, position): subtract the maximum (exactly x - m, the GEMM update has a single product per element), exponentiate,
+ * divide by the sum over channels. The reference sums in its GEMV's order; here channels are added in ascending order
+ * (compared at 1e-4). */
+void exo_softmax_channels_f32(const float* x, float* y, int n, int c, int hw) {
+    for (int img = 0; img < n; ++img)
+        for (int k = 0; k < hw; ++k) {
+            const float* in = x + (size_t)img * c * hw + k;
+            float* out = y + (size_t)img * c * hw + k;
+            float m = in[0];
+            for (int j = 0; j < c; ++j) m = m < in[(size_t)j * hw] ? in[(size_t)j * hw] : m;
+            float sum = 0.f;
+            for (int j = 0; j < c; ++j) {
+                out[(size_t)j * hw] = expf(in[(size_t)j * hw] - m);
+                sum += out[(size_t)j * hw];
+            }
+            for (int j = 0; j < c; ++j) out[(size_t)j * hw] = out[(size_t)j * hw] / sum;
+        }
+}
+
+/* operation_transpose::forward_cpu_f32, order (1, 0, 2), src/Excalibur/operation_transpose.cpp:51-70: rows and columns
+ * of every channel plane change places, y[n][c][i][j] = x[n][c][j][i], output shape [n][c][w][h]. */
+void exo_transpose_hw_f32(const float* x, float* y, long planes, int h, int w) {
+    for (long p = 0; p < planes; ++p)
+        for (int i = 0; i < w; ++i)
+            for (int j = 0; j < h; ++j) y[((size_t)p * w + i) * h + j] = x[((size_t)p * h + j) * w + i];
+}

@@ -23,6 +23,8 @@
  *   concat_channels / interp_nearest       reference fixtures (bit-exact), element counts with and without a vector tail
  *   exo_deconv2d_f32                       float64 evaluation of the definition, reference fixtures at 1e-4
  *   exo_focus_f32                          reference fixture (bit-exact) for one image; further images by the same formula
+ *   exo_clip_f32, exo_transpose_hw_f32     reference fixtures (bit-exact)
+ *   exo_softmax_channels_f32               reference fixtures at 1e-4; rows sum to 1, invariance under a shift of the input
  * No function here is "parity unpinned".
  */
 #ifndef EXCALIBUR_ORACLE_H_
@@ -84,6 +86,9 @@ void exo_hardswish_f32(const float* x, float* y, long count, float alpha, float 
 void exo_leakyrelu_f32(const float* x, float* y, long count, float alpha);
 void exo_sigmoid_f32(const float* x, float* y, long count);
 void exo_hardsigmoid_f32(const float* x, float* y, long count, float alpha, float beta);
+void exo_clip_f32(const float* x, float* y, long count, float lo, float hi);
+void exo_softmax_channels_f32(const float* x, float* y, int n, int c, int hw);
+void exo_transpose_hw_f32(const float* x, float* y, long planes, int h, int w);
 void exo_prelu_f32(const float* x, float* y, int n, int c, int hw, const float* slope, int shared);
 void exo_batchnorm_f32(const float* x, float* y, int n, int c, int hw, const float* slope, const float* mean,
                        const float* var, const float* bias, float eps, float* ab);

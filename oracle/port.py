@@ -247,6 +247,27 @@ def hardsigmoid(x, alpha=0.2, beta=0.5):
     return _unary(lib().exo_hardsigmoid_f32, x, alpha, beta)
 
 
+def clip(x, lo, hi):
+    return _unary(lib().exo_clip_f32, x, lo, hi)
+
+
+def softmax_channels(x):
+    """Softmax over the channel axis of an NCHW tensor (the reference's only axis)."""
+    x = _f32(x)
+    n, c = x.shape[:2]
+    y = np.empty(x.shape, np.float32)
+    lib().exo_softmax_channels_f32(_p(x), _p(y), n, c, int(np.prod(x.shape[2:], dtype=np.int64)))
+    return y
+
+
+def transpose_hw(x):
+    x = _f32(x)
+    n, c, h, w = x.shape
+    y = np.empty((n, c, w, h), np.float32)
+    lib().exo_transpose_hw_f32(_p(x), _p(y), ctypes.c_long(n * c), h, w)
+    return y
+
+
 def prelu(x, slope):
     x, slope = _f32(x), _f32(slope)
     n, c, h, w = x.shape

@@ -86,6 +86,21 @@ def unary_case(seed, kind, shape, **params):
     return dict(op=kind, x=_rng(seed).uniform(-4, 4, shape).astype(np.float32), **params)
 
 
+def reshape_shape(case):
+    """The layer's shape rule (src/Excalibur/operation_reshape.cpp:49-86): given dimensions replace the old ones, absent
+    ones (or negative ones) follow from the element count, channels first, then height, then width."""
+    shape = list(case["x"].shape)
+    given = [None, case.get("new_c"), case.get("new_h"), case.get("new_w")]
+    for axis in (1, 2, 3):
+        if given[axis] is not None and given[axis] > 0:
+            shape[axis] = given[axis]
+    for axis in (1, 2, 3):
+        if given[axis] is None or given[axis] < 0:
+            others = int(np.prod([shape[i] for i in range(4) if i != axis]))
+            shape[axis] = case["x"].size // others
+    return tuple(shape)
+
+
 def prelu_case(seed, shape, shared=False):
     r = _rng(seed)
     return dict(op="prelu", x=r.uniform(-2, 2, shape).astype(np.float32),
@@ -160,6 +175,17 @@ def reference_io(case):
     if op == "interp":
         # key 1 is read into the width scale and key 2 into the height scale (src/Excalibur/operation_interp.cpp:196-201)
         return mf.topology([f"Interp layer 1 1 data out 0=1 1={case['width_scale']!r} 2={case['height_scale']!r}"]), b"", [case["x"]], "out"
+    if op == "clip":
+        return mf.topology([f"Clip layer 1 1 data out 0={case['lo']!r} 1={case['hi']!r}"]), b"", [case["x"]], "out"
+    if op == "softmax":
+        return mf.topology(["Softmax layer 1 1 data out 0=0"]), b"", [case["x"]], "out"
+    if op == "transpose":
+        return mf.topology(["Transpose layer 1 1 data out 0=" + ",".join(str(v) for v in case["order"])]), b"", [case["x"]], "out"
+    if op == "reshape":
+        keys = " ".join(f"{k}={case[name]}" for k, name in ((0, "new_w"), (1, "new_h"), (2, "new_c")) if case.get(name) is not None)
+        return mf.topology([f"Reshape layer 1 1 data out {keys}"]), b"", [case["x"]], "out"
+    if op == "flatten":
+        return mf.topology([f"Flatten layer 1 1 data out 0={case['axis']}"]), b"", [case["x"]], "out"
     if op == "prelu":
         return mf.topology([f"PReLU layer 1 1 data out 0={case['slope'].size}"]), mf.floats_blob(case["slope"]), [case["x"]], "out"
     if op == "batchnorm":
@@ -229,6 +255,18 @@ def oracle_eval(case):
         return port.focus(case["x"])
     if op == "interp":
         return port.interp_nearest(case["x"], case["height_scale"], case["width_scale"])
+    if op == "clip":
+        return port.clip(case["x"], case["lo"], case["hi"])
+    if op == "softmax":
+        return port.softmax_channels(case["x"])
+    if op == "transpose":
+        return port.transpose_hw(case["x"]) if tuple(case["order"]) == (1, 0, 2) else case["x"].copy()
+    if op == "reshape":
+        return case["x"].reshape(reshape_shape(case))
+    if op == "flatten":
+        n, c, h, w = case["x"].shape
+        hw = {0: (c * h * w, 1), 1: (c * h, w), 2: (c, h * w)}.get(case["axis"], (1, c * h * w))
+        return case["x"].reshape(n, 1, *hw)
     if op == "prelu":
         return port.prelu(case["x"], case["slope"])
     if op == "batchnorm":

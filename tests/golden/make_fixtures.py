@@ -78,6 +78,16 @@ def fixture_cases():
         "interp_nearest_x2": c.unary_case(71, "interp", (2, 3, 5, 7), height_scale=2.0, width_scale=2.0),
         "interp_nearest_frac": c.unary_case(72, "interp", (1, 2, 6, 5), height_scale=1.5, width_scale=2.5),
         "focus": c.unary_case(73, "focus", (1, 3, 8, 10)),
+        # shape and normalisation layers of the shipped topologies
+        "clip": c.unary_case(77, "clip", (2, 3, 5, 7), lo=-1.5, hi=2.25),
+        "clip_relu6": c.unary_case(78, "clip", (1, 4, 4, 4), lo=0.0, hi=6.0),
+        "softmax_channels": c.unary_case(79, "softmax", (2, 6, 5, 7)),
+        "softmax_vector": c.unary_case(80, "softmax", (3, 10, 1, 1)),
+        "transpose_hw": c.unary_case(81, "transpose", (2, 3, 5, 7), order=(1, 0, 2)),
+        "transpose_identity": c.unary_case(82, "transpose", (1, 2, 4, 6), order=(0, 1, 2)),
+        "reshape_yolo_head": c.unary_case(83, "reshape", (2, 12, 5, 4), new_w=20, new_h=4, new_c=3),
+        "reshape_infer_c": c.unary_case(84, "reshape", (1, 6, 4, 5), new_w=10, new_h=3),
+        "flatten_axis1": c.unary_case(85, "flatten", (2, 3, 4, 5), axis=1),
         # transposed convolution (the detection head's 2x2 stride-2 upsampling, and overlapping taps with padding)
         "deconv_2x2s2": c.deconv_case(74, 2, 6, 5, 7, 4, 2, 2),
         "deconv_4x4s2p1": c.deconv_case(75, 1, 5, 6, 6, 3, 4, 2, 1),

