@@ -180,6 +180,11 @@ public:
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
     void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
+    // The reference reads the int8 blob (one weight scale, one feature-map scale) but has no forward for it
+    // (include/Excalibur/operation.hpp:353-357). Here the layer is the int8 1x1 convolution of the flattened input, with
+    // the int8 convolution's arithmetic: q8(x * fs), int32 sum, fmaf(acc, 1 / (ws * fs), bias).
+    void forward_gpu_i8(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    std::shared_ptr<memory::tensor<float>> scale_dev_;
 };
 
 // ---- activation / glue layers of the shipped topologies (float32 kernels; fp16 pipelines take the base class's

@@ -778,6 +778,36 @@ void operation_innerproduct<Dtype>::forward_gpu_f32(const tensor_list<float>& bo
 }
 
 template <typename Dtype>
+void operation_innerproduct<Dtype>::forward_gpu_i8(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    require_nchw(bottoms[0]->order());
+    if (this->weights_i8_.empty()) {  // a float blob in a layer flagged int8: the float path
+        forward_gpu_f32(bottoms, tops);
+        return;
+    }
+    const int dev = this->params_.device_;
+    const int m = bottoms[0]->num(), n = num_output_, k = bottoms[0]->count(1, 4);
+    CHECK_EQ(k * n, weight_data_size_);
+    const float fs = this->featmap_scaletable_i8_->cpu_data()[0];
+    if (!scale_dev_) {
+        const float ws = this->weights_scaletable_i8_->cpu_data()[0];
+        volatile float prod = ws * fs;  // float product, then float division, as for the convolution
+        const float s = std::fabs(ws) <= 1e-6 ? 0.f : 1.0f / prod;
+        scale_dev_ = vec_tensor<float>(n, dev);
+        for (int i = 0; i < n; ++i) scale_dev_->mutable_cpu_data()[i] = s;
+    }
+    exhip_conv_desc d;
+    std::memset(&d, 0, sizeof(d));
+    d.n = m; d.c = k; d.h = 1; d.w = 1; d.k = n; d.kh = d.kw = 1; d.sh = d.sw = 1;
+    d.c_stride = k; d.k_stride = n;
+    tops[0] = new_tensor<float>({m, n, 1, 1}, dev);
+    EXHIP_FATAL(exhip_conv2d_direct_nchw(this->ctx(), &d, 1, bottoms[0]->gpu_data(), nullptr,
+                                         reinterpret_cast<const int8_t*>(this->weights_i8_[0]->gpu_data()), fs, scale_dev_->gpu_data(),
+                                         bias_term_ ? this->weights_f32_[1]->gpu_data() : nullptr, tops[0]->mutable_gpu_data()));
+}
+
+template <typename Dtype>
 void operation_innerproduct<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
     CHECK_EQ(bottoms.size(), 1);
     CHECK_EQ(tops.size(), 1);

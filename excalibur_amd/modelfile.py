@@ -55,6 +55,7 @@ def conv_blob_i8(w, bias, ws, fs):
 
 
 fc_blob_f32 = conv_blob_f32
+fc_blob_i8 = conv_blob_i8  # one weight scale and one feature-map scale (src/Excalibur/operation_innerproduct.cpp:95-113)
 
 
 def floats_blob(*arrays):

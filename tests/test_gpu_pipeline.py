@@ -225,6 +225,36 @@ def test_classifier_tail_flatten_innerproduct_softmax():
         os.unlink(path)
 
 
+@pytest.mark.parametrize("bias", [True, False])
+def test_int8_innerproduct_is_the_int8_1x1_convolution_of_the_flattened_input(bias):
+    """The reference reads the int8 InnerProduct blob but has no forward for it (include/Excalibur/operation.hpp:353-357).
+    The layer is defined here by the int8 convolution's arithmetic, so the pinned int8 convolution restatement, run as a
+    1x1 convolution over the [m][c*h*w][1][1] view of the input, is its oracle: bit-exact."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(71)
+    x = r.uniform(-3, 3, (5, 6, 3, 4)).astype(np.float32)
+    k, n_out = 72, 10
+    wq = r.integers(-127, 128, (n_out, k)).astype(np.int8)
+    fs = np.float32(127.0 / np.abs(x).max() * 1.05)
+    ws = np.float32(1.0 / (3e-3 * fs))
+    b = r.normal(0, 0.5, (n_out,)).astype(np.float32) if bias else None
+    line = f"InnerProduct fc 1 1 data out 0={n_out} 1={int(bias)} 2={wq.size} 8=1"
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        f.write(mf.fc_blob_i8(wq, b, np.array([ws], np.float32), fs))
+        path = f.name
+    try:
+        p = xp.Pipeline(mf.topology([line]), path, 0)
+        p.forward(x)
+        g = port.geom((5, k, 1, 1), n_out, 1)
+        want = port.conv2d_i8(x.reshape(5, k, 1, 1), wq.reshape(n_out, k, 1, 1), b, np.full((n_out,), ws, np.float32), fs, 0, g)
+        got = p.get("out")
+        assert got.shape == (5, n_out, 1, 1)
+        assert np.array_equal(got, want)
+        p.close()
+    finally:
+        os.unlink(path)
+
+
 def test_input_layer_without_bottoms_normalises_the_pipeline_input():
     """`Input name 0 1 blob ...` (no bottoms): the pipeline input is `<name>_input`, the layer subtracts the means and
     scales (one scale repeated over the channels), then a float convolution with PReLU behind it: fp32 and fp16."""
