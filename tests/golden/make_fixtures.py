@@ -19,7 +19,7 @@ from tests import cases  # noqa: E402
 from tests.refrun import run_reference  # noqa: E402
 
 
-NETWORKS = ("net_mobilefacenet_f32",)  # whole-topology fixtures: not single-layer cases
+NETWORKS = ("net_mobilefacenet_f32", "net_yolov5_shaped_f32")  # whole-topology fixtures: not single-layer cases
 
 
 def fixture_cases():
@@ -162,6 +162,17 @@ def main():
     out = ref.run(net.topology(), path, x, [net.output])[net.output]
     os.unlink(path)
     np.savez_compressed(os.path.join(HERE, "net_mobilefacenet_f32.npz"), input_seed=np.asarray(8), expected=out)
+    # a YOLOv5s-shaped float topology (excalibur_amd.yolo), one image: the reference's outputs of both heads
+    from excalibur_amd.yolo import YoloV5ShapedF32
+    net = YoloV5ShapedF32()
+    x = np.random.default_rng(9).uniform(0, 255, (1, 3, net.hw, net.hw)).astype(np.float32)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    net.write_model(path)
+    outs = ref.run(net.topology(), path, x, net.outputs)
+    os.unlink(path)
+    np.savez_compressed(os.path.join(HERE, "net_yolov5_shaped_f32.npz"), input_seed=np.asarray(9),
+                        **{f"expected{i}": outs[n] for i, n in enumerate(net.outputs)})
     total = sum(os.path.getsize(os.path.join(HERE, f)) for f in os.listdir(HERE) if f.endswith(".npz"))
     print(f"wrote {len(fixture_cases()) + len(f16_cases())} fixtures, {total / 1024:.0f} KiB")
 

@@ -77,3 +77,42 @@ def oracle_forward_mobilenet(net, x):
         elif kind == "fc":
             blobs[op[2]] = port.innerproduct(blobs[op[1]], op[3], op[4])
     return blobs[net.output], blobs
+
+
+def oracle_forward_yolo(net, x):
+    """The float YOLOv5-shaped network (excalibur_amd.yolo) op by op through the oracle restatement."""
+    blobs = {"images_input": np.ascontiguousarray(x, np.float32)}
+    for op in net.ops:
+        kind = op[0]
+        if kind == "input":
+            blobs[op[2]] = port.input_layer(blobs[op[1]], [0.0, 0.0, 0.0], [net.scale] * 3)
+        elif kind == "focus":
+            blobs[op[2]] = port.focus(blobs[op[1]])
+        elif kind == "conv":
+            _, bottom, top, w, b, kernel, stride, pad = op
+            xin = blobs[bottom]
+            blobs[top] = port.conv2d_f32(xin, w, b, 0, port.geom(xin.shape, w.shape[0], kernel, kernel, stride, pad))
+        elif kind == "hardswish":
+            blobs[op[2]] = port.hardswish(blobs[op[1]], op[3], op[4])
+        elif kind == "leakyrelu":
+            blobs[op[2]] = port.leakyrelu(blobs[op[1]], op[3])
+        elif kind == "split":
+            for t in op[2]:
+                blobs[t] = blobs[op[1]]
+        elif kind == "add":
+            blobs[op[2]] = port.binaryop_add(blobs[op[1][0]], blobs[op[1][1]])
+        elif kind == "concat":
+            blobs[op[2]] = port.concat_channels([blobs[n] for n in op[1]])
+        elif kind == "batchnorm":
+            blobs[op[2]] = port.batchnorm(blobs[op[1]], op[3], op[4], op[5], op[6], 0.0)
+        elif kind == "maxpool":
+            blobs[op[2]] = port.pool2d(blobs[op[1]], port.POOL_MAX, op[3], 1, op[3] // 2)
+        elif kind == "interp":
+            blobs[op[2]] = port.interp_nearest(blobs[op[1]], op[3], op[4])
+        elif kind == "reshape":
+            blobs[op[2]] = blobs[op[1]].reshape((blobs[op[1]].shape[0],) + tuple(op[3]))
+        elif kind == "transpose":
+            blobs[op[2]] = port.transpose_hw(blobs[op[1]])
+        else:
+            raise ValueError(kind)
+    return [blobs[n] for n in net.outputs], blobs

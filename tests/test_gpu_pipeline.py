@@ -315,3 +315,33 @@ def test_mobilefacenet_shaped_float_topology_matches_the_reference_fixture():
         p16.close()
     finally:
         os.unlink(path)
+
+
+def test_yolov5_shaped_float_topology_matches_the_reference_fixture():
+    """Focus -> HardSwish convolutions -> cross-stage block (BinaryOp sum, Concat, BatchNorm, LeakyRelu) -> pyramid of
+    5 / 9 / 13 max pools -> upsampling + Concat -> two heads ending in Reshape + Transpose, loaded from generated
+    `.phai` + `.racy`: float32 against the compiled reference's outputs, float16 alongside."""
+    from excalibur_amd.yolo import YoloV5ShapedF32
+    net = YoloV5ShapedF32()
+    z = np.load(os.path.join(GOLDEN, "net_yolov5_shaped_f32.npz"))
+    x = np.random.default_rng(int(z["input_seed"])).uniform(0, 255, (1, 3, net.hw, net.hw)).astype(np.float32)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        net.write_model(path)
+        p = xp.Pipeline(net.topology(), path, 0)
+        p.forward(x)
+        assert not p.fused
+        for i, name in enumerate(net.outputs):
+            got = p.get(name)
+            assert got.shape == z[f"expected{i}"].shape
+            assert cases.check_value(got, z[f"expected{i}"], 1e-4) == 0
+        p.close()
+        p16 = xp.Pipeline(net.topology(), path, 0, "f16")
+        p16.forward(x.astype(np.float16).view(np.uint16))
+        for i, name in enumerate(net.outputs):
+            got16 = p16.get(name).view(np.float16).astype(np.float32)
+            assert cases.check_value(got16, z[f"expected{i}"], 3e-2) == 0  # every layer rounds to half
+        p16.close()
+    finally:
+        os.unlink(path)

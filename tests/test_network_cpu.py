@@ -49,3 +49,28 @@ def test_mobilefacenet_shaped_topology_oracle_equals_compiled_reference():
         os.unlink(path)
     assert np.array_equal(got, z["expected"])
     assert cases.check_value(got.reshape(want.shape), want, 1e-4) == 0
+
+
+@pytest.mark.ref
+def test_yolov5_shaped_topology_oracle_equals_compiled_reference():
+    """The float detector topology of excalibur_amd.yolo (Focus, HardSwish convolutions, cross-stage block, pyramid of
+    5 / 9 / 13 max pools, upsampling, two Reshape + Transpose heads): the op-by-op oracle evaluation against the
+    compiled reference running the generated `.phai` / `.racy`, and against the committed fixture."""
+    import tempfile
+    from excalibur_amd.yolo import YoloV5ShapedF32
+    from oracle import ref
+    net = YoloV5ShapedF32()
+    z = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "net_yolov5_shaped_f32.npz"))
+    x = np.random.default_rng(int(z["input_seed"])).uniform(0, 255, (1, 3, net.hw, net.hw)).astype(np.float32)
+    want, _ = netref.oracle_forward_yolo(net, x)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        net.write_model(path)
+        got = ref.run(net.topology(), path, x, net.outputs)
+    finally:
+        os.unlink(path)
+    for i, name in enumerate(net.outputs):
+        assert np.array_equal(got[name], z[f"expected{i}"])
+        assert got[name].shape == want[i].shape == (1, 3, (net.hw // (4 << i)) ** 2, 6)
+        assert cases.check_value(got[name], want[i], 1e-4) == 0
