@@ -269,16 +269,23 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
             iy += wrap;
         }
     } else {
-        const int npix = p.IH * p.IW;
+        // the same without branches; pixel tid + THREADS * i advances by (adv_iy, adv_ix) per i
+        const int H = p.H, W = p.W, IW = p.IW, cs_b = p.cstride_b, oob = (int)p.img_bytes, row_b = p.lds_row_b, pix_b = p.lds_pix_b;
+        const int d_iy = p.adv_iy, d_ix = p.adv_ix;
+        const int npix = p.IH * IW;
+        int iy = fast_div(tid, p.magic_iw), ix = tid - iy * IW;
 #pragma unroll
         for (int i = 0; i < NPP; ++i) {
-            const int v = tid + THREADS * i;
-            const int iy = fast_div(v, p.magic_iw), ix = v - iy * p.IW;
             const int gy = iy0 + iy, gx = ix0 + ix;
-            const bool in_tile = v < npix;
-            const bool in_img = in_tile && gy >= 0 && gy < p.H && gx >= 0 && gx < p.W;
-            a_loff[i] = in_tile ? iy * p.lds_row_b + ix * p.lds_pix_b : -1;
-            a_goff[i] = in_img ? (gy * p.W + gx) * p.cstride_b : (int)p.img_bytes;
+            const bool in_tile = tid + THREADS * i < npix;
+            const bool in_img = in_tile & ((unsigned)gy < (unsigned)H) & ((unsigned)gx < (unsigned)W);
+            a_loff[i] = in_tile ? iy * row_b + ix * pix_b : -1;
+            a_goff[i] = in_img ? (gy * W + gx) * cs_b : oob;
+            ix += d_ix;
+            iy += d_iy;
+            const int wrap = ix >= IW ? 1 : 0;
+            ix -= wrap ? IW : 0;
+            iy += wrap;
         }
     }
 
@@ -1287,7 +1294,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.vp_shift = pl.chunk_b == 64 ? 2 : 1;
     p.SL = pl.SL; p.act_need_b = pl.act_need_b;
     p.magic_sl = (unsigned)(((1ull << 32) + pl.SL - 1) / pl.SL);
-    p.adv_part = pl.threads % pl.SL; p.adv_pix = pl.threads / pl.SL;
+    p.adv_part = pl.threads % pl.SL; p.adv_pix = pl.packed ? pl.threads : pl.threads / pl.SL;  // packed: a slot is a pixel
     p.adv_iy = p.adv_pix / pl.IW; p.adv_ix = p.adv_pix % pl.IW;
     p.tile_dy = pl.PH; p.tile_dx = pl.PW;
     if (pool) {
