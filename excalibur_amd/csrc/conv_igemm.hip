@@ -368,7 +368,11 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
                     for (int s_ = 0; s_ < NS; ++s_) {
                         if (s_ + 1 < NS) fetch_at((P0 + s_ + 1) & 1, wl, ar, s_ + 1);
                         else if (has_next) fetch_at((P0 + s_ + 1) & 1, wl + NS * STEPB, nr, 0);
+                        // keep the order written here: the next k-step's fragment reads go out before this k-step's
+                        // MFMAs and are waited for after them (left alone, the scheduler sinks the reads to their uses)
+                        __builtin_amdgcn_sched_barrier(0);
                         compute((P0 + s_) & 1);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                     wl += NS * STEPB;
 #pragma unroll
