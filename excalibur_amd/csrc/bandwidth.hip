@@ -844,6 +844,53 @@ __global__ __launch_bounds__(kBlock) void eltwise_f32_v4_kernel(EltArgs a, float
     y[j] = r;
 }
 
+// BinaryOp ADD / SUB / MUL / DIV (OP 0..3) with a smaller second operand. MODE 0: equal shapes, op(large, small);
+// 1: one value per image, op(large, value); 2: one value per (image, channel), op(value, large) -- the reference puts
+// the smaller operand first there; 3: one value per (image, pixel), op(value, large). The smaller operand's images
+// repeat modulo its batch size. Four floats per thread along a plane.
+template <int OP>
+__device__ __forceinline__ float binop_value(float x, float y) {
+    if constexpr (OP == 0) return x + y;
+    else if constexpr (OP == 1) return x - y;
+    else if constexpr (OP == 2) return x * y;
+    else return x / y;
+}
+template <int OP, int MODE, int VEC>
+__global__ __launch_bounds__(kBlock) void binaryop_f32_kernel(const float* __restrict__ big, const float* __restrict__ small,
+                                                              float* __restrict__ y, int C, int HW, int small_n, size_t total) {
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;  // one thread per VEC consecutive values of a plane
+    if (t >= total) return;
+    const int per_plane = HW / VEC;
+    const size_t plane = t / per_plane;
+    const int p = (int)(t - plane * per_plane) * VEC;
+    const int c = (int)(plane % C);
+    const size_t img = plane / C;
+    const size_t at = plane * HW + p;
+    const size_t simg = img % small_n;
+    float b[VEC], s[VEC], r[VEC];
+    if constexpr (VEC == 4) {
+        const v4f v = *reinterpret_cast<const v4f*>(big + at);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) b[e] = v[e];
+    } else {
+        b[0] = big[at];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        if constexpr (MODE == 0) s[e] = small[at + e];
+        else if constexpr (MODE == 1) s[e] = small[simg];
+        else if constexpr (MODE == 2) s[e] = small[simg * C + c];
+        else s[e] = small[simg * HW + p + e];
+        r[e] = MODE <= 1 ? binop_value<OP>(b[e], s[e]) : binop_value<OP>(s[e], b[e]);
+    }
+    if constexpr (VEC == 4) {
+        const v4f o = {r[0], r[1], r[2], r[3]};
+        *reinterpret_cast<v4f*>(y + at) = o;
+    } else {
+        y[at] = r[0];
+    }
+}
+
 // ---- activation / glue layers ----
 // One value of an elementwise activation. OP 0 HardSwish, 1 LeakyReLU, 2 sigmoid, 3 HardSigmoid, 4 Clip; the multiply-adds
 // are fused where the CPU path's are (vector fmadd, and scalar expressions contracted by its compiler flags).
@@ -1724,6 +1771,45 @@ extern "C" int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, 
     hipLaunchKernelGGL(focus_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total);
     EXHIP_LAUNCH_CHECK();
     return 0;
+}
+
+template <int OP, int MODE>
+static int launch_binaryop(exhip_ctx* ctx, const float* big, const float* small, float* y, int n, int c, int hw, int small_n) {
+    const bool vec = hw % 4 == 0 && (uintptr_t)big % 16 == 0 && (uintptr_t)y % 16 == 0;
+    const size_t total = (size_t)n * c * (vec ? hw / 4 : hw);
+    if (vec)
+        hipLaunchKernelGGL((binaryop_f32_kernel<OP, MODE, 4>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, big, small, y, c,
+                           hw, small_n, total);
+    else
+        hipLaunchKernelGGL((binaryop_f32_kernel<OP, MODE, 1>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, big, small, y, c,
+                           hw, small_n, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+template <int OP>
+static int launch_binaryop_mode(exhip_ctx* ctx, int mode, const float* big, const float* small, float* y, int n, int c, int hw,
+                                int small_n) {
+    switch (mode) {
+    case EXHIP_BINARY_EQUAL: return launch_binaryop<OP, 0>(ctx, big, small, y, n, c, hw, small_n);
+    case EXHIP_BINARY_PER_IMAGE: return launch_binaryop<OP, 1>(ctx, big, small, y, n, c, hw, small_n);
+    case EXHIP_BINARY_PER_CHANNEL: return launch_binaryop<OP, 2>(ctx, big, small, y, n, c, hw, small_n);
+    case EXHIP_BINARY_PER_PIXEL: return launch_binaryop<OP, 3>(ctx, big, small, y, n, c, hw, small_n);
+    default: exhip_set_error("exhip_binaryop_f32: unknown mode %d", mode); return EXHIP_ERR_ARG;
+    }
+}
+
+extern "C" int exhip_binaryop_f32(exhip_ctx* ctx, int op, int mode, const float* large, const float* small, float* y, int n, int c,
+                                  int hw, int small_n) {
+    REQ_CTX("exhip_binaryop_f32");
+    EXHIP_REQUIRE(large && small && y && n > 0 && c > 0 && hw > 0 && small_n > 0, "exhip_binaryop_f32: bad argument");
+    EXHIP_REQUIRE(mode != EXHIP_BINARY_EQUAL || small_n == n, "exhip_binaryop_f32: equal shapes need equal batch sizes");
+    switch (op) {
+    case 0: return launch_binaryop_mode<0>(ctx, mode, large, small, y, n, c, hw, small_n);
+    case 1: return launch_binaryop_mode<1>(ctx, mode, large, small, y, n, c, hw, small_n);
+    case 2: return launch_binaryop_mode<2>(ctx, mode, large, small, y, n, c, hw, small_n);
+    case 3: return launch_binaryop_mode<3>(ctx, mode, large, small, y, n, c, hw, small_n);
+    default: exhip_set_error("exhip_binaryop_f32: unknown op %d (0 ADD, 1 SUB, 2 MUL, 3 DIV)", op); return EXHIP_ERR_ARG;
+    }
 }
 
 extern "C" int exhip_softmax_channels_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int hw) {

@@ -41,8 +41,8 @@ extern "C" int exhip_init(int device, exhip_ctx** out) {
 
 extern "C" int exhip_destroy(exhip_ctx* ctx) {
     if (!ctx) return 0;
-    hipStreamSynchronize(ctx->stream);
-    hipStreamDestroy(ctx->stream);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return 0;
 }

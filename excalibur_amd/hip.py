@@ -344,6 +344,13 @@ class Ctx:
         _check(lib().exhip_focus_f32(self.h, x.ptr, y.ptr, n, c, h, w))
         return y
 
+    def binaryop_f32(self, op, mode, large, small):
+        """op 0 ADD / 1 SUB / 2 MUL / 3 DIV; mode 0 equal shapes, 1 per image, 2 per (image, channel), 3 per (image, pixel)."""
+        n, c, h, w = large.shape
+        y = self.empty(large.shape, np.float32)
+        _check(lib().exhip_binaryop_f32(self.h, int(op), int(mode), large.ptr, small.ptr, y.ptr, n, c, h * w, small.shape[0]))
+        return y
+
     def softmax_channels_f32(self, x):
         n, c = x.shape[:2]
         y = self.empty(x.shape, np.float32)

@@ -126,7 +126,7 @@ public:
     using tensor_list = typename operation<Dtype>::template tensor_list<T>;
     explicit operation_binaryop(const operation_param& param);
     const char* type() const override { return this->params_.type_.c_str(); }
-    int op_type_ = 0;  // 0 ADD (the only one on the hot path)
+    int op_type_ = 0;  // 0 ADD, 1 SUB, 2 MUL, 3 DIV
     int with_scalar_ = 0;
     float coef_ = 0.f;
 

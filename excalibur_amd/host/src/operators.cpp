@@ -621,17 +621,47 @@ template <typename Dtype>
 void operation_binaryop<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
     CHECK_GE(bottoms.size(), 1);
     CHECK_EQ(tops.size(), 1);
-    if (op_type_ != 0 || with_scalar_ || bottoms.size() != 2 || bottoms[0]->data_shape() != bottoms[1]->data_shape())
-        LOG(FATAL) << "layer " << this->params_.name_ << ": this backend implements BinaryOp as equal-shape ADD only (the residual add)";
-    tops[0] = std::make_shared<tensor<float>>(bottoms[0]->data_shape(), this->params_.device_, bottoms[0]->order());
-    EXHIP_FATAL(exhip_add_f32(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
+    if (with_scalar_ || bottoms.size() != 2 || op_type_ < 0 || op_type_ > 3) NOT_IMPLEMENTED << " BinaryOp with a scalar, one operand or op " << op_type_;
+    require_nchw(bottoms[0]->order());
+    if (op_type_ == 0 && bottoms[0]->data_shape() == bottoms[1]->data_shape()) {  // the residual add
+        tops[0] = std::make_shared<tensor<float>>(bottoms[0]->data_shape(), this->params_.device_, bottoms[0]->order());
+        EXHIP_FATAL(exhip_add_f32(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
+        return;
+    }
+    // which operand gives the output its shape: src/Excalibur/operation_binaryop.cpp:9-42
+    auto dims_of = [](const tensor<float>& t) { return (t.width() != 1) + (t.height() != 1) + (t.channels() != 1); };
+    const std::vector<int> s1 = bottoms[0]->data_shape(), s2 = bottoms[1]->data_shape();
+    bool second_larger = false;
+    if (s1 != s2) {
+        const int d1 = dims_of(*bottoms[0]), d2 = dims_of(*bottoms[1]);
+        if (d2 > d1) second_larger = true;
+        else if (d2 == d1)
+            for (int i = 1; i < 4; ++i)
+                if (s2[i] > s1[i]) { second_larger = true; break; }
+    }
+    const auto& large = second_larger ? bottoms[1] : bottoms[0];
+    const auto& small = second_larger ? bottoms[0] : bottoms[1];
+    const int hw = large->height() * large->width();
+    const int small_chw = small->channels() * small->height() * small->width();
+    const int large_dims = std::max(1, dims_of(*large)), small_dims = std::max(1, dims_of(*small));
+    int mode = -1;
+    if (s1 == s2) mode = EXHIP_BINARY_EQUAL;
+    else if (small_chw == 1) mode = EXHIP_BINARY_PER_IMAGE;
+    else if (large_dims == 3 && small_dims == 2 && small->channels() == 1 && small->height() * small->width() == hw) mode = EXHIP_BINARY_PER_PIXEL;
+    else if (large_dims == 3 && small_dims == 1 && small->channels() > 1 && small->channels() == large->channels()) mode = EXHIP_BINARY_PER_CHANNEL;
+    if (mode < 0) NOT_IMPLEMENTED << " BinaryOp on these two shapes";
+    tops[0] = std::make_shared<tensor<float>>(large->data_shape(), this->params_.device_, large->order());
+    EXHIP_FATAL(exhip_binaryop_f32(this->ctx(), op_type_, mode, large->gpu_data(), small->gpu_data(), tops[0]->mutable_gpu_data(),
+                                   large->num(), large->channels(), hw, small->num()));
 }
 
 template <typename Dtype>
 void operation_binaryop<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
     CHECK_EQ(tops.size(), 1);
-    if (op_type_ != 0 || with_scalar_ || bottoms.size() != 2 || bottoms[0]->data_shape() != bottoms[1]->data_shape())
-        LOG(FATAL) << "layer " << this->params_.name_ << ": this backend implements BinaryOp as equal-shape ADD only (the residual add)";
+    if (op_type_ != 0 || with_scalar_ || bottoms.size() != 2 || bottoms[0]->data_shape() != bottoms[1]->data_shape()) {
+        operation<Dtype>::forward_gpu_f16(bottoms, tops);  // everything but the residual add: convert, float kernel, convert back
+        return;
+    }
     tops[0] = std::make_shared<tensor<unsigned short>>(bottoms[0]->data_shape(), this->params_.device_, bottoms[0]->order());
     EXHIP_FATAL(exhip_add_f16(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
 }

@@ -178,6 +178,17 @@ int exhip_relu_f32(exhip_ctx* ctx, const float* x, float* y, size_t count);
 int exhip_add_f16(exhip_ctx* ctx, const uint16_t* a, const uint16_t* b, uint16_t* y, size_t count, int relu);
 int exhip_relu_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, size_t count);
 
+/* operation_binaryop::forward_cpu_f32 beyond the equal-shape add (src/Excalibur/operation_binaryop.cpp:44-199,395-448):
+ * op 0 ADD, 1 SUB, 2 MUL, 3 DIV; `large` [n][c][hw] gives the output its shape, `small` is, by mode, the same shape
+ * (op(large, small)), one value per image (op(large, value)), [small_n][c] (op(value, large): the reference puts the
+ * smaller operand first here) or [small_n][hw] (op(value, large)); its images repeat modulo small_n. */
+#define EXHIP_BINARY_EQUAL 0
+#define EXHIP_BINARY_PER_IMAGE 1
+#define EXHIP_BINARY_PER_CHANNEL 2
+#define EXHIP_BINARY_PER_PIXEL 3
+int exhip_binaryop_f32(exhip_ctx* ctx, int op, int mode, const float* large, const float* small, float* y, int n, int c, int hw,
+                       int small_n);
+
 /* Elementwise activations of the shipped topologies. HardSwish x * clamp(alpha*x + beta, 0, 1)
  * (src/Excalibur/operation_hardswish.cpp:32-63), LeakyReLU (operation_leakyrelu.cpp:31-58), sigmoid evaluated in double
  * (operation_sigmoid.cpp:17-33), HardSigmoid clamp(alpha*x + beta, 0, 1) (operation_hardsigmoid.cpp:33-46). */

@@ -593,3 +593,64 @@ void exo_transpose_hw_f32(const float* x, float* y, long planes, int h, int w) {
         for (int i = 0; i < w; ++i)
             for (int j = 0; j < h; ++j) y[((size_t)p * w + i) * h + j] = x[((size_t)p * h + j) * w + i];
 }
+
+/* operation_binaryop::forward_cpu_f32 without the scalar form, src/Excalibur/operation_binaryop.cpp:9-96,152-199,395-448:
+ * op 0 ADD, 1 SUB, 2 MUL, 3 DIV on two NCHW tensors. The operand with more non-unit dimensions among (C, H, W) (on a
+ * tie: the second if one of its dimensions is larger) is the "larger" one and gives the output its shape. Cases
+ * restated: equal shapes, op(a, b); a smaller operand of one value per image, op(large, value); [N][C][H][W] with
+ * [N][C][1][1], op(small[c], large) -- the small operand comes first; [N][C][H][W] with [N][1][H][W],
+ * op(small[pixel], large). The smaller operand's images repeat modulo its batch size. Returns 0, or -1 for a shape
+ * pair the reference does not implement or that is not restated here. */
+static float exo_binop(int op, float x, float y) {
+    switch (op) {
+    case 0: return x + y;
+    case 1: return x - y;
+    case 2: return x * y;
+    default: return x / y;
+    }
+}
+int exo_binaryop_f32(int op, const float* a, const int* a_shape, const float* b, const int* b_shape, float* y, int* y_shape) {
+    int second_larger = 0, same = 1;
+    for (int i = 0; i < 4; ++i) same = same && a_shape[i] == b_shape[i];
+    if (!same) {
+        const int d1 = (a_shape[3] != 1) + (a_shape[2] != 1) + (a_shape[1] != 1);
+        const int d2 = (b_shape[3] != 1) + (b_shape[2] != 1) + (b_shape[1] != 1);
+        if (d2 > d1) second_larger = 1;
+        else if (d2 == d1)
+            for (int i = 1; i < 4; ++i)
+                if (b_shape[i] > a_shape[i]) { second_larger = 1; break; }
+    }
+    const float* big = second_larger ? b : a;
+    const float* small = second_larger ? a : b;
+    const int* bs = second_larger ? b_shape : a_shape;
+    const int* ss = second_larger ? a_shape : b_shape;
+    for (int i = 0; i < 4; ++i) y_shape[i] = bs[i];
+    const long chw = (long)bs[1] * bs[2] * bs[3], hw = (long)bs[2] * bs[3], small_chw = (long)ss[1] * ss[2] * ss[3];
+    int big_dims = (bs[3] != 1) + (bs[2] != 1) + (bs[1] != 1), small_dims = (ss[3] != 1) + (ss[2] != 1) + (ss[1] != 1);
+    big_dims = big_dims ? big_dims : 1;
+    small_dims = small_dims ? small_dims : 1;
+    if (same) {
+        for (long i = 0; i < bs[0] * chw; ++i) y[i] = exo_binop(op, big[i], small[i]);
+        return 0;
+    }
+    if (small_chw == 1) {
+        for (int n = 0; n < bs[0]; ++n)
+            for (long i = 0; i < chw; ++i) y[n * chw + i] = exo_binop(op, big[n * chw + i], small[n % ss[0]]);
+        return 0;
+    }
+    if (big_dims == 3 && small_dims == 2 && ss[1] == 1 && (long)ss[2] * ss[3] == hw) {
+        for (int n = 0; n < bs[0]; ++n)
+            for (int c = 0; c < bs[1]; ++c)
+                for (long i = 0; i < hw; ++i)
+                    y[n * chw + c * hw + i] = exo_binop(op, small[(n % ss[0]) * small_chw + i], big[n * chw + c * hw + i]);
+        return 0;
+    }
+    if (big_dims == 3 && small_dims == 1 && ss[1] > 1 && ss[1] == bs[1]) {
+        for (int n = 0; n < bs[0]; ++n)
+            for (int c = 0; c < bs[1]; ++c)
+                for (long i = 0; i < hw; ++i)
+                    y[n * chw + c * hw + i] = exo_binop(op, small[(n % ss[0]) * small_chw + c], big[n * chw + c * hw + i]);
+        return 0;
+    }
+    return -1;
+}

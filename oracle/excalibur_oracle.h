@@ -24,6 +24,7 @@
  *   exo_deconv2d_f32                       float64 evaluation of the definition, reference fixtures at 1e-4
  *   exo_focus_f32                          reference fixture (bit-exact) for one image; further images by the same formula
  *   exo_clip_f32, exo_transpose_hw_f32     reference fixtures (bit-exact)
+ *   exo_binaryop_f32                       reference fixtures (bit-exact) for every op and every restated shape pair
  *   exo_softmax_channels_f32               reference fixtures at 1e-4; rows sum to 1, invariance under a shift of the input
  * No function here is "parity unpinned".
  */
@@ -87,6 +88,7 @@ void exo_leakyrelu_f32(const float* x, float* y, long count, float alpha);
 void exo_sigmoid_f32(const float* x, float* y, long count);
 void exo_hardsigmoid_f32(const float* x, float* y, long count, float alpha, float beta);
 void exo_clip_f32(const float* x, float* y, long count, float lo, float hi);
+int exo_binaryop_f32(int op, const float* a, const int* a_shape, const float* b, const int* b_shape, float* y, int* y_shape);
 void exo_softmax_channels_f32(const float* x, float* y, int n, int c, int hw);
 void exo_transpose_hw_f32(const float* x, float* y, long planes, int h, int w);
 void exo_prelu_f32(const float* x, float* y, int n, int c, int hw, const float* slope, int shared);

@@ -247,6 +247,19 @@ def hardsigmoid(x, alpha=0.2, beta=0.5):
     return _unary(lib().exo_hardsigmoid_f32, x, alpha, beta)
 
 
+def binaryop(a, b, op):
+    """BinaryOp ADD / SUB / MUL / DIV (op 0..3) with the reference's broadcasting rules; the result has the shape of the
+    operand the reference calls the larger one."""
+    a, b = _f32(a), _f32(b)
+    sa = (ctypes.c_int * 4)(*a.shape)
+    sb = (ctypes.c_int * 4)(*b.shape)
+    so = (ctypes.c_int * 4)()
+    y = np.empty(max(a.size, b.size), np.float32)
+    if lib().exo_binaryop_f32(int(op), _p(a), sa, _p(b), sb, _p(y), so) != 0:
+        raise NotImplementedError(f"BinaryOp on shapes {a.shape} and {b.shape}")
+    return y.reshape(tuple(so))
+
+
 def clip(x, lo, hi):
     return _unary(lib().exo_clip_f32, x, lo, hi)
 

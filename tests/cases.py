@@ -86,6 +86,28 @@ def unary_case(seed, kind, shape, **params):
     return dict(op=kind, x=_rng(seed).uniform(-4, 4, shape).astype(np.float32), **params)
 
 
+def binaryop_bc_case(seed, shape, op_type, small, swap=False):
+    """BinaryOp (0 ADD, 1 SUB, 2 MUL, 3 DIV) of a tensor with a smaller operand derived from it inside the topology, the
+    way the shipped networks do (squeeze-and-excite gates): `small` = "equal" (the tensor clipped to [0.5, 3]), "channel"
+    (global average, [n][c][1][1]), "pixel" (a 1x1 convolution to one channel, [n][1][h][w]) or "image" (the global
+    average of that, [n][1][1][1]). swap: the smaller operand is written first in the layer line."""
+    r = _rng(seed)
+    x = r.uniform(0.5, 2.0, shape).astype(np.float32) * r.choice([-1.0, 1.0], shape).astype(np.float32)
+    w = r.uniform(0.2, 1.0, (1, shape[1], 1, 1)).astype(np.float32)
+    return dict(op="binaryop_bc", x=x, op_type=op_type, small=small, swap=swap, wt=w)
+
+
+def binaryop_bc_small(case):
+    """The smaller operand, evaluated by the oracle restatement."""
+    x = case["x"]
+    if case["small"] == "equal":
+        return port.clip(x, 0.5, 3.0)
+    if case["small"] == "channel":
+        return port.pool2d(x, port.POOL_AVE, global_pool=True)
+    plane = port.conv2d_f32(x, case["wt"], None, 0, port.geom(x.shape, 1, 1))
+    return plane if case["small"] == "pixel" else port.pool2d(plane, port.POOL_AVE, global_pool=True)
+
+
 def reshape_shape(case):
     """The layer's shape rule (src/Excalibur/operation_reshape.cpp:49-86): given dimensions replace the old ones, absent
     ones (or negative ones) follow from the element count, channels first, then height, then width."""
@@ -175,6 +197,21 @@ def reference_io(case):
     if op == "interp":
         # key 1 is read into the width scale and key 2 into the height scale (src/Excalibur/operation_interp.cpp:196-201)
         return mf.topology([f"Interp layer 1 1 data out 0=1 1={case['width_scale']!r} 2={case['height_scale']!r}"]), b"", [case["x"]], "out"
+    if op == "binaryop_bc":
+        lines, blob = ["Split s 1 2 data a b"], b""
+        if case["small"] == "equal":
+            lines.append("Clip k 1 1 b small 0=0.5 1=3.0")
+        elif case["small"] == "channel":
+            lines.append(mf.pool_line("gap", "b", "small", 1, global_pool=True))
+        else:
+            lines.append(mf.conv_line("Convolution", "c1", "b", "plane" if case["small"] == "image" else "small", 1, 1, 1, 0, False,
+                                      case["wt"].size, 1, act=0))
+            blob = mf.conv_blob_f32(case["wt"], None)
+            if case["small"] == "image":
+                lines.append(mf.pool_line("gap", "plane", "small", 1, global_pool=True))
+        operands = "small a" if case["swap"] else "a small"
+        lines.append(f"BinaryOp e 2 1 {operands} out 0={case['op_type']}")
+        return mf.topology(lines), blob, [case["x"]], "out"
     if op == "clip":
         return mf.topology([f"Clip layer 1 1 data out 0={case['lo']!r} 1={case['hi']!r}"]), b"", [case["x"]], "out"
     if op == "softmax":
@@ -255,6 +292,9 @@ def oracle_eval(case):
         return port.focus(case["x"])
     if op == "interp":
         return port.interp_nearest(case["x"], case["height_scale"], case["width_scale"])
+    if op == "binaryop_bc":
+        small = binaryop_bc_small(case)
+        return port.binaryop(small, case["x"], case["op_type"]) if case["swap"] else port.binaryop(case["x"], small, case["op_type"])
     if op == "clip":
         return port.clip(case["x"], case["lo"], case["hi"])
     if op == "softmax":

@@ -88,6 +88,17 @@ def fixture_cases():
         "reshape_yolo_head": c.unary_case(83, "reshape", (2, 12, 5, 4), new_w=20, new_h=4, new_c=3),
         "reshape_infer_c": c.unary_case(84, "reshape", (1, 6, 4, 5), new_w=10, new_h=3),
         "flatten_axis1": c.unary_case(85, "flatten", (2, 3, 4, 5), axis=1),
+        # BinaryOp beyond the residual add: every op, every operand shape pair of the restatement, both operand orders
+        "binaryop_mul_channel": c.binaryop_bc_case(86, (2, 6, 5, 8), 2, "channel"),
+        "binaryop_sub_channel": c.binaryop_bc_case(87, (2, 6, 5, 7), 1, "channel"),
+        "binaryop_div_channel_swapped": c.binaryop_bc_case(88, (2, 5, 4, 4), 3, "channel", swap=True),
+        "binaryop_sub_equal": c.binaryop_bc_case(89, (2, 4, 5, 7), 1, "equal"),
+        "binaryop_div_equal_swapped": c.binaryop_bc_case(90, (2, 4, 6, 6), 3, "equal", swap=True),
+        "binaryop_mul_equal": c.binaryop_bc_case(91, (1, 3, 5, 5), 2, "equal"),
+        "binaryop_pixel_mul": c.binaryop_bc_case(92, (2, 5, 6, 8), 2, "pixel"),
+        "binaryop_pixel_sub": c.binaryop_bc_case(93, (2, 5, 5, 7), 1, "pixel"),
+        "binaryop_image_add": c.binaryop_bc_case(94, (3, 4, 5, 6), 0, "image"),
+        "binaryop_image_div": c.binaryop_bc_case(95, (3, 4, 4, 4), 3, "image"),
         # transposed convolution (the detection head's 2x2 stride-2 upsampling, and overlapping taps with padding)
         "deconv_2x2s2": c.deconv_case(74, 2, 6, 5, 7, 4, 2, 2),
         "deconv_4x4s2p1": c.deconv_case(75, 1, 5, 6, 6, 3, 4, 2, 1),

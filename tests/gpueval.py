@@ -116,6 +116,20 @@ def gpu_eval(ctx, case):
         return ctx.unary_f32(op, ctx.array(case["x"]), case["alpha"]).download()
     if op == "sigmoid":
         return ctx.unary_f32(op, ctx.array(case["x"])).download()
+    if op == "binaryop_bc":
+        x = ctx.array(case["x"])
+        kind = case["small"]
+        if kind == "equal":
+            small, mode = ctx.unary_f32("clip", x, 0.5, 3.0), 0
+        elif kind == "channel":
+            small, mode = ctx.pool2d_nchw_f32(x, 1, global_pool=True), 2
+        else:
+            small, mode = ctx.array(cases.binaryop_bc_small(dict(case, small="pixel"))), 3  # the 1x1 convolution is not under test
+            if kind == "image":
+                small, mode = ctx.pool2d_nchw_f32(small, 1, global_pool=True), 1
+        if kind == "equal" and case["swap"]:
+            return ctx.binaryop_f32(case["op_type"], 0, small, x).download()
+        return ctx.binaryop_f32(case["op_type"], mode, x, small).download()
     if op == "clip":
         return ctx.unary_f32("clip", ctx.array(case["x"]), case["lo"], case["hi"]).download()
     if op == "softmax":

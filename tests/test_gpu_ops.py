@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(f).startswith("net_"))
-TOLERANT = ("conv_f32", "fc_", "deconv", "softmax")
+TOLERANT = ("conv_f32", "fc_", "deconv", "softmax", "binaryop_pixel", "binaryop_image")
 
 
 @pytest.fixture(scope="module")

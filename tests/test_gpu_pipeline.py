@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(f).startswith("net_"))
-TOLERANT = ("conv_f32", "fc_", "deconv", "softmax")
+TOLERANT = ("conv_f32", "fc_", "deconv", "softmax", "binaryop_pixel", "binaryop_image")
 
 
 def run_case(case, dtype="f32"):
@@ -221,6 +221,39 @@ def test_classifier_tail_flatten_innerproduct_softmax():
         assert cases.check_value(got.reshape(want.shape), want, 1e-4) == 0
         assert np.allclose(got.reshape(3, 7).sum(1), 1.0, atol=1e-6)
         p.close()
+    finally:
+        os.unlink(path)
+
+
+def test_squeeze_and_excite_gate():
+    """The gate of models/angle_cool_best.phai:10-16: Split, global average, 1x1 convolution + ReLU, 1x1 convolution +
+    HardSigmoid, BinaryOp MUL of the [n][c][h][w] tensor with the [n][c][1][1] gate; float32 and fp16."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(81)
+    x = r.uniform(-2, 2, (2, 16, 7, 9)).astype(np.float32)
+    c1 = cases.conv_f32_case(82, 2, 16, 1, 1, 4, 1, 1, 0, act=0)
+    c2 = cases.conv_f32_case(83, 2, 4, 1, 1, 16, 1, 1, 0, act=0)
+    lines = ["Split s 1 2 data a b", mf.pool_line("gap", "b", "g", 1, global_pool=True),
+             mf.conv_line("Convolution", "c1", "g", "g1", 4, 1, 1, 0, True, c1["wt"].size, 1, act=0), "ReLU r 1 1 g1 g2",
+             mf.conv_line("Convolution", "c2", "g2", "g3", 16, 1, 1, 0, True, c2["wt"].size, 1, act=0),
+             "HardSigmoid h 1 1 g3 gate 0=1.666667e-01 1=5.000000e-01", "BinaryOp m 2 1 a gate out 0=2"]
+    g = port.pool2d(x, port.POOL_AVE, global_pool=True)
+    g = port.relu(cases.oracle_eval(dict(c1, x=g)))
+    gate = port.hardsigmoid(cases.oracle_eval(dict(c2, x=g)), 1.666667e-01, 0.5)
+    want = port.binaryop(x, gate, 2)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        f.write(mf.conv_blob_f32(c1["wt"], c1["bias"]) + mf.conv_blob_f32(c2["wt"], c2["bias"]))
+        path = f.name
+    try:
+        p = xp.Pipeline(mf.topology(lines), path, 0)
+        p.forward(x)
+        assert cases.check_value(p.get("gate"), gate, 1e-4) == 0
+        assert cases.check_value(p.get("out"), want, 1e-4) == 0
+        p.close()
+        p16 = xp.Pipeline(mf.topology(lines), path, 0, "f16")
+        p16.forward(x.astype(np.float16).view(np.uint16))
+        assert cases.check_value(p16.get("out").view(np.float16).astype(np.float32), want, 5e-3) == 0
+        p16.close()
     finally:
         os.unlink(path)
 
