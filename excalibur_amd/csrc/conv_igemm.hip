@@ -46,6 +46,8 @@ constexpr int kEpiRowQ = 64 + 16;
 constexpr int kPoolRowB = 32 * 4 + 16;  // pooled epilogue: one tile pixel, 32 float32 channels + padding
 constexpr int kEpiWaveBytes = 32 * kEpiRowF + 32 * kEpiRowQ + 128;
 constexpr size_t kLdsLimit = 158 * 1024;  // dynamic LDS one group may use
+constexpr size_t kLdsThird = 53 * 1024;   // at most this much each and three groups fit a CU's 160 KiB
+constexpr long long kCUs = 256;           // compute units of the MI355X
 constexpr int kSbBytes = 1024;  // LDS kept for per-channel scale and bias of the group's (at most 128) channels
 constexpr unsigned kEpiInvalid = 0x3FFFFF00u;  // element offset whose byte offsets (x1, x4) lie past any accepted tensor
 
@@ -525,7 +527,9 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
         for (int st = 0; st < n_stages; ++st) {
             const bool more = st + 1 < n_stages;
             const bool next_chunk = rg + 1 == p.n_rg;
-            const bool want_a = rg == 0 && a_req_left > 0;
+            // With one tile buffer the next chunk's tile can only be requested once every wave has left this chunk's
+            // last stage (below); with two it is requested during the chunk's first stage.
+            const bool want_a = p.act_bufs > 1 && rg == 0 && a_req_left > 0;
             // The requests go out after the stage's first filter row has been issued: their issue cost then
             // overlaps with MFMAs already in the pipe instead of standing in front of them. The request needed
             // sooner goes first, so that the wait below can leave the other in flight.
@@ -547,6 +551,13 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igem
                 d[9] += t1 - t0;
                 d[10] += t2 - t1;
                 d[11] += t3 - t2;
+            }
+            if (p.act_bufs == 1 && next_chunk && more) {
+                // single tile buffer: refill it now and wait for it in the open; the other groups of the CU (this layout
+                // is chosen where it lets a third one in) run meanwhile
+                request_a();
+                wait_vmcnt(0);
+                __syncthreads();
             }
             after_w[0] = after_w[1];
             w_cur += p.lds_w_b;
@@ -1064,6 +1075,7 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
     static const int force_variant = getenv("EXHIP_FORCE_VARIANT") ? atoi(getenv("EXHIP_FORCE_VARIANT")) : -1;
     static const int force_chunk = getenv("EXHIP_FORCE_CHUNK") ? atoi(getenv("EXHIP_FORCE_CHUNK")) : 0;
     static const int force_rs = getenv("EXHIP_FORCE_RS") ? atoi(getenv("EXHIP_FORCE_RS")) : 0;
+    static const int force_abufs = getenv("EXHIP_FORCE_ABUFS") ? atoi(getenv("EXHIP_FORCE_ABUFS")) : 0;
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
         if (force_variant >= 0 && variant != force_variant) continue;
@@ -1120,6 +1132,8 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
         p.MPH = p.MPW = 0;
         // fills the patch-dependent fields; false when the patch exceeds a staging or LDS limit
         auto shape_patch = [&](int PH, int PW) {
+            const long long wgs = (long long)d->n * ceil_div(pool ? pool->oh : OH, pool ? std::max(1, (PH - 1) / 2) : PH) *
+                                  ceil_div(pool ? pool->ow : OW, pool ? std::max(1, (PW - 1) / 2) : PW) * ktiles;
             p.PH = PH;
             p.PW = PW;
             p.IH = (PH - 1) * p.S + d->kh;
@@ -1157,6 +1171,14 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
                         const size_t with2 = p.lds_bytes();
                         const bool fits3 = with3 <= kLdsLimit;
                         if (fits3 && kLdsLimit / with2 <= kLdsLimit / with3) p.w_bufs = 3;
+                    }
+                    if (p.n_chunks > 1 && p.lds_bytes() > kLdsThird) {
+                        // A single tile buffer if that lets three groups share the CU and the launch has the groups to
+                        // use the room: three per CU must need fewer rounds than two, by more than the 15 % a group
+                        // loses to the tile's load latency, then in the open at every chunk boundary.
+                        const long long r2 = (wgs + 2 * kCUs - 1) / (2 * kCUs), r3 = (wgs + 3 * kCUs - 1) / (3 * kCUs);
+                        p.act_bufs = 1;
+                        if (force_abufs == 2 || p.lds_bytes() > kLdsThird || (force_abufs != 1 && r3 * 115 >= r2 * 100)) p.act_bufs = 2;
                     }
                     if (p.lds_bytes() <= kLdsLimit) return true;
                 }
