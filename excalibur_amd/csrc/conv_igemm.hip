@@ -47,6 +47,7 @@ constexpr int kPoolRowB = 32 * 4 + 16;  // pooled epilogue: one tile pixel, 32 f
 constexpr int kEpiWaveBytes = 32 * kEpiRowF + 32 * kEpiRowQ + 128;
 constexpr size_t kLdsLimit = 158 * 1024;  // dynamic LDS one group may use
 constexpr size_t kLdsThird = 53 * 1024;   // at most this much each and three groups fit a CU's 160 KiB
+constexpr size_t kLdsHalf = 80 * 1024;    // two groups per CU
 constexpr long long kCUs = 256;           // compute units of the MI355X
 constexpr int kSbBytes = 1024;  // LDS kept for per-channel scale and bias of the group's (at most 128) channels
 constexpr unsigned kEpiInvalid = 0x3FFFFF00u;  // element offset whose byte offsets (x1, x4) lie past any accepted tensor
@@ -188,8 +189,9 @@ __device__ __forceinline__ void wait_vmcnt(int keep) {
 
 // KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
 // turns every LDS fragment address of a row into an immediate offset; KWE == 0 keeps them as run-time values.
-template <int DT, int MT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
-__global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : 2)) void conv_igemm_kernel(const ConvParams p) {
+// LOWREG: held to 128 registers (a few spills) so that two 512-thread groups can share a CU.
+template <int DT, int MT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC, bool LOWREG = false>
+__global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2))) void conv_igemm_kernel(const ConvParams p) {
     constexpr int THREADS = 64 * WM * WN;
     constexpr int TM = 32 * MT * WM;
     // staging limits scale with the group size so that a 512-thread group needs half the registers
@@ -1031,6 +1033,7 @@ struct Plan {
     int tiles_x, tiles_y, ktiles;
     int OH, OW;
     int MPH, MPW;  // pooled form: pooled pixels per patch (0 otherwise); the patch is then (2 MPH + 1) x (2 MPW + 1)
+    bool two_per_cu = false;  // a 512-thread plan whose launch counts on two groups per CU (the 128-register kernel)
     size_t staging_bytes() const { return (size_t)act_bufs * lds_act_b + (size_t)w_bufs * lds_w_b; }
     // What the launch asks for: the staging buffers, reused by the epilogue's tiles. epi_wave_b: bytes of LDS
     // each wave's epilogue uses.
@@ -1172,13 +1175,20 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
                         const bool fits3 = with3 <= kLdsLimit;
                         if (fits3 && kLdsLimit / with2 <= kLdsLimit / with3) p.w_bufs = 3;
                     }
-                    if (p.n_chunks > 1 && p.lds_bytes() > kLdsThird) {
+                    const size_t room = p.threads == 512 ? kLdsHalf : kLdsThird;   // 512-thread groups: two per CU at most
+                    const long long per_cu = p.threads == 512 ? 2 : 3;
+                    if (p.n_chunks > 1 && p.lds_bytes() > room) {
                         // A single tile buffer if that lets three groups share the CU and the launch has the groups to
                         // use the room: three per CU must need fewer rounds than two, by more than the 15 % a group
                         // loses to the tile's load latency, then in the open at every chunk boundary.
-                        const long long r2 = (wgs + 2 * kCUs - 1) / (2 * kCUs), r3 = (wgs + 3 * kCUs - 1) / (3 * kCUs);
+                        const long long r2 = (wgs + (per_cu - 1) * kCUs - 1) / ((per_cu - 1) * kCUs), r3 = (wgs + per_cu * kCUs - 1) / (per_cu * kCUs);
+                        const int w_bufs_before = p.w_bufs;
                         p.act_bufs = 1;
-                        if (force_abufs == 2 || p.lds_bytes() > kLdsThird || (force_abufs != 1 && r3 * 115 >= r2 * 100)) p.act_bufs = 2;
+                        if (p.lds_bytes() > room && p.w_bufs == 3) p.w_bufs = 2;
+                        if (force_abufs == 2 || p.lds_bytes() > room || (force_abufs != 1 && r3 * 115 >= r2 * 100)) {
+                            p.act_bufs = 2;
+                            p.w_bufs = w_bufs_before;
+                        }
                     }
                     if (p.lds_bytes() <= kLdsLimit) return true;
                 }
@@ -1263,6 +1273,12 @@ int launch_kernel(exhip_ctx* ctx, K kernel, bool* attr_set, const Plan& pl, cons
 
 template <int DT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC>
 int launch_inst(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
+    if constexpr (WM * WN == 8 && !PACKED && EPI == 1 && KWE == 3) {
+        if (pl.two_per_cu) {
+            static bool attr_low = false;
+            return launch_kernel(ctx, conv_igemm_kernel<DT, 2, NT, WM, WN, PACKED, EPI, KWE, KSC, true>, &attr_low, pl, p, grid);
+        }
+    }
     static bool attr = false;
     return launch_kernel(ctx, conv_igemm_kernel<DT, 2, NT, WM, WN, PACKED, EPI, KWE, KSC>, &attr, pl, p, grid);
 }
@@ -1276,6 +1292,7 @@ int launch_shape(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) 
         return launch_inst<DT, NT, WM, WN, true, EPI, 1, 1>(ctx, pl, p, grid);
     } else {
         if (pl.KWe == 3 && pl.KS == 2) return launch_inst<DT, NT, WM, WN, false, EPI, 3, 2>(ctx, pl, p, grid);
+        if (pl.KWe == 3 && pl.KS == 1) return launch_inst<DT, NT, WM, WN, false, EPI, 3, 1>(ctx, pl, p, grid);
         if (pl.KWe == 1 && pl.KS == 2) return launch_inst<DT, NT, WM, WN, false, EPI, 1, 2>(ctx, pl, p, grid);
         return launch_inst<DT, NT, WM, WN, false, EPI, 0, 0>(ctx, pl, p, grid);
     }
@@ -1290,12 +1307,47 @@ int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid
     }
 }
 
+// The plan assumes the largest epilogue so that the weight packing does not depend on a call's outputs; the number of
+// staging buffers does not enter the packing, so a launch that knows its epilogue's LDS may trade the second tile
+// buffer (and the third weight buffer) for one more group per CU, under make_plan's rule: the extra group must save
+// more rounds than the exposed tile loads cost. `fused_3x3`: the launch runs the fused int8 epilogue on a 3-tap row
+// shape, the instantiations whose 512-thread form is held to 128 registers and so may run two groups per CU.
+void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3) {
+    static const int force_abufs = getenv("EXHIP_FORCE_ABUFS") ? atoi(getenv("EXHIP_FORCE_ABUFS")) : 0;
+    if (pl.packed || pl.MPH || pl.n_chunks < 2 || pl.act_bufs == 1 || force_abufs == 2) return;
+    const long long cap = pl.threads == 512 ? (fused_3x3 ? 2 : 1) : 3;
+    auto groups = [&](const Plan& q) {
+        const long long g = (long long)(160 * 1024 / q.launch_lds_bytes(epi_wave_b));
+        return std::max(1ll, std::min(g, cap));
+    };
+    Plan one = pl;
+    one.act_bufs = 1;
+    if (groups(one) <= groups(pl) && one.w_bufs == 3) one.w_bufs = 2;
+    const long long g_now = groups(pl), g_one = groups(one);
+    if (g_one <= g_now) return;
+    const long long wgs = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
+    const long long r_now = (wgs + g_now * kCUs - 1) / (g_now * kCUs), r_one = (wgs + g_one * kCUs - 1) / (g_one * kCUs);
+    if (force_abufs == 1 || r_one * 115 < r_now * 100) {
+        pl = one;
+        pl.two_per_cu = pl.threads == 512;
+    }
+}
+
 template <int DT>
 int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolSpec* pool = nullptr) {
     EXHIP_REQUIRE(ctx, "conv: NULL ctx");
     Plan pl;
     int rc = make_plan(d, DT, &pl, pool);
     if (rc) return rc;
+    if constexpr (DT == EXHIP_I8) {
+        if (!pool) {
+            const long long elems = (long long)d->n * pl.OH * pl.OW * d->k;
+            const bool fused = !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 && elems * 4 < 0xFFFFF000ll &&
+                               elems < (long long)kEpiInvalid;
+            const int epi_wave_b = !fused ? 0 : ((p.residual || p.y_nhwc) ? kEpiWaveBytes : 32 * kEpiRowQ + 128);
+            rebuffer(pl, d, epi_wave_b, fused && pl.KWe == 3);
+        }
+    }
     EXHIP_REQUIRE(p.x && p.wp, "conv: NULL input or weights");
     EXHIP_REQUIRE(d->k_stride >= d->k || (!p.y_q && !p.y_nhwc && !p.residual), "conv: k_stride %d < k %d", d->k_stride, d->k);
     EXHIP_REQUIRE(!(p.y_q) || d->k_stride % 16 == 0, "conv: NHWC int8/half output needs k_stride %% 16 == 0");
