@@ -1078,7 +1078,8 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
     static const int force_variant = getenv("EXHIP_FORCE_VARIANT") ? atoi(getenv("EXHIP_FORCE_VARIANT")) : -1;
     static const int force_chunk = getenv("EXHIP_FORCE_CHUNK") ? atoi(getenv("EXHIP_FORCE_CHUNK")) : 0;
     static const int force_rs = getenv("EXHIP_FORCE_RS") ? atoi(getenv("EXHIP_FORCE_RS")) : 0;
-    static const int force_abufs = getenv("EXHIP_FORCE_ABUFS") ? atoi(getenv("EXHIP_FORCE_ABUFS")) : 0;
+    const char* const abufs_env = getenv("EXHIP_FORCE_ABUFS");  // read per call: tests switch it inside one process
+    const int force_abufs = abufs_env ? atoi(abufs_env) : 0;
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
         if (force_variant >= 0 && variant != force_variant) continue;
@@ -1313,7 +1314,8 @@ int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid
 // more rounds than the exposed tile loads cost. `fused_3x3`: the launch runs the fused int8 epilogue on a 3-tap row
 // shape, the instantiations whose 512-thread form is held to 128 registers and so may run two groups per CU.
 void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3) {
-    static const int force_abufs = getenv("EXHIP_FORCE_ABUFS") ? atoi(getenv("EXHIP_FORCE_ABUFS")) : 0;
+    const char* const abufs_env = getenv("EXHIP_FORCE_ABUFS");  // read per call: tests switch it inside one process
+    const int force_abufs = abufs_env ? atoi(abufs_env) : 0;
     if (pl.packed || pl.MPH || pl.n_chunks < 2 || pl.act_bufs == 1 || force_abufs == 2) return;
     const long long cap = pl.threads == 512 ? (fused_3x3 ? 2 : 1) : 3;
     auto groups = [&](const Plan& q) {
@@ -1330,6 +1332,10 @@ void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3
     if (force_abufs == 1 || r_one * 115 < r_now * 100) {
         pl = one;
         pl.two_per_cu = pl.threads == 512;
+        static const bool show = getenv("EXHIP_DEBUG_PLAN") != nullptr;
+        if (show)
+            fprintf(stderr, "  launch: act x%d w x%d, %lld groups per CU instead of %lld (%lld groups, LDS %zu)\n", pl.act_bufs, pl.w_bufs,
+                    g_one, g_now, wgs, pl.launch_lds_bytes(epi_wave_b));
     }
 }
 

@@ -97,6 +97,39 @@ def test_conv_i8_fused_residual_relu_requant(ctx):
     assert np.array_equal(got["i8"], want_q.transpose(0, 2, 3, 1))
 
 
+ONE_BUFFER_SHAPES = [
+    # seed, n, c, h, w, k, kernel, stride, pad
+    (225, 2, 128, 40, 40, 128, 3, 1, 1),   # two 64-byte chunks, three groups per CU
+    (226, 1, 256, 24, 20, 64, 3, 1, 1),    # four chunks
+    (227, 2, 128, 41, 39, 256, 3, 2, 1),   # strided: the 512-thread variant in its 128-register form, four 32-byte chunks
+    (228, 2, 128, 24, 24, 128, 1, 1, 0),   # 1x1
+]
+
+
+@pytest.mark.parametrize("args", ONE_BUFFER_SHAPES, ids=[f"s{a[0]}" for a in ONE_BUFFER_SHAPES])
+def test_conv_i8_single_tile_buffer_bit_exact(ctx, args, monkeypatch):
+    """The planner trades the second activation tile buffer for one more workgroup per CU only on launches large enough
+    to gain from it; EXHIP_FORCE_ABUFS=1 (read per call) makes these small launches take that path: fused int8 and
+    float32 outputs with a shortcut, and the plain NCHW output, all bit-exact."""
+    monkeypatch.setenv("EXHIP_FORCE_ABUFS", "1")
+    case = cases.conv_i8_case(*args, act=0)
+    g = cases.geom_of(case)
+    want_y, want_acc = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], case["act"], g, want_acc=True)
+    got = gpueval.conv_i8(ctx, case)
+    assert np.array_equal(got["acc"], want_acc)
+    assert np.array_equal(got["nchw"], want_y)
+    r = np.random.default_rng(args[0] + 1000)
+    res_nchw = r.uniform(-4, 4, want_y.shape).astype(np.float32)
+    fs_out = np.float32(11.7)
+    z = port.relu(port.binaryop_add(want_y, res_nchw))
+    fused = gpueval.conv_i8(ctx, case, fs_out=fs_out, residual=np.ascontiguousarray(res_nchw.transpose(0, 2, 3, 1)), post_relu=1,
+                            want=("nhwc",))
+    assert np.array_equal(fused["nhwc"], z.transpose(0, 2, 3, 1))
+    assert np.array_equal(fused["i8"], port.quantize(z, fs_out).transpose(0, 2, 3, 1))
+    q_only = gpueval.conv_i8(ctx, dict(case, act=1), fs_out=fs_out, want=())
+    assert np.array_equal(q_only["i8"], port.quantize(port.relu(want_y), fs_out).transpose(0, 2, 3, 1))
+
+
 def test_conv_i8_requant_pad_channels_are_zero(ctx):
     case = cases.conv_i8_case(222, 1, 32, 12, 12, 40, 3, 1, 1)
     fs_out = np.float32(9.0)
