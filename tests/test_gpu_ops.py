@@ -1,6 +1,6 @@
 """GPU parity tests: every operator of the hot path through the exhip C ABI against
 (1) the golden fixtures written by the compiled reference, (2) the CPU restatement on larger seeded
-shapes, (3) size-independent properties at the BASELINE sizes.
+shapes, (3) size-independent properties at the benchmark sizes.
 
 Bars: int32 accumulators, dequantized outputs of the int8 path, requantized int8 outputs, depthwise,
 pooling and elementwise results bit-exact (== on floats, so +0.0 equals -0.0); fp32 convolution and
@@ -380,7 +380,7 @@ FULL = [
 
 @pytest.mark.parametrize("name,args", FULL, ids=[f[0] for f in FULL])
 def test_full_size_sampled_and_linear(ctx, name, args):
-    """At BASELINE sizes: (a) sampled accumulators against brute force, (b) linearity in the weights:
+    """At the benchmark sizes: (a) sampled accumulators against brute force, (b) linearity in the weights:
     acc(w1) + acc(w2) == acc(w1 + w2), (c) the dequantized output recomputed from the GPU's own
     accumulators with the closed form fmaf(acc, s, b) + ReLU."""
     case = cases.conv_i8_case(*args, integer_x=True)

@@ -9,7 +9,7 @@ from excalibur_amd.resnet18 import ResNet18Int8
 from tests import cases, netref
 
 
-def test_algorithmic_work_matches_the_survey_figure():
+def test_algorithmic_work_of_the_benchmark_network():
     net = ResNet18Int8(seed=3, calib_hw=32)
     # 14.80 GMAC per 640x640 image: stem 0.963 + stage1 4x0.944 + three stages of (0.472 + 0.052 + 3x0.944)
     assert abs(net.gmac_per_image(640, 640) - 14.805) < 0.01
