@@ -665,6 +665,44 @@ __global__ __launch_bounds__(kBlock) void pool_s2_nchw_f32_strip_kernel(const fl
     }
 }
 
+// Stride-1 max pooling with an odd window and "same" padding (the 5 / 9 / 13 pyramid of the detection topologies):
+// the maximum is separable, so a workgroup stages a 32 x 32 output tile's halo in LDS, takes row maxima into a second
+// LDS array and column maxima of those into the output: 2K compares per output instead of K * K. Cells outside the
+// image hold -FLT_MAX, the clipped window's identity.
+template <int K>
+__global__ __launch_bounds__(kBlock) void maxpool_same_nchw_f32_kernel(const float* __restrict__ x, float* __restrict__ y, int H,
+                                                                       int W) {
+    constexpr int P = K / 2, T = 32, S = T + 2 * P;
+    __shared__ float in[S][S + 1];
+    __shared__ float rowmax[S][T + 1];
+    const size_t plane = blockIdx.z;
+    const int x0 = blockIdx.x * T, y0 = blockIdx.y * T;
+    const float* src = x + plane * H * W;
+    for (int i = threadIdx.x; i < S * S; i += kBlock) {
+        const int r = i / S, c = i - r * S;
+        const int gy = y0 - P + r, gx = x0 - P + c;
+        in[r][c] = (gy >= 0 && gy < H && gx >= 0 && gx < W) ? src[(size_t)gy * W + gx] : -FLT_MAX;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < S * T; i += kBlock) {
+        const int r = i / T, c = i - r * T;
+        float m = in[r][c];
+#pragma unroll
+        for (int k = 1; k < K; ++k) m = m < in[r][c + k] ? in[r][c + k] : m;
+        rowmax[r][c] = m;
+    }
+    __syncthreads();
+    float* dst = y + plane * H * W;
+    for (int i = threadIdx.x; i < T * T; i += kBlock) {
+        const int r = i / T, c = i - r * T;
+        if (y0 + r >= H || x0 + c >= W) continue;
+        float m = rowmax[r][c];
+#pragma unroll
+        for (int k = 1; k < K; ++k) m = m < rowmax[r + k][c] ? rowmax[r + k][c] : m;
+        dst[(size_t)(y0 + r) * W + x0 + c] = m;
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void maxpool_nhwc_f32_kernel(const float* __restrict__ x, float* __restrict__ y,
                                                                   int8_t* __restrict__ yq, float fs_out, int H, int W, int cs,
                                                                   int OH, int OW, int kh, int kw, int sh, int sw, int pt,
@@ -1501,6 +1539,16 @@ extern "C" int exhip_pool2d_nchw_f32(exhip_ctx* ctx, const float* x, float* y, i
     REQ_CTX("exhip_pool2d_nchw_f32");
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && oh > 0 && ow > 0 && kh > 0 && kw > 0, "exhip_pool2d_nchw_f32: bad argument");
     EXHIP_REQUIRE(type == 0 || type == 1, "exhip_pool2d_nchw_f32: unknown pooling type %d", type);
+    const bool same_window = type == 0 && kh == kw && (kh == 5 || kh == 9 || kh == 13) && sh == 1 && sw == 1 && pt == kh / 2 &&
+                             pb == kh / 2 && pl == kh / 2 && pr == kh / 2 && oh == h && ow == w && (long long)n * c <= 65535;
+    if (same_window) {
+        const dim3 grid((w + 31) / 32, (h + 31) / 32, n * c);
+        if (kh == 5) hipLaunchKernelGGL((maxpool_same_nchw_f32_kernel<5>), grid, dim3(kBlock), 0, ctx->stream, x, y, h, w);
+        else if (kh == 9) hipLaunchKernelGGL((maxpool_same_nchw_f32_kernel<9>), grid, dim3(kBlock), 0, ctx->stream, x, y, h, w);
+        else hipLaunchKernelGGL((maxpool_same_nchw_f32_kernel<13>), grid, dim3(kBlock), 0, ctx->stream, x, y, h, w);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const bool strip_window = kh == kw && (kh == 2 || kh == 3) && sh == 2 && sw == 2 && pl >= 0 && pl <= 1 && pt >= 0 &&
                               w % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     if (strip_window) {
