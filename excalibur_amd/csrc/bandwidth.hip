@@ -969,6 +969,53 @@ __global__ __launch_bounds__(kBlock) void unary_f32_kernel(const float* __restri
     }
 }
 
+// The same on half storage: widened to float, the float formula, rounded to half once (what the reference's fp16 layers
+// do through their convert-and-call wrapper). Eight values per thread over the aligned body.
+template <int OP>
+__global__ __launch_bounds__(kBlock) void unary_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y, size_t n8,
+                                                           size_t count, float alpha, float beta) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n8) {
+        v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(x)[i]), v8f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = unary_value<OP>(v[e], alpha, beta);
+        reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
+    } else {
+        const size_t j = n8 * 8 + (i - n8);
+        if (j < count) y[j] = exhip_f2h(unary_value<OP>(exhip_h2f(x[j]), alpha, beta));
+    }
+}
+
+template <int OP>
+__device__ __forceinline__ float channel_value(float v, float a, float b) {
+    if constexpr (OP == 0) return v >= 0.f ? v : a * v;
+    else if constexpr (OP == 1) return __builtin_fmaf(b, v, a);
+    else return (v - a) * b;
+}
+
+// Per-channel layers on NCHW half storage, one block row per (image, channel) plane, eight values per thread where the
+// plane is a multiple of eight halves long.
+template <int OP, int VEC>
+__global__ __launch_bounds__(kBlock) void channelwise_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int C,
+                                                                 int HW, const float* __restrict__ p0,
+                                                                 const float* __restrict__ p1, int shared) {
+    const int plane = blockIdx.y;
+    const int c = plane % C;
+    const float a = p0[shared ? 0 : c];
+    const float b = p1 ? p1[c] : 0.f;
+    const size_t base = (size_t)plane * HW;
+    for (int j = (blockIdx.x * kBlock + threadIdx.x) * VEC; j < HW; j += gridDim.x * kBlock * VEC) {
+        if constexpr (VEC == 8) {
+            v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(x + base + j)), v8f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = channel_value<OP>(v[e], a, b);
+            *reinterpret_cast<v4i*>(y + base + j) = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
+        } else {
+            y[base + j] = exhip_f2h(channel_value<OP>(exhip_h2f(x[base + j]), a, b));
+        }
+    }
+}
+
 // Per-channel layers on NCHW. OP 0 PReLU (p0 = slope, one per channel or one shared), 1 BatchNorm as
 // fma(p1[c], x, p0[c]) with the load-time a / b, 2 Input (x - p0[c]) * p1[c]. One block row per (image, channel) plane.
 template <int OP>
@@ -1725,6 +1772,57 @@ extern "C" int exhip_unary_f32(exhip_ctx* ctx, int op, const float* x, float* y,
     case EXHIP_UNARY_CLIP: return launch_unary<4>(ctx, x, y, count, alpha, beta);
     default: exhip_set_error("exhip_unary_f32: unknown op %d", op); return EXHIP_ERR_ARG;
     }
+}
+
+template <int OP>
+static int launch_unary_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, size_t count, float alpha, float beta) {
+    if (!count) return 0;
+    const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)y % 16 == 0);
+    const size_t n8 = aligned ? count / 8 : 0;
+    const size_t threads = n8 + (count - n8 * 8);
+    hipLaunchKernelGGL((unary_f16_kernel<OP>), dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, x, y, n8, count, alpha, beta);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_unary_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, size_t count, float alpha, float beta) {
+    REQ_CTX("exhip_unary_f16");
+    EXHIP_REQUIRE((x && y) || !count, "exhip_unary_f16: NULL tensor");
+    switch (op) {
+    case EXHIP_UNARY_HARDSWISH: return launch_unary_f16<0>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_LEAKYRELU: return launch_unary_f16<1>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_SIGMOID: return launch_unary_f16<2>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_HARDSIGMOID: return launch_unary_f16<3>(ctx, x, y, count, alpha, beta);
+    case EXHIP_UNARY_CLIP: return launch_unary_f16<4>(ctx, x, y, count, alpha, beta);
+    default: exhip_set_error("exhip_unary_f16: unknown op %d", op); return EXHIP_ERR_ARG;
+    }
+}
+
+template <int OP>
+static void launch_channelwise_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int hw, const float* p0,
+                                   const float* p1, int shared) {
+    const bool vec = hw % 8 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0;
+    unsigned bx = blocks_for((size_t)(vec ? hw / 8 : hw));
+    if (bx > 64) bx = 64;
+    const dim3 grid(bx, (unsigned)(n * c));
+    if (vec) hipLaunchKernelGGL((channelwise_f16_kernel<OP, 8>), grid, dim3(kBlock), 0, ctx->stream, x, y, c, hw, p0, p1, shared);
+    else hipLaunchKernelGGL((channelwise_f16_kernel<OP, 1>), grid, dim3(kBlock), 0, ctx->stream, x, y, c, hw, p0, p1, shared);
+}
+
+extern "C" int exhip_channelwise_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, int n, int c, int hw, const float* p0,
+                                     const float* p1, int shared) {
+    REQ_CTX("exhip_channelwise_f16");
+    EXHIP_REQUIRE(x && y && p0 && n > 0 && c > 0 && hw > 0, "exhip_channelwise_f16: bad argument");
+    EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || p1, "exhip_channelwise_f16: this op needs two parameter arrays");
+    EXHIP_REQUIRE((long long)n * c <= 65535, "exhip_channelwise_f16: more than 65535 (image, channel) planes");
+    switch (op) {
+    case EXHIP_CHANNEL_PRELU: launch_channelwise_f16<0>(ctx, x, y, n, c, hw, p0, p1, shared); break;
+    case EXHIP_CHANNEL_BATCHNORM: launch_channelwise_f16<1>(ctx, x, y, n, c, hw, p0, p1, 0); break;
+    case EXHIP_CHANNEL_INPUT: launch_channelwise_f16<2>(ctx, x, y, n, c, hw, p0, p1, 0); break;
+    default: exhip_set_error("exhip_channelwise_f16: unknown op %d", op); return EXHIP_ERR_ARG;
+    }
+    EXHIP_LAUNCH_CHECK();
+    return 0;
 }
 
 extern "C" int exhip_channelwise_f32(exhip_ctx* ctx, int op, const float* x, float* y, int n, int c, int hw, const float* p0,

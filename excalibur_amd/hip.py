@@ -324,6 +324,18 @@ class Ctx:
         _check(lib().exhip_channelwise_f32(self.h, self.CHANNEL[op], x.ptr, y.ptr, n, c, h * w, p0.ptr, _ptr(p1), int(shared)))
         return y
 
+    def unary_f16(self, op, x, alpha=0.0, beta=0.0):
+        y = self.empty(x.shape, np.uint16)
+        _check(lib().exhip_unary_f16(self.h, self.UNARY[op], x.ptr, y.ptr, ctypes.c_size_t(y.size), ctypes.c_float(float(alpha)),
+                                     ctypes.c_float(float(beta))))
+        return y
+
+    def channelwise_f16(self, op, x, p0, p1=None, shared=False):
+        n, c, h, w = x.shape
+        y = self.empty(x.shape, np.uint16)
+        _check(lib().exhip_channelwise_f16(self.h, self.CHANNEL[op], x.ptr, y.ptr, n, c, h * w, p0.ptr, _ptr(p1), int(shared)))
+        return y
+
     def concat_channels_f32(self, inputs):
         n, _, h, w = inputs[0].shape
         ptrs = (ctypes.c_void_p * len(inputs))(*[a.ptr.value for a in inputs])

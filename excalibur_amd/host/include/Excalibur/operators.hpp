@@ -205,6 +205,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 template <typename Dtype>
 struct operation_hardswish : operation_unary<Dtype> {
@@ -244,6 +245,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 
 // src/Excalibur/operation_batchnorm.cpp:10-156: keys 0 = channels, 1 = eps; blob = slope, mean, var, bias;
@@ -263,6 +265,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
     void fold();
 };
 

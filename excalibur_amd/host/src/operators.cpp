@@ -590,6 +590,13 @@ void operation_eltwise<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>
     CHECK_GE(bottoms.size(), 2);
     CHECK_EQ(tops.size(), 1);
     const int dev = this->params_.device_;
+    if (type_ == 1 && bottoms.size() == 2 && coeffs_[0] == 1.f && coeffs_[1] == 1.f) {  // the residual add, in one pass
+        CHECK(bottoms[1]->data_shape() == bottoms[0]->data_shape());
+        tops[0] = std::make_shared<tensor<unsigned short>>(bottoms[0]->data_shape(), dev, bottoms[0]->order());
+        EXHIP_FATAL(exhip_add_f16(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(),
+                                  tops[0]->count(), 0));
+        return;
+    }
     tensor_list<float> f(bottoms.size());
     std::vector<const float*> in;
     for (size_t i = 0; i < bottoms.size(); ++i) {
@@ -890,6 +897,15 @@ void operation_unary<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, 
 }
 
 template <typename Dtype>
+void operation_unary<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        tops[i] = std::make_shared<tensor<unsigned short>>(bottoms[i]->data_shape(), this->params_.device_, bottoms[i]->order());
+        EXHIP_FATAL(exhip_unary_f16(this->ctx(), op_, bottoms[i]->gpu_data(), tops[i]->mutable_gpu_data(), tops[i]->count(), alpha_, beta_));
+    }
+}
+
+template <typename Dtype>
 operation_prelu<Dtype>::operation_prelu(const operation_param& param) : operation<Dtype>(param) {
     for (const layer_attr& a : parse_attrs(param.specific_params_)) {
         const int key = std::atoi(a.key.c_str());
@@ -929,6 +945,19 @@ void operation_prelu<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, 
         if (!share_channel_) CHECK_EQ(b->channels(), num_slope_);
         tops[i] = std::make_shared<tensor<float>>(b->data_shape(), this->params_.device_, b->order());
         EXHIP_FATAL(exhip_channelwise_f32(this->ctx(), EXHIP_CHANNEL_PRELU, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(), b->channels(),
+                                          b->height() * b->width(), this->weights_f32_[0]->gpu_data(), nullptr, share_channel_ ? 1 : 0));
+    }
+}
+
+template <typename Dtype>
+void operation_prelu<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        const auto& b = bottoms[i];
+        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+        if (!share_channel_) CHECK_EQ(b->channels(), num_slope_);
+        tops[i] = std::make_shared<tensor<unsigned short>>(b->data_shape(), this->params_.device_, b->order());
+        EXHIP_FATAL(exhip_channelwise_f16(this->ctx(), EXHIP_CHANNEL_PRELU, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(), b->channels(),
                                           b->height() * b->width(), this->weights_f32_[0]->gpu_data(), nullptr, share_channel_ ? 1 : 0));
     }
 }
@@ -995,6 +1024,19 @@ void operation_batchnorm<Dtype>::forward_gpu_f32(const tensor_list<float>& botto
         CHECK_EQ(b->channels(), channels_);
         tops[i] = std::make_shared<tensor<float>>(b->data_shape(), this->params_.device_, b->order());
         EXHIP_FATAL(exhip_channelwise_f32(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(),
+                                          b->channels(), b->height() * b->width(), a_->gpu_data(), b_->gpu_data(), 0));
+    }
+}
+
+template <typename Dtype>
+void operation_batchnorm<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        const auto& b = bottoms[i];
+        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
+        CHECK_EQ(b->channels(), channels_);
+        tops[i] = std::make_shared<tensor<unsigned short>>(b->data_shape(), this->params_.device_, b->order());
+        EXHIP_FATAL(exhip_channelwise_f16(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(),
                                           b->channels(), b->height() * b->width(), a_->gpu_data(), b_->gpu_data(), 0));
     }
 }

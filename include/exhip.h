@@ -198,6 +198,9 @@ int exhip_binaryop_f32(exhip_ctx* ctx, int op, int mode, const float* large, con
 #define EXHIP_UNARY_HARDSIGMOID 3
 #define EXHIP_UNARY_CLIP 4 /* max(alpha, min(beta, x)), src/Excalibur/operation_clip.cpp:32-58 */
 int exhip_unary_f32(exhip_ctx* ctx, int op, const float* x, float* y, size_t count, float alpha, float beta);
+/* The same on half storage: the reference's fp16 layer is float2half(op(half2float(x))) (include/Excalibur/operation.hpp:204-266);
+ * here in one pass, rounding to nearest even. */
+int exhip_unary_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, size_t count, float alpha, float beta);
 /* Per-channel layers on NCHW float tensors: PReLU, p0 = slope[c] or one shared slope (operation_prelu.cpp:57-124);
  * BatchNorm as fma(p1[c], x, p0[c]) with a = p0, b = p1 computed at load time (operation_batchnorm.cpp:52-64,122-156);
  * Input (x - p0[c]) * p1[c] (operation_input.cpp:61-151). p0 / p1: device arrays of c floats. */
@@ -205,6 +208,9 @@ int exhip_unary_f32(exhip_ctx* ctx, int op, const float* x, float* y, size_t cou
 #define EXHIP_CHANNEL_BATCHNORM 1
 #define EXHIP_CHANNEL_INPUT 2
 int exhip_channelwise_f32(exhip_ctx* ctx, int op, const float* x, float* y, int n, int c, int hw, const float* p0,
+                          const float* p1, int shared);
+/* The same on half storage (float parameters and arithmetic, one rounding to half). */
+int exhip_channelwise_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, int n, int c, int hw, const float* p0,
                           const float* p1, int shared);
 /* operation_concat::forward_cpu_f32 along the channel axis (operation_concat.cpp:31-103): inputs is a host array of
  * device pointers to NCHW tensors [n][channels[i]][hw]. */

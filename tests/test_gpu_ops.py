@@ -320,6 +320,51 @@ def test_pool_nhwc_f16(ctx):
     assert np.array_equal(got, port.pool2d(x16.astype(np.float32), port.POOL_MAX, 3, 2, 1))
 
 
+def _half(a):
+    """Round-to-nearest-even to half storage, widened again (what a tensor of the fp16 path holds)."""
+    return a.astype(np.float16)
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 20, 24), (1, 3, 5, 7), (1, 1, 1, 1)])
+@pytest.mark.parametrize("kind,params", [("hardswish", dict(alpha=1 / 6, beta=0.5)), ("leakyrelu", dict(alpha=0.1)), ("sigmoid", {}),
+                                         ("hardsigmoid", dict(alpha=0.2, beta=0.5))])
+def test_unary_half_storage_bit_exact(ctx, kind, params, shape):
+    """The fp16 activation layers in one pass: half in, the float formula, one rounding to half out."""
+    case = cases.unary_case(325, kind, shape, **params)
+    x16 = _half(case["x"])
+    want = _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32))))
+    got = ctx.unary_f16(kind, ctx.array(x16.view(np.uint16)), params.get("alpha", 0.0), params.get("beta", 0.0)).download()
+    assert np.array_equal(got, want.view(np.uint16))
+
+
+def test_clip_half_storage_bit_exact(ctx):
+    x16 = _half(np.random.default_rng(326).uniform(-4, 4, (2, 5, 9, 11)).astype(np.float32))
+    got = ctx.unary_f16("clip", ctx.array(x16.view(np.uint16)), 0.5, 3.0).download()
+    assert np.array_equal(got, _half(port.clip(x16.astype(np.float32), 0.5, 3.0)).view(np.uint16))
+
+
+@pytest.mark.parametrize("shape", [(2, 16, 20, 24), (2, 5, 7, 9), (1, 3, 1, 1)])
+def test_channelwise_half_storage_bit_exact(ctx, shape):
+    """PReLU (per-channel and shared slope), BatchNorm and Input on half storage with float parameters."""
+    for shared in (False, True):
+        case = cases.prelu_case(327, shape, shared)
+        x16 = _half(case["x"])
+        got = ctx.channelwise_f16("prelu", ctx.array(x16.view(np.uint16)), ctx.array(case["slope"]), shared=shared).download()
+        assert np.array_equal(got, _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.uint16))
+    case = cases.batchnorm_case(328, shape)
+    x16 = _half(case["x"])
+    sqrt_var = np.sqrt((case["var"] + np.float32(case["eps"])).astype(np.float64)).astype(np.float32)
+    a = (case["bias"] - case["slope"] * case["mean"] / sqrt_var).astype(np.float32)
+    b = (case["slope"] / sqrt_var).astype(np.float32)
+    got = ctx.channelwise_f16("batchnorm", ctx.array(x16.view(np.uint16)), ctx.array(a), ctx.array(b)).download()
+    assert np.array_equal(got, _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.uint16))
+    case = cases.input_case(329, (shape[0], 3) + shape[2:], [127.5, 120.0, 110.25], [1 / 128.0, 0.017, 0.0175])
+    x16 = _half(case["x"])
+    got = ctx.channelwise_f16("input", ctx.array(x16.view(np.uint16)), ctx.array(np.asarray(case["means"], np.float32)),
+                              ctx.array(np.asarray(case["scales"], np.float32))).download()
+    assert np.array_equal(got, _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.uint16))
+
+
 @pytest.mark.parametrize("etype,n,coeffs", [(1, 2, None), (1, 3, [0.5, -1.25, 2.0]), (2, 3, None), (0, 3, None)])
 def test_eltwise_bit_exact(ctx, etype, n, coeffs):
     case = cases.eltwise_case(320 + etype, (2, 16, 21, 23), etype, n, coeffs)
