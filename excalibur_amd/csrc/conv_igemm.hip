@@ -452,6 +452,13 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
             float v = 0.f;
             if (ch < p.K) v = tid < TM ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
             lds_sb[(tid < TM ? 0 : 128) + c] = v;
+            if constexpr (EPI == 2) {
+                // pooled form: does any channel have a negative scale? (wave 0 holds all 64 scales; slot 64 is spare)
+                if (tid < TM) {
+                    const unsigned long long neg = __ballot(__builtin_bit_cast(int, v) < 0);
+                    if (tid == 0) reinterpret_cast<int*>(lds_sb)[64] = neg != 0ull;
+                }
+            }
         }
     }
 
@@ -826,12 +833,34 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_nhwc, 0, (int)(out_px * (unsigned)p.K * 4u), kRsrcWord3);
         const bool has_f = p.y_nhwc != nullptr, has_q = p.y_q != nullptr;
         const int items = p.MPH * p.MPW * 8;  // 4-channel vectors of the pooled patch, per 32-channel block
+        // With a scale >= 0 the dequantization fmaf((float)acc, scale, bias) and the ReLU are non-decreasing in acc, so the
+        // maximum can be taken on the int32 accumulators and only the pooled pixels are dequantized: the same values
+        // (the float of the largest accumulator is the largest float), a quarter of the conversions. The tile then
+        // holds int32 and INT_MIN marks pixels outside the convolution's output. Any negative scale (never the case
+        // for scales made as 1 / (ws * fs), but allowed) selects the float form.
+        const bool int_pool = reinterpret_cast<const int*>(lds_sb)[64] == 0;  // written before the stage loop's barriers
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             if (m > 0) __syncthreads();  // the previous block's tile has been read
 #pragma unroll
             for (int nn = 0; nn < NT; ++nn) {
                 const int pp = (wn * NT + nn) * 32 + px_l;
+                if (int_pool) {
+                    if (pp < npatch) {
+                        char* const dst = pool + pp * kPoolRowB + hh * 64;
+                        if ((pvalid >> nn) & 1) {
+#pragma unroll
+                            for (int e4 = 0; e4 < 4; ++e4)
+                                *reinterpret_cast<v4i*>(dst + e4 * 16) =
+                                    v4i{acc[m][nn][e4 * 4], acc[m][nn][e4 * 4 + 1], acc[m][nn][e4 * 4 + 2], acc[m][nn][e4 * 4 + 3]};
+                        } else {
+                            const int lowest = (int)0x80000000;
+#pragma unroll
+                            for (int e4 = 0; e4 < 4; ++e4) *reinterpret_cast<v4i*>(dst + e4 * 16) = v4i{lowest, lowest, lowest, lowest};
+                        }
+                    }
+                    continue;
+                }
                 // median(v, lo, hi): a valid pixel gets max(v, 0) with ReLU (lo = 0, hi = +inf) or v without
                 // (lo = -inf); a pixel outside the convolution's output gets -inf (lo = hi = -inf)
                 const bool valid = (pvalid >> nn) & 1;
@@ -855,16 +884,35 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 const int pyy = fast_div(pq, p.magic_mpw), pxx = pq - pyy * p.MPW;
                 const int gy = ty * p.MPH + pyy, gx = tx * p.MPW + pxx;
                 const char* w0 = pool + ((2 * pyy) * p.PW + 2 * pxx) * kPoolRowB + part * 16;
-                v4f best = *reinterpret_cast<const v4f*>(w0);
+                v4f best;
+                if (int_pool) {
+                    v4i top = *reinterpret_cast<const v4i*>(w0);
 #pragma unroll
-                for (int dr = 0; dr < 3; ++dr)
+                    for (int dr = 0; dr < 3; ++dr)
 #pragma unroll
-                    for (int dc = 0; dc < 3; ++dc) {
-                        if (dr == 0 && dc == 0) continue;
-                        const v4f t = *reinterpret_cast<const v4f*>(w0 + (dr * p.PW + dc) * kPoolRowB);
+                        for (int dc = 0; dc < 3; ++dc) {
+                            if (dr == 0 && dc == 0) continue;
+                            const v4i t = *reinterpret_cast<const v4i*>(w0 + (dr * p.PW + dc) * kPoolRowB);
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) best[e] = __builtin_fmaxf(best[e], t[e]);
-                    }
+                            for (int e = 0; e < 4; ++e) top[e] = top[e] > t[e] ? top[e] : t[e];
+                        }
+                    const v4f s4 = *reinterpret_cast<const v4f*>(lds_sb + m * 32 + part * 4);
+                    const v4f b4 = *reinterpret_cast<const v4f*>(lds_sb + 128 + m * 32 + part * 4);
+                    const float floor = p.act == 1 ? 0.f : ninf;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) best[e] = __builtin_fmaxf(__builtin_fmaf((float)top[e], s4[e], b4[e]), floor);
+                } else {
+                    best = *reinterpret_cast<const v4f*>(w0);
+#pragma unroll
+                    for (int dr = 0; dr < 3; ++dr)
+#pragma unroll
+                        for (int dc = 0; dc < 3; ++dc) {
+                            if (dr == 0 && dc == 0) continue;
+                            const v4f t = *reinterpret_cast<const v4f*>(w0 + (dr * p.PW + dc) * kPoolRowB);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) best[e] = __builtin_fmaxf(best[e], t[e]);
+                        }
+                }
                 const bool ok = gy < p.POH && gx < p.POW;
                 const unsigned elem = ((unsigned)(n * p.POH + gy) * (unsigned)p.POW + gx) * (unsigned)p.K + kt * TM + m * 32 + part * 4;
                 const unsigned off = ok ? elem : kEpiInvalid;

@@ -149,17 +149,23 @@ CONV_POOL_SHAPES = [
 ]
 
 
+@pytest.mark.parametrize("act,negate", [(1, False), (0, False), (1, True), (0, True)], ids=["relu", "linear", "relu-negscale", "linear-negscale"])
 @pytest.mark.parametrize("args", CONV_POOL_SHAPES, ids=[f"s{a[0]}" for a in CONV_POOL_SHAPES])
-def test_conv_i8_maxpool_one_launch_bit_exact(ctx, args):
-    """Convolution (+ReLU) and the 3x3 stride-2 max pool behind it in one kernel == oracle conv then oracle pool."""
+def test_conv_i8_maxpool_one_launch_bit_exact(ctx, args, act, negate):
+    """Convolution (+ReLU) and the 3x3 stride-2 max pool behind it in one kernel == oracle conv then oracle pool. With
+    scales >= 0 the kernel pools the int32 accumulators and dequantizes the pooled pixels; a negative weight scale in
+    some channels makes it pool the dequantized floats instead."""
     seed, n, c, h, w, k, kernel, stride, pad, ppad, pad_mode = args
-    case = cases.conv_i8_case(seed, n, c, h, w, k, kernel, stride, pad, act=1)
+    case = cases.conv_i8_case(seed, n, c, h, w, k, kernel, stride, pad, act=act)
+    if negate:
+        case["ws"] = case["ws"].copy()
+        case["ws"][::3] *= np.float32(-1)
     fs_out = np.float32(23.5)
     y = cases.oracle_eval(case)
     want = port.pool2d(y, port.POOL_MAX, 3, 2, ppad, pad_mode=pad_mode)
     poh, pow_ = want.shape[2:]
     cs = gpueval.in_stride(c, gpueval.hip.I8, kernel)
-    d = ctx.conv_desc(n, c, h, w, k, kernel, stride, pad, 1, cs, k, 0, float(fs_out))
+    d = ctx.conv_desc(n, c, h, w, k, kernel, stride, pad, act, cs, k, 0, float(fs_out))
     xq = ctx.quantize_nchw_to_nhwc_i8(ctx.array(case["x"]), case["fs"], cs)
     wp = ctx.pack_conv_weights(d, gpueval.hip.I8, case["wt"])
     scale = ctx.array(gpueval.dequant_scales(case["ws"], case["fs"], k))
