@@ -50,6 +50,12 @@ constexpr size_t kLdsThird = 53 * 1024;   // at most this much each and three gr
 constexpr size_t kLdsHalf = 80 * 1024;    // two groups per CU
 constexpr long long kCUs = 256;           // compute units of the MI355X
 constexpr int kSbBytes = 1024;  // LDS kept for per-channel scale and bias of the group's (at most 128) channels
+// Phase timestamps (a development aid) are compiled in only with -DEXHIP_STAMPS=1: even as a never-taken branch
+// they cost the stage loop scalar registers and a dozen instructions per stage.
+#ifndef EXHIP_STAMPS
+#define EXHIP_STAMPS 0
+#endif
+constexpr bool kStamps = EXHIP_STAMPS != 0;
 constexpr unsigned kEpiInvalid = 0x3FFFFF00u;  // element offset whose byte offsets (x1, x4) lie past any accepted tensor
 
 struct ConvParams {
@@ -210,7 +216,8 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     auto stamp = [&](int k) {
-        if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * (THREADS / 64) + wave) * 16 + k] = wall_clock64();
+        if constexpr (kStamps)
+            if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * (THREADS / 64) + wave) * 16 + k] = wall_clock64();
     };
     stamp(0);
 
@@ -548,13 +555,13 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 if (want_a && !(next_chunk && dist == 2)) request_a();
             };
             long long t0 = 0, t1 = 0, t2 = 0;
-            if (p.dbg) t0 = wall_clock64();
+            if (kStamps && p.dbg) t0 = wall_clock64();
             mfma_stage(w_cur, a_cur, p.RS, requests);
-            if (p.dbg) t1 = wall_clock64();
+            if (kStamps && p.dbg) t1 = wall_clock64();
             if (more) wait_vmcnt(next_chunk && after_act < after_w[0] ? after_act : after_w[0]);
-            if (p.dbg) t2 = wall_clock64();
+            if (kStamps && p.dbg) t2 = wall_clock64();
             __syncthreads();
-            if (p.dbg && lane == 0) {
+            if (kStamps && p.dbg && lane == 0) {
                 const long long t3 = wall_clock64();
                 long long* d = p.dbg + ((size_t)blockIdx.x * (THREADS / 64) + wave) * 16;
                 d[9] += t1 - t0;
@@ -1419,7 +1426,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.n_chunks = pl.n_chunks; p.chunk_b = pl.chunk_b; p.RS = pl.RS; p.n_rg = pl.n_rg;
     p.tiles_x = pl.tiles_x; p.tiles_y = pl.tiles_y; p.ktiles = pl.ktiles;
     p.act = d->act; p.post_relu = d->post_relu; p.fs_out = d->fs_out; p.b_align = pl.b_align;
-    p.dbg = getenv("EXHIP_DEBUG_STAMPS") ? (long long*)strtoull(getenv("EXHIP_DEBUG_STAMPS"), nullptr, 0) : nullptr;
+    p.dbg = (kStamps && getenv("EXHIP_DEBUG_STAMPS")) ? (long long*)strtoull(getenv("EXHIP_DEBUG_STAMPS"), nullptr, 0) : nullptr;
     p.img_bytes = (unsigned)((size_t)d->h * d->w * p.cstride_b);
     p.magic_iw = (unsigned)(((1ull << 32) + pl.IW - 1) / pl.IW);
     p.magic_pw = (unsigned)(((1ull << 32) + pl.PW - 1) / pl.PW);
