@@ -539,13 +539,16 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         const char* a_cur = lds_a0;                // current tile, first filter row of the current stage
         const int a_stage_b = p.RS * p.lds_row_b;
         bool cur_odd = false;
-        int rg = 0;
-        for (int st = 0; st < n_stages; ++st) {
+        // One stage. first_rg / next_chunk: it is the first / last stage of its channel chunk; nrows: its filter rows.
+        // The three arrive as compile-time constants from the drivers below where the layer's shape fixes them: a stage
+        // is two dozen MFMAs per wave, and every wave-uniform test the compiler can drop from it counts.
+        auto stage = [&](int st, auto first_rg_t, auto next_chunk_t, auto nrows_t) {
+            const bool first_rg = first_rg_t, next_chunk = next_chunk_t;
+            const int nrows = nrows_t;
             const bool more = st + 1 < n_stages;
-            const bool next_chunk = rg + 1 == p.n_rg;
             // With one tile buffer the next chunk's tile can only be requested once every wave has left this chunk's
             // last stage (below); with two it is requested during the chunk's first stage.
-            const bool want_a = p.act_bufs > 1 && rg == 0 && a_req_left > 0;
+            const bool want_a = p.act_bufs > 1 && first_rg && a_req_left > 0;
             // The requests go out after the stage's first filter row has been issued: their issue cost then
             // overlaps with MFMAs already in the pipe instead of standing in front of them. The request needed
             // sooner goes first, so that the wait below can leave the other in flight.
@@ -556,7 +559,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
             };
             long long t0 = 0, t1 = 0, t2 = 0;
             if (kStamps && p.dbg) t0 = wall_clock64();
-            mfma_stage(w_cur, a_cur, p.RS, requests);
+            mfma_stage(w_cur, a_cur, nrows, requests);
             if (kStamps && p.dbg) t1 = wall_clock64();
             if (more) wait_vmcnt(next_chunk && after_act < after_w[0] ? after_act : after_w[0]);
             if (kStamps && p.dbg) t2 = wall_clock64();
@@ -579,12 +582,35 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
             w_cur += p.lds_w_b;
             if (w_cur == w_cur_end) w_cur = lds_w0 + aoff;
             if (next_chunk) {
-                rg = 0;
                 a_cur = lds_a0 + (cur_odd ? 0 : a_flip);
                 cur_odd = !cur_odd;
             } else {
-                ++rg;
                 a_cur += a_stage_b;
+            }
+        };
+        constexpr std::true_type yes{};
+        constexpr std::false_type no{};
+        constexpr std::integral_constant<int, 1> one_row{};
+        bool done = false;
+        if constexpr (EPI == 1 && KWE > 0) {
+            if (p.n_rg == 3 && p.RS == 1) {  // three filter rows, one per stage (the 3x3 layers)
+                for (int st = 0; st < n_stages; st += 3) {
+                    stage(st, yes, no, one_row);
+                    stage(st + 1, no, no, one_row);
+                    stage(st + 2, no, yes, one_row);
+                }
+                done = true;
+            } else if (p.n_rg == 1) {        // one stage per chunk (1x1 layers, 3x3 with all rows in a stage)
+                for (int st = 0; st < n_stages; ++st) stage(st, yes, yes, p.RS);
+                done = true;
+            }
+        }
+        if (!done) {
+            int rg = 0;
+            for (int st = 0; st < n_stages; ++st) {
+                const bool next_chunk = rg + 1 == p.n_rg;
+                stage(st, rg == 0, next_chunk, p.RS);
+                rg = next_chunk ? 0 : rg + 1;
             }
         }
     } else {
