@@ -70,6 +70,15 @@ extern "C" void exc_pipeline_set_fusion(exc_pipeline* p, int on) {
 
 extern "C" int exc_pipeline_last_fused(exc_pipeline* p) { return p->f32 ? p->f32->fused() : 0; }
 
+extern "C" void exc_pipeline_time_fused_span(exc_pipeline* p, int first_launch) {
+    if (p->f32) p->f32->time_fused_span(first_launch);
+}
+
+extern "C" float exc_pipeline_last_span(exc_pipeline* p, int* launches) {
+    if (launches) *launches = 0;
+    return p->f32 ? p->f32->last_span(launches) : 0.f;
+}
+
 extern "C" int exc_pipeline_set_input(exc_pipeline* p, const void* input, const int shape[4]) {
     if (p->dtype == 0) set_input(p->in32, p->device, input, shape);
     else set_input(p->in16, p->device, input, shape);

@@ -166,6 +166,9 @@ public:
     bool fusion_ = true;
     bool last_fused_ = false;
     double last_ms_ = 0;
+    int span_first_ = -1, span_launches_ = 0;  // time_fused_span / last_span
+    void* span_ev_[2] = {nullptr, nullptr};
+    int device() const { return device_; }
 
 private:
     // ---------------------------------------------------------------- per-layer executor
@@ -474,7 +477,22 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
         plan_ = plan;
     }
     plan_->input_ptr = input->gpu_data();
-    for (auto& launch : plan_->launches) launch();
+    if (span_first_ >= 0 && span_first_ < static_cast<int>(plan_->launches.size())) {
+        exhip_ctx* ctx = memory::device_context(device_);
+        if (!span_ev_[0]) {
+            EXHIP_FATAL(exhip_event_create(&span_ev_[0]));
+            EXHIP_FATAL(exhip_event_create(&span_ev_[1]));
+        }
+        for (int i = 0; i < static_cast<int>(plan_->launches.size()); ++i) {
+            if (i == span_first_) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+            plan_->launches[i]();
+        }
+        EXHIP_FATAL(exhip_event_record(ctx, span_ev_[1]));
+        span_launches_ = static_cast<int>(plan_->launches.size()) - span_first_;
+    } else {
+        for (auto& launch : plan_->launches) launch();
+        span_launches_ = 0;
+    }
     last_fused_ = true;
     for (auto& kv : plan_->outputs) {
         kv.second->mutable_gpu_data();  // the kernels just wrote it: the device copy is the newest
@@ -521,6 +539,19 @@ template <typename Dtype>
 void pipeline<Dtype>::set_fusion(bool on) { impl_->fusion_ = on; }
 template <typename Dtype>
 bool pipeline<Dtype>::fused() const { return impl_->last_fused_; }
+
+template <typename Dtype>
+void pipeline<Dtype>::time_fused_span(int first_launch) { impl_->span_first_ = first_launch; }
+
+template <typename Dtype>
+float pipeline<Dtype>::last_span(int* launches) {
+    if (launches) *launches = impl_->span_launches_;
+    if (!impl_->span_launches_) return 0.f;
+    EXHIP_FATAL(exhip_sync(memory::device_context(impl_->device())));
+    float ms = 0.f;
+    EXHIP_FATAL(exhip_event_elapsed_ms(impl_->span_ev_[0], impl_->span_ev_[1], &ms));
+    return ms;
+}
 template <typename Dtype>
 double pipeline<Dtype>::last_forward_ms() const { return impl_->last_ms_; }
 template <typename Dtype>

@@ -30,6 +30,9 @@ def lib():
         L.exc_pipeline_get.restype = ctypes.c_long
         L.exc_pipeline_get.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_long,
                                        ctypes.POINTER(ctypes.c_int)]
+        L.exc_pipeline_time_fused_span.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        L.exc_pipeline_last_span.restype = ctypes.c_float
+        L.exc_pipeline_last_span.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
         L.exc_registered_operations.restype = ctypes.c_size_t
         L.exc_registered_operations.argtypes = [ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
         _lib = L
@@ -75,6 +78,17 @@ class Pipeline:
         self.set_input(x)
         self.run()
         self.sync()
+
+    def time_fused_span(self, first_launch):
+        """Every later fused forward records device events around its launches first_launch .. last (0 = the input
+        quantizer); -1 switches that off."""
+        lib().exc_pipeline_time_fused_span(self.h, int(first_launch))
+
+    def last_span(self):
+        """(milliseconds, launches) between the events of the last fused forward; waits for the device."""
+        n = ctypes.c_int(0)
+        ms = lib().exc_pipeline_last_span(self.h, ctypes.byref(n))
+        return float(ms), n.value
 
     @property
     def fused(self):

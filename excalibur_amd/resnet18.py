@@ -247,6 +247,25 @@ class FusedRunner:
         for _, _, fn in self.steps:
             fn()
 
+    def forward_conv_span(self):
+        """One forward with one HIP event pair around its convolution launches (from in front of the first one to
+        behind the last launch); returns (ms, convolution launches). Everything else in the span must be
+        convolutions too, which holds when the stem's pool is fused."""
+        kinds = [kind for _, kind, _ in self.steps]
+        first = kinds.index("conv")
+        assert all(k == "conv" for k in kinds[first:]), "a non-convolution launch inside the span"
+        if not hasattr(self, "_span"):
+            self._span = (self.hip.Event(), self.hip.Event())
+        record, ctx_h = self.hip.lib().exhip_event_record, self.ctx.h
+        e0, e1 = self._span
+        for i, (_, _, fn) in enumerate(self.steps):
+            if i == first:
+                record(ctx_h, e0.h)
+            fn()
+        record(ctx_h, e1.h)
+        self.ctx.sync()
+        return e0.elapsed_ms(e1), len(kinds) - first
+
     def forward_timed(self):
         """One forward with a HIP event pair around every launch; returns [(label, kind, ms)].
 

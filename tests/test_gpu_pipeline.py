@@ -81,6 +81,15 @@ def test_resnet18_topology_through_the_pipeline(fusion):
         if not fusion:  # every intermediate blob exists as a float NCHW tensor, as in the reference
             assert np.array_equal(p.get("pool1"), blobs["pool1"])
             assert np.array_equal(p.get("l3b1_out"), blobs["l3b1_out"])
+        # device time of the convolution launches of a fused forward (what the benchmark's roofline divides by)
+        p.time_fused_span(1)
+        p.forward(x)
+        ms, launches = p.last_span()
+        assert (launches, ms > 0) == ((20, True) if fusion else (0, False))
+        assert np.array_equal(p.get(net.output), want)
+        p.time_fused_span(-1)
+        p.forward(x)
+        assert p.last_span() == (0.0, 0)
         # a second input of another shape rebuilds the plan
         x2 = np.random.default_rng(23).uniform(-1, 1, (1, 3, 64, 64)).astype(np.float32)
         p.forward(x2)
