@@ -71,6 +71,87 @@ def measured_traffic(n, hw):
     return None
 
 
+def bandwidth_table(iters=20):
+    """The path's memory-bound kernels at the benchmark network's tensor sizes, through the C ABI with preallocated
+    operands: HIP events around `iters` back-to-back launches, algorithmic bytes (every operand read once, every result
+    written once) over the 8 TB/s HBM peak. Returns [{"kernel", "us", "GB/s", "frac"}]."""
+    from excalibur_amd import hip
+    ctx = hip.Ctx(0)
+    L = hip.lib()
+    rng = np.random.default_rng(0)
+    cf, sz = ctypes.c_float, ctypes.c_size_t
+    rows = []
+
+    def bw(label, nbytes, fn):
+        for _ in range(3):
+            rc = fn()
+            assert rc == 0, (label, rc, L.exhip_last_error())
+        ctx.sync()
+        e0, e1 = hip.Event(), hip.Event()
+        e0.record(ctx)
+        for _ in range(iters):
+            fn()
+        e1.record(ctx)
+        ctx.sync()
+        ms = e0.elapsed_ms(e1) / iters
+        rows.append({"kernel": label, "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
+                     "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 3)})
+        print(f"{label:66s} {ms * 1e3:8.1f} us {nbytes / ms / 1e6:8.1f} GB/s {100 * nbytes / ms / 1e6 / PEAK_HBM_GBS:5.1f} %", file=sys.stderr, flush=True)
+
+    n, c, h, w = 32, 64, 160, 160          # the stage-1 tensors of the benchmark network
+    cnt = n * c * h * w
+    xf = ctx.array(rng.normal(0, 1, (n, c, h, w)).astype(np.float32))
+    yf, zf = ctx.empty((n, c, h, w), np.float32).zero(), ctx.empty((n, c, h, w), np.float32)
+    xh = ctx.array(rng.normal(0, 1, (n, c, h, w)).astype(np.float16).view(np.uint16))
+    yh, zh = ctx.empty((n, c, h, w), np.uint16).zero(), ctx.empty((n, c, h, w), np.uint16)
+    xin = ctx.array(rng.uniform(-1, 1, (n, 3, 640, 640)).astype(np.float32))
+    q = ctx.empty((n, 640, 640, 4), np.int8)
+    bw("first-layer quantizer, f32 NCHW 32x3x640x640 -> int8 NHWC4", xin.size * 4 + n * 640 * 640 * 4,
+       lambda: L.exhip_quantize_nchw_f32_to_nhwc_i8(ctx.h, xin.ptr, n, 3, 640, 640, cf(20.0), None, 4, q.ptr))
+    bw("layout NCHW f32 -> NHWC f32", cnt * 8, lambda: L.exhip_nchw_f32_to_nhwc_f32(ctx.h, xf.ptr, n, c, h, w, c, zf.ptr))
+    bw("layout NHWC f32 -> NCHW f32", cnt * 8, lambda: L.exhip_nhwc_f32_to_nchw_f32(ctx.h, xf.ptr, n, c, h, w, c, zf.ptr))
+    bw("layout NCHW f16 -> NHWC f16", cnt * 4, lambda: L.exhip_nchw_f16_to_nhwc_f16(ctx.h, xh.ptr, n, c, h, w, c, zh.ptr))
+    bw("layout NHWC f16 -> NCHW f16", cnt * 4, lambda: L.exhip_nhwc_f16_to_nchw_f16(ctx.h, xh.ptr, n, c, h, w, c, zh.ptr))
+    bw("f32 -> f16", cnt * 6, lambda: L.exhip_f32_to_f16(ctx.h, xf.ptr, zh.ptr, sz(cnt)))
+    bw("f16 -> f32", cnt * 6, lambda: L.exhip_f16_to_f32(ctx.h, xh.ptr, zf.ptr, sz(cnt)))
+    bw("eltwise add + ReLU f32", cnt * 12, lambda: L.exhip_add_f32(ctx.h, xf.ptr, yf.ptr, zf.ptr, sz(cnt), 1))
+    bw("eltwise add + ReLU f16", cnt * 6, lambda: L.exhip_add_f16(ctx.h, xh.ptr, yh.ptr, zh.ptr, sz(cnt), 1))
+    bw("ReLU f32", cnt * 8, lambda: L.exhip_relu_f32(ctx.h, xf.ptr, zf.ptr, sz(cnt)))
+    ptrs, coef = (ctypes.c_void_p * 2)(xf.ptr, yf.ptr), (ctypes.c_float * 2)(1.0, 1.0)
+    bw("Eltwise SUM f32, two inputs", cnt * 12, lambda: L.exhip_eltwise_f32(ctx.h, ptrs, 2, coef, 1, zf.ptr, sz(cnt)))
+    bw("HardSwish f32", cnt * 8, lambda: L.exhip_unary_f32(ctx.h, 0, xf.ptr, zf.ptr, sz(cnt), cf(1 / 6), cf(0.5)))
+    bw("HardSwish f16", cnt * 4, lambda: L.exhip_unary_f16(ctx.h, 0, xh.ptr, zh.ptr, sz(cnt), cf(1 / 6), cf(0.5)))
+    p0, p1 = ctx.array(rng.normal(0, 1, c).astype(np.float32)), ctx.array(rng.normal(0, 1, c).astype(np.float32))
+    bw("BatchNorm f32", cnt * 8, lambda: L.exhip_channelwise_f32(ctx.h, 1, xf.ptr, zf.ptr, n, c, h * w, p0.ptr, p1.ptr, 0))
+    bw("BatchNorm f16", cnt * 4, lambda: L.exhip_channelwise_f16(ctx.h, 1, xh.ptr, zh.ptr, n, c, h * w, p0.ptr, p1.ptr, 0))
+    big = ctx.empty((n, 2 * c, h, w), np.float32)
+    chs = (ctypes.c_int * 2)(c, c)
+    bw("Concat f32, 2 x 64 channels", cnt * 16, lambda: L.exhip_concat_channels_f32(ctx.h, ptrs, chs, 2, n, h * w, big.ptr))
+    small = ctx.array(rng.normal(0, 1, (n, c, h // 2, w // 2)).astype(np.float32))
+    bw("Interp nearest x2 f32", cnt * 5, lambda: L.exhip_interp_nearest_f32(ctx.h, small.ptr, zf.ptr, n, c, h // 2, w // 2, h, w))
+    pf = ctx.empty((n, c, h // 2, w // 2), np.float32)
+    bw("max pool 3x3 s2 p1 f32 NCHW", cnt * 5,
+       lambda: L.exhip_pool2d_nchw_f32(ctx.h, xf.ptr, pf.ptr, n, c, h, w, h // 2, w // 2, 0, 3, 3, 2, 2, 1, 1, 1, 1, 0))
+    pq = ctx.empty((n, h // 2, w // 2, c), np.int8)
+    bw("max pool 3x3 s2 p1 f32 NHWC + int8 copy", cnt * 5 + cnt // 4,
+       lambda: L.exhip_maxpool2d_nhwc_f32(ctx.h, xf.ptr, pf.ptr, pq.ptr, cf(20.0), n, c, h, w, c, h // 2, w // 2, 3, 3, 2, 2, 1, 1))
+    ph = ctx.empty((n, h // 2, w // 2, c), np.uint16)
+    bw("max pool 3x3 s2 p1 f16 NHWC", cnt * 2 + cnt // 2,
+       lambda: L.exhip_pool2d_nhwc_f16(ctx.h, xh.ptr, ph.ptr, n, c, h, w, c, h // 2, w // 2, 0, 3, 3, 2, 2, 1, 1, 1, 1, 0))
+    w9, b9 = ctx.array(rng.normal(0, 0.1, (128, 9)).astype(np.float32)), ctx.array(rng.normal(0, 0.1, 128).astype(np.float32))
+    bw("depthwise 3x3 s1 f32 NCHW, 32x64x160x160", cnt * 8,
+       lambda: L.exhip_dwconv3x3_nchw_f32(ctx.h, xf.ptr, w9.ptr, b9.ptr, zf.ptr, n, c, h, w, 1, 1, 1, 1, 1, 1))
+    dn, dc, dh = 64, 128, 56               # the MobileNet-style stack's middle maps
+    dx = ctx.array(rng.normal(0, 1, (dn, dh, dh, dc)).astype(np.float16).view(np.uint16))
+    dy = ctx.empty((dn, dh, dh, dc), np.uint16)
+    bw("depthwise 3x3 s1 f16 NHWC, 64x128x56x56", dx.size * 4,
+       lambda: L.exhip_dwconv3x3_nhwc_f16(ctx.h, dx.ptr, w9.ptr, b9.ptr, dy.ptr, dn, dc, dh, dh, dc, 1, 1, 1, 1, 1, 1))
+    bw("depthwise 3x3 s2 f16 NHWC, 64x128x56x56", dx.size * 2 + dx.size // 2,
+       lambda: L.exhip_dwconv3x3_nhwc_f16(ctx.h, dx.ptr, w9.ptr, b9.ptr, dy.ptr, dn, dc, dh, dh, dc, 2, 1, 1, 1, 1, 1))
+    ctx.close()
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -80,11 +161,18 @@ def main():
     ap.add_argument("--hw", type=int, default=640)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--per-layer", action="store_true", help="print per-launch timings to stderr")
+    ap.add_argument("--bandwidth", action="store_true",
+                    help="instead of the network: time the memory-bound kernels of the path and print their GB/s")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; the batch shards trivially across GPUs but no multi-GPU path "
               "is part of it (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
+
+    if args.bandwidth:
+        print(json.dumps({"metric": "achieved HBM GB/s of the memory-bound kernels", "peak_GB/s": PEAK_HBM_GBS,
+                          "kernels": bandwidth_table()}))
+        return
 
     import tempfile
 
