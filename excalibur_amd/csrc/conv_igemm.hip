@@ -168,29 +168,41 @@ __device__ __forceinline__ void async_load16(__amdgpu_buffer_rsrc_t rsrc, int vo
 }
 
 // Waits until at most `keep` of this wave's loads are in flight. The instruction takes an immediate, so a
-// wave-uniform value picks the largest supported immediate that does not exceed it.
+// wave-uniform value selects one of seventeen waits (16 stands for "16 or more"): a computed jump into a table of
+// (s_waitcnt, s_branch) pairs, eight bytes each. Written out by hand because the compiler turns the equivalent switch
+// into a chain of some twenty-five scalar instructions and eight branches, once per stage of the convolution loop.
 template <int N>
 __device__ __forceinline__ void wait_vmcnt_imm() { __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 __device__ __forceinline__ void wait_vmcnt(int keep) {
-    switch (keep < 16 ? keep : 16) {  // a balanced compare tree: four branches deep
-    case 0: wait_vmcnt_imm<0>(); break;
-    case 1: wait_vmcnt_imm<1>(); break;
-    case 2: wait_vmcnt_imm<2>(); break;
-    case 3: wait_vmcnt_imm<3>(); break;
-    case 4: wait_vmcnt_imm<4>(); break;
-    case 5: wait_vmcnt_imm<5>(); break;
-    case 6: wait_vmcnt_imm<6>(); break;
-    case 7: wait_vmcnt_imm<7>(); break;
-    case 8: wait_vmcnt_imm<8>(); break;
-    case 9: wait_vmcnt_imm<9>(); break;
-    case 10: wait_vmcnt_imm<10>(); break;
-    case 11: wait_vmcnt_imm<11>(); break;
-    case 12: wait_vmcnt_imm<12>(); break;
-    case 13: wait_vmcnt_imm<13>(); break;
-    case 14: wait_vmcnt_imm<14>(); break;
-    case 15: wait_vmcnt_imm<15>(); break;
-    default: wait_vmcnt_imm<16>(); break;
-    }
+    const int k = __builtin_amdgcn_readfirstlane(keep < 0 ? 0 : keep < 16 ? keep : 16);  // the jump must land inside the table
+    int entry;
+    __asm__ volatile(
+        "s_getpc_b64 vcc\n\t"                    // address of the next instruction
+        "s_lshl3_add_u32 %0, %1, 16\n\t"         // 8 * k + the 16 bytes from there to the table
+        "s_add_u32 vcc_lo, vcc_lo, %0\n\t"
+        "s_addc_u32 vcc_hi, vcc_hi, 0\n\t"
+        "s_setpc_b64 vcc\n\t"
+        "s_waitcnt vmcnt(0)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(1)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(2)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(3)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(4)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(5)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(6)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(7)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(8)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(9)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(10)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(11)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(12)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(13)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(14)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(15)\n\ts_branch .Lwait_done%=\n\t"
+        "s_waitcnt vmcnt(16)\n"
+        ".Lwait_done%=:"
+        : "=&s"(entry)
+        : "s"(k)
+        : "vcc", "scc", "memory");
 }
 
 // KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
