@@ -33,3 +33,46 @@ def test_fused_resnet18_int8_bit_exact(ctx, n, hw):
     run.forward()
     ctx.sync()
     assert np.array_equal(run.out.download(), want)
+
+
+def test_benchmark_batch_at_full_size():
+    """The benchmark's own workload (32 x 3 x 640 x 640 through the host pipeline) checked by what does not need a CPU
+    pass over 32 images: (a) images are independent, so a single image run alone (other tile plans, other groups per CU)
+    gives the bytes of its row of the batch; (b) the per-layer executor (float NCHW blobs between layers, every kernel
+    at its real size) agrees with the fused plan; (c) where the compiled reference is present, one 640 x 640 image through
+    the reference's CPU path, bit for bit."""
+    import os
+    import tempfile
+
+    from excalibur_amd import pipeline as xp
+    from oracle import ref
+
+    net = ResNet18Int8(seed=1234, calib_hw=64)
+    n, hw = 32, 640
+    x = np.random.default_rng(99).uniform(-1, 1, (n, 3, hw, hw)).astype(np.float32)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        net.write_model(path)
+        p = xp.Pipeline(net.topology(), path, 0, "f32", fusion=True)
+        p.forward(x)
+        assert p.fused
+        batch = p.get(net.output)
+        assert batch.shape == (n, 512, 20, 20)
+        assert np.count_nonzero(batch) > batch.size // 8
+        for i in (0, 17, 31):
+            p.forward(x[i:i + 1])
+            assert np.array_equal(p.get(net.output)[0], batch[i]), f"image {i} alone differs from its row of the batch"
+        p.close()
+        layers = xp.Pipeline(net.topology(), path, 0, "f32", fusion=False)
+        layers.forward(x[:2])
+        assert not layers.fused
+        assert np.array_equal(layers.get(net.output), batch[:2])
+        layers.close()
+        if ref.available():
+            r = ref.Pipeline(net.topology(), path, "f32")
+            r.forward(x[17:18])
+            assert np.array_equal(r.get(net.output)[0], batch[17])
+            r.close()
+    finally:
+        os.unlink(path)
