@@ -588,24 +588,27 @@ __global__ __launch_bounds__(kBlock) void pool2d_nchw_f32_kernel(const float* __
 // makes four neighbouring outputs of one row from two aligned 16-byte loads per input row (plus one halo float to
 // the left for left padding 1, or to the right for a 3-wide window without left padding), so a wave reads whole
 // rows contiguously. Window clipping, the divisor and the row-major summation order are those of the general kernel.
-template <int K, int TYPE>
+template <int K, int TYPE, int ROWS, int PL>
 __global__ __launch_bounds__(kBlock) void pool_s2_nchw_f32_strip_kernel(const float* __restrict__ x, float* __restrict__ y,
-                                                                        int H, int W, int OH, int OW, int pt, int pb, int pl,
-                                                                        int pr, int include_pad, int strips, size_t total) {
+                                                                        int H, int W, int OH, int OW, int pt, int pb,
+                                                                        int pr, int include_pad, int strips, int row_blocks,
+                                                                        size_t total) {
+    constexpr int pl = PL;  // left padding, 0 or 1: a constant so that every index into v[] is one (registers, not scratch)
     const size_t gi = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (gi >= total) return;
     const int t = (int)(gi % strips);
     const size_t rest = gi / strips;
-    const int ph = (int)(rest % OH);
-    const size_t nc = rest / OH;
+    const int ph0 = (int)(rest % row_blocks) * ROWS;  // this thread's first output row; it makes ROWS of them
+    const size_t nc = rest / row_blocks;
     const float* in = x + nc * H * W;
     const int c0 = 8 * t;  // first column of the aligned chunk; v[i] below holds column c0 - 1 + i
     const float fill = TYPE == 0 ? -FLT_MAX : 0.f;
-    float v[K][10];
-    const int hs0 = ph * 2 - pt;
+    constexpr int NR = 2 * (ROWS - 1) + K;  // input rows under ROWS consecutive windows: neighbouring windows share K - 2 of them
+    float v[NR][10];
+    const int hs00 = ph0 * 2 - pt;
 #pragma unroll
-    for (int a = 0; a < K; ++a) {
-        const int iy = hs0 + a;
+    for (int a = 0; a < NR; ++a) {
+        const int iy = hs00 + a;
         const bool row_ok = iy >= 0 && iy < H;
         const float* row = in + (size_t)iy * W;
         v4f lo = {fill, fill, fill, fill}, hi = lo;
@@ -619,49 +622,54 @@ __global__ __launch_bounds__(kBlock) void pool_s2_nchw_f32_strip_kernel(const fl
             v[a][5 + e] = hi[e];
         }
     }
-    v4f out;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int first = 2 * j - pl + 1;  // index into v[] of the window's first column
-        float res;
-        if (TYPE == 0) {
-            res = -FLT_MAX;
+    for (int r = 0; r < ROWS; ++r) {
+        const int ph = ph0 + r, hs0 = hs00 + 2 * r;
+        const bool row_out = ph < OH;  // no early exit: the loop must unroll for v[] to stay in registers
+        v4f out;
 #pragma unroll
-            for (int a = 0; a < K; ++a)
+        for (int j = 0; j < 4; ++j) {
+            const int first = 2 * j - pl + 1;  // index into v[] of the window's first column
+            float res;
+            if (TYPE == 0) {
+                res = -FLT_MAX;
 #pragma unroll
-                for (int b = 0; b < K; ++b) {
-                    const float tap = v[a][first + b];
-                    res = res < tap ? tap : res;
-                }
-        } else {
-            const int pw = 4 * t + j;
-            int hs = hs0, wsx = pw * 2 - pl;
-            int he = min(hs + K, H + pb), we = min(wsx + K, W + pr);
-            int pool = (he - hs) * (we - wsx);
-            hs = max(hs, 0);
-            wsx = max(wsx, 0);
-            he = min(he, H);
-            we = min(we, W);
-            if (!include_pad) pool = (he - hs) * (we - wsx);
-            res = 0.f;
+                for (int a = 0; a < K; ++a)
 #pragma unroll
-            for (int a = 0; a < K; ++a)
+                    for (int b = 0; b < K; ++b) {
+                        const float tap = v[2 * r + a][first + b];
+                        res = res < tap ? tap : res;
+                    }
+            } else {
+                const int pw = 4 * t + j;
+                int hs = hs0, wsx = pw * 2 - pl;
+                int he = min(hs + K, H + pb), we = min(wsx + K, W + pr);
+                int pool = (he - hs) * (we - wsx);
+                hs = max(hs, 0);
+                wsx = max(wsx, 0);
+                he = min(he, H);
+                we = min(we, W);
+                if (!include_pad) pool = (he - hs) * (we - wsx);
+                res = 0.f;
 #pragma unroll
-                for (int b = 0; b < K; ++b) {
-                    const int iy = hs0 + a, ix = pw * 2 - pl + b;
-                    if (iy >= hs && iy < he && ix >= wsx && ix < we) res += v[a][first + b];
-                }
-            res = res / (float)pool;
+                for (int a = 0; a < K; ++a)
+#pragma unroll
+                    for (int b = 0; b < K; ++b) {
+                        const int iy = hs0 + a, ix = pw * 2 - pl + b;
+                        if (iy >= hs && iy < he && ix >= wsx && ix < we) res += v[2 * r + a][first + b];
+                    }
+                res = res / (float)pool;
+            }
+            out[j] = res;
         }
-        out[j] = res;
-    }
-    float* dst = y + (nc * OH + ph) * OW + 4 * t;
-    if ((OW & 3) == 0) {
-        *reinterpret_cast<v4f*>(dst) = out;
-    } else {
+        float* dst = y + (nc * OH + ph) * OW + 4 * t;
+        if ((OW & 3) == 0) {
+            if (row_out) *reinterpret_cast<v4f*>(dst) = out;
+        } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (4 * t + j < OW) dst[j] = out[j];
+            for (int j = 0; j < 4; ++j)
+                if (row_out && 4 * t + j < OW) dst[j] = out[j];
+        }
     }
 }
 
@@ -735,6 +743,56 @@ __global__ __launch_bounds__(kBlock) void maxpool_nhwc_f32_kernel(const float* _
     }
 }
 
+// 3x3 stride-2 max pooling on NHWC float32, a 2 x 2 block of output pixels per thread (four channels each): the four
+// windows share a row and a column, so 25 loads instead of 36, all in flight at once. Taps outside the image count as
+// -FLT_MAX, the clipped window of the general kernel. Optional requantized int8 copy as there.
+__global__ __launch_bounds__(kBlock) void maxpool3x3s2_nhwc_f32_block_kernel(const float* __restrict__ x, float* __restrict__ y,
+                                                                             int8_t* __restrict__ yq, float fs_out, int H, int W,
+                                                                             int cs, int OH, int OW, int pt, int pl, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 4, pairs = (OW + 1) / 2, row_pairs = (OH + 1) / 2;
+    const int g = (int)(i % groups);
+    size_t pix = i / groups;
+    const int ox = (int)(pix % pairs) * 2;
+    pix /= pairs;
+    const int oy = (int)(pix % row_pairs) * 2;
+    const size_t n = pix / row_pairs;
+    const int iy0 = oy * 2 - pt, ix0 = ox * 2 - pl;
+    const v4f lowest = {-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX};
+    v4f t[5][5];
+#pragma unroll
+    for (int a = 0; a < 5; ++a)
+#pragma unroll
+        for (int b = 0; b < 5; ++b) {
+            const int iy = iy0 + a, ix = ix0 + b;
+            const bool ok = (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+            t[a][b] = ok ? *reinterpret_cast<const v4f*>(x + ((n * H + iy) * W + ix) * cs + g * 4) : lowest;
+        }
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            v4f m = lowest;
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+#pragma unroll
+                for (int b = 0; b < 3; ++b)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) m[e] = m[e] < t[2 * r + a][2 * j + b][e] ? t[2 * r + a][2 * j + b][e] : m[e];
+            if (oy + r < OH && ox + j < OW) {
+                const size_t o = ((n * OH + oy + r) * OW + ox + j) * cs + g * 4;
+                if (y) *reinterpret_cast<v4f*>(y + o) = m;
+                if (yq) {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(m[e] * fs_out) & 0xff) << (8 * e);
+                    *reinterpret_cast<int*>(yq + o) = (int)w;
+                }
+            }
+        }
+}
+
 // Max pooling with a small fixed window on half storage: the maximum of halves is exact, so the taps are compared
 // as packed halves, all window loads in flight at once. Taps outside the image count as -inf (the clipped window of
 // the general kernel); an all-padding window cannot occur for the output sizes the layer computes.
@@ -769,6 +827,47 @@ __global__ __launch_bounds__(kBlock) void maxpool_nhwc_f16_window_kernel(const u
 #pragma unroll
         for (int b = 0; b < K; ++b) best = __builtin_elementwise_max(best, tap[a][b]);
     *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 8) = __builtin_bit_cast(v4i, best);
+}
+
+// The 3x3 stride-2 window on half storage, a 2 x 2 block of output pixels per thread (eight channels each): 25 loads
+// instead of 36, since neighbouring windows share a row and a column.
+__global__ __launch_bounds__(kBlock) void maxpool3x3s2_nhwc_f16_block_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                                             int H, int W, int cs, int OH, int OW, int pt, int pl,
+                                                                             size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 8, pairs = (OW + 1) / 2, row_pairs = (OH + 1) / 2;
+    const int g = (int)(i % groups);
+    size_t pix = i / groups;
+    const int ox = (int)(pix % pairs) * 2;
+    pix /= pairs;
+    const int oy = (int)(pix % row_pairs) * 2;
+    const size_t n = pix / row_pairs;
+    const int iy0 = oy * 2 - pt, ix0 = ox * 2 - pl;
+    const _Float16 ninf = -__builtin_inff16();
+    const v8h lowest = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+    v8h tap[5][5];
+#pragma unroll
+    for (int a = 0; a < 5; ++a)
+#pragma unroll
+        for (int b = 0; b < 5; ++b) {
+            const int iy = iy0 + a, ix = ix0 + b;
+            tap[a][b] = lowest;
+            if ((unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W)
+                tap[a][b] = __builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(x + ((n * H + iy) * W + ix) * cs + g * 8));
+        }
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            v8h best = lowest;
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+#pragma unroll
+                for (int b = 0; b < 3; ++b) best = __builtin_elementwise_max(best, tap[2 * r + a][2 * j + b]);
+            if (oy + r < OH && ox + j < OW)
+                *reinterpret_cast<v4i*>(y + ((n * OH + oy + r) * OW + ox + j) * cs + g * 8) = __builtin_bit_cast(v4i, best);
+        }
 }
 
 __global__ __launch_bounds__(kBlock) void pool2d_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int H,
@@ -1600,14 +1699,24 @@ extern "C" int exhip_pool2d_nchw_f32(exhip_ctx* ctx, const float* x, float* y, i
                               w % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     if (strip_window) {
         const int strips = (ow + 3) / 4;
-        const size_t threads = (size_t)n * c * oh * strips;
-#define EXHIP_POOL_STRIP(K, T)                                                                                              \
-    hipLaunchKernelGGL((pool_s2_nchw_f32_strip_kernel<K, T>), dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, x, y, \
-                       h, w, oh, ow, pt, pb, pl, pr, include_pad, strips, threads)
-        if (kh == 2 && type == 0) EXHIP_POOL_STRIP(2, 0);
-        else if (kh == 2) EXHIP_POOL_STRIP(2, 1);
-        else if (type == 0) EXHIP_POOL_STRIP(3, 0);
-        else EXHIP_POOL_STRIP(3, 1);
+        // maximum: two output rows per thread (five input rows instead of six: the windows share one); the averages keep
+        // one row per thread
+        const int rows = type == 0 ? 2 : 1;
+        const int row_blocks = (oh + rows - 1) / rows;
+        const size_t threads = (size_t)n * c * row_blocks * strips;
+#define EXHIP_POOL_STRIP(K, T, R)                                                                                                  \
+    do {                                                                                                                           \
+        if (pl == 0)                                                                                                               \
+            hipLaunchKernelGGL((pool_s2_nchw_f32_strip_kernel<K, T, R, 0>), dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, \
+                               x, y, h, w, oh, ow, pt, pb, pr, include_pad, strips, row_blocks, threads);                          \
+        else                                                                                                                       \
+            hipLaunchKernelGGL((pool_s2_nchw_f32_strip_kernel<K, T, R, 1>), dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, \
+                               x, y, h, w, oh, ow, pt, pb, pr, include_pad, strips, row_blocks, threads);                          \
+    } while (0)
+        if (kh == 2 && type == 0) EXHIP_POOL_STRIP(2, 0, 2);
+        else if (kh == 2) EXHIP_POOL_STRIP(2, 1, 1);
+        else if (type == 0) EXHIP_POOL_STRIP(3, 0, 2);
+        else EXHIP_POOL_STRIP(3, 1, 1);
 #undef EXHIP_POOL_STRIP
         EXHIP_LAUNCH_CHECK();
         return 0;
@@ -1623,6 +1732,14 @@ extern "C" int exhip_maxpool2d_nhwc_f32(exhip_ctx* ctx, const float* x, float* y
                                         int h, int w, int cs, int oh, int ow, int kh, int kw, int sh, int sw, int pt, int pl) {
     REQ_CTX("exhip_maxpool2d_nhwc_f32");
     EXHIP_REQUIRE(x && (y || y_i8) && n > 0 && c > 0 && cs >= c && cs % 4 == 0, "exhip_maxpool2d_nhwc_f32: bad argument");
+    if (kh == 3 && kw == 3 && sh == 2 && sw == 2 && pt >= 0 && pl >= 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+        (!y || (reinterpret_cast<uintptr_t>(y) & 15) == 0)) {
+        const size_t threads = (size_t)n * ((oh + 1) / 2) * ((ow + 1) / 2) * (cs / 4);
+        hipLaunchKernelGGL(maxpool3x3s2_nhwc_f32_block_kernel, dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, x, y, y_i8,
+                           fs_out, h, w, cs, oh, ow, pt, pl, threads);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const size_t total = (size_t)n * oh * ow * (cs / 4);
     hipLaunchKernelGGL(maxpool_nhwc_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, y_i8, fs_out, h, w,
                        cs, oh, ow, kh, kw, sh, sw, pt, pl, total);
@@ -1639,10 +1756,11 @@ extern "C" int exhip_pool2d_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t
     const size_t total = (size_t)n * oh * ow * (cs / 8);
     if (type == 0 && kh == kw && sh == sw && sh == 2 && (kh == 2 || kh == 3) && pt >= 0 && pl >= 0 && pt < kh && pl < kw &&
         (oh - 1) * 2 - pt < h && (ow - 1) * 2 - pl < w) {
-        if (kh == 3)
-            hipLaunchKernelGGL((maxpool_nhwc_f16_window_kernel<3, 2>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h,
-                               w, cs, oh, ow, pt, pl, total);
-        else
+        if (kh == 3) {
+            const size_t threads = (size_t)n * ((oh + 1) / 2) * ((ow + 1) / 2) * (cs / 8);
+            hipLaunchKernelGGL(maxpool3x3s2_nhwc_f16_block_kernel, dim3(blocks_for(threads)), dim3(kBlock), 0, ctx->stream, x, y, h, w,
+                               cs, oh, ow, pt, pl, threads);
+        } else
             hipLaunchKernelGGL((maxpool_nhwc_f16_window_kernel<2, 2>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h,
                                w, cs, oh, ow, pt, pl, total);
         EXHIP_LAUNCH_CHECK();
