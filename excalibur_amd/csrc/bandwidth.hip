@@ -279,12 +279,14 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_kernel(const float*
 // band of output rows with the three input rows it needs in registers. A row arrives as one (stride 1) or two
 // (stride 2) aligned 16-byte loads plus the halo floats the padding asks for, through a buffer descriptor whose
 // range check turns taps outside the image into zeros. slot i of a row holds column c0 - 1 + i.
-template <int STRIDE, int ACT>
+template <int STRIDE, int ACT, int PL>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_strip_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                                           const float* __restrict__ bias, float* __restrict__ y,
-                                                                          int C, int H, int W, int OH, int OW, int pt, int pl,
+                                                                          int C, int H, int W, int OH, int OW, int pt,
                                                                           int band_rows, int bands, int strips, unsigned x_bytes,
                                                                           unsigned y_bytes, size_t total) {
+    constexpr int pl = PL;  // left padding (0 or 1) as a constant: which register a tap reads is then fixed, and the halo
+                            // floats that this padding does not use are not loaded
     constexpr int CH = STRIDE == 1 ? 1 : 2;  // aligned 16-byte chunks per row
     constexpr int NI = 4 * CH + 3, KEEP = 3 - STRIDE;
     constexpr unsigned kRowOutside = 0x80000000u, kColOutside = 0x40000000u;  // tensors are at most 2^30 bytes
@@ -321,9 +323,12 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_strip_kernel(const 
 #pragma unroll
             for (int e = 0; e < 4; ++e) dst[1 + 4 * q + e] = v[e];
         }
-        dst[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[0]), 0, 0));
-        dst[NI - 2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[1]), 0, 0));
-        dst[NI - 1] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[2]), 0, 0));
+        dst[0] = dst[NI - 2] = dst[NI - 1] = 0.f;
+        if constexpr (pl == 1) dst[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[0]), 0, 0));
+        if constexpr (STRIDE == 1 || pl == 0)
+            dst[NI - 2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[1]), 0, 0));
+        if constexpr (STRIDE == 1 && pl == 0)
+            dst[NI - 1] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(xr, (int)(row_off + halo_off[2]), 0, 0));
     };
     const int oy0 = band * band_rows, oy1 = min(OH, oy0 + band_rows);
 #pragma unroll
@@ -1588,10 +1593,17 @@ extern "C" int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const fl
         if (env_rows > 0) band_rows = std::min(env_rows, oh);
         bands = (oh + band_rows - 1) / band_rows;
         const size_t total = per_band * bands;
-#define EXHIP_DW_STRIP(S, A)                                                                                              \
-    hipLaunchKernelGGL((dwconv3x3_nchw_f32_strip_kernel<S, A>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, \
-                       w9, bias, y, c, h, w, oh, ow, pt, pl, band_rows, bands, strips, (unsigned)x_bytes, (unsigned)y_bytes, \
-                       total)
+#define EXHIP_DW_STRIP(S, A)                                                                                                     \
+    do {                                                                                                                         \
+        if (pl == 0)                                                                                                             \
+            hipLaunchKernelGGL((dwconv3x3_nchw_f32_strip_kernel<S, A, 0>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, \
+                               w9, bias, y, c, h, w, oh, ow, pt, band_rows, bands, strips, (unsigned)x_bytes, (unsigned)y_bytes,  \
+                               total);                                                                                           \
+        else                                                                                                                     \
+            hipLaunchKernelGGL((dwconv3x3_nchw_f32_strip_kernel<S, A, 1>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, \
+                               w9, bias, y, c, h, w, oh, ow, pt, band_rows, bands, strips, (unsigned)x_bytes, (unsigned)y_bytes,  \
+                               total);                                                                                           \
+    } while (0)
         if (stride == 1) {
             if (act == 0) EXHIP_DW_STRIP(1, 0);
             else if (act == 1) EXHIP_DW_STRIP(1, 1);
