@@ -432,7 +432,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nhwc_f16_kernel(const uint16
 // by vector ALU issue as much as by memory, hence the template on the activation and the masked, packed stores.
 // Arithmetic order per output is that of dw_pixel.
 template <int STRIDE, int PX, int ACT>
-__global__ __launch_bounds__(kBlock) void dwconv3x3_nhwc_f16_strip_kernel(const uint16_t* __restrict__ x,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void dwconv3x3_nhwc_f16_strip_kernel(const uint16_t* __restrict__ x,
                                                                           const float* __restrict__ w,
                                                                           const float* __restrict__ bias,
                                                                           uint16_t* __restrict__ y, int C, int H, int W,
