@@ -1120,6 +1120,21 @@ __global__ __launch_bounds__(kBlock) void channelwise_f16_kernel(const uint16_t*
     }
 }
 
+// The per-channel layers on NHWC half storage (channel = element index modulo C, C a multiple of eight): eight
+// consecutive channels of one pixel per thread.
+template <int OP>
+__global__ __launch_bounds__(kBlock) void channelwise_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                                      size_t n8, int C, const float* __restrict__ p0,
+                                                                      const float* __restrict__ p1, int shared) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n8) return;
+    const int c0 = (int)((i * 8) % (size_t)C);
+    v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(x)[i]), v8f);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = channel_value<OP>(v[e], p0[shared ? 0 : c0 + e], p1 ? p1[c0 + e] : 0.f);
+    reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
+}
+
 // Per-channel layers on NCHW. OP 0 PReLU (p0 = slope, one per channel or one shared), 1 BatchNorm as
 // fma(p1[c], x, p0[c]) with the load-time a / b, 2 Input (x - p0[c]) * p1[c]. One block row per (image, channel) plane.
 template <int OP>
@@ -1950,6 +1965,31 @@ extern "C" int exhip_channelwise_f16(exhip_ctx* ctx, int op, const uint16_t* x, 
     case EXHIP_CHANNEL_BATCHNORM: launch_channelwise_f16<1>(ctx, x, y, n, c, hw, p0, p1, 0); break;
     case EXHIP_CHANNEL_INPUT: launch_channelwise_f16<2>(ctx, x, y, n, c, hw, p0, p1, 0); break;
     default: exhip_set_error("exhip_channelwise_f16: unknown op %d", op); return EXHIP_ERR_ARG;
+    }
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_channelwise_nhwc_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, size_t pixels, int c,
+                                          const float* p0, const float* p1, int shared) {
+    REQ_CTX("exhip_channelwise_nhwc_f16");
+    EXHIP_REQUIRE(x && y && p0 && pixels > 0 && c > 0, "exhip_channelwise_nhwc_f16: bad argument");
+    EXHIP_REQUIRE(c % 8 == 0, "exhip_channelwise_nhwc_f16: %d channels, need a multiple of 8", c);
+    EXHIP_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0,
+                  "exhip_channelwise_nhwc_f16: tensors must be 16-byte aligned");
+    EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || p1, "exhip_channelwise_nhwc_f16: this op needs two parameter arrays");
+    const size_t n8 = pixels * (size_t)c / 8;
+    switch (op) {
+    case EXHIP_CHANNEL_PRELU:
+        hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<0>), dim3(blocks_for(n8)), dim3(kBlock), 0, ctx->stream, x, y, n8, c, p0, p1, shared);
+        break;
+    case EXHIP_CHANNEL_BATCHNORM:
+        hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<1>), dim3(blocks_for(n8)), dim3(kBlock), 0, ctx->stream, x, y, n8, c, p0, p1, 0);
+        break;
+    case EXHIP_CHANNEL_INPUT:
+        hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<2>), dim3(blocks_for(n8)), dim3(kBlock), 0, ctx->stream, x, y, n8, c, p0, p1, 0);
+        break;
+    default: exhip_set_error("exhip_channelwise_nhwc_f16: unknown op %d", op); return EXHIP_ERR_ARG;
     }
     EXHIP_LAUNCH_CHECK();
     return 0;

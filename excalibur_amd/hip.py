@@ -336,6 +336,13 @@ class Ctx:
         _check(lib().exhip_channelwise_f16(self.h, self.CHANNEL[op], x.ptr, y.ptr, n, c, h * w, p0.ptr, _ptr(p1), int(shared)))
         return y
 
+    def channelwise_nhwc_f16(self, op, x, p0, p1=None, shared=False):
+        n, h, w, c = x.shape
+        y = self.empty(x.shape, np.uint16)
+        _check(lib().exhip_channelwise_nhwc_f16(self.h, self.CHANNEL[op], x.ptr, y.ptr, ctypes.c_size_t(n * h * w), c, p0.ptr, _ptr(p1),
+                                                int(shared)))
+        return y
+
     def concat_channels_f32(self, inputs):
         n, _, h, w = inputs[0].shape
         ptrs = (ctypes.c_void_p * len(inputs))(*[a.ptr.value for a in inputs])

@@ -117,6 +117,7 @@ public:
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
     void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
+    void eltwise_general_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops);
 };
 
 template <typename Dtype>

@@ -3,6 +3,7 @@
 // blobs; the kernels' NHWC / int8 forms are produced and consumed inside each forward call.
 #include "../include/Excalibur/operators.hpp"
 
+#include <cstdlib>
 #include <cmath>
 #include <cstring>
 #include <random>
@@ -66,8 +67,8 @@ namespace {
 inline int pad_to(int v, int m) { return (v + m - 1) / m * m; }
 
 template <typename T>
-std::shared_ptr<tensor<T>> new_tensor(std::vector<int> shape, int device) {
-    return std::make_shared<tensor<T>>(shape, device, memory::NCHW, nullptr);
+std::shared_ptr<tensor<T>> new_tensor(std::vector<int> shape, int device, memory::orderType order = memory::NCHW) {
+    return std::make_shared<tensor<T>>(shape, device, order, nullptr);
 }
 
 // 1 x 1 x 1 x n vector blob (the reference's tensor(w, device, order, allocator) constructor)
@@ -109,6 +110,41 @@ int conv_in_stride(int c, int dtype, int kw) {
 
 void require_nchw(memory::orderType o) {
     if (o != memory::NCHW) LOG(FATAL) << "this backend takes NCHW blobs at the operator interface";
+}
+
+// The fp16 pipeline keeps blobs NHWC between the layers whose kernels work on that layout (convolution, depthwise,
+// pooling, the elementwise and per-channel layers): a blob of order NHWC has shape {n, h, w, c} (the reference's
+// convention for that order, include/Primitives/tensor.hpp:124-134), channel stride == c, c a multiple of 8. Every other
+// layer, and whoever reads a blob from outside, gets the NCHW form through as_nchw.
+using half_ptr = std::shared_ptr<tensor<unsigned short>>;
+// EXCALIBUR_F16_NCHW=1 (read at every call: tests switch it inside one process) keeps every blob NCHW, the form the
+// NHWC-resident one must agree with bit for bit.
+bool nhwc_allowed() {
+    const char* e = std::getenv("EXCALIBUR_F16_NCHW");
+    return !(e && std::atoi(e) != 0);
+}
+bool nhwc_channels_ok(int c) { return c % 8 == 0 && nhwc_allowed(); }
+
+half_ptr as_nchw(exhip_ctx* ctx, const half_ptr& t, int device) {
+    if (t->order() == memory::NCHW) return t;
+    auto out = new_tensor<unsigned short>({t->num(), t->channels(), t->height(), t->width()}, device);
+    EXHIP_FATAL(exhip_nhwc_f16_to_nchw_f16(ctx, t->gpu_data(), t->num(), t->channels(), t->height(), t->width(), t->channels(),
+                                           out->mutable_gpu_data()));
+    return out;
+}
+
+half_ptr as_order(exhip_ctx* ctx, const half_ptr& t, memory::orderType order, int device);
+
+half_ptr as_nhwc(exhip_ctx* ctx, const half_ptr& t, int device) {
+    if (t->order() == memory::NHWC) return t;
+    auto out = new_tensor<unsigned short>({t->num(), t->height(), t->width(), t->channels()}, device, memory::NHWC);
+    EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(ctx, t->gpu_data(), t->num(), t->channels(), t->height(), t->width(), t->channels(),
+                                           out->mutable_gpu_data()));
+    return out;
+}
+
+half_ptr as_order(exhip_ctx* ctx, const half_ptr& t, memory::orderType order, int device) {
+    return order == memory::NHWC ? as_nhwc(ctx, t, device) : as_nchw(ctx, t, device);
 }
 
 }  // namespace
@@ -384,29 +420,41 @@ template <typename Dtype>
 void operation_convolution<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
     CHECK_EQ(bottoms.size(), 1);
     CHECK_EQ(tops.size(), 1);
-    require_nchw(bottoms[0]->order());
     const int dev = this->params_.device_;
     const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
     CHECK_EQ(c, this->input_channels());
     exhip_conv_desc d = describe(n, h, w, c, this->output_channel_);
     int oh, ow;
     EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
-    tops[0] = new_tensor<unsigned short>({n, this->output_channel_, oh, ow}, dev);
     if (!mfma_path_ok()) {
         // definition-order kernel in float on converted tensors, result rounded to half
+        const half_ptr in = as_nchw(this->ctx(), bottoms[0], dev);
+        tops[0] = new_tensor<unsigned short>({n, this->output_channel_, oh, ow}, dev);
         auto xf = new_tensor<float>({n, c, h, w}, dev);
         auto yf = new_tensor<float>({n, this->output_channel_, oh, ow}, dev);
-        EXHIP_FATAL(exhip_f16_to_f32(this->ctx(), bottoms[0]->gpu_data(), xf->mutable_gpu_data(), xf->count()));
+        EXHIP_FATAL(exhip_f16_to_f32(this->ctx(), in->gpu_data(), xf->mutable_gpu_data(), xf->count()));
         EXHIP_FATAL(exhip_conv2d_direct_nchw(this->ctx(), &d, this->group_, xf->gpu_data(), this->weights_f32_[0]->gpu_data(), nullptr,
                                              1.f, nullptr, bias_gpu(), yf->mutable_gpu_data()));
         EXHIP_FATAL(exhip_f32_to_f16(this->ctx(), yf->gpu_data(), tops[0]->mutable_gpu_data(), yf->count()));
         return;
     }
+    // The kernel reads NHWC with the channel stride it wants (16 halves per 32-byte step) and writes NHWC, NCHW or both:
+    // an NHWC blob with such a stride goes in as it is, and the result stays NHWC where its channel count allows.
     d.c_stride = conv_in_stride(c, EXHIP_F16, d.kw);
-    auto x = new_tensor<unsigned short>({n, h, w, d.c_stride}, dev);
-    EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, d.c_stride, x->mutable_gpu_data()));
-    EXHIP_FATAL(exhip_conv2d_f16(this->ctx(), &d, x->gpu_data(), packed_weights(EXHIP_F16, d), bias_gpu(), nullptr, nullptr,
-                                 tops[0]->mutable_gpu_data(), nullptr));
+    half_ptr x;
+    if (bottoms[0]->order() == memory::NHWC && d.c_stride == c) {
+        x = bottoms[0];
+    } else {
+        const half_ptr in = as_nchw(this->ctx(), bottoms[0], dev);
+        x = new_tensor<unsigned short>({n, h, w, d.c_stride}, dev);
+        EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), in->gpu_data(), n, c, h, w, d.c_stride, x->mutable_gpu_data()));
+    }
+    const bool out_nhwc = this->output_channel_ % 16 == 0 && nhwc_allowed();
+    tops[0] = out_nhwc ? new_tensor<unsigned short>({n, oh, ow, this->output_channel_}, dev, memory::NHWC)
+                       : new_tensor<unsigned short>({n, this->output_channel_, oh, ow}, dev);
+    unsigned short* y = tops[0]->mutable_gpu_data();
+    EXHIP_FATAL(exhip_conv2d_f16(this->ctx(), &d, x->gpu_data(), packed_weights(EXHIP_F16, d), bias_gpu(), nullptr,
+                                 out_nhwc ? y : nullptr, out_nhwc ? nullptr : y, nullptr));
 }
 
 // ------------------------------------------------------------------ depthwise convolution
@@ -463,16 +511,24 @@ void operation_convolutiondepthwise<Dtype>::forward_gpu_f16(const tensor_list<un
         operation_convolution<Dtype>::forward_gpu_f16(bottoms, tops);
         return;
     }
-    require_nchw(bottoms[0]->order());
     const int dev = this->params_.device_;
     const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
     const int oh = (h + this->pad_top_ + this->pad_bottom_ - 3) / this->stride_h_ + 1;
     const int ow = (w + this->pad_left_ + this->pad_right_ - 3) / this->stride_w_ + 1;
+    if (nhwc_channels_ok(c)) {  // NHWC in, NHWC out
+        const half_ptr x = as_nhwc(this->ctx(), bottoms[0], dev);
+        tops[0] = new_tensor<unsigned short>({n, oh, ow, c}, dev, memory::NHWC);
+        EXHIP_FATAL(exhip_dwconv3x3_nhwc_f16(this->ctx(), x->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
+                                             tops[0]->mutable_gpu_data(), n, c, h, w, c, this->stride_h_, this->pad_top_,
+                                             this->pad_bottom_, this->pad_left_, this->pad_right_, this->activation_type_));
+        return;
+    }
+    const half_ptr in = as_nchw(this->ctx(), bottoms[0], dev);
     const int cs = pad_to(c, 8);
     auto x = new_tensor<unsigned short>({n, h, w, cs}, dev);
     auto y = new_tensor<unsigned short>({n, oh, ow, cs}, dev);
     tops[0] = new_tensor<unsigned short>({n, c, oh, ow}, dev);
-    EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, cs, x->mutable_gpu_data()));
+    EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), in->gpu_data(), n, c, h, w, cs, x->mutable_gpu_data()));
     EXHIP_FATAL(exhip_dwconv3x3_nhwc_f16(this->ctx(), x->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
                                          y->mutable_gpu_data(), n, c, h, w, cs, this->stride_h_, this->pad_top_, this->pad_bottom_,
                                          this->pad_left_, this->pad_right_, this->activation_type_));
@@ -535,15 +591,22 @@ void operation_pooling<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>
     CHECK_EQ(bottoms.size(), tops.size());
     const int dev = this->params_.device_;
     for (size_t i = 0; i < bottoms.size(); ++i) {
-        require_nchw(bottoms[i]->order());
         const int n = bottoms[i]->num(), c = bottoms[i]->channels(), h = bottoms[i]->height(), w = bottoms[i]->width();
         int kh, kw, sh, sw, pt, pb, pl, pr, oh, ow;
         geometry(h, w, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &oh, &ow);
+        if (nhwc_channels_ok(c)) {  // NHWC in, NHWC out
+            const half_ptr x = as_nhwc(this->ctx(), bottoms[i], dev);
+            tops[i] = new_tensor<unsigned short>({n, oh, ow, c}, dev, memory::NHWC);
+            EXHIP_FATAL(exhip_pool2d_nhwc_f16(this->ctx(), x->gpu_data(), tops[i]->mutable_gpu_data(), n, c, h, w, c, oh, ow, type_, kh,
+                                              kw, sh, sw, pt, pb, pl, pr, avgpool_count_include_pad_));
+            continue;
+        }
+        const half_ptr in = as_nchw(this->ctx(), bottoms[i], dev);
         const int cs = pad_to(c, 8);
         auto x = new_tensor<unsigned short>({n, h, w, cs}, dev);
         auto y = new_tensor<unsigned short>({n, oh, ow, cs}, dev);
         tops[i] = new_tensor<unsigned short>({n, c, oh, ow}, dev);
-        EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), bottoms[i]->gpu_data(), n, c, h, w, cs, x->mutable_gpu_data()));
+        EXHIP_FATAL(exhip_nchw_f16_to_nhwc_f16(this->ctx(), in->gpu_data(), n, c, h, w, cs, x->mutable_gpu_data()));
         EXHIP_FATAL(exhip_pool2d_nhwc_f16(this->ctx(), x->gpu_data(), y->mutable_gpu_data(), n, c, h, w, cs, oh, ow, type_, kh, kw, sh,
                                           sw, pt, pb, pl, pr, avgpool_count_include_pad_));
         EXHIP_FATAL(exhip_nhwc_f16_to_nchw_f16(this->ctx(), y->gpu_data(), n, c, oh, ow, cs, tops[i]->mutable_gpu_data()));
@@ -591,12 +654,21 @@ void operation_eltwise<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>
     CHECK_EQ(tops.size(), 1);
     const int dev = this->params_.device_;
     if (type_ == 1 && bottoms.size() == 2 && coeffs_[0] == 1.f && coeffs_[1] == 1.f) {  // the residual add, in one pass
-        CHECK(bottoms[1]->data_shape() == bottoms[0]->data_shape());
+        const half_ptr b1 = as_order(this->ctx(), bottoms[1], bottoms[0]->order(), dev);  // element by element: any common layout
+        CHECK(b1->data_shape() == bottoms[0]->data_shape());
         tops[0] = std::make_shared<tensor<unsigned short>>(bottoms[0]->data_shape(), dev, bottoms[0]->order());
-        EXHIP_FATAL(exhip_add_f16(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(),
-                                  tops[0]->count(), 0));
+        EXHIP_FATAL(exhip_add_f16(this->ctx(), bottoms[0]->gpu_data(), b1->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
         return;
     }
+    // the general form in NCHW: the SUM kernel reproduces a rounding that depends on an element's position in the blob
+    tensor_list<unsigned short> nchw;
+    for (const auto& b : bottoms) nchw.push_back(as_nchw(this->ctx(), b, dev));
+    eltwise_general_f16(nchw, tops);
+}
+
+template <typename Dtype>
+void operation_eltwise<Dtype>::eltwise_general_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    const int dev = this->params_.device_;
     tensor_list<float> f(bottoms.size());
     std::vector<const float*> in;
     for (size_t i = 0; i < bottoms.size(); ++i) {
@@ -665,12 +737,17 @@ void operation_binaryop<Dtype>::forward_gpu_f32(const tensor_list<float>& bottom
 template <typename Dtype>
 void operation_binaryop<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
     CHECK_EQ(tops.size(), 1);
-    if (op_type_ != 0 || with_scalar_ || bottoms.size() != 2 || bottoms[0]->data_shape() != bottoms[1]->data_shape()) {
+    const int dev = this->params_.device_;
+    const bool same_blob_shape = bottoms.size() == 2 && bottoms[0]->num() == bottoms[1]->num() &&
+                                 bottoms[0]->channels() == bottoms[1]->channels() && bottoms[0]->height() == bottoms[1]->height() &&
+                                 bottoms[0]->width() == bottoms[1]->width();
+    if (op_type_ != 0 || with_scalar_ || !same_blob_shape) {
         operation<Dtype>::forward_gpu_f16(bottoms, tops);  // everything but the residual add: convert, float kernel, convert back
         return;
     }
-    tops[0] = std::make_shared<tensor<unsigned short>>(bottoms[0]->data_shape(), this->params_.device_, bottoms[0]->order());
-    EXHIP_FATAL(exhip_add_f16(this->ctx(), bottoms[0]->gpu_data(), bottoms[1]->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
+    const half_ptr b1 = as_order(this->ctx(), bottoms[1], bottoms[0]->order(), dev);  // element by element: any common layout
+    tops[0] = std::make_shared<tensor<unsigned short>>(bottoms[0]->data_shape(), dev, bottoms[0]->order());
+    EXHIP_FATAL(exhip_add_f16(this->ctx(), bottoms[0]->gpu_data(), b1->gpu_data(), tops[0]->mutable_gpu_data(), tops[0]->count(), 0));
 }
 
 template <typename Dtype>
@@ -850,8 +927,9 @@ void operation_innerproduct<Dtype>::forward_gpu_f16(const tensor_list<unsigned s
     CHECK_EQ(tops.size(), 1);
     const int dev = this->params_.device_;
     tensor_list<float> fb(1), ft(1);
-    fb[0] = std::make_shared<tensor<float>>(bottoms[0]->data_shape(), dev, bottoms[0]->order());
-    EXHIP_FATAL(exhip_f16_to_f32(this->ctx(), bottoms[0]->gpu_data(), fb[0]->mutable_gpu_data(), fb[0]->count()));
+    const half_ptr in = as_nchw(this->ctx(), bottoms[0], dev);  // the flattening order is NCHW's
+    fb[0] = std::make_shared<tensor<float>>(in->data_shape(), dev, in->order());
+    EXHIP_FATAL(exhip_f16_to_f32(this->ctx(), in->gpu_data(), fb[0]->mutable_gpu_data(), fb[0]->count()));
     forward_gpu_f32(fb, ft);
     tops[0] = std::make_shared<tensor<unsigned short>>(ft[0]->data_shape(), dev, ft[0]->order());
     EXHIP_FATAL(exhip_f32_to_f16(this->ctx(), ft[0]->gpu_data(), tops[0]->mutable_gpu_data(), ft[0]->count()));
@@ -861,7 +939,8 @@ void operation_innerproduct<Dtype>::forward_gpu_f16(const tensor_list<unsigned s
 template <typename Dtype>
 void operation<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
     tensor_list<float> in32, out32(tops.size());
-    for (const auto& b : bottoms) {
+    for (const auto& blob : bottoms) {
+        const half_ptr b = as_nchw(ctx(), blob, params_.device_);  // the float layers take NCHW
         auto f = std::make_shared<tensor<float>>(b->data_shape(), params_.device_, b->order());
         EXHIP_FATAL(exhip_f16_to_f32(ctx(), b->gpu_data(), f->mutable_gpu_data(), f->count()));
         in32.push_back(f);
@@ -954,9 +1033,14 @@ void operation_prelu<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& 
     CHECK_EQ(bottoms.size(), tops.size());
     for (size_t i = 0; i < bottoms.size(); ++i) {
         const auto& b = bottoms[i];
-        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
         if (!share_channel_) CHECK_EQ(b->channels(), num_slope_);
         tops[i] = std::make_shared<tensor<unsigned short>>(b->data_shape(), this->params_.device_, b->order());
+        if (b->order() == memory::NHWC) {
+            EXHIP_FATAL(exhip_channelwise_nhwc_f16(this->ctx(), EXHIP_CHANNEL_PRELU, b->gpu_data(), tops[i]->mutable_gpu_data(),
+                                                   static_cast<size_t>(b->num()) * b->height() * b->width(), b->channels(),
+                                                   this->weights_f32_[0]->gpu_data(), nullptr, share_channel_ ? 1 : 0));
+            continue;
+        }
         EXHIP_FATAL(exhip_channelwise_f16(this->ctx(), EXHIP_CHANNEL_PRELU, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(), b->channels(),
                                           b->height() * b->width(), this->weights_f32_[0]->gpu_data(), nullptr, share_channel_ ? 1 : 0));
     }
@@ -1033,9 +1117,14 @@ void operation_batchnorm<Dtype>::forward_gpu_f16(const tensor_list<unsigned shor
     CHECK_EQ(bottoms.size(), tops.size());
     for (size_t i = 0; i < bottoms.size(); ++i) {
         const auto& b = bottoms[i];
-        if (b->order() != memory::NCHW) NOT_IMPLEMENTED;
         CHECK_EQ(b->channels(), channels_);
         tops[i] = std::make_shared<tensor<unsigned short>>(b->data_shape(), this->params_.device_, b->order());
+        if (b->order() == memory::NHWC) {
+            EXHIP_FATAL(exhip_channelwise_nhwc_f16(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(),
+                                                   static_cast<size_t>(b->num()) * b->height() * b->width(), b->channels(),
+                                                   a_->gpu_data(), b_->gpu_data(), 0));
+            continue;
+        }
         EXHIP_FATAL(exhip_channelwise_f16(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(),
                                           b->channels(), b->height() * b->width(), a_->gpu_data(), b_->gpu_data(), 0));
     }

@@ -12,6 +12,7 @@
 //    (+ shortcut add + ReLU) and writing what its consumers read. Same values as the per-layer executor.
 #include "../include/Excalibur/pipeline.hpp"
 
+#include <type_traits>
 #include <chrono>
 #include <cmath>
 #include <cstring>
@@ -159,7 +160,20 @@ public:
     tensor_ptr get_featmap(std::string_view name) {
         auto it = blob_index_.find(std::string(name));
         if (it == blob_index_.end()) return nullptr;
-        return featmaps_[it->second];
+        return nchw(featmaps_[it->second]);
+    }
+
+    // The fp16 layers pass NHWC blobs among themselves; what leaves the pipeline is NCHW as in the reference.
+    tensor_ptr nchw(const tensor_ptr& t) const {
+        if constexpr (std::is_same_v<Dtype, unsigned short>) {
+            if (t && t->order() == memory::NHWC) {
+                auto out = std::make_shared<tensor<Dtype>>(std::vector<int>{t->num(), t->channels(), t->height(), t->width()}, device_);
+                EXHIP_FATAL(exhip_nhwc_f16_to_nchw_f16(memory::device_context(device_), t->gpu_data(), t->num(), t->channels(),
+                                                       t->height(), t->width(), t->channels(), out->mutable_gpu_data()));
+                return out;
+            }
+        }
+        return t;
     }
 
     bool profile_ = false;
@@ -185,7 +199,11 @@ private:
             for (size_t j = 0; j < out.size(); ++j) featmaps_[op_outputs_[i][j]] = out[j];
         }
         blob_map results;
-        for (const std::string& o : output_names_) results[o] = featmaps_[blob_index_[o]];
+        for (const std::string& o : output_names_) {
+            tensor_ptr& blob = featmaps_[blob_index_[o]];
+            blob = nchw(blob);
+            results[o] = blob;
+        }
         return results;
     }
 

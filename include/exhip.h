@@ -212,6 +212,10 @@ int exhip_channelwise_f32(exhip_ctx* ctx, int op, const float* x, float* y, int 
 /* The same on half storage (float parameters and arithmetic, one rounding to half). */
 int exhip_channelwise_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, int n, int c, int hw, const float* p0,
                           const float* p1, int shared);
+/* ... and on NHWC half storage with channel stride == c (a multiple of 8): the layout the fp16 pipeline keeps between
+ * its convolution, depthwise and pooling layers. */
+int exhip_channelwise_nhwc_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, size_t pixels, int c,
+                               const float* p0, const float* p1, int shared);
 /* operation_concat::forward_cpu_f32 along the channel axis (operation_concat.cpp:31-103): inputs is a host array of
  * device pointers to NCHW tensors [n][channels[i]][hw]. */
 int exhip_concat_channels_f32(exhip_ctx* ctx, const float* const* inputs, const int* channels, int n_inputs, int n, int hw,

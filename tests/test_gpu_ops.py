@@ -371,6 +371,26 @@ def test_channelwise_half_storage_bit_exact(ctx, shape):
     assert np.array_equal(got, _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.uint16))
 
 
+def test_channelwise_nhwc_half_storage_bit_exact(ctx):
+    """PReLU and BatchNorm on the NHWC half tensors the fp16 pipeline keeps between layers == the NCHW layer transposed."""
+    shape = (2, 16, 9, 11)
+    for shared in (False, True):
+        case = cases.prelu_case(331, shape, shared)
+        x16 = _half(case["x"])
+        want = _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.uint16).transpose(0, 2, 3, 1)
+        xd = ctx.array(np.ascontiguousarray(x16.view(np.uint16).transpose(0, 2, 3, 1)))
+        got = ctx.channelwise_nhwc_f16("prelu", xd, ctx.array(case["slope"]), shared=shared).download()
+        assert np.array_equal(got, want)
+    case = cases.batchnorm_case(332, shape)
+    x16 = _half(case["x"])
+    sqrt_var = np.sqrt((case["var"] + np.float32(case["eps"])).astype(np.float64)).astype(np.float32)
+    a = (case["bias"] - case["slope"] * case["mean"] / sqrt_var).astype(np.float32)
+    b = (case["slope"] / sqrt_var).astype(np.float32)
+    want = _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.uint16).transpose(0, 2, 3, 1)
+    xd = ctx.array(np.ascontiguousarray(x16.view(np.uint16).transpose(0, 2, 3, 1)))
+    assert np.array_equal(ctx.channelwise_nhwc_f16("batchnorm", xd, ctx.array(a), ctx.array(b)).download(), want)
+
+
 @pytest.mark.parametrize("etype,n,coeffs", [(1, 2, None), (1, 3, [0.5, -1.25, 2.0]), (2, 3, None), (0, 3, None)])
 def test_eltwise_bit_exact(ctx, etype, n, coeffs):
     case = cases.eltwise_case(320 + etype, (2, 16, 21, 23), etype, n, coeffs)
