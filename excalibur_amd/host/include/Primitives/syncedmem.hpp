@@ -31,7 +31,7 @@ public:
 
 private:
     void to_cpu();
-    void to_gpu();
+    void to_gpu(bool will_overwrite);
     Dtype* cpu_ptr_ = nullptr;
     Dtype* gpu_ptr_ = nullptr;
     size_t size_;

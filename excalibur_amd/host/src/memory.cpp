@@ -66,11 +66,9 @@ syncedmem<Dtype>::syncedmem(size_t size, int device) : size_(size), device_(devi
 template <typename Dtype>
 syncedmem<Dtype>::~syncedmem() {
     if (cpu_ptr_) std::free(cpu_ptr_);
-    if (gpu_ptr_) {
-        // kernels reading this buffer may still be queued: recycle only after the stream has drained
-        exhip_sync(device_context(device_));
-        device_release(device_, gpu_ptr_, size_ * sizeof(Dtype));
-    }
+    // Kernels using this buffer may still be queued, and that is fine: every device operation of a device (kernels,
+    // copies, fills) goes through that device's one stream, so whatever touches a recycled block is queued behind them.
+    if (gpu_ptr_) device_release(device_, gpu_ptr_, size_ * sizeof(Dtype));
 }
 
 template <typename Dtype>
@@ -91,15 +89,18 @@ void syncedmem<Dtype>::to_cpu() {
     }
 }
 
+// will_overwrite: the caller asks for the buffer to write all of it (mutable_gpu_data of a fresh blob, which is how every
+// layer makes its output): the zero fill the reference gives a fresh blob is then skipped. Reading a blob nobody wrote
+// (gpu_data first) still yields zeros.
 template <typename Dtype>
-void syncedmem<Dtype>::to_gpu() {
+void syncedmem<Dtype>::to_gpu(bool will_overwrite) {
     if (device_ < 0) LOG(FATAL) << "gpu_data() on a tensor created without a device";
     const size_t bytes = size_ * sizeof(Dtype);
     exhip_ctx* ctx = device_context(device_);
     switch (head_) {
     case UNINITIALIZED:
         gpu_ptr_ = static_cast<Dtype*>(device_alloc(device_, bytes));
-        EXHIP_FATAL(exhip_memset(ctx, gpu_ptr_, 0, bytes));
+        if (!will_overwrite) EXHIP_FATAL(exhip_memset(ctx, gpu_ptr_, 0, bytes));
         head_ = HEAD_AT_GPU;
         break;
     case HEAD_AT_CPU:
@@ -114,11 +115,11 @@ void syncedmem<Dtype>::to_gpu() {
 template <typename Dtype>
 const Dtype* syncedmem<Dtype>::cpu_data() { to_cpu(); return cpu_ptr_; }
 template <typename Dtype>
-const Dtype* syncedmem<Dtype>::gpu_data() { to_gpu(); return gpu_ptr_; }
+const Dtype* syncedmem<Dtype>::gpu_data() { to_gpu(false); return gpu_ptr_; }
 template <typename Dtype>
 Dtype* syncedmem<Dtype>::mutable_cpu_data() { to_cpu(); head_ = HEAD_AT_CPU; return cpu_ptr_; }
 template <typename Dtype>
-Dtype* syncedmem<Dtype>::mutable_gpu_data() { to_gpu(); head_ = HEAD_AT_GPU; return gpu_ptr_; }
+Dtype* syncedmem<Dtype>::mutable_gpu_data() { to_gpu(true); head_ = HEAD_AT_GPU; return gpu_ptr_; }
 
 template <typename Dtype>
 void tensor<Dtype>::init(const std::vector<int>& shape, int device) {
