@@ -1195,6 +1195,71 @@ __global__ __launch_bounds__(kBlock) void concat_block_v4_kernel(const v4f* __re
         y[img * out_image4 + out_offset4 + j] = x[img * block4 + j];
 }
 
+// Channel concatenation of NHWC half blobs (every channel count a multiple of 8): a thread moves one 16-byte vector of
+// one output pixel; `first[i]` is the first output channel of input i.
+struct ConcatNhwcArgs {
+    const uint16_t* src[8];
+    int first[9];  // first[n_inputs] = total channels
+    int n_inputs;
+};
+__global__ __launch_bounds__(kBlock) void concat_nhwc_f16_kernel(ConcatNhwcArgs a, uint16_t* __restrict__ y, size_t total8) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total8) return;
+    const int vecs = a.first[a.n_inputs] / 8;
+    const int v = (int)(i % vecs);
+    const size_t pix = i / vecs;
+    const int c = v * 8;
+    int k = 0;
+#pragma unroll
+    for (int j = 1; j < 8; ++j)
+        if (j < a.n_inputs && c >= a.first[j]) k = j;
+    const int ck = a.first[k + 1] - a.first[k];
+    reinterpret_cast<v4i*>(y)[i] = *reinterpret_cast<const v4i*>(a.src[k] + pix * ck + (c - a.first[k]));
+}
+
+// Nearest-neighbour resize of an NHWC half blob (channels a multiple of 8), the index rule of the NCHW kernel below.
+__global__ __launch_bounds__(kBlock) void interp_nearest_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                                         int H, int W, int C8, int OH, int OW, float hs, float ws,
+                                                                         size_t total8) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total8) return;
+    const int v = (int)(i % C8);
+    size_t t = i / C8;
+    const int ox = (int)(t % OW);
+    t /= OW;
+    const int oy = (int)(t % OH);
+    const size_t n = t / OH;
+    int iy = (int)(oy * hs), ix = (int)(ox * ws);
+    iy = iy > H - 1 ? H - 1 : iy;
+    ix = ix > W - 1 ? W - 1 : ix;
+    reinterpret_cast<v4i*>(y)[i] = reinterpret_cast<const v4i*>(x)[((n * H + iy) * W + ix) * C8 + v];
+}
+
+// One direction of a stride-1 "same" max pooling on NHWC half storage (window K, padding K / 2, taps outside the image
+// do not count): the K x K maximum is the maximum over rows of the maxima over columns, so two launches of 2K taps
+// replace K * K. ALONG_W: the window runs along x, else along y.
+template <int K, bool ALONG_W>
+__global__ __launch_bounds__(kBlock) void maxpool_same_1d_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                                          int H, int W, int C8, size_t total8) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total8) return;
+    const int v = (int)(i % C8);
+    size_t t = i / C8;
+    const int ox = (int)(t % W);
+    t /= W;
+    const int oy = (int)(t % H);
+    const size_t n = t / H;
+    const _Float16 ninf = -__builtin_inff16();
+    v8h best = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+#pragma unroll
+    for (int d = -(K / 2); d <= K / 2; ++d) {
+        const int iy = ALONG_W ? oy : oy + d, ix = ALONG_W ? ox + d : ox;
+        if ((unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W)
+            best = __builtin_elementwise_max(best, __builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(x)[((n * H + iy) * W + ix) * C8 + v]));
+    }
+    reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, best);
+}
+
 // Nearest-neighbour resize: in = min((int)(out * scale), size - 1), scale = size / (float)out_size.
 __global__ __launch_bounds__(kBlock) void interp_nearest_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W,
                                                                 int OH, int OW, float hs, float ws, size_t total) {
@@ -1966,6 +2031,63 @@ extern "C" int exhip_channelwise_f16(exhip_ctx* ctx, int op, const uint16_t* x, 
     case EXHIP_CHANNEL_INPUT: launch_channelwise_f16<2>(ctx, x, y, n, c, hw, p0, p1, 0); break;
     default: exhip_set_error("exhip_channelwise_f16: unknown op %d", op); return EXHIP_ERR_ARG;
     }
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_concat_channels_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs, const int* channels, int n_inputs,
+                                              size_t pixels, uint16_t* y) {
+    REQ_CTX("exhip_concat_channels_nhwc_f16");
+    EXHIP_REQUIRE(inputs && channels && y && n_inputs >= 1 && n_inputs <= 8 && pixels > 0, "exhip_concat_channels_nhwc_f16: bad argument");
+    ConcatNhwcArgs a = {};
+    a.n_inputs = n_inputs;
+    int total = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        EXHIP_REQUIRE(inputs[i] && channels[i] > 0 && channels[i] % 8 == 0 && (reinterpret_cast<uintptr_t>(inputs[i]) & 15) == 0,
+                      "exhip_concat_channels_nhwc_f16: input %d needs a multiple of 8 channels and 16-byte alignment", i);
+        a.src[i] = inputs[i];
+        a.first[i] = total;
+        total += channels[i];
+    }
+    a.first[n_inputs] = total;
+    EXHIP_REQUIRE((reinterpret_cast<uintptr_t>(y) & 15) == 0, "exhip_concat_channels_nhwc_f16: output must be 16-byte aligned");
+    const size_t total8 = pixels * (size_t)(total / 8);
+    hipLaunchKernelGGL(concat_nhwc_f16_kernel, dim3(blocks_for(total8)), dim3(kBlock), 0, ctx->stream, a, y, total8);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_interp_nearest_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int oh,
+                                             int ow) {
+    REQ_CTX("exhip_interp_nearest_nhwc_f16");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && c % 8 == 0 && h > 0 && w > 0 && oh > 0 && ow > 0, "exhip_interp_nearest_nhwc_f16: bad argument");
+    EXHIP_REQUIRE((reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0,
+                  "exhip_interp_nearest_nhwc_f16: tensors must be 16-byte aligned");
+    const size_t total8 = (size_t)n * oh * ow * (c / 8);
+    hipLaunchKernelGGL(interp_nearest_nhwc_f16_kernel, dim3(blocks_for(total8)), dim3(kBlock), 0, ctx->stream, x, y, h, w, c / 8, oh, ow,
+                       h / (float)oh, w / (float)ow, total8);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_maxpool_same_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* tmp, uint16_t* y, int n, int c, int h, int w,
+                                           int k) {
+    REQ_CTX("exhip_maxpool_same_nhwc_f16");
+    EXHIP_REQUIRE(x && tmp && y && n > 0 && c > 0 && c % 8 == 0 && h > 0 && w > 0, "exhip_maxpool_same_nhwc_f16: bad argument");
+    EXHIP_REQUIRE(k == 5 || k == 9 || k == 13, "exhip_maxpool_same_nhwc_f16: window %d (5, 9 or 13)", k);
+    EXHIP_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(tmp) | reinterpret_cast<uintptr_t>(y)) & 15) == 0,
+                  "exhip_maxpool_same_nhwc_f16: tensors must be 16-byte aligned");
+    const size_t total8 = (size_t)n * h * w * (c / 8);
+    const dim3 grid(blocks_for(total8)), block(kBlock);
+#define EXHIP_SAME_POOL(K)                                                                                                   \
+    do {                                                                                                                     \
+        hipLaunchKernelGGL((maxpool_same_1d_nhwc_f16_kernel<K, true>), grid, block, 0, ctx->stream, x, tmp, h, w, c / 8, total8); \
+        hipLaunchKernelGGL((maxpool_same_1d_nhwc_f16_kernel<K, false>), grid, block, 0, ctx->stream, tmp, y, h, w, c / 8, total8); \
+    } while (0)
+    if (k == 5) EXHIP_SAME_POOL(5);
+    else if (k == 9) EXHIP_SAME_POOL(9);
+    else EXHIP_SAME_POOL(13);
+#undef EXHIP_SAME_POOL
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

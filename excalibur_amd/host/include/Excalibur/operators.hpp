@@ -284,6 +284,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 
 // src/Excalibur/operation_concat.cpp:10-103: key 0 = axis - 2 (the files carry -1 for the channel axis).
@@ -298,6 +299,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 
 // src/Excalibur/operation_interp.cpp:185-268: keys 0 = type (1 nearest), 1 -> width scale, 2 -> height scale,
@@ -314,6 +316,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 
 // src/Excalibur/operation_yolov5focus.cpp:12-50.

@@ -597,6 +597,13 @@ void operation_pooling<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>
         if (nhwc_channels_ok(c)) {  // NHWC in, NHWC out
             const half_ptr x = as_nhwc(this->ctx(), bottoms[i], dev);
             tops[i] = new_tensor<unsigned short>({n, oh, ow, c}, dev, memory::NHWC);
+            if (type_ == 0 && kh == kw && (kh == 5 || kh == 9 || kh == 13) && sh == 1 && sw == 1 && pt == kh / 2 && pb == kh / 2 &&
+                pl == kh / 2 && pr == kh / 2 && oh == h && ow == w) {  // the detection topologies' 5 / 9 / 13 pyramid: rows, then columns
+                auto tmp = new_tensor<unsigned short>({n, h, w, c}, dev, memory::NHWC);
+                EXHIP_FATAL(exhip_maxpool_same_nhwc_f16(this->ctx(), x->gpu_data(), tmp->mutable_gpu_data(), tops[i]->mutable_gpu_data(), n,
+                                                        c, h, w, kh));
+                continue;
+            }
             EXHIP_FATAL(exhip_pool2d_nhwc_f16(this->ctx(), x->gpu_data(), tops[i]->mutable_gpu_data(), n, c, h, w, c, oh, ow, type_, kh,
                                               kw, sh, sw, pt, pb, pl, pr, avgpool_count_include_pad_));
             continue;
@@ -1176,6 +1183,29 @@ void operation_input<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, 
 }
 
 template <typename Dtype>
+void operation_input<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), tops.size());
+    for (size_t i = 0; i < bottoms.size(); ++i) {
+        const half_ptr b = as_nchw(this->ctx(), bottoms[i], this->params_.device_);
+        const int ch = b->channels();
+        if (ch != 1 && ch != 3) LOG(FATAL) << "Un-supprted channel num: " << ch;
+        CHECK_EQ(static_cast<size_t>(ch), means_.size());
+        CHECK_GE(vars_.size(), static_cast<size_t>(ch));
+        if (!means_dev_) {
+            means_dev_ = vec_tensor<float>(ch, this->params_.device_);
+            vars_dev_ = vec_tensor<float>(ch, this->params_.device_);
+            for (int c = 0; c < ch; ++c) {
+                means_dev_->mutable_cpu_data()[c] = means_[c];
+                vars_dev_->mutable_cpu_data()[c] = vars_[c];
+            }
+        }
+        tops[i] = std::make_shared<tensor<unsigned short>>(b->data_shape(), this->params_.device_, b->order());
+        EXHIP_FATAL(exhip_channelwise_f16(this->ctx(), EXHIP_CHANNEL_INPUT, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(), ch,
+                                          b->height() * b->width(), means_dev_->gpu_data(), vars_dev_->gpu_data(), 0));
+    }
+}
+
+template <typename Dtype>
 operation_concat<Dtype>::operation_concat(const operation_param& param) : operation<Dtype>(param) {
     for (const layer_attr& a : parse_attrs(param.specific_params_)) {
         const int key = std::atoi(a.key.c_str());
@@ -1208,6 +1238,37 @@ void operation_concat<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms,
 }
 
 template <typename Dtype>
+void operation_concat<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_GE(bottoms.size(), 2);
+    CHECK_EQ(tops.size(), 1);
+    bool nhwc = axis_ + 2 == 1 && bottoms.size() <= 8;
+    for (const auto& b : bottoms) nhwc = nhwc && nhwc_channels_ok(b->channels());
+    if (!nhwc) {
+        operation<Dtype>::forward_gpu_f16(bottoms, tops);  // convert, float kernel, convert back
+        return;
+    }
+    const int dev = this->params_.device_;
+    tensor_list<unsigned short> in;
+    std::vector<const unsigned short*> ptrs;
+    std::vector<int> channels;
+    int total = 0;
+    for (const auto& blob : bottoms) {
+        const half_ptr b = as_nhwc(this->ctx(), blob, dev);
+        CHECK_EQ(b->num(), bottoms[0]->num());
+        CHECK_EQ(b->height(), bottoms[0]->height());
+        CHECK_EQ(b->width(), bottoms[0]->width());
+        in.push_back(b);
+        ptrs.push_back(b->gpu_data());
+        channels.push_back(b->channels());
+        total += b->channels();
+    }
+    const auto& b0 = in[0];
+    tops[0] = new_tensor<unsigned short>({b0->num(), b0->height(), b0->width(), total}, dev, memory::NHWC);
+    EXHIP_FATAL(exhip_concat_channels_nhwc_f16(this->ctx(), ptrs.data(), channels.data(), static_cast<int>(ptrs.size()),
+                                               static_cast<size_t>(b0->num()) * b0->height() * b0->width(), tops[0]->mutable_gpu_data()));
+}
+
+template <typename Dtype>
 operation_interp<Dtype>::operation_interp(const operation_param& param) : operation<Dtype>(param) {
     for (const layer_attr& a : parse_attrs(param.specific_params_)) {
         switch (std::atoi(a.key.c_str())) {
@@ -1236,6 +1297,27 @@ void operation_interp<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms,
     tops[0] = new_tensor<float>({b->num(), b->channels(), oh, ow}, this->params_.device_);
     EXHIP_FATAL(exhip_interp_nearest_f32(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num(), b->channels(), b->height(),
                                          b->width(), oh, ow));
+}
+
+template <typename Dtype>
+void operation_interp<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const auto& blob = bottoms[0];
+    if (resize_type_ != 1 || align_corner_ != 0 || !nhwc_channels_ok(blob->channels())) {
+        operation<Dtype>::forward_gpu_f16(bottoms, tops);  // convert, float kernel, convert back
+        return;
+    }
+    const int dev = this->params_.device_;
+    const half_ptr b = as_nhwc(this->ctx(), blob, dev);
+    int oh = output_height_, ow = output_width_;
+    if (oh == 0 || ow == 0) {
+        oh = static_cast<int>(b->height() * height_scale_);
+        ow = static_cast<int>(b->width() * width_scale_);
+    }
+    tops[0] = new_tensor<unsigned short>({b->num(), oh, ow, b->channels()}, dev, memory::NHWC);
+    EXHIP_FATAL(exhip_interp_nearest_nhwc_f16(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num(), b->channels(),
+                                              b->height(), b->width(), oh, ow));
 }
 
 template <typename Dtype>

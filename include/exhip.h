@@ -216,6 +216,14 @@ int exhip_channelwise_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y
  * its convolution, depthwise and pooling layers. */
 int exhip_channelwise_nhwc_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, size_t pixels, int c,
                                const float* p0, const float* p1, int shared);
+/* Layers that only move or compare values, on those NHWC half blobs (channel counts multiples of 8): Concat along the
+ * channels (src/Excalibur/operation_concat.cpp:31-103; inputs: host array of up to 8 device pointers), nearest Interp
+ * (operation_interp.cpp:247-268) and the stride-1 max pooling with window k = 5 / 9 / 13 and padding k / 2 of the
+ * detection topologies (operation_pooling.cpp:145-159), as a row pass into tmp (same size as x) and a column pass. */
+int exhip_concat_channels_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs, const int* channels, int n_inputs,
+                                   size_t pixels, uint16_t* y);
+int exhip_interp_nearest_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int oh, int ow);
+int exhip_maxpool_same_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* tmp, uint16_t* y, int n, int c, int h, int w, int k);
 /* operation_concat::forward_cpu_f32 along the channel axis (operation_concat.cpp:31-103): inputs is a host array of
  * device pointers to NCHW tensors [n][channels[i]][hw]. */
 int exhip_concat_channels_f32(exhip_ctx* ctx, const float* const* inputs, const int* channels, int n_inputs, int n, int hw,

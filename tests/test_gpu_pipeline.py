@@ -389,21 +389,28 @@ def test_yolov5_shaped_float_topology_matches_the_reference_fixture():
         os.unlink(path)
 
 
-def test_fp16_pipeline_nhwc_resident_equals_nchw_blobs(monkeypatch):
+@pytest.mark.parametrize("which", ["mobilefacenet", "yolov5"])
+def test_fp16_pipeline_nhwc_resident_equals_nchw_blobs(monkeypatch, which):
     """pipeline<unsigned short> keeps blobs NHWC between its convolution, depthwise, pooling, elementwise and per-channel
     layers; with that switched off every blob is NCHW as in the reference. Layer by layer the arithmetic is the same, so
     the two agree bit for bit: on the output and on blobs in the middle, which come out of the pipeline as NCHW."""
-    from excalibur_amd.mobilenet import MobileFaceNetF32
-    net = MobileFaceNetF32(seed=5, hw=32, width=16, blocks=((2, 16, 2), (1, 16, 2), (2, 32, 4)), embed=32)
-    x = np.random.default_rng(6).uniform(0, 255, (3, 3, 32, 32)).astype(np.float32)
+    if which == "mobilefacenet":
+        from excalibur_amd.mobilenet import MobileFaceNetF32
+        net = MobileFaceNetF32(seed=5, hw=32, width=16, blocks=((2, 16, 2), (1, 16, 2), (2, 32, 4)), embed=32)
+        outputs, kinds = [net.output], ("ConvolutionDepthWise", "PReLU", "Eltwise")
+    else:  # Focus, Concat, nearest Interp, the 5 / 9 / 13 pooling pyramid, heads whose channel count is no multiple of 8
+        from excalibur_amd.yolo import YoloV5ShapedF32
+        net = YoloV5ShapedF32(seed=7, hw=64, width=8)
+        outputs, kinds = list(net.outputs), ("Concat", "Interp", "Pooling", "HardSwish")
+    x = np.random.default_rng(6).uniform(0, 255, (3, 3, net.hw, net.hw)).astype(np.float32)
     x16 = x.astype(np.float16).view(np.uint16)
     with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
         path = f.name
     try:
         net.write_model(path)
-        names = [net.output]
+        names = outputs
         # the first output blob of a few layers in the middle (line: type name n_in n_out bottoms... tops... keys)
-        middle = [l.split()[4 + int(l.split()[2])] for l in net.lines if l.split()[0] in ("ConvolutionDepthWise", "PReLU", "Eltwise")][:8]
+        middle = [l.split()[4 + int(l.split()[2])] for l in net.lines if l.split()[0] in kinds][:12]
         got = {}
         for flag in ("0", "1"):
             monkeypatch.setenv("EXCALIBUR_F16_NCHW", flag)
