@@ -55,3 +55,26 @@ __device__ __forceinline__ float exhip_act(float v, int act) {
 
 __device__ __forceinline__ float exhip_h2f(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t exhip_f2h(float f) { return __builtin_bit_cast(uint16_t, (_Float16)f); }
+
+// One value of an elementwise activation. OP 0 HardSwish, 1 LeakyReLU, 2 sigmoid, 3 HardSigmoid, 4 Clip; the multiply-adds
+// are fused where the CPU path's are (vector fmadd, and scalar expressions contracted by its compiler flags).
+template <int OP>
+__device__ __forceinline__ float unary_value(float x, float alpha, float beta) {
+    if constexpr (OP == 0) {
+        float t = __builtin_fmaf(x, alpha, beta);
+        t = t > 0.f ? t : 0.f;
+        t = t < 1.f ? t : 1.f;
+        return t * x;
+    } else if constexpr (OP == 1) {
+        return x < 0.f ? alpha * x : x;
+    } else if constexpr (OP == 2) {
+        return (float)(1. / (1. + exp(-(double)x)));
+    } else if constexpr (OP == 3) {
+        float t = __builtin_fmaf(alpha, x, beta);
+        t = 1.f < t ? 1.f : t;
+        return 0.f < t ? t : 0.f;
+    } else {
+        const float t = beta < x ? beta : x;  // clip to [alpha, beta]
+        return alpha < t ? t : alpha;
+    }
+}

@@ -86,6 +86,8 @@ struct ConvParams {
     int RS, n_rg;             // filter rows per stage, stages per chunk
     int tiles_x, tiles_y, ktiles;
     int act, post_relu;
+    int post_op;              // 0, or 1 + EXHIP_UNARY_*: the activation layer behind the convolution (general epilogue)
+    float post_alpha, post_beta;
     float fs_out;
     int b_align;              // alignment of B fragment reads in packed-row form (4, 8 or 16)
     unsigned img_bytes;       // bytes of one input image (buffer range for the bounds-checked loads)
@@ -203,6 +205,28 @@ __device__ __forceinline__ void wait_vmcnt(int keep) {
         : "=&s"(entry)
         : "s"(k)
         : "vcc", "scc", "memory");
+}
+
+// The activation layer behind a convolution, applied in the convolution's epilogue to the values this layer would have
+// stored: halves in the fp16 pipeline, so each value is rounded to half and widened again first. The sigmoid layer
+// (double-precision exp) stays a layer of its own.
+template <int OP, int DT>
+__device__ __forceinline__ void post_activation_op(float (&v)[16], float alpha, float beta) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        float t = v[e];
+        if constexpr (DT == EXHIP_F16) t = exhip_h2f(exhip_f2h(t));
+        v[e] = unary_value<OP>(t, alpha, beta);
+    }
+}
+template <int DT>
+__device__ __forceinline__ void post_activation(float (&v)[16], int op, float alpha, float beta) {
+    switch (op) {
+    case EXHIP_UNARY_HARDSWISH: post_activation_op<0, DT>(v, alpha, beta); break;
+    case EXHIP_UNARY_LEAKYRELU: post_activation_op<1, DT>(v, alpha, beta); break;
+    case EXHIP_UNARY_HARDSIGMOID: post_activation_op<3, DT>(v, alpha, beta); break;
+    default: post_activation_op<4, DT>(v, alpha, beta); break;
+    }
 }
 
 // KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
@@ -1033,9 +1057,15 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                     }
                 }
                 if (p.post_relu) {
+                    // a ReLU layer reads what this layer stored: in the fp16 pipeline the rounded half (a tiny negative
+                    // value is -0 there and stays -0)
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) v[e] = (0.f > v[e]) ? 0.f : v[e];
+                    for (int e = 0; e < 16; ++e) {
+                        if constexpr (DT == EXHIP_F16) v[e] = exhip_h2f(exhip_f2h(v[e]));
+                        v[e] = (0.f > v[e]) ? 0.f : v[e];
+                    }
                 }
+                if (p.post_op) post_activation<DT>(v, p.post_op - 1, p.post_alpha, p.post_beta);
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
@@ -1441,8 +1471,8 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     if constexpr (DT == EXHIP_I8) {
         if (!pool) {
             const long long elems = (long long)d->n * pl.OH * pl.OW * d->k;
-            const bool fused = !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 && elems * 4 < 0xFFFFF000ll &&
-                               elems < (long long)kEpiInvalid;
+            const bool fused = !p.acc_nchw && !d->post_op && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
+                               elems * 4 < 0xFFFFF000ll && elems < (long long)kEpiInvalid;
             const int epi_wave_b = !fused ? 0 : ((p.residual || p.y_nhwc) ? kEpiWaveBytes : 32 * kEpiRowQ + 128);
             rebuffer(pl, d, epi_wave_b, fused && pl.KWe == 3);
         }
@@ -1464,6 +1494,9 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.n_chunks = pl.n_chunks; p.chunk_b = pl.chunk_b; p.RS = pl.RS; p.n_rg = pl.n_rg;
     p.tiles_x = pl.tiles_x; p.tiles_y = pl.tiles_y; p.ktiles = pl.ktiles;
     p.act = d->act; p.post_relu = d->post_relu; p.fs_out = d->fs_out; p.b_align = pl.b_align;
+    p.post_op = d->post_op; p.post_alpha = d->post_alpha; p.post_beta = d->post_beta;
+    EXHIP_REQUIRE(d->post_op >= 0 && d->post_op <= 1 + EXHIP_UNARY_CLIP && d->post_op != 1 + EXHIP_UNARY_SIGMOID,
+                  "conv: post_op %d is not an activation the epilogue applies", d->post_op);
     p.dbg = (kStamps && getenv("EXHIP_DEBUG_STAMPS")) ? (long long*)strtoull(getenv("EXHIP_DEBUG_STAMPS"), nullptr, 0) : nullptr;
     p.img_bytes = (unsigned)((size_t)d->h * d->w * p.cstride_b);
     p.magic_iw = (unsigned)(((1ull << 32) + pl.IW - 1) / pl.IW);
@@ -1493,7 +1526,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         }
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
-        const bool fused = !p.acc_nchw && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
+        const bool fused = !p.acc_nchw && !d->post_op && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
                            out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
         if (fused) {
             p.epi_mode = 1;
@@ -1583,7 +1616,7 @@ extern "C" int exhip_conv2d_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_des
     EXHIP_REQUIRE(d && scale, "exhip_conv2d_i8_maxpool3x3s2: NULL descriptor or scale");
     EXHIP_REQUIRE(y_i8 || y_f32_nhwc, "exhip_conv2d_i8_maxpool3x3s2: no output requested");
     EXHIP_REQUIRE(d->k % 64 == 0 && d->k_stride == d->k, "conv+pool: needs k %% 64 == 0 and k_stride == k (k %d, k_stride %d)", d->k, d->k_stride);
-    EXHIP_REQUIRE(d->act <= 1 && !d->post_relu, "conv+pool: activation must be none or ReLU");
+    EXHIP_REQUIRE(d->act <= 1 && !d->post_relu && !d->post_op, "conv+pool: activation must be none or ReLU");
     int oh = 0, ow = 0;
     int rc = exhip_conv_out_hw(d, &oh, &ow);
     if (rc) return rc;

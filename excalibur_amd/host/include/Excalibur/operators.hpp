@@ -54,12 +54,19 @@ public:
     // weights packed for the MFMA kernel for one input geometry; cached per (dtype, n, h, w, c_stride)
     const void* packed_weights(int dtype, const exhip_conv_desc& d);
     exhip_conv_desc describe(int n, int h, int w, int c_stride, int k_stride) const;
+    // The activation layer behind this one, applied in the kernel's epilogue by the next forward calls: post_op 0 = none,
+    // else 1 + EXHIP_UNARY_* with its two parameters; relu = a ReLU layer. False, and nothing set, where this layer's
+    // kernel cannot apply it (the definition-order kernel of grouped layers, the sigmoid's double-precision exp).
+    virtual bool set_post_activation(int post_op, float alpha, float beta, bool relu);
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
     void forward_gpu_i8(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
     void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
     bool mfma_path_ok() const;
+    int post_op_ = 0;
+    float post_alpha_ = 0.f, post_beta_ = 0.f;
+    bool post_relu_ = false;
 
 private:
     struct packed_entry { void* ptr; size_t bytes; };
@@ -73,6 +80,7 @@ public:
     template <typename T>
     using tensor_list = typename operation<Dtype>::template tensor_list<T>;
     explicit operation_convolutiondepthwise(const operation_param& param) : operation_convolution<Dtype>(param) {}
+    bool set_post_activation(int, float, float, bool) override { return false; }
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;

@@ -327,7 +327,16 @@ exhip_conv_desc operation_convolution<Dtype>::describe(int n, int h, int w, int 
     d.kh = this->kernel_size_h_; d.kw = this->kernel_size_w_; d.sh = this->stride_h_; d.sw = this->stride_w_;
     d.pt = this->pad_top_; d.pb = this->pad_bottom_; d.pl = this->pad_left_; d.pr = this->pad_right_;
     d.act = this->activation_type_; d.c_stride = c_stride; d.k_stride = k_stride;
+    d.post_relu = post_relu_ ? 1 : 0; d.post_op = post_op_; d.post_alpha = post_alpha_; d.post_beta = post_beta_;
     return d;
+}
+
+template <typename Dtype>
+bool operation_convolution<Dtype>::set_post_activation(int post_op, float alpha, float beta, bool relu) {
+    if ((post_op || relu) && (this->group_ != 1 || this->stride_h_ != this->stride_w_ || post_op == 1 + EXHIP_UNARY_SIGMOID))
+        return false;
+    post_op_ = post_op; post_alpha_ = alpha; post_beta_ = beta; post_relu_ = relu;
+    return true;
 }
 
 template <typename Dtype>

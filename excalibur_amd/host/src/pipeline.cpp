@@ -132,6 +132,39 @@ public:
                 if (!consumed.count(b)) output_names_.push_back(b);
         if (input_names_.empty()) LOG(FATAL) << "the topology has no input blob";
         featmaps_.resize(blob_names_.size());
+        find_activation_pairs();
+    }
+
+    // A convolution whose only reader is the activation layer on the next line runs that layer in its epilogue: the
+    // values are the ones the two layers produce one after the other, and the blob between them is never stored. The
+    // pair qualifies when the activation writes over its input (the blob name is reused) or when nothing else reads
+    // the convolution's blob and it is not a result of the network.
+    void find_activation_pairs() {
+        pair_.assign(operations_.size(), post_activation{});
+        std::vector<int> readers(blob_names_.size(), 0);
+        for (const auto& in : op_inputs_)
+            for (int b : in) ++readers[b];
+        for (size_t i = 0; i + 1 < operations_.size(); ++i) {
+            auto* conv = dynamic_cast<operation_convolution<Dtype>*>(operations_[i].get());
+            if (!conv || op_outputs_[i].size() != 1 || op_inputs_[i + 1].size() != 1 || op_outputs_[i + 1].size() != 1) continue;
+            const int mid = op_outputs_[i][0];
+            if (op_inputs_[i + 1][0] != mid) continue;
+            post_activation pa;
+            if (auto* u = dynamic_cast<operation_unary<Dtype>*>(operations_[i + 1].get())) {
+                pa.post_op = 1 + u->op_; pa.alpha = u->alpha_; pa.beta = u->beta_;
+            } else if (dynamic_cast<operation_relu<Dtype>*>(operations_[i + 1].get())) {
+                pa.relu = true;
+            } else {
+                continue;
+            }
+            const bool in_place = op_outputs_[i + 1][0] == mid;
+            const bool is_result = std::find(output_names_.begin(), output_names_.end(), blob_names_[mid]) != output_names_.end();
+            if (!in_place && (readers[mid] != 1 || is_result)) continue;
+            if (!conv->set_post_activation(pa.post_op, pa.alpha, pa.beta, pa.relu)) continue;
+            conv->set_post_activation(0, 0.f, 0.f, false);
+            pa.on = true;
+            pair_[i] = pa;
+        }
     }
 
     blob_map forward(const tensor_ptr& input) {
@@ -195,6 +228,16 @@ private:
                 if (!featmaps_[b]) LOG(FATAL) << "layer " << op_params_[i].name_ << " reads blob " << blob_names_[b] << " before it is produced";
                 in.push_back(featmaps_[b]);
             }
+            if (fusion_ && pair_[i].on) {
+                auto* conv = static_cast<operation_convolution<Dtype>*>(operations_[i].get());
+                conv->set_post_activation(pair_[i].post_op, pair_[i].alpha, pair_[i].beta, pair_[i].relu);
+                conv->forward_gpu(in, out);
+                conv->set_post_activation(0, 0.f, 0.f, false);
+                featmaps_[op_outputs_[i][0]] = nullptr;
+                featmaps_[op_outputs_[i + 1][0]] = out[0];
+                ++i;  // the activation layer has run
+                continue;
+            }
             operations_[i]->forward_gpu(in, out);
             for (size_t j = 0; j < out.size(); ++j) featmaps_[op_outputs_[i][j]] = out[j];
         }
@@ -222,6 +265,12 @@ private:
     std::vector<std::vector<int>> op_inputs_, op_outputs_;
     std::vector<std::string> input_names_, output_names_;
     std::vector<tensor_ptr> featmaps_;
+    struct post_activation {
+        bool on = false, relu = false;
+        int post_op = 0;
+        float alpha = 0.f, beta = 0.f;
+    };
+    std::vector<post_activation> pair_;  // per layer: the activation layer on the next line runs in this one's epilogue
     int weights_mem_cost_ = 0;
 };
 

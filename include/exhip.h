@@ -86,6 +86,10 @@ typedef struct exhip_conv_desc {
     int k_stride;               /* channel stride of the NHWC outputs, in elements (>= k) */
     int post_relu;              /* ReLU applied after the residual add (0/1) */
     float fs_out;               /* scale of the optional int8 output: q = sat8(trunc(v*fs_out +- 0.5)) */
+    int post_op;                /* 0, or 1 + EXHIP_UNARY_*: the activation layer behind the convolution, applied to the
+                                 * value the convolution layer would have stored (rounded to half first in the fp16
+                                 * kernel) by the general epilogue; not available with the fused int8 outputs */
+    float post_alpha, post_beta; /* that layer's parameters (operation_hardswish.cpp:32-63, operation_leakyrelu.cpp:31-58) */
 } exhip_conv_desc;
 
 /* Output spatial size, (H + pt + pb - kh)/sh + 1 (src/Excalibur/operation_convolution.cpp:270-271). */

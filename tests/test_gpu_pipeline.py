@@ -425,3 +425,85 @@ def test_fp16_pipeline_nhwc_resident_equals_nchw_blobs(monkeypatch, which):
         assert np.isfinite(out).all() and np.count_nonzero(out) > out.size // 2
     finally:
         os.unlink(path)
+
+
+def _activation_pairs_net(seed, int8):
+    """Convolutions followed by every activation layer the convolution kernel can apply itself, plus the cases it must
+    leave alone: a sigmoid, a blob with a second reader, a blob that is a result of the network, a grouped layer."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(seed)
+    lines, blobs = ["Input data 0 1 data 0=20 1=20 2=3 3=0,0,0 4=1.0"], []
+
+    def conv(bottom, top, cin, k, kernel, stride, groups=1):
+        w = r.normal(0, np.sqrt(2.0 / (cin // groups * kernel * kernel)), (k, cin // groups, kernel, kernel)).astype(np.float32)
+        b = r.normal(0, 0.5, (k,)).astype(np.float32)
+        if int8 and groups == 1:
+            ws = (np.float32(127.0) / np.abs(w).reshape(k, -1).max(axis=1)).astype(np.float32)
+            wq = np.clip(np.rint(w * ws[:, None, None, None]), -127, 127).astype(np.int8)
+            lines.append(mf.conv_line("Convolution", top + "_l", bottom, top, k, kernel, stride, kernel // 2, True, w.size, 1, int8=True))
+            blobs.append(mf.conv_blob_i8(wq, b, ws, np.float32(40.0)))
+        else:
+            kind = "Convolution" if groups == 1 else "ConvolutionDepthWise"
+            lines.append(mf.conv_line(kind, top + "_l", bottom, top, k, kernel, stride, kernel // 2, True, w.size, groups))
+            blobs.append(mf.conv_blob_f32(w, b))
+
+    conv("data", "c1", 3, 16, 3, 1)
+    lines.append("HardSwish hs1 1 1 c1 a1 0=1.666667e-01 1=5.000000e-01")
+    conv("a1", "c2", 16, 32, 1, 1)
+    lines.append("LeakyRelu lk2 1 1 c2 c2 0=1.000000e-01")              # writes over its input
+    conv("c2", "c3", 32, 32, 3, 2)
+    lines.append("ReLU r3 1 1 c3 a3")
+    conv("a3", "c4", 32, 24, 1, 1)                                        # 24 channels: no multiple of 16
+    lines.append("Clip cl4 1 1 c4 a4 0=-0.25 1=0.75")
+    conv("a4", "c5", 24, 16, 3, 1)
+    lines.append("HardSigmoid hg5 1 1 c5 a5 0=2.000000e-01 1=5.000000e-01")
+    conv("a5", "c6", 16, 16, 1, 1)
+    lines.append("Sigmoid sg6 1 1 c6 a6")                                 # stays a layer
+    conv("a6", "c7", 16, 16, 3, 1)
+    lines.append("HardSwish hs7 1 1 c7 a7 0=1.666667e-01 1=5.000000e-01")  # c7 has a second reader below
+    lines.append("Eltwise sum7 2 1 c7 a7 s7 0=1")
+    conv("s7", "c8", 16, 16, 3, 1, groups=16)                             # depthwise: its kernel has no such epilogue
+    lines.append("HardSwish hs8 1 1 c8 a8 0=1.666667e-01 1=5.000000e-01")
+    conv("a8", "c9", 16, 16, 1, 1)
+    lines.append("Split sp9 1 2 c9 c9a c9b")
+    lines.append("ReLU r9 1 1 c9a a9")                                    # c9b stays a result of the network
+    return lines, blobs, ["a9", "c9b"], ["a1", "c2", "a3", "a4", "a5", "a6", "a7", "s7", "a8"]
+
+
+@pytest.mark.parametrize("kind", ["f32", "f16", "int8"])
+def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
+    """With fusion on, the per-layer executor hands a HardSwish / LeakyRelu / ReLU / Clip / HardSigmoid layer that is the
+    only reader of a convolution to that convolution's epilogue. The values are bit for bit those of the two layers run
+    one after the other (fusion off), in float32, in float16 (where the layer between rounds to half) and behind the
+    int8 convolution; the blob between the two is not kept."""
+    from excalibur_amd import modelfile as mf
+    lines, blobs, outputs, middle = _activation_pairs_net(21, kind == "int8")
+    x = np.random.default_rng(22).normal(0, 1.5, (2, 3, 20, 20)).astype(np.float32)
+    dtype = "f16" if kind == "f16" else "f32"
+    xin = x.astype(np.float16).view(np.uint16) if kind == "f16" else x
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        mf.write_model(path, blobs)
+        got = {}
+        for fusion in (False, True):
+            p = xp.Pipeline(mf.topology(lines, "pairs"), path, 0, dtype, fusion=fusion)
+            p.forward(xin)
+            assert not p.fused
+            got[fusion] = {b: p.get(b) for b in outputs + middle}
+            if fusion:
+                for gone in ("c1", "c3", "c4", "c5"):
+                    with pytest.raises(KeyError):
+                        p.get(gone)
+                for kept in ("c6", "c7", "c8", "c9b"):
+                    p.get(kept)
+            p.close()
+        for b in outputs + middle:
+            assert got[False][b].shape == got[True][b].shape
+            assert np.array_equal(got[False][b].view(np.uint32 if dtype == "f32" else np.uint16),
+                                  got[True][b].view(np.uint32 if dtype == "f32" else np.uint16)), b
+        last = got[True]["a9"]
+        last = last.view(np.float16).astype(np.float32) if kind == "f16" else last
+        assert np.isfinite(last).all() and np.count_nonzero(last) > last.size // 8
+    finally:
+        os.unlink(path)
