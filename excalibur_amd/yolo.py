@@ -1,4 +1,4 @@
-"""A YOLOv5s-shaped float detector as `.phai` topology text + `.racy` weights, built from a seed.
+"""A YOLOv5s-shaped detector (float, or with int8 convolutions) as `.phai` topology text + `.racy` weights, built from a seed.
 
 The layer mix of the detection topology the library ships with (Input scaling, Focus, convolutions with HardSwish, a
 cross-stage block with a residual BinaryOp sum, Concat + BatchNorm + LeakyRelu, a spatial pyramid of 5 / 9 / 13 max
@@ -11,9 +11,13 @@ from . import modelfile as mf
 
 
 class YoloV5ShapedF32:
-    def __init__(self, seed=11, hw=64, width=8, anchors=3, outputs=6):
+    def __init__(self, seed=11, hw=64, width=8, anchors=3, outputs=6, int8=False, fs=96.0):
+        """int8: every convolution carries int8 weights with per-channel scales ws = 127 / max|w| and quantizes its
+        input with the feature-map scale `fs` (activations of this network stay below 1.6, so a few saturate); the other layers stay
+        float, as in the library's int8 topologies."""
         r = np.random.default_rng(seed)
         self.hw = hw
+        self.int8 = int8
         self.lines, self.blobs, self.ops = [], [], []
         self.scale = 0.0039215
         self.lines.append(f"Input images 0 1 images 0={hw} 1={hw} 2=3 3=0,0,0 4={self.scale!r}")
@@ -30,9 +34,15 @@ class YoloV5ShapedF32:
             w = r.normal(0, np.sqrt(2.0 / (cin * kernel * kernel)), (k, cin, kernel, kernel)).astype(np.float32)
             b = r.normal(0, 0.05, (k,)).astype(np.float32) if bias else None
             top = name("conv")
-            self.lines.append(mf.conv_line("Convolution", top + "_l", bottom, top, k, kernel, stride, pad, bias, w.size, 1, act=0))
-            self.blobs.append(mf.conv_blob_f32(w, b))
-            self.ops.append(("conv", bottom, top, w, b, kernel, stride, pad))
+            self.lines.append(mf.conv_line("Convolution", top + "_l", bottom, top, k, kernel, stride, pad, bias, w.size, 1, int8=int8, act=0))
+            if int8:
+                ws = (np.float32(127.0) / np.abs(w).reshape(k, -1).max(axis=1)).astype(np.float32)
+                wq = np.clip(np.rint(w * ws[:, None, None, None]), -127, 127).astype(np.int8)
+                self.blobs.append(mf.conv_blob_i8(wq, b, ws, np.float32(fs)))
+                self.ops.append(("conv_i8", bottom, top, wq, b, kernel, stride, pad, ws, np.float32(fs)))
+            else:
+                self.blobs.append(mf.conv_blob_f32(w, b))
+                self.ops.append(("conv", bottom, top, w, b, kernel, stride, pad))
             if not act:
                 return top
             out = name("hs")
@@ -109,7 +119,7 @@ class YoloV5ShapedF32:
         self.output = self.outputs[0]
 
     def topology(self):
-        return mf.topology(self.lines, "yolov5_shaped_f32")
+        return mf.topology(self.lines, "yolov5_shaped_int8" if self.int8 else "yolov5_shaped_f32")
 
     def write_model(self, path):
         mf.write_model(path, self.blobs)

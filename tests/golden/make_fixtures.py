@@ -19,7 +19,7 @@ from tests import cases  # noqa: E402
 from tests.refrun import run_reference  # noqa: E402
 
 
-NETWORKS = ("net_mobilefacenet_f32", "net_yolov5_shaped_f32")  # whole-topology fixtures: not single-layer cases
+NETWORKS = ("net_mobilefacenet_f32", "net_yolov5_shaped_f32", "net_yolov5_shaped_int8")  # whole-topology fixtures: not single-layer cases
 
 
 def fixture_cases():
@@ -154,6 +154,27 @@ def load_case(path):
     return case, z["expected"]
 
 
+def write_yolo_fixture(int8):
+    """A YOLOv5s-shaped topology (excalibur_amd.yolo; float, or with int8 convolutions), one image: the reference's
+    outputs of both heads."""
+    import tempfile
+    from excalibur_amd.yolo import YoloV5ShapedF32
+    from oracle import ref
+    # int8: 3 x 8 head channels; with 3 x 6 the reference's int8 GEMM runs its loop for output channels left over after
+    # groups of eight and four, which applies the first weight of every four to all four inputs
+    # (src/Excalibur/operation_convolution.cpp:2898-2906)
+    net = YoloV5ShapedF32(int8=True, outputs=8) if int8 else YoloV5ShapedF32()
+    seed = 10 if int8 else 9
+    x = np.random.default_rng(seed).uniform(0, 255, (1, 3, net.hw, net.hw)).astype(np.float32)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    net.write_model(path)
+    outs = ref.run(net.topology(), path, x, net.outputs)
+    os.unlink(path)
+    np.savez_compressed(os.path.join(HERE, "net_yolov5_shaped_int8.npz" if int8 else "net_yolov5_shaped_f32.npz"),
+                        input_seed=np.asarray(seed), **{f"expected{i}": outs[n] for i, n in enumerate(net.outputs)})
+
+
 def main():
     for name, case in fixture_cases().items():
         save_case(os.path.join(HERE, name + ".npz"), case, run_reference(case))
@@ -173,17 +194,8 @@ def main():
     out = ref.run(net.topology(), path, x, [net.output])[net.output]
     os.unlink(path)
     np.savez_compressed(os.path.join(HERE, "net_mobilefacenet_f32.npz"), input_seed=np.asarray(8), expected=out)
-    # a YOLOv5s-shaped float topology (excalibur_amd.yolo), one image: the reference's outputs of both heads
-    from excalibur_amd.yolo import YoloV5ShapedF32
-    net = YoloV5ShapedF32()
-    x = np.random.default_rng(9).uniform(0, 255, (1, 3, net.hw, net.hw)).astype(np.float32)
-    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
-        path = f.name
-    net.write_model(path)
-    outs = ref.run(net.topology(), path, x, net.outputs)
-    os.unlink(path)
-    np.savez_compressed(os.path.join(HERE, "net_yolov5_shaped_f32.npz"), input_seed=np.asarray(9),
-                        **{f"expected{i}": outs[n] for i, n in enumerate(net.outputs)})
+    write_yolo_fixture(False)
+    write_yolo_fixture(True)
     total = sum(os.path.getsize(os.path.join(HERE, f)) for f in os.listdir(HERE) if f.endswith(".npz"))
     print(f"wrote {len(fixture_cases()) + len(f16_cases())} fixtures, {total / 1024:.0f} KiB")
 

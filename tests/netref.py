@@ -80,7 +80,7 @@ def oracle_forward_mobilenet(net, x):
 
 
 def oracle_forward_yolo(net, x):
-    """The float YOLOv5-shaped network (excalibur_amd.yolo) op by op through the oracle restatement."""
+    """The YOLOv5-shaped network (excalibur_amd.yolo, float or int8 convolutions) op by op through the oracle restatement."""
     blobs = {"images_input": np.ascontiguousarray(x, np.float32)}
     for op in net.ops:
         kind = op[0]
@@ -92,6 +92,10 @@ def oracle_forward_yolo(net, x):
             _, bottom, top, w, b, kernel, stride, pad = op
             xin = blobs[bottom]
             blobs[top] = port.conv2d_f32(xin, w, b, 0, port.geom(xin.shape, w.shape[0], kernel, kernel, stride, pad))
+        elif kind == "conv_i8":
+            _, bottom, top, wq, b, kernel, stride, pad, ws, fs = op
+            xin = blobs[bottom]
+            blobs[top] = port.conv2d_i8(xin, wq, b, ws, fs, 0, port.geom(xin.shape, wq.shape[0], kernel, kernel, stride, pad))
         elif kind == "hardswish":
             blobs[op[2]] = port.hardswish(blobs[op[1]], op[3], op[4])
         elif kind == "leakyrelu":

@@ -507,3 +507,28 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
         assert np.isfinite(last).all() and np.count_nonzero(last) > last.size // 8
     finally:
         os.unlink(path)
+
+
+@pytest.mark.parametrize("fusion", [False, True])
+def test_yolov5_shaped_int8_topology_matches_the_reference_fixture(fusion):
+    """The detector topology with int8 convolutions through pipeline<float>: each convolution quantizes its float input,
+    accumulates in int32 and dequantizes with fmaf, every other layer is float, so the outputs equal the compiled
+    reference's bit for bit, with the HardSwish layers in the convolutions' epilogues (fusion) and as layers."""
+    from excalibur_amd.yolo import YoloV5ShapedF32
+    net = YoloV5ShapedF32(int8=True, outputs=8)
+    z = np.load(os.path.join(GOLDEN, "net_yolov5_shaped_int8.npz"))
+    x = np.random.default_rng(int(z["input_seed"])).uniform(0, 255, (1, 3, net.hw, net.hw)).astype(np.float32)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        net.write_model(path)
+        p = xp.Pipeline(net.topology(), path, 0, fusion=fusion)
+        p.forward(x)
+        assert not p.fused
+        for i, name in enumerate(net.outputs):
+            got = p.get(name)
+            assert got.shape == z[f"expected{i}"].shape
+            assert np.array_equal(got, z[f"expected{i}"])
+        p.close()
+    finally:
+        os.unlink(path)
