@@ -51,6 +51,18 @@ public:
     void reshape(std::vector<int> data_shape) { shape_ = data_shape; }
     pool_allocator<Dtype>* allocator() const { return nullptr; }
 
+    // An int8 NHWC copy of this blob, q8(x * scale) with `stride` channels per pixel (pad channels zero), written by the
+    // layer that produced the blob beside its float data, or instead of it (`only`: the float data was never written).
+    // An int8 convolution that reads the blob with that scale and stride takes the copy in place of running its
+    // quantizer. The pipeline sets this up and is the only one to hand out `only` blobs, to such readers alone.
+    struct quantized_copy {
+        std::shared_ptr<tensor<signed char>> data;
+        float scale = 0.f;
+        int stride = 0;
+        bool only = false;
+    };
+    std::shared_ptr<quantized_copy> quantized;
+
 private:
     void init(const std::vector<int>& shape, int device);
     std::shared_ptr<syncedmem<Dtype>> data_;

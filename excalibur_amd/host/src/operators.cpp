@@ -340,6 +340,24 @@ bool operation_convolution<Dtype>::set_post_activation(int post_op, float alpha,
 }
 
 template <typename Dtype>
+bool operation_convolution<Dtype>::set_quantized_output(float fs, int stride, bool only) {
+    if (fs != 0.f && (!this->params_.int8_quantization_ || this->group_ != 1 || this->stride_h_ != this->stride_w_ ||
+                      stride < this->output_channel_ || stride % 32 != 0))
+        return false;
+    q_out_fs_ = fs; q_out_stride_ = fs != 0.f ? stride : 0; q_out_only_ = fs != 0.f && only;
+    return true;
+}
+
+template <typename Dtype>
+void operation_convolution<Dtype>::quantized_input(float* fs, int* stride) const {
+    *fs = 0.f; *stride = 0;
+    if (!this->params_.int8_quantization_ || this->group_ != 1 || this->stride_h_ != this->stride_w_) return;
+    if (!this->featmap_scaletable_i8_ || this->featmap_scaletable_i8_->count() != 1) return;
+    *fs = featmap_scale();
+    *stride = conv_in_stride(this->input_channels(), EXHIP_I8, this->kernel_size_w_);
+}
+
+template <typename Dtype>
 const void* operation_convolution<Dtype>::packed_weights(int dtype, const exhip_conv_desc& d) {
     const std::vector<int> key{dtype, d.n, d.h, d.w, d.c_stride};
     auto it = packed_.find(key);
@@ -418,11 +436,31 @@ void operation_convolution<Dtype>::forward_gpu_i8(const tensor_list<float>& bott
         return;
     }
     d.c_stride = conv_in_stride(c, EXHIP_I8, d.kw);
-    auto q = new_tensor<signed char>({n, h, w, d.c_stride}, dev);
-    EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, featmap_scale(), nullptr,
-                                                   d.c_stride, reinterpret_cast<int8_t*>(q->mutable_gpu_data())));
+    // the producer's int8 copy of the input if it was made with this layer's scale and stride, else the quantizer
+    std::shared_ptr<tensor<signed char>> q;
+    const auto& copy = bottoms[0]->quantized;
+    if (copy && copy->scale == featmap_scale() && copy->stride == d.c_stride &&
+        copy->data->data_shape() == std::vector<int>{n, h, w, d.c_stride}) {
+        q = copy->data;
+    } else {
+        if (copy && copy->only) LOG(FATAL) << "layer " << this->params_.name_ << ": the input blob holds int8 data for another reader";
+        q = new_tensor<signed char>({n, h, w, d.c_stride}, dev);
+        EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(this->ctx(), bottoms[0]->gpu_data(), n, c, h, w, featmap_scale(), nullptr,
+                                                       d.c_stride, reinterpret_cast<int8_t*>(q->mutable_gpu_data())));
+    }
+    int8_t* y_q = nullptr;
+    if (q_out_fs_ != 0.f) {
+        auto out = std::make_shared<typename tensor<float>::quantized_copy>();
+        out->data = new_tensor<signed char>({n, oh, ow, q_out_stride_}, dev);
+        out->scale = q_out_fs_; out->stride = q_out_stride_; out->only = q_out_only_;
+        tops[0]->quantized = out;
+        y_q = reinterpret_cast<int8_t*>(out->data->mutable_gpu_data());
+        d.fs_out = q_out_fs_;
+        d.k_stride = q_out_stride_;
+    }
     EXHIP_FATAL(exhip_conv2d_i8(this->ctx(), &d, reinterpret_cast<const int8_t*>(q->gpu_data()), packed_weights(EXHIP_I8, d),
-                                scale_gpu(), bias_gpu(), nullptr, nullptr, nullptr, tops[0]->mutable_gpu_data(), nullptr));
+                                scale_gpu(), bias_gpu(), nullptr, y_q, nullptr, q_out_only_ ? nullptr : tops[0]->mutable_gpu_data(),
+                                nullptr));
 }
 
 template <typename Dtype>

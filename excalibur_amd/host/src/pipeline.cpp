@@ -165,6 +165,49 @@ public:
             pa.on = true;
             pair_[i] = pa;
         }
+        find_quantized_links();
+    }
+
+    // An int8 convolution whose result is read by int8 convolutions writes the int8 NHWC tensor those readers would
+    // make of it (their feature-map scale, their channel stride) from its epilogue, and they skip their quantizer:
+    // q8(v * fs) of the value the layer stores is what the reader's quantizer computes from the stored value. Readers
+    // are found through Split layers (their tops are the bottom itself) and behind the activation layer paired with the
+    // convolution; if every reader is such a convolution and the blob is no result of the network, the float tensor
+    // is not written at all.
+    void find_quantized_links() {
+        link_.assign(operations_.size(), quantized_link{});
+        for (size_t i = 0; i < operations_.size(); ++i) {
+            auto* conv = dynamic_cast<operation_convolution<Dtype>*>(operations_[i].get());
+            if (!conv || op_outputs_[i].size() != 1 || !conv->set_quantized_output(1.f, 1 << 20, false)) continue;
+            conv->set_quantized_output(0.f, 0, false);
+            const size_t last = pair_[i].on ? i + 1 : i;  // the layer whose top the readers see
+            std::vector<int> names{op_outputs_[last][0]};
+            quantized_link lk;
+            bool float_reader = false;
+            for (size_t b = 0; b < names.size(); ++b) {
+                if (std::find(output_names_.begin(), output_names_.end(), blob_names_[names[b]]) != output_names_.end()) float_reader = true;
+                for (size_t j = 0; j < operations_.size(); ++j) {
+                    if (j == last && pair_[i].on) continue;  // the paired activation writing over its input
+                    if (std::find(op_inputs_[j].begin(), op_inputs_[j].end(), names[b]) == op_inputs_[j].end()) continue;
+                    if (j <= last) { float_reader = true; continue; }  // a reused name: not this layer's blob, stay safe
+                    if (dynamic_cast<operation_split<Dtype>*>(operations_[j].get())) {
+                        for (int t : op_outputs_[j])
+                            if (std::find(names.begin(), names.end(), t) == names.end()) names.push_back(t);
+                        continue;
+                    }
+                    float fs = 0.f;
+                    int stride = 0;
+                    if (auto* reader = dynamic_cast<operation_convolution<Dtype>*>(operations_[j].get())) reader->quantized_input(&fs, &stride);
+                    if (fs == 0.f || stride % 32 != 0) { float_reader = true; continue; }
+                    if (!lk.on) { lk.on = true; lk.fs = fs; lk.stride = stride; }
+                    else if (lk.fs != fs || lk.stride != stride) float_reader = true;  // that reader runs its quantizer
+                }
+            }
+            if (!lk.on || !conv->set_quantized_output(lk.fs, lk.stride, false)) continue;
+            conv->set_quantized_output(0.f, 0, false);
+            lk.only = !float_reader;
+            link_[i] = lk;
+        }
     }
 
     blob_map forward(const tensor_ptr& input) {
@@ -193,7 +236,9 @@ public:
     tensor_ptr get_featmap(std::string_view name) {
         auto it = blob_index_.find(std::string(name));
         if (it == blob_index_.end()) return nullptr;
-        return nchw(featmaps_[it->second]);
+        const tensor_ptr& t = featmaps_[it->second];
+        if (t && t->quantized && t->quantized->only) return nullptr;  // only its int8 form was written
+        return nchw(t);
     }
 
     // The fp16 layers pass NHWC blobs among themselves; what leaves the pipeline is NCHW as in the reference.
@@ -228,14 +273,20 @@ private:
                 if (!featmaps_[b]) LOG(FATAL) << "layer " << op_params_[i].name_ << " reads blob " << blob_names_[b] << " before it is produced";
                 in.push_back(featmaps_[b]);
             }
-            if (fusion_ && pair_[i].on) {
+            if (fusion_ && (pair_[i].on || link_[i].on)) {
                 auto* conv = static_cast<operation_convolution<Dtype>*>(operations_[i].get());
-                conv->set_post_activation(pair_[i].post_op, pair_[i].alpha, pair_[i].beta, pair_[i].relu);
+                if (pair_[i].on) conv->set_post_activation(pair_[i].post_op, pair_[i].alpha, pair_[i].beta, pair_[i].relu);
+                if (link_[i].on) conv->set_quantized_output(link_[i].fs, link_[i].stride, link_[i].only);
                 conv->forward_gpu(in, out);
                 conv->set_post_activation(0, 0.f, 0.f, false);
-                featmaps_[op_outputs_[i][0]] = nullptr;
-                featmaps_[op_outputs_[i + 1][0]] = out[0];
-                ++i;  // the activation layer has run
+                conv->set_quantized_output(0.f, 0, false);
+                if (pair_[i].on) {
+                    featmaps_[op_outputs_[i][0]] = nullptr;
+                    featmaps_[op_outputs_[i + 1][0]] = out[0];
+                    ++i;  // the activation layer has run
+                } else {
+                    featmaps_[op_outputs_[i][0]] = out[0];
+                }
                 continue;
             }
             operations_[i]->forward_gpu(in, out);
@@ -271,6 +322,12 @@ private:
         float alpha = 0.f, beta = 0.f;
     };
     std::vector<post_activation> pair_;  // per layer: the activation layer on the next line runs in this one's epilogue
+    struct quantized_link {
+        bool on = false, only = false;
+        float fs = 0.f;
+        int stride = 0;
+    };
+    std::vector<quantized_link> link_;   // per layer: an int8 convolution that writes its readers' int8 input
     int weights_mem_cost_ = 0;
 };
 

@@ -490,7 +490,12 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
             p = xp.Pipeline(mf.topology(lines, "pairs"), path, 0, dtype, fusion=fusion)
             p.forward(xin)
             assert not p.fused
-            got[fusion] = {b: p.get(b) for b in outputs + middle}
+            got[fusion] = {b: p.get(b) for b in outputs}
+            for b in middle:  # with int8 convolutions, a blob read by int8 convolutions alone has no float form
+                try:
+                    got[fusion][b] = p.get(b)
+                except KeyError:
+                    assert fusion and kind == "int8"
             if fusion:
                 for gone in ("c1", "c3", "c4", "c5"):
                     with pytest.raises(KeyError):
@@ -498,7 +503,8 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
                 for kept in ("c6", "c7", "c8", "c9b"):
                     p.get(kept)
             p.close()
-        for b in outputs + middle:
+        assert len(got[True]) >= len(outputs) + 4
+        for b in got[True]:
             assert got[False][b].shape == got[True][b].shape
             assert np.array_equal(got[False][b].view(np.uint32 if dtype == "f32" else np.uint16),
                                   got[True][b].view(np.uint32 if dtype == "f32" else np.uint16)), b
@@ -530,5 +536,67 @@ def test_yolov5_shaped_int8_topology_matches_the_reference_fixture(fusion):
             assert got.shape == z[f"expected{i}"].shape
             assert np.array_equal(got, z[f"expected{i}"])
         p.close()
+    finally:
+        os.unlink(path)
+
+
+def test_int8_convolutions_hand_their_readers_int8_tensors():
+    """With fusion on, an int8 convolution read by int8 convolutions (directly, through Split layers, behind its paired
+    activation) writes their quantized input itself and they skip the quantizer; a blob all of whose readers are such
+    convolutions is never stored as float. Same values as layer by layer, bit for bit: conv -> conv, conv -> HardSwish
+    -> Split -> two convs, a convolution read by a float layer as well, one whose reader uses another scale, one with
+    fewer output channels than the reader's channel stride."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(51)
+    lines, blobs = ["Input data 0 1 data 0=24 1=24 2=3 3=0,0,0 4=1.0"], []
+
+    def conv(bottom, top, cin, k, kernel, stride, fs):
+        w = r.normal(0, np.sqrt(2.0 / (cin * kernel * kernel)), (k, cin, kernel, kernel)).astype(np.float32)
+        b = r.normal(0, 0.3, (k,)).astype(np.float32)
+        ws = (np.float32(127.0) / np.abs(w).reshape(k, -1).max(axis=1)).astype(np.float32)
+        wq = np.clip(np.rint(w * ws[:, None, None, None]), -127, 127).astype(np.int8)
+        lines.append(mf.conv_line("Convolution", top + "_l", bottom, top, k, kernel, stride, kernel // 2, True, w.size, 1, int8=True))
+        blobs.append(mf.conv_blob_i8(wq, b, ws, np.float32(fs)))
+
+    conv("data", "c1", 3, 64, 3, 1, 40.0)
+    conv("c1", "c2", 64, 24, 3, 2, 30.0)                     # c1: one int8 reader, float never stored; 24 of 32 channels
+    lines.append("HardSwish hs2 1 1 c2 a2 0=1.666667e-01 1=5.000000e-01")
+    lines.append("Split sp2 1 2 a2 a2x a2y")
+    conv("a2x", "c3", 24, 32, 1, 1, 50.0)                    # both readers of a2 quantize with 50
+    conv("a2y", "c4", 24, 32, 3, 1, 50.0)
+    lines.append("Split sp3 1 2 c3 c3x c3y")                 # c3: an int8 reader and a float reader
+    conv("c3x", "c5", 32, 32, 1, 1, 20.0)
+    lines.append("Eltwise sum 2 1 c3y c4 s 0=1")             # c4: float reader only
+    conv("s", "c6", 32, 64, 3, 1, 25.0)
+    lines.append("Split sp6 1 2 c6 c6x c6y")                 # c6: two int8 readers with different scales
+    conv("c6x", "c7", 64, 16, 1, 1, 35.0)
+    conv("c6y", "c8", 64, 16, 1, 1, 45.0)
+    outputs = ["c5", "c7", "c8"]
+    x = np.random.default_rng(52).normal(0, 1.0, (2, 3, 24, 24)).astype(np.float32)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        mf.write_model(path, blobs)
+        got = {}
+        for fusion in (False, True):
+            p = xp.Pipeline(mf.topology(lines, "links"), path, 0, fusion=fusion)
+            p.forward(x)
+            assert not p.fused
+            got[fusion] = {b: p.get(b) for b in outputs + ["c3", "c4", "s"]}
+            if fusion:
+                for gone in ("c1", "c2", "a2"):         # int8 only, or inside the pair
+                    with pytest.raises(KeyError):
+                        p.get(gone)
+                assert np.isfinite(p.get("c6")).all()    # its second reader quantizes the float form itself
+                p.forward(x)                              # a second forward reuses the pooled blocks
+                for b in outputs:
+                    assert np.array_equal(p.get(b), got[True][b])
+            else:
+                for b in ("c1", "c2", "a2", "c6"):
+                    assert np.isfinite(p.get(b)).all()
+            p.close()
+        for b in got[False]:
+            assert np.array_equal(got[False][b].view(np.uint32), got[True][b].view(np.uint32)), b
+        assert all(np.count_nonzero(got[True][b]) > got[True][b].size // 4 for b in outputs)
     finally:
         os.unlink(path)
