@@ -124,6 +124,8 @@ def bandwidth_table(iters=20):
     p0, p1 = ctx.array(rng.normal(0, 1, c).astype(np.float32)), ctx.array(rng.normal(0, 1, c).astype(np.float32))
     bw("BatchNorm f32", cnt * 8, lambda: L.exhip_channelwise_f32(ctx.h, 1, xf.ptr, zf.ptr, n, c, h * w, p0.ptr, p1.ptr, 0))
     bw("BatchNorm f16", cnt * 4, lambda: L.exhip_channelwise_f16(ctx.h, 1, xh.ptr, zh.ptr, n, c, h * w, p0.ptr, p1.ptr, 0))
+    bw("BatchNorm f16 NHWC", cnt * 4,
+       lambda: L.exhip_channelwise_nhwc_f16(ctx.h, 1, xh.ptr, zh.ptr, ctypes.c_size_t(n * h * w), c, p0.ptr, p1.ptr, 0))
     big = ctx.empty((n, 2 * c, h, w), np.float32)
     chs = (ctypes.c_int * 2)(c, c)
     bw("Concat f32, 2 x 64 channels", cnt * 16, lambda: L.exhip_concat_channels_f32(ctx.h, ptrs, chs, 2, n, h * w, big.ptr))

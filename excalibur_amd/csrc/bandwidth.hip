@@ -1099,18 +1099,33 @@ __global__ __launch_bounds__(kBlock) void channelwise_f16_kernel(const uint16_t*
 }
 
 // The per-channel layers on NHWC half storage (channel = element index modulo C, C a multiple of eight): eight
-// consecutive channels of one pixel per thread.
-template <int OP>
+// consecutive channels of one pixel per 16-byte vector. The launch has a multiple of C / 8 threads, so a thread's
+// vectors (one every `gridDim.x * kBlock`) all belong to the same eight channels and their parameters are read once.
+template <int OP, bool VEC_PARAMS>
 __global__ __launch_bounds__(kBlock) void channelwise_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
-                                                                      size_t n8, int C, const float* __restrict__ p0,
+                                                                      size_t n8, unsigned groups, const float* __restrict__ p0,
                                                                       const float* __restrict__ p1, int shared) {
-    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= n8) return;
-    const int c0 = (int)((i * 8) % (size_t)C);
-    v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(x)[i]), v8f);
+    const unsigned first = blockIdx.x * kBlock + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * kBlock;
+    const unsigned c0 = (first % groups) * 8;
+    float a[8], b[8];
+    if constexpr (VEC_PARAMS) {
+        const v4f a0 = shared ? v4f{p0[0], p0[0], p0[0], p0[0]} : *reinterpret_cast<const v4f*>(p0 + c0);
+        const v4f a1 = shared ? a0 : *reinterpret_cast<const v4f*>(p0 + c0 + 4);
+        const v4f b0 = p1 ? *reinterpret_cast<const v4f*>(p1 + c0) : v4f{0.f, 0.f, 0.f, 0.f};
+        const v4f b1 = p1 ? *reinterpret_cast<const v4f*>(p1 + c0 + 4) : b0;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = channel_value<OP>(v[e], p0[shared ? 0 : c0 + e], p1 ? p1[c0 + e] : 0.f);
-    reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
+        for (int e = 0; e < 4; ++e) { a[e] = a0[e]; a[e + 4] = a1[e]; b[e] = b0[e]; b[e + 4] = b1[e]; }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { a[e] = p0[shared ? 0 : c0 + e]; b[e] = p1 ? p1[c0 + e] : 0.f; }
+    }
+    for (size_t i = first; i < n8; i += step) {
+        v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, reinterpret_cast<const v4i*>(x)[i]), v8f);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = channel_value<OP>(v[e], a[e], b[e]);
+        reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
+    }
 }
 
 // Per-channel layers on NCHW. OP 0 PReLU (p0 = slope, one per channel or one shared), 1 BatchNorm as
@@ -2079,18 +2094,26 @@ extern "C" int exhip_channelwise_nhwc_f16(exhip_ctx* ctx, int op, const uint16_t
                   "exhip_channelwise_nhwc_f16: tensors must be 16-byte aligned");
     EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || p1, "exhip_channelwise_nhwc_f16: this op needs two parameter arrays");
     const size_t n8 = pixels * (size_t)c / 8;
+    // about eight vectors per thread, in a launch whose thread count is a multiple of the channel groups
+    const unsigned groups = (unsigned)c / 8;
+    unsigned g = groups, r = kBlock;
+    while (r) { const unsigned t = g % r; g = r; r = t; }           // g = gcd(groups, kBlock)
+    const unsigned unit = groups / g;
+    size_t blocks = (n8 + (size_t)kBlock * 8 - 1) / ((size_t)kBlock * 8);
+    blocks = (blocks + unit - 1) / unit * unit;
+    EXHIP_REQUIRE(blocks * kBlock < (1ull << 32), "exhip_channelwise_nhwc_f16: tensor too large");
+    const bool vp = (reinterpret_cast<uintptr_t>(p0) & 15) == 0 && (reinterpret_cast<uintptr_t>(p1) & 15) == 0;
+    const dim3 grid((unsigned)blocks);
+#define EXHIP_CW_NHWC(OP, SH)                                                                                                 \
+    if (vp) hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<OP, true>), grid, dim3(kBlock), 0, ctx->stream, x, y, n8, groups, p0, p1, SH); \
+    else hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<OP, false>), grid, dim3(kBlock), 0, ctx->stream, x, y, n8, groups, p0, p1, SH)
     switch (op) {
-    case EXHIP_CHANNEL_PRELU:
-        hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<0>), dim3(blocks_for(n8)), dim3(kBlock), 0, ctx->stream, x, y, n8, c, p0, p1, shared);
-        break;
-    case EXHIP_CHANNEL_BATCHNORM:
-        hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<1>), dim3(blocks_for(n8)), dim3(kBlock), 0, ctx->stream, x, y, n8, c, p0, p1, 0);
-        break;
-    case EXHIP_CHANNEL_INPUT:
-        hipLaunchKernelGGL((channelwise_nhwc_f16_kernel<2>), dim3(blocks_for(n8)), dim3(kBlock), 0, ctx->stream, x, y, n8, c, p0, p1, 0);
-        break;
+    case EXHIP_CHANNEL_PRELU: EXHIP_CW_NHWC(0, shared); break;
+    case EXHIP_CHANNEL_BATCHNORM: EXHIP_CW_NHWC(1, 0); break;
+    case EXHIP_CHANNEL_INPUT: EXHIP_CW_NHWC(2, 0); break;
     default: exhip_set_error("exhip_channelwise_nhwc_f16: unknown op %d", op); return EXHIP_ERR_ARG;
     }
+#undef EXHIP_CW_NHWC
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
