@@ -899,14 +899,23 @@ __global__ __launch_bounds__(kBlock) void pool2d_nhwc_f16_kernel(const uint16_t*
     float acc[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[e] = type == 0 ? -FLT_MAX : 0.f;
+    // eight taps of a row are loaded before the first is used (a global pool is one thread walking the whole plane);
+    // the taps are taken in window order, as in the definition
     for (int a = hs; a < he; ++a)
-        for (int b = wsx; b < we; ++b) {
-            const v4i v = *reinterpret_cast<const v4i*>(x + ((n * H + a) * W + b) * cs + g * 8);
+        for (int b0 = wsx; b0 < we; b0 += 8) {
+            v4i v[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float t = exhip_h2f((uint16_t)(((uint32_t)v[e >> 1] >> ((e & 1) * 16)) & 0xffff));
-                if (type == 0) acc[e] = acc[e] < t ? t : acc[e];
-                else acc[e] += t;
+            for (int t = 0; t < 8; ++t)
+                v[t] = *reinterpret_cast<const v4i*>(x + ((n * H + a) * W + min(b0 + t, we - 1)) * cs + g * 8);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                if (b0 + t >= we) break;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float f = exhip_h2f((uint16_t)(((uint32_t)v[t][e >> 1] >> ((e & 1) * 16)) & 0xffff));
+                    if (type == 0) acc[e] = acc[e] < f ? f : acc[e];
+                    else acc[e] += f;
+                }
             }
         }
     v4i o = {0, 0, 0, 0};
@@ -1464,7 +1473,7 @@ __global__ __launch_bounds__(kBlock) void innerproduct_f32_kernel(const float* _
     if (j >= n_out) return;
     const float* wr = w + (size_t)j * k_in;
     const bool vec = (k_in % 4 == 0);
-    for (int m0 = 0; m0 < m; m0 += 8) {
+    for (int m0 = blockIdx.y * 8; m0 < m; m0 += gridDim.y * 8) {  // groups of eight batch rows across blockIdx.y
         float acc[8];
 #pragma unroll
         for (int r = 0; r < 8; ++r) acc[r] = 0.f;
@@ -1931,7 +1940,8 @@ extern "C" int exhip_innerproduct_f32(exhip_ctx* ctx, const float* x, const floa
                                       int n_out, int k_in) {
     REQ_CTX("exhip_innerproduct_f32");
     EXHIP_REQUIRE(x && w && y && m > 0 && n_out > 0 && k_in > 0, "exhip_innerproduct_f32: bad argument");
-    hipLaunchKernelGGL(innerproduct_f32_kernel, dim3((n_out + 3) / 4), dim3(kBlock), 0, ctx->stream, x, w, bias, y, m, n_out, k_in);
+    const unsigned row_groups = (unsigned)std::min((m + 7) / 8, 1024);
+    hipLaunchKernelGGL(innerproduct_f32_kernel, dim3((n_out + 3) / 4, row_groups), dim3(kBlock), 0, ctx->stream, x, w, bias, y, m, n_out, k_in);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

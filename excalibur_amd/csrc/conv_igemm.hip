@@ -88,6 +88,8 @@ struct ConvParams {
     int act, post_relu;
     int post_op;              // 0, or 1 + EXHIP_UNARY_*: the activation layer behind the convolution (general epilogue)
     float post_alpha, post_beta;
+    const float* post_slope;  // post_op == EXHIP_POST_PRELU: slopes per output channel (one for all if post_slope_shared)
+    int post_slope_shared;
     float fs_out;
     int b_align;              // alignment of B fragment reads in packed-row form (4, 8 or 16)
     unsigned img_bytes;       // bytes of one input image (buffer range for the bounds-checked loads)
@@ -1065,7 +1067,17 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                         v[e] = (0.f > v[e]) ? 0.f : v[e];
                     }
                 }
-                if (p.post_op) post_activation<DT>(v, p.post_op - 1, p.post_alpha, p.post_beta);
+                if (p.post_op == EXHIP_POST_PRELU) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        float t = v[e];
+                        if constexpr (DT == EXHIP_F16) t = exhip_h2f(exhip_f2h(t));
+                        const float slope = p.post_slope[p.post_slope_shared || ch0 + e >= p.K ? 0 : ch0 + e];
+                        v[e] = t >= 0.f ? t : slope * t;
+                    }
+                } else if (p.post_op) {
+                    post_activation<DT>(v, p.post_op - 1, p.post_alpha, p.post_beta);
+                }
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
@@ -1495,7 +1507,9 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.tiles_x = pl.tiles_x; p.tiles_y = pl.tiles_y; p.ktiles = pl.ktiles;
     p.act = d->act; p.post_relu = d->post_relu; p.fs_out = d->fs_out; p.b_align = pl.b_align;
     p.post_op = d->post_op; p.post_alpha = d->post_alpha; p.post_beta = d->post_beta;
-    EXHIP_REQUIRE(d->post_op >= 0 && d->post_op <= 1 + EXHIP_UNARY_CLIP && d->post_op != 1 + EXHIP_UNARY_SIGMOID,
+    p.post_slope = d->post_slope; p.post_slope_shared = d->post_slope_shared;
+    EXHIP_REQUIRE((d->post_op >= 0 && d->post_op <= 1 + EXHIP_UNARY_CLIP && d->post_op != 1 + EXHIP_UNARY_SIGMOID) ||
+                      (d->post_op == EXHIP_POST_PRELU && d->post_slope),
                   "conv: post_op %d is not an activation the epilogue applies", d->post_op);
     p.dbg = (kStamps && getenv("EXHIP_DEBUG_STAMPS")) ? (long long*)strtoull(getenv("EXHIP_DEBUG_STAMPS"), nullptr, 0) : nullptr;
     p.img_bytes = (unsigned)((size_t)d->h * d->w * p.cstride_b);

@@ -23,7 +23,8 @@ class ConvDesc(ctypes.Structure):
     _fields_ = [(k, ctypes.c_int) for k in
                 ("n", "c", "h", "w", "k", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr", "act", "c_stride", "k_stride",
                  "post_relu")] + [("fs_out", ctypes.c_float), ("post_op", ctypes.c_int), ("post_alpha", ctypes.c_float),
-                                  ("post_beta", ctypes.c_float)]
+                                  ("post_beta", ctypes.c_float), ("post_slope", ctypes.c_void_p),
+                                  ("post_slope_shared", ctypes.c_int)]
 
 
 _lib = None

@@ -58,6 +58,8 @@ public:
     // else 1 + EXHIP_UNARY_* with its two parameters; relu = a ReLU layer. False, and nothing set, where this layer's
     // kernel cannot apply it (the definition-order kernel of grouped layers, the sigmoid's double-precision exp).
     virtual bool set_post_activation(int post_op, float alpha, float beta, bool relu);
+    // the same for a PReLU layer: its device-resident slopes, one per output channel or one for all
+    virtual bool set_post_prelu(const float* slopes, bool shared);
     // int8 layers on the MFMA kernel. The next forward calls also write the int8 NHWC form of the output that a reader
     // quantizing with `fs` into `stride` channels per pixel would make of it (attached to the top blob as its
     // `quantized` copy), and with `only` leave the float data unwritten; fs = 0 switches it off. False where this
@@ -74,6 +76,8 @@ protected:
     int post_op_ = 0;
     float post_alpha_ = 0.f, post_beta_ = 0.f;
     bool post_relu_ = false;
+    const float* post_slope_ = nullptr;
+    bool post_slope_shared_ = false;
     float q_out_fs_ = 0.f;
     int q_out_stride_ = 0;
     bool q_out_only_ = false;
@@ -91,6 +95,7 @@ public:
     using tensor_list = typename operation<Dtype>::template tensor_list<T>;
     explicit operation_convolutiondepthwise(const operation_param& param) : operation_convolution<Dtype>(param) {}
     bool set_post_activation(int, float, float, bool) override { return false; }
+    bool set_post_prelu(const float*, bool) override { return false; }
     bool set_quantized_output(float, int, bool) override { return false; }
     void quantized_input(float* fs, int* stride) const override { *fs = 0.f; *stride = 0; }
 

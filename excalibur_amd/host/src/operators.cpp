@@ -328,7 +328,16 @@ exhip_conv_desc operation_convolution<Dtype>::describe(int n, int h, int w, int 
     d.pt = this->pad_top_; d.pb = this->pad_bottom_; d.pl = this->pad_left_; d.pr = this->pad_right_;
     d.act = this->activation_type_; d.c_stride = c_stride; d.k_stride = k_stride;
     d.post_relu = post_relu_ ? 1 : 0; d.post_op = post_op_; d.post_alpha = post_alpha_; d.post_beta = post_beta_;
+    d.post_slope = post_slope_; d.post_slope_shared = post_slope_shared_ ? 1 : 0;
     return d;
+}
+
+template <typename Dtype>
+bool operation_convolution<Dtype>::set_post_prelu(const float* slopes, bool shared) {
+    if (!slopes || this->group_ != 1 || this->stride_h_ != this->stride_w_) return false;
+    post_op_ = EXHIP_POST_PRELU; post_alpha_ = post_beta_ = 0.f; post_relu_ = false;
+    post_slope_ = slopes; post_slope_shared_ = shared;
+    return true;
 }
 
 template <typename Dtype>
@@ -336,6 +345,7 @@ bool operation_convolution<Dtype>::set_post_activation(int post_op, float alpha,
     if ((post_op || relu) && (this->group_ != 1 || this->stride_h_ != this->stride_w_ || post_op == 1 + EXHIP_UNARY_SIGMOID))
         return false;
     post_op_ = post_op; post_alpha_ = alpha; post_beta_ = beta; post_relu_ = relu;
+    post_slope_ = nullptr; post_slope_shared_ = false;
     return true;
 }
 

@@ -154,13 +154,17 @@ public:
                 pa.post_op = 1 + u->op_; pa.alpha = u->alpha_; pa.beta = u->beta_;
             } else if (dynamic_cast<operation_relu<Dtype>*>(operations_[i + 1].get())) {
                 pa.relu = true;
+            } else if (auto* pr = dynamic_cast<operation_prelu<Dtype>*>(operations_[i + 1].get())) {
+                if (!pr->share_channel_ && pr->num_slope_ != conv->output_channel_) continue;
+                pa.prelu = pr;
             } else {
                 continue;
             }
             const bool in_place = op_outputs_[i + 1][0] == mid;
             const bool is_result = std::find(output_names_.begin(), output_names_.end(), blob_names_[mid]) != output_names_.end();
             if (!in_place && (readers[mid] != 1 || is_result)) continue;
-            if (!conv->set_post_activation(pa.post_op, pa.alpha, pa.beta, pa.relu)) continue;
+            static const float probe = 0.f;  // any non-null address: asks whether the layer can, sets nothing up for a launch
+            if (!(pa.prelu ? conv->set_post_prelu(&probe, true) : conv->set_post_activation(pa.post_op, pa.alpha, pa.beta, pa.relu))) continue;
             conv->set_post_activation(0, 0.f, 0.f, false);
             pa.on = true;
             pair_[i] = pa;
@@ -275,7 +279,10 @@ private:
             }
             if (fusion_ && (pair_[i].on || link_[i].on)) {
                 auto* conv = static_cast<operation_convolution<Dtype>*>(operations_[i].get());
-                if (pair_[i].on) conv->set_post_activation(pair_[i].post_op, pair_[i].alpha, pair_[i].beta, pair_[i].relu);
+                if (pair_[i].on && pair_[i].prelu)
+                    conv->set_post_prelu(pair_[i].prelu->weights_f32()[0]->gpu_data(), pair_[i].prelu->share_channel_);
+                else if (pair_[i].on)
+                    conv->set_post_activation(pair_[i].post_op, pair_[i].alpha, pair_[i].beta, pair_[i].relu);
                 if (link_[i].on) conv->set_quantized_output(link_[i].fs, link_[i].stride, link_[i].only);
                 conv->forward_gpu(in, out);
                 conv->set_post_activation(0, 0.f, 0.f, false);
@@ -320,6 +327,7 @@ private:
         bool on = false, relu = false;
         int post_op = 0;
         float alpha = 0.f, beta = 0.f;
+        operation_prelu<Dtype>* prelu = nullptr;
     };
     std::vector<post_activation> pair_;  // per layer: the activation layer on the next line runs in this one's epilogue
     struct quantized_link {

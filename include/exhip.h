@@ -90,7 +90,12 @@ typedef struct exhip_conv_desc {
                                  * value the convolution layer would have stored (rounded to half first in the fp16
                                  * kernel) by the general epilogue; not available with the fused int8 outputs */
     float post_alpha, post_beta; /* that layer's parameters (operation_hardswish.cpp:32-63, operation_leakyrelu.cpp:31-58) */
+    const float* post_slope;    /* post_op == EXHIP_POST_PRELU: the PReLU layer behind the convolution
+                                 * (operation_prelu.cpp:57-124), v >= 0 ? v : slope * v with these device-resident
+                                 * slopes, one per output channel, or one for all if post_slope_shared */
+    int post_slope_shared;
 } exhip_conv_desc;
+#define EXHIP_POST_PRELU 16
 
 /* Output spatial size, (H + pt + pb - kh)/sh + 1 (src/Excalibur/operation_convolution.cpp:270-271). */
 int exhip_conv_out_hw(const exhip_conv_desc* d, int* oh, int* ow);

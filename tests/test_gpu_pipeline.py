@@ -449,7 +449,13 @@ def _activation_pairs_net(seed, int8):
 
     conv("data", "c1", 3, 16, 3, 1)
     lines.append("HardSwish hs1 1 1 c1 a1 0=1.666667e-01 1=5.000000e-01")
-    conv("a1", "c2", 16, 32, 1, 1)
+    conv("a1", "c1b", 16, 16, 3, 1)
+    lines.append("PReLU pr1b 1 1 c1b a1b 0=16")                          # one slope per channel
+    blobs.append(mf.floats_blob(r.uniform(-0.5, 0.5, 16).astype(np.float32)))
+    conv("a1b", "c1c", 16, 24, 1, 1)
+    lines.append("PReLU pr1c 1 1 c1c a1c 0=1")                           # one slope for all
+    blobs.append(mf.floats_blob(np.asarray([0.25], np.float32)))
+    conv("a1c", "c2", 24, 32, 1, 1)
     lines.append("LeakyRelu lk2 1 1 c2 c2 0=1.000000e-01")              # writes over its input
     conv("c2", "c3", 32, 32, 3, 2)
     lines.append("ReLU r3 1 1 c3 a3")
@@ -467,12 +473,12 @@ def _activation_pairs_net(seed, int8):
     conv("a8", "c9", 16, 16, 1, 1)
     lines.append("Split sp9 1 2 c9 c9a c9b")
     lines.append("ReLU r9 1 1 c9a a9")                                    # c9b stays a result of the network
-    return lines, blobs, ["a9", "c9b"], ["a1", "c2", "a3", "a4", "a5", "a6", "a7", "s7", "a8"]
+    return lines, blobs, ["a9", "c9b"], ["a1", "a1b", "a1c", "c2", "a3", "a4", "a5", "a6", "a7", "s7", "a8"]
 
 
 @pytest.mark.parametrize("kind", ["f32", "f16", "int8"])
 def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
-    """With fusion on, the per-layer executor hands a HardSwish / LeakyRelu / ReLU / Clip / HardSigmoid layer that is the
+    """With fusion on, the per-layer executor hands a HardSwish / LeakyRelu / ReLU / Clip / HardSigmoid / PReLU layer that is the
     only reader of a convolution to that convolution's epilogue. The values are bit for bit those of the two layers run
     one after the other (fusion off), in float32, in float16 (where the layer between rounds to half) and behind the
     int8 convolution; the blob between the two is not kept."""
@@ -497,7 +503,7 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
                 except KeyError:
                     assert fusion and kind == "int8"
             if fusion:
-                for gone in ("c1", "c3", "c4", "c5"):
+                for gone in ("c1", "c1b", "c1c", "c3", "c4", "c5"):
                     with pytest.raises(KeyError):
                         p.get(gone)
                 for kept in ("c6", "c7", "c8", "c9b"):
