@@ -279,12 +279,14 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_kernel(const float*
 // band of output rows with the three input rows it needs in registers. A row arrives as one (stride 1) or two
 // (stride 2) aligned 16-byte loads plus the halo floats the padding asks for, through a buffer descriptor whose
 // range check turns taps outside the image into zeros. slot i of a row holds column c0 - 1 + i.
+constexpr int kDwPrelu = 100;  // ACT of the strip kernels: no activation of the layer's own, then the PReLU layer behind it
 template <int STRIDE, int ACT, int PL>
 __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_strip_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                                           const float* __restrict__ bias, float* __restrict__ y,
                                                                           int C, int H, int W, int OH, int OW, int pt,
                                                                           int band_rows, int bands, int strips, unsigned x_bytes,
-                                                                          unsigned y_bytes, size_t total) {
+                                                                          unsigned y_bytes, size_t total,
+                                                                          const float* __restrict__ slope, int slope_shared) {
     constexpr int pl = PL;  // left padding (0 or 1) as a constant: which register a tap reads is then fixed, and the halo
                             // floats that this padding does not use are not loaded
     constexpr int CH = STRIDE == 1 ? 1 : 2;  // aligned 16-byte chunks per row
@@ -301,6 +303,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_strip_kernel(const 
 #pragma unroll
     for (int q = 0; q < 9; ++q) k[q] = w[c * 9 + q];
     const float b = bias ? bias[c] : 0.f;
+    const float sl = ACT == kDwPrelu ? slope[slope_shared ? 0 : c] : 0.f;  // the PReLU layer behind this one
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(x), 0, (int)x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t yr = __builtin_amdgcn_make_buffer_rsrc(y, 0, (int)y_bytes, 0x00020000);
     const int c0 = 4 * CH * t;
@@ -360,7 +363,8 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_strip_kernel(const 
                 for (int a = 0; a < 3; ++a) col = __builtin_fmaf(pl == 1 ? r[a][j * STRIDE + q] : r[a][j * STRIDE + q + 1], k[a * 3 + q], col);
                 sum += col;
             }
-            if (ACT != 0) sum = (0.f > sum) ? 0.f : sum;
+            if (ACT == kDwPrelu) sum = sum >= 0.f ? sum : sl * sum;
+            else if (ACT != 0) sum = (0.f > sum) ? 0.f : sum;
             if (ACT == 3) sum = sum <= 6.f ? sum : 0.f;
             out[j] = sum;
         }
@@ -438,7 +442,8 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                                                                           uint16_t* __restrict__ y, int C, int H, int W,
                                                                           int cs, int OH, int OW, int pt, int pl,
                                                                           int band_rows, int bands, int strips,
-                                                                          unsigned x_bytes, unsigned y_bytes, size_t total) {
+                                                                          unsigned x_bytes, unsigned y_bytes, size_t total,
+                                                                          const float* __restrict__ slope, int slope_shared) {
     constexpr int NC = (PX - 1) * STRIDE + 3, KEEP = 3 - STRIDE;
     // out-of-range markers: a tensor is at most 2^30 bytes, so a valid row offset plus the column marker, the row
     // marker plus anything, and both markers together all land beyond the descriptor's range without wrapping
@@ -470,6 +475,11 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) b[e] = bias ? bias[min(c0 + e, C - 1)] : 0.f;
+    float sl[4] = {0.f, 0.f, 0.f, 0.f};  // the PReLU layer behind this one
+    if (ACT == kDwPrelu) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sl[e] = slope[slope_shared ? 0 : min(c0 + e, C - 1)];
+    }
     // channels of the padding are stored as zero halves
     const int keep_lo = (c0 < C ? 0xffff : 0) | (c0 + 1 < C ? 0xffff0000 : 0);
     const int keep_hi = (c0 + 2 < C ? 0xffff : 0) | (c0 + 3 < C ? 0xffff0000 : 0);
@@ -526,7 +536,12 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                     sum += s;
                 }
                 // activations 0 (none), 1 (ReLU), 3 (ReLU6 as the reference writes it)
-                if (ACT != 0) sum = (0.f > sum) ? 0.f : sum;
+                if (ACT == kDwPrelu) {
+                    sum = exhip_h2f(exhip_f2h(sum));  // the PReLU layer reads the stored half
+                    sum = sum >= 0.f ? sum : sl[e] * sum;
+                } else if (ACT != 0) {
+                    sum = (0.f > sum) ? 0.f : sum;
+                }
                 if (ACT == 3) sum = sum <= 6.f ? sum : 0.f;
                 res[e] = sum;
             }
@@ -1654,8 +1669,8 @@ static int dw_out(int h, int w, int stride, int pt, int pb, int pl, int pr, int*
     return 0;
 }
 
-extern "C" int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const float* w9, const float* bias, float* y, int n,
-                                        int c, int h, int w, int stride, int pt, int pb, int pl, int pr, int act) {
+static int dw_nchw_f32(exhip_ctx* ctx, const float* x, const float* w9, const float* bias, float* y, int n, int c, int h, int w,
+                       int stride, int pt, int pb, int pl, int pr, int act, const float* slope, int slope_shared) {
     REQ_CTX("exhip_dwconv3x3_nchw_f32");
     EXHIP_REQUIRE(x && w9 && y && n > 0 && c > 0, "exhip_dwconv3x3_nchw_f32: bad argument");
     int oh, ow;
@@ -1680,24 +1695,30 @@ extern "C" int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const fl
         if (pl == 0)                                                                                                             \
             hipLaunchKernelGGL((dwconv3x3_nchw_f32_strip_kernel<S, A, 0>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, \
                                w9, bias, y, c, h, w, oh, ow, pt, band_rows, bands, strips, (unsigned)x_bytes, (unsigned)y_bytes,  \
-                               total);                                                                                           \
+                               total, slope, slope_shared);                                                                      \
         else                                                                                                                     \
             hipLaunchKernelGGL((dwconv3x3_nchw_f32_strip_kernel<S, A, 1>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, \
                                w9, bias, y, c, h, w, oh, ow, pt, band_rows, bands, strips, (unsigned)x_bytes, (unsigned)y_bytes,  \
-                               total);                                                                                           \
+                               total, slope, slope_shared);                                                                      \
     } while (0)
         if (stride == 1) {
-            if (act == 0) EXHIP_DW_STRIP(1, 0);
+            if (slope) EXHIP_DW_STRIP(1, kDwPrelu);
+            else if (act == 0) EXHIP_DW_STRIP(1, 0);
             else if (act == 1) EXHIP_DW_STRIP(1, 1);
             else EXHIP_DW_STRIP(1, 3);
         } else {
-            if (act == 0) EXHIP_DW_STRIP(2, 0);
+            if (slope) EXHIP_DW_STRIP(2, kDwPrelu);
+            else if (act == 0) EXHIP_DW_STRIP(2, 0);
             else if (act == 1) EXHIP_DW_STRIP(2, 1);
             else EXHIP_DW_STRIP(2, 3);
         }
 #undef EXHIP_DW_STRIP
         EXHIP_LAUNCH_CHECK();
         return 0;
+    }
+    if (slope) {
+        exhip_set_error("exhip_dwconv3x3_nchw_f32_prelu: this shape runs the general kernel, which has no PReLU epilogue");
+        return EXHIP_ERR_UNSUPPORTED;
     }
     const size_t total = (size_t)n * c * oh * ow;
     hipLaunchKernelGGL(dwconv3x3_nchw_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, w9, bias, y, c, h, w,
@@ -1706,9 +1727,21 @@ extern "C" int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const fl
     return 0;
 }
 
-extern "C" int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const float* bias, uint16_t* y,
-                                        int n, int c, int h, int w, int cs, int stride, int pt, int pb, int pl, int pr,
-                                        int act) {
+extern "C" int exhip_dwconv3x3_nchw_f32(exhip_ctx* ctx, const float* x, const float* w9, const float* bias, float* y, int n,
+                                        int c, int h, int w, int stride, int pt, int pb, int pl, int pr, int act) {
+    return dw_nchw_f32(ctx, x, w9, bias, y, n, c, h, w, stride, pt, pb, pl, pr, act, nullptr, 0);
+}
+
+extern "C" int exhip_dwconv3x3_nchw_f32_prelu(exhip_ctx* ctx, const float* x, const float* w9, const float* bias,
+                                              const float* slope, int slope_shared, float* y, int n, int c, int h, int w,
+                                              int stride, int pt, int pb, int pl, int pr) {
+    EXHIP_REQUIRE(slope, "exhip_dwconv3x3_nchw_f32_prelu: NULL slopes");
+    return dw_nchw_f32(ctx, x, w9, bias, y, n, c, h, w, stride, pt, pb, pl, pr, 0, slope, slope_shared);
+}
+
+static int dw_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const float* bias, uint16_t* y, int n, int c, int h,
+                       int w, int cs, int stride, int pt, int pb, int pl, int pr, int act, const float* slope,
+                       int slope_shared) {
     REQ_CTX("exhip_dwconv3x3_nhwc_f16");
     EXHIP_REQUIRE(x && w9 && y && n > 0 && c > 0 && cs >= c && cs % 8 == 0, "exhip_dwconv3x3_nhwc_f16: bad argument (c_stride %% 8)");
     int oh, ow;
@@ -1732,13 +1765,15 @@ extern "C" int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const
 #define EXHIP_DW_STRIP(S, P, A)                                                                                          \
     hipLaunchKernelGGL((dwconv3x3_nhwc_f16_strip_kernel<S, P, A>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, \
                        x, w9, bias, y, c, h, w, cs, oh, ow, pt, pl, band_rows, bands, strips, (unsigned)x_bytes,        \
-                       (unsigned)y_bytes, total)
+                       (unsigned)y_bytes, total, slope, slope_shared)
         if (stride == 1) {
-            if (act == 0) EXHIP_DW_STRIP(1, 4, 0);
+            if (slope) EXHIP_DW_STRIP(1, 4, kDwPrelu);
+            else if (act == 0) EXHIP_DW_STRIP(1, 4, 0);
             else if (act == 1) EXHIP_DW_STRIP(1, 4, 1);
             else EXHIP_DW_STRIP(1, 4, 3);
         } else {
-            if (act == 0) EXHIP_DW_STRIP(2, 3, 0);
+            if (slope) EXHIP_DW_STRIP(2, 3, kDwPrelu);
+            else if (act == 0) EXHIP_DW_STRIP(2, 3, 0);
             else if (act == 1) EXHIP_DW_STRIP(2, 3, 1);
             else EXHIP_DW_STRIP(2, 3, 3);
         }
@@ -1746,11 +1781,28 @@ extern "C" int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const
         EXHIP_LAUNCH_CHECK();
         return 0;
     }
+    if (slope) {
+        exhip_set_error("exhip_dwconv3x3_nhwc_f16_prelu: this shape runs the general kernel, which has no PReLU epilogue");
+        return EXHIP_ERR_UNSUPPORTED;
+    }
     const size_t total = (size_t)n * oh * ow * (cs / 8);
     hipLaunchKernelGGL(dwconv3x3_nhwc_f16_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, w9, bias, y, c, h, w,
                        cs, oh, ow, stride, pt, pl, act, total);
     EXHIP_LAUNCH_CHECK();
     return 0;
+}
+
+extern "C" int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const float* bias, uint16_t* y,
+                                        int n, int c, int h, int w, int cs, int stride, int pt, int pb, int pl, int pr,
+                                        int act) {
+    return dw_nhwc_f16(ctx, x, w9, bias, y, n, c, h, w, cs, stride, pt, pb, pl, pr, act, nullptr, 0);
+}
+
+extern "C" int exhip_dwconv3x3_nhwc_f16_prelu(exhip_ctx* ctx, const uint16_t* x, const float* w9, const float* bias,
+                                              const float* slope, int slope_shared, uint16_t* y, int n, int c, int h, int w,
+                                              int cs, int stride, int pt, int pb, int pl, int pr) {
+    EXHIP_REQUIRE(slope, "exhip_dwconv3x3_nhwc_f16_prelu: NULL slopes");
+    return dw_nhwc_f16(ctx, x, w9, bias, y, n, c, h, w, cs, stride, pt, pb, pl, pr, 0, slope, slope_shared);
 }
 
 extern "C" int exhip_dw_dequant_weights(exhip_ctx* ctx, const int8_t* w, const float* ws, float* wf, int k, int per_group) {

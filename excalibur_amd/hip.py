@@ -246,6 +246,24 @@ class Ctx:
                                               act))
         return y
 
+    def dwconv3x3_nchw_f32_prelu(self, x, w9, bias, slope, shared, stride, pad):
+        n, c, h, w = x.shape
+        pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+        oh, ow = (h + pt + pb - 3) // stride + 1, (w + pl + pr - 3) // stride + 1
+        y = self.empty((n, c, oh, ow), np.float32)
+        _check(lib().exhip_dwconv3x3_nchw_f32_prelu(self.h, x.ptr, w9.ptr, _ptr(bias), slope.ptr, int(shared), y.ptr, n, c, h, w,
+                                                    stride, pt, pb, pl, pr))
+        return y
+
+    def dwconv3x3_nhwc_f16_prelu(self, x, c, w9, bias, slope, shared, stride, pad):
+        n, h, w, cs = x.shape
+        pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
+        oh, ow = (h + pt + pb - 3) // stride + 1, (w + pl + pr - 3) // stride + 1
+        y = self.empty((n, oh, ow, cs), np.uint16)
+        _check(lib().exhip_dwconv3x3_nhwc_f16_prelu(self.h, x.ptr, w9.ptr, _ptr(bias), slope.ptr, int(shared), y.ptr, n, c, h, w,
+                                                    cs, stride, pt, pb, pl, pr))
+        return y
+
     def dw_dequant_weights(self, w_i8, ws):
         k = w_i8.shape[0]
         wf = self.empty(w_i8.shape, np.float32)

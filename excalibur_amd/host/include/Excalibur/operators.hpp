@@ -60,6 +60,10 @@ public:
     virtual bool set_post_activation(int post_op, float alpha, float beta, bool relu);
     // the same for a PReLU layer: its device-resident slopes, one per output channel or one for all
     virtual bool set_post_prelu(const float* slopes, bool shared);
+    void clear_post() {
+        post_op_ = 0; post_alpha_ = post_beta_ = 0.f; post_relu_ = false;
+        post_slope_ = nullptr; post_slope_shared_ = false;
+    }
     // int8 layers on the MFMA kernel. The next forward calls also write the int8 NHWC form of the output that a reader
     // quantizing with `fs` into `stride` channels per pixel would make of it (attached to the top blob as its
     // `quantized` copy), and with `only` leave the float data unwritten; fs = 0 switches it off. False where this
@@ -95,7 +99,7 @@ public:
     using tensor_list = typename operation<Dtype>::template tensor_list<T>;
     explicit operation_convolutiondepthwise(const operation_param& param) : operation_convolution<Dtype>(param) {}
     bool set_post_activation(int, float, float, bool) override { return false; }
-    bool set_post_prelu(const float*, bool) override { return false; }
+    bool set_post_prelu(const float* slopes, bool shared) override;  // the 3x3 kernels apply it; other shapes do not pair
     bool set_quantized_output(float, int, bool) override { return false; }
     void quantized_input(float* fs, int* stride) const override { *fs = 0.f; *stride = 0; }
 

@@ -536,9 +536,32 @@ void operation_convolutiondepthwise<Dtype>::forward_gpu_f32(const tensor_list<fl
     const int oh = (h + this->pad_top_ + this->pad_bottom_ - 3) / this->stride_h_ + 1;
     const int ow = (w + this->pad_left_ + this->pad_right_ - 3) / this->stride_w_ + 1;
     tops[0] = new_tensor<float>({n, c, oh, ow}, this->params_.device_);
+    if (this->post_slope_) {  // the PReLU layer behind this one in the same kernel, or as a second launch where the shape needs it
+        const int rc = exhip_dwconv3x3_nchw_f32_prelu(this->ctx(), bottoms[0]->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
+                                                      this->post_slope_, this->post_slope_shared_, tops[0]->mutable_gpu_data(), n, c, h, w,
+                                                      this->stride_h_, this->pad_top_, this->pad_bottom_, this->pad_left_, this->pad_right_);
+        if (rc != EXHIP_ERR_UNSUPPORTED) {
+            EXHIP_FATAL(rc);
+            return;
+        }
+        auto mid = new_tensor<float>({n, c, oh, ow}, this->params_.device_);
+        EXHIP_FATAL(exhip_dwconv3x3_nchw_f32(this->ctx(), bottoms[0]->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
+                                             mid->mutable_gpu_data(), n, c, h, w, this->stride_h_, this->pad_top_, this->pad_bottom_,
+                                             this->pad_left_, this->pad_right_, 0));
+        EXHIP_FATAL(exhip_channelwise_f32(this->ctx(), EXHIP_CHANNEL_PRELU, mid->gpu_data(), tops[0]->mutable_gpu_data(), n, c, oh * ow,
+                                          this->post_slope_, nullptr, this->post_slope_shared_ ? 1 : 0));
+        return;
+    }
     EXHIP_FATAL(exhip_dwconv3x3_nchw_f32(this->ctx(), bottoms[0]->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
                                          tops[0]->mutable_gpu_data(), n, c, h, w, this->stride_h_, this->pad_top_, this->pad_bottom_,
                                          this->pad_left_, this->pad_right_, this->activation_type_));
+}
+
+template <typename Dtype>
+bool operation_convolutiondepthwise<Dtype>::set_post_prelu(const float* slopes, bool shared) {
+    if (!slopes || !fast3x3() || this->activation_type_ != 0 || this->output_channel_ != this->group_) return false;
+    this->post_op_ = EXHIP_POST_PRELU; this->post_slope_ = slopes; this->post_slope_shared_ = shared;
+    return true;
 }
 
 // Weight-only quantization: the int8 weights are dequantized once and the float path runs
@@ -575,6 +598,24 @@ void operation_convolutiondepthwise<Dtype>::forward_gpu_f16(const tensor_list<un
     if (nhwc_channels_ok(c)) {  // NHWC in, NHWC out
         const half_ptr x = as_nhwc(this->ctx(), bottoms[0], dev);
         tops[0] = new_tensor<unsigned short>({n, oh, ow, c}, dev, memory::NHWC);
+        if (this->post_slope_) {
+            const int rc = exhip_dwconv3x3_nhwc_f16_prelu(this->ctx(), x->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
+                                                          this->post_slope_, this->post_slope_shared_, tops[0]->mutable_gpu_data(), n, c, h,
+                                                          w, c, this->stride_h_, this->pad_top_, this->pad_bottom_, this->pad_left_,
+                                                          this->pad_right_);
+            if (rc != EXHIP_ERR_UNSUPPORTED) {
+                EXHIP_FATAL(rc);
+                return;
+            }
+            auto mid = new_tensor<unsigned short>({n, oh, ow, c}, dev, memory::NHWC);
+            EXHIP_FATAL(exhip_dwconv3x3_nhwc_f16(this->ctx(), x->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
+                                                 mid->mutable_gpu_data(), n, c, h, w, c, this->stride_h_, this->pad_top_,
+                                                 this->pad_bottom_, this->pad_left_, this->pad_right_, 0));
+            EXHIP_FATAL(exhip_channelwise_nhwc_f16(this->ctx(), EXHIP_CHANNEL_PRELU, mid->gpu_data(), tops[0]->mutable_gpu_data(),
+                                                   static_cast<size_t>(n) * oh * ow, c, this->post_slope_, nullptr,
+                                                   this->post_slope_shared_ ? 1 : 0));
+            return;
+        }
         EXHIP_FATAL(exhip_dwconv3x3_nhwc_f16(this->ctx(), x->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
                                              tops[0]->mutable_gpu_data(), n, c, h, w, c, this->stride_h_, this->pad_top_,
                                              this->pad_bottom_, this->pad_left_, this->pad_right_, this->activation_type_));
@@ -589,6 +630,13 @@ void operation_convolutiondepthwise<Dtype>::forward_gpu_f16(const tensor_list<un
     EXHIP_FATAL(exhip_dwconv3x3_nhwc_f16(this->ctx(), x->gpu_data(), this->weights_f32_[0]->gpu_data(), this->bias_gpu(),
                                          y->mutable_gpu_data(), n, c, h, w, cs, this->stride_h_, this->pad_top_, this->pad_bottom_,
                                          this->pad_left_, this->pad_right_, this->activation_type_));
+    if (this->post_slope_) {  // channel counts off the NHWC layout: the PReLU layer as a launch of its own on the NCHW result
+        auto mid = new_tensor<unsigned short>({n, c, oh, ow}, dev);
+        EXHIP_FATAL(exhip_nhwc_f16_to_nchw_f16(this->ctx(), y->gpu_data(), n, c, oh, ow, cs, mid->mutable_gpu_data()));
+        EXHIP_FATAL(exhip_channelwise_f16(this->ctx(), EXHIP_CHANNEL_PRELU, mid->gpu_data(), tops[0]->mutable_gpu_data(), n, c, oh * ow,
+                                          this->post_slope_, nullptr, this->post_slope_shared_ ? 1 : 0));
+        return;
+    }
     EXHIP_FATAL(exhip_nhwc_f16_to_nchw_f16(this->ctx(), y->gpu_data(), n, c, oh, ow, cs, tops[0]->mutable_gpu_data()));
 }
 

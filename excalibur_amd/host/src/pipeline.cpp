@@ -165,7 +165,7 @@ public:
             if (!in_place && (readers[mid] != 1 || is_result)) continue;
             static const float probe = 0.f;  // any non-null address: asks whether the layer can, sets nothing up for a launch
             if (!(pa.prelu ? conv->set_post_prelu(&probe, true) : conv->set_post_activation(pa.post_op, pa.alpha, pa.beta, pa.relu))) continue;
-            conv->set_post_activation(0, 0.f, 0.f, false);
+            conv->clear_post();
             pa.on = true;
             pair_[i] = pa;
         }
@@ -285,7 +285,7 @@ private:
                     conv->set_post_activation(pair_[i].post_op, pair_[i].alpha, pair_[i].beta, pair_[i].relu);
                 if (link_[i].on) conv->set_quantized_output(link_[i].fs, link_[i].stride, link_[i].only);
                 conv->forward_gpu(in, out);
-                conv->set_post_activation(0, 0.f, 0.f, false);
+                conv->clear_post();
                 conv->set_quantized_output(0.f, 0, false);
                 if (pair_[i].on) {
                     featmaps_[op_outputs_[i][0]] = nullptr;

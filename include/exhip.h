@@ -157,6 +157,15 @@ int exhip_dwconv3x3_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9,
                              int n, int c, int h, int w, int c_stride, int stride, int pt, int pb, int pl, int pr,
                              int act);
 /* operation_convolutiondepthwise::dequantize_int8 (:195-222): wf = w_i8 * (ws <= 1e-6 ? 0 : 1/ws). */
+/* The same followed by the PReLU layer behind it (operation_prelu.cpp:57-124), v >= 0 ? v : slope * v on the value the
+ * depthwise layer stores (the rounded half in the f16 form), slopes per channel or one for all; the layer's own activation
+ * is none. EXHIP_ERR_UNSUPPORTED for shapes only the general kernel takes: run the two layers one after the other then. */
+int exhip_dwconv3x3_nchw_f32_prelu(exhip_ctx* ctx, const float* x, const float* w9, const float* bias, const float* slope,
+                                   int slope_shared, float* y, int n, int c, int h, int w, int stride, int pt, int pb, int pl,
+                                   int pr);
+int exhip_dwconv3x3_nhwc_f16_prelu(exhip_ctx* ctx, const uint16_t* x, const float* w9, const float* bias, const float* slope,
+                                   int slope_shared, uint16_t* y, int n, int c, int h, int w, int cs, int stride, int pt, int pb,
+                                   int pl, int pr);
 int exhip_dw_dequant_weights(exhip_ctx* ctx, const int8_t* w, const float* ws, float* wf, int k, int per_group);
 
 /* operation_pooling::forward_cpu_f32 (src/Excalibur/operation_pooling.cpp:80-208). type 0 max, 1 average.

@@ -270,6 +270,27 @@ def test_depthwise_nhwc_f16(ctx, stride, c, h, w, act):
         assert np.array_equal(got, want32.astype(np.float16).view(np.uint16))
 
 
+@pytest.mark.parametrize("stride,c,h,w,shared", [(1, 24, 28, 32, False), (2, 40, 41, 36, False), (1, 16, 9, 12, True)])
+def test_depthwise_with_the_prelu_layer_behind_it(ctx, stride, c, h, w, shared):
+    """exhip_dwconv3x3_*_prelu: the depthwise layer (no activation of its own) and the PReLU layer behind it in one
+    kernel, against the two restated layers one after the other: float32 bit for bit; half storage with the PReLU on the
+    rounded half, as the fp16 pipeline's two layers compute it."""
+    from excalibur_amd import hip
+    case = cases.conv_f32_case(310 + h, 2, c, h, w, c, 3, stride, 1, act=0, groups=c, dw=True)
+    slope = np.random.default_rng(311).uniform(-0.5, 0.5, 1 if shared else c).astype(np.float32)
+    want = port.prelu(cases.oracle_eval(case), slope)
+    got = ctx.dwconv3x3_nchw_f32_prelu(ctx.array(case["x"]), ctx.array(case["wt"]), ctx.array(case["bias"]), ctx.array(slope), shared,
+                                       stride, 1).download()
+    assert np.array_equal(got, want)
+    x16 = case["x"].astype(np.float16).view(np.uint16)
+    # halves rounded to nearest even, as the hardware conversion of the two separate kernels does
+    mid = cases.oracle_eval(dict(case, x=port.half2float(x16))).astype(np.float16)
+    want16 = port.prelu(mid.astype(np.float32), slope).astype(np.float16).view(np.uint16)
+    x = ctx.nchw_to_nhwc(ctx.array(x16), hip.pad_to(c, 16), "f16")
+    y = ctx.dwconv3x3_nhwc_f16_prelu(x, c, ctx.array(case["wt"]), ctx.array(case["bias"]), ctx.array(slope), shared, stride, 1)
+    assert np.array_equal(ctx.nhwc_to_nchw(y, c, "f16").download(), want16)
+
+
 POOLS = [
     dict(ptype=0, kernel=3, stride=2, pad=1), dict(ptype=0, kernel=5, stride=1, pad=2),
     dict(ptype=0, kernel=9, stride=1, pad=4), dict(ptype=0, kernel=13, stride=1, pad=6),

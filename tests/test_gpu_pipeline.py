@@ -397,7 +397,7 @@ def test_fp16_pipeline_nhwc_resident_equals_nchw_blobs(monkeypatch, which):
     if which == "mobilefacenet":
         from excalibur_amd.mobilenet import MobileFaceNetF32
         net = MobileFaceNetF32(seed=5, hw=32, width=16, blocks=((2, 16, 2), (1, 16, 2), (2, 32, 4)), embed=32)
-        outputs, kinds = [net.output], ("ConvolutionDepthWise", "PReLU", "Eltwise")
+        outputs, kinds = [net.output], ("PReLU", "Eltwise")  # convolution and depthwise blobs live inside their PReLU pair
     else:  # Focus, Concat, nearest Interp, the 5 / 9 / 13 pooling pyramid, heads whose channel count is no multiple of 8
         from excalibur_amd.yolo import YoloV5ShapedF32
         net = YoloV5ShapedF32(seed=7, hw=64, width=8)
@@ -470,10 +470,13 @@ def _activation_pairs_net(seed, int8):
     lines.append("Eltwise sum7 2 1 c7 a7 s7 0=1")
     conv("s7", "c8", 16, 16, 3, 1, groups=16)                             # depthwise: its kernel has no such epilogue
     lines.append("HardSwish hs8 1 1 c8 a8 0=1.666667e-01 1=5.000000e-01")
-    conv("a8", "c9", 16, 16, 1, 1)
+    conv("a8", "c8b", 16, 16, 3, 2, groups=16)                           # depthwise 3x3 + PReLU: one kernel
+    lines.append("PReLU pr8b 1 1 c8b a8b 0=16")
+    blobs.append(mf.floats_blob(r.uniform(-0.5, 0.5, 16).astype(np.float32)))
+    conv("a8b", "c9", 16, 16, 1, 1)
     lines.append("Split sp9 1 2 c9 c9a c9b")
     lines.append("ReLU r9 1 1 c9a a9")                                    # c9b stays a result of the network
-    return lines, blobs, ["a9", "c9b"], ["a1", "a1b", "a1c", "c2", "a3", "a4", "a5", "a6", "a7", "s7", "a8"]
+    return lines, blobs, ["a9", "c9b"], ["a1", "a1b", "a1c", "c2", "a3", "a4", "a5", "a6", "a7", "s7", "a8", "a8b"]
 
 
 @pytest.mark.parametrize("kind", ["f32", "f16", "int8"])
@@ -503,7 +506,7 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
                 except KeyError:
                     assert fusion and kind == "int8"
             if fusion:
-                for gone in ("c1", "c1b", "c1c", "c3", "c4", "c5"):
+                for gone in ("c1", "c1b", "c1c", "c3", "c4", "c5", "c8b"):
                     with pytest.raises(KeyError):
                         p.get(gone)
                 for kept in ("c6", "c7", "c8", "c9b"):
