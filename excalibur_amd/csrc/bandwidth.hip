@@ -924,12 +924,12 @@ __global__ __launch_bounds__(kBlock) void pool2d_nhwc_f16_kernel(const uint16_t*
                 v[t] = *reinterpret_cast<const v4i*>(x + ((n * H + a) * W + min(b0 + t, we - 1)) * cs + g * 8);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
-                if (b0 + t >= we) break;
+                const bool in_window = b0 + t < we;  // a select, not a branch: the loads above stay ahead of all of this
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float f = exhip_h2f((uint16_t)(((uint32_t)v[t][e >> 1] >> ((e & 1) * 16)) & 0xffff));
-                    if (type == 0) acc[e] = acc[e] < f ? f : acc[e];
-                    else acc[e] += f;
+                    const float next = type == 0 ? (acc[e] < f ? f : acc[e]) : acc[e] + f;
+                    acc[e] = in_window ? next : acc[e];
                 }
             }
         }
