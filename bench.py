@@ -71,6 +71,55 @@ def measured_traffic(n, hw):
     return None
 
 
+def network_table(iters=10):
+    """The generated topologies of the other configurations through pipeline<float> / pipeline<unsigned short> layer by
+    layer (every output blob allocated per forward, as in the reference), input resident on the device: wall time per
+    forward over `iters` forwards, device drained before and after. Returns [{"network", "dtype", "ms", "images/s"}]."""
+    import tempfile
+    from excalibur_amd import pipeline as xp
+    from excalibur_amd.mobilenet import MobileFaceNetF32
+    from excalibur_amd.yolo import YoloV5ShapedF32
+    r = np.random.default_rng(0)
+    rows = []
+
+    def run(label, net, x, dtype, pipe_dtype):
+        with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+            path = f.name
+        net.write_model(path)
+        p = xp.Pipeline(net.topology(), path, 0, pipe_dtype)
+        os.unlink(path)
+        p.set_input(x if pipe_dtype == "f32" else x.astype(np.float16).view(np.uint16))
+        for _ in range(3):
+            p.run()
+        p.sync()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            p.run()
+        p.sync()
+        ms = (time.perf_counter() - t0) / iters * 1e3
+        p.close()
+        rows.append({"network": label, "dtype": dtype, "layers": len(net.lines), "ms": round(ms, 3),
+                     "images/s": round(x.shape[0] / ms * 1e3, 1)})
+        print(f"{label:72s} {dtype:5s} {ms:7.2f} ms {x.shape[0] / ms * 1e3:9.0f} images/s", file=sys.stderr, flush=True)
+
+    face = MobileFaceNetF32(hw=112, width=64, blocks=((2, 64, 2), (1, 64, 2), (1, 64, 2), (2, 128, 4), (1, 128, 2), (1, 128, 2),
+                                                     (2, 128, 4), (1, 128, 2)), embed=128)
+    x = r.uniform(0, 255, (64, 3, 112, 112)).astype(np.float32)
+    for dt in ("f32", "f16"):
+        run("MobileFaceNet-shaped (PReLU behind every convolution), 64x3x112x112", face, x, dt, dt)
+    mobile = MobileFaceNetF32(hw=224, width=32, blocks=((2, 64, 2), (1, 64, 2), (2, 128, 2), (1, 128, 2), (2, 256, 2), (1, 256, 2),
+                                                       (1, 256, 2), (2, 512, 2), (1, 512, 2)), embed=128)
+    x = r.uniform(0, 255, (64, 3, 224, 224)).astype(np.float32)
+    for dt in ("f32", "f16"):
+        run("3x3 s2 stem -> 32, dw3x3 + pw1x1 blocks 64..512, residual adds, 64x3x224x224", mobile, x, dt, dt)
+    x = r.uniform(0, 255, (16, 3, 640, 640)).astype(np.float32)
+    yolo = YoloV5ShapedF32(hw=640, width=32)
+    for dt in ("f32", "f16"):
+        run("YOLOv5s-shaped, 16x3x640x640", yolo, x, dt, dt)
+    run("YOLOv5s-shaped, 16x3x640x640", YoloV5ShapedF32(hw=640, width=32, int8=True, outputs=8), x, "int8", "f32")
+    return rows
+
+
 def bandwidth_table(iters=20):
     """The path's memory-bound kernels at the benchmark network's tensor sizes, through the C ABI with preallocated
     operands: HIP events around `iters` back-to-back launches, algorithmic bytes (every operand read once, every result
@@ -163,6 +212,9 @@ def main():
     ap.add_argument("--hw", type=int, default=640)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--per-layer", action="store_true", help="print per-launch timings to stderr")
+    ap.add_argument("--networks", action="store_true",
+                    help="time the other configurations' whole topologies (MobileNet- and YOLOv5s-shaped, f32 / f16 / int8) "
+                         "through the per-layer executor instead of the headline benchmark")
     ap.add_argument("--bandwidth", action="store_true",
                     help="instead of the network: time the memory-bound kernels of the path and print their GB/s")
     args = ap.parse_args()
@@ -174,6 +226,10 @@ def main():
     if args.bandwidth:
         print(json.dumps({"metric": "achieved HBM GB/s of the memory-bound kernels", "peak_GB/s": PEAK_HBM_GBS,
                           "kernels": bandwidth_table()}))
+        return
+    if args.networks:
+        print(json.dumps({"metric": "forward time of the generated topologies through the per-layer executor",
+                          "networks": network_table()}))
         return
 
     import tempfile

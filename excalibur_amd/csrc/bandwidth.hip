@@ -2079,14 +2079,19 @@ extern "C" int exhip_channelwise_f16(exhip_ctx* ctx, int op, const uint16_t* x, 
     REQ_CTX("exhip_channelwise_f16");
     EXHIP_REQUIRE(x && y && p0 && n > 0 && c > 0 && hw > 0, "exhip_channelwise_f16: bad argument");
     EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || p1, "exhip_channelwise_f16: this op needs two parameter arrays");
-    EXHIP_REQUIRE((long long)n * c <= 65535, "exhip_channelwise_f16: more than 65535 (image, channel) planes");
-    switch (op) {
-    case EXHIP_CHANNEL_PRELU: launch_channelwise_f16<0>(ctx, x, y, n, c, hw, p0, p1, shared); break;
-    case EXHIP_CHANNEL_BATCHNORM: launch_channelwise_f16<1>(ctx, x, y, n, c, hw, p0, p1, 0); break;
-    case EXHIP_CHANNEL_INPUT: launch_channelwise_f16<2>(ctx, x, y, n, c, hw, p0, p1, 0); break;
-    default: exhip_set_error("exhip_channelwise_f16: unknown op %d", op); return EXHIP_ERR_ARG;
+    EXHIP_REQUIRE(c <= 65535, "exhip_channelwise_f16: more than 65535 channels");
+    EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || op == EXHIP_CHANNEL_BATCHNORM || op == EXHIP_CHANNEL_INPUT,
+                  "exhip_channelwise_f16: unknown op %d", op);
+    // one block row per (image, channel) plane, at most 65535 rows to a launch: whole images per launch
+    const int per_launch = 65535 / c;
+    for (int n0 = 0; n0 < n; n0 += per_launch) {
+        const int nn = std::min(per_launch, n - n0);
+        const size_t off = (size_t)n0 * c * hw;
+        if (op == EXHIP_CHANNEL_PRELU) launch_channelwise_f16<0>(ctx, x + off, y + off, nn, c, hw, p0, p1, shared);
+        else if (op == EXHIP_CHANNEL_BATCHNORM) launch_channelwise_f16<1>(ctx, x + off, y + off, nn, c, hw, p0, p1, 0);
+        else launch_channelwise_f16<2>(ctx, x + off, y + off, nn, c, hw, p0, p1, 0);
+        EXHIP_LAUNCH_CHECK();
     }
-    EXHIP_LAUNCH_CHECK();
     return 0;
 }
 
@@ -2180,12 +2185,27 @@ extern "C" int exhip_channelwise_nhwc_f16(exhip_ctx* ctx, int op, const uint16_t
     return 0;
 }
 
+static int channelwise_f32_launch(exhip_ctx* ctx, int op, const float* x, float* y, int n, int c, int hw, const float* p0,
+                                  const float* p1, int shared);
+
 extern "C" int exhip_channelwise_f32(exhip_ctx* ctx, int op, const float* x, float* y, int n, int c, int hw, const float* p0,
                                      const float* p1, int shared) {
     REQ_CTX("exhip_channelwise_f32");
     EXHIP_REQUIRE(x && y && p0 && n > 0 && c > 0 && hw > 0, "exhip_channelwise_f32: bad argument");
     EXHIP_REQUIRE(op == EXHIP_CHANNEL_PRELU || p1, "exhip_channelwise_f32: this op needs two parameter arrays");
-    EXHIP_REQUIRE((long long)n * c <= 65535, "exhip_channelwise_f32: more than 65535 (image, channel) planes");
+    EXHIP_REQUIRE(c <= 65535, "exhip_channelwise_f32: more than 65535 channels");
+    // one block row per (image, channel) plane, at most 65535 rows to a launch: whole images per launch
+    const int per_launch = 65535 / c;
+    for (int n0 = 0; n0 < n; n0 += per_launch) {
+        const size_t off = (size_t)n0 * c * hw;
+        const int rc = channelwise_f32_launch(ctx, op, x + off, y + off, std::min(per_launch, n - n0), c, hw, p0, p1, shared);
+        if (rc) return rc;
+    }
+    return 0;
+}
+
+static int channelwise_f32_launch(exhip_ctx* ctx, int op, const float* x, float* y, int n, int c, int hw, const float* p0,
+                                  const float* p1, int shared) {
     if (hw % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) {
         unsigned bx4 = blocks_for((size_t)hw / 4);
         if (bx4 > 64) bx4 = 64;

@@ -392,6 +392,20 @@ def test_channelwise_half_storage_bit_exact(ctx, shape):
     assert np.array_equal(got, _half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.uint16))
 
 
+def test_channelwise_more_planes_than_one_launch_takes(ctx):
+    """A per-channel layer over more than 65535 (image, channel) planes (a launch's limit on block rows) runs as several
+    launches of whole images: 3 images x 30000 channels of PReLU, float32 and half storage, against the closed form."""
+    r = np.random.default_rng(333)
+    x = r.normal(0, 1, (3, 30000, 2, 4)).astype(np.float32)
+    slope = r.uniform(-0.5, 0.5, 30000).astype(np.float32)
+    want = np.where(x >= 0, x, slope[None, :, None, None] * x).astype(np.float32)
+    assert np.array_equal(ctx.channelwise_f32("prelu", ctx.array(x), ctx.array(slope)).download(), want)
+    x16 = _half(x)
+    want16 = _half(np.where(x16 >= 0, x16.astype(np.float32), slope[None, :, None, None] * x16.astype(np.float32)).astype(np.float32))
+    got16 = ctx.channelwise_f16("prelu", ctx.array(x16.view(np.uint16)), ctx.array(slope)).download()
+    assert np.array_equal(got16, want16.view(np.uint16))
+
+
 def test_channelwise_nhwc_half_storage_bit_exact(ctx):
     """PReLU and BatchNorm on the NHWC half tensors the fp16 pipeline keeps between layers == the NCHW layer transposed."""
     shape = (2, 16, 9, 11)
