@@ -1217,7 +1217,7 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
     const int force_abufs = abufs_env ? atoi(abufs_env) : 0;
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
-        if (force_variant >= 0 && variant != force_variant) continue;
+        if (force_variant >= 0 && !pool && !packed && variant != force_variant) continue;  // not the first-layer forms
         if (force_chunk > 0 && !packed && chunk_opt != force_chunk) continue;
         if (pool && variant != 0) continue;  // the pooled epilogue holds one 64-channel slab per group
         if (packed && chunk_opt == 64) continue;
