@@ -1047,10 +1047,20 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 }
                 if (p.residual) {
                     if constexpr (DT == EXHIP_F16) {
+                        // the add layer behind this one reads the stored (rounded) half
                         const uint16_t* r = reinterpret_cast<const uint16_t*>(p.residual) + pix * p.kstride + ch0;
+                        if (ch0 + 16 <= p.K) {  // 32 aligned bytes: two loads
+                            const v4i r0 = reinterpret_cast<const v4i*>(r)[0], r1 = reinterpret_cast<const v4i*>(r)[1];
 #pragma unroll
-                        for (int e = 0; e < 16; ++e)
-                            if (ch0 + e < p.K) v[e] += exhip_h2f(r[e]);
+                            for (int e = 0; e < 16; ++e) {
+                                const int word = e < 8 ? r0[e >> 1] : r1[(e - 8) >> 1];
+                                v[e] = exhip_h2f(exhip_f2h(v[e])) + exhip_h2f((uint16_t)(((uint32_t)word >> ((e & 1) * 16)) & 0xffff));
+                            }
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 16; ++e)
+                                if (ch0 + e < p.K) v[e] = exhip_h2f(exhip_f2h(v[e])) + exhip_h2f(r[e]);
+                        }
                     } else {
                         const float* r = reinterpret_cast<const float*>(p.residual) + pix * p.kstride + ch0;
 #pragma unroll

@@ -170,6 +170,36 @@ public:
             pair_[i] = pa;
         }
         find_quantized_links();
+        find_sum_pairs();
+    }
+
+    // fp16 pipeline: a convolution whose only reader is the two-input sum on the next line (Eltwise SUM with unit
+    // coefficients, BinaryOp ADD of two blobs: the residual add of a bottleneck block) adds the other operand in its
+    // epilogue, to its own result rounded to half as the sum layer would read it. Whether it can is known only when the
+    // blobs are there (both NHWC, same shape), so the convolution reports it and the sum layer runs if it could not.
+    void find_sum_pairs() {
+        sum_other_.assign(operations_.size(), -1);
+        if constexpr (std::is_same_v<Dtype, unsigned short>) {
+            std::vector<int> readers(blob_names_.size(), 0);
+            for (const auto& in : op_inputs_)
+                for (int b : in) ++readers[b];
+            for (size_t i = 0; i + 1 < operations_.size(); ++i) {
+                auto* conv = dynamic_cast<operation_convolution<Dtype>*>(operations_[i].get());
+                if (!conv || dynamic_cast<operation_convolutiondepthwise<Dtype>*>(conv) || pair_[i].on) continue;
+                if (op_outputs_[i].size() != 1 || op_inputs_[i + 1].size() != 2 || op_outputs_[i + 1].size() != 1) continue;
+                const int mid = op_outputs_[i][0];
+                const int a = op_inputs_[i + 1][0], b = op_inputs_[i + 1][1];
+                if ((a == mid) == (b == mid)) continue;  // exactly one operand is the convolution's blob
+                bool plain_sum = false;
+                if (auto* e = dynamic_cast<operation_eltwise<Dtype>*>(operations_[i + 1].get()))
+                    plain_sum = e->type_ == 1 && e->coeffs_.size() == 2 && e->coeffs_[0] == 1.f && e->coeffs_[1] == 1.f;
+                else if (auto* bo = dynamic_cast<operation_binaryop<Dtype>*>(operations_[i + 1].get()))
+                    plain_sum = bo->op_type_ == 0 && !bo->with_scalar_;
+                if (!plain_sum || readers[mid] != 1 || op_outputs_[i + 1][0] == mid) continue;
+                if (std::find(output_names_.begin(), output_names_.end(), blob_names_[mid]) != output_names_.end()) continue;
+                sum_other_[i] = a == mid ? b : a;
+            }
+        }
     }
 
     // An int8 convolution whose result is read by int8 convolutions writes the int8 NHWC tensor those readers would
@@ -277,6 +307,23 @@ private:
                 if (!featmaps_[b]) LOG(FATAL) << "layer " << op_params_[i].name_ << " reads blob " << blob_names_[b] << " before it is produced";
                 in.push_back(featmaps_[b]);
             }
+            if constexpr (std::is_same_v<Dtype, unsigned short>) {
+                if (fusion_ && sum_other_[i] >= 0 && featmaps_[sum_other_[i]]) {
+                    auto* conv = static_cast<operation_convolution<Dtype>*>(operations_[i].get());
+                    conv->set_post_sum(featmaps_[sum_other_[i]]);
+                    conv->forward_gpu(in, out);
+                    const bool summed = conv->post_sum_used();
+                    conv->clear_post();
+                    if (summed) {
+                        featmaps_[op_outputs_[i][0]] = nullptr;
+                        featmaps_[op_outputs_[i + 1][0]] = out[0];
+                        ++i;  // the sum layer has run
+                    } else {
+                        featmaps_[op_outputs_[i][0]] = out[0];
+                    }
+                    continue;
+                }
+            }
             if (fusion_ && (pair_[i].on || link_[i].on)) {
                 auto* conv = static_cast<operation_convolution<Dtype>*>(operations_[i].get());
                 if (pair_[i].on && pair_[i].prelu)
@@ -335,6 +382,7 @@ private:
         float fs = 0.f;
         int stride = 0;
     };
+    std::vector<int> sum_other_;         // per layer: the other operand's blob of the sum layer this convolution absorbs, or -1
     std::vector<quantized_link> link_;   // per layer: an int8 convolution that writes its readers' int8 input
     int weights_mem_cost_ = 0;
 };

@@ -132,7 +132,9 @@ int exhip_conv2d_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_desc* d, int p
 
 /* operation_convolution::forward_cpu_f32 (src/Excalibur/operation_convolution.cpp:251-329) with fp16
  * storage and f32 accumulation (include/Excalibur/operation.hpp:234-260 describes the fp16 layer):
- * x NHWC f16; outputs NHWC f16 and/or NCHW f16 and/or NCHW f32; residual NHWC f16. */
+ * x NHWC f16; outputs NHWC f16 and/or NCHW f16 and/or NCHW f32. residual_nhwc (NHWC f16, the output's shape and
+ * stride) is the other operand of the two-input sum layer behind the convolution (operation_eltwise.cpp:43-94 SUM,
+ * operation_binaryop.cpp:75-84): added to the layer's result rounded to half, as that layer would read it. */
 int exhip_conv2d_f16(exhip_ctx* ctx, const exhip_conv_desc* d, const uint16_t* x_nhwc, const void* w_packed,
                      const float* bias, const uint16_t* residual_nhwc, uint16_t* y_f16_nhwc, uint16_t* y_f16_nchw,
                      float* y_f32_nchw);

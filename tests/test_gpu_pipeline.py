@@ -473,10 +473,14 @@ def _activation_pairs_net(seed, int8):
     conv("a8", "c8b", 16, 16, 3, 2, groups=16)                           # depthwise 3x3 + PReLU: one kernel
     lines.append("PReLU pr8b 1 1 c8b a8b 0=16")
     blobs.append(mf.floats_blob(r.uniform(-0.5, 0.5, 16).astype(np.float32)))
-    conv("a8b", "c9", 16, 16, 1, 1)
+    conv("a8b", "c8c", 16, 16, 1, 1)                                      # fp16: the sum behind it joins its epilogue
+    lines.append("Eltwise sum8 2 1 c8c a8b s8 0=1")
+    conv("s8", "c8d", 16, 16, 3, 1)
+    lines.append("BinaryOp add8 2 1 s8 c8d s8d 0=0")                      # the convolution's blob as second operand
+    conv("s8d", "c9", 16, 16, 1, 1)
     lines.append("Split sp9 1 2 c9 c9a c9b")
     lines.append("ReLU r9 1 1 c9a a9")                                    # c9b stays a result of the network
-    return lines, blobs, ["a9", "c9b"], ["a1", "a1b", "a1c", "c2", "a3", "a4", "a5", "a6", "a7", "s7", "a8", "a8b"]
+    return lines, blobs, ["a9", "c9b"], ["a1", "a1b", "a1c", "c2", "a3", "a4", "a5", "a6", "a7", "s7", "a8", "a8b", "s8", "s8d"]
 
 
 @pytest.mark.parametrize("kind", ["f32", "f16", "int8"])
@@ -509,6 +513,12 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
                 for gone in ("c1", "c1b", "c1c", "c3", "c4", "c5", "c8b"):
                     with pytest.raises(KeyError):
                         p.get(gone)
+                for summed in ("c8c", "c8d"):  # the residual adds: in the convolution only on NHWC half blobs
+                    if kind == "f16":
+                        with pytest.raises(KeyError):
+                            p.get(summed)
+                    else:
+                        p.get(summed)
                 for kept in ("c6", "c7", "c8", "c9b"):
                     p.get(kept)
             p.close()
