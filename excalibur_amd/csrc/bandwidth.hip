@@ -1752,7 +1752,9 @@ static int dw_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const
     if ((stride == 1 || stride == 2) && (act == 0 || act == 1 || act == 3) && x_bytes <= desc_limit && y_bytes <= desc_limit) {
         // bands of output rows: about fourteen rows each (the per-thread set-up is worth several rows of work),
         // shorter where that would leave fewer than four waves for every compute unit
-        const int px = stride == 1 ? 4 : 3;
+        // stride 2: strips of two pixels (five input columns a row); three pixels (seven columns) sit at the register
+        // limit of four waves per SIMD, spill with the PReLU epilogue, and measured slower without it
+        const int px = stride == 1 ? 4 : 2;
         const int strips = (ow + px - 1) / px;
         const size_t per_band = (size_t)n * strips * (cs / 4);
         static const int env_rows = getenv("EXHIP_DW_BAND_ROWS") ? atoi(getenv("EXHIP_DW_BAND_ROWS")) : 0;
@@ -1772,10 +1774,10 @@ static int dw_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const
             else if (act == 1) EXHIP_DW_STRIP(1, 4, 1);
             else EXHIP_DW_STRIP(1, 4, 3);
         } else {
-            if (slope) EXHIP_DW_STRIP(2, 3, kDwPrelu);
-            else if (act == 0) EXHIP_DW_STRIP(2, 3, 0);
-            else if (act == 1) EXHIP_DW_STRIP(2, 3, 1);
-            else EXHIP_DW_STRIP(2, 3, 3);
+            if (slope) EXHIP_DW_STRIP(2, 2, kDwPrelu);
+            else if (act == 0) EXHIP_DW_STRIP(2, 2, 0);
+            else if (act == 1) EXHIP_DW_STRIP(2, 2, 1);
+            else EXHIP_DW_STRIP(2, 2, 3);
         }
 #undef EXHIP_DW_STRIP
         EXHIP_LAUNCH_CHECK();
