@@ -1750,16 +1750,17 @@ static int dw_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const
     const size_t x_bytes = (size_t)n * h * w * cs * 2, y_bytes = (size_t)n * oh * ow * cs * 2;
     const size_t desc_limit = (size_t)1 << 30;
     if ((stride == 1 || stride == 2) && (act == 0 || act == 1 || act == 3) && x_bytes <= desc_limit && y_bytes <= desc_limit) {
-        // bands of output rows: about fourteen rows each (the per-thread set-up is worth several rows of work),
-        // shorter where that would leave fewer than four waves for every compute unit
+        // bands of output rows: about fourteen rows each (the per-thread set-up and the two halo rows are worth several
+        // rows of work), shorter where that would leave fewer than fourteen waves for every compute unit, never under
+        // seven rows (measured at 64x128x56x56: 7 rows beat 4, 10, 14 and 28 at both strides)
         // stride 2: strips of two pixels (five input columns a row); three pixels (seven columns) sit at the register
         // limit of four waves per SIMD, spill with the PReLU epilogue, and measured slower without it
         const int px = stride == 1 ? 4 : 2;
         const int strips = (ow + px - 1) / px;
         const size_t per_band = (size_t)n * strips * (cs / 4);
         static const int env_rows = getenv("EXHIP_DW_BAND_ROWS") ? atoi(getenv("EXHIP_DW_BAND_ROWS")) : 0;
-        const size_t want = (size_t)256 * 4 * 64;
-        int bands = (int)std::min<size_t>((size_t)oh, std::max<size_t>((oh + 13) / 14, (want + per_band - 1) / per_band));
+        const size_t want = (size_t)256 * 14 * 64;
+        int bands = (int)std::min<size_t>((size_t)std::max(1, oh / 7), std::max<size_t>((oh + 13) / 14, (want + per_band - 1) / per_band));
         int band_rows = (oh + bands - 1) / bands;
         if (env_rows > 0) band_rows = std::min(env_rows, oh);
         bands = (oh + band_rows - 1) / band_rows;
