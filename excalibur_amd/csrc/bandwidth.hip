@@ -1684,7 +1684,8 @@ static int dw_nchw_f32(exhip_ctx* ctx, const float* x, const float* w9, const fl
         const int strips = (ow + 3) / 4;
         const size_t per_band = (size_t)n * c * strips;
         const size_t want = (size_t)256 * 8 * 64;
-        int bands = (int)std::min<size_t>((size_t)oh, std::max<size_t>((oh + 15) / 16, (want + per_band - 1) / per_band));
+        // about eight rows to a band (measured at 32x64x160x160: 5 to 10 rows 65 % of the HBM peak, 16 rows 61 %, 20 and more 59 %)
+        int bands = (int)std::min<size_t>((size_t)oh, std::max<size_t>((oh + 7) / 8, (want + per_band - 1) / per_band));
         static const int env_rows = getenv("EXHIP_DW_BAND_ROWS") ? atoi(getenv("EXHIP_DW_BAND_ROWS")) : 0;
         int band_rows = (oh + bands - 1) / bands;
         if (env_rows > 0) band_rows = std::min(env_rows, oh);
