@@ -5,6 +5,8 @@
 // saxpby rounding), so these kernels are bit-exact against it in fp32.
 #include <float.h>
 
+#include <mutex>
+
 #include "common.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -2154,6 +2156,51 @@ extern "C" int exhip_maxpool_same_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, ui
 #undef EXHIP_SAME_POOL
     EXHIP_LAUNCH_CHECK();
     return 0;
+}
+
+// ---- the one entry point that allocates nothing ----
+// The row pass of the separable pooling above needs an intermediate tensor of the input's size. For callers that cannot
+// allocate device memory (code under graph capture, serving loops, harnesses that forbid hipMalloc) it lives in this
+// file-scope device array: each GPU the library runs on holds its own copy until the process ends.
+static constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// The array's name is only a host-side handle; its device address differs per GPU and is looked up once per device,
+// with that device current (exhip_init does so), and kept here.
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {};
+
+int exhip_static_scratch_setup(int device) {
+    EXHIP_REQUIRE(device >= 0 && device < kMaxDevices, "static scratch: device %d out of range", device);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[device]) return 0;
+    void* ptr = nullptr;
+    EXHIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    EXHIP_REQUIRE(ptr != nullptr && (reinterpret_cast<uintptr_t>(ptr) & 255) == 0, "static scratch: bad device address %p", ptr);
+    g_scratch_ptr[device] = ptr;
+    return 0;
+}
+
+extern "C" size_t exhip_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int exhip_maxpool_same_nhwc_f16_static(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int k) {
+    REQ_CTX("exhip_maxpool_same_nhwc_f16_static");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && c % 8 == 0 && h > 0 && w > 0, "exhip_maxpool_same_nhwc_f16_static: bad argument");
+    const size_t bytes = (size_t)n * h * w * c * sizeof(uint16_t);
+    EXHIP_REQUIRE(bytes <= kStaticScratchBytes,
+                  "exhip_maxpool_same_nhwc_f16_static: the tensor has %zu bytes, the static scratch array holds %zu; use "
+                  "exhip_maxpool_same_nhwc_f16 with a workspace of the caller's",
+                  bytes, kStaticScratchBytes);
+    EXHIP_REQUIRE(ctx->device >= 0 && ctx->device < kMaxDevices, "exhip_maxpool_same_nhwc_f16_static: device %d out of range", ctx->device);
+    void* ptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        ptr = g_scratch_ptr[ctx->device];
+    }
+    EXHIP_REQUIRE(ptr != nullptr, "exhip_maxpool_same_nhwc_f16_static: device %d was not set up by exhip_init", ctx->device);
+    // The row pass writes every element of the part of the array the column pass reads: nothing needs clearing.
+    return exhip_maxpool_same_nhwc_f16(ctx, x, static_cast<uint16_t*>(ptr), y, n, c, h, w, k);
 }
 
 extern "C" int exhip_channelwise_nhwc_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16_t* y, size_t pixels, int c,

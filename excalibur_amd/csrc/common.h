@@ -13,6 +13,10 @@ struct exhip_ctx {
 
 void exhip_set_error(const char* fmt, ...);
 
+// Looks up, once per device and with that device current, the address of the static scratch array behind
+// exhip_maxpool_same_nhwc_f16_static (defined beside that array).
+int exhip_static_scratch_setup(int device);
+
 #define EXHIP_CHECK(expr)                                                                          \
     do {                                                                                           \
         hipError_t e_ = (expr);                                                                    \

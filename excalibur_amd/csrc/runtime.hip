@@ -27,6 +27,8 @@ extern "C" int exhip_init(int device, exhip_ctx** out) {
         exhip_set_error("exhip_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
         return EXHIP_ERR_UNSUPPORTED;
     }
+    const int rc = exhip_static_scratch_setup(device);
+    if (rc != 0) return rc;
     exhip_ctx* c = new exhip_ctx();
     c->device = device;
     hipError_t e = hipStreamCreate(&c->stream);  // default priority

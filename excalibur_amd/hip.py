@@ -39,6 +39,7 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         L.exhip_last_error.restype = ctypes.c_char_p
         L.exhip_conv_packed_bytes.restype = ctypes.c_size_t
+        L.exhip_static_scratch_bytes.restype = ctypes.c_size_t
         _lib = L
     return _lib
 
@@ -309,6 +310,20 @@ class Ctx:
         y = self.empty((n, oh, ow, cs), np.uint16)
         _check(lib().exhip_pool2d_nhwc_f16(self.h, x.ptr, y.ptr, n, c, h, w, cs, oh, ow, ptype, kh, kw, sh, sw, pt, pb, pl, pr,
                                            count_include_pad))
+        return y
+
+    def maxpool_same_nhwc_f16(self, x, k, y=None, tmp=None):
+        """Stride-1 max pooling with window k and padding k // 2 on an NHWC half tensor; tmp is the caller's workspace."""
+        n, h, w, c = x.shape
+        y = y if y is not None else self.empty(x.shape, np.uint16)
+        tmp = tmp if tmp is not None else self.empty(x.shape, np.uint16)
+        _check(lib().exhip_maxpool_same_nhwc_f16(self.h, x.ptr, tmp.ptr, y.ptr, n, c, h, w, int(k)))
+        return y
+
+    def maxpool_same_nhwc_f16_static(self, x, k, y):
+        """The same through the entry point that allocates nothing: y is preallocated by the caller."""
+        n, h, w, c = x.shape
+        _check(lib().exhip_maxpool_same_nhwc_f16_static(self.h, x.ptr, y.ptr, n, c, h, w, int(k)))
         return y
 
     def eltwise_f32(self, inputs, etype, coeffs=None):

@@ -244,6 +244,13 @@ int exhip_concat_channels_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs
                                    size_t pixels, uint16_t* y);
 int exhip_interp_nearest_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int oh, int ow);
 int exhip_maxpool_same_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* tmp, uint16_t* y, int n, int c, int h, int w, int k);
+/* exhip_maxpool_same_nhwc_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. The row pass's intermediate tensor
+ * lives in a static device array of exhip_static_scratch_bytes() bytes (8 MiB) per GPU instead of a caller workspace;
+ * a tensor of more than that many bytes (n*h*w*c*2) is refused with EXHIP_ERR_ARG. The call allocates and frees
+ * nothing. All calls on one GPU share that array: calls that overlap on one GPU (two contexts, two threads) race. */
+size_t exhip_static_scratch_bytes(void);
+int exhip_maxpool_same_nhwc_f16_static(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int k);
 /* operation_concat::forward_cpu_f32 along the channel axis (operation_concat.cpp:31-103): inputs is a host array of
  * device pointers to NCHW tensors [n][channels[i]][hw]. */
 int exhip_concat_channels_f32(exhip_ctx* ctx, const float* const* inputs, const int* channels, int n_inputs, int n, int hw,
