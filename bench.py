@@ -77,7 +77,7 @@ def network_table(iters=10):
     forward over `iters` forwards, device drained before and after. Returns [{"network", "dtype", "ms", "images/s"}]."""
     import tempfile
     from excalibur_amd import pipeline as xp
-    from excalibur_amd.mobilenet import MobileFaceNetF32
+    from excalibur_amd.mobilenet import CFG3, MobileFaceNetF32
     from excalibur_amd.yolo import YoloV5ShapedF32
     r = np.random.default_rng(0)
     rows = []
@@ -107,8 +107,7 @@ def network_table(iters=10):
     x = r.uniform(0, 255, (64, 3, 112, 112)).astype(np.float32)
     for dt in ("f32", "f16"):
         run("MobileFaceNet-shaped (PReLU behind every convolution), 64x3x112x112", face, x, dt, dt)
-    mobile = MobileFaceNetF32(hw=224, width=32, blocks=((2, 64, 2), (1, 64, 2), (2, 128, 2), (1, 128, 2), (2, 256, 2), (1, 256, 2),
-                                                       (1, 256, 2), (2, 512, 2), (1, 512, 2)), embed=128)
+    mobile = MobileFaceNetF32(**CFG3)
     x = r.uniform(0, 255, (64, 3, 224, 224)).astype(np.float32)
     for dt in ("f32", "f16"):
         run("3x3 s2 stem -> 32, dw3x3 + pw1x1 blocks 64..512, residual adds, 64x3x224x224", mobile, x, dt, dt)

@@ -53,10 +53,12 @@ public:
     }
 };
 
-// This backend instantiates pipeline<float> and pipeline<unsigned short>; the reference also has
-// pipeline<double>, whose operators are all unimplemented on its CPU path as well.
-#define INSTANCE_CLASS(CLASS_NAME)    \
-    template class CLASS_NAME<float>; \
+// The three element types of the reference (operation_reflector.hpp:55-93). Operators of a pipeline<double> can be
+// created and loaded; their forward is NOT_IMPLEMENTED, as the reference's forward_*_d64 defaults are
+// (include/Excalibur/operation.hpp:185-201).
+#define INSTANCE_CLASS(CLASS_NAME)     \
+    template class CLASS_NAME<float>;  \
+    template class CLASS_NAME<double>; \
     template class CLASS_NAME<unsigned short>;
 
 #define REGISTE_SHORT(CLASS_NAME)                                                                  \
@@ -69,9 +71,15 @@ public:
         #CLASS_NAME, [](const operation_param& param) -> std::shared_ptr<operation<float>> { \
             return std::make_shared<CLASS_NAME<float>>(param);                       \
         });
-#define REGISTE(CLASS_NAME)  \
+#define REGISTE_DOUBLE(CLASS_NAME)                                                     \
+    register_action<double> g_d_register_action_##CLASS_NAME(                         \
+        #CLASS_NAME, [](const operation_param& param) -> std::shared_ptr<operation<double>> { \
+            return std::make_shared<CLASS_NAME<double>>(param);                       \
+        });
+#define REGISTE(CLASS_NAME)   \
     REGISTE_SHORT(CLASS_NAME) \
-    REGISTE_FLOAT(CLASS_NAME)
+    REGISTE_FLOAT(CLASS_NAME) \
+    REGISTE_DOUBLE(CLASS_NAME)
 
 }  // namespace excalibur
 }  // namespace glasssix

@@ -19,6 +19,7 @@ public:
     class impl;
     using blob_map = std::unordered_map<std::string, std::shared_ptr<memory::tensor<Dtype>>>;
 
+    explicit pipeline();
     explicit pipeline(std::string_view param_file, std::string_view model_file, int device = -1);
     explicit pipeline(std::string_view param_file, int device = -1);
     explicit pipeline(const std::vector<std::string>& hardcode_params, std::string_view model_file, int device = -1);
@@ -33,9 +34,11 @@ public:
     void disable_profiler();
 
     // Backend switch without a counterpart in the reference: run int8 convolution chains with fused
-    // epilogues and int8 NHWC tensors between layers (default on). Intermediate blobs are then not
-    // materialised as float tensors; get_featmap() returns pipeline outputs only.
+    // epilogues and int8 NHWC tensors between layers, let convolutions absorb the activation / sum layer
+    // behind them (default on). A forward then stores only some blobs as float tensors; get_featmap() of
+    // another blob runs the last input once more layer by layer. blob_stored() tells the two apart.
     void set_fusion(bool on);
+    bool blob_stored(std::string_view featmap_name) const;
     bool fused() const;
     double last_forward_ms() const;
     // Device time of part of a fused forward: with first_launch >= 0 every fused forward records one event in front

@@ -18,6 +18,8 @@ struct exc_pipeline {
     std::shared_ptr<tensor<unsigned short>> in16;
     pipeline<float>::blob_map out32;
     pipeline<unsigned short>::blob_map out16;
+    std::vector<pipeline<float>::blob_map> kept32;  // results of earlier forwards held on purpose (exc_pipeline_run_keeping)
+    std::vector<pipeline<unsigned short>::blob_map> kept16;
 };
 
 namespace {
@@ -62,10 +64,25 @@ extern "C" exc_pipeline* exc_pipeline_create(const char* topology, const char* m
     return p;
 }
 
+extern "C" exc_pipeline* exc_pipeline_create_from_files(const char* param_file, const char* model_file, int device, int dtype) {
+    auto* p = new exc_pipeline();
+    p->dtype = dtype;
+    p->device = device;
+    const bool dummy = !model_file || !*model_file;
+    if (dtype == 0) p->f32.reset(dummy ? new pipeline<float>(param_file, device) : new pipeline<float>(param_file, model_file, device));
+    else p->f16.reset(dummy ? new pipeline<unsigned short>(param_file, device) : new pipeline<unsigned short>(param_file, model_file, device));
+    return p;
+}
+
 extern "C" void exc_pipeline_destroy(exc_pipeline* p) { delete p; }
 
 extern "C" void exc_pipeline_set_fusion(exc_pipeline* p, int on) {
     if (p->f32) p->f32->set_fusion(on != 0);
+    if (p->f16) p->f16->set_fusion(on != 0);
+}
+
+extern "C" int exc_pipeline_blob_stored(exc_pipeline* p, const char* name) {
+    return p->f32 ? p->f32->blob_stored(name) : p->f16 ? p->f16->blob_stored(name) : 0;
 }
 
 extern "C" int exc_pipeline_last_fused(exc_pipeline* p) { return p->f32 ? p->f32->fused() : 0; }
@@ -86,9 +103,54 @@ extern "C" int exc_pipeline_set_input(exc_pipeline* p, const void* input, const 
 }
 
 extern "C" int exc_pipeline_run(exc_pipeline* p) {
-    if (p->dtype == 0) p->out32 = p->f32->forward(p->in32);
-    else p->out16 = p->f16->forward(p->in16);
+    // the previous results are released first: a result still held when a forward starts stays its holder's, and the
+    // pipeline would write into newly allocated tensors
+    if (p->dtype == 0) {
+        p->out32.clear();
+        p->out32 = p->f32->forward(p->in32);
+    } else {
+        p->out16.clear();
+        p->out16 = p->f16->forward(p->in16);
+    }
     return 0;
+}
+
+extern "C" int exc_pipeline_run_keeping(exc_pipeline* p) {
+    if (p->dtype == 0) {
+        p->kept32.push_back(std::move(p->out32));
+        p->out32 = p->f32->forward(p->in32);
+    } else {
+        p->kept16.push_back(std::move(p->out16));
+        p->out16 = p->f16->forward(p->in16);
+    }
+    return 0;
+}
+
+extern "C" long exc_pipeline_get_kept(exc_pipeline* p, int back, const char* name, void* out, long capacity, int shape[4]) {
+    std::shared_ptr<tensor<float>> t32;
+    std::shared_ptr<tensor<unsigned short>> t16;
+    if (back < 1) return -1;
+    if (p->dtype == 0) {
+        if (static_cast<size_t>(back) > p->kept32.size()) return -1;
+        auto& m = p->kept32[p->kept32.size() - back];
+        auto it = m.find(name);
+        if (it == m.end()) return -1;
+        t32 = it->second;
+    } else {
+        if (static_cast<size_t>(back) > p->kept16.size()) return -1;
+        auto& m = p->kept16[p->kept16.size() - back];
+        auto it = m.find(name);
+        if (it == m.end()) return -1;
+        t16 = it->second;
+    }
+    const std::vector<int> s = t32 ? t32->data_shape() : t16->data_shape();
+    for (int i = 0; i < 4; ++i) shape[i] = s[i];
+    const long n = t32 ? t32->count() : t16->count();
+    if (out && n <= capacity) {
+        if (t32) std::memcpy(out, t32->cpu_data(), sizeof(float) * static_cast<size_t>(n));
+        else std::memcpy(out, t16->cpu_data(), sizeof(unsigned short) * static_cast<size_t>(n));
+    }
+    return n;
 }
 
 extern "C" int exc_pipeline_sync(exc_pipeline* p) { return exhip_sync(glasssix::memory::device_context(p->device)); }
@@ -106,8 +168,9 @@ extern "C" long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, l
 
 extern "C" size_t exc_registered_operations(int dtype, char* buf, size_t len) {
     std::string all;
-    const std::vector<std::string> names = dtype == 0 ? glasssix::excalibur::operation_reflector<float>::instance().registered()
-                                                      : glasssix::excalibur::operation_reflector<unsigned short>::instance().registered();
+    const std::vector<std::string> names = dtype == 0   ? glasssix::excalibur::operation_reflector<float>::instance().registered()
+                                           : dtype == 1 ? glasssix::excalibur::operation_reflector<unsigned short>::instance().registered()
+                                                        : glasssix::excalibur::operation_reflector<double>::instance().registered();
     for (const std::string& n : names) all += n + "\n";
     if (buf && len) {
         std::strncpy(buf, all.c_str(), len - 1);

@@ -59,7 +59,16 @@ template <>
 void operation<unsigned short>::forward_gpu(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
     forward_gpu_f16(bottoms, tops);
 }
+// pipeline<double>: the reference dispatches to forward_*_d64, which no operator of this path overrides
+// (include/Excalibur/operation.hpp:185-201): NOT_IMPLEMENTED.
+template <>
+void operation<double>::forward_cpu(const tensor_list<double>&, tensor_list<double>&) { NO_CPU; }
+template <>
+void operation<double>::forward_gpu(const tensor_list<double>&, tensor_list<double>&) {
+    NOT_IMPLEMENTED << " double-precision layers have no forward";
+}
 template class operation<float>;
+template class operation<double>;
 template class operation<unsigned short>;
 
 namespace {
@@ -434,7 +443,10 @@ void operation_convolution<Dtype>::forward_gpu_i8(const tensor_list<float>& bott
     const int dev = this->params_.device_;
     const int n = bottoms[0]->num(), c = bottoms[0]->channels(), h = bottoms[0]->height(), w = bottoms[0]->width();
     CHECK_EQ(c, this->input_channels());
-    CHECK_EQ(this->featmap_scaletable_i8_->count(), 1) << "per-channel feature-map scales are not supported";
+    // Both loaders of the reference give a convolution exactly one feature-map scale (model file: operation_convolution.cpp:130-131,
+    // dummy weights: :230-231), so the per-input-channel branch of its quantizer (operation_general_conv.cpp:596) cannot be
+    // reached through this operator; the quantizer entry point of the C ABI covers that branch on its own.
+    CHECK_EQ(this->featmap_scaletable_i8_->count(), 1) << "a convolution carries one feature-map scale";
     exhip_conv_desc d = describe(n, h, w, c, this->output_channel_);
     int oh, ow;
     EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
@@ -1128,8 +1140,12 @@ int operation_prelu<Dtype>::init_weights(FILE* fp) {
 template <typename Dtype>
 int operation_prelu<Dtype>::init_weights() {
     this->weights_f32_.push_back(vec_tensor<float>(num_slope_, this->params_.device_));
+    // dummy weights as the reference draws them (src/Excalibur/operation_prelu.cpp:45-55): |N(0, 0.3)| from a
+    // default-seeded engine
+    std::default_random_engine e;
+    std::normal_distribution<float> n(0, 0.3);
     float* s = this->weights_f32_[0]->mutable_cpu_data();
-    for (int i = 0; i < num_slope_; ++i) s[i] = 0.25f;  // dummy weights
+    for (int i = 0; i < num_slope_; ++i) s[i] = std::fabs(n(e));
     return num_slope_ * static_cast<int>(sizeof(float));
 }
 
@@ -1207,11 +1223,14 @@ int operation_batchnorm<Dtype>::init_weights(FILE* fp) {
 
 template <typename Dtype>
 int operation_batchnorm<Dtype>::init_weights() {
-    const float init[4] = {1.f, 0.f, 1.f, 0.f};  // dummy weights: identity
+    // dummy weights as the reference draws them (src/Excalibur/operation_batchnorm.cpp:69-121): slope, mean, var and
+    // bias are N(0, 0.3) from one default-seeded engine; a negative var gives NaN there and here
+    std::default_random_engine e;
+    std::normal_distribution<float> n(0, 0.3);
     for (int k = 0; k < 4; ++k) {
         this->weights_f32_.push_back(vec_tensor<float>(channels_, this->params_.device_));
         float* p = this->weights_f32_[k]->mutable_cpu_data();
-        for (int i = 0; i < channels_; ++i) p[i] = init[k];
+        for (int i = 0; i < channels_; ++i) p[i] = n(e);
     }
     fold();
     return channels_ * static_cast<int>(sizeof(float)) * 4;
@@ -1590,11 +1609,16 @@ template <typename Dtype>
 int operation_deconvolution<Dtype>::init_weights() {
     if (this->params_.int8_quantization_) NOT_IMPLEMENTED;
     this->weights_f32_.push_back(vec_tensor<float>(this->weight_data_size_, this->params_.device_));
+    // dummy weights as the reference draws them (src/Excalibur/operation_deconvolution.cpp:44-76)
+    std::default_random_engine e;
+    std::normal_distribution<float> n(0, 0.3);
     float* w = this->weights_f32_[0]->mutable_cpu_data();
-    for (int i = 0; i < this->weight_data_size_; ++i) w[i] = 0.01f * static_cast<float>((i % 7) - 3);  // dummy weights
+    for (int i = 0; i < this->weight_data_size_; ++i) w[i] = n(e);
     int mem = this->weight_data_size_ * static_cast<int>(sizeof(float));
     if (this->bias_term_) {
         this->weights_f32_.push_back(vec_tensor<float>(this->output_channel_, this->params_.device_));
+        float* b = this->weights_f32_[1]->mutable_cpu_data();
+        for (int i = 0; i < this->output_channel_; ++i) b[i] = n(e);
         mem += this->output_channel_ * static_cast<int>(sizeof(float));
     }
     return mem;

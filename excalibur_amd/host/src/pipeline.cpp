@@ -16,6 +16,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstring>
+#include <deque>
 #include <fstream>
 #include <functional>
 #include <map>
@@ -58,6 +59,8 @@ template <typename Dtype>
 class pipeline<Dtype>::impl {
 public:
     using tensor_ptr = std::shared_ptr<tensor<Dtype>>;
+
+    impl() : device_(-1) {}  // the reference's default-constructed pipeline (pipeline.cpp:575-577): no layers; forward is fatal
 
     impl(const std::vector<std::string>& lines, std::string_view model_file, int device) : device_(device) {
         if (device >= 0) memory::device_context(device);  // opens the device, fatal if it is not an MI355X
@@ -267,12 +270,34 @@ public:
         return results;
     }
 
+    // A blob of the last forward by name, NCHW (nullptr for an unknown name, as in the reference). The fused executors
+    // do not store every blob (a fused plan keeps int8 tensors between layers, a convolution absorbs the activation or
+    // sum behind it, int8 readers get an int8 form only): asking for such a blob runs the last input once more through the
+    // per-layer executor with fusion off, which stores them all, so what comes back always belongs to the last input.
     tensor_ptr get_featmap(std::string_view name) {
         auto it = blob_index_.find(std::string(name));
         if (it == blob_index_.end()) return nullptr;
+        auto missing = [&]() {
+            const tensor_ptr& t = featmaps_[it->second];
+            return !t || (t->quantized && t->quantized->only);
+        };
+        if (missing() && last_input_ && !all_blobs_stored_) {
+            const bool fusion = fusion_, fused = last_fused_;
+            fusion_ = false;
+            forward_layers(last_input_);
+            fusion_ = fusion;
+            last_fused_ = fused;
+        }
+        if (missing()) return nullptr;
+        return nchw(featmaps_[it->second]);
+    }
+
+    // Whether the last forward itself stored blob `name` in float form (false for blobs a fused executor skipped).
+    bool blob_stored(std::string_view name) const {
+        auto it = blob_index_.find(std::string(name));
+        if (it == blob_index_.end()) return false;
         const tensor_ptr& t = featmaps_[it->second];
-        if (t && t->quantized && t->quantized->only) return nullptr;  // only its int8 form was written
-        return nchw(t);
+        return t && !(t->quantized && t->quantized->only);
     }
 
     // The fp16 layers pass NHWC blobs among themselves; what leaves the pipeline is NCHW as in the reference.
@@ -300,6 +325,8 @@ private:
     // ---------------------------------------------------------------- per-layer executor
     blob_map forward_layers(const tensor_ptr& input) {
         last_fused_ = false;
+        last_input_ = input;
+        all_blobs_stored_ = !fusion_;
         featmaps_[blob_index_[input_names_[0]]] = input;
         for (size_t i = 0; i < operations_.size(); ++i) {
             std::vector<tensor_ptr> in, out(op_outputs_[i].size());
@@ -370,6 +397,8 @@ private:
     std::vector<std::vector<int>> op_inputs_, op_outputs_;
     std::vector<std::string> input_names_, output_names_;
     std::vector<tensor_ptr> featmaps_;
+    tensor_ptr last_input_;           // for get_featmap of a blob the fused executors did not store
+    bool all_blobs_stored_ = false;   // the last forward was a per-layer one with fusion off
     struct post_activation {
         bool on = false, relu = false;
         int post_op = 0;
@@ -393,13 +422,30 @@ struct pipeline<Dtype>::impl::fused_plan {
     std::vector<int> in_shape;
     std::vector<dev_buffer> buffers;
     std::vector<std::function<void()>> launches;
-    std::vector<std::pair<std::string, std::shared_ptr<tensor<float>>>> outputs;
-    const float** input_slot = nullptr;
+    // Results: the launches write through `slot` into `t`, which forward() hands out. A result the caller still holds
+    // when the next forward starts is left to the caller: the plan then writes into a new tensor.
+    struct result {
+        std::string name;
+        std::shared_ptr<tensor<float>> t;
+        std::vector<int> shape;
+        float* slot = nullptr;
+    };
+    std::deque<result> outputs;  // stable addresses: the launches keep pointers to the slots
     const float* input_ptr = nullptr;
+    float** new_result(const std::vector<int>& shape, int device) {
+        outputs.emplace_back();
+        result& r = outputs.back();
+        r.shape = shape;
+        r.t = std::make_shared<tensor<float>>(shape, device);
+        r.slot = r.t->mutable_gpu_data();
+        return &r.slot;
+    }
 };
 
 template <>
 bool pipeline<unsigned short>::impl::try_fused(const tensor_ptr&, blob_map*) { return false; }
+template <>
+bool pipeline<double>::impl::try_fused(const tensor_ptr&, blob_map*) { return false; }
 
 template <>
 bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results) {
@@ -506,7 +552,7 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
             float fs = 0.f;
             int n = 0, c = 0, h = 0, w = 0, cs = 0;
             void *f32 = nullptr, *i8 = nullptr;
-            std::shared_ptr<tensor<float>> nchw;  // pipeline outputs
+            float** nchw = nullptr;  // pipeline outputs: the plan's result slot
         };
         std::vector<value_info> vals(blob_names_.size());
         const int in_value = root(blob_index_[input_names_[0]]);
@@ -567,11 +613,8 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                 const bool pooled_node = nd.pool_op >= 0;  // its output tensors have the pooled size: allocated below
                 if (out.need_i8 && !pooled_node) out.i8 = alloc(elems);
                 if (out.need_f32 && !pooled_node) out.f32 = alloc(elems * sizeof(float));
-                float* nchw = nullptr;
-                if (is_output[nd.out_value] && !pooled_node) {
-                    out.nchw = std::make_shared<tensor<float>>(std::vector<int>{out.n, out.c, oh, ow}, dev);
-                    nchw = out.nchw->mutable_gpu_data();
-                }
+                float** nchw = nullptr;
+                if (is_output[nd.out_value] && !pooled_node) nchw = out.nchw = plan->new_result({out.n, out.c, oh, ow}, dev);
                 const float* res = nullptr;
                 if (nd.res_value >= 0) {
                     const value_info& r = vals[nd.res_value];
@@ -616,16 +659,16 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                         });
                     }
                     if (out_is_result) {
-                        out.nchw = std::make_shared<tensor<float>>(std::vector<int>{out.n, out.c, ph, pw}, dev);
-                        float* nchw = out.nchw->mutable_gpu_data();
-                        plan->launches.push_back([=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, yf, o.n, o.c, ph, pw, o.cs, nchw)); });
+                        float** nchw = out.nchw = plan->new_result({out.n, out.c, ph, pw}, dev);
+                        plan->launches.push_back([=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, yf, o.n, o.c, ph, pw, o.cs, *nchw)); });
                     }
                     continue;
                 }
                 int8_t* yq = static_cast<int8_t*>(out.i8);
                 float* yf = static_cast<float*>(out.f32);
                 if (!yq && !yf && !nchw) yf = static_cast<float*>(out.f32 = alloc(elems * sizeof(float)));  // dead value: still computed
-                plan->launches.push_back([=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, res, yq, yf, nchw, nullptr)); });
+                plan->launches.push_back(
+                    [=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, res, yq, yf, nchw ? *nchw : nullptr, nullptr)); });
             } else {
                 auto* p = static_cast<operation_pooling<float>*>(operations_[nd.op].get());
                 if (!in.f32) return give_up();
@@ -643,20 +686,31 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                     EXHIP_FATAL(exhip_maxpool2d_nhwc_f32(ctx, x, yf, yq, o.fs, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl));
                 });
                 if (is_output[nd.out_value]) {
-                    out.nchw = std::make_shared<tensor<float>>(std::vector<int>{out.n, out.c, oh, ow}, dev);
-                    float* nchw = out.nchw->mutable_gpu_data();
-                    plan->launches.push_back([=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, yf, o.n, o.c, oh, ow, o.cs, nchw)); });
+                    float** nchw = out.nchw = plan->new_result({out.n, out.c, oh, ow}, dev);
+                    plan->launches.push_back([=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, yf, o.n, o.c, oh, ow, o.cs, *nchw)); });
                 }
             }
         }
+        // several output names may be Split copies of one value: they share its tensor, as in the per-layer executor
         for (const std::string& o : output_names_) {
             const value_info& v = vals[root(blob_index_[o])];
             if (!v.nchw) return give_up();
-            plan->outputs.push_back({o, v.nchw});
+            for (auto& r : plan->outputs)
+                if (&r.slot == v.nchw) r.name += (r.name.empty() ? "" : "\n") + o;
         }
         plan_ = plan;
     }
     plan_->input_ptr = input->gpu_data();
+    last_input_ = input;
+    all_blobs_stored_ = false;
+    for (tensor_ptr& t : featmaps_) t = nullptr;  // nothing of an earlier input stays readable
+    featmaps_[blob_index_[input_names_[0]]] = input;
+    for (auto& r : plan_->outputs) {
+        if (r.t.use_count() > 1) {  // a result of an earlier forward is still held outside: it stays the caller's
+            r.t = std::make_shared<tensor<float>>(r.shape, device_);
+            r.slot = r.t->mutable_gpu_data();
+        }
+    }
     if (span_first_ >= 0 && span_first_ < static_cast<int>(plan_->launches.size())) {
         exhip_ctx* ctx = memory::device_context(device_);
         if (!span_ev_[0]) {
@@ -674,10 +728,12 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
         span_launches_ = 0;
     }
     last_fused_ = true;
-    for (auto& kv : plan_->outputs) {
-        kv.second->mutable_gpu_data();  // the kernels just wrote it: the device copy is the newest
-        (*results)[kv.first] = kv.second;
-        featmaps_[blob_index_[kv.first]] = kv.second;
+    for (auto& r : plan_->outputs) {
+        r.t->mutable_gpu_data();  // the kernels just wrote it: the device copy is the newest
+        for (const std::string& name : split_string(r.name, "\n")) {
+            (*results)[name] = r.t;
+            featmaps_[blob_index_[name]] = r.t;
+        }
     }
     return true;
 }
@@ -693,6 +749,8 @@ std::vector<std::string> read_lines(std::string_view path) {
 }
 }  // namespace
 
+template <typename Dtype>
+pipeline<Dtype>::pipeline() : impl_(new impl()) {}
 template <typename Dtype>
 pipeline<Dtype>::pipeline(std::string_view param_file, std::string_view model_file, int device)
     : impl_(new impl(read_lines(param_file), model_file, device)) {}
@@ -711,6 +769,8 @@ template <typename Dtype>
 typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward_gpu(const std::shared_ptr<memory::tensor<Dtype>>& t) { return impl_->forward_gpu(t); }
 template <typename Dtype>
 std::shared_ptr<memory::tensor<Dtype>> pipeline<Dtype>::get_featmap(std::string_view name) { return impl_->get_featmap(name); }
+template <typename Dtype>
+bool pipeline<Dtype>::blob_stored(std::string_view name) const { return impl_->blob_stored(name); }
 template <typename Dtype>
 void pipeline<Dtype>::enable_profiler() { impl_->profile_ = true; }
 template <typename Dtype>
@@ -738,6 +798,7 @@ template <typename Dtype>
 std::string pipeline<Dtype>::version() { return "1.0.0"; }
 
 template class pipeline<float>;
+template class pipeline<double>;
 template class pipeline<unsigned short>;
 
 }  // namespace excalibur

@@ -76,3 +76,9 @@ class MobileFaceNetF32:
 
     def write_model(self, path):
         mf.write_model(path, self.blobs)
+
+
+# The MobileNet-style fp16 configuration of the benchmark set: 3x3 stride-2 stem to 32 channels, depthwise 3x3 (stride 1 / 2)
+# + pointwise 1x1 blocks of 64 ... 512 channels with residual sums where the shapes match, global average pooling; 224 x 224.
+CFG3 = dict(hw=224, width=32, blocks=((2, 64, 2), (1, 64, 2), (2, 128, 2), (1, 128, 2), (2, 256, 2), (1, 256, 2),
+                                      (1, 256, 2), (2, 512, 2), (1, 512, 2)), embed=128)

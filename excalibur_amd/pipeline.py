@@ -20,9 +20,16 @@ def lib():
         L = ctypes.CDLL(LIB_PATH)
         L.exc_pipeline_create.restype = ctypes.c_void_p
         L.exc_pipeline_create.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
+        L.exc_pipeline_create_from_files.restype = ctypes.c_void_p
+        L.exc_pipeline_create_from_files.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
+        L.exc_pipeline_run_keeping.argtypes = [ctypes.c_void_p]
+        L.exc_pipeline_get_kept.restype = ctypes.c_long
+        L.exc_pipeline_get_kept.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_long,
+                                            ctypes.POINTER(ctypes.c_int)]
         L.exc_pipeline_destroy.argtypes = [ctypes.c_void_p]
         L.exc_pipeline_set_fusion.argtypes = [ctypes.c_void_p, ctypes.c_int]
         L.exc_pipeline_last_fused.argtypes = [ctypes.c_void_p]
+        L.exc_pipeline_blob_stored.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
         L.exc_pipeline_set_input.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
         L.exc_pipeline_run.argtypes = [ctypes.c_void_p]
         L.exc_pipeline_sync.argtypes = [ctypes.c_void_p]
@@ -41,16 +48,22 @@ def lib():
 
 def registered_operations(dtype="f32"):
     buf = ctypes.create_string_buffer(4096)
-    lib().exc_registered_operations(0 if dtype == "f32" else 1, buf, 4096)
+    lib().exc_registered_operations({"f32": 0, "f16": 1, "f64": 2}[dtype], buf, 4096)
     return buf.value.decode().split()
 
 
 class Pipeline:
     """pipeline<float> (dtype 'f32') or pipeline<unsigned short> (dtype 'f16') on HIP device `device`."""
 
-    def __init__(self, topology, model_path="", device=0, dtype="f32", fusion=True):
+    def __init__(self, topology, model_path="", device=0, dtype="f32", fusion=True, topology_file=None):
+        """topology: the `.phai` text; topology_file: instead, the path of a `.phai` file (the reference's file-path
+        constructors); model_path "" loads dummy weights."""
         self.dtype = np.float32 if dtype == "f32" else np.uint16
-        self.h = lib().exc_pipeline_create(topology.encode(), (model_path or "").encode(), device, 0 if dtype == "f32" else 1)
+        code = 0 if dtype == "f32" else 1
+        if topology_file is not None:
+            self.h = lib().exc_pipeline_create_from_files(topology_file.encode(), (model_path or "").encode(), device, code)
+        else:
+            self.h = lib().exc_pipeline_create(topology.encode(), (model_path or "").encode(), device, code)
         lib().exc_pipeline_set_fusion(self.h, int(fusion))
 
     def close(self):
@@ -68,6 +81,19 @@ class Pipeline:
 
     def run(self):
         lib().exc_pipeline_run(self.h)
+
+    def run_keeping(self):
+        """forward() while the results of the earlier forwards stay held; get_kept(back, name) reads them."""
+        lib().exc_pipeline_run_keeping(self.h)
+
+    def get_kept(self, back, name):
+        shape = (ctypes.c_int * 4)()
+        n = lib().exc_pipeline_get_kept(self.h, back, name.encode(), None, 0, shape)
+        if n < 0:
+            raise KeyError(name)
+        out = np.empty(tuple(shape), self.dtype)
+        lib().exc_pipeline_get_kept(self.h, back, name.encode(), out.ctypes.data, out.size, shape)
+        return out
 
     def sync(self):
         rc = lib().exc_pipeline_sync(self.h)
@@ -93,6 +119,10 @@ class Pipeline:
     @property
     def fused(self):
         return bool(lib().exc_pipeline_last_fused(self.h))
+
+    def stored(self, name):
+        """Whether the last forward itself stored this blob (get() materialises the others by a per-layer rerun)."""
+        return bool(lib().exc_pipeline_blob_stored(self.h, name.encode()))
 
     def get(self, name):
         shape = (ctypes.c_int * 4)()

@@ -15,18 +15,30 @@ typedef struct exc_pipeline exc_pipeline;
 /* topology: the `.phai` text ('\n' separated); model_path: a `.racy` file or "" for dummy weights;
  * device: HIP ordinal (>= 0); dtype: 0 = pipeline<float>, 1 = pipeline<unsigned short> (fp16 storage). */
 exc_pipeline* exc_pipeline_create(const char* topology, const char* model_path, int device, int dtype);
+/* The reference's file-path constructors (include/Excalibur/pipeline.hpp:24-25, src/Excalibur/pipeline.cpp:580-587):
+ * param_file is the path of a `.phai` file, model_file the path of a `.racy` file, or NULL / "" for dummy weights. */
+exc_pipeline* exc_pipeline_create_from_files(const char* param_file, const char* model_file, int device, int dtype);
 void exc_pipeline_destroy(exc_pipeline* p);
-/* 1 (default): int8 convolution chains run as one fused plan; 0: every layer through forward_gpu on NCHW blobs. */
+/* 1 (default): int8 convolution chains run as one fused plan, convolutions absorb the activation / sum layer behind
+ * them; 0: every layer through forward_gpu, every blob stored. */
 void exc_pipeline_set_fusion(exc_pipeline* p, int on);
 int exc_pipeline_last_fused(exc_pipeline* p);
+/* 1 if the last forward itself stored blob `name` as a float tensor; 0 for a blob a fused executor skipped, which
+ * exc_pipeline_get then obtains by running the last input once more layer by layer. */
+int exc_pipeline_blob_stored(exc_pipeline* p, const char* name);
 /* Copies a host NCHW tensor into the pipeline's input blob and uploads it to the device. */
 int exc_pipeline_set_input(exc_pipeline* p, const void* input, const int shape[4]);
 /* pipeline::forward on the resident input; kernels are queued, not awaited. */
 int exc_pipeline_run(exc_pipeline* p);
+/* The same, but the results of the earlier forwards stay held, as a C++ caller may hold the blob_map of one forward
+ * across the next: exc_pipeline_get_kept reads blob `name` of the forward `back` runs before the last one (1 = the one
+ * before) like exc_pipeline_get. */
+int exc_pipeline_run_keeping(exc_pipeline* p);
+long exc_pipeline_get_kept(exc_pipeline* p, int back, const char* name, void* out, long capacity, int shape[4]);
 int exc_pipeline_sync(exc_pipeline* p);
 /* set_input + run + sync */
 int exc_pipeline_forward(exc_pipeline* p, const void* input, const int shape[4]);
-/* Copies output blob (or, with fusion off, any feature map) `name` to `out` if it fits in `capacity` elements;
+/* Copies output blob or feature map `name` of the last forward to `out` if it fits in `capacity` elements;
  * returns its element count (-1 if unknown) and its shape. */
 long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, long capacity, int shape[4]);
 /* Device time of part of a fused forward (no counterpart in the reference: a measurement aid). With
@@ -36,7 +48,8 @@ long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, long capacit
  * launches lay between them (0 and 0.0 if the last forward was not a fused one). */
 void exc_pipeline_time_fused_span(exc_pipeline* p, int first_launch);
 float exc_pipeline_last_span(exc_pipeline* p, int* launches);
-/* Newline-separated list of registered operator class names for a dtype. Returns the length needed. */
+/* Newline-separated list of registered operator class names for a dtype (0 float, 1 unsigned short, 2 double).
+ * Returns the length needed. */
 size_t exc_registered_operations(int dtype, char* buf, size_t len);
 
 #ifdef __cplusplus

@@ -102,7 +102,9 @@ void exo_dequant_i32_f32(const int32_t* acc, float* y, int n, int k, int hw, con
 
 /* src/Excalibur/operation_general_conv.cpp:127-272. 1: max(0,x) keeping -0.0 and mapping NaN to NaN
  * as _mm256_max_ps(zero, x) does (:157); 3: the reference's "ReLU6" zeroes values above 6
- * (:206-229); 4: sigmoid evaluated in double (:251); 5: mish in double (:264). */
+ * (:206-229); 4: sigmoid evaluated in double (:251); 5: mish in double (:264: the unqualified exp / log / tanh
+ * on a float resolve to the C library's double functions; pinned by the fixtures conv_f32_mish / conv_i8_mish of
+ * the compiled reference, which the float functions expf / logf / tanhf miss in half of the elements). */
 void exo_activation_f32(float* y, long count, int act) {
     switch (act) {
     case EXO_ACT_NONE: return;

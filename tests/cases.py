@@ -24,7 +24,7 @@ def conv_f32_case(seed, n, c, h, w, k, kernel, stride=1, pad=0, act=1, groups=1,
                 bias=r.normal(0, 0.01, (k,)).astype(np.float32) if bias else None)
 
 
-def conv_i8_case(seed, n, c, h, w, k, kernel, stride=1, pad=0, act=1, bias=True, integer_x=False, groups=1):
+def conv_i8_case(seed, n, c, h, w, k, kernel, stride=1, pad=0, act=1, bias=True, integer_x=False, groups=1, out_scale=1.0):
     r = _rng(seed)
     kh, kw = (kernel, kernel) if np.isscalar(kernel) else kernel
     if integer_x:
@@ -34,7 +34,7 @@ def conv_i8_case(seed, n, c, h, w, k, kernel, stride=1, pad=0, act=1, bias=True,
         x = r.uniform(-3, 3, (n, c, h, w)).astype(np.float32)
         fs = np.float32(127.0 / np.abs(x).max() * 1.1)  # a few values saturate
     wt = r.integers(-127, 128, (k, c // groups, kh, kw)).astype(np.int8)
-    s = r.uniform(1e-4, 1e-2, (k,)).astype(np.float32)       # wanted dequant scale
+    s = (r.uniform(1e-4, 1e-2, (k,)) * out_scale).astype(np.float32)  # wanted dequant scale (out_scale < 1: outputs of a few units, where sigmoid / mish bend)
     ws = (np.float32(1.0) / (s * fs)).astype(np.float32)     # stored weight scale
     ws[0] = np.float32(5e-7)                                  # |ws| <= 1e-6 -> scale forced to 0
     return dict(op="conv_i8", n=n, c=c, h=h, w=w, k=k, kh=kh, kw=kw, stride=stride, pad=pad, act=act, groups=groups,

@@ -120,3 +120,200 @@ def oracle_forward_yolo(net, x):
         else:
             raise ValueError(kind)
     return [blobs[n] for n in net.outputs], blobs
+
+
+# ---- any topology, layer by layer through the oracle restatement ----
+def _half_round(a):
+    """float -> nearest half -> float (the fp16 pipeline's storage between layers)."""
+    return np.asarray(a, np.float32).astype(np.float16).astype(np.float32)
+
+
+def _pads(L, key_all, key_top, key_right, key_bottom):
+    """Padding keys in file order, as the constructors apply them: `key_all` sets the four sides, the others one each."""
+    pl = pr = pt = pb = 0
+    for k, v in L.params.items():
+        k = int(k)
+        if k == key_all:
+            pl = pr = pt = pb = int(v)
+        elif k == key_top:
+            pt = int(v)
+        elif k == key_right:
+            pr = int(v)
+        elif k == key_bottom:
+            pb = int(v)
+    return pt, pb, pl, pr
+
+
+def layer_forward(L, ins, weights, half=False):
+    """One layer of a topology on float NCHW arrays -> list of outputs. Follows the constructors' parameter keys
+    (src/Excalibur/operation_general_conv.cpp:14-115, operation_pooling.cpp:15-75, operation_eltwise.cpp:18-39,
+    operation_innerproduct.cpp:40-72, operation_interp.cpp:186-214, operation_reshape.cpp:17-40). half: the fp16
+    pipeline's layer, float operator on half-rounded inputs with the result rounded to half
+    (include/Excalibur/operation.hpp:204-266); int8 layers do not exist there."""
+    kind = L.kind.lower()
+    wt = weights.get(L.name, {})
+    if half:
+        ins = [_half_round(a) for a in ins]
+    x = ins[0]
+    if kind in ("convolution", "convolutiondepthwise"):
+        k, kw = L.get(0), L.get(1)
+        kh, sw = L.get(11, kw), L.get(3, 1)
+        sh, groups, act = L.get(13, sw), L.get(7, 1), L.get(9, 0)
+        assert L.get(2, 1) == 1 and L.get(12, 1) == 1, "dilation"
+        g = port.geom(x.shape, k, kh, kw, (sh, sw), _pads(L, 4, 14, 15, 16), groups)
+        int8 = L.get(8, 0) != 0 and not half
+        if kind == "convolutiondepthwise":
+            w = port.dw_dequant_weights(wt["w_i8"], wt["ws"]) if int8 else wt["w"]
+            out = port.dwconv_f32(x, w, wt["bias"], act, g)
+        elif int8:
+            assert groups == 1
+            out = port.conv2d_i8(x, wt["w_i8"], wt["bias"], wt["ws"], wt["fs"], act, g)
+        else:
+            out = port.conv2d_f32(x, wt["w"], wt["bias"], act, g)
+    elif kind == "deconvolution":
+        sw = L.get(3, 1)
+        out = port.deconv2d_f32(x, wt["w"], wt["bias"], (L.get(13, sw), sw), _pads(L, 4, 14, 15, 16))
+    elif kind == "innerproduct":
+        out = port.innerproduct(x, wt["w"], wt["bias"])
+    elif kind == "pooling":
+        kw, sw = L.get(1, 0), L.get(2, 1)
+        out = port.pool2d(x, L.get(0, 0), (L.get(11, kw), kw), (L.get(12, sw), sw), _pads(L, 3, 13, 14, 15), L.get(4, 0) != 0,
+                          L.get(5, 1), L.get(6, 0))
+    elif kind == "relu":
+        out = port.relu(x)
+    elif kind == "prelu":
+        out = port.prelu(x, wt["slope"])
+    elif kind == "hardswish":
+        out = port.hardswish(x, L.get(0, 1.0 / 6.0, np.float32), L.get(1, 0.5, np.float32))
+    elif kind == "leakyrelu":
+        out = port.leakyrelu(x, L.get(0, 0.0, np.float32))
+    elif kind == "sigmoid":
+        out = port.sigmoid(x)
+    elif kind == "batchnorm":
+        out = port.batchnorm(x, wt["slope"], wt["mean"], wt["var"], wt["bias"], L.get(1, 0.0, float))
+    elif kind == "input":
+        mean = [float(v) for v in L.params.get("3", "0").split(",")]
+        scale = [float(v) for v in L.params.get("4", "1").split(",")]
+        c = x.shape[1]
+        if len(scale) != c:
+            scale = [scale[0]] * c
+        out = port.input_layer(x, mean, scale)
+    elif kind == "yolov5focus":
+        out = port.focus(x)
+    elif kind == "split":
+        return [x for _ in L.tops]
+    elif kind == "concat":
+        out = port.concat_channels(ins)
+    elif kind == "binaryop":
+        assert L.get(0, 0) == 0 and all(a.shape == x.shape for a in ins)
+        out = port.binaryop_add(ins[0], ins[1])
+    elif kind == "eltwise":
+        coeffs = None
+        if "-23301" in L.params:
+            parts = L.params["-23301"].split(",")
+            coeffs = [1.0] * len(ins)
+            for j in range(1, min(int(parts[0]), len(parts))):
+                coeffs[j - 1] = float(parts[j])
+        out = port.eltwise(ins, L.get(0, 1), coeffs)
+    elif kind == "interp":
+        assert L.get(0) == 1, "nearest only"
+        out = port.interp_nearest(x, L.get(2, 1.0, float), L.get(1, 1.0, float))
+    elif kind == "reshape":
+        shape = [x.shape[0], L.get(2, x.shape[1]), L.get(1, x.shape[2]), L.get(0, x.shape[3])]
+        out = x.reshape(shape)
+    elif kind == "transpose":
+        assert L.params.get("0") == "1,0,2"
+        out = port.transpose_hw(x)
+    else:
+        raise NotImplementedError(L.kind)
+    return [_half_round(out) if half else out]
+
+
+def evaluate(layers, weights, x, half=False, forced=None):
+    """The whole topology on x -> {blob name: float array}. forced: {blob: array} of blobs measured elsewhere; a layer
+    whose inputs are all forced reads them instead of this evaluation's own ("teacher forcing": every layer is then
+    checked on the very inputs the other side had, so errors do not add up through the stack)."""
+    first = layers[0].bottoms[0]
+    blobs = {first: _half_round(x) if half else np.ascontiguousarray(x, np.float32)}
+    for L in layers:
+        ins = [forced[b] if forced is not None and b in forced else blobs[b] for b in L.bottoms]
+        for t, o in zip(L.tops, layer_forward(L, ins, weights, half)):
+            blobs[t] = o
+    return blobs
+
+
+def calibrate_int8(layers, weights, x, margin=1.0):
+    """Feature-map scales for the int8 convolutions of a topology: one float forward with the float weights, then
+    fs = 127 / (margin * max|input of the layer|). -> {layer name: fs}"""
+    float_layers = []
+    for L in layers:
+        if L.get(8, 0) != 0:
+            params = {k: v for k, v in L.params.items() if k != "8"}
+            L = type(L)(L.kind, L.name, L.bottoms, L.tops, params)
+        float_layers.append(L)
+    blobs = evaluate(float_layers, weights, x)
+    return {L.name: np.float32(127.0 / (margin * max(float(np.abs(blobs[L.bottoms[0]]).max()), 1e-6)))
+            for L in layers if L.get(8, 0) != 0 and L.kind == "Convolution"}
+
+
+# ---- comparing a GPU pipeline with the oracle layer by layer ----
+def _as_float(a):
+    return a.view(np.float16).astype(np.float32) if a.dtype == np.uint16 else np.asarray(a, np.float32)
+
+
+def forced_layer_violations(pipe, layers, weights, half, tol, check, skip=()):
+    """Every layer of a topology on the very inputs the GPU pipeline had (its own blobs, read back by name; the pipeline
+    ran with fusion off so that every blob exists): -> [(layer name, blob, violations of `check` at `tol`)] for the
+    blobs that differ. Errors cannot add up through the stack this way: each blob is held to the tolerance on its own."""
+    bad = []
+    cache = {}
+
+    def blob(name):
+        if name not in cache:
+            cache[name] = _as_float(pipe.get(name))
+        return cache[name]
+
+    for L in layers:
+        if L.kind in skip:
+            continue
+        ins = [blob(b) for b in L.bottoms]
+        if L.kind == "Reshape":   # in place on the GPU side: the bottom already carries the new shape
+            continue
+        for t, want in zip(L.tops, layer_forward(L, ins, weights, half)):
+            got = blob(t)
+            n = check(got.reshape(want.shape), want, tol) if tol else int((got.reshape(want.shape) != want).sum())
+            if n:
+                bad.append((L.name, t, n))
+    return bad
+
+
+def _window_layer(L):
+    """The layer with its padding keys set to zero: for crops that carry their own border."""
+    params = {k: v for k, v in L.params.items() if k not in ("4", "14", "15", "16")}
+    return type(L)(L.kind, L.name, L.bottoms, L.tops, params)
+
+
+def sampled_conv_violations(pipe, L, weights, half, tol, check, image, windows=((0, 0), (-1, -1), (None, None)), size=6):
+    """A convolution / depthwise layer of a full-size forward checked on output windows of size x size of one image:
+    the oracle runs the layer on the crop of the GPU's own input blob that the window depends on (zero border added
+    where the window touches the image's edge). windows: (row, column) of the window's corner, -1 = the last window,
+    None = the middle. -> violations of `check` at `tol` (bit equality if tol is None)."""
+    x = _as_float(pipe.get(L.bottoms[0]))[image:image + 1]
+    y = _as_float(pipe.get(L.tops[0]))[image:image + 1]
+    kw, sw = L.get(1), L.get(3, 1)
+    kh, sh = L.get(11, kw), L.get(13, sw)
+    pt, pb, pl, pr = _pads(L, 4, 14, 15, 16)
+    oh, ow = (x.shape[2] + pt + pb - kh) // sh + 1, (x.shape[3] + pl + pr - kw) // sw + 1
+    y = y.reshape(1, L.get(0), oh, ow)   # a Reshape layer behind it works in place: the blob may carry that layer's shape
+    xp = np.pad(x, ((0, 0), (0, 0), (pt, pb), (pl, pr)))
+    Lw = _window_layer(L)
+    bad = 0
+    for wy, wx in windows:
+        hgt, wid = min(size, oh), min(size, ow)
+        oy = 0 if wy == 0 else oh - hgt if wy == -1 else (oh - hgt) // 2
+        ox = 0 if wx == 0 else ow - wid if wx == -1 else (ow - wid) // 2
+        crop = xp[:, :, oy * sh:(oy + hgt - 1) * sh + kh, ox * sw:(ox + wid - 1) * sw + kw]
+        want = layer_forward(Lw, [np.ascontiguousarray(crop)], weights, half)[0]
+        got = y[:, :, oy:oy + hgt, ox:ox + wid]
+        bad += check(got, want, tol) if tol else int((got != want).sum())
+    return bad

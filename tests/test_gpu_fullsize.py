@@ -1,0 +1,148 @@
+"""The benchmark set's network configurations at their full sizes on the GPU: the MobileNet-style fp16 stack at
+64 x 3 x 224 x 224 and the YOLOv5s detector (the shipped topology: 70 convolutions, three heads of 255 channels) at
+16 x 3 x 640 x 640 in fp16 and with int8 convolutions. The oracle cannot evaluate these sizes in a test's time, so the
+checks are the ones that do not depend on size:
+
+* rows of the batch against the same images run alone (other tile plans, other launch shapes);
+* the fused forms (convolutions absorbing the layer behind them, int8 tensors handed between convolutions, NHWC-resident
+  half blobs) against the plain per-layer form;
+* layers sampled through the stack against the oracle on the GPU's own input blobs of one image: output windows of
+  convolutions and depthwise layers (corners with their zero border, and the middle), whole small blobs elsewhere.
+"""
+import os
+import tempfile
+
+import numpy as np
+import pytest
+
+from excalibur_amd import modelfile as mf
+from excalibur_amd import pipeline as xp
+from excalibur_amd import topologies
+from tests import cases, netref
+
+pytestmark = pytest.mark.gpu
+
+
+class Net:
+    def __init__(self, text, seed, gain=2.0, fs=None):
+        self.text = text
+        self.layers = mf.parse_topology(text)
+        self.model = mf.SeededModel(self.layers, seed, fs=fs, gain=gain)
+        with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+            self.path = f.name
+        self.model.write(self.path)
+
+    def close(self):
+        os.unlink(self.path)
+
+
+def _run(net, x, dtype, fusion=True):
+    p = xp.Pipeline(net.text, net.path, 0, dtype, fusion=fusion)
+    p.forward(x if dtype == "f32" else x.astype(np.float16).view(np.uint16))
+    return p
+
+
+def _f(a):
+    return a.view(np.float16).astype(np.float32) if a.dtype == np.uint16 else a
+
+
+def _sampled(p, net, half, tol, image, every):
+    """Every `every`-th convolution / depthwise layer on windows, plus the small layers whole, on image `image`."""
+    check = cases.check_value if tol else None
+    convs = [L for L in net.layers if L.kind in ("Convolution", "ConvolutionDepthWise")]
+    picked = convs[::every] + convs[-3:]
+    bad = [(L.name, netref.sampled_conv_violations(p, L, net.model.weights, half, tol, check, image)) for L in picked]
+    return [b for b in bad if b[1]]
+
+
+def test_cfg3_mobilenet_style_fp16_at_full_size(monkeypatch):
+    from excalibur_amd.mobilenet import CFG3, MobileFaceNetF32
+    net = Net(MobileFaceNetF32(**CFG3).topology(), 61, gain=1.0)
+    try:
+        x = np.random.default_rng(62).uniform(0, 255, (64, 3, 224, 224)).astype(np.float32)
+        p = _run(net, x, "f16")
+        out = p.get("out")
+        assert out.shape == (64, 128, 1, 1) and np.isfinite(_f(out)).all()
+        p.close()
+        # (a) rows of the batch against single-image runs: the float accumulation order inside a tile does not depend on
+        # the batch, the tile plan may; both are held to the fp16 contract
+        for i in (0, 37, 63):
+            q = _run(net, x[i:i + 1], "f16")
+            assert cases.check_value(_f(q.get("out")), _f(out[i:i + 1]), 2e-3) == 0, i
+            q.close()
+        # (b) per-layer form without the fused epilogues: bit for bit
+        plain = _run(net, x, "f16", fusion=False)
+        assert np.array_equal(plain.get("out"), out)
+        # (d) layers through the stack against the fp16 oracle on the GPU's own blobs
+        assert _sampled(plain, net, True, 2e-3, 37, 4) == []
+        tail = [L for L in net.layers if L.kind in ("Pooling", "InnerProduct")]
+        assert netref.forced_layer_violations(plain, tail, net.model.weights, True, 2e-3, cases.check_value) == []
+        plain.close()
+        # (c) every blob kept NCHW: other kernels for the per-channel and elementwise layers, whose float-to-half
+        # conversions may round a product once where the other layout's rounds twice (one half ulp, rarely)
+        monkeypatch.setenv("EXCALIBUR_F16_NCHW", "1")
+        q = _run(net, x, "f16")
+        assert cases.check_value(_f(q.get("out")), _f(out), 2e-3) == 0
+        q.close()
+    finally:
+        net.close()
+
+
+def test_cfg5_yolov5s_fp16_at_full_size(monkeypatch):
+    text, outs = topologies.yolov5s_simp(640)
+    net = Net(text, 63)
+    try:
+        x = np.random.default_rng(64).uniform(0, 255, (16, 3, 640, 640)).astype(np.float32)
+        p = _run(net, x, "f16")
+        got = {o: p.get(o) for o in outs}
+        assert [got[o].shape for o in outs] == [(16, 3, 6400, 85), (16, 3, 1600, 85), (16, 3, 400, 85)]
+        assert all(np.isfinite(_f(v)).all() for v in got.values())
+        p.close()
+        for i in (0, 11):
+            q = _run(net, x[i:i + 1], "f16")
+            for o in outs:
+                assert cases.check_value(_f(q.get(o)), _f(got[o][i:i + 1]), 2e-3) == 0, (i, o)
+            q.close()
+        plain = _run(net, x, "f16", fusion=False)
+        for o in outs:
+            assert np.array_equal(plain.get(o), got[o]), o
+        assert _sampled(plain, net, True, 2e-3, 11, 6) == []
+        small = [L for L in net.layers if L.kind in ("Pooling", "Interp", "BatchNorm", "LeakyRelu") or L.name in ("Concat_300", "Concat_517")]
+        assert netref.forced_layer_violations(plain, small[-8:], net.model.weights, True, 2e-3, cases.check_value) == []
+        plain.close()
+        monkeypatch.setenv("EXCALIBUR_F16_NCHW", "1")
+        q = _run(net, x[:4], "f16")
+        for o in outs:
+            assert cases.check_value(_f(q.get(o)), _f(got[o][:4]), 2e-3) == 0, o
+        q.close()
+    finally:
+        net.close()
+
+
+def test_cfg5_yolov5s_int8_at_full_size():
+    text, outs = topologies.yolov5s_simp(640, int8=True)
+    layers = mf.parse_topology(text)
+    # feature-map scales from a float forward of the same weights at a reduced input
+    small_text, _ = topologies.yolov5s_simp(64, int8=True)
+    small_layers = mf.parse_topology(small_text)
+    fs = netref.calibrate_int8(small_layers, mf.SeededModel(small_layers, 65).weights,
+                               np.random.default_rng(66).uniform(0, 255, (1, 3, 64, 64)).astype(np.float32), margin=1.5)
+    net = Net(text, 65, fs=fs)
+    try:
+        x = np.random.default_rng(67).uniform(0, 255, (16, 3, 640, 640)).astype(np.float32)
+        p = _run(net, x, "f32")
+        got = {o: p.get(o) for o in outs}
+        assert got[outs[0]].shape == (16, 3, 6400, 85)
+        p.close()
+        for i in (0, 11):   # int8 accumulation has one right answer and the float layers work element by element: bit for bit
+            q = _run(net, x[i:i + 1], "f32")
+            for o in outs:
+                assert np.array_equal(q.get(o), got[o][i:i + 1]), (i, o)
+            q.close()
+        plain = _run(net, x, "f32", fusion=False)
+        for o in outs:
+            assert np.array_equal(plain.get(o), got[o]), o
+        assert _sampled(plain, net, False, None, 11, 6) == []
+        plain.close()
+    finally:
+        net.close()

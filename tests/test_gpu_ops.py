@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(f).startswith("net_"))
-TOLERANT = ("conv_f32", "fc_", "deconv", "softmax", "binaryop_pixel", "binaryop_image")
+TOLERANT = ("conv_f32", "fc_", "deconv", "softmax", "binaryop_pixel", "binaryop_image", "conv_i8_mish")
 
 
 @pytest.fixture(scope="module")
@@ -479,6 +479,8 @@ def _sampled_acc(case, q_nchw, samples, rng):
 FULL = [
     ("cfg2_3x3", (400, 8, 128, 80, 80, 128, 3, 1, 1)),
     ("cfg2_1x1_k256", (401, 8, 128, 80, 80, 256, 1, 1, 0)),
+    ("cfg2_3x3_k256", (404, 8, 128, 80, 80, 256, 3, 1, 1)),
+    ("cfg2_1x1_k128", (405, 8, 128, 80, 80, 128, 1, 1, 0)),
     ("resnet_stage1_n8", (402, 8, 64, 160, 160, 64, 3, 1, 1)),
     ("resnet_stem_n4", (403, 4, 3, 640, 640, 64, 7, 2, 3)),
 ]
@@ -502,3 +504,38 @@ def test_full_size_sampled_and_linear(ctx, name, args):
     assert np.array_equal(a1 + a2, got["acc"])
     want = port.dequant(got["acc"], case["ws"], case["fs"], case["bias"])
     assert np.array_equal(got["nchw"], port.relu(want))
+
+
+@pytest.mark.parametrize("k,kernel", [(128, 3), (256, 3), (128, 1), (256, 1)], ids=["3x3k128", "3x3k256", "1x1k128", "1x1k256"])
+def test_cfg2_requantized_int8_output_at_full_size(ctx, k, kernel):
+    """8 x 128 x 80 x 80 -> K with ReLU and the next layer's quantizer in the epilogue (the fused int8 output): the int8
+    NHWC tensor recomputed from the GPU's own accumulators (checked against brute force by the test above) with the closed
+    form q8(relu(fmaf(acc, s, b)) * fs_out), every element; and with a float32 shortcut added before the ReLU."""
+    case = cases.conv_i8_case(410 + k + kernel, 8, 128, 80, 80, k, kernel, 1, kernel // 2, act=0)
+    fs_out = np.float32(23.7)
+    r = np.random.default_rng(k + kernel)
+    res = r.uniform(-3, 3, (8, 80, 80, k)).astype(np.float32)
+    base = gpueval.conv_i8(ctx, case, want=("acc",))
+    y = port.dequant(base["acc"], case["ws"], case["fs"], case["bias"])
+    got = gpueval.conv_i8(ctx, case, fs_out=fs_out, post_relu=1, want=())
+    assert np.array_equal(got["i8"], port.quantize(port.relu(y), fs_out).transpose(0, 2, 3, 1))
+    got = gpueval.conv_i8(ctx, case, fs_out=fs_out, residual=res, post_relu=1, want=("nhwc",))
+    z = port.relu(port.binaryop_add(y, np.ascontiguousarray(res.transpose(0, 3, 1, 2))))
+    assert np.array_equal(got["nhwc"], z.transpose(0, 2, 3, 1))
+    assert np.array_equal(got["i8"], port.quantize(z, fs_out).transpose(0, 2, 3, 1))
+
+
+@pytest.mark.parametrize("shape,cs", [((2, 5, 7, 9), 32), ((1, 3, 6, 6), 4), ((2, 40, 5, 4), 64)], ids=str)
+def test_quantizer_with_per_input_channel_scales(ctx, shape, cs):
+    """quantize_float32_to_int8's second branch (src/Excalibur/operation_general_conv.cpp:596): one scale per input
+    channel. Values at +-0.5 ties and beyond saturation included; pad channels are zero."""
+    r = np.random.default_rng(shape[1])
+    fs = r.uniform(0.5, 60, (shape[1],)).astype(np.float32)
+    x = r.uniform(-4, 4, shape).astype(np.float32)
+    x[0, :, 0, 0] = (np.float32(2.5) / fs).astype(np.float32)    # ties after scaling, where they are representable
+    x[0, :, 0, 1] = np.float32(1000.0)
+    x[0, :, 0, 2] = np.float32(-1000.0)
+    got = ctx.quantize_nchw_to_nhwc_i8(ctx.array(x), 0.0, cs, fs_per_channel=ctx.array(fs)).download()
+    want = port.quantize(x, fs).transpose(0, 2, 3, 1)
+    assert np.array_equal(got[..., :shape[1]], want)
+    assert not got[..., shape[1]:].any()

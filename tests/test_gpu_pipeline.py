@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 NAMES = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(f).startswith("net_"))
-TOLERANT = ("conv_f32", "fc_", "deconv", "softmax", "binaryop_pixel", "binaryop_image")
+TOLERANT = ("conv_f32", "fc_", "deconv", "softmax", "binaryop_pixel", "binaryop_image", "conv_i8_mish")
 
 
 def run_case(case, dtype="f32"):
@@ -504,23 +504,23 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
             p.forward(xin)
             assert not p.fused
             got[fusion] = {b: p.get(b) for b in outputs}
-            for b in middle:  # with int8 convolutions, a blob read by int8 convolutions alone has no float form
-                try:
-                    got[fusion][b] = p.get(b)
-                except KeyError:
-                    assert fusion and kind == "int8"
-            if fusion:
+            if fusion:  # which blobs the forward itself stored (asked before get() materialises the others)
                 for gone in ("c1", "c1b", "c1c", "c3", "c4", "c5", "c8b"):
-                    with pytest.raises(KeyError):
-                        p.get(gone)
+                    assert not p.stored(gone), gone
                 for summed in ("c8c", "c8d"):  # the residual adds: in the convolution only on NHWC half blobs
-                    if kind == "f16":
-                        with pytest.raises(KeyError):
-                            p.get(summed)
-                    else:
-                        p.get(summed)
+                    assert p.stored(summed) == (kind != "f16"), summed
                 for kept in ("c6", "c7", "c8", "c9b"):
-                    p.get(kept)
+                    assert p.stored(kept), kept
+                for b in middle:  # with int8 convolutions, a blob read by int8 convolutions alone has no float form
+                    assert p.stored(b) or kind == "int8", b
+            else:
+                assert all(p.stored(b) for b in middle)
+            for b in middle:
+                got[fusion][b] = p.get(b)
+            if fusion:  # a skipped blob comes from a per-layer rerun of the same input: the plain pipeline's bytes
+                assert np.array_equal(p.get("c1"), plain_c1)
+            else:
+                plain_c1 = p.get("c1")
             p.close()
         assert len(got[True]) >= len(outputs) + 4
         for b in got[True]:
@@ -604,8 +604,7 @@ def test_int8_convolutions_hand_their_readers_int8_tensors():
             got[fusion] = {b: p.get(b) for b in outputs + ["c3", "c4", "s"]}
             if fusion:
                 for gone in ("c1", "c2", "a2"):         # int8 only, or inside the pair
-                    with pytest.raises(KeyError):
-                        p.get(gone)
+                    assert not p.stored(gone), gone
                 assert np.isfinite(p.get("c6")).all()    # its second reader quantizes the float form itself
                 p.forward(x)                              # a second forward reuses the pooled blocks
                 for b in outputs:

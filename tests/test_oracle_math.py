@@ -28,6 +28,15 @@ def test_quantize_dense_sweep_against_closed_form():
     x2 = np.ones((1, 3, 2, 2), np.float32)
     q2 = port.quantize(x2, np.array([1, 2, 3], np.float32))
     assert [int(q2[0, c, 0, 0]) for c in range(3)] == [1, 2, 3]
+    # ... for every image and position, against the closed form written per element
+    r = np.random.default_rng(12)
+    x3 = r.uniform(-5, 5, (2, 4, 3, 5)).astype(np.float32)
+    fs = r.uniform(0.5, 40, 4).astype(np.float32)
+    q3 = port.quantize(x3, fs)
+    for idx in np.ndindex(x3.shape):
+        v = np.float32(x3[idx] * fs[idx[1]])
+        t = np.float32(v + np.float32(0.5)) if v >= 0 else np.float32(v - np.float32(0.5))
+        assert int(q3[idx]) == int(np.clip(np.trunc(np.float64(t)), -128, 127)), idx
 
 
 def _brute_conv(q, w, stride, pad, groups=1):
