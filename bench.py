@@ -28,44 +28,72 @@ PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0
 
 
-def cpu_baseline(net, hw, budget_s=20.0):
-    """Reference CPU path (one core) on one image of the workload's own resolution; the number of timed forwards is
-    sized so that the sample takes roughly `budget_s` seconds."""
+def cpu_baseline(net, hw, budget_s=10.0):
+    """The reference's CPU path on one image of the workload's own resolution, two legs of about `budget_s` seconds each:
+    one core (the reference's default build: OpenMP off), and batch-parallel over the host cores with one pipeline and one
+    image per worker thread (a pipeline instance is single-threaded). -> (one-core record, all-cores record or None)"""
     from oracle import ref
     x = np.random.default_rng(7).uniform(-1, 1, (1, 3, hw, hw)).astype(np.float32)
     gmac = net.gmac_per_image(hw, hw)
-    if ref.available():
-        import tempfile
-        with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
-            path = f.name
-        net.write_model(path)
+    if not ref.available():
+        from tests import netref
+        t0 = time.perf_counter()
+        netref.oracle_forward(net, x)
+        sec = time.perf_counter() - t0
+        return {"value": round(1.0 / sec, 4), "unit": "images/s", "cores": 1, "kind": "port",
+                "sample": f"one 3x{hw}x{hw} image through the same int8 topology, 1 timed forward, "
+                          f"{sec * 1e3:.0f} ms = {2 * gmac / sec:.1f} GOP/s"}, None
+    import tempfile
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    net.write_model(path)
+    try:
         p = ref.Pipeline(net.topology(), path, "f32")
-        os.unlink(path)
         t0 = time.perf_counter()
         p.forward(x)
         first = time.perf_counter() - t0
         iters = max(2, min(60, int(budget_s / max(first, 1e-3)) - 1))
         sec = p.time(x, 0, iters)
         p.close()
-        kind = "reference"
-    else:
-        from tests import netref
-        t0 = time.perf_counter()
-        netref.oracle_forward(net, x)
-        sec = time.perf_counter() - t0
-        iters, kind = 1, "port"
-    return {"value": round(1.0 / sec, 4), "unit": "images/s", "cores": 1, "kind": kind,
-            "sample": f"one 3x{hw}x{hw} image through the same int8 topology, {iters} timed forward(s), "
-                      f"{sec * 1e3:.0f} ms each = {2 * gmac / sec:.1f} GOP/s"}
+        one = {"value": round(1.0 / sec, 4), "unit": "images/s", "cores": 1, "kind": "reference",
+               "sample": f"one 3x{hw}x{hw} image through the same int8 topology, {iters} timed forward(s), "
+                         f"{sec * 1e3:.0f} ms each = {2 * gmac / sec:.1f} GOP/s"}
+        # the GPU boxes give a job 16 cores, whatever the machine has
+        workers = max(1, min(os.cpu_count() or 1, 16))
+        each = max(1, int(budget_s / max(sec, 1e-3)))
+        wall = ref.time_parallel(net.topology(), path, x, workers, 1, each)
+        rate = workers * each / wall
+        many = {"value": round(rate, 4), "unit": "images/s", "cores": workers, "kind": "reference",
+                "sample": f"{workers} worker threads, each its own pipeline and one 3x{hw}x{hw} image, {each} timed forward(s) "
+                          f"each in {wall:.1f} s = {2 * gmac * rate:.1f} GOP/s"}
+    finally:
+        os.unlink(path)
+    return one, many
+
+
+def csrc_digest():
+    """A digest of the kernel sources: profiles taken under rocprofv3 carry it, so that a figure read back from a profile
+    file is dropped once a kernel has changed."""
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "excalibur_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h")):
+            h.update(open(os.path.join(d, name), "rb").read())
+    return h.hexdigest()[:16]
 
 
 def measured_traffic(n, hw):
     """HBM bytes per conv launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE, scaled by a
-    plain copy kernel); it was taken on the default workload only."""
+    plain copy kernel). The counters cannot be read inside this process, so the figure comes from the profile file, which
+    names the workload and the kernel sources it was taken with: None for another workload or other sources."""
     path = os.path.join(ROOT, "profiles", "conv_igemm_resnet18_int8_n32_640_hbm_traffic.txt")
     if (n, hw) != (32, 640) or not os.path.exists(path):
         return None
-    for line in open(path):
+    text = open(path).read()
+    if f"kernel sources {csrc_digest()}" not in text:
+        return None
+    for line in text.splitlines():
         if line.startswith("conv_igemm_kernel HBM traffic per forward"):
             return {"value": float(line.split("=")[-1].split("MB")[0]), "unit": "MB per launch (mean of 20 launches)"}
     return None
@@ -119,12 +147,13 @@ def network_table(iters=10):
     return rows
 
 
-def bandwidth_table(iters=20):
+def bandwidth_table(iters=20, quiet=False, ctx=None):
     """The path's memory-bound kernels at the benchmark network's tensor sizes, through the C ABI with preallocated
     operands: HIP events around `iters` back-to-back launches, algorithmic bytes (every operand read once, every result
     written once) over the 8 TB/s HBM peak. Returns [{"kernel", "us", "GB/s", "frac"}]."""
     from excalibur_amd import hip
-    ctx = hip.Ctx(0)
+    own_ctx = ctx is None
+    ctx = hip.Ctx(0) if own_ctx else ctx
     L = hip.lib()
     rng = np.random.default_rng(0)
     cf, sz = ctypes.c_float, ctypes.c_size_t
@@ -144,7 +173,8 @@ def bandwidth_table(iters=20):
         ms = e0.elapsed_ms(e1) / iters
         rows.append({"kernel": label, "us": round(ms * 1e3, 1), "GB/s": round(nbytes / ms / 1e6, 1),
                      "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 3)})
-        print(f"{label:66s} {ms * 1e3:8.1f} us {nbytes / ms / 1e6:8.1f} GB/s {100 * nbytes / ms / 1e6 / PEAK_HBM_GBS:5.1f} %", file=sys.stderr, flush=True)
+        if not quiet:
+            print(f"{label:66s} {ms * 1e3:8.1f} us {nbytes / ms / 1e6:8.1f} GB/s {100 * nbytes / ms / 1e6 / PEAK_HBM_GBS:5.1f} %", file=sys.stderr, flush=True)
 
     n, c, h, w = 32, 64, 160, 160          # the stage-1 tensors of the benchmark network
     cnt = n * c * h * w
@@ -198,7 +228,8 @@ def bandwidth_table(iters=20):
        lambda: L.exhip_dwconv3x3_nhwc_f16(ctx.h, dx.ptr, w9.ptr, b9.ptr, dy.ptr, dn, dc, dh, dh, dc, 1, 1, 1, 1, 1, 1))
     bw("depthwise 3x3 s2 f16 NHWC, 64x128x56x56", dx.size * 2 + dx.size // 2,
        lambda: L.exhip_dwconv3x3_nhwc_f16(ctx.h, dx.ptr, w9.ptr, b9.ptr, dy.ptr, dn, dc, dh, dh, dc, 2, 1, 1, 1, 1, 1))
-    ctx.close()
+    if own_ctx:
+        ctx.close()
     return rows
 
 
@@ -210,6 +241,7 @@ def main():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--hw", type=int, default=640)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-memory-bound", action="store_true", help="skip the memory-bound kernels' block of the line")
     ap.add_argument("--per-layer", action="store_true", help="print per-launch timings to stderr")
     ap.add_argument("--networks", action="store_true",
                     help="time the other configurations' whole topologies (MobileNet- and YOLOv5s-shaped, f32 / f16 / int8) "
@@ -334,8 +366,20 @@ def main():
                      "algorithmic_gop_per_step": round(conv_gop, 1), "avg_launch_ms": round(conv_ms / n_conv, 4),
                      "timing": f"HIP events around the {n_conv} consecutive launches of a forward of the timed pipeline, mean of {reps} forwards"},
     }
+    if not args.no_memory_bound:
+        rows = bandwidth_table(iters=10, quiet=True, ctx=ctx)
+        fr = sorted(r["frac"] for r in rows)
+        worst = min(rows, key=lambda r: r["frac"])
+        line["memory_bound"] = {"bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s", "kernels": len(rows),
+                                "worst_frac": worst["frac"], "worst_kernel": worst["kernel"], "median_frac": fr[len(fr) // 2],
+                                "below_0.60": [r["kernel"] for r in rows if r["frac"] < 0.60],
+                                "timing": "HIP events around 10 back-to-back launches of each memory-bound kernel of the path, "
+                                          "algorithmic bytes over the 8 TB/s peak (python bench.py --bandwidth prints every row)"}
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(net, hw)
+        one, many = cpu_baseline(net, hw)
+        line["cpu_baseline"] = one
+        if many:
+            line["cpu_baseline_all_cores"] = many
     print(json.dumps(line))
     pipe.close()
     ctx.close()

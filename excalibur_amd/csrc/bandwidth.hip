@@ -1688,7 +1688,7 @@ static int dw_nchw_f32(exhip_ctx* ctx, const float* x, const float* w9, const fl
         const size_t want = (size_t)256 * 8 * 64;
         // about eight rows to a band (measured at 32x64x160x160: 5 to 10 rows 65 % of the HBM peak, 16 rows 61 %, 20 and more 59 %)
         int bands = (int)std::min<size_t>((size_t)oh, std::max<size_t>((oh + 7) / 8, (want + per_band - 1) / per_band));
-        static const int env_rows = getenv("EXHIP_DW_BAND_ROWS") ? atoi(getenv("EXHIP_DW_BAND_ROWS")) : 0;
+        const int env_rows = g_exhip_options.dw_band_rows;
         int band_rows = (oh + bands - 1) / bands;
         if (env_rows > 0) band_rows = std::min(env_rows, oh);
         bands = (oh + band_rows - 1) / band_rows;
@@ -1761,7 +1761,7 @@ static int dw_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, const float* w9, const
         const int px = stride == 1 ? 4 : 2;
         const int strips = (ow + px - 1) / px;
         const size_t per_band = (size_t)n * strips * (cs / 4);
-        static const int env_rows = getenv("EXHIP_DW_BAND_ROWS") ? atoi(getenv("EXHIP_DW_BAND_ROWS")) : 0;
+        const int env_rows = g_exhip_options.dw_band_rows;
         const size_t want = (size_t)256 * 14 * 64;
         int bands = (int)std::min<size_t>((size_t)std::max(1, oh / 7), std::max<size_t>((oh + 13) / 14, (want + per_band - 1) / per_band));
         int band_rows = (oh + bands - 1) / bands;

@@ -37,6 +37,18 @@ int exhip_static_scratch_setup(int device);
 // Kernel launch check: launch errors are reported at once, execution errors at the next sync.
 #define EXHIP_LAUNCH_CHECK() EXHIP_CHECK(hipGetLastError())
 
+// Switches for tests and development, set through exhip_set_option (never read from the environment): a test
+// pins a plan choice to reach a code path small shapes would not take; zero / negative values mean "not set".
+struct exhip_options {
+    int force_variant = -1;  // tile variant of the convolution planner
+    int force_chunk = 0;     // its channel chunk in bytes (32 / 64)
+    int force_rs = 0;        // filter rows per stage
+    int force_abufs = 0;     // activation tile buffers (1 / 2)
+    int debug_plan = 0;      // one line per planned layer on stderr
+    int dw_band_rows = 0;    // row-band height of the depthwise strip kernels
+};
+extern exhip_options g_exhip_options;
+
 // ---- device helpers shared by the kernels ----
 // float32_to_int8 of the reference (src/Primitives/simd_types.cpp:140-152): add +-0.5, saturate, truncate.
 __device__ __forceinline__ int exhip_q8(float v) {

@@ -21,6 +21,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
 #include <type_traits>
 #include <vector>
 
@@ -1220,11 +1221,8 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
     const int es = esize_of(dt), cb = d->c_stride * es;
     const int OH = (d->h + d->pt + d->pb - d->kh) / d->sh + 1, OW = (d->w + d->pl + d->pr - d->kw) / d->sw + 1;
     const bool packed = cb < 32;
-    static const int force_variant = getenv("EXHIP_FORCE_VARIANT") ? atoi(getenv("EXHIP_FORCE_VARIANT")) : -1;
-    static const int force_chunk = getenv("EXHIP_FORCE_CHUNK") ? atoi(getenv("EXHIP_FORCE_CHUNK")) : 0;
-    static const int force_rs = getenv("EXHIP_FORCE_RS") ? atoi(getenv("EXHIP_FORCE_RS")) : 0;
-    const char* const abufs_env = getenv("EXHIP_FORCE_ABUFS");  // read per call: tests switch it inside one process
-    const int force_abufs = abufs_env ? atoi(abufs_env) : 0;
+    const int force_variant = g_exhip_options.force_variant, force_chunk = g_exhip_options.force_chunk;
+    const int force_rs = g_exhip_options.force_rs, force_abufs = g_exhip_options.force_abufs;
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
         if (force_variant >= 0 && !pool && !packed && variant != force_variant) continue;  // not the first-layer forms
@@ -1395,22 +1393,28 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
         return EXHIP_ERR_UNSUPPORTED;
     }
     *out = best;
-    static const bool show = getenv("EXHIP_DEBUG_PLAN") != nullptr;  // development aid: one line per planned layer
-    if (show)
+    if (g_exhip_options.debug_plan)
         fprintf(stderr, "plan %dx%dx%dx%d k%d %dx%d s%d%s: variant %d chunk %d RS %d patch %dx%d tile %dx%d act %d B x%d w %d B x%d lds %zu\n", d->n,
                 d->c, d->h, d->w, d->k, d->kh, d->kw, d->sh, pool ? " +pool" : "", best.variant, best.chunk_b, best.RS, best.PH, best.PW,
                 best.IH, best.IW, best.lds_act_b, best.act_bufs, best.lds_w_b, best.w_bufs, best.lds_bytes());
     return 0;
 }
 
+// Per kernel: on which devices its dynamic LDS limit has been raised (bit i = device i), guarded by one mutex.
+std::mutex g_attr_mutex;
+
 template <typename K>
-int launch_kernel(exhip_ctx* ctx, K kernel, bool* attr_set, const Plan& pl, const ConvParams& p, int grid) {
+int launch_kernel(exhip_ctx* ctx, K kernel, unsigned long long* attr_set, const Plan& pl, const ConvParams& p, int grid) {
     // per-wave epilogue LDS: none in the general form, the int8 tile and offset table in the fused form, plus
     // the float32 tile when a float32 tensor is read or written
     const int epi_wave_b = p.epi_mode == 0 ? 0 : (p.epi_f ? kEpiWaveBytes : 32 * kEpiRowQ + 128);
-    if (!*attr_set) {  // raise the dynamic LDS limit once per kernel
-        EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        *attr_set = true;
+    {
+        std::lock_guard<std::mutex> lock(g_attr_mutex);
+        const unsigned long long bit = 1ull << (ctx->device & 63);
+        if (!(*attr_set & bit)) {  // raise the dynamic LDS limit once per kernel and device
+            EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            *attr_set |= bit;
+        }
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(pl.threads), pl.launch_lds_bytes(epi_wave_b), ctx->stream, p);
     EXHIP_LAUNCH_CHECK();
@@ -1421,11 +1425,11 @@ template <int DT, int NT, int WM, int WN, bool PACKED, int EPI, int KWE, int KSC
 int launch_inst(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid) {
     if constexpr (WM * WN == 8 && !PACKED && EPI == 1 && KWE == 3) {
         if (pl.two_per_cu) {
-            static bool attr_low = false;
+            static unsigned long long attr_low = 0;
             return launch_kernel(ctx, conv_igemm_kernel<DT, 2, NT, WM, WN, PACKED, EPI, KWE, KSC, true>, &attr_low, pl, p, grid);
         }
     }
-    static bool attr = false;
+    static unsigned long long attr = 0;
     return launch_kernel(ctx, conv_igemm_kernel<DT, 2, NT, WM, WN, PACKED, EPI, KWE, KSC>, &attr, pl, p, grid);
 }
 
@@ -1459,8 +1463,7 @@ int launch_variant(exhip_ctx* ctx, const Plan& pl, const ConvParams& p, int grid
 // more rounds than the exposed tile loads cost. `fused_3x3`: the launch runs the fused int8 epilogue on a 3-tap row
 // shape, the instantiations whose 512-thread form is held to 128 registers and so may run two groups per CU.
 void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3) {
-    const char* const abufs_env = getenv("EXHIP_FORCE_ABUFS");  // read per call: tests switch it inside one process
-    const int force_abufs = abufs_env ? atoi(abufs_env) : 0;
+    const int force_abufs = g_exhip_options.force_abufs;
     if (pl.packed || pl.MPH || pl.n_chunks < 2 || pl.act_bufs == 1 || force_abufs == 2) return;
     const long long cap = pl.threads == 512 ? (fused_3x3 ? 2 : 1) : 3;
     auto groups = [&](const Plan& q) {
@@ -1477,8 +1480,7 @@ void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3
     if (force_abufs == 1 || r_one * 115 < r_now * 100) {
         pl = one;
         pl.two_per_cu = pl.threads == 512;
-        static const bool show = getenv("EXHIP_DEBUG_PLAN") != nullptr;
-        if (show)
+        if (g_exhip_options.debug_plan)
             fprintf(stderr, "  launch: act x%d w x%d, %lld groups per CU instead of %lld (%lld groups, LDS %zu)\n", pl.act_bufs, pl.w_bufs,
                     g_one, g_now, wgs, pl.launch_lds_bytes(epi_wave_b));
     }

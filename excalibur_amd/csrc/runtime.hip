@@ -15,6 +15,24 @@ void exhip_set_error(const char* fmt, ...) {
 
 extern "C" const char* exhip_last_error(void) { return g_err; }
 
+exhip_options g_exhip_options;
+
+extern "C" int exhip_set_option(const char* name, int value) {
+    EXHIP_REQUIRE(name, "exhip_set_option: NULL name");
+    exhip_options& o = g_exhip_options;
+    if (!strcmp(name, "force_variant")) o.force_variant = value;
+    else if (!strcmp(name, "force_chunk")) o.force_chunk = value;
+    else if (!strcmp(name, "force_rs")) o.force_rs = value;
+    else if (!strcmp(name, "force_abufs")) o.force_abufs = value;
+    else if (!strcmp(name, "debug_plan")) o.debug_plan = value;
+    else if (!strcmp(name, "dw_band_rows")) o.dw_band_rows = value;
+    else {
+        exhip_set_error("exhip_set_option: unknown option %s", name);
+        return EXHIP_ERR_ARG;
+    }
+    return 0;
+}
+
 extern "C" int exhip_init(int device, exhip_ctx** out) {
     EXHIP_REQUIRE(out != nullptr, "exhip_init: ctx is NULL");
     int count = 0;

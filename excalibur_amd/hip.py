@@ -44,6 +44,11 @@ def lib():
     return _lib
 
 
+def set_option(name, value):
+    """Test / development switches of the library (exhip_set_option)."""
+    _check(lib().exhip_set_option(name.encode(), int(value)))
+
+
 def _check(rc):
     if rc != 0:
         raise ExhipError(f"exhip error {rc}: {lib().exhip_last_error().decode()}")

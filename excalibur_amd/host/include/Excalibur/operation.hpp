@@ -38,6 +38,10 @@ struct operation_param {
 // adjacent separators are kept, a trailing separator adds none.
 std::vector<std::string> split_string(const std::string& s, const std::string& c);
 
+// Test switch of this backend (process-wide): the fp16 pipeline keeps blobs NHWC between the layers whose kernels work on
+// that layout; `true` keeps every blob NCHW as in the reference.
+void set_f16_nchw_only(bool on);
+
 // key=value attributes of a layer line, in order of appearance
 struct layer_attr {
     std::string key;

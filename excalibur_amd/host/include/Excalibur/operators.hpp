@@ -94,7 +94,8 @@ protected:
     bool q_out_only_ = false;
 
 private:
-    struct packed_entry { void* ptr; size_t bytes; };
+    struct packed_entry { void* ptr; size_t bytes; unsigned long long last_use; };
+    unsigned long long packed_clock_ = 0;
     std::map<std::vector<int>, packed_entry> packed_;
     std::shared_ptr<memory::tensor<float>> scale_dev_;
 };

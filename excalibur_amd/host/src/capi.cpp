@@ -81,6 +81,14 @@ extern "C" void exc_pipeline_set_fusion(exc_pipeline* p, int on) {
     if (p->f16) p->f16->set_fusion(on != 0);
 }
 
+extern "C" int exc_set_option(const char* name, int value) {
+    if (name && !std::strcmp(name, "f16_nchw_only")) {
+        glasssix::excalibur::set_f16_nchw_only(value != 0);
+        return 0;
+    }
+    return exhip_set_option(name, value);
+}
+
 extern "C" int exc_pipeline_blob_stored(exc_pipeline* p, const char* name) {
     return p->f32 ? p->f32->blob_stored(name) : p->f16 ? p->f16->blob_stored(name) : 0;
 }

@@ -13,6 +13,10 @@ namespace {
 std::mutex g_mu;
 std::map<int, exhip_ctx*> g_ctx;
 std::map<std::pair<int, size_t>, std::vector<void*>> g_free;  // (device, rounded bytes) -> idle blocks
+std::map<int, size_t> g_idle_bytes;                            // device -> bytes held idle in g_free
+// Idle blocks are kept for reuse up to this many bytes per device; beyond it a released block goes back to the driver, so
+// a pipeline fed many different resolutions does not grow without bound.
+constexpr size_t kIdleLimit = (size_t)8 << 30;
 
 size_t round_block(size_t bytes) {
     size_t b = 256;
@@ -37,6 +41,21 @@ exhip_ctx* device_context(int device) {
     return ctx;
 }
 
+// Returns every idle block of a device to the driver (exhip_free waits for the device's stream first).
+static void trim_idle(int device, exhip_ctx* ctx) {
+    std::vector<void*> blocks;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        for (auto& kv : g_free)
+            if (kv.first.first == device) {
+                blocks.insert(blocks.end(), kv.second.begin(), kv.second.end());
+                kv.second.clear();
+            }
+        g_idle_bytes[device] = 0;
+    }
+    for (void* b : blocks) exhip_free(ctx, b);
+}
+
 void* device_alloc(int device, size_t bytes) {
     exhip_ctx* ctx = device_context(device);
     const size_t rb = round_block(bytes);
@@ -46,18 +65,30 @@ void* device_alloc(int device, size_t bytes) {
         if (!pool.empty()) {
             void* p = pool.back();
             pool.pop_back();
+            g_idle_bytes[device] -= rb;
             return p;
         }
     }
     void* p = nullptr;
-    EXHIP_FATAL(exhip_malloc(ctx, rb, &p));
+    if (exhip_malloc(ctx, rb, &p) != 0) {  // out of device memory: give the idle blocks back and try once more
+        trim_idle(device, ctx);
+        EXHIP_FATAL(exhip_malloc(ctx, rb, &p));
+    }
     return p;
 }
 
 void device_release(int device, void* ptr, size_t bytes) {
     if (!ptr) return;
-    std::lock_guard<std::mutex> lock(g_mu);
-    g_free[{device, round_block(bytes)}].push_back(ptr);
+    const size_t rb = round_block(bytes);
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        if (g_idle_bytes[device] + rb <= kIdleLimit) {
+            g_free[{device, rb}].push_back(ptr);
+            g_idle_bytes[device] += rb;
+            return;
+        }
+    }
+    exhip_free(device_context(device), ptr);  // over the limit: back to the driver (waits for the stream)
 }
 
 template <typename Dtype>

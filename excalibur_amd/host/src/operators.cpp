@@ -126,12 +126,9 @@ void require_nchw(memory::orderType o) {
 // convention for that order, include/Primitives/tensor.hpp:124-134), channel stride == c, c a multiple of 8. Every other
 // layer, and whoever reads a blob from outside, gets the NCHW form through as_nchw.
 using half_ptr = std::shared_ptr<tensor<unsigned short>>;
-// EXCALIBUR_F16_NCHW=1 (read at every call: tests switch it inside one process) keeps every blob NCHW, the form the
-// NHWC-resident one must agree with bit for bit.
-bool nhwc_allowed() {
-    const char* e = std::getenv("EXCALIBUR_F16_NCHW");
-    return !(e && std::atoi(e) != 0);
-}
+// set_f16_nchw_only(true) keeps every blob NCHW, the form the NHWC-resident one is checked against.
+bool g_f16_nchw_only = false;
+bool nhwc_allowed() { return !g_f16_nchw_only; }
 bool nhwc_channels_ok(int c) { return c % 8 == 0 && nhwc_allowed(); }
 
 half_ptr as_nchw(exhip_ctx* ctx, const half_ptr& t, int device) {
@@ -157,6 +154,8 @@ half_ptr as_order(exhip_ctx* ctx, const half_ptr& t, memory::orderType order, in
 }
 
 }  // namespace
+
+void set_f16_nchw_only(bool on) { g_f16_nchw_only = on; }
 
 // ------------------------------------------------------------------ convolution parameters
 template <typename Dtype>
@@ -380,7 +379,19 @@ template <typename Dtype>
 const void* operation_convolution<Dtype>::packed_weights(int dtype, const exhip_conv_desc& d) {
     const std::vector<int> key{dtype, d.n, d.h, d.w, d.c_stride};
     auto it = packed_.find(key);
-    if (it != packed_.end()) return it->second.ptr;
+    if (it != packed_.end()) {
+        it->second.last_use = ++packed_clock_;
+        return it->second.ptr;
+    }
+    // One packed copy per input geometry, the few most recently used: a detector fed many resolutions would otherwise
+    // keep a copy of its weights for each. (A fused plan holds the pointers of its own geometry, always the latest.)
+    while (packed_.size() >= 4) {
+        auto oldest = packed_.begin();
+        for (auto jt = packed_.begin(); jt != packed_.end(); ++jt)
+            if (jt->second.last_use < oldest->second.last_use) oldest = jt;
+        memory::device_release(this->params_.device_, oldest->second.ptr, oldest->second.bytes);
+        packed_.erase(oldest);
+    }
     const size_t bytes = exhip_conv_packed_bytes(&d, dtype);
     if (bytes == 0) LOG(FATAL) << "layer " << this->params_.name_ << ": " << exhip_last_error();
     std::vector<char> host(bytes);
@@ -400,7 +411,7 @@ const void* operation_convolution<Dtype>::packed_weights(int dtype, const exhip_
     EXHIP_FATAL(exhip_conv_pack_weights(&d, dtype, src, host.data()));
     void* dev = memory::device_alloc(this->params_.device_, bytes);
     EXHIP_FATAL(exhip_memcpy_h2d(this->ctx(), dev, host.data(), bytes));
-    packed_[key] = {dev, bytes};
+    packed_[key] = {dev, bytes, ++packed_clock_};
     return dev;
 }
 

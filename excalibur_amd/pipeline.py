@@ -46,6 +46,13 @@ def lib():
     return _lib
 
 
+def set_option(name, value):
+    """Test / development switches of the backend (see include/excalibur_capi.h)."""
+    rc = lib().exc_set_option(name.encode(), int(value))
+    if rc:
+        raise ValueError(f"unknown option {name}")
+
+
 def registered_operations(dtype="f32"):
     buf = ctypes.create_string_buffer(4096)
     lib().exc_registered_operations({"f32": 0, "f16": 1, "f64": 2}[dtype], buf, 4096)

@@ -48,6 +48,10 @@ long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, long capacit
  * launches lay between them (0 and 0.0 if the last forward was not a fused one). */
 void exc_pipeline_time_fused_span(exc_pipeline* p, int first_launch);
 float exc_pipeline_last_span(exc_pipeline* p, int* launches);
+/* Test and development switches, process-wide (nothing is read from the environment): "f16_nchw_only" = 1 keeps every
+ * blob of pipeline<unsigned short> NCHW instead of NHWC between layers; any other name goes to exhip_set_option.
+ * Returns 0, or an error code for an unknown name. */
+int exc_set_option(const char* name, int value);
 /* Newline-separated list of registered operator class names for a dtype (0 float, 1 unsigned short, 2 double).
  * Returns the length needed. */
 size_t exc_registered_operations(int dtype, char* buf, size_t len);

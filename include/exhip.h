@@ -44,6 +44,12 @@ int exhip_memcpy_d2h(exhip_ctx* ctx, void* dst, const void* src, size_t bytes);
 int exhip_memcpy_d2d(exhip_ctx* ctx, void* dst, const void* src, size_t bytes);
 int exhip_sync(exhip_ctx* ctx);
 const char* exhip_last_error(void);
+/* Switches for tests and development (no counterpart in the reference; the library reads nothing from the environment):
+ * "force_variant" / "force_chunk" / "force_rs" / "force_abufs" pin the convolution planner's tile variant, channel chunk
+ * bytes, filter rows per stage and activation tile buffers, "debug_plan" prints one line per planned layer,
+ * "dw_band_rows" pins the depthwise strip kernels' band height. 0 (-1 for force_variant) restores the planner's choice.
+ * Process-wide; packed weights depend on the first three, so set them before packing. */
+int exhip_set_option(const char* name, int value);
 int exhip_device_name(exhip_ctx* ctx, char* buf, size_t len);
 
 /* HIP events on the context's stream, for timing kernels where they are launched

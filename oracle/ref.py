@@ -31,8 +31,20 @@ def lib():
         L.exref_pipeline_time.restype = ctypes.c_double
         L.exref_pipeline_time.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int),
                                           ctypes.c_int, ctypes.c_int]
+        L.exref_pipeline_time_parallel.restype = ctypes.c_double
+        L.exref_pipeline_time_parallel.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_void_p,
+                                                   ctypes.POINTER(ctypes.c_int), ctypes.c_int, ctypes.c_int, ctypes.c_int]
         _lib = L
     return _lib
+
+
+def time_parallel(topology, model_path, image, workers, warmup, iters, dtype="f32"):
+    """`workers` threads, each with its own pipeline<Dtype> and the same single image (shape 1 x C x H x W), run `iters`
+    timed forwards each -> wall-clock seconds of the timed part."""
+    image = np.ascontiguousarray(image, np.float32 if dtype == "f32" else np.uint16)
+    shape = (ctypes.c_int * 4)(*image.shape)
+    return lib().exref_pipeline_time_parallel(topology.encode(), (model_path or "").encode(), 0 if dtype == "f32" else 1,
+                                              image.ctypes.data, shape, int(workers), int(warmup), int(iters))
 
 
 class Pipeline:

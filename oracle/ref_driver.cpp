@@ -19,6 +19,7 @@
 #include <cstring>
 #include <memory>
 #include <sstream>
+#include <thread>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -110,4 +111,28 @@ EXREF_API double exref_pipeline_time(void* p, const void* input, const int* shap
     for (int i = 0; i < iters; ++i) exref_pipeline_forward(h, input, shape);
     auto t1 = std::chrono::steady_clock::now();
     return std::chrono::duration<double>(t1 - t0).count() / (iters > 0 ? iters : 1);
+}
+
+// The batch-parallel form of the CPU baseline: `workers` threads, each with a pipeline of its own (an instance is
+// single-threaded and keeps per-call state in its operators) and one image, run `iters` forwards after `warmup` untimed
+// ones. Returns the wall-clock seconds of the timed part; images per second = workers * iters / that. The reference's own
+// OpenMP use is off in this build and would be pinned to two threads (src/Excalibur/operation_convolution.cpp:436).
+EXREF_API double exref_pipeline_time_parallel(const char* topology, const char* model_path, int dtype, const void* image,
+                                              const int* shape, int workers, int warmup, int iters) {
+    std::vector<void*> pipes;
+    for (int w = 0; w < workers; ++w) pipes.push_back(exref_pipeline_create(topology, model_path, dtype));
+    auto run = [&](int n) {
+        std::vector<std::thread> threads;
+        for (int w = 0; w < workers; ++w)
+            threads.emplace_back([&, w]() {
+                for (int i = 0; i < n; ++i) exref_pipeline_forward(pipes[w], image, shape);
+            });
+        for (auto& t : threads) t.join();
+    };
+    run(warmup);
+    auto t0 = std::chrono::steady_clock::now();
+    run(iters);
+    auto t1 = std::chrono::steady_clock::now();
+    for (void* p : pipes) exref_pipeline_destroy(p);
+    return std::chrono::duration<double>(t1 - t0).count();
 }

@@ -55,7 +55,7 @@ def _sampled(p, net, half, tol, image, every):
     return [b for b in bad if b[1]]
 
 
-def test_cfg3_mobilenet_style_fp16_at_full_size(monkeypatch):
+def test_cfg3_mobilenet_style_fp16_at_full_size():
     from excalibur_amd.mobilenet import CFG3, MobileFaceNetF32
     net = Net(MobileFaceNetF32(**CFG3).topology(), 61, gain=1.0)
     try:
@@ -80,15 +80,18 @@ def test_cfg3_mobilenet_style_fp16_at_full_size(monkeypatch):
         plain.close()
         # (c) every blob kept NCHW: other kernels for the per-channel and elementwise layers, whose float-to-half
         # conversions may round a product once where the other layout's rounds twice (one half ulp, rarely)
-        monkeypatch.setenv("EXCALIBUR_F16_NCHW", "1")
-        q = _run(net, x, "f16")
-        assert cases.check_value(_f(q.get("out")), _f(out), 2e-3) == 0
-        q.close()
+        xp.set_option("f16_nchw_only", 1)
+        try:
+            q = _run(net, x, "f16")
+            assert cases.check_value(_f(q.get("out")), _f(out), 2e-3) == 0
+            q.close()
+        finally:
+            xp.set_option("f16_nchw_only", 0)
     finally:
         net.close()
 
 
-def test_cfg5_yolov5s_fp16_at_full_size(monkeypatch):
+def test_cfg5_yolov5s_fp16_at_full_size():
     text, outs = topologies.yolov5s_simp(640)
     net = Net(text, 63)
     try:
@@ -110,11 +113,14 @@ def test_cfg5_yolov5s_fp16_at_full_size(monkeypatch):
         small = [L for L in net.layers if L.kind in ("Pooling", "Interp", "BatchNorm", "LeakyRelu") or L.name in ("Concat_300", "Concat_517")]
         assert netref.forced_layer_violations(plain, small[-8:], net.model.weights, True, 2e-3, cases.check_value) == []
         plain.close()
-        monkeypatch.setenv("EXCALIBUR_F16_NCHW", "1")
-        q = _run(net, x[:4], "f16")
-        for o in outs:
-            assert cases.check_value(_f(q.get(o)), _f(got[o][:4]), 2e-3) == 0, o
-        q.close()
+        xp.set_option("f16_nchw_only", 1)
+        try:
+            q = _run(net, x[:4], "f16")
+            for o in outs:
+                assert cases.check_value(_f(q.get(o)), _f(got[o][:4]), 2e-3) == 0, o
+            q.close()
+        finally:
+            xp.set_option("f16_nchw_only", 0)
     finally:
         net.close()
 

@@ -106,12 +106,19 @@ ONE_BUFFER_SHAPES = [
 ]
 
 
+@pytest.fixture
+def one_tile_buffer():
+    from excalibur_amd import hip
+    hip.set_option("force_abufs", 1)
+    yield
+    hip.set_option("force_abufs", 0)
+
+
 @pytest.mark.parametrize("args", ONE_BUFFER_SHAPES, ids=[f"s{a[0]}" for a in ONE_BUFFER_SHAPES])
-def test_conv_i8_single_tile_buffer_bit_exact(ctx, args, monkeypatch):
+def test_conv_i8_single_tile_buffer_bit_exact(ctx, args, one_tile_buffer):
     """The planner trades the second activation tile buffer for one more workgroup per CU only on launches large enough
-    to gain from it; EXHIP_FORCE_ABUFS=1 (read per call) makes these small launches take that path: fused int8 and
+    to gain from it; the option force_abufs = 1 makes these small launches take that path: fused int8 and
     float32 outputs with a shortcut, and the plain NCHW output, all bit-exact."""
-    monkeypatch.setenv("EXHIP_FORCE_ABUFS", "1")
     case = cases.conv_i8_case(*args, act=0)
     g = cases.geom_of(case)
     want_y, want_acc = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], case["act"], g, want_acc=True)

@@ -390,7 +390,7 @@ def test_yolov5_shaped_float_topology_matches_the_reference_fixture():
 
 
 @pytest.mark.parametrize("which", ["mobilefacenet", "yolov5"])
-def test_fp16_pipeline_nhwc_resident_equals_nchw_blobs(monkeypatch, which):
+def test_fp16_pipeline_nhwc_resident_equals_nchw_blobs(which):
     """pipeline<unsigned short> keeps blobs NHWC between its convolution, depthwise, pooling, elementwise and per-channel
     layers; with that switched off every blob is NCHW as in the reference. Layer by layer the arithmetic is the same, so
     the two agree bit for bit: on the output and on blobs in the middle, which come out of the pipeline as NCHW."""
@@ -412,12 +412,15 @@ def test_fp16_pipeline_nhwc_resident_equals_nchw_blobs(monkeypatch, which):
         # the first output blob of a few layers in the middle (line: type name n_in n_out bottoms... tops... keys)
         middle = [l.split()[4 + int(l.split()[2])] for l in net.lines if l.split()[0] in kinds][:12]
         got = {}
-        for flag in ("0", "1"):
-            monkeypatch.setenv("EXCALIBUR_F16_NCHW", flag)
-            p = xp.Pipeline(net.topology(), path, 0, "f16")
-            p.forward(x16)
-            got[flag] = {b: p.get(b) for b in names + middle}
-            p.close()
+        try:
+            for flag in ("0", "1"):
+                xp.set_option("f16_nchw_only", int(flag))
+                p = xp.Pipeline(net.topology(), path, 0, "f16")
+                p.forward(x16)
+                got[flag] = {b: p.get(b) for b in names + middle}
+                p.close()
+        finally:
+            xp.set_option("f16_nchw_only", 0)
         for b in names + middle:
             assert got["0"][b].shape == got["1"][b].shape
             assert np.array_equal(got["0"][b], got["1"][b]), b
