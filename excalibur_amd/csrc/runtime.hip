@@ -151,3 +151,38 @@ extern "C" int exhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms) 
     EXHIP_CHECK(hipEventElapsedTime(ms, (hipEvent_t)ev_start, (hipEvent_t)ev_stop));
     return 0;
 }
+
+// ---- stream capture: a fixed sequence of launches recorded once and replayed as one graph ----
+extern "C" int exhip_graph_begin(exhip_ctx* ctx) {
+    EXHIP_REQUIRE(ctx, "exhip_graph_begin: NULL ctx");
+    EXHIP_CHECK(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    return 0;
+}
+
+extern "C" int exhip_graph_end(exhip_ctx* ctx, void** graph_exec) {
+    EXHIP_REQUIRE(ctx && graph_exec, "exhip_graph_end: NULL argument");
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    EXHIP_CHECK(hipStreamEndCapture(ctx->stream, &graph));
+    EXHIP_REQUIRE(graph != nullptr, "exhip_graph_end: the capture recorded nothing");
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+        exhip_set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+        return (int)e;
+    }
+    *graph_exec = (void*)exec;
+    return 0;
+}
+
+extern "C" int exhip_graph_launch(exhip_ctx* ctx, void* graph_exec) {
+    EXHIP_REQUIRE(ctx && graph_exec, "exhip_graph_launch: NULL argument");
+    EXHIP_CHECK(hipGraphLaunch((hipGraphExec_t)graph_exec, ctx->stream));
+    return 0;
+}
+
+extern "C" int exhip_graph_destroy(void* graph_exec) {
+    if (graph_exec) EXHIP_CHECK(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    return 0;
+}

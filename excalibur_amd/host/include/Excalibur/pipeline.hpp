@@ -39,6 +39,9 @@ public:
     // another blob runs the last input once more layer by layer. blob_stored() tells the two apart.
     void set_fusion(bool on);
     bool blob_stored(std::string_view featmap_name) const;
+    // on: a fused int8 plan replays its launches (all but the input quantizer) as one HIP graph from its second
+    // forward on; off (default: the replay measured no faster than the calls): one call per launch.
+    void set_graphs(bool on);
     bool fused() const;
     double last_forward_ms() const;
     // Device time of part of a fused forward: with first_launch >= 0 every fused forward records one event in front

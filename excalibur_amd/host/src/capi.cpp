@@ -93,6 +93,10 @@ extern "C" int exc_pipeline_blob_stored(exc_pipeline* p, const char* name) {
     return p->f32 ? p->f32->blob_stored(name) : p->f16 ? p->f16->blob_stored(name) : 0;
 }
 
+extern "C" void exc_pipeline_set_graphs(exc_pipeline* p, int on) {
+    if (p->f32) p->f32->set_graphs(on != 0);
+}
+
 extern "C" int exc_pipeline_last_fused(exc_pipeline* p) { return p->f32 ? p->f32->fused() : 0; }
 
 extern "C" void exc_pipeline_time_fused_span(exc_pipeline* p, int first_launch) {

@@ -315,6 +315,10 @@ public:
 
     bool profile_ = false;
     bool fusion_ = true;
+    // Fused plans can replay their launches as one HIP graph (set_graphs). Off by default: measured on MI355X the replay
+    // is no faster than the calls (the pause between two dependent launches is the device's own hand-over and is there
+    // inside a graph too), at batch 32 x 640 x 640 as at one 64 x 64 image.
+    bool graphs_ = false;
     bool last_fused_ = false;
     double last_ms_ = 0;
     int span_first_ = -1, span_launches_ = 0;  // time_fused_span / last_span
@@ -432,6 +436,15 @@ struct pipeline<Dtype>::impl::fused_plan {
     };
     std::deque<result> outputs;  // stable addresses: the launches keep pointers to the slots
     const float* input_ptr = nullptr;
+    // Launches 1 .. end (everything behind the input quantizer, which alone reads the caller's input pointer) recorded as
+    // one HIP graph: made on the plan's second forward (the first runs eagerly, which also sets the kernels' attributes),
+    // replayed afterwards, made again when a result tensor was replaced.
+    void* graph = nullptr;
+    std::vector<float*> graph_slots;
+    int forwards = 0;
+    ~fused_plan() {
+        if (graph) exhip_graph_destroy(graph);
+    }
     float** new_result(const std::vector<int>& shape, int device) {
         outputs.emplace_back();
         result& r = outputs.back();
@@ -711,22 +724,46 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
             r.slot = r.t->mutable_gpu_data();
         }
     }
-    if (span_first_ >= 0 && span_first_ < static_cast<int>(plan_->launches.size())) {
-        exhip_ctx* ctx = memory::device_context(device_);
-        if (!span_ev_[0]) {
-            EXHIP_FATAL(exhip_event_create(&span_ev_[0]));
-            EXHIP_FATAL(exhip_event_create(&span_ev_[1]));
+    exhip_ctx* const ctx = memory::device_context(device_);
+    const int n_launches = static_cast<int>(plan_->launches.size());
+    const bool timed = span_first_ >= 0 && span_first_ < n_launches;
+    if (timed && !span_ev_[0]) {
+        EXHIP_FATAL(exhip_event_create(&span_ev_[0]));
+        EXHIP_FATAL(exhip_event_create(&span_ev_[1]));
+    }
+    // the graph form: launch 0 eagerly, the rest as one replay (a timed span must start at launch 0 or 1 to use it)
+    bool use_graph = graphs_ && n_launches > 2 && plan_->forwards >= 1 && (!timed || span_first_ <= 1);
+    if (use_graph) {
+        std::vector<float*> slots;
+        for (auto& r : plan_->outputs) slots.push_back(r.slot);
+        if (plan_->graph && slots != plan_->graph_slots) {
+            EXHIP_FATAL(exhip_graph_destroy(plan_->graph));
+            plan_->graph = nullptr;
         }
-        for (int i = 0; i < static_cast<int>(plan_->launches.size()); ++i) {
+        if (!plan_->graph) {
+            EXHIP_FATAL(exhip_graph_begin(ctx));
+            for (int i = 1; i < n_launches; ++i) plan_->launches[i]();
+            EXHIP_FATAL(exhip_graph_end(ctx, &plan_->graph));
+            plan_->graph_slots = slots;
+        }
+        if (timed && span_first_ == 0) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+        plan_->launches[0]();
+        if (timed && span_first_ == 1) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+        EXHIP_FATAL(exhip_graph_launch(ctx, plan_->graph));
+        if (timed) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[1]));
+        span_launches_ = timed ? n_launches - span_first_ : 0;
+    } else if (timed) {
+        for (int i = 0; i < n_launches; ++i) {
             if (i == span_first_) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
             plan_->launches[i]();
         }
         EXHIP_FATAL(exhip_event_record(ctx, span_ev_[1]));
-        span_launches_ = static_cast<int>(plan_->launches.size()) - span_first_;
+        span_launches_ = n_launches - span_first_;
     } else {
         for (auto& launch : plan_->launches) launch();
         span_launches_ = 0;
     }
+    ++plan_->forwards;
     last_fused_ = true;
     for (auto& r : plan_->outputs) {
         r.t->mutable_gpu_data();  // the kernels just wrote it: the device copy is the newest
@@ -779,6 +816,8 @@ template <typename Dtype>
 void pipeline<Dtype>::set_fusion(bool on) { impl_->fusion_ = on; }
 template <typename Dtype>
 bool pipeline<Dtype>::fused() const { return impl_->last_fused_; }
+template <typename Dtype>
+void pipeline<Dtype>::set_graphs(bool on) { impl_->graphs_ = on; }
 
 template <typename Dtype>
 void pipeline<Dtype>::time_fused_span(int first_launch) { impl_->span_first_ = first_launch; }

@@ -29,6 +29,7 @@ def lib():
         L.exc_pipeline_destroy.argtypes = [ctypes.c_void_p]
         L.exc_pipeline_set_fusion.argtypes = [ctypes.c_void_p, ctypes.c_int]
         L.exc_pipeline_last_fused.argtypes = [ctypes.c_void_p]
+        L.exc_pipeline_set_graphs.argtypes = [ctypes.c_void_p, ctypes.c_int]
         L.exc_pipeline_blob_stored.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
         L.exc_pipeline_set_input.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
         L.exc_pipeline_run.argtypes = [ctypes.c_void_p]
@@ -88,6 +89,10 @@ class Pipeline:
 
     def run(self):
         lib().exc_pipeline_run(self.h)
+
+    def set_graphs(self, on):
+        """Fused int8 plans replay their launches as one HIP graph, or (default) issue them one by one."""
+        lib().exc_pipeline_set_graphs(self.h, int(on))
 
     def run_keeping(self):
         """forward() while the results of the earlier forwards stay held; get_kept(back, name) reads them."""

@@ -23,6 +23,9 @@ void exc_pipeline_destroy(exc_pipeline* p);
  * them; 0: every layer through forward_gpu, every blob stored. */
 void exc_pipeline_set_fusion(exc_pipeline* p, int on);
 int exc_pipeline_last_fused(exc_pipeline* p);
+/* 1: a fused int8 plan replays its launches as one HIP graph from its second forward on; 0 (default; the replay
+ * measured no faster than the calls on MI355X): one call per launch. */
+void exc_pipeline_set_graphs(exc_pipeline* p, int on);
 /* 1 if the last forward itself stored blob `name` as a float tensor; 0 for a blob a fused executor skipped, which
  * exc_pipeline_get then obtains by running the last input once more layer by layer. */
 int exc_pipeline_blob_stored(exc_pipeline* p, const char* name);

@@ -59,6 +59,16 @@ int exhip_event_destroy(void* ev);
 int exhip_event_record(exhip_ctx* ctx, void* ev);
 int exhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms); /* synchronises on ev_stop */
 
+/* A fixed sequence of launches recorded once and replayed as one HIP graph (no counterpart in the reference, whose
+ * executor issues one call per layer, src/Excalibur/pipeline.cpp:326-392): between exhip_graph_begin and exhip_graph_end
+ * every kernel an entry point of this library launches on the context's stream is recorded instead of run (entry points
+ * that copy, fill or synchronise must not be called there); exhip_graph_launch replays the recording with the pointers
+ * and sizes it was made with. */
+int exhip_graph_begin(exhip_ctx* ctx);
+int exhip_graph_end(exhip_ctx* ctx, void** graph_exec);
+int exhip_graph_launch(exhip_ctx* ctx, void* graph_exec);
+int exhip_graph_destroy(void* graph_exec);
+
 /* ---- layout / precision conversion at the boundary ---- */
 /* quantize_float32_to_int8 (src/Excalibur/operation_general_conv.cpp:584-720) fused with NCHW->NHWC:
  * y[n,h,w,c] = sat8(trunc(x[n,c,h,w]*fs +- 0.5)); fs per tensor (fs_per_channel == NULL) or a device
