@@ -9,7 +9,16 @@
 struct exhip_ctx {
     int device;
     hipStream_t stream;
+    // scratch of the convolution's split reduction, grown on demand and kept until the context is destroyed
+    int* split_acc = nullptr;
+    size_t split_acc_bytes = 0;
+    unsigned* split_count = nullptr;
+    size_t split_count_n = 0;
 };
+
+// Makes the context's split-reduction scratch at least this large (partial accumulators, and one zeroed arrival counter per
+// tile) and returns it. Growing it waits for the stream; no allocation happens when it is large enough already.
+int exhip_split_scratch(exhip_ctx* ctx, size_t acc_bytes, size_t tiles, int** acc, unsigned** count);
 
 void exhip_set_error(const char* fmt, ...);
 
@@ -46,6 +55,7 @@ struct exhip_options {
     int force_abufs = 0;     // activation tile buffers (1 / 2)
     int debug_plan = 0;      // one line per planned layer on stderr
     int dw_band_rows = 0;    // row-band height of the depthwise strip kernels
+    int force_splits = 0;    // groups per tile of the convolution's split reduction (1 = never split)
 };
 extern exhip_options g_exhip_options;
 

@@ -108,6 +108,12 @@ struct ConvParams {
     int tile_dy, tile_dx;     // output pixels between the origins of neighbouring patches (PH, PW unless pooled)
     int tile_oy, tile_ox;     // the first patch starts this many pixels before output pixel 0 (pooled form: the pool's padding)
     int MPH, MPW, POH, POW;   // pooled form: pooled pixels per patch and pooled image size
+    // Split reduction (launches with too few tiles to fill the chip): `splits` groups share a tile, each reduces a run of
+    // channel chunks and leaves its raw accumulators in split_acc; the group that arrives last at the tile's counter
+    // adds the parts in split order and runs the epilogue. 1 = off.
+    int splits;
+    int* split_acc;           // [tile][split][16 vectors][THREADS][4] accumulator words (int32 or float bits)
+    unsigned* split_count;    // [tile] arrivals, back to 0 when the tile is done
 };
 
 template <int DT> struct Acc { typedef v16i type; };
@@ -267,6 +273,10 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         const int per = gridDim.x >> 3;
         if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
     }
+    // a split reduction's groups of one tile are neighbours in the grid
+    const int sp = __builtin_amdgcn_readfirstlane(p.splits > 1 ? bid % p.splits : 0);
+    if (p.splits > 1) bid /= p.splits;
+    const int tile_id = bid;
     const int kt = __builtin_amdgcn_readfirstlane(bid % p.ktiles);
     int t = bid / p.ktiles;
     const int tx = __builtin_amdgcn_readfirstlane(t % p.tiles_x);
@@ -365,8 +375,11 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
     const int row_w_b = p.KWe * p.KS * (TM / 32) * 1024;  // packed weight bytes of one filter row
-    const int n_stages = p.n_chunks * p.n_rg;
-    const char* const wkt = p.wp + (size_t)kt * p.n_chunks * p.KH * row_w_b;
+    // this group's run of channel chunks: all of them, or its share of a split reduction
+    const int chunk0 = __builtin_amdgcn_readfirstlane(p.splits > 1 ? sp * p.n_chunks / p.splits : 0);
+    const int my_chunks = __builtin_amdgcn_readfirstlane(p.splits > 1 ? (sp + 1) * p.n_chunks / p.splits - chunk0 : p.n_chunks);
+    const int n_stages = my_chunks * p.n_rg;
+    const char* const wkt = p.wp + ((size_t)kt * p.n_chunks + chunk0) * p.KH * row_w_b;
     auto stage_rows = [&](int rg) { const int r0 = rg * p.RS; return (p.KH - r0 < p.RS ? p.KH - r0 : p.RS); };
     // (chunk, row group) of the stage `by` stages after (cc, rg), without dividing
     auto stage_after = [&](int cc, int rg, int by, int& cc_out, int& rg_out) {
@@ -547,9 +560,9 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 if (w_dst == w_lds_end) w_dst = w_lds0;
             }
         };
-        const char* a_src = ximg;                  // channel chunk of the next tile to request
-        int a_range = (int)p.img_bytes;
-        int a_req_left = p.n_chunks;
+        const char* a_src = ximg + chunk0 * p.chunk_b;  // channel chunk of the next tile to request
+        int a_range = (int)p.img_bytes - chunk0 * p.chunk_b;
+        int a_req_left = my_chunks;
         unsigned a_dst = lds_base + kSbBytes + wave_slot;
         const unsigned a_flip = p.act_bufs > 1 ? (unsigned)p.lds_act_b : 0u;  // the two tile buffers alternate
         bool a_odd = false;
@@ -743,6 +756,62 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
     }
 
     stamp(5);
+    if (p.splits > 1) {
+        // every group leaves its accumulators (a lane's 64 words as 16 vectors, lanes contiguous per vector); the one
+        // that finds the tile's counter at splits - 1 is the last: it adds the parts in split order, so the result
+        // does not depend on who came last, and goes on to the epilogue
+        // (the counter's value travels through the first word of the staging area: the loop ended with a barrier, so
+        // nobody reads that area any more, and the epilogue's tiles are written only after this exchange)
+        volatile unsigned* const arrived = reinterpret_cast<volatile unsigned*>(smem + kSbBytes);
+        // The parts travel with the cache policy of device-scope atomic accesses (sc0 sc1: stores are written through,
+        // loads are not served from a cache that another XCD's stores cannot reach), so that no fence has to write back
+        // or invalidate a whole L2: all that is needed is that a group's stores have completed before its arrival counts.
+        constexpr int kDeviceCoherent = 1 | 16;  // sc0 | sc1
+        const unsigned part_b = 16u * THREADS * 16u;  // bytes of one group's part
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            reinterpret_cast<char*>(p.split_acc) + (size_t)tile_id * p.splits * part_b, 0, (int)(p.splits * part_b), kRsrcWord3);
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    v4i v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const auto a = acc[i][j][e4 * 4 + e];  // a scalar copy: a bit cast of a vector element reads element 0
+                        v[e] = __builtin_bit_cast(int, a);
+                    }
+                    __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)(((((i * NT + j) * 4 + e4) * THREADS) + tid) * 16u), (int)(sp * part_b),
+                                                           kDeviceCoherent);
+                }
+        __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) *arrived = atomicAdd(p.split_count + tile_id, 1u);
+        __syncthreads();
+        const unsigned before_me = *arrived;
+        __syncthreads();  // everyone has read the word before the epilogue reuses the area
+        if (before_me != (unsigned)(p.splits - 1)) return;
+        if (tid == 0) p.split_count[tile_id] = 0;  // ready for the next launch (launches on one stream run in order)
+        for (int q = 0; q < p.splits; ++q) {
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(((((i * NT + j) * 4 + e4) * THREADS) + tid) * 16u),
+                                                                            (int)(q * part_b), kDeviceCoherent);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            typedef decltype(acc[i][j][0] + acc[i][j][0]) elem_t;
+                            const int word = v[e];
+                            const elem_t x = __builtin_bit_cast(elem_t, word);
+                            acc[i][j][e4 * 4 + e] = q == 0 ? x : acc[i][j][e4 * 4 + e] + x;
+                        }
+                    }
+        }
+    }
     // ---- epilogue ----
     // A lane holds, per accumulator tile, 16 consecutive output channels of one pixel.
     const int img_px = p.OH * p.OW;
@@ -1539,8 +1608,27 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         p.magic_mpw = (unsigned)(((1ull << 32) + pl.MPW - 1) / pl.MPW);
     }
     EXHIP_REQUIRE((long long)d->n * pl.OH * pl.OW < (1ll << 31), "conv: more than 2^31 output pixels");
-    const long long grid = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
-    EXHIP_REQUIRE(grid > 0 && grid < (1ll << 31), "conv: grid too large");
+    const long long tiles = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
+    EXHIP_REQUIRE(tiles > 0 && tiles < (1ll << 31), "conv: grid too large");
+    // A launch with too few tiles for the chip's 256 CUs (one image, deep layers) walks its whole reduction on a handful
+    // of groups, one stage after the other. Such a launch splits each tile's channel chunks over several groups (at least
+    // three stages each, which the loop's prologue counts on), up to about two groups per CU; the parts are added in a
+    // fixed order, exactly for int32 and reproducibly for float.
+    p.splits = 1;
+    if (!pl.packed && !pool && g_exhip_options.force_splits != 1) {
+        const int min_chunks = (3 + pl.n_rg - 1) / pl.n_rg;
+        long long s = std::min<long long>(pl.n_chunks / min_chunks, kCUs / tiles);  // measured: no gain once every CU has a group
+        s = std::min<long long>(s, 16);
+        if (g_exhip_options.force_splits > 1) s = std::min<long long>(g_exhip_options.force_splits, pl.n_chunks / min_chunks);
+        if (s >= 2) {
+            const size_t acc_bytes = (size_t)tiles * s * pl.threads * 256;  // 64 words per lane
+            rc = exhip_split_scratch(ctx, acc_bytes, (size_t)tiles, &p.split_acc, &p.split_count);
+            if (rc) return rc;
+            p.splits = (int)s;
+        }
+    }
+    const long long grid = tiles * p.splits;
+    EXHIP_REQUIRE(grid < (1ll << 31), "conv: grid too large");
     if constexpr (DT == EXHIP_I8) {
         if (pool) {
             const long long out_elems = (long long)d->n * pool->oh * pool->ow * d->k;

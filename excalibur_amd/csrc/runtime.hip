@@ -2,6 +2,8 @@
 #include <stdarg.h>
 #include <string.h>
 
+#include <algorithm>
+
 #include "common.h"
 
 static thread_local char g_err[512] = "";
@@ -26,6 +28,7 @@ extern "C" int exhip_set_option(const char* name, int value) {
     else if (!strcmp(name, "force_abufs")) o.force_abufs = value;
     else if (!strcmp(name, "debug_plan")) o.debug_plan = value;
     else if (!strcmp(name, "dw_band_rows")) o.dw_band_rows = value;
+    else if (!strcmp(name, "force_splits")) o.force_splits = value;
     else {
         exhip_set_error("exhip_set_option: unknown option %s", name);
         return EXHIP_ERR_ARG;
@@ -62,6 +65,8 @@ extern "C" int exhip_init(int device, exhip_ctx** out) {
 extern "C" int exhip_destroy(exhip_ctx* ctx) {
     if (!ctx) return 0;
     (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->split_acc) (void)hipFree(ctx->split_acc);
+    if (ctx->split_count) (void)hipFree(ctx->split_count);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return 0;
@@ -184,5 +189,30 @@ extern "C" int exhip_graph_launch(exhip_ctx* ctx, void* graph_exec) {
 
 extern "C" int exhip_graph_destroy(void* graph_exec) {
     if (graph_exec) EXHIP_CHECK(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    return 0;
+}
+
+int exhip_split_scratch(exhip_ctx* ctx, size_t acc_bytes, size_t tiles, int** acc, unsigned** count) {
+    if (acc_bytes > ctx->split_acc_bytes) {
+        EXHIP_CHECK(hipStreamSynchronize(ctx->stream));
+        if (ctx->split_acc) EXHIP_CHECK(hipFree(ctx->split_acc));
+        ctx->split_acc = nullptr;
+        ctx->split_acc_bytes = 0;
+        const size_t want = std::max(acc_bytes, (size_t)4 << 20);
+        EXHIP_CHECK(hipMalloc(reinterpret_cast<void**>(&ctx->split_acc), want));
+        ctx->split_acc_bytes = want;
+    }
+    if (tiles > ctx->split_count_n) {
+        EXHIP_CHECK(hipStreamSynchronize(ctx->stream));
+        if (ctx->split_count) EXHIP_CHECK(hipFree(ctx->split_count));
+        ctx->split_count = nullptr;
+        ctx->split_count_n = 0;
+        const size_t want = std::max(tiles, (size_t)1024);
+        EXHIP_CHECK(hipMalloc(reinterpret_cast<void**>(&ctx->split_count), want * sizeof(unsigned)));
+        EXHIP_CHECK(hipMemset(ctx->split_count, 0, want * sizeof(unsigned)));  // every launch leaves its counters at zero
+        ctx->split_count_n = want;
+    }
+    *acc = ctx->split_acc;
+    *count = ctx->split_count;
     return 0;
 }

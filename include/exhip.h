@@ -47,7 +47,8 @@ const char* exhip_last_error(void);
 /* Switches for tests and development (no counterpart in the reference; the library reads nothing from the environment):
  * "force_variant" / "force_chunk" / "force_rs" / "force_abufs" pin the convolution planner's tile variant, channel chunk
  * bytes, filter rows per stage and activation tile buffers, "debug_plan" prints one line per planned layer,
- * "dw_band_rows" pins the depthwise strip kernels' band height. 0 (-1 for force_variant) restores the planner's choice.
+ * "dw_band_rows" pins the depthwise strip kernels' band height, "force_splits" the groups per tile of the convolution's
+ * split reduction (1 = never split). 0 (-1 for force_variant) restores the planner's choice.
  * Process-wide; packed weights depend on the first three, so set them before packing. */
 int exhip_set_option(const char* name, int value);
 int exhip_device_name(exhip_ctx* ctx, char* buf, size_t len);

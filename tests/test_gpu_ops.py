@@ -546,3 +546,59 @@ def test_quantizer_with_per_input_channel_scales(ctx, shape, cs):
     want = port.quantize(x, fs).transpose(0, 2, 3, 1)
     assert np.array_equal(got[..., :shape[1]], want)
     assert not got[..., shape[1]:].any()
+
+
+@pytest.fixture(params=[1, 0, 3])
+def splits(request):
+    """The convolution's split reduction: never (1), the planner's choice (0), three groups per tile where the layer allows."""
+    from excalibur_amd import hip
+    hip.set_option("force_splits", request.param)
+    yield request.param
+    hip.set_option("force_splits", 0)
+
+
+SPLIT_SHAPES = [
+    # seed, n, c, h, w, k, kernel, stride, pad: launches of a few tiles with several channel chunks
+    (600, 1, 256, 14, 14, 64, 3, 1, 1),
+    (601, 1, 512, 7, 9, 128, 3, 1, 1),
+    (602, 2, 384, 6, 6, 72, 1, 1, 0),      # 1x1: three chunks to a part; ragged channel count (general epilogue)
+    (603, 1, 128, 20, 20, 256, 3, 2, 1),
+]
+
+
+@pytest.mark.parametrize("args", SPLIT_SHAPES, ids=[f"s{a[0]}" for a in SPLIT_SHAPES])
+def test_conv_split_reduction_int8_bit_exact(ctx, args, splits):
+    """Few tiles, deep reduction: the tile's channel chunks are reduced by several groups and the int32 parts added by
+    the last one to arrive. Accumulators, float output and the fused shortcut / requantized outputs equal the oracle's
+    whichever way the launch is split; run twice in a row (the arrival counters must be back at zero)."""
+    case = cases.conv_i8_case(*args, act=0)
+    g = cases.geom_of(case)
+    want_y, want_acc = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], 0, g, want_acc=True)
+    for _ in range(2):
+        got = gpueval.conv_i8(ctx, case)
+        assert np.array_equal(got["acc"], want_acc)
+        assert np.array_equal(got["nchw"], want_y)
+    if args[5] % 64 == 0:
+        r = np.random.default_rng(args[0] + 1)
+        res = r.uniform(-4, 4, want_y.shape).astype(np.float32)
+        fs_out = np.float32(13.1)
+        z = port.relu(port.binaryop_add(want_y, res))
+        fused = gpueval.conv_i8(ctx, case, fs_out=fs_out, residual=np.ascontiguousarray(res.transpose(0, 2, 3, 1)), post_relu=1, want=("nhwc",))
+        assert np.array_equal(fused["nhwc"], z.transpose(0, 2, 3, 1))
+        assert np.array_equal(fused["i8"], port.quantize(z, fs_out).transpose(0, 2, 3, 1))
+
+
+def test_conv_split_reduction_float_within_tolerance(ctx, splits):
+    """The benchmark set's single float32 layer (1 x 64 x 56 x 56 -> 64, 3x3, bias, ReLU: 13 tiles on 256 CUs) and a half
+    layer: the parts are added in split order, so a launch gives the same bits every time, within 1e-4 / 2e-3 of the oracle."""
+    case = cases.conv_f32_case(610, 1, 64, 56, 56, 64, 3, 1, 1)
+    want = cases.oracle_eval(case)
+    a = gpueval.conv_f32(ctx, case)
+    assert cases.check_value(a, want, 1e-4) == 0
+    assert np.array_equal(a, gpueval.conv_f32(ctx, case))
+    case = cases.conv_f32_case(611, 1, 256, 14, 14, 128, 3, 1, 1)
+    x16 = case["x"].astype(np.float16)
+    want = cases.oracle_eval(dict(case, x=x16.astype(np.float32)))
+    h = gpueval.conv_f16(ctx, case, x16.view(np.uint16))
+    assert cases.check_value(h.view(np.float16).astype(np.float32), want, 2e-3) == 0
+    assert np.array_equal(h, gpueval.conv_f16(ctx, case, x16.view(np.uint16)))
