@@ -228,6 +228,15 @@ def bandwidth_table(iters=20, quiet=False, ctx=None):
        lambda: L.exhip_dwconv3x3_nhwc_f16(ctx.h, dx.ptr, w9.ptr, b9.ptr, dy.ptr, dn, dc, dh, dh, dc, 1, 1, 1, 1, 1, 1))
     bw("depthwise 3x3 s2 f16 NHWC, 64x128x56x56", dx.size * 2 + dx.size // 2,
        lambda: L.exhip_dwconv3x3_nhwc_f16(ctx.h, dx.ptr, w9.ptr, b9.ptr, dy.ptr, dn, dc, dh, dh, dc, 2, 1, 1, 1, 1, 1))
+    # global average pooling, the last layer of the MobileNet-style stack (64 x 1024 x 7 x 7) and of a 20 x 20 backbone
+    gx = ctx.array(rng.normal(0, 1, (64, 7, 7, 1024)).astype(np.float16).view(np.uint16))
+    gy = ctx.empty((64, 1, 1, 1024), np.uint16)
+    bw("global average pool f16 NHWC, 64x1024x7x7", gx.size * 2 + gy.size * 2,
+       lambda: L.exhip_pool2d_nhwc_f16(ctx.h, gx.ptr, gy.ptr, 64, 1024, 7, 7, 1024, 1, 1, 1, 7, 7, 1, 1, 0, 0, 0, 0, 0))
+    gf = ctx.array(rng.normal(0, 1, (32, 512, 20, 20)).astype(np.float32))
+    gfy = ctx.empty((32, 512, 1, 1), np.float32)
+    bw("global average pool f32 NCHW, 32x512x20x20", gf.size * 4 + gfy.size * 4,
+       lambda: L.exhip_pool2d_nchw_f32(ctx.h, gf.ptr, gfy.ptr, 32, 512, 20, 20, 1, 1, 1, 20, 20, 1, 1, 0, 0, 0, 0, 0))
     if own_ctx:
         ctx.close()
     return rows

@@ -6,6 +6,7 @@
 #include <float.h>
 
 #include <mutex>
+#include <type_traits>
 
 #include "common.h"
 
@@ -251,6 +252,14 @@ __device__ __forceinline__ float dw_pixel(const float r[3][3], const float* k, f
     return sum;
 }
 
+// Workgroup ids are dealt round-robin to the chip's 8 XCDs, each with an L2 of its own. Remapped like this every XCD
+// works on one contiguous run of a kernel's blocks, so that neighbouring blocks (row bands of one image, which read each
+// other's border rows) meet in one L2.
+__device__ __forceinline__ unsigned xcd_contiguous_block() {
+    const unsigned per = gridDim.x >> 3, b = blockIdx.x;
+    return b < (per << 3) ? (b & 7) * per + (b >> 3) : b;
+}
+
 __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                                     const float* __restrict__ bias, float* __restrict__ y,
                                                                     int C, int H, int W, int OH, int OW, int stride, int pt,
@@ -294,7 +303,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nchw_f32_strip_kernel(const 
     constexpr int CH = STRIDE == 1 ? 1 : 2;  // aligned 16-byte chunks per row
     constexpr int NI = 4 * CH + 3, KEEP = 3 - STRIDE;
     constexpr unsigned kRowOutside = 0x80000000u, kColOutside = 0x40000000u;  // tensors are at most 2^30 bytes
-    const size_t gi = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t gi = (size_t)xcd_contiguous_block() * kBlock + threadIdx.x;
     if (gi >= total) return;
     const int t = (int)(gi % strips);
     size_t rest = gi / strips;
@@ -438,7 +447,7 @@ __global__ __launch_bounds__(kBlock) void dwconv3x3_nhwc_f16_kernel(const uint16
 // by vector ALU issue as much as by memory, hence the template on the activation and the masked, packed stores.
 // Arithmetic order per output is that of dw_pixel.
 template <int STRIDE, int PX, int ACT>
-__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) void dwconv3x3_nhwc_f16_strip_kernel(const uint16_t* __restrict__ x,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(3, 4))) void dwconv3x3_nhwc_f16_strip_kernel(const uint16_t* __restrict__ x,
                                                                           const float* __restrict__ w,
                                                                           const float* __restrict__ bias,
                                                                           uint16_t* __restrict__ y, int C, int H, int W,
@@ -450,7 +459,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     // out-of-range markers: a tensor is at most 2^30 bytes, so a valid row offset plus the column marker, the row
     // marker plus anything, and both markers together all land beyond the descriptor's range without wrapping
     constexpr unsigned kRowOutside = 0x80000000u, kColOutside = 0x40000000u;
-    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t i = (size_t)xcd_contiguous_block() * kBlock + threadIdx.x;
     if (i >= total) return;
     const int groups = cs / 4;
     const int g = (int)(i % groups);
@@ -485,6 +494,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     // channels of the padding are stored as zero halves
     const int keep_lo = (c0 < C ? 0xffff : 0) | (c0 + 1 < C ? 0xffff0000 : 0);
     const int keep_hi = (c0 + 2 < C ? 0xffff : 0) | (c0 + 3 < C ? 0xffff0000 : 0);
+    const bool ragged_c = (C & 3) != 0 || cs != C;  // uniform over the launch: whole groups of four channels need no masks
     const int oy0 = band * band_rows, oy1 = min(OH, oy0 + band_rows);
     const int ox0 = xs * PX, ix0 = ox0 * STRIDE - pl;
     const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(x), 0, (int)x_bytes, 0x00020000);
@@ -499,30 +509,30 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
     }
 #pragma unroll
     for (int px = 0; px < PX; ++px) ocol_off[px] = ox0 + px < OW ? (unsigned)((ox0 + px) * cs * 2) : kColOutside;
-    v4h r[3][NC], nxt[STRIDE][NC];
+    // The input rows live in a ring of 3 + D * STRIDE register rows: output row t reads ring slots (t * STRIDE + a) % R,
+    // a = 0 .. 2, while the rows the next D output rows add are already on their way into the slots behind them. The
+    // row loop is unrolled over one turn of the ring, so every slot index is a constant and no row is ever copied.
+    // D: how many output rows ahead the input rows are requested (two at stride 1, where a row's arithmetic is too short to
+    // cover the memory latency with three waves per SIMD).
+    constexpr int D = STRIDE == 1 ? 2 : 1;
+    constexpr int R = 3 + D * STRIDE, TURN = R;  // R and STRIDE are coprime (4 or 5 and 1, 5 and 2): a turn is R output rows
+    v4h r[R][NC];
     auto fetch = [&](int iy, v4h (&dst)[NC]) {
         const unsigned row_off = iy >= 0 && iy < H ? (unsigned)(img_off + iy * row_b) : kRowOutside;
 #pragma unroll
         for (int cidx = 0; cidx < NC; ++cidx)
             dst[cidx] = __builtin_bit_cast(v4h, __builtin_amdgcn_raw_buffer_load_b64(xr, (int)(row_off + col_off[cidx]), 0, 0));
     };
-    // rows that the first step keeps from "the step before" go where the shift below expects them
 #pragma unroll
-    for (int a = 0; a < KEEP; ++a) fetch(oy0 * STRIDE - pt + a, r[STRIDE + a]);
-#pragma unroll
-    for (int a = 0; a < STRIDE; ++a) fetch(oy0 * STRIDE - pt + KEEP + a, nxt[a]);
+    for (int a = 0; a < (D - 1) * STRIDE + 3; ++a) fetch(oy0 * STRIDE - pt + a, r[a]);
     unsigned orow_off = (unsigned)((n * OH + oy0) * orow_b + c0 * 2);
-    for (int oy = oy0; oy < oy1; ++oy, orow_off += orow_b) {
+    // one output row, PH = its position in the turn
+    auto row = [&](auto ph, int oy) {
+        constexpr int PH = decltype(ph)::value;
+        if (oy + D < oy1) {
 #pragma unroll
-        for (int cidx = 0; cidx < NC; ++cidx) {
-#pragma unroll
-            for (int a = 0; a < KEEP; ++a) r[a][cidx] = r[a + STRIDE][cidx];
-#pragma unroll
-            for (int a = 0; a < STRIDE; ++a) r[KEEP + a][cidx] = nxt[a][cidx];
-        }
-        if (oy + 1 < oy1) {
-#pragma unroll
-            for (int a = 0; a < STRIDE; ++a) fetch((oy + 1) * STRIDE - pt + KEEP + a, nxt[a]);
+            for (int a = 0; a < STRIDE; ++a)
+                fetch((oy + D) * STRIDE - pt + 3 - STRIDE + a, r[((PH + D) * STRIDE + 3 - STRIDE + a) % R]);
         }
 #pragma unroll
         for (int px = 0; px < PX; ++px) {
@@ -534,7 +544,7 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                 for (int j = 0; j < 3; ++j) {
                     float s = 0.f;
 #pragma unroll
-                    for (int a = 0; a < 3; ++a) s = __builtin_fmaf((float)r[a][px * STRIDE + j][e], k[e][a * 3 + j], s);
+                    for (int a = 0; a < 3; ++a) s = __builtin_fmaf((float)r[(PH * STRIDE + a) % R][px * STRIDE + j][e], k[e][a * 3 + j], s);
                     sum += s;
                 }
                 // activations 0 (none), 1 (ReLU), 3 (ReLU6 as the reference writes it)
@@ -548,11 +558,24 @@ __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4, 4))) 
                 res[e] = sum;
             }
             v2i o = __builtin_bit_cast(v2i, __builtin_convertvector(res, v4h));
-            o[0] &= keep_lo;
-            o[1] &= keep_hi;
+            if (ragged_c) {
+                o[0] &= keep_lo;
+                o[1] &= keep_hi;
+            }
             __builtin_amdgcn_raw_buffer_store_b64(o, yr, (int)(orow_off + ocol_off[px]), 0, 0);
         }
-    }
+        orow_off += orow_b;
+    };
+    auto turn = [&](auto self, auto ph, int oy) -> void {
+        constexpr int PH = decltype(ph)::value;
+        if constexpr (PH < TURN) {
+            if (oy < oy1) {
+                row(ph, oy);
+                self(self, std::integral_constant<int, PH + 1>{}, oy + 1);
+            }
+        }
+    };
+    for (int oy = oy0; oy < oy1; oy += TURN) turn(turn, std::integral_constant<int, 0>{}, oy);
 }
 
 __global__ __launch_bounds__(kBlock) void dw_dequant_kernel(const int8_t* __restrict__ w, const float* __restrict__ ws,
@@ -942,6 +965,60 @@ __global__ __launch_bounds__(kBlock) void pool2d_nhwc_f16_kernel(const uint16_t*
         o[e >> 1] |= (int)((uint32_t)exhip_f2h(r) << ((e & 1) * 16));
     }
     *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 8) = o;
+}
+
+// Global average pooling, src/Excalibur/operation_pooling.cpp:90-100,181-201 with the window = the whole plane. The
+// reference adds a plane's values one after the other; here a plane is cut into interleaved runs that are summed side by
+// side and combined in a fixed order (a launch gives the same bits every time; against the reference the float sum differs
+// in its last bits, inside the 1e-4 the path allows for this layer).
+// NHWC half: a block takes G groups of 8 channels of one image; thread (phase, group) adds pixels phase, phase + P, ...
+// of its group, the P partial sums of a group meet in LDS and are added in phase order.
+__global__ __launch_bounds__(kBlock) void global_avgpool_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
+                                                                         int HW, int cs, int G, int slabs) {
+    __shared__ float part[kBlock][9];  // 8 sums per thread, rows padded against bank conflicts
+    const int n = blockIdx.x / slabs, slab = blockIdx.x % slabs;
+    const int P = kBlock / G;
+    const int g = threadIdx.x % G, phase = threadIdx.x / G;
+    const int group = slab * G + g;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (group * 8 < cs && phase < P) {
+        const uint16_t* src = x + (size_t)n * HW * cs + group * 8;
+        for (int p = phase; p < HW; p += P) {
+            const v8h v = __builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(src + (size_t)p * cs));
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += (float)v[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[threadIdx.x][e] = acc[e];
+    __syncthreads();
+    if (phase == 0 && group * 8 < cs) {
+        float s[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[e] = part[g][e];
+        for (int q = 1; q < P; ++q)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s[e] += part[q * G + g][e];
+        v8h o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (_Float16)(s[e] / (float)HW);
+        *reinterpret_cast<v4i*>(y + (size_t)n * cs + group * 8) = __builtin_bit_cast(v4i, o);
+    }
+}
+
+// NCHW float: one wave per plane; lane l adds elements l, l + 64, ..., then the 64 partial sums are folded
+// 32 + 32, 16 + 16, ... in a fixed tree.
+__global__ __launch_bounds__(kBlock) void global_avgpool_nchw_f32_kernel(const float* __restrict__ x, float* __restrict__ y, int HW,
+                                                                         size_t planes) {
+    const size_t plane = (size_t)blockIdx.x * (kBlock / 64) + threadIdx.x / 64;
+    if (plane >= planes) return;
+    const int lane = threadIdx.x & 63;
+    const float* src = x + plane * HW;
+    float s = 0.f;
+    for (int i = lane; i < HW; i += 64) s += src[i];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) s += __shfl_down(s, d, 64);
+    if (lane == 0) y[plane] = s / (float)HW;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1847,6 +1924,14 @@ extern "C" int exhip_pool2d_nchw_f32(exhip_ctx* ctx, const float* x, float* y, i
         EXHIP_LAUNCH_CHECK();
         return 0;
     }
+    if (type == 1 && oh == 1 && ow == 1 && kh == h && kw == w && pt == 0 && pb == 0 && pl == 0 && pr == 0 && h * w >= 64) {
+        // the whole plane in one window: a wave per plane instead of one thread walking it
+        const size_t planes = (size_t)n * c;
+        hipLaunchKernelGGL(global_avgpool_nchw_f32_kernel, dim3((unsigned)((planes + kBlock / 64 - 1) / (kBlock / 64))), dim3(kBlock), 0,
+                           ctx->stream, x, y, h * w, planes);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     const bool strip_window = kh == kw && (kh == 2 || kh == 3) && sh == 2 && sw == 2 && pl >= 0 && pl <= 1 && pt >= 0 &&
                               w % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     if (strip_window) {
@@ -1915,6 +2000,15 @@ extern "C" int exhip_pool2d_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t
         } else
             hipLaunchKernelGGL((maxpool_nhwc_f16_window_kernel<2, 2>), dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h,
                                w, cs, oh, ow, pt, pl, total);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
+    if (type == 1 && oh == 1 && ow == 1 && kh == h && kw == w && pt == 0 && pb == 0 && pl == 0 && pr == 0 && h * w >= 16) {
+        // the whole plane in one window: parallel partial sums instead of one thread walking the plane
+        int G = 32;
+        while (G > 1 && (cs / 8) % G != 0) G >>= 1;
+        const int slabs = (cs / 8) / G;
+        hipLaunchKernelGGL(global_avgpool_nhwc_f16_kernel, dim3(n * slabs), dim3(kBlock), 0, ctx->stream, x, y, h * w, cs, G, slabs);
         EXHIP_LAUNCH_CHECK();
         return 0;
     }
