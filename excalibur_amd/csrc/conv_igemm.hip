@@ -503,23 +503,30 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
     };
 
     stamp(1);
+    // Per-channel scale and bias of this group's channels go to LDS for the epilogue. The load is issued here, ahead of
+    // the staging requests, and its value is stored behind the wait for the first stage's operands (loads return in
+    // order, so it has arrived by then): a wait here would put a whole memory round trip in front of the first request.
+    float sb_value = 0.f;
     if constexpr (EPI >= 1) {
-        // per-channel scale and bias of this group's channels, fetched now so that the epilogue finds them in LDS
         if (tid < 2 * TM) {
-            const int c = tid < TM ? tid : tid - TM;
-            const int ch = kt * TM + c;
-            float v = 0.f;
-            if (ch < p.K) v = tid < TM ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
-            lds_sb[(tid < TM ? 0 : 128) + c] = v;
-            if constexpr (EPI == 2) {
-                // pooled form: does any channel have a negative scale? (wave 0 holds all 64 scales; slot 64 is spare)
-                if (tid < TM) {
-                    const unsigned long long neg = __ballot(__builtin_bit_cast(int, v) < 0);
-                    if (tid == 0) reinterpret_cast<int*>(lds_sb)[64] = neg != 0ull;
+            const int ch = kt * TM + (tid < TM ? tid : tid - TM);
+            if (ch < p.K) sb_value = tid < TM ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
+        }
+    }
+    auto publish_scale_bias = [&]() {
+        if constexpr (EPI >= 1) {
+            if (tid < 2 * TM) {
+                lds_sb[(tid < TM ? 0 : 128) + (tid < TM ? tid : tid - TM)] = sb_value;
+                if constexpr (EPI == 2) {
+                    // pooled form: does any channel have a negative scale? (wave 0 holds all 64 scales; slot 64 is spare)
+                    if (tid < TM) {
+                        const unsigned long long neg = __ballot(__builtin_bit_cast(int, sb_value) < 0);
+                        if (tid == 0) reinterpret_cast<int*>(lds_sb)[64] = neg != 0ull;
+                    }
                 }
             }
         }
-    }
+    };
 
     if constexpr (!PACKED) {
         // ---- asynchronous pipeline ----
@@ -583,6 +590,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         if (dist == 2) request_w(0);
         stamp(2);
         wait_vmcnt(dist == 2 ? nwl : 0);
+        publish_scale_bias();
         stamp(3);
         __syncthreads();
         stamp(4);
@@ -734,6 +742,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         stamp(2);
         store_act(lds_a0);
         store_w(lds_w0, w_set0);
+        publish_scale_bias();
         stamp(3);
         __syncthreads();
         stamp(4);
