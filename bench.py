@@ -144,6 +144,28 @@ def network_table(iters=10):
     for dt in ("f32", "f16"):
         run("YOLOv5s-shaped, 16x3x640x640", yolo, x, dt, dt)
     run("YOLOv5s-shaped, 16x3x640x640", YoloV5ShapedF32(hw=640, width=32, int8=True, outputs=8), x, "int8", "f32")
+
+    # The detection configuration itself: the topology of the shipped yolov5s_simp (70 convolutions, 13 Concat, three
+    # 255-channel heads), generated line for line, with seeded weights (int8: unit-range feature-map scales, which
+    # decide values, not time).
+    from excalibur_amd import modelfile as mf
+    from excalibur_amd import topologies
+
+    class Seeded:
+        def __init__(self, text, seed):
+            self.lines = [l for l in text.splitlines()[2:] if l.strip()]
+            self._text = text
+            self._model = mf.SeededModel(mf.parse_topology(text), seed, default_fs=0.25)
+
+        def topology(self):
+            return self._text
+
+        def write_model(self, path):
+            mf.write_model(path, self._model.blobs)
+
+    for dt, int8 in (("f32", False), ("f16", False), ("int8", True)):
+        text, _ = topologies.yolov5s_simp(640, int8=int8)
+        run("yolov5s_simp topology (3 heads x 255 channels), 16x3x640x640", Seeded(text, 5), x, dt, "f32" if int8 else dt)
     return rows
 
 
