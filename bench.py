@@ -272,6 +272,8 @@ def main():
     ap.add_argument("--batch", type=int, default=32)
     ap.add_argument("--hw", type=int, default=640)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--in-flight", type=int, default=2,
+                    help="forwards in flight: steps are dealt in turn to this many pipelines, each on a HIP stream of its own (1..8)")
     ap.add_argument("--no-memory-bound", action="store_true", help="skip the memory-bound kernels' block of the line")
     ap.add_argument("--per-layer", action="store_true", help="print per-launch timings to stderr")
     ap.add_argument("--networks", action="store_true",
@@ -310,18 +312,36 @@ def main():
     with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
         model_path = f.name
     net.write_model(model_path)
-    pipe = xp.Pipeline(net.topology(), model_path, 0, "f32", fusion=True)
+    # Steps are dealt in turn to `in_flight` pipelines of the same network, each in a stream slot of its own (its own HIP
+    # stream, activation buffers and input copy): step i + 1 is queued while step i runs, so the second forward's groups
+    # fill the CUs the first leaves idle in the tail of every launch and in the hand-over between launches. Every step is
+    # a whole forward of the batch; all K of them finish inside the timed region.
+    in_flight = max(1, min(args.in_flight, 8))
+    pipes = []
+    for k in range(in_flight):
+        xp.set_stream_slot(k)
+        q = xp.Pipeline(net.topology(), model_path, 0, "f32", fusion=True)
+        q.set_input(x)
+        pipes.append(q)
+    xp.set_stream_slot(0)
     os.unlink(model_path)
-    pipe.set_input(x)
-    for _ in range(args.warmup):
-        pipe.run()
-    pipe.sync()
+    pipe = pipes[0]
+
+    def timed(group, steps, warmup):
+        for i in range(warmup):
+            group[i % len(group)].run()
+        for q in group:
+            q.sync()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            group[i % len(group)].run()
+        for q in group:
+            q.sync()
+        return time.perf_counter() - t0
+
+    one_elapsed = timed(pipes[:1], args.steps, args.warmup)
     assert pipe.fused, "the int8 ResNet-18 topology did not take the fused plan"
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        pipe.run()
-    pipe.sync()
-    elapsed = time.perf_counter() - t0
+    elapsed = timed(pipes, args.steps, args.warmup) if in_flight > 1 else one_elapsed
     ms_per_step = elapsed / args.steps * 1e3
     images_per_s = n * args.steps / elapsed
 
@@ -389,13 +409,15 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"ResNet-18-shaped int8 backbone (7x7 s2 stem, 3x3 s2 maxpool, 4 stages of BasicBlocks "
                                f"64/128/256/512, add+ReLU, per-channel requant), input {n}x3x{hw}x{hw}",
-                   "batch": n, "device": ctx.device_name().strip(),
+                   "batch": n, "device": ctx.device_name().strip(), "forwards_in_flight": in_flight,
+                   "one_in_flight": {"value": round(n * args.steps / one_elapsed, 1), "ms_per_step": round(one_elapsed / args.steps * 1e3, 4)},
                    "int8_tops_whole_step": round(conv_gop / ms_per_step, 1)},
         "roofline": {"bound": "mfma", "kernel": "conv_igemm_kernel (int8, 20 launches per step)",
                      "achieved": round(achieved_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(achieved_tops / PEAK_INT8_TOPS, 4), "traffic": measured_traffic(n, hw),
                      "algorithmic_gop_per_step": round(conv_gop, 1), "avg_launch_ms": round(conv_ms / n_conv, 4),
-                     "timing": f"HIP events around the {n_conv} consecutive launches of a forward of the timed pipeline, mean of {reps} forwards"},
+                     "timing": f"HIP events around the {n_conv} consecutive launches of a forward of the timed pipeline with "
+                               f"nothing else in flight, mean of {reps} forwards"},
     }
     if not args.no_memory_bound:
         rows = bandwidth_table(iters=10, quiet=True, ctx=ctx)
@@ -412,7 +434,8 @@ def main():
         if many:
             line["cpu_baseline_all_cores"] = many
     print(json.dumps(line))
-    pipe.close()
+    for q in pipes:
+        q.close()
     ctx.close()
 
 

@@ -50,6 +50,13 @@ public:
     void time_fused_span(int first_launch);
     float last_span(int* launches);
 
+    // Stream slots (no counterpart in the reference, whose pipelines are synchronous): a pipeline does its device work on
+    // the HIP stream of the slot its constructing thread was in (memory::set_stream_slot; 0 unless set), so pipelines made
+    // in different slots may have forwards in flight at the same time. forward() returns when the work is queued;
+    // reading a result (cpu_data) or synchronize() waits for it.
+    int stream_slot() const;
+    void synchronize();
+
     static std::string version();
 
 private:

@@ -37,6 +37,7 @@ private:
     size_t size_;
     SyncedHead head_ = UNINITIALIZED;
     int device_;
+    int slot_;  // stream slot whose block cache gpu_ptr_ came from
     DISABLE_COPY_AND_ASSIGN(syncedmem);
 };
 

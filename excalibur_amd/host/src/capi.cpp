@@ -12,6 +12,7 @@ using glasssix::memory::tensor;
 
 struct exc_pipeline {
     int dtype = 0, device = 0;
+    int slot = glasssix::memory::stream_slot();  // the pipeline's stream slot: the input tensor lives there too
     std::unique_ptr<pipeline<float>> f32;
     std::unique_ptr<pipeline<unsigned short>> f16;
     std::shared_ptr<tensor<float>> in32;
@@ -109,6 +110,7 @@ extern "C" float exc_pipeline_last_span(exc_pipeline* p, int* launches) {
 }
 
 extern "C" int exc_pipeline_set_input(exc_pipeline* p, const void* input, const int shape[4]) {
+    glasssix::memory::stream_scope scope(p->slot);  // the input's device block belongs to the pipeline's slot
     if (p->dtype == 0) set_input(p->in32, p->device, input, shape);
     else set_input(p->in16, p->device, input, shape);
     return 0;
@@ -165,7 +167,15 @@ extern "C" long exc_pipeline_get_kept(exc_pipeline* p, int back, const char* nam
     return n;
 }
 
-extern "C" int exc_pipeline_sync(exc_pipeline* p) { return exhip_sync(glasssix::memory::device_context(p->device)); }
+extern "C" int exc_pipeline_sync(exc_pipeline* p) { return exhip_sync(glasssix::memory::device_context(p->device, p->slot)); }
+
+extern "C" int exc_set_stream_slot(int slot) {
+    if (slot < 0 || slot >= glasssix::memory::kMaxStreamSlots) return -1;
+    glasssix::memory::set_stream_slot(slot);
+    return 0;
+}
+
+extern "C" int exc_pipeline_stream_slot(exc_pipeline* p) { return p->slot; }
 
 extern "C" int exc_pipeline_forward(exc_pipeline* p, const void* input, const int shape[4]) {
     exc_pipeline_set_input(p, input, shape);

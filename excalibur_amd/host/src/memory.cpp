@@ -3,6 +3,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <tuple>
 
 #include "../include/Primitives/tensor.hpp"
 
@@ -11,9 +12,10 @@ namespace memory {
 
 namespace {
 std::mutex g_mu;
-std::map<int, exhip_ctx*> g_ctx;
-std::map<std::pair<int, size_t>, std::vector<void*>> g_free;  // (device, rounded bytes) -> idle blocks
-std::map<int, size_t> g_idle_bytes;                            // device -> bytes held idle in g_free
+thread_local int t_slot = 0;
+std::map<std::pair<int, int>, exhip_ctx*> g_ctx;                       // (device, slot)
+std::map<std::tuple<int, int, size_t>, std::vector<void*>> g_free;     // (device, slot, rounded bytes) -> idle blocks
+std::map<int, size_t> g_idle_bytes;                                    // device -> bytes held idle in g_free
 // Idle blocks are kept for reuse up to this many bytes per device; beyond it a released block goes back to the driver, so
 // a pipeline fed many different resolutions does not grow without bound.
 constexpr size_t kIdleLimit = (size_t)8 << 30;
@@ -30,38 +32,51 @@ size_t round_block(size_t bytes) {
 }
 }  // namespace
 
-exhip_ctx* device_context(int device) {
+int stream_slot() { return t_slot; }
+
+void set_stream_slot(int slot) {
+    if (slot < 0 || slot >= kMaxStreamSlots) LOG(FATAL) << "stream slot " << slot << " outside 0.." << kMaxStreamSlots - 1;
+    t_slot = slot;
+}
+
+exhip_ctx* device_context(int device) { return device_context(device, t_slot); }
+
+exhip_ctx* device_context(int device, int slot) {
     std::lock_guard<std::mutex> lock(g_mu);
-    auto it = g_ctx.find(device);
+    auto it = g_ctx.find({device, slot});
     if (it != g_ctx.end()) return it->second;
     exhip_ctx* ctx = nullptr;
     int rc = exhip_init(device, &ctx);
     if (rc != 0) LOG(FATAL) << "cannot open HIP device " << device << ": " << exhip_last_error();
-    g_ctx[device] = ctx;
+    g_ctx[{device, slot}] = ctx;
     return ctx;
 }
 
-// Returns every idle block of a device to the driver (exhip_free waits for the device's stream first).
-static void trim_idle(int device, exhip_ctx* ctx) {
-    std::vector<void*> blocks;
+// Returns every idle block of a device to the driver, each through its own slot's context (exhip_free waits for that
+// slot's stream first, behind which the block's last user is queued).
+static void trim_idle(int device) {
+    std::vector<std::pair<int, void*>> blocks;
     {
         std::lock_guard<std::mutex> lock(g_mu);
         for (auto& kv : g_free)
-            if (kv.first.first == device) {
-                blocks.insert(blocks.end(), kv.second.begin(), kv.second.end());
+            if (std::get<0>(kv.first) == device) {
+                for (void* b : kv.second) blocks.push_back({std::get<1>(kv.first), b});
                 kv.second.clear();
             }
         g_idle_bytes[device] = 0;
     }
-    for (void* b : blocks) exhip_free(ctx, b);
+    for (auto& b : blocks) exhip_free(device_context(device, b.first), b.second);
 }
 
-void* device_alloc(int device, size_t bytes) {
-    exhip_ctx* ctx = device_context(device);
+void* device_alloc(int device, size_t bytes) { return device_alloc(device, t_slot, bytes); }
+void device_release(int device, void* ptr, size_t bytes) { device_release(device, t_slot, ptr, bytes); }
+
+void* device_alloc(int device, int slot, size_t bytes) {
+    exhip_ctx* ctx = device_context(device, slot);
     const size_t rb = round_block(bytes);
     {
         std::lock_guard<std::mutex> lock(g_mu);
-        auto& pool = g_free[{device, rb}];
+        auto& pool = g_free[{device, slot, rb}];
         if (!pool.empty()) {
             void* p = pool.back();
             pool.pop_back();
@@ -71,35 +86,36 @@ void* device_alloc(int device, size_t bytes) {
     }
     void* p = nullptr;
     if (exhip_malloc(ctx, rb, &p) != 0) {  // out of device memory: give the idle blocks back and try once more
-        trim_idle(device, ctx);
+        trim_idle(device);
         EXHIP_FATAL(exhip_malloc(ctx, rb, &p));
     }
     return p;
 }
 
-void device_release(int device, void* ptr, size_t bytes) {
+void device_release(int device, int slot, void* ptr, size_t bytes) {
     if (!ptr) return;
     const size_t rb = round_block(bytes);
     {
         std::lock_guard<std::mutex> lock(g_mu);
         if (g_idle_bytes[device] + rb <= kIdleLimit) {
-            g_free[{device, rb}].push_back(ptr);
+            g_free[{device, slot, rb}].push_back(ptr);
             g_idle_bytes[device] += rb;
             return;
         }
     }
-    exhip_free(device_context(device), ptr);  // over the limit: back to the driver (waits for the stream)
+    exhip_free(device_context(device, slot), ptr);  // over the limit: back to the driver (waits for the slot's stream)
 }
 
 template <typename Dtype>
-syncedmem<Dtype>::syncedmem(size_t size, int device) : size_(size), device_(device) {}
+syncedmem<Dtype>::syncedmem(size_t size, int device) : size_(size), device_(device), slot_(stream_slot()) {}
 
 template <typename Dtype>
 syncedmem<Dtype>::~syncedmem() {
     if (cpu_ptr_) std::free(cpu_ptr_);
-    // Kernels using this buffer may still be queued, and that is fine: every device operation of a device (kernels,
-    // copies, fills) goes through that device's one stream, so whatever touches a recycled block is queued behind them.
-    if (gpu_ptr_) device_release(device_, gpu_ptr_, size_ * sizeof(Dtype));
+    // Kernels using this buffer may still be queued, and that is fine: every device operation of a slot (kernels,
+    // copies, fills) goes through that slot's one stream, and the block returns to the cache of the slot it was taken
+    // from, so whatever touches the recycled block is queued behind them.
+    if (gpu_ptr_) device_release(device_, slot_, gpu_ptr_, size_ * sizeof(Dtype));
 }
 
 template <typename Dtype>
@@ -113,7 +129,10 @@ void syncedmem<Dtype>::to_cpu() {
         break;
     case HEAD_AT_GPU:
         if (!cpu_ptr_) cpu_ptr_ = static_cast<Dtype*>(std::aligned_alloc(64, (bytes + 63) / 64 * 64 + 64));
-        EXHIP_FATAL(exhip_memcpy_d2h(device_context(device_), cpu_ptr_, gpu_ptr_, bytes));  // synchronises the stream
+        // synchronises the stream of the slot the block was taken in (a pipeline's outputs: the pipeline's); a reader working
+        // in another slot may have queued the writer there, so that stream is drained as well
+        if (stream_slot() != slot_) EXHIP_FATAL(exhip_sync(device_context(device_)));
+        EXHIP_FATAL(exhip_memcpy_d2h(device_context(device_, slot_), cpu_ptr_, gpu_ptr_, bytes));
         head_ = SYNCED;
         break;
     default: break;
@@ -130,12 +149,16 @@ void syncedmem<Dtype>::to_gpu(bool will_overwrite) {
     exhip_ctx* ctx = device_context(device_);
     switch (head_) {
     case UNINITIALIZED:
+        slot_ = stream_slot();  // the block comes from, is first used in, and returns to the slot of this call
         gpu_ptr_ = static_cast<Dtype*>(device_alloc(device_, bytes));
         if (!will_overwrite) EXHIP_FATAL(exhip_memset(ctx, gpu_ptr_, 0, bytes));
         head_ = HEAD_AT_GPU;
         break;
     case HEAD_AT_CPU:
-        if (!gpu_ptr_) gpu_ptr_ = static_cast<Dtype*>(device_alloc(device_, bytes));
+        if (!gpu_ptr_) {
+            slot_ = stream_slot();
+            gpu_ptr_ = static_cast<Dtype*>(device_alloc(device_, bytes));
+        }
         EXHIP_FATAL(exhip_memcpy_h2d(ctx, gpu_ptr_, cpu_ptr_, bytes));
         head_ = SYNCED;
         break;

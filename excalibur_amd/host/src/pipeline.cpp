@@ -324,6 +324,7 @@ public:
     int span_first_ = -1, span_launches_ = 0;  // time_fused_span / last_span
     void* span_ev_[2] = {nullptr, nullptr};
     int device() const { return device_; }
+    const int slot_ = memory::stream_slot();  // the stream slot the constructing thread was in: all device work goes there
 
 private:
     // ---------------------------------------------------------------- per-layer executor
@@ -796,16 +797,35 @@ pipeline<Dtype>::pipeline(std::string_view param_file, int device) : impl_(new i
 template <typename Dtype>
 pipeline<Dtype>::pipeline(const std::vector<std::string>& hardcode_params, std::string_view model_file, int device)
     : impl_(new impl(hardcode_params, model_file, device)) {}
+// Every entry that touches the device works in the pipeline's own stream slot, whichever slot the caller is in.
 template <typename Dtype>
-pipeline<Dtype>::~pipeline() { delete impl_; }
+pipeline<Dtype>::~pipeline() {
+    memory::stream_scope scope(impl_->slot_);
+    delete impl_;
+}
 template <typename Dtype>
-typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward(const std::shared_ptr<memory::tensor<Dtype>>& t) { return impl_->forward(t); }
+typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward(const std::shared_ptr<memory::tensor<Dtype>>& t) {
+    memory::stream_scope scope(impl_->slot_);
+    return impl_->forward(t);
+}
 template <typename Dtype>
 typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward_cpu(const std::shared_ptr<memory::tensor<Dtype>>& t) { return impl_->forward_cpu(t); }
 template <typename Dtype>
-typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward_gpu(const std::shared_ptr<memory::tensor<Dtype>>& t) { return impl_->forward_gpu(t); }
+typename pipeline<Dtype>::blob_map pipeline<Dtype>::forward_gpu(const std::shared_ptr<memory::tensor<Dtype>>& t) {
+    memory::stream_scope scope(impl_->slot_);
+    return impl_->forward_gpu(t);
+}
 template <typename Dtype>
-std::shared_ptr<memory::tensor<Dtype>> pipeline<Dtype>::get_featmap(std::string_view name) { return impl_->get_featmap(name); }
+std::shared_ptr<memory::tensor<Dtype>> pipeline<Dtype>::get_featmap(std::string_view name) {
+    memory::stream_scope scope(impl_->slot_);
+    return impl_->get_featmap(name);
+}
+template <typename Dtype>
+int pipeline<Dtype>::stream_slot() const { return impl_->slot_; }
+template <typename Dtype>
+void pipeline<Dtype>::synchronize() {
+    if (impl_->device() >= 0) EXHIP_FATAL(exhip_sync(memory::device_context(impl_->device(), impl_->slot_)));
+}
 template <typename Dtype>
 bool pipeline<Dtype>::blob_stored(std::string_view name) const { return impl_->blob_stored(name); }
 template <typename Dtype>
@@ -826,7 +846,7 @@ template <typename Dtype>
 float pipeline<Dtype>::last_span(int* launches) {
     if (launches) *launches = impl_->span_launches_;
     if (!impl_->span_launches_) return 0.f;
-    EXHIP_FATAL(exhip_sync(memory::device_context(impl_->device())));
+    EXHIP_FATAL(exhip_sync(memory::device_context(impl_->device(), impl_->slot_)));
     float ms = 0.f;
     EXHIP_FATAL(exhip_event_elapsed_ms(impl_->span_ev_[0], impl_->span_ev_[1], &ms));
     return ms;

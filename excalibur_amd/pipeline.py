@@ -34,6 +34,8 @@ def lib():
         L.exc_pipeline_set_input.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
         L.exc_pipeline_run.argtypes = [ctypes.c_void_p]
         L.exc_pipeline_sync.argtypes = [ctypes.c_void_p]
+        L.exc_set_stream_slot.argtypes = [ctypes.c_int]
+        L.exc_pipeline_stream_slot.argtypes = [ctypes.c_void_p]
         L.exc_pipeline_forward.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
         L.exc_pipeline_get.restype = ctypes.c_long
         L.exc_pipeline_get.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_long,
@@ -52,6 +54,12 @@ def set_option(name, value):
     rc = lib().exc_set_option(name.encode(), int(value))
     if rc:
         raise ValueError(f"unknown option {name}")
+
+
+def set_stream_slot(slot):
+    """Pipelines this thread creates from now on work on the HIP stream of `slot` (0..7; see include/excalibur_capi.h)."""
+    if lib().exc_set_stream_slot(int(slot)):
+        raise ValueError(f"stream slot {slot} out of range")
 
 
 def registered_operations(dtype="f32"):
@@ -106,6 +114,10 @@ class Pipeline:
         out = np.empty(tuple(shape), self.dtype)
         lib().exc_pipeline_get_kept(self.h, back, name.encode(), out.ctypes.data, out.size, shape)
         return out
+
+    @property
+    def stream_slot(self):
+        return lib().exc_pipeline_stream_slot(self.h)
 
     def sync(self):
         rc = lib().exc_pipeline_sync(self.h)

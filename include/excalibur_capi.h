@@ -39,6 +39,12 @@ int exc_pipeline_run(exc_pipeline* p);
 int exc_pipeline_run_keeping(exc_pipeline* p);
 long exc_pipeline_get_kept(exc_pipeline* p, int back, const char* name, void* out, long capacity, int shape[4]);
 int exc_pipeline_sync(exc_pipeline* p);
+/* Stream slots (memory::set_stream_slot, pipeline::stream_slot; no counterpart in the reference): the calling thread works
+ * in slot 0 unless it sets another (0..7); a pipeline created afterwards does all its device work on that slot's own HIP
+ * stream, so exc_pipeline_run of pipelines made in different slots overlap on the GPU. exc_pipeline_sync and
+ * exc_pipeline_get wait for the pipeline's own stream. Returns -1 for a slot outside the range. */
+int exc_set_stream_slot(int slot);
+int exc_pipeline_stream_slot(exc_pipeline* p);
 /* set_input + run + sync */
 int exc_pipeline_forward(exc_pipeline* p, const void* input, const int shape[4]);
 /* Copies output blob or feature map `name` of the last forward to `out` if it fits in `capacity` elements;
