@@ -314,6 +314,12 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         int iy = fast_div(pix, p.magic_iw), ix = pix - iy * IW;
 #pragma unroll
         for (int i = 0; i < NAV; ++i) {
+            // loads past the tile's last slot are never issued (the tile of a layer rarely needs all NAV): their two
+            // dozen instructions are skipped as a whole, which a wave-uniform test per load does pay for
+            if (i > 0 && i * THREADS * 16 >= p.act_need_b) {
+                a_goff[i] = oob;
+                continue;
+            }
             const int gy = iy0 + iy * step, gx = ix0 + ix * step;
             const bool in_img = (pix < npix) & (part < SL - 1) & ((unsigned)gy < (unsigned)H) & ((unsigned)gx < (unsigned)W);
             const int off = (gy * W + gx) * cs_b + part * 16;
@@ -336,6 +342,11 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         int iy = fast_div(tid, p.magic_iw), ix = tid - iy * IW;
 #pragma unroll
         for (int i = 0; i < NPP; ++i) {
+            if (i > 0 && THREADS * i >= npix) {  // past the tile for every thread: skipped as a whole
+                a_loff[i] = -1;
+                a_goff[i] = oob;
+                continue;
+            }
             const int gy = iy0 + iy, gx = ix0 + ix;
             const bool in_tile = tid + THREADS * i < npix;
             const bool in_img = in_tile & ((unsigned)gy < (unsigned)H) & ((unsigned)gx < (unsigned)W);
