@@ -348,6 +348,11 @@ def main():
     elapsed = timed(pipes, args.steps, args.warmup) if in_flight > 1 else one_elapsed
     ms_per_step = elapsed / args.steps * 1e3
     images_per_s = n * args.steps / elapsed
+    # every pipeline was fed the same batch: after the timed loops their results must be the same bytes
+    first_out = pipes[0].get(net.output)
+    assert np.isfinite(first_out).all() and np.count_nonzero(first_out) > first_out.size // 8
+    for q in pipes[1:]:
+        assert np.array_equal(q.get(net.output), first_out), "pipelines in different stream slots disagree"
 
     # One plain copy-like kernel of known size (ReLU over 64 Mi floats: 256 MiB read + 256 MiB written), outside
     # the timed region: it calibrates the FETCH_SIZE / WRITE_SIZE counters when this command runs under rocprofv3 --pmc.
