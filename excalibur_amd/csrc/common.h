@@ -56,6 +56,7 @@ struct exhip_options {
     int debug_plan = 0;      // one line per planned layer on stderr
     int dw_band_rows = 0;    // row-band height of the depthwise strip kernels
     int force_splits = 0;    // groups per tile of the convolution's split reduction (1 = never split)
+    int share_gpu = 0;       // launches of several streams overlap: the planner then counts groups per CU, not rounds of one launch
 };
 extern exhip_options g_exhip_options;
 

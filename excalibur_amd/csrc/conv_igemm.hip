@@ -1312,6 +1312,9 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
     const bool packed = cb < 32;
     const int force_variant = g_exhip_options.force_variant, force_chunk = g_exhip_options.force_chunk;
     const int force_rs = g_exhip_options.force_rs, force_abufs = g_exhip_options.force_abufs;
+    // With launches of other streams on the GPU a launch's own rounds stop mattering (whatever it leaves idle is taken):
+    // one more group per CU is then worth the exposed tile loads whenever it fits.
+    const bool crowd = g_exhip_options.share_gpu != 0 && force_abufs == 0;
     for (int vc = 0; vc < 2 * kNumVariants; ++vc) {
         const int variant = vc >> 1, chunk_opt = (vc & 1) ? 32 : 64;
         if (force_variant >= 0 && !pool && !packed && variant != force_variant) continue;  // not the first-layer forms
@@ -1418,7 +1421,7 @@ int make_plan(const exhip_conv_desc* d, int dt, Plan* out, const PoolSpec* pool 
                         const int w_bufs_before = p.w_bufs;
                         p.act_bufs = 1;
                         if (p.lds_bytes() > room && p.w_bufs == 3) p.w_bufs = 2;
-                        if (force_abufs == 2 || p.lds_bytes() > room || (force_abufs != 1 && r3 * 115 >= r2 * 100)) {
+                        if (force_abufs == 2 || p.lds_bytes() > room || (force_abufs != 1 && !crowd && r3 * 115 >= r2 * 100)) {
                             p.act_bufs = 2;
                             p.w_bufs = w_bufs_before;
                         }
@@ -1566,7 +1569,7 @@ void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3
     if (g_one <= g_now) return;
     const long long wgs = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
     const long long r_now = (wgs + g_now * kCUs - 1) / (g_now * kCUs), r_one = (wgs + g_one * kCUs - 1) / (g_one * kCUs);
-    if (force_abufs == 1 || r_one * 115 < r_now * 100) {
+    if (force_abufs == 1 || (g_exhip_options.share_gpu != 0 && force_abufs == 0) || r_one * 115 < r_now * 100) {
         pl = one;
         pl.two_per_cu = pl.threads == 512;
         if (g_exhip_options.debug_plan)

@@ -48,7 +48,9 @@ const char* exhip_last_error(void);
  * "force_variant" / "force_chunk" / "force_rs" / "force_abufs" pin the convolution planner's tile variant, channel chunk
  * bytes, filter rows per stage and activation tile buffers, "debug_plan" prints one line per planned layer,
  * "dw_band_rows" pins the depthwise strip kernels' band height, "force_splits" the groups per tile of the convolution's
- * split reduction (1 = never split). 0 (-1 for force_variant) restores the planner's choice.
+ * split reduction (1 = never split). 0 (-1 for force_variant) restores the planner's choice. "share_gpu" = 1 tells the
+ * planner that launches of several streams overlap on the GPU (it then prefers one more group per CU over fewer rounds
+ * of a launch: measured 3 % faster with two forwards in flight, 2 % slower alone; off unless set).
  * Process-wide; packed weights depend on the first three, so set them before packing. */
 int exhip_set_option(const char* name, int value);
 int exhip_device_name(exhip_ctx* ctx, char* buf, size_t len);
