@@ -55,3 +55,26 @@ def test_argument_errors_need_no_gpu():
     assert hip.Ctx.pool_out_hw(20, 20, 3, 3, 2, 2, 1, 1, 1, 1, 1) == (10, 10)
     assert hip.Ctx.pool_out_hw(14, 14, 3, 3, 2, 2, 0, 0, 0, 0, 0) == (7, 7)
     assert hip.Ctx.pool_out_hw(14, 14, 3, 3, 2, 2, 0, 0, 0, 0, 1) == (6, 6)
+
+
+def test_stream_slots_and_options_need_no_gpu():
+    """The slot of a thread is thread-local state of the host library, and unknown option names are refused."""
+    import threading
+
+    from excalibur_amd import pipeline
+    L = pipeline.lib()
+    assert L.exc_set_stream_slot(3) == 0
+    assert L.exc_set_stream_slot(8) == -1 and L.exc_set_stream_slot(-1) == -1
+    seen = []
+
+    def other():
+        seen.append(L.exc_set_stream_slot(5))  # another thread's slot does not move this one's
+
+    t = threading.Thread(target=other)
+    t.start()
+    t.join()
+    assert seen == [0]
+    assert L.exc_set_stream_slot(0) == 0
+    with pytest.raises(ValueError):
+        pipeline.set_option("no_such_option", 1)
+    pipeline.set_option("share_gpu", 0)
