@@ -1,0 +1,19 @@
+// The 3x3 stride-1 int8 convolution with the fused epilogue as a lean, optionally persistent kernel
+// (conv_i8_lean.hip). conv_igemm.hip plans the layer and hands the launch over when the geometry fits.
+#pragma once
+#include "common.h"
+
+struct exhip_lean_geom {
+    int n, h, w, c_bytes, k, oh, ow;     // input / output shape; c_bytes: bytes per input pixel (a multiple of 64)
+    int pt, pl;                          // top / left zero padding
+    int ph, pw, ih, iw;                  // output patch of a group and its staged input tile, in pixels
+    int tiles_x, tiles_y, ktiles;        // patches per image and 64-channel slabs
+    int act, post_relu;                  // ReLU before / after the shortcut sum
+    float fs_out;                        // scale of the int8 output
+};
+
+// Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then
+// runs the general kernel), another code on failure. Weights are the general kernel's packing for 64-channel slabs and
+// 64-byte channel chunks.
+int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
+                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw);

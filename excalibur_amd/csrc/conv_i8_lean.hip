@@ -1,0 +1,599 @@
+// 3x3 stride-1 int8 convolution with the fused epilogue (dequantize, ReLU, float32 shortcut, float32 / int8 NHWC and
+// float32 NCHW results): the layers that carry most of a ResNet-shaped int8 stack. Same implicit GEMM as
+// conv_igemm.hip -- rows = 64 output channels, columns = a patch of up to 256 output pixels, v_mfma_i32_32x32x32_i8,
+// every wave a 64 x 64 accumulator tile, operands from global memory straight into LDS -- but with everything the
+// general kernel decides at run time fixed at compile time, so that a wave issues little besides its MFMAs:
+//
+//  * a group is persistent: it walks several patches of one 64-channel slab. Lane constants (fragment offsets, the
+//    gather offsets of the staging loads relative to a patch's origin, output offsets) are computed once; per patch only
+//    the border tests remain, and those only for patches that touch the image's border.
+//  * the weight slices and the activation tiles of a group's whole run form one pipeline: what the next patch needs is
+//    requested while the current one computes, so a patch boundary costs no refill.
+//  * every wave issues the same, fixed number of staging loads per stage (a request without data gets a zero-length
+//    buffer view), which makes every s_waitcnt an immediate.
+//  * with 64 input channels the slab's whole filter (36 KiB) stays in LDS for the life of the group and a patch needs two
+//    barriers in all.
+//  * the epilogue works from registers: a lane holds 16 consecutive channels of a pixel per accumulator tile, and one
+//    v_permlane32_swap per register pair turns the two half-waves' 64-byte runs into 32-byte pieces that two lanes
+//    read or write side by side, so float32 tensors move as whole 32-byte sectors without an exchange through LDS.
+//
+// Arithmetic and rounding are the general kernel's (and so the reference's, src/Excalibur/operation_convolution.cpp:373-408,
+// src/Primitives/simd_types.cpp:140-152): results are bit for bit the same.
+#include <mutex>
+
+#include "conv_i8_lean.h"
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kNAL = 7;                   // staging loads per thread for one activation tile (7 x 4 KiB)
+constexpr int kActStride = 27 * 1024;     // LDS bytes of an activation tile buffer; the 28th KiB a request writes is a spare one
+constexpr int kPixB = 80;                 // a staged pixel: a 64-byte channel chunk and 16 bytes that keep fragment reads off the same banks
+constexpr int kWSlice = 3 * 2 * 2 * 1024; // weights of one filter row of one chunk: 3 taps x 2 k-steps x 2 channel tiles x 1 KiB
+constexpr int kSbB = 512;                 // scale and bias of the slab's 64 channels
+constexpr int kSpareB = 1024;
+constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer: out-of-range loads return 0, stores are dropped
+constexpr int kOob = 0x7FFFFF00;              // a byte offset past any tensor
+constexpr unsigned kOobElem = 0x3FFFFF00u;    // an element offset whose byte offsets (x1, x4, + 255) lie past any accepted tensor
+
+enum { E_RES = 1, E_F = 2, E_Q = 4, E_NCHW = 8, E_ACT = 16, E_POST = 32, E_QNN = 64 };
+
+struct LeanParams {
+    const char* x;
+    const char* wp;
+    const float* scale;
+    const float* bias;
+    const float* residual;
+    int8_t* y_q;
+    float* y_f;
+    float* y_nchw;
+    int H, W, K, OH, OW, PT, PL;
+    int C_b, n_chunks;
+    int PH, PW, IH, IW;
+    int tiles_x, tiles_xy, ktiles, n_ptiles;
+    unsigned img_bytes, out_elems;
+    unsigned magic_iw, magic_pw, magic_tx, magic_txy;
+    int adv_iy, adv_ix;  // (256 / 5) / IW, (256 / 5) % IW: how a thread's tile pixel advances from one staging load to the next
+    float fs_out;
+    int flags;
+};
+
+__device__ __forceinline__ int fast_div(int n, unsigned magic) { return (int)__umulhi((unsigned)n, magic); }
+__device__ __forceinline__ v4i lds_read16(const char* p) { return *reinterpret_cast<const v4i*>(p); }
+
+// One 16-byte element per lane from a bounds-checked buffer view straight into LDS: lane l's data lands at
+// lds_base + 16 * l (lds_base wave-uniform, in M0). Completion is counted by vmcnt like any other load.
+__device__ __forceinline__ void async_load16(__amdgpu_buffer_rsrc_t rsrc, int voff, int soff, unsigned lds_base) {
+    __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voff),
+                     "s"(rsrc), "s"(soff)
+                     : "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() { __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+// v_permlane32_swap: the upper half-wave of `a` changes places with the lower half-wave of `b`.
+__device__ __forceinline__ void half_swap(int& a, int& b) {
+    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)a, (unsigned)b, false, false);
+    a = (int)r[0];
+    b = (int)r[1];
+}
+__device__ __forceinline__ void half_swap4(v4i& a, v4i& b) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        int x = a[e], y = b[e];
+        half_swap(x, y);
+        a[e] = x;
+        b[e] = y;
+    }
+}
+
+// WRES: the slab's whole filter is resident (one 64-byte chunk); otherwise weight slices rotate through NWB buffers and
+// activation tiles through NAB. EPI >= 0: the epilogue's switches as compile-time constants; EPI < 0: read from p.flags.
+template <bool WRES, int NAB, int NWB, int EPI>
+__global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) void conv3x3_i8_lean_kernel(const LeanParams p) {
+    constexpr int NWS = WRES ? 3 : NWB;
+    constexpr int A0 = NWS * kWSlice;
+    constexpr int SB0 = A0 + NAB * kActStride;
+    constexpr int SPARE0 = SB0 + kSbB;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    float* const lds_sb = reinterpret_cast<float*>(smem + SB0);
+
+    const int flags = EPI >= 0 ? EPI : p.flags;
+    const bool has_res = flags & E_RES, has_f = flags & E_F, has_q = flags & E_Q, has_nchw = flags & E_NCHW;
+    const bool act_relu = flags & E_ACT, post_relu = flags & E_POST, q_nonneg = flags & E_QNN;
+    const bool q_only = q_nonneg && has_q && !has_res && !has_f && !has_nchw;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int hh = lane >> 5;
+
+    // ---- which patches this group walks: groups of one XCD (ids are dealt round-robin to the 8 XCDs) take neighbouring
+    // patches, so that halos and the slabs of one patch meet in that XCD's L2 ----
+    const int G = gridDim.x;
+    int lb = blockIdx.x;
+    if ((G & 7) == 0) lb = (lb & 7) * (G >> 3) + (lb >> 3);
+    const int kt = __builtin_amdgcn_readfirstlane(lb % p.ktiles);
+    const int pj = __builtin_amdgcn_readfirstlane(lb / p.ktiles);
+    const int GP = G / p.ktiles;
+    const int my_tiles = __builtin_amdgcn_readfirstlane((p.n_ptiles - pj + GP - 1) / GP);
+
+    // ---- lane constants ----
+    // staging: slot v = tid + 256 * i of a tile is 16 bytes of pixel v / 5, part v % 5 (part 4 is the padding)
+    int a_rel[kNAL], a_yx[kNAL], a_off[kNAL];
+    {
+        const int IW = p.IW, npix = p.IH * IW, W = p.W, cb = p.C_b;
+        int pix = fast_div(tid, 0x33333334u), part = tid - pix * 5;
+        int iy = fast_div(pix, p.magic_iw), ix = pix - iy * IW;
+#pragma unroll
+        for (int i = 0; i < kNAL; ++i) {
+            const bool ok = (pix < npix) & (part < 4);
+            a_rel[i] = ok ? (iy * W + ix) * cb + part * 16 : kOob;
+            a_yx[i] = ok ? (iy | (ix << 16)) : -1;
+            part += 1;
+            const int carry = part >= 5 ? 1 : 0;
+            part -= carry ? 5 : 0;
+            pix += 51 + carry;
+            ix += p.adv_ix + carry;
+            iy += p.adv_iy;
+            const int wrap = ix >= IW ? 1 : 0;
+            ix -= wrap ? IW : 0;
+            iy += wrap;
+        }
+    }
+    // the lane's two pixels (one per 32-pixel column block of its wave): fragment offset in a tile, position in the patch
+    int boff[2], o_rel[2], o_y[2], o_x[2];
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn) {
+        int pp = (wave * 2 + nn) * 32 + (lane & 31);
+        const bool ok = pp < p.PH * p.PW;
+        pp = ok ? pp : 0;
+        const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
+        boff[nn] = py * (p.IW * kPixB) + px * kPixB + hh * 16;
+        o_rel[nn] = (py * p.OW + px) * p.K;
+        o_y[nn] = ok ? py : 0x4000;  // a row past any image
+        o_x[nn] = px;
+    }
+    const int row_b = p.IW * kPixB;
+    const int img_px = p.OH * p.OW;
+
+    v16i acc[2][2];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[m][nn][e] = 0;
+    };
+
+    // ---- patch bookkeeping (all wave-uniform) ----
+    auto decode = [&](int t, int& n, int& oy0, int& ox0) {
+        n = fast_div(t, p.magic_txy);
+        const int r = t - n * p.tiles_xy;
+        const int ty = fast_div(r, p.magic_tx), tx = r - ty * p.tiles_x;
+        oy0 = ty * p.PH;
+        ox0 = tx * p.PW;
+    };
+    // gather offsets of a patch's staging loads; returns what goes into the buffer view's base instead
+    auto set_offsets = [&](int oy0, int ox0) -> int {
+        const int iy0 = oy0 - p.PT, ix0 = ox0 - p.PL;
+        const int tile_base = (iy0 * p.W + ix0) * p.C_b;
+        const bool interior = iy0 >= 0 && ix0 >= 0 && iy0 + p.IH <= p.H && ix0 + p.IW <= p.W;
+        if (interior) {
+#pragma unroll
+            for (int i = 0; i < kNAL; ++i) a_off[i] = a_rel[i];
+            return tile_base;
+        }
+#pragma unroll
+        for (int i = 0; i < kNAL; ++i) {
+            const int gy = iy0 + (a_yx[i] & 0xFFFF), gx = ix0 + (int)((unsigned)a_yx[i] >> 16);
+            const bool in = ((unsigned)gy < (unsigned)p.H) & ((unsigned)gx < (unsigned)p.W);
+            a_off[i] = in ? a_rel[i] + tile_base : kOob;
+        }
+        return 0;
+    };
+
+    // ---- staging requests ----
+    const unsigned wave_slot = (unsigned)wave * 1024u;
+    const int w_voff = tid * 16;
+    const char* const wkt = p.wp + (size_t)kt * p.n_chunks * (3 * kWSlice);  // this slab's slices, in (chunk, filter row) order
+    const int w_run_b = p.n_chunks * 3 * kWSlice;
+    int w_off = 0;                                  // next slice to request
+    int w_left = my_tiles * p.n_chunks * 3;         // slices of the whole run not requested yet
+    auto request_w = [&](unsigned dst) {
+        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(wkt + w_off), 0, w_left > 0 ? kWSlice : 0, kRsrcWord3);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) async_load16(wr, w_voff, i * 4096, dst + wave_slot + i * 4096);
+        --w_left;
+        w_off += kWSlice;
+        if (w_off == w_run_b) w_off = 0;
+    };
+    auto request_a = [&](const char* img, int base, int cc, bool valid, unsigned dst) {
+        const int off = base + cc * 64;
+        const __amdgpu_buffer_rsrc_t xr =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(img + off), 0, valid ? (int)p.img_bytes - off : 0, kRsrcWord3);
+#pragma unroll
+        for (int i = 0; i < kNAL; ++i) {
+            unsigned d = dst + wave_slot + i * 4096;
+            if (i == kNAL - 1) d = wave == 3 ? lds0 + SPARE0 : d;  // the KiB past the buffer
+            async_load16(xr, a_off[i], 0, d);
+        }
+    };
+
+    // ---- MFMAs of filter rows: k-steps in (tap, channel half) order, fragments fetched one step ahead ----
+    v4i af[2][2], bf[2][2];
+    auto compute = [&](int buf) {
+#pragma unroll
+        for (int m = 0; m < 2; ++m)
+#pragma unroll
+            for (int nn = 0; nn < 2; ++nn) acc[m][nn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][m], bf[buf][nn], acc[m][nn], 0, 0, 0);
+    };
+    auto fetch = [&](int buf, const char* wrow, const char* a0, const char* a1, int s) {
+        af[buf][0] = lds_read16(wrow + s * 2048);
+        af[buf][1] = lds_read16(wrow + s * 2048 + 1024);
+        bf[buf][0] = lds_read16(a0 + (s >> 1) * kPixB + (s & 1) * 32);
+        bf[buf][1] = lds_read16(a1 + (s >> 1) * kPixB + (s & 1) * 32);
+    };
+    // NR filter rows whose weights lie kWSlice apart from wrow on and whose tile rows lie row_b apart from a0 / a1 on;
+    // `requests` runs once, behind the first k-step's MFMAs
+    auto mfma_rows = [&](auto nr_t, const char* wrow, const char* a0, const char* a1, auto&& requests) {
+        constexpr int NR = decltype(nr_t)::value;
+        fetch(0, wrow, a0, a1, 0);
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+#pragma unroll
+            for (int s = 0; s < 6; ++s) {
+                const int k = r * 6 + s;
+                if (s + 1 < 6) fetch((k + 1) & 1, wrow + r * kWSlice, a0 + r * row_b, a1 + r * row_b, s + 1);
+                else if (r + 1 < NR) fetch((k + 1) & 1, wrow + (r + 1) * kWSlice, a0 + (r + 1) * row_b, a1 + (r + 1) * row_b, 0);
+                // keep this order: the next k-step's fragment reads go out before this k-step's MFMAs
+                __builtin_amdgcn_sched_barrier(0);
+                compute(k & 1);
+                __builtin_amdgcn_sched_barrier(0);
+                if (k == 0) requests();
+            }
+        }
+    };
+    constexpr std::integral_constant<int, 1> one_row{};
+    constexpr std::integral_constant<int, 3> three_rows{};
+
+    // ---- epilogue of one patch, from registers ----
+    const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(p.y_q, 0, (int)p.out_elems, kRsrcWord3);
+    const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_f, 0, (int)(p.out_elems * 4u), kRsrcWord3);
+    const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.residual), 0, (int)(p.out_elems * 4u), kRsrcWord3);
+    const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc(p.y_nchw, 0, (int)(p.out_elems * 4u), kRsrcWord3);
+    // 32-byte pieces of a pixel's 32 channels in the order the register pairs hold them after the half-wave swap
+    auto piece = [](int j) { return j == 0 ? 0 : j == 1 ? 64 : j == 2 ? 32 : 96; };
+    auto epilogue = [&](int n, int oy0, int ox0) {
+        const bool full = oy0 + p.PH <= p.OH && ox0 + p.PW <= p.OW;
+        const unsigned obase = ((unsigned)n * (unsigned)img_px + (unsigned)(oy0 * p.OW + ox0)) * (unsigned)p.K + (unsigned)(kt * 64);
+        unsigned eoff[2], noff[2];
+#pragma unroll
+        for (int nn = 0; nn < 2; ++nn) {
+            const bool valid = full ? o_y[nn] < 0x4000 : ((oy0 + o_y[nn] < p.OH) & (ox0 + o_x[nn] < p.OW));
+            eoff[nn] = valid ? obase + (unsigned)o_rel[nn] : kOobElem;
+            if (has_nchw) {
+                const unsigned e = ((unsigned)n * (unsigned)p.K + (unsigned)(kt * 64 + hh * 16)) * (unsigned)img_px +
+                                   (unsigned)((oy0 + o_y[nn]) * p.OW + ox0 + o_x[nn]);
+                noff[nn] = valid ? e * 4u : (unsigned)kOob;
+            }
+        }
+        // the shortcut's values first, so that all of them are in flight while the first are used
+        v4i rs[2][2][4];
+        if (has_res) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        rs[m][nn][j] = __builtin_amdgcn_raw_buffer_load_b128(rr, (int)(eoff[nn] * 4u + hh * 16 + m * 128 + piece(j)), 0, 0);
+        }
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            v4f s4[4], b4[4];
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                s4[e4] = *reinterpret_cast<const v4f*>(lds_sb + m * 32 + hh * 16 + e4 * 4);
+                b4[e4] = *reinterpret_cast<const v4f*>(lds_sb + 64 + m * 32 + hh * 16 + e4 * 4);
+            }
+#pragma unroll
+            for (int nn = 0; nn < 2; ++nn) {
+                v4i q4;
+                if (q_only) {
+                    // int8 output only, ReLU last: q = trunc(max(v, 0) * fs + 0.5) capped at 127. With fs > 0 the maximum
+                    // commutes with the product, and max(t, 0) + 0.5 == max(t + 0.5, 0.5) in float arithmetic (the sum is
+                    // monotone in t), so one median does ReLU and saturation.
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        int b[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float v = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e4][e], b4[e4][e]);
+                            b[e] = (int)__builtin_amdgcn_fmed3f(v * p.fs_out + 0.5f, 0.5f, 127.f);
+                        }
+                        q4[e4] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                    }
+                    __builtin_amdgcn_raw_buffer_store_b128(q4, rq, (int)(eoff[nn] + hh * 16 + m * 32), 0, 0);
+                    continue;
+                }
+                v4i r4[4];
+                if (has_res) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) r4[j] = rs[m][nn][j];
+                    half_swap4(r4[0], r4[1]);
+                    half_swap4(r4[2], r4[3]);
+                }
+                v4i o4[4];
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    v4f v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e4][e], b4[e4][e]);
+                    if (act_relu) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
+                    }
+                    if (has_res) {
+                        const v4f rv = __builtin_bit_cast(v4f, r4[e4]);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += rv[e];
+                    }
+                    if (post_relu) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
+                    }
+                    o4[e4] = __builtin_bit_cast(v4i, v);
+                    if (has_nchw) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            __builtin_amdgcn_raw_buffer_store_b32(o4[e4][e], rn, (int)noff[nn], (m * 32 + e4 * 4 + e) * img_px * 4, 0);
+                    }
+                    if (has_q) {
+                        // float32_to_int8(v * fs): product rounded first, then +-0.5, saturate, truncate. After a final
+                        // ReLU every product is >= 0: the sign select and the lower clamp fall away.
+                        int b[4];
+                        if (q_nonneg) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) b[e] = (int)__builtin_fminf(v[e] * p.fs_out + 0.5f, 127.f);
+                            q4[e4] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                const float t = v[e] * p.fs_out;
+                                b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
+                            }
+                            q4[e4] = (b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24);
+                        }
+                    }
+                }
+                if (has_f) {
+                    half_swap4(o4[0], o4[1]);
+                    half_swap4(o4[2], o4[3]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        __builtin_amdgcn_raw_buffer_store_b128(o4[j], rf, (int)(eoff[nn] * 4u + hh * 16 + m * 128 + piece(j)), 0, 0);
+                }
+                if (has_q) __builtin_amdgcn_raw_buffer_store_b128(q4, rq, (int)(eoff[nn] + hh * 16 + m * 32), 0, 0);
+            }
+        }
+    };
+    // stores an epilogue issues (they stand behind the next tile's request in the wave's memory queue)
+    constexpr int kEpiStores = EPI < 0 ? 64 : ((EPI & E_F) ? 16 : 0) + ((EPI & E_Q) ? 4 : 0) + ((EPI & E_NCHW) ? 64 : 0);
+    constexpr int kWaitBehindEpi = EPI < 0 ? 0 : (kEpiStores < 60 ? kEpiStores : 60);
+
+    // ---- the run ----
+    int n, oy0, ox0;                 // the patch being computed
+    int pt = pj;
+    decode(pt, n, oy0, ox0);
+    const char* img = p.x + (size_t)n * p.img_bytes;   // image and view base of the next tile request
+    int base = set_offsets(oy0, ox0);
+    if (tid < 128) {
+        const int ch = kt * 64 + (tid & 63);
+        lds_sb[tid] = tid < 64 ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
+    }
+    clear_acc();
+
+    if constexpr (WRES) {
+        request_a(img, base, 0, true, lds0 + A0);
+        for (int r = 0; r < 3; ++r) request_w(lds0 + r * kWSlice);
+        wait_vmcnt<0>();
+        __syncthreads();
+        const char* const wrow = smem + lane * 16;
+        const char* const a0 = smem + A0 + boff[0];
+        const char* const a1 = smem + A0 + boff[1];
+        for (int done = 0;;) {
+            mfma_rows(three_rows, wrow, a0, a1, []() {});
+            __syncthreads();  // every wave has read the tile
+            const bool has_next = ++done < my_tiles;
+            int nn_, ny, nx;
+            if (has_next) {
+                pt += GP;
+                decode(pt, nn_, ny, nx);
+                img = p.x + (size_t)nn_ * p.img_bytes;
+                base = set_offsets(ny, nx);
+                request_a(img, base, 0, true, lds0 + A0);
+            }
+            epilogue(n, oy0, ox0);
+            if (!has_next) break;
+            clear_acc();
+            n = nn_; oy0 = ny; ox0 = nx;
+            wait_vmcnt<kWaitBehindEpi>();
+            __syncthreads();
+        }
+    } else {
+        // waits at the end of a stage's MFMAs: the next stage's slice must have landed; what was requested behind it stays
+        // in flight (the order of a stage's requests: its slice first, then the next chunk's tile)
+        constexpr int kWait0 = (NWB == 3 ? 3 : 0) + (NAB == 2 ? kNAL : 0);
+        constexpr int kWait1 = NWB == 3 ? 3 + (NAB == 2 ? kNAL : 0) : 0;
+        constexpr int kWait2 = NWB == 3 ? 3 : 0;
+        request_a(img, base, 0, true, lds0 + A0);
+        request_w(lds0);
+        if constexpr (NWB == 3) request_w(lds0 + kWSlice);
+        wait_vmcnt<(NWB == 3 ? 3 : 0)>();
+        __syncthreads();
+        int abuf = 0;   // tile buffer of the current chunk
+        int wbuf = 0;   // NWB == 2: slice buffer of the current stage (with three buffers filter row r is in buffer r)
+        int nn_ = n, ny = oy0, nx = ox0;
+        for (int done = 0;;) {
+            const bool has_next = done + 1 < my_tiles;
+            for (int cc = 0; cc < p.n_chunks; ++cc) {
+                const bool last_cc = cc + 1 == p.n_chunks;
+                // what the next chunk's tile request asks for: the next chunk of this patch, or the next patch's first
+                auto request_next_a = [&](unsigned dst) {
+                    if (last_cc) {
+                        if (has_next) {
+                            pt += GP;
+                            decode(pt, nn_, ny, nx);
+                            img = p.x + (size_t)nn_ * p.img_bytes;
+                            base = set_offsets(ny, nx);
+                        }
+                        request_a(img, base, 0, has_next, dst);
+                    } else {
+                        request_a(img, base, cc + 1, true, dst);
+                    }
+                };
+                const char* const ab = smem + A0 + (NAB == 2 ? abuf * kActStride : 0);
+                const char* const a0 = ab + boff[0];
+                const char* const a1 = ab + boff[1];
+                const unsigned a_other = lds0 + A0 + (NAB == 2 ? (1 - abuf) * kActStride : 0);
+                if constexpr (NWB == 3) {
+                    mfma_rows(one_row, smem + lane * 16, a0, a1, [&]() {
+                        request_w(lds0 + 2 * kWSlice);
+                        if constexpr (NAB == 2) request_next_a(a_other);
+                    });
+                    wait_vmcnt<kWait0>();
+                    __syncthreads();
+                    mfma_rows(one_row, smem + kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0); });
+                    wait_vmcnt<kWait1>();
+                    __syncthreads();
+                    mfma_rows(one_row, smem + 2 * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b, [&]() { request_w(lds0 + kWSlice); });
+                    wait_vmcnt<kWait2>();
+                    __syncthreads();
+                } else {
+                    mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0, a1, [&]() {
+                        request_w(lds0 + (1 - wbuf) * kWSlice);
+                        if constexpr (NAB == 2) request_next_a(a_other);
+                    });
+                    wait_vmcnt<kWait0>();
+                    __syncthreads();
+                    wbuf = 1 - wbuf;
+                    mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
+                    wait_vmcnt<kWait1>();
+                    __syncthreads();
+                    wbuf = 1 - wbuf;
+                    mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b,
+                              [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
+                    wait_vmcnt<kWait2>();
+                    __syncthreads();
+                    wbuf = 1 - wbuf;
+                }
+                if constexpr (NAB == 2) {
+                    abuf = 1 - abuf;
+                } else {
+                    // a single tile buffer: refilled once every wave has left the chunk; between chunks the load is waited
+                    // for in the open (the CU's other groups run meanwhile), behind a patch it lands under the epilogue
+                    request_next_a(lds0 + A0);
+                    if (!last_cc) {
+                        wait_vmcnt<0>();
+                        __syncthreads();
+                    }
+                }
+            }
+            epilogue(n, oy0, ox0);
+            if (!has_next) break;
+            ++done;
+            clear_acc();
+            n = nn_; oy0 = ny; ox0 = nx;
+            if constexpr (NAB == 1) {
+                wait_vmcnt<kWaitBehindEpi>();
+                __syncthreads();
+            }
+        }
+    }
+    wait_vmcnt<0>();  // no staging load may land after the group's LDS has been given to another
+}
+
+std::mutex g_attr_mutex;
+
+template <bool WRES, int NAB, int NWB, int EPI>
+int launch(exhip_ctx* ctx, const LeanParams& p, int grid) {
+    constexpr int lds = ((WRES ? 3 : NWB) * kWSlice) + NAB * kActStride + kSbB + kSpareB;
+    static unsigned long long attr_set = 0;
+    auto kernel = conv3x3_i8_lean_kernel<WRES, NAB, NWB, EPI>;
+    {
+        std::lock_guard<std::mutex> lock(g_attr_mutex);
+        const unsigned long long bit = 1ull << (ctx->device & 63);
+        if (!(attr_set & bit)) {
+            EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            attr_set |= bit;
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, ctx->stream, p);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+template <bool WRES, int NAB, int NWB>
+int launch_epi(exhip_ctx* ctx, const LeanParams& p, int grid) {
+    switch (p.flags) {
+    case E_Q | E_ACT | E_QNN: return launch<WRES, NAB, NWB, (E_Q | E_ACT | E_QNN)>(ctx, p, grid);
+    case E_RES | E_F | E_Q | E_POST | E_QNN: return launch<WRES, NAB, NWB, (E_RES | E_F | E_Q | E_POST | E_QNN)>(ctx, p, grid);
+    default: return launch<WRES, NAB, NWB, -1>(ctx, p, grid);
+    }
+}
+
+}  // namespace
+
+int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
+                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw) {
+    const int mode = g_exhip_options.lean;
+    if (mode == 0) return EXHIP_ERR_UNSUPPORTED;
+    const long long n_ptiles = (long long)g.n * g.tiles_y * g.tiles_x;
+    const long long out_elems = (long long)g.n * g.oh * g.ow * g.k;
+    if (g.c_bytes % 64 != 0 || g.k % 64 != 0 || g.ph * g.pw > 256 || g.ih * g.iw * kPixB + 16 > kActStride || n_ptiles >= 65536 ||
+        g.h >= 0x4000 || g.w >= 0x4000 || g.ih >= 0x4000 || g.iw >= 0x4000 || g.ph >= 0x4000 || out_elems * 4 >= 0xFFFFF000ll ||
+        out_elems >= (long long)kOobElem || (long long)g.h * g.w * g.c_bytes >= 0x7FFFFF00ll || g.act > 1 || g.ktiles != g.k / 64)
+        return EXHIP_ERR_UNSUPPORTED;
+    LeanParams p = {};
+    p.x = (const char*)x; p.wp = (const char*)wp; p.scale = scale; p.bias = bias; p.residual = residual;
+    p.y_q = y_q; p.y_f = y_f; p.y_nchw = y_nchw;
+    p.H = g.h; p.W = g.w; p.K = g.k; p.OH = g.oh; p.OW = g.ow; p.PT = g.pt; p.PL = g.pl;
+    p.C_b = g.c_bytes; p.n_chunks = g.c_bytes / 64;
+    p.PH = g.ph; p.PW = g.pw; p.IH = g.ih; p.IW = g.iw;
+    p.tiles_x = g.tiles_x; p.tiles_xy = g.tiles_x * g.tiles_y; p.ktiles = g.ktiles; p.n_ptiles = (int)n_ptiles;
+    p.img_bytes = (unsigned)((size_t)g.h * g.w * g.c_bytes);
+    p.out_elems = (unsigned)out_elems;
+    auto magic = [](int d) { return (unsigned)(((1ull << 32) + d - 1) / d); };
+    p.magic_iw = magic(g.iw); p.magic_pw = magic(g.pw); p.magic_tx = magic(g.tiles_x); p.magic_txy = magic(p.tiles_xy);
+    p.adv_iy = 51 / g.iw; p.adv_ix = 51 % g.iw;
+    p.fs_out = g.fs_out;
+    const bool q_nonneg = g.fs_out > 0.f && (g.post_relu || (g.act == 1 && !residual));
+    p.flags = (residual ? E_RES : 0) | (y_f ? E_F : 0) | (y_q ? E_Q : 0) | (y_nchw ? E_NCHW : 0) | (g.act == 1 ? E_ACT : 0) |
+              (g.post_relu ? E_POST : 0) | (q_nonneg ? E_QNN : 0);
+
+    // groups: as many as stay resident (persistent), or one per patch and slab (mode 2)
+    const bool wres = p.n_chunks == 1;
+    const int cfg = wres ? 0 : g_exhip_options.lean_cfg;  // 0: one tile buffer, two slice buffers; 1: two and two; 2: one and three
+    const int per_cu = wres ? 2 : (cfg == 0 ? 3 : 2);
+    const long long total = n_ptiles * g.ktiles;
+    long long G = total;
+    if (mode != 2 && total > per_cu * 256ll) {
+        const long long unit = 8ll * g.ktiles;  // the XCD mapping and the slab of a group need whole units
+        G = per_cu * 256ll / unit * unit;
+        if (G <= 0) G = g.ktiles;
+    }
+    if (g_exhip_options.lean_groups > 0 && G > (long long)g_exhip_options.lean_groups * g.ktiles)
+        G = (long long)g_exhip_options.lean_groups * g.ktiles;
+    if (g_exhip_options.debug_plan)
+        fprintf(stderr, "  lean: %s cfg %d, %lld groups for %lld tiles, flags %d\n", wres ? "resident filter" : "streamed filter", cfg, G, total,
+                p.flags);
+    if (wres) return launch_epi<true, 1, 2>(ctx, p, (int)G);
+    if (cfg == 1) return launch_epi<false, 2, 2>(ctx, p, (int)G);
+    if (cfg == 2) return launch_epi<false, 1, 3>(ctx, p, (int)G);
+    return launch_epi<false, 1, 2>(ctx, p, (int)G);
+}

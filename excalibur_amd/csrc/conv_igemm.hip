@@ -26,6 +26,7 @@
 #include <vector>
 
 #include "common.h"
+#include "conv_i8_lean.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
@@ -1665,6 +1666,18 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = !p.acc_nchw && !d->post_op && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
                            out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
+        if (fused && !pl.packed && p.splits == 1 && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
+            p.cstride_b % 64 == 0) {
+            // the lean kernel takes these layers with the same packed weights; EXHIP_ERR_UNSUPPORTED leaves them to this one
+            exhip_lean_geom g = {};
+            g.n = d->n; g.h = d->h; g.w = d->w; g.c_bytes = p.cstride_b; g.k = d->k; g.oh = pl.OH; g.ow = pl.OW;
+            g.pt = d->pt; g.pl = d->pl; g.ph = pl.PH; g.pw = pl.PW; g.ih = pl.IH; g.iw = pl.IW;
+            g.tiles_x = pl.tiles_x; g.tiles_y = pl.tiles_y; g.ktiles = pl.ktiles;
+            g.act = d->act; g.post_relu = d->post_relu; g.fs_out = d->fs_out;
+            rc = exhip_conv3x3_i8_lean(ctx, g, reinterpret_cast<const int8_t*>(p.x), p.wp, p.scale, p.bias, reinterpret_cast<const float*>(p.residual),
+                                       reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc), reinterpret_cast<float*>(p.y_nchw));
+            if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
+        }
         if (fused) {
             p.epi_mode = 1;
             p.epi_f = p.residual || p.y_nhwc;

@@ -30,6 +30,9 @@ extern "C" int exhip_set_option(const char* name, int value) {
     else if (!strcmp(name, "dw_band_rows")) o.dw_band_rows = value;
     else if (!strcmp(name, "force_splits")) o.force_splits = value;
     else if (!strcmp(name, "share_gpu")) o.share_gpu = value;
+    else if (!strcmp(name, "lean")) o.lean = value;
+    else if (!strcmp(name, "lean_cfg")) o.lean_cfg = value;
+    else if (!strcmp(name, "lean_groups")) o.lean_groups = value;
     else {
         exhip_set_error("exhip_set_option: unknown option %s", name);
         return EXHIP_ERR_ARG;
