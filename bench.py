@@ -282,6 +282,8 @@ def main():
                     help="set the planner option share_gpu: one more group per CU wherever a single activation tile buffer allows "
                          "it (3 %% faster with two forwards in flight, 2 %% slower with one; off by default)")
     ap.add_argument("--no-memory-bound", action="store_true", help="skip the memory-bound kernels' block of the line")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="set a library option (exhip_set_option) before the network is planned; may be repeated")
     ap.add_argument("--per-layer", action="store_true", help="print per-launch timings to stderr")
     ap.add_argument("--networks", action="store_true",
                     help="time the other configurations' whole topologies (MobileNet- and YOLOv5s-shaped, f32 / f16 / int8) "
@@ -326,6 +328,9 @@ def main():
     in_flight = max(1, min(args.in_flight, 8))
     if args.shared_gpu_plans:
         xp.set_option("share_gpu", 1)
+    for item in args.option:
+        name, _, value = item.partition("=")
+        xp.set_option(name, int(value))
     pipes = []
     for k in range(in_flight):
         xp.set_stream_slot(k)

@@ -59,6 +59,8 @@ struct exhip_options {
     int share_gpu = 0;       // launches of several streams overlap: the planner then counts groups per CU, not rounds of one launch
     int lean = 1;            // 3x3 stride-1 int8 layers with the fused epilogue: 0 general kernel, 1 lean persistent kernel, 2 lean, one group per patch
     int lean_cfg = 0;        // its staging buffers for layers of more than 64 input channels: 0 one tile + two slices, 1 two + two, 2 one + three
+    int lean_wres = 1;       // 64 input channels: keep the slab's whole filter in LDS (0: stream it like the deeper layers)
+    int lean_stagger = 0;    // experiment: start delay per hardware wave slot, in units of 64 cycles
     int lean_groups = 0;     // at most this many groups per 64-channel slab (tests: a few groups that walk many patches each)
 };
 extern exhip_options g_exhip_options;

@@ -40,6 +40,12 @@ constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer: out-of-range loads 
 constexpr int kOob = 0x7FFFFF00;              // a byte offset past any tensor
 constexpr unsigned kOobElem = 0x3FFFFF00u;    // an element offset whose byte offsets (x1, x4, + 255) lie past any accepted tensor
 
+#ifndef EXHIP_STAMPS
+#define EXHIP_STAMPS 0
+#endif
+constexpr bool kStamps = EXHIP_STAMPS != 0;
+long long* g_lean_dbg = nullptr;
+
 enum { E_RES = 1, E_F = 2, E_Q = 4, E_NCHW = 8, E_ACT = 16, E_POST = 32, E_QNN = 64 };
 
 struct LeanParams {
@@ -60,6 +66,8 @@ struct LeanParams {
     int adv_iy, adv_ix;  // (256 / 5) / IW, (256 / 5) % IW: how a thread's tile pixel advances from one staging load to the next
     float fs_out;
     int flags;
+    int stagger;     // persistent launches: a group whose waves sit in hardware wave slot s starts s * stagger * 64 cycles late
+    long long* dbg;  // phase timestamps (builds with -DEXHIP_STAMPS=1 only)
 };
 
 __device__ __forceinline__ int fast_div(int n, unsigned magic) { return (int)__umulhi((unsigned)n, magic); }
@@ -69,8 +77,16 @@ __device__ __forceinline__ v4i lds_read16(const char* p) { return *reinterpret_c
 // lds_base + 16 * l (lds_base wave-uniform, in M0). Completion is counted by vmcnt like any other load.
 __device__ __forceinline__ void async_load16(__amdgpu_buffer_rsrc_t rsrc, int voff, int soff, unsigned lds_base) {
     __asm__ volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voff),
-                     "s"(rsrc), "s"(soff)
+                     "s"(rsrc), "s"(__builtin_amdgcn_readfirstlane(soff))
                      : "m0");
+}
+// A buffer view whose base and range are pinned to scalar registers (the staging loads are inline assembly: the compiler
+// cannot wrap them in the loop it would put around a view it keeps in vector registers).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_view(const char* base, int range) {
+    const unsigned long long a = (unsigned long long)(uintptr_t)base;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)a), hi = __builtin_amdgcn_readfirstlane((unsigned)(a >> 32));
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<char*>((uintptr_t)(((unsigned long long)hi << 32) | lo)), 0,
+                                             __builtin_amdgcn_readfirstlane(range), kRsrcWord3);
 }
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() { __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -110,6 +126,21 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int hh = lane >> 5;
+    long long t_mfma = 0, t_wait = 0, t_bar = 0, t_epi = 0, t_gap = 0, t_mark = 0;
+    auto now = [&]() -> long long { return kStamps && p.dbg ? (long long)clock64() : 0ll; };
+    auto put = [&](int k, long long v) {
+        if constexpr (kStamps)
+            if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * 4 + wave) * 16 + k] = v;
+    };
+    put(0, now());
+    if (p.stagger > 0) {
+        // Groups that share a CU start together and would reach their MFMA runs, waits and epilogues together, the matrix
+        // pipes idle in between. The hardware wave slot (HW_ID bits 3:0) counts the waves a SIMD already holds: delaying a
+        // group by its slot spreads the phases of a CU's groups over a patch's period.
+        const int slot = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | ((4 - 1) << 11));  // HW_REG_HW_ID, offset 0, width 4
+        for (int i = 0; i < slot * p.stagger; ++i) __builtin_amdgcn_s_sleep(1);
+    }
+    if constexpr (kStamps) put(10, (long long)wall_clock64());
 
     // ---- which patches this group walks: groups of one XCD (ids are dealt round-robin to the 8 XCDs) take neighbouring
     // patches, so that halos and the slabs of one patch meet in that XCD's L2 ----
@@ -205,7 +236,7 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     int w_off = 0;                                  // next slice to request
     int w_left = my_tiles * p.n_chunks * 3;         // slices of the whole run not requested yet
     auto request_w = [&](unsigned dst) {
-        const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(wkt + w_off), 0, w_left > 0 ? kWSlice : 0, kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t wr = uniform_view(wkt + w_off, w_left > 0 ? kWSlice : 0);
 #pragma unroll
         for (int i = 0; i < 3; ++i) async_load16(wr, w_voff, i * 4096, dst + wave_slot + i * 4096);
         --w_left;
@@ -214,8 +245,7 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     };
     auto request_a = [&](const char* img, int base, int cc, bool valid, unsigned dst) {
         const int off = base + cc * 64;
-        const __amdgpu_buffer_rsrc_t xr =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(img + off), 0, valid ? (int)p.img_bytes - off : 0, kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t xr = uniform_view(img + off, valid ? (int)p.img_bytes - off : 0);
 #pragma unroll
         for (int i = 0; i < kNAL; ++i) {
             unsigned d = dst + wave_slot + i * 4096;
@@ -401,14 +431,19 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     if constexpr (WRES) {
         request_a(img, base, 0, true, lds0 + A0);
         for (int r = 0; r < 3; ++r) request_w(lds0 + r * kWSlice);
+        put(1, now());
         wait_vmcnt<0>();
         __syncthreads();
+        put(2, now());
         const char* const wrow = smem + lane * 16;
         const char* const a0 = smem + A0 + boff[0];
         const char* const a1 = smem + A0 + boff[1];
         for (int done = 0;;) {
+            t_mark = now();
             mfma_rows(three_rows, wrow, a0, a1, []() {});
+            { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
             __syncthreads();  // every wave has read the tile
+            { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
             const bool has_next = ++done < my_tiles;
             int nn_, ny, nx;
             if (has_next) {
@@ -418,12 +453,16 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                 base = set_offsets(ny, nx);
                 request_a(img, base, 0, true, lds0 + A0);
             }
+            { const long long t = now(); t_gap += t - t_mark; t_mark = t; }
             epilogue(n, oy0, ox0);
+            { const long long t = now(); t_epi += t - t_mark; t_mark = t; }
             if (!has_next) break;
             clear_acc();
             n = nn_; oy0 = ny; ox0 = nx;
             wait_vmcnt<kWaitBehindEpi>();
+            { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
             __syncthreads();
+            { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
         }
     } else {
         // waits at the end of a stage's MFMAs: the next stage's slice must have landed; what was requested behind it stays
@@ -434,8 +473,11 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
         request_a(img, base, 0, true, lds0 + A0);
         request_w(lds0);
         if constexpr (NWB == 3) request_w(lds0 + kWSlice);
+        put(1, now());
         wait_vmcnt<(NWB == 3 ? 3 : 0)>();
         __syncthreads();
+        put(2, now());
+        t_mark = now();
         int abuf = 0;   // tile buffer of the current chunk
         int wbuf = 0;   // NWB == 2: slice buffer of the current stage (with three buffers filter row r is in buffer r)
         int nn_ = n, ny = oy0, nx = ox0;
@@ -466,30 +508,48 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                         request_w(lds0 + 2 * kWSlice);
                         if constexpr (NAB == 2) request_next_a(a_other);
                     });
+                    { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait0>();
+                    { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
+                    { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                     mfma_rows(one_row, smem + kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0); });
+                    { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait1>();
+                    { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
+                    { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                     mfma_rows(one_row, smem + 2 * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b, [&]() { request_w(lds0 + kWSlice); });
+                    { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait2>();
+                    { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
+                    { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                 } else {
                     mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0, a1, [&]() {
                         request_w(lds0 + (1 - wbuf) * kWSlice);
                         if constexpr (NAB == 2) request_next_a(a_other);
                     });
+                    { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait0>();
+                    { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
+                    { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                     wbuf = 1 - wbuf;
                     mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
+                    { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait1>();
+                    { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
+                    { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                     wbuf = 1 - wbuf;
                     mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b,
                               [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
+                    { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait2>();
+                    { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
+                    { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                     wbuf = 1 - wbuf;
                 }
                 if constexpr (NAB == 2) {
@@ -502,9 +562,11 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                         wait_vmcnt<0>();
                         __syncthreads();
                     }
+                    { const long long t = now(); t_gap += t - t_mark; t_mark = t; }
                 }
             }
             epilogue(n, oy0, ox0);
+            { const long long t = now(); t_epi += t - t_mark; t_mark = t; }
             if (!has_next) break;
             ++done;
             clear_acc();
@@ -512,10 +574,444 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
             if constexpr (NAB == 1) {
                 wait_vmcnt<kWaitBehindEpi>();
                 __syncthreads();
+                { const long long t = now(); t_gap += t - t_mark; t_mark = t; }
             }
         }
     }
     wait_vmcnt<0>();  // no staging load may land after the group's LDS has been given to another
+    put(3, t_mfma); put(4, t_wait); put(5, t_bar); put(6, t_epi); put(7, t_gap); put(8, now()); put(9, my_tiles);
+    if constexpr (kStamps) put(11, (long long)wall_clock64());
+}
+
+// ---- the same convolution with the work of a group split between two kinds of waves ----
+// A group of eight waves owns a CU: waves 0-3 stage operands and run the MFMAs of a patch (a 64 x 64 accumulator tile each),
+// then leave the accumulators in LDS; waves 4-7 take them from there one patch later and do everything that is not an
+// MFMA -- dequantization, shortcut, ReLU, requantization, all traffic to and from the result tensors -- while the first
+// four are already at the next patch. On every SIMD an MFMA wave and an epilogue wave run side by side, so the matrix
+// pipe does not wait for vector work, and the shortcut's loads (requested a patch ahead) and the result stores have a
+// memory queue of their own: the staging waits of the MFMA waves never stand behind them. The two kinds meet only at
+// the stage barriers both execute in equal number. With one group per CU the whole LDS is the group's: three weight
+// slice buffers (or the resident filter), two activation tile buffers, 64 KiB for the accumulators.
+template <bool WRES, int EPI>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv3x3_i8_ws_kernel(const LeanParams p) {
+    constexpr int A0 = 3 * kWSlice;
+    constexpr int H0 = A0 + 2 * kActStride;          // accumulators on their way to the epilogue waves: 4 x 16 KiB
+    constexpr int SB0 = H0 + 4 * 16384;
+    constexpr int SPARE0 = SB0 + kSbB;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+    float* const lds_sb = reinterpret_cast<float*>(smem + SB0);
+
+    const int flags = EPI >= 0 ? EPI : p.flags;
+    const bool has_res = flags & E_RES, has_f = flags & E_F, has_q = flags & E_Q, has_nchw = flags & E_NCHW;
+    const bool act_relu = flags & E_ACT, post_relu = flags & E_POST, q_nonneg = flags & E_QNN;
+    const bool q_only = q_nonneg && has_q && !has_res && !has_f && !has_nchw;
+
+    const int wave8 = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const bool mma_role = wave8 < 4;
+    const int wave = wave8 & 3, lane = threadIdx.x & 63, tid = threadIdx.x & 255, hh = lane >> 5;
+
+    // waits for this wave's LDS operations, then for the group: what was written before is visible behind it. No memory
+    // fence: that would also wait for every global access in flight, which is what the epilogue waves must not do.
+    auto barrier = [&]() { __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    const int G = gridDim.x;
+    int lb = blockIdx.x;
+    if ((G & 7) == 0) lb = (lb & 7) * (G >> 3) + (lb >> 3);
+    const int kt = __builtin_amdgcn_readfirstlane(lb % p.ktiles);
+    const int pj = __builtin_amdgcn_readfirstlane(lb / p.ktiles);
+    const int GP = G / p.ktiles;
+    const int my_tiles = __builtin_amdgcn_readfirstlane((p.n_ptiles - pj + GP - 1) / GP);
+    const int nst = WRES ? 2 : p.n_chunks * 3;   // barriers per patch
+    const int row_b = p.IW * kPixB;
+    const int img_px = p.OH * p.OW;
+
+    auto decode = [&](int t, int& n, int& oy0, int& ox0) {
+        n = fast_div(t, p.magic_txy);
+        const int r = t - n * p.tiles_xy;
+        const int ty = fast_div(r, p.magic_tx), tx = r - ty * p.tiles_x;
+        oy0 = ty * p.PH;
+        ox0 = tx * p.PW;
+    };
+    // the lane's two pixels (one per 32-pixel column block of its wave)
+    int boff[2], o_rel[2], o_y[2], o_x[2];
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn) {
+        int pp = (wave * 2 + nn) * 32 + (lane & 31);
+        const bool ok = pp < p.PH * p.PW;
+        pp = ok ? pp : 0;
+        const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
+        boff[nn] = py * row_b + px * kPixB + hh * 16;
+        o_rel[nn] = (py * p.OW + px) * p.K;
+        o_y[nn] = ok ? py : 0x4000;
+        o_x[nn] = px;
+    }
+    char* const hand = smem + H0 + wave * 16384 + lane * 16;   // this wave pair's accumulators: 16 x 1 KiB
+
+    if (mma_role) {
+        // ================= staging and MFMAs =================
+        int a_rel[kNAL], a_yx[kNAL], a_off[kNAL];
+        {
+            const int IW = p.IW, npix = p.IH * IW, W = p.W, cb = p.C_b;
+            int pix = fast_div(tid, 0x33333334u), part = tid - pix * 5;
+            int iy = fast_div(pix, p.magic_iw), ix = pix - iy * IW;
+#pragma unroll
+            for (int i = 0; i < kNAL; ++i) {
+                const bool ok = (pix < npix) & (part < 4);
+                a_rel[i] = ok ? (iy * W + ix) * cb + part * 16 : kOob;
+                a_yx[i] = ok ? (iy | (ix << 16)) : -1;
+                part += 1;
+                const int carry = part >= 5 ? 1 : 0;
+                part -= carry ? 5 : 0;
+                pix += 51 + carry;
+                ix += p.adv_ix + carry;
+                iy += p.adv_iy;
+                const int wrap = ix >= IW ? 1 : 0;
+                ix -= wrap ? IW : 0;
+                iy += wrap;
+            }
+        }
+        auto set_offsets = [&](int oy0, int ox0) -> int {
+            const int iy0 = oy0 - p.PT, ix0 = ox0 - p.PL;
+            const int tile_base = (iy0 * p.W + ix0) * p.C_b;
+            const bool interior = iy0 >= 0 && ix0 >= 0 && iy0 + p.IH <= p.H && ix0 + p.IW <= p.W;
+            if (interior) {
+#pragma unroll
+                for (int i = 0; i < kNAL; ++i) a_off[i] = a_rel[i];
+                return tile_base;
+            }
+#pragma unroll
+            for (int i = 0; i < kNAL; ++i) {
+                const int gy = iy0 + (a_yx[i] & 0xFFFF), gx = ix0 + (int)((unsigned)a_yx[i] >> 16);
+                const bool in = ((unsigned)gy < (unsigned)p.H) & ((unsigned)gx < (unsigned)p.W);
+                a_off[i] = in ? a_rel[i] + tile_base : kOob;
+            }
+            return 0;
+        };
+        const unsigned wave_slot = (unsigned)wave * 1024u;
+        const int w_voff = tid * 16;
+        const char* const wkt = p.wp + (size_t)kt * p.n_chunks * (3 * kWSlice);
+        const int w_run_b = p.n_chunks * 3 * kWSlice;
+        int w_off = 0;
+        int w_left = my_tiles * p.n_chunks * 3;
+        auto request_w = [&](unsigned dst) {
+            const __amdgpu_buffer_rsrc_t wr = uniform_view(wkt + w_off, w_left > 0 ? kWSlice : 0);
+#pragma unroll
+            for (int i = 0; i < 3; ++i) async_load16(wr, w_voff, i * 4096, dst + wave_slot + i * 4096);
+            --w_left;
+            w_off += kWSlice;
+            if (w_off == w_run_b) w_off = 0;
+        };
+        auto request_a = [&](const char* img, int base, int cc, bool valid, unsigned dst) {
+            const int off = base + cc * 64;
+            const __amdgpu_buffer_rsrc_t xr =
+                uniform_view(img + off, valid ? (int)p.img_bytes - off : 0);
+#pragma unroll
+            for (int i = 0; i < kNAL; ++i) {
+                unsigned d = dst + wave_slot + i * 4096;
+                if (i == kNAL - 1) d = wave == 3 ? lds0 + SPARE0 : d;
+                async_load16(xr, a_off[i], 0, d);
+            }
+        };
+        v16i acc[2][2];
+        auto clear_acc = [&]() {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[m][nn][e] = 0;
+        };
+        auto hand_over = [&]() {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4)
+                        *reinterpret_cast<v4i*>(hand + ((m * 2 + nn) * 4 + e4) * 1024) =
+                            v4i{acc[m][nn][e4 * 4], acc[m][nn][e4 * 4 + 1], acc[m][nn][e4 * 4 + 2], acc[m][nn][e4 * 4 + 3]};
+        };
+        v4i af[2][2], bf[2][2];
+        auto compute = [&](int buf) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int nn = 0; nn < 2; ++nn) acc[m][nn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][m], bf[buf][nn], acc[m][nn], 0, 0, 0);
+        };
+        auto fetch = [&](int buf, const char* wrow, const char* a0, const char* a1, int s) {
+            af[buf][0] = lds_read16(wrow + s * 2048);
+            af[buf][1] = lds_read16(wrow + s * 2048 + 1024);
+            bf[buf][0] = lds_read16(a0 + (s >> 1) * kPixB + (s & 1) * 32);
+            bf[buf][1] = lds_read16(a1 + (s >> 1) * kPixB + (s & 1) * 32);
+        };
+        auto mfma_rows = [&](auto nr_t, const char* wrow, const char* a0, const char* a1, auto&& requests) {
+            constexpr int NR = decltype(nr_t)::value;
+            fetch(0, wrow, a0, a1, 0);
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+#pragma unroll
+                for (int s = 0; s < 6; ++s) {
+                    const int k = r * 6 + s;
+                    if (s + 1 < 6) fetch((k + 1) & 1, wrow + r * kWSlice, a0 + r * row_b, a1 + r * row_b, s + 1);
+                    else if (r + 1 < NR) fetch((k + 1) & 1, wrow + (r + 1) * kWSlice, a0 + (r + 1) * row_b, a1 + (r + 1) * row_b, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    compute(k & 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (k == 0) requests();
+                }
+            }
+        };
+        constexpr std::integral_constant<int, 1> one_row{};
+        constexpr std::integral_constant<int, 2> two_rows{};
+
+        int n, oy0, ox0, pt = pj;
+        decode(pt, n, oy0, ox0);
+        const char* img = p.x + (size_t)n * p.img_bytes;
+        int base = set_offsets(oy0, ox0);
+        if (tid < 128) {
+            const int ch = kt * 64 + (tid & 63);
+            lds_sb[tid] = tid < 64 ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
+        }
+        clear_acc();
+        int abuf = 0;
+        // the next tile request: the next chunk of this patch, or the first chunk of the group's next patch
+        auto request_next_a = [&](int cc, bool last_cc, bool has_next, unsigned dst) {
+            if (last_cc) {
+                if (has_next) {
+                    pt += GP;
+                    decode(pt, n, oy0, ox0);
+                    img = p.x + (size_t)n * p.img_bytes;
+                    base = set_offsets(oy0, ox0);
+                }
+                request_a(img, base, 0, has_next, dst);
+            } else {
+                request_a(img, base, cc + 1, true, dst);
+            }
+        };
+        if constexpr (WRES) {
+            request_a(img, base, 0, true, lds0 + A0);
+            for (int r = 0; r < 3; ++r) request_w(lds0 + r * kWSlice);
+            wait_vmcnt<0>();
+            barrier();
+            for (int done = 0; done < my_tiles; ++done) {
+                const bool has_next = done + 1 < my_tiles;
+                const char* const ab = smem + A0 + abuf * kActStride;
+                const unsigned a_other = lds0 + A0 + (1 - abuf) * kActStride;
+                mfma_rows(one_row, smem + lane * 16, ab + boff[0], ab + boff[1], [&]() { request_next_a(0, true, has_next, a_other); });
+                barrier();   // the epilogue waves have taken the previous patch's accumulators
+                mfma_rows(two_rows, smem + kWSlice + lane * 16, ab + row_b + boff[0], ab + row_b + boff[1], []() {});
+                hand_over();
+                wait_vmcnt<0>();
+                barrier();
+                clear_acc();
+                abuf = 1 - abuf;
+            }
+        } else {
+            request_a(img, base, 0, true, lds0 + A0);
+            request_w(lds0);
+            request_w(lds0 + kWSlice);
+            wait_vmcnt<3>();
+            barrier();
+            for (int done = 0; done < my_tiles; ++done) {
+                const bool has_next = done + 1 < my_tiles;
+                for (int cc = 0; cc < p.n_chunks; ++cc) {
+                    const bool last_cc = cc + 1 == p.n_chunks;
+                    const char* const ab = smem + A0 + abuf * kActStride;
+                    const char* const a0 = ab + boff[0];
+                    const char* const a1 = ab + boff[1];
+                    const unsigned a_other = lds0 + A0 + (1 - abuf) * kActStride;
+                    mfma_rows(one_row, smem + lane * 16, a0, a1, [&]() {
+                        request_w(lds0 + 2 * kWSlice);
+                        request_next_a(cc, last_cc, has_next, a_other);
+                    });
+                    wait_vmcnt<3 + kNAL>();
+                    barrier();
+                    mfma_rows(one_row, smem + kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0); });
+                    wait_vmcnt<3 + kNAL>();
+                    barrier();
+                    mfma_rows(one_row, smem + 2 * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b, [&]() { request_w(lds0 + kWSlice); });
+                    if (last_cc) hand_over();
+                    wait_vmcnt<3>();
+                    barrier();
+                    abuf = 1 - abuf;
+                }
+                clear_acc();
+            }
+        }
+        wait_vmcnt<0>();  // no staging load may land after the group's LDS has been given to another
+    } else {
+        // ================= epilogues, one patch behind =================
+        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(p.y_q, 0, (int)p.out_elems, kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rf = __builtin_amdgcn_make_buffer_rsrc(p.y_f, 0, (int)(p.out_elems * 4u), kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.residual), 0, (int)(p.out_elems * 4u), kRsrcWord3);
+        const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc(p.y_nchw, 0, (int)(p.out_elems * 4u), kRsrcWord3);
+        auto piece = [](int j) { return j == 0 ? 0 : j == 1 ? 64 : j == 2 ? 32 : 96; };
+        // element offsets of the lane's two pixels in a patch's result tensors
+        auto offsets = [&](int n, int oy0, int ox0, unsigned (&eoff)[2], unsigned (&noff)[2]) {
+            const bool full = oy0 + p.PH <= p.OH && ox0 + p.PW <= p.OW;
+            const unsigned obase = ((unsigned)n * (unsigned)img_px + (unsigned)(oy0 * p.OW + ox0)) * (unsigned)p.K + (unsigned)(kt * 64);
+#pragma unroll
+            for (int nn = 0; nn < 2; ++nn) {
+                const bool valid = full ? o_y[nn] < 0x4000 : ((oy0 + o_y[nn] < p.OH) & (ox0 + o_x[nn] < p.OW));
+                eoff[nn] = valid ? obase + (unsigned)o_rel[nn] : kOobElem;
+                noff[nn] = 0;
+                if (has_nchw) {
+                    const unsigned e = ((unsigned)n * (unsigned)p.K + (unsigned)(kt * 64 + hh * 16)) * (unsigned)img_px +
+                                       (unsigned)((oy0 + o_y[nn]) * p.OW + ox0 + o_x[nn]);
+                    noff[nn] = valid ? e * 4u : (unsigned)kOob;
+                }
+            }
+        };
+        v4i rs[2][2][4];   // the shortcut's values of the patch whose epilogue comes next
+        auto request_shortcut = [&](const unsigned (&eoff)[2]) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int nn = 0; nn < 2; ++nn)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        rs[m][nn][j] = __builtin_amdgcn_raw_buffer_load_b128(rr, (int)(eoff[nn] * 4u + hh * 16 + m * 128 + piece(j)), 0, 0);
+        };
+        // The accumulators taken over. With the resident filter all four tiles are read at once (the MFMA waves write the
+        // next patch's before this patch's last blocks run); otherwise each block reads its own when its turn comes.
+        v4i accq[WRES ? 4 : 1][4];
+        auto take_over = [&](int b) {
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) accq[WRES ? b : 0][e4] = *reinterpret_cast<const v4i*>(hand + (b * 4 + e4) * 1024);
+        };
+        // one accumulator tile (32 channels x 32 pixels of the wave's 64 x 64)
+        auto block = [&](auto m_t, auto nn_t, const unsigned (&eoff)[2], const unsigned (&noff)[2]) {
+            constexpr int m = decltype(m_t)::value, nn = decltype(nn_t)::value;
+            if constexpr (!WRES) take_over(m * 2 + nn);
+            v4f s4[4], b4[4];
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                s4[e4] = *reinterpret_cast<const v4f*>(lds_sb + m * 32 + hh * 16 + e4 * 4);
+                b4[e4] = *reinterpret_cast<const v4f*>(lds_sb + 64 + m * 32 + hh * 16 + e4 * 4);
+            }
+            v4i q4;
+            if (q_only) {
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    int b[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float v = __builtin_fmaf((float)accq[WRES ? m * 2 + nn : 0][e4][e], s4[e4][e], b4[e4][e]);
+                        b[e] = (int)__builtin_amdgcn_fmed3f(v * p.fs_out + 0.5f, 0.5f, 127.f);
+                    }
+                    q4[e4] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                }
+                __builtin_amdgcn_raw_buffer_store_b128(q4, rq, (int)(eoff[nn] + hh * 16 + m * 32), 0, 0);
+                return;
+            }
+            v4i r4[4];
+            if (has_res) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) r4[j] = rs[m][nn][j];
+                half_swap4(r4[0], r4[1]);
+                half_swap4(r4[2], r4[3]);
+            }
+            v4i o4[4];
+#pragma unroll
+            for (int e4 = 0; e4 < 4; ++e4) {
+                v4f v;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)accq[WRES ? m * 2 + nn : 0][e4][e], s4[e4][e], b4[e4][e]);
+                if (act_relu) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
+                }
+                if (has_res) {
+                    const v4f rv = __builtin_bit_cast(v4f, r4[e4]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += rv[e];
+                }
+                if (post_relu) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
+                }
+                o4[e4] = __builtin_bit_cast(v4i, v);
+                if (has_nchw) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        __builtin_amdgcn_raw_buffer_store_b32(o4[e4][e], rn, (int)noff[nn], (m * 32 + e4 * 4 + e) * img_px * 4, 0);
+                }
+                if (has_q) {
+                    int b[4];
+                    if (q_nonneg) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) b[e] = (int)__builtin_fminf(v[e] * p.fs_out + 0.5f, 127.f);
+                        q4[e4] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float t = v[e] * p.fs_out;
+                            b[e] = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
+                        }
+                        q4[e4] = (b[0] & 0xff) | ((b[1] & 0xff) << 8) | ((b[2] & 0xff) << 16) | (b[3] << 24);
+                    }
+                }
+            }
+            if (has_f) {
+                half_swap4(o4[0], o4[1]);
+                half_swap4(o4[2], o4[3]);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[j], rf, (int)(eoff[nn] * 4u + hh * 16 + m * 128 + piece(j)), 0, 0);
+            }
+            if (has_q) __builtin_amdgcn_raw_buffer_store_b128(q4, rq, (int)(eoff[nn] + hh * 16 + m * 32), 0, 0);
+        };
+        constexpr std::integral_constant<int, 0> c0{};
+        constexpr std::integral_constant<int, 1> c1{};
+        auto block_i = [&](int b, const unsigned (&eoff)[2], const unsigned (&noff)[2]) {
+            if (b == 0) block(c0, c0, eoff, noff);
+            else if (b == 1) block(c0, c1, eoff, noff);
+            else if (b == 2) block(c1, c0, eoff, noff);
+            else block(c1, c1, eoff, noff);
+        };
+        // which of a patch's four blocks run before its barrier `s`: spread so that no step holds the MFMA waves up
+        const int per_step = nst >= 4 ? 1 : 2;
+        auto first_block = [&](int s) { return WRES ? (s == 0 ? 0 : 1) : s * per_step; };
+        auto end_block = [&](int s) { const int e = WRES ? (s == 0 ? 1 : 4) : (s + 1) * per_step; return e < 4 ? e : 4; };
+
+        unsigned e_prev[2] = {0, 0}, n_prev[2] = {0, 0};   // offsets of the patch whose accumulators are next
+        unsigned e_cur[2], n_cur[2];
+        int n, oy0, ox0, pt = pj;
+        decode(pt, n, oy0, ox0);
+        offsets(n, oy0, ox0, e_cur, n_cur);
+        if (has_res) request_shortcut(e_cur);
+        barrier();
+        for (int t = 0; t < my_tiles; ++t) {
+            // during patch t's stages: the epilogue of patch t - 1 (offsets e_prev), then the request for patch t's shortcut
+            for (int s = 0; s < nst; ++s) {
+                if (t > 0) {
+                    if constexpr (WRES) {
+                        if (s == 0) {
+#pragma unroll
+                            for (int b = 0; b < 4; ++b) take_over(b);
+                        }
+                    }
+                    const int b0 = first_block(s), b1 = end_block(s);
+                    for (int b = b0; b < b1; ++b) block_i(b, e_prev, n_prev);
+                    if (has_res && b0 < 4 && b1 == 4) request_shortcut(e_cur);
+                }
+                barrier();
+            }
+            e_prev[0] = e_cur[0]; e_prev[1] = e_cur[1]; n_prev[0] = n_cur[0]; n_prev[1] = n_cur[1];
+            if (t + 1 < my_tiles) {
+                pt += GP;
+                decode(pt, n, oy0, ox0);
+                offsets(n, oy0, ox0, e_cur, n_cur);
+            }
+        }
+        if constexpr (WRES) {
+#pragma unroll
+            for (int b = 0; b < 4; ++b) take_over(b);
+        }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) block_i(b, e_prev, n_prev);
+    }
 }
 
 std::mutex g_attr_mutex;
@@ -547,7 +1043,39 @@ int launch_epi(exhip_ctx* ctx, const LeanParams& p, int grid) {
     }
 }
 
+template <bool WRES, int EPI>
+int launch_ws(exhip_ctx* ctx, const LeanParams& p, int grid) {
+    constexpr int lds = 3 * kWSlice + 2 * kActStride + 4 * 16384 + kSbB + kSpareB;
+    static unsigned long long attr_set = 0;
+    auto kernel = conv3x3_i8_ws_kernel<WRES, EPI>;
+    {
+        std::lock_guard<std::mutex> lock(g_attr_mutex);
+        const unsigned long long bit = 1ull << (ctx->device & 63);
+        if (!(attr_set & bit)) {
+            EXHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+            attr_set |= bit;
+        }
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(512), lds, ctx->stream, p);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+template <bool WRES>
+int launch_ws_epi(exhip_ctx* ctx, const LeanParams& p, int grid) {
+    switch (p.flags) {
+    case E_Q | E_ACT | E_QNN: return launch_ws<WRES, (E_Q | E_ACT | E_QNN)>(ctx, p, grid);
+    case E_RES | E_F | E_Q | E_POST | E_QNN: return launch_ws<WRES, (E_RES | E_F | E_Q | E_POST | E_QNN)>(ctx, p, grid);
+    default: return launch_ws<WRES, -1>(ctx, p, grid);
+    }
+}
+
 }  // namespace
+
+#if EXHIP_STAMPS
+// development builds only: where the kernel's waves leave their phase timestamps (16 words per wave), or NULL
+extern "C" void exhip_dev_lean_stamps(void* device_buffer) { g_lean_dbg = (long long*)device_buffer; }
+#endif
 
 int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
                           const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw) {
@@ -572,13 +1100,28 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
     p.magic_iw = magic(g.iw); p.magic_pw = magic(g.pw); p.magic_tx = magic(g.tiles_x); p.magic_txy = magic(p.tiles_xy);
     p.adv_iy = 51 / g.iw; p.adv_ix = 51 % g.iw;
     p.fs_out = g.fs_out;
+    p.dbg = g_lean_dbg;
+    p.stagger = g_exhip_options.lean_stagger;
     const bool q_nonneg = g.fs_out > 0.f && (g.post_relu || (g.act == 1 && !residual));
     p.flags = (residual ? E_RES : 0) | (y_f ? E_F : 0) | (y_q ? E_Q : 0) | (y_nchw ? E_NCHW : 0) | (g.act == 1 ? E_ACT : 0) |
               (g.post_relu ? E_POST : 0) | (q_nonneg ? E_QNN : 0);
 
+    if (mode == 3) {
+        // eight-wave groups, one per CU: MFMA waves and epilogue waves
+        const long long total = n_ptiles * g.ktiles;
+        long long G = total;
+        if (total > 256) G = 256;   // 256 is a multiple of 8 x the slab counts this path meets
+        if (G % g.ktiles != 0) G = G / g.ktiles * g.ktiles;
+        if (G <= 0 || (G % 8 == 0 && (G / 8) % g.ktiles != 0 && G != total)) return EXHIP_ERR_UNSUPPORTED;
+        if (g_exhip_options.lean_groups > 0 && G > (long long)g_exhip_options.lean_groups * g.ktiles)
+            G = (long long)g_exhip_options.lean_groups * g.ktiles;
+        if (g_exhip_options.debug_plan) fprintf(stderr, "  lean: wave-specialised, %lld groups for %lld tiles, flags %d\n", G, total, p.flags);
+        if (p.n_chunks == 1 && g_exhip_options.lean_wres != 0) return launch_ws_epi<true>(ctx, p, (int)G);
+        return launch_ws_epi<false>(ctx, p, (int)G);
+    }
     // groups: as many as stay resident (persistent), or one per patch and slab (mode 2)
-    const bool wres = p.n_chunks == 1;
-    const int cfg = wres ? 0 : g_exhip_options.lean_cfg;  // 0: one tile buffer, two slice buffers; 1: two and two; 2: one and three
+    const bool wres = p.n_chunks == 1 && g_exhip_options.lean_wres != 0;
+    const int cfg = g_exhip_options.lean_cfg;  // 0: one tile buffer, two slice buffers; 1: two and two; 2: one and three
     const int per_cu = wres ? 2 : (cfg == 0 ? 3 : 2);
     const long long total = n_ptiles * g.ktiles;
     long long G = total;

@@ -76,8 +76,9 @@ def all_epilogues(ctx, case, want_y):
     return out
 
 
-@pytest.mark.parametrize("mode,cfg,groups", [(1, 0, 0), (1, 1, 0), (1, 2, 0), (2, 0, 0), (1, 0, 2), (1, 1, 3), (1, 2, 1)],
-                         ids=["persist-a1w2", "persist-a2w2", "persist-a1w3", "oneshot", "walk2-a1w2", "walk3-a2w2", "walk1-a1w3"])
+@pytest.mark.parametrize("mode,cfg,groups", [(1, 0, 0), (1, 1, 0), (1, 2, 0), (2, 0, 0), (1, 0, 2), (1, 1, 3), (1, 2, 1), (3, 0, 0), (3, 0, 2), (3, 0, 1)],
+                         ids=["persist-a1w2", "persist-a2w2", "persist-a1w3", "oneshot", "walk2-a1w2", "walk3-a2w2", "walk1-a1w3",
+                              "roles", "roles-walk2", "roles-walk1"])
 @pytest.mark.parametrize("args", LEAN_SHAPES, ids=[f"s{a[0]}" for a in LEAN_SHAPES])
 def test_lean_kernel_bit_exact(ctx, options, args, mode, cfg, groups):
     seed, n, c, h, w, k = args
@@ -100,8 +101,8 @@ def test_lean_and_general_kernel_agree_on_a_stage_sized_launch(ctx, options):
     fs_out = np.float32(9.3)
     options("lean", 0)
     want = gpueval.conv_i8(ctx, case, fs_out=fs_out, residual=res, post_relu=1, want=("nhwc",))
-    for groups in (0, 5):
-        options("lean", 1)
+    for mode, groups in ((1, 0), (1, 5), (3, 0), (3, 5)):
+        options("lean", mode)
         options("lean_groups", groups)
         got = gpueval.conv_i8(ctx, case, fs_out=fs_out, residual=res, post_relu=1, want=("nhwc",))
         assert np.array_equal(got["nhwc"], want["nhwc"])
