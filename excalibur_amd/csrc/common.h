@@ -57,7 +57,8 @@ struct exhip_options {
     int dw_band_rows = 0;    // row-band height of the depthwise strip kernels
     int force_splits = 0;    // groups per tile of the convolution's split reduction (1 = never split)
     int share_gpu = 0;       // launches of several streams overlap: the planner then counts groups per CU, not rounds of one launch
-    int lean = 1;            // 3x3 stride-1 int8 layers with the fused epilogue: 0 general kernel, 1 lean persistent kernel, 2 lean, one group per patch
+    int lean = 4;            // 3x3 stride-1 int8 layers with the fused epilogue: 0 general kernel, 1 lean kernel with persistent groups, 2 lean, one
+                             // group per patch, 3 lean with MFMA and epilogue waves, 4 the form measured fastest for the layer's class
     int lean_cfg = 0;        // its staging buffers for layers of more than 64 input channels: 0 one tile + two slices, 1 two + two, 2 one + three
     int lean_wres = 1;       // 64 input channels: keep the slab's whole filter in LDS (0: stream it like the deeper layers)
     int lean_stagger = 0;    // experiment: start delay per hardware wave slot, in units of 64 cycles

@@ -613,7 +613,22 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
     // waits for this wave's LDS operations, then for the group: what was written before is visible behind it. No memory
     // fence: that would also wait for every global access in flight, which is what the epilogue waves must not do.
-    auto barrier = [&]() { __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    long long t_mfma = 0, t_wait = 0, t_bar = 0, t_epi = 0, t_mark = 0;
+    auto now = [&]() -> long long { return kStamps && p.dbg ? (long long)clock64() : 0ll; };
+    auto put = [&](int k, long long v) {
+        if constexpr (kStamps)
+            if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * 8 + wave8) * 16 + k] = v;
+    };
+    auto lap = [&](long long& acc_t) {
+        if constexpr (kStamps) { const long long t = now(); acc_t += t - t_mark; t_mark = t; }
+    };
+    put(0, now());
+    if constexpr (kStamps) put(10, (long long)wall_clock64());
+    auto barrier = [&]() {
+        lap(t_mfma);
+        __asm__ volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        lap(t_bar);
+    };
 
     const int G = gridDim.x;
     int lb = blockIdx.x;
@@ -792,8 +807,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         if constexpr (WRES) {
             request_a(img, base, 0, true, lds0 + A0);
             for (int r = 0; r < 3; ++r) request_w(lds0 + r * kWSlice);
-            wait_vmcnt<0>();
+            lap(t_mfma); wait_vmcnt<0>(); lap(t_wait);
+            put(1, now());
             barrier();
+            put(2, now());
+            t_mark = now(); t_mfma = 0; t_bar = 0; t_wait = 0;
             for (int done = 0; done < my_tiles; ++done) {
                 const bool has_next = done + 1 < my_tiles;
                 const char* const ab = smem + A0 + abuf * kActStride;
@@ -802,7 +820,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                 barrier();   // the epilogue waves have taken the previous patch's accumulators
                 mfma_rows(two_rows, smem + kWSlice + lane * 16, ab + row_b + boff[0], ab + row_b + boff[1], []() {});
                 hand_over();
-                wait_vmcnt<0>();
+                lap(t_mfma); wait_vmcnt<0>(); lap(t_wait);
                 barrier();
                 clear_acc();
                 abuf = 1 - abuf;
@@ -811,8 +829,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             request_a(img, base, 0, true, lds0 + A0);
             request_w(lds0);
             request_w(lds0 + kWSlice);
-            wait_vmcnt<3>();
+            lap(t_mfma); wait_vmcnt<3>(); lap(t_wait);
+            put(1, now());
             barrier();
+            put(2, now());
+            t_mark = now(); t_mfma = 0; t_bar = 0; t_wait = 0;
             for (int done = 0; done < my_tiles; ++done) {
                 const bool has_next = done + 1 < my_tiles;
                 for (int cc = 0; cc < p.n_chunks; ++cc) {
@@ -825,14 +846,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                         request_w(lds0 + 2 * kWSlice);
                         request_next_a(cc, last_cc, has_next, a_other);
                     });
-                    wait_vmcnt<3 + kNAL>();
+                    lap(t_mfma); wait_vmcnt<3 + kNAL>(); lap(t_wait);
                     barrier();
                     mfma_rows(one_row, smem + kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0); });
-                    wait_vmcnt<3 + kNAL>();
+                    lap(t_mfma); wait_vmcnt<3 + kNAL>(); lap(t_wait);
                     barrier();
                     mfma_rows(one_row, smem + 2 * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b, [&]() { request_w(lds0 + kWSlice); });
                     if (last_cc) hand_over();
-                    wait_vmcnt<3>();
+                    lap(t_mfma); wait_vmcnt<3>(); lap(t_wait);
                     barrier();
                     abuf = 1 - abuf;
                 }
@@ -981,7 +1002,10 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         decode(pt, n, oy0, ox0);
         offsets(n, oy0, ox0, e_cur, n_cur);
         if (has_res) request_shortcut(e_cur);
+        put(1, now());
         barrier();
+        put(2, now());
+        t_mark = now(); t_mfma = 0; t_bar = 0;
         for (int t = 0; t < my_tiles; ++t) {
             // during patch t's stages: the epilogue of patch t - 1 (offsets e_prev), then the request for patch t's shortcut
             for (int s = 0; s < nst; ++s) {
@@ -1012,6 +1036,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int b = 0; b < 4; ++b) block_i(b, e_prev, n_prev);
     }
+    lap(t_epi);
+    put(3, t_mfma); put(4, t_wait); put(5, t_bar); put(6, t_epi); put(8, now()); put(9, my_tiles);
+    if constexpr (kStamps) put(11, (long long)wall_clock64());
 }
 
 std::mutex g_attr_mutex;
@@ -1079,8 +1106,24 @@ extern "C" void exhip_dev_lean_stamps(void* device_buffer) { g_lean_dbg = (long 
 
 int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
                           const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw) {
-    const int mode = g_exhip_options.lean;
+    int mode = g_exhip_options.lean;
     if (mode == 0) return EXHIP_ERR_UNSUPPORTED;
+    int cfg = g_exhip_options.lean_cfg;  // 0: one tile buffer, two slice buffers; 1: two and two; 2: one and three
+    if (mode == 4) {
+        // The form that measured fastest per layer class on the ResNet-18-shaped stack at 32 x 640 x 640: without a shortcut
+        // the resident filter (64 channels) or one group per patch with three groups per CU; with a shortcut, whose float32
+        // traffic is the larger part of the launch, the general kernel up to 128 channels (its three groups per CU keep
+        // more of it in flight) and persistent groups with deeper buffers beyond.
+        const int chunks = g.c_bytes / 64;
+        if (!residual) {
+            mode = chunks == 1 ? 1 : (chunks <= 4 ? 2 : 1);
+            cfg = chunks <= 4 ? 0 : 2;
+        } else {
+            if (chunks <= 2) return EXHIP_ERR_UNSUPPORTED;
+            mode = 1;
+            cfg = chunks <= 4 ? 1 : 2;
+        }
+    }
     const long long n_ptiles = (long long)g.n * g.tiles_y * g.tiles_x;
     const long long out_elems = (long long)g.n * g.oh * g.ow * g.k;
     if (g.c_bytes % 64 != 0 || g.k % 64 != 0 || g.ph * g.pw > 256 || g.ih * g.iw * kPixB + 16 > kActStride || n_ptiles >= 65536 ||
@@ -1121,7 +1164,6 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
     }
     // groups: as many as stay resident (persistent), or one per patch and slab (mode 2)
     const bool wres = p.n_chunks == 1 && g_exhip_options.lean_wres != 0;
-    const int cfg = g_exhip_options.lean_cfg;  // 0: one tile buffer, two slice buffers; 1: two and two; 2: one and three
     const int per_cu = wres ? 2 : (cfg == 0 ? 3 : 2);
     const long long total = n_ptiles * g.ktiles;
     long long G = total;

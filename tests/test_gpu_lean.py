@@ -27,7 +27,7 @@ def options():
         hip.set_option(name, value)
         changed.append(name)
     yield set_
-    defaults = dict(lean=1, lean_cfg=0, lean_groups=0)
+    defaults = dict(lean=4, lean_cfg=0, lean_groups=0)
     for name in changed:
         hip.set_option(name, defaults[name])
 
