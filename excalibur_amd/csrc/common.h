@@ -22,6 +22,10 @@ int exhip_split_scratch(exhip_ctx* ctx, size_t acc_bytes, size_t tiles, int** ac
 
 void exhip_set_error(const char* fmt, ...);
 
+// How exhip_conv_pack_weights lays this layer's weights out: output channels per slab, and whether it is the packed
+// first-layer form (4- or 8-byte pixels, one k-step per filter row).
+int exhip_conv_packed_layout(const exhip_conv_desc* d, int dtype, int* slab_channels, int* packed_form);
+
 // Looks up, once per device and with that device current, the address of the static scratch array behind
 // exhip_maxpool_same_nhwc_f16_static (defined beside that array).
 int exhip_static_scratch_setup(int device);
@@ -62,6 +66,7 @@ struct exhip_options {
     int lean_cfg = 0;        // its staging buffers for layers of more than 64 input channels: 0 one tile + two slices, 1 two + two, 2 one + three
     int lean_wres = 1;       // 64 input channels: keep the slab's whole filter in LDS (0: stream it like the deeper layers)
     int lean_stagger = 0;    // experiment: start delay per hardware wave slot, in units of 64 cycles
+    int stem = 1;            // the stem (quantizer + first convolution + max pooling) as one kernel where the entry point offers it
     int lean_groups = 0;     // at most this many groups per 64-channel slab (tests: a few groups that walk many patches each)
 };
 extern exhip_options g_exhip_options;

@@ -70,7 +70,8 @@ struct LeanParams {
     long long* dbg;  // phase timestamps (builds with -DEXHIP_STAMPS=1 only)
 };
 
-__device__ __forceinline__ int fast_div(int n, unsigned magic) { return (int)__umulhi((unsigned)n, magic); }
+// n / d for n < 2^16 with magic = ceil(2^32 / d) as a 32-bit word: one multiply-high; d == 1 arrives as 0
+__device__ __forceinline__ int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
 __device__ __forceinline__ v4i lds_read16(const char* p) { return *reinterpret_cast<const v4i*>(p); }
 
 // One 16-byte element per lane from a bounds-checked buffer view straight into LDS: lane l's data lands at

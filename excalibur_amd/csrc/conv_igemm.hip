@@ -1723,6 +1723,15 @@ void pack_weights_t(const exhip_conv_desc* d, int dt, const Plan& pl, const T* w
 
 }  // namespace
 
+int exhip_conv_packed_layout(const exhip_conv_desc* d, int dtype, int* slab_channels, int* packed_form) {
+    Plan pl;
+    const int rc = make_plan(d, dtype, &pl);
+    if (rc) return rc;
+    *slab_channels = pl.TM;
+    *packed_form = pl.packed ? 1 : 0;
+    return 0;
+}
+
 extern "C" int exhip_conv_out_hw(const exhip_conv_desc* d, int* oh, int* ow) {
     EXHIP_REQUIRE(d && oh && ow, "exhip_conv_out_hw: NULL argument");
     EXHIP_REQUIRE(d->sh > 0 && d->sw > 0, "exhip_conv_out_hw: bad stride");

@@ -34,6 +34,7 @@ extern "C" int exhip_set_option(const char* name, int value) {
     else if (!strcmp(name, "lean_cfg")) o.lean_cfg = value;
     else if (!strcmp(name, "lean_groups")) o.lean_groups = value;
     else if (!strcmp(name, "lean_wres")) o.lean_wres = value;
+    else if (!strcmp(name, "stem")) o.stem = value;
     else if (!strcmp(name, "lean_stagger")) o.lean_stagger = value;
     else {
         exhip_set_error("exhip_set_option: unknown option %s", name);

@@ -222,6 +222,17 @@ class Ctx:
         _check(lib().exhip_conv2d_i8_maxpool3x3s2(self.h, ctypes.byref(d), pool_pad, pool_pad, pool_oh, pool_ow, x.ptr, wp.ptr,
                                                   scale.ptr, _ptr(bias), _ptr(y_i8), _ptr(y_f32_nhwc)))
 
+    def stem_f32_conv_i8_maxpool3x3s2(self, d, pool_pad, pool_oh, pool_ow, x_nchw, fs_in, wp, scale, scales_nonnegative, bias=None,
+                                      y_i8=None, y_f32_nhwc=None):
+        """Returns False when the library leaves the shape to the quantizer + exhip_conv2d_i8_maxpool3x3s2."""
+        rc = lib().exhip_stem_f32_conv_i8_maxpool3x3s2(self.h, ctypes.byref(d), pool_pad, pool_pad, pool_oh, pool_ow, x_nchw.ptr,
+                                                       ctypes.c_float(fs_in), wp.ptr, scale.ptr, int(scales_nonnegative), _ptr(bias),
+                                                       _ptr(y_i8), _ptr(y_f32_nhwc))
+        if rc == 10002:
+            return False
+        _check(rc)
+        return True
+
     def conv2d_f16(self, d, x, wp, bias=None, residual=None, y_f16_nhwc=None, y_f16_nchw=None, y_f32_nchw=None):
         _check(lib().exhip_conv2d_f16(self.h, ctypes.byref(d), x.ptr, wp.ptr, _ptr(bias), _ptr(residual), _ptr(y_f16_nhwc),
                                       _ptr(y_f16_nchw), _ptr(y_f32_nchw)))

@@ -45,7 +45,8 @@ public:
     bool fused() const;
     double last_forward_ms() const;
     // Device time of part of a fused forward: with first_launch >= 0 every fused forward records one event in front
-    // of its launch number first_launch (0 is the input quantizer) and one behind its last launch;
+    // of its launch number first_launch (0 is the input quantizer, unless the stem kernel quantizes its own input; -2 stands
+    // for the first convolution's launch, whichever number it has) and one behind its last launch;
     // last_span(&launches) waits for them and returns the milliseconds between the two and the launches in between.
     void time_fused_span(int first_launch);
     float last_span(int* launches);

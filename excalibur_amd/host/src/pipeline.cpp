@@ -437,6 +437,7 @@ struct pipeline<Dtype>::impl::fused_plan {
     };
     std::deque<result> outputs;  // stable addresses: the launches keep pointers to the slots
     const float* input_ptr = nullptr;
+    int first_conv_launch = 1;  // 1: launch 0 is the input quantizer; 0: the stem kernel quantizes its own input
     // Launches 1 .. end (everything behind the input quantizer, which alone reads the caller's input pointer) recorded as
     // one HIP graph: made on the plan's second forward (the first runs eagerly, which also sets the kernels' attributes),
     // replayed afterwards, made again when a result tensor was replaced.
@@ -608,6 +609,7 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
             plan->launches.push_back([=]() {
                 EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(ctx, pl->input_ptr, vi.n, vi.c, vi.h, vi.w, vi.fs, nullptr, vi.cs, q));
             });
+            plan->first_conv_launch = 1;
         }
         for (const node& nd : nodes) {
             const value_info in = vals[nd.in_value];
@@ -660,7 +662,28 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                         if (rc == EXHIP_ERR_UNSUPPORTED) one_kernel = false;
                         else EXHIP_FATAL(rc);
                     }
-                    if (one_kernel) {
+                    // the network's input read by this layer alone: the stem kernel quantizes it on the way in
+                    bool stem_kernel = false;
+                    if (one_kernel && nd.in_value == in_value && consumers[in_value].size() == 1 && plan->launches.size() == 1) {
+                        bool nonneg = true;
+                        for (float sc : c->dequantize_scales()) nonneg = nonneg && sc >= 0.f;
+                        fused_plan* fp = plan.get();
+                        const float fs_in = in.fs;
+                        const int nn = nonneg ? 1 : 0;
+                        const int rc = exhip_stem_f32_conv_i8_maxpool3x3s2(ctx, &d, pt, pl, ph, pw, input->gpu_data(), fs_in, wp, scale, nn, bias, yq, yf);
+                        if (rc == 0) {
+                            stem_kernel = true;
+                            plan->launches.clear();  // the quantizer's launch
+                            plan->first_conv_launch = 0;
+                            plan->launches.push_back([=]() {
+                                EXHIP_FATAL(exhip_stem_f32_conv_i8_maxpool3x3s2(ctx, &d, pt, pl, ph, pw, fp->input_ptr, fs_in, wp, scale, nn, bias, yq, yf));
+                            });
+                        } else if (rc != EXHIP_ERR_UNSUPPORTED) {
+                            EXHIP_FATAL(rc);
+                        }
+                    }
+                    if (stem_kernel) {
+                    } else if (one_kernel) {
                         plan->launches.push_back(
                             [=]() { EXHIP_FATAL(exhip_conv2d_i8_maxpool3x3s2(ctx, &d, pt, pl, ph, pw, x, wp, scale, bias, yq, yf)); });
                     } else {
@@ -727,13 +750,14 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
     }
     exhip_ctx* const ctx = memory::device_context(device_);
     const int n_launches = static_cast<int>(plan_->launches.size());
-    const bool timed = span_first_ >= 0 && span_first_ < n_launches;
+    const int span_first = span_first_ == -2 ? plan_->first_conv_launch : span_first_;  // -2: from the first convolution on
+    const bool timed = span_first >= 0 && span_first < n_launches;
     if (timed && !span_ev_[0]) {
         EXHIP_FATAL(exhip_event_create(&span_ev_[0]));
         EXHIP_FATAL(exhip_event_create(&span_ev_[1]));
     }
     // the graph form: launch 0 eagerly, the rest as one replay (a timed span must start at launch 0 or 1 to use it)
-    bool use_graph = graphs_ && n_launches > 2 && plan_->forwards >= 1 && (!timed || span_first_ <= 1);
+    bool use_graph = graphs_ && n_launches > 2 && plan_->forwards >= 1 && (!timed || span_first <= 1);
     if (use_graph) {
         std::vector<float*> slots;
         for (auto& r : plan_->outputs) slots.push_back(r.slot);
@@ -747,19 +771,19 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
             EXHIP_FATAL(exhip_graph_end(ctx, &plan_->graph));
             plan_->graph_slots = slots;
         }
-        if (timed && span_first_ == 0) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+        if (timed && span_first == 0) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
         plan_->launches[0]();
-        if (timed && span_first_ == 1) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+        if (timed && span_first == 1) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
         EXHIP_FATAL(exhip_graph_launch(ctx, plan_->graph));
         if (timed) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[1]));
-        span_launches_ = timed ? n_launches - span_first_ : 0;
+        span_launches_ = timed ? n_launches - span_first : 0;
     } else if (timed) {
         for (int i = 0; i < n_launches; ++i) {
-            if (i == span_first_) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+            if (i == span_first) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
             plan_->launches[i]();
         }
         EXHIP_FATAL(exhip_event_record(ctx, span_ev_[1]));
-        span_launches_ = n_launches - span_first_;
+        span_launches_ = n_launches - span_first;
     } else {
         for (auto& launch : plan_->launches) launch();
         span_launches_ = 0;

@@ -131,7 +131,8 @@ class Pipeline:
 
     def time_fused_span(self, first_launch):
         """Every later fused forward records device events around its launches first_launch .. last (0 = the input
-        quantizer); -1 switches that off."""
+        quantizer unless the stem kernel quantizes the input itself, -2 = the first convolution's launch); -1 switches
+        that off."""
         lib().exc_pipeline_time_fused_span(self.h, int(first_launch))
 
     def last_span(self):

@@ -186,6 +186,29 @@ class FusedRunner:
         self.steps.append((layer.name, "conv", lambda: ctx.conv2d_i8_maxpool3x3s2(d, 1, ph, pw, x_i8, wp, scale_d, bias_d, yq, y)))
         return y, yq, ph, pw, layer.k
 
+    def _stem(self, layer, x, fs_out):
+        """Quantizer, stem convolution and max pool as one launch where the library offers it (None otherwise)."""
+        ctx, hip = self.ctx, self.hip
+        d = ctx.conv_desc(self.n, layer.c, self.h, self.w, layer.k, layer.kernel, layer.stride, layer.pad, layer.act, 4, layer.k,
+                          0, float(fs_out))
+        oh, ow = ctx.conv_out_hw(d)
+        ph, pw = (oh + 2 - 3) // 2 + 1, (ow + 2 - 3) // 2 + 1
+        wp = ctx.pack_conv_weights(d, hip.I8, layer.w_i8)
+        ws, fs = layer.ws, layer.fs
+        with np.errstate(divide="ignore"):
+            scale = np.where(np.abs(ws.astype(np.float64)) <= 1e-6, np.float32(0),
+                             np.float32(1.0) / (ws * fs).astype(np.float32)).astype(np.float32)
+        nonneg = bool((scale >= 0).all())
+        scale_d, bias_d = ctx.array(scale), ctx.array(layer.bias)
+        y = ctx.empty((self.n, ph, pw, layer.k), np.float32)
+        yq = ctx.empty((self.n, ph, pw, layer.k), np.int8)
+        if not ctx.stem_f32_conv_i8_maxpool3x3s2(d, 1, ph, pw, x, float(fs), wp, scale_d, nonneg, bias_d, yq, y):
+            return None
+        self.conv_gop[layer.name] = 2.0 * self.n * oh * ow * layer.k * layer.c * layer.kernel * layer.kernel / 1e9
+        self.steps.append((layer.name, "conv", lambda: ctx.stem_f32_conv_i8_maxpool3x3s2(d, 1, ph, pw, x, float(fs), wp, scale_d, nonneg,
+                                                                                         bias_d, yq, y)))
+        return y, yq, ph, pw, layer.k
+
     def _quantize_input(self, x, q, fs):
         import ctypes
         ctx, n, h, w = self.ctx, self.n, self.h, self.w
@@ -215,10 +238,14 @@ class FusedRunner:
         ctx, net, n = self.ctx, self.net, self.n
         self.x = ctx.empty((n, 3, self.h, self.w), np.float32)
         self.q0 = ctx.empty((n, self.h, self.w, 4), np.int8)
-        self._quantize_input(self.x, self.q0, net.stem.fs)
-        if self.fuse_pool:
+        stem = self._stem(net.stem, self.x, net.blocks[0][0].fs) if self.fuse_pool else None
+        if stem is not None:
+            pool_f32, pool_i8, ph, pw, ks = stem
+        elif self.fuse_pool:
+            self._quantize_input(self.x, self.q0, net.stem.fs)
             pool_f32, pool_i8, ph, pw, ks = self._conv_maxpool(net.stem, self.q0, self.h, self.w, 4, net.blocks[0][0].fs)
         else:
+            self._quantize_input(self.x, self.q0, net.stem.fs)
             _, stem_f32, _, oh, ow, ks = self._conv(net.stem, self.q0, self.h, self.w, 4, None, 0, None, True, False)
             pool_f32, pool_i8, ph, pw = self._maxpool(stem_f32, 64, oh, ow, ks, net.blocks[0][0].fs)
         cur_i8, cur_f32, hh, ww, cs = pool_i8, pool_f32, ph, pw, ks

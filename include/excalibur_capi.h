@@ -52,7 +52,8 @@ int exc_pipeline_forward(exc_pipeline* p, const void* input, const int shape[4])
 long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, long capacity, int shape[4]);
 /* Device time of part of a fused forward (no counterpart in the reference: a measurement aid). With
  * first_launch >= 0 every later fused forward records one event in front of its launch number first_launch
- * (0 = the input quantizer) and one behind its last launch; -1 switches that off. exc_pipeline_last_span waits for
+ * (0 = the input quantizer, or the stem when its kernel quantizes the input itself; -2 = the first convolution's launch,
+ * whichever number it has) and one behind its last launch; -1 switches that off. exc_pipeline_last_span waits for
  * the device and returns the milliseconds between the two events of the last forward and, in *launches, how many
  * launches lay between them (0 and 0.0 if the last forward was not a fused one). */
 void exc_pipeline_time_fused_span(exc_pipeline* p, int first_launch);

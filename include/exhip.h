@@ -149,6 +149,19 @@ int exhip_conv2d_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_desc* d, int p
                                  int pool_ow, const int8_t* x_nhwc, const void* w_packed, const float* scale,
                                  const float* bias, int8_t* y_i8_nhwc, float* y_f32_nhwc);
 
+/* The stem of an int8 network in one kernel: quantize_float32_to_int8 of the float32 NCHW input with the per-tensor scale
+ * fs_in (src/Excalibur/operation_general_conv.cpp:584-720), the first convolution (operation_convolution::forward_cpu_i8,
+ * src/Excalibur/operation_convolution.cpp:373-408) and MAX pooling 3x3 stride 2 (src/Excalibur/operation_pooling.cpp:145-159)
+ * as in exhip_conv2d_i8_maxpool3x3s2; neither the quantized input nor the convolution's output reaches memory. d describes
+ * the convolution on 4-byte pixels (c <= 4, c_stride 4, kw <= 8, kh 3 / 5 / 7, stride 2, k % 64 == 0, act 0 or 1), w_packed
+ * is exhip_conv_pack_weights' output for it. The maximum is taken on the int32 accumulators, which is the reference's
+ * result when no dequantization scale is negative: the caller states that with scales_nonnegative != 0.
+ * EXHIP_ERR_UNSUPPORTED for anything else (the caller then runs the quantizer and exhip_conv2d_i8_maxpool3x3s2). */
+int exhip_stem_f32_conv_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_desc* d, int pool_pt, int pool_pl, int pool_oh,
+                                        int pool_ow, const float* x_f32_nchw, float fs_in, const void* w_packed,
+                                        const float* scale, int scales_nonnegative, const float* bias, int8_t* y_i8_nhwc,
+                                        float* y_f32_nhwc);
+
 /* operation_convolution::forward_cpu_f32 (src/Excalibur/operation_convolution.cpp:251-329) with fp16
  * storage and f32 accumulation (include/Excalibur/operation.hpp:234-260 describes the fp16 layer):
  * x NHWC f16; outputs NHWC f16 and/or NCHW f16 and/or NCHW f32. residual_nhwc (NHWC f16, the output's shape and

@@ -40,6 +40,8 @@ LEAN_SHAPES = [
     (903, 1, 256, 20, 20, 64),    # four chunks
     (904, 3, 128, 9, 11, 192),    # an image smaller than a patch, three slabs
     (905, 2, 512, 20, 20, 128),   # eight chunks, patch wider than tall
+    (906, 2, 256, 40, 40, 64),    # patches as wide as the image (one per row band)
+    (907, 3, 64, 12, 14, 64),     # one patch per image
 ]
 
 
