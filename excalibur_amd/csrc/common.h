@@ -16,8 +16,10 @@ struct exhip_ctx {
     size_t split_count_n = 0;
 };
 
-// Makes the context's split-reduction scratch at least this large (partial accumulators, and one zeroed arrival counter per
-// tile) and returns it. Growing it waits for the stream; no allocation happens when it is large enough already.
+// The context's split-reduction scratch (partial accumulators, and one zeroed arrival counter per tile): allocated on first
+// use at its fixed upper bound -- kSplitGroups groups per launch -- and never moved or grown afterwards; a request beyond
+// the bound is an error (the planner clamps its splits to it).
+constexpr int kSplitGroups = 256;
 int exhip_split_scratch(exhip_ctx* ctx, size_t acc_bytes, size_t tiles, int** acc, unsigned** count);
 
 void exhip_set_error(const char* fmt, ...);

@@ -1644,6 +1644,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         long long s = std::min<long long>(pl.n_chunks / min_chunks, kCUs / tiles);  // measured: no gain once every CU has a group
         s = std::min<long long>(s, 16);
         if (g_exhip_options.force_splits > 1) s = std::min<long long>(g_exhip_options.force_splits, pl.n_chunks / min_chunks);
+        s = std::min<long long>(s, kSplitGroups / tiles);  // the scratch holds kSplitGroups groups' accumulators, whatever forces the split
         if (s >= 2) {
             const size_t acc_bytes = (size_t)tiles * s * pl.threads * 256;  // 64 words per lane
             rc = exhip_split_scratch(ctx, acc_bytes, (size_t)tiles, &p.split_acc, &p.split_count);

@@ -81,7 +81,14 @@ extern "C" int exhip_destroy(exhip_ctx* ctx) {
 
 extern "C" int exhip_malloc(exhip_ctx* ctx, size_t bytes, void** dptr) {
     EXHIP_REQUIRE(ctx && dptr, "exhip_malloc: NULL argument");
-    EXHIP_CHECK(hipMalloc(dptr, bytes ? bytes : 1));
+    const hipError_t e = hipMalloc(dptr, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        // the runtime keeps a failed call's code as the thread's last error, where the next launch check would find it: a
+        // caller that recovers (frees blocks, asks again) must not be failed by it later
+        (void)hipGetLastError();
+        exhip_set_error("hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+        return (int)e;
+    }
     return 0;
 }
 
@@ -199,25 +206,31 @@ extern "C" int exhip_graph_destroy(void* graph_exec) {
     return 0;
 }
 
+// The scratch never moves once it exists: a recorded HIP graph keeps its address in kernel nodes, so it is allocated once per
+// context at its upper bound (the planner splits a launch into at most kSplitGroups groups of at most 512 threads, 256 bytes
+// of accumulators per thread) together with one arrival counter per possible tile.
 int exhip_split_scratch(exhip_ctx* ctx, size_t acc_bytes, size_t tiles, int** acc, unsigned** count) {
-    if (acc_bytes > ctx->split_acc_bytes) {
-        EXHIP_CHECK(hipStreamSynchronize(ctx->stream));
-        if (ctx->split_acc) EXHIP_CHECK(hipFree(ctx->split_acc));
-        ctx->split_acc = nullptr;
-        ctx->split_acc_bytes = 0;
-        const size_t want = std::max(acc_bytes, (size_t)4 << 20);
-        EXHIP_CHECK(hipMalloc(reinterpret_cast<void**>(&ctx->split_acc), want));
-        ctx->split_acc_bytes = want;
-    }
-    if (tiles > ctx->split_count_n) {
-        EXHIP_CHECK(hipStreamSynchronize(ctx->stream));
-        if (ctx->split_count) EXHIP_CHECK(hipFree(ctx->split_count));
-        ctx->split_count = nullptr;
-        ctx->split_count_n = 0;
-        const size_t want = std::max(tiles, (size_t)1024);
-        EXHIP_CHECK(hipMalloc(reinterpret_cast<void**>(&ctx->split_count), want * sizeof(unsigned)));
-        EXHIP_CHECK(hipMemset(ctx->split_count, 0, want * sizeof(unsigned)));  // every launch leaves its counters at zero
-        ctx->split_count_n = want;
+    constexpr size_t kAccBytes = (size_t)kSplitGroups * 512 * 256, kCounters = kSplitGroups;
+    EXHIP_REQUIRE(acc_bytes <= kAccBytes && tiles <= kCounters, "split reduction: %zu bytes for %zu tiles exceed the scratch's fixed size", acc_bytes,
+                  tiles);
+    if (!ctx->split_acc) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        EXHIP_CHECK(hipStreamIsCapturing(ctx->stream, &capturing));
+        EXHIP_REQUIRE(capturing == hipStreamCaptureStatusNone,
+                      "split reduction: its scratch cannot be allocated while the stream records a graph; run the launch once before recording");
+        EXHIP_CHECK(hipMalloc(reinterpret_cast<void**>(&ctx->split_acc), kAccBytes));
+        ctx->split_acc_bytes = kAccBytes;
+        hipError_t e = hipMalloc(reinterpret_cast<void**>(&ctx->split_count), kCounters * sizeof(unsigned));
+        if (e == hipSuccess) e = hipMemset(ctx->split_count, 0, kCounters * sizeof(unsigned));  // every launch leaves its counters at zero
+        if (e != hipSuccess) {
+            (void)hipFree(ctx->split_acc);
+            if (ctx->split_count) (void)hipFree(ctx->split_count);
+            ctx->split_acc = nullptr;
+            ctx->split_count = nullptr;
+            exhip_set_error("split reduction: allocating the arrival counters failed: %s", hipGetErrorString(e));
+            return (int)e;
+        }
+        ctx->split_count_n = kCounters;
     }
     *acc = ctx->split_acc;
     *count = ctx->split_count;

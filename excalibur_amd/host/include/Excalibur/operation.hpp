@@ -67,6 +67,7 @@ public:
     void forward_cpu(const tensor_list<Dtype>& bottoms, tensor_list<Dtype>& tops);
     void forward_gpu(const tensor_list<Dtype>& bottoms, tensor_list<Dtype>& tops);
 
+    tensor_list<double>& weights_d64() { return weights_d64_; }
     tensor_list<float>& weights_f32() { return weights_f32_; }
     tensor_list<unsigned short>& weights_f16() { return weights_f16_; }
     tensor_list<signed char>& weights_i8() { return weights_i8_; }
@@ -74,6 +75,7 @@ public:
     virtual const char* type() const { return "Unknown Type"; }
 
 protected:
+    tensor_list<double> weights_d64_;   // declared as in the reference (include/Excalibur/operation.hpp:158); no layer of the path fills it
     tensor_list<float> weights_f32_;
     tensor_list<unsigned short> weights_f16_;
     tensor_list<signed char> weights_i8_;
@@ -85,6 +87,9 @@ protected:
     virtual void forward_cpu_f16(const tensor_list<unsigned short>&, tensor_list<unsigned short>&) { NO_CPU; }
     virtual void forward_cpu_i8(const tensor_list<float>&, tensor_list<float>&) { NO_CPU; }
     virtual void forward_gpu_f32(const tensor_list<float>&, tensor_list<float>&) { NOT_IMPLEMENTED; }
+    // the reference's double-precision hooks (include/Excalibur/operation.hpp:185-201): NOT_IMPLEMENTED there and here
+    virtual void forward_cpu_d64(const tensor_list<double>&, tensor_list<double>&) { NOT_IMPLEMENTED; }
+    virtual void forward_gpu_d64(const tensor_list<double>&, tensor_list<double>&) { NOT_IMPLEMENTED; }
     // Default fp16 layer: the float32 operator on converted data, as the reference's CPU wrapper does
     // (include/Excalibur/operation.hpp:204-266): half -> float, forward_gpu_f32, float -> half.
     virtual void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops);

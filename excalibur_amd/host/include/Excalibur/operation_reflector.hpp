@@ -81,5 +81,14 @@ public:
     REGISTE_FLOAT(CLASS_NAME) \
     REGISTE_DOUBLE(CLASS_NAME)
 
+// The reference's way of giving an operator without device code a forward_gpu_f32 that stops
+// (include/Excalibur/operation_reflector.hpp:95-100): kept so that operator sources written against it compile.
+#define STUB_GPU(Operation_Name)                                                                          \
+    template <typename Dtype>                                                                            \
+    void Operation_Name<Dtype>::forward_gpu_f32(const std::vector<std::shared_ptr<memory::tensor<float>>>& bottoms, \
+                                                std::vector<std::shared_ptr<memory::tensor<float>>>& tops) {        \
+        NO_GPU;                                                                                          \
+    }
+
 }  // namespace excalibur
 }  // namespace glasssix

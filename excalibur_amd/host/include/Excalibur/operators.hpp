@@ -53,6 +53,9 @@ public:
     const float* scale_gpu();
     // weights packed for the MFMA kernel for one input geometry; cached per (dtype, n, h, w, c_stride)
     const void* packed_weights(int dtype, const exhip_conv_desc& d);
+    // A holder that keeps the pointer across forwards (a fused plan) pins the copy: pinned copies are never evicted.
+    const void* pin_packed_weights(int dtype, const exhip_conv_desc& d);
+    void unpin_packed_weights(const void* ptr);
     exhip_conv_desc describe(int n, int h, int w, int c_stride, int k_stride) const;
     // The activation layer behind this one, applied in the kernel's epilogue by the next forward calls: post_op 0 = none,
     // else 1 + EXHIP_UNARY_* with its two parameters; relu = a ReLU layer. False, and nothing set, where this layer's
@@ -94,7 +97,7 @@ protected:
     bool q_out_only_ = false;
 
 private:
-    struct packed_entry { void* ptr; size_t bytes; unsigned long long last_use; };
+    struct packed_entry { void* ptr; size_t bytes; unsigned long long last_use; int pins = 0; };
     unsigned long long packed_clock_ = 0;
     std::map<std::vector<int>, packed_entry> packed_;
     std::shared_ptr<memory::tensor<float>> scale_dev_;

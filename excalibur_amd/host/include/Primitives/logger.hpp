@@ -40,6 +40,7 @@ private:
 #define CHECK_GE(a, b) CHECK_OP(a, b, >=)
 #define CHECK_GT(a, b) CHECK_OP(a, b, >)
 #define NOT_IMPLEMENTED LOG(FATAL) << "Not Implemented Yet"
+#define NO_GPU LOG(FATAL) << "This operator has no device code."
 #define NO_CPU LOG(FATAL) << "This backend computes on an MI355X only: construct the pipeline with device >= 0."
 #define DISABLE_COPY_AND_ASSIGN(classname) \
     classname(const classname&) = delete;  \

@@ -23,6 +23,8 @@ public:
 
     SyncedHead head() const { return head_; }
     size_t size() const { return size_; }
+    // counts the mutable_*_data() calls: a holder that remembers the value can tell whether the bytes may have changed since
+    unsigned long long writes() const { return writes_; }
     void set_allocator(pool_allocator<Dtype>*) {}
     const Dtype* cpu_data();
     const Dtype* gpu_data();
@@ -36,6 +38,7 @@ private:
     Dtype* gpu_ptr_ = nullptr;
     size_t size_;
     SyncedHead head_ = UNINITIALIZED;
+    unsigned long long writes_ = 0;
     int device_;
     int slot_;  // stream slot whose block cache gpu_ptr_ came from
     DISABLE_COPY_AND_ASSIGN(syncedmem);

@@ -29,6 +29,7 @@ public:
     const Dtype* gpu_data() const { return data_->gpu_data(); }
     Dtype* mutable_cpu_data() const { return data_->mutable_cpu_data(); }
     Dtype* mutable_gpu_data() const { return data_->mutable_gpu_data(); }
+    unsigned long long writes() const { return data_->writes(); }  // mutable_*_data() calls so far
     void copy_from(const void* data, size_t size);
 
     int num() const { return shape_[0]; }

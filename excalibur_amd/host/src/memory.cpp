@@ -171,9 +171,9 @@ const Dtype* syncedmem<Dtype>::cpu_data() { to_cpu(); return cpu_ptr_; }
 template <typename Dtype>
 const Dtype* syncedmem<Dtype>::gpu_data() { to_gpu(false); return gpu_ptr_; }
 template <typename Dtype>
-Dtype* syncedmem<Dtype>::mutable_cpu_data() { to_cpu(); head_ = HEAD_AT_CPU; return cpu_ptr_; }
+Dtype* syncedmem<Dtype>::mutable_cpu_data() { to_cpu(); head_ = HEAD_AT_CPU; ++writes_; return cpu_ptr_; }
 template <typename Dtype>
-Dtype* syncedmem<Dtype>::mutable_gpu_data() { to_gpu(true); head_ = HEAD_AT_GPU; return gpu_ptr_; }
+Dtype* syncedmem<Dtype>::mutable_gpu_data() { to_gpu(true); head_ = HEAD_AT_GPU; ++writes_; return gpu_ptr_; }
 
 template <typename Dtype>
 void tensor<Dtype>::init(const std::vector<int>& shape, int device) {

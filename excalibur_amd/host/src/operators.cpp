@@ -384,11 +384,16 @@ const void* operation_convolution<Dtype>::packed_weights(int dtype, const exhip_
         return it->second.ptr;
     }
     // One packed copy per input geometry, the few most recently used: a detector fed many resolutions would otherwise
-    // keep a copy of its weights for each. (A fused plan holds the pointers of its own geometry, always the latest.)
-    while (packed_.size() >= 4) {
-        auto oldest = packed_.begin();
-        for (auto jt = packed_.begin(); jt != packed_.end(); ++jt)
-            if (jt->second.last_use < oldest->second.last_use) oldest = jt;
+    // keep a copy of its weights for each. Copies a fused plan holds are pinned and stay.
+    for (;;) {
+        size_t loose = 0;
+        auto oldest = packed_.end();
+        for (auto jt = packed_.begin(); jt != packed_.end(); ++jt) {
+            if (jt->second.pins > 0) continue;
+            ++loose;
+            if (oldest == packed_.end() || jt->second.last_use < oldest->second.last_use) oldest = jt;
+        }
+        if (loose < 4) break;
         memory::device_release(this->params_.device_, oldest->second.ptr, oldest->second.bytes);
         packed_.erase(oldest);
     }
@@ -411,8 +416,22 @@ const void* operation_convolution<Dtype>::packed_weights(int dtype, const exhip_
     EXHIP_FATAL(exhip_conv_pack_weights(&d, dtype, src, host.data()));
     void* dev = memory::device_alloc(this->params_.device_, bytes);
     EXHIP_FATAL(exhip_memcpy_h2d(this->ctx(), dev, host.data(), bytes));
-    packed_[key] = {dev, bytes, ++packed_clock_};
+    packed_[key] = {dev, bytes, ++packed_clock_, 0};
     return dev;
+}
+
+template <typename Dtype>
+const void* operation_convolution<Dtype>::pin_packed_weights(int dtype, const exhip_conv_desc& d) {
+    const void* ptr = packed_weights(dtype, d);
+    for (auto& kv : packed_)
+        if (kv.second.ptr == ptr) ++kv.second.pins;
+    return ptr;
+}
+
+template <typename Dtype>
+void operation_convolution<Dtype>::unpin_packed_weights(const void* ptr) {
+    for (auto& kv : packed_)
+        if (kv.second.ptr == ptr && kv.second.pins > 0) --kv.second.pins;
 }
 
 template <typename Dtype>

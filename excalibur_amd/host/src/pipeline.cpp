@@ -62,6 +62,9 @@ public:
 
     impl() : device_(-1) {}  // the reference's default-constructed pipeline (pipeline.cpp:575-577): no layers; forward is fatal
 
+    // the plan lets go of the operators' packed weights: it goes first, while the operators still exist
+    ~impl() { plan_.reset(); }
+
     impl(const std::vector<std::string>& lines, std::string_view model_file, int device) : device_(device) {
         if (device >= 0) memory::device_context(device);  // opens the device, fatal if it is not an MI355X
         if (lines.empty()) LOG(FATAL) << "Incorrect param file.";
@@ -273,7 +276,9 @@ public:
     // A blob of the last forward by name, NCHW (nullptr for an unknown name, as in the reference). The fused executors
     // do not store every blob (a fused plan keeps int8 tensors between layers, a convolution absorbs the activation or
     // sum behind it, int8 readers get an int8 form only): asking for such a blob runs the last input once more through the
-    // per-layer executor with fusion off, which stores them all, so what comes back always belongs to the last input.
+    // per-layer executor with fusion off, which stores them all, so what comes back always belongs to the last input. If the
+    // caller has written to the input tensor since that forward, the rerun would mix two inputs' blobs: the request is
+    // refused (nullptr and an error line) until the next forward.
     tensor_ptr get_featmap(std::string_view name) {
         auto it = blob_index_.find(std::string(name));
         if (it == blob_index_.end()) return nullptr;
@@ -281,6 +286,11 @@ public:
             const tensor_ptr& t = featmaps_[it->second];
             return !t || (t->quantized && t->quantized->only);
         };
+        if (missing() && last_input_ && !all_blobs_stored_ && last_input_->writes() != last_input_writes_) {
+            LOG(ERROR) << name_ << ": blob " << name << " was not stored by the last forward and the input tensor has been written to since; "
+                       << "run forward again before asking for it";
+            return nullptr;
+        }
         if (missing() && last_input_ && !all_blobs_stored_) {
             const bool fusion = fusion_, fused = last_fused_;
             fusion_ = false;
@@ -331,6 +341,7 @@ private:
     blob_map forward_layers(const tensor_ptr& input) {
         last_fused_ = false;
         last_input_ = input;
+        last_input_writes_ = input->writes();
         all_blobs_stored_ = !fusion_;
         featmaps_[blob_index_[input_names_[0]]] = input;
         for (size_t i = 0; i < operations_.size(); ++i) {
@@ -403,6 +414,7 @@ private:
     std::vector<std::string> input_names_, output_names_;
     std::vector<tensor_ptr> featmaps_;
     tensor_ptr last_input_;           // for get_featmap of a blob the fused executors did not store
+    unsigned long long last_input_writes_ = 0;  // its write count when the last forward took it
     bool all_blobs_stored_ = false;   // the last forward was a per-layer one with fusion off
     struct post_activation {
         bool on = false, relu = false;
@@ -444,8 +456,10 @@ struct pipeline<Dtype>::impl::fused_plan {
     void* graph = nullptr;
     std::vector<float*> graph_slots;
     int forwards = 0;
+    std::vector<std::function<void()>> pinned;  // releases of the packed weight copies the launches point to
     ~fused_plan() {
         if (graph) exhip_graph_destroy(graph);
+        for (auto& release : pinned) release();
     }
     float** new_result(const std::vector<int>& shape, int device) {
         outputs.emplace_back();
@@ -637,7 +651,8 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                     if (!r.f32 || r.n != out.n || r.h != oh || r.w != ow || r.cs != ks) return give_up();
                     res = static_cast<const float*>(r.f32);
                 }
-                const void* wp = c->packed_weights(EXHIP_I8, d);
+                const void* wp = c->pin_packed_weights(EXHIP_I8, d);  // the launches below keep this pointer
+                plan->pinned.emplace_back([c, wp]() { c->unpin_packed_weights(wp); });
                 const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
                 const int8_t* x = static_cast<const int8_t*>(in.i8);
                 if (nd.pool_op >= 0) {
@@ -739,6 +754,7 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
     }
     plan_->input_ptr = input->gpu_data();
     last_input_ = input;
+    last_input_writes_ = input->writes();
     all_blobs_stored_ = false;
     for (tensor_ptr& t : featmaps_) t = nullptr;  // nothing of an earlier input stays readable
     featmaps_[blob_index_[input_names_[0]]] = input;

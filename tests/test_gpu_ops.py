@@ -612,6 +612,24 @@ def test_conv_split_reduction_int8_bit_exact(ctx, args, splits):
         assert np.array_equal(fused["i8"], port.quantize(z, fs_out).transpose(0, 2, 3, 1))
 
 
+def test_conv_split_reduction_many_tiles_equals_the_unsplit_launch(ctx):
+    """128 tiles x 2 groups each (8 x 512 x 20 x 20 -> 512, eight chunks): every accumulator and every output of the split
+    launch equals the unsplit launch's, which the tests above pin against the oracle. The forced split of three is clamped
+    to what the fixed scratch holds."""
+    from excalibur_amd import hip
+    case = cases.conv_i8_case(620, 8, 512, 20, 20, 512, 3, 1, 1, act=0)
+    hip.set_option("force_splits", 1)
+    try:
+        want = gpueval.conv_i8(ctx, case)
+        hip.set_option("force_splits", 3)
+        got = gpueval.conv_i8(ctx, case)
+    finally:
+        hip.set_option("force_splits", 0)
+    for name in ("acc", "nchw"):
+        bad = np.flatnonzero(got[name].ravel() != want[name].ravel())
+        assert bad.size == 0, f"{name}: first of {bad.size} mismatches at flat index {bad[0]}"
+
+
 def test_conv_split_reduction_float_within_tolerance(ctx, splits):
     """The benchmark set's single float32 layer (1 x 64 x 56 x 56 -> 64, 3x3, bias, ReLU: 13 tiles on 256 CUs) and a half
     layer: the parts are added in split order, so a launch gives the same bits every time, within 1e-4 / 2e-3 of the oracle."""

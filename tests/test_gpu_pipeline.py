@@ -82,7 +82,7 @@ def test_resnet18_topology_through_the_pipeline(fusion):
             assert np.array_equal(p.get("pool1"), blobs["pool1"])
             assert np.array_equal(p.get("l3b1_out"), blobs["l3b1_out"])
         # device time of the convolution launches of a fused forward (what the benchmark's roofline divides by)
-        p.time_fused_span(1)
+        p.time_fused_span(-2)  # from the first convolution's launch on, whether or not an input quantizer stands in front of it
         p.forward(x)
         ms, launches = p.last_span()
         assert (launches, ms > 0) == ((20, True) if fusion else (0, False))
