@@ -1067,6 +1067,8 @@ int launch_epi(exhip_ctx* ctx, const LeanParams& p, int grid) {
     switch (p.flags) {
     case E_Q | E_ACT | E_QNN: return launch<WRES, NAB, NWB, (E_Q | E_ACT | E_QNN)>(ctx, p, grid);
     case E_RES | E_F | E_Q | E_POST | E_QNN: return launch<WRES, NAB, NWB, (E_RES | E_F | E_Q | E_POST | E_QNN)>(ctx, p, grid);
+    case E_RES | E_Q | E_POST | E_QNN: return launch<WRES, NAB, NWB, (E_RES | E_Q | E_POST | E_QNN)>(ctx, p, grid);  // a block's end read by int8 layers only
+    case E_RES | E_NCHW | E_POST: return launch<WRES, NAB, NWB, (E_RES | E_NCHW | E_POST)>(ctx, p, grid);            // a network's last block
     default: return launch<WRES, NAB, NWB, -1>(ctx, p, grid);
     }
 }

@@ -101,6 +101,7 @@ __global__ __launch_bounds__(256, 3) void stem_conv_pool_kernel(const StemParams
         }
     }
     // staging: tile pixel v = tid + 256 i
+    const int spare_off = p.IH * p.IW * 4;  // the 16 spare bytes behind a tile buffer's pixels
     int l_rel[kNP], l_yx[kNP], l_lds[kNP];
     {
         const int IW = p.IW, npix = p.IH * IW;
@@ -110,7 +111,7 @@ __global__ __launch_bounds__(256, 3) void stem_conv_pool_kernel(const StemParams
             const bool ok = tid + 256 * i < npix;
             l_rel[i] = ok ? (iy * p.W + ix) * 4 : kOob;
             l_yx[i] = ok ? (iy | (ix << 16)) : -1;
-            l_lds[i] = ok ? (iy * IW + ix) * 4 : -1;
+            l_lds[i] = ok ? (iy * IW + ix) * 4 : spare_off;  // lanes past the tile write a spare word
             ix += p.adv_ix;
             iy += p.adv_iy;
             const int wrap = ix >= IW ? 1 : 0;
@@ -177,7 +178,7 @@ __global__ __launch_bounds__(256, 3) void stem_conv_pool_kernel(const StemParams
                 const int q = (int)__builtin_amdgcn_fmed3f(t + __builtin_copysignf(0.5f, t), -128.f, 127.f);
                 pix |= c == 3 ? (q << 24) : ((q & 0xff) << (8 * c));
             }
-            if (l_lds[i] >= 0) *reinterpret_cast<int*>(dst + l_lds[i]) = pix;
+            *reinterpret_cast<int*>(dst + l_lds[i]) = pix;
         }
     };
 
@@ -249,8 +250,9 @@ __global__ __launch_bounds__(256, 3) void stem_conv_pool_kernel(const StemParams
             }
         }
         {
-            char* const dst = lds_pool + (py * MPW + pc) * kPoolPixB + hh * 64;
+            // lanes outside the patch's pooled columns write a spare pixel behind the buffer (a branch per store costs more)
             const bool wr = pc < MPW && py < rows;
+            char* const dst = lds_pool + (wr ? (py * MPW + pc) * kPoolPixB : rows * MPW * kPoolPixB) + hh * 64;
 #pragma unroll
             for (int m = 0; m < 2; ++m)
 #pragma unroll
@@ -263,7 +265,7 @@ __global__ __launch_bounds__(256, 3) void stem_conv_pool_kernel(const StemParams
                         const int t = even > odd ? even : odd;
                         h[e] = t > next ? t : next;
                     }
-                    if (wr) *reinterpret_cast<v4i*>(dst + (m * 32 + e4 * 4) * 4) = h;
+                    *reinterpret_cast<v4i*>(dst + (m * 32 + e4 * 4) * 4) = h;
                 }
         }
         barrier();
@@ -367,7 +369,7 @@ extern "C" int exhip_stem_f32_conv_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_c
     p.IW = (2 * p.MPW) * 2 + 8;       // columns 0 .. 2 MPW, eight taps each (taps past KW meet zero weights)
     if (p.IH * p.IW > kNP * 256) return EXHIP_ERR_UNSUPPORTED;
     p.tile_b = (p.IH * p.IW * 4 + 16 + 15) / 16 * 16;  // a fragment read may run 8 bytes past the last pixel it needs
-    p.pool_b = (2 * p.MPH + 1) * p.MPW * kPoolPixB;
+    p.pool_b = ((2 * p.MPH + 1) * p.MPW + 1) * kPoolPixB;  // and one spare pixel
     p.tiles_x = (pool_ow + p.MPW - 1) / p.MPW;
     const int tiles_y = (pool_oh + p.MPH - 1) / p.MPH;
     p.tiles_xy = p.tiles_x * tiles_y;
@@ -385,7 +387,7 @@ extern "C" int exhip_stem_f32_conv_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_c
     p.adv_iy = 256 / p.IW; p.adv_ix = 256 % p.IW;
     p.fs_in = fs_in; p.fs_out = d->fs_out;
     p.act = d->act; p.q_nonneg = d->fs_out > 0.f && d->act == 1;
-    const int lds = d->kh * 2048 + 2 * p.tile_b + p.pool_b;  // 53264 bytes for a 7x7 filter: three groups per CU
+    const int lds = d->kh * 2048 + 2 * p.tile_b + p.pool_b;  // 53536 bytes for a 7x7 filter: three groups per CU
     const long long total = n_ptiles * p.ktiles;
     long long G = total;
     if (total > 3 * 256) {
