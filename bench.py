@@ -440,7 +440,7 @@ def main():
                                                       f"different forwards overlap, none is shortened"},
                    "int8_tops_whole_step": round(conv_gop / ms_per_step, 1)},
         "roofline": {"bound": "mfma", "kernel": "the int8 convolution launches of a step (stem_conv_pool_kernel, conv3x3_i8_lean_kernel, "
-                                                 "conv_igemm_kernel: 20 launches)",
+                                                 f"conv_igemm_kernel: {n_conv} launches for the 20 convolutions)",
                      "achieved": round(achieved_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(achieved_tops / PEAK_INT8_TOPS, 4), "traffic": measured_traffic(n, hw),
                      "algorithmic_gop_per_step": round(conv_gop, 1), "avg_launch_ms": round(conv_ms / n_conv, 4),

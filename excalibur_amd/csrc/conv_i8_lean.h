@@ -12,8 +12,20 @@ struct exhip_lean_geom {
     float fs_out;                        // scale of the int8 output
 };
 
+// A 1x1 convolution of another int8 tensor (stride 1 or 2, no padding, no activation) whose float32 result is the
+// shortcut the 3x3 layer adds: a residual block's projection. The kernel accumulates it beside the 3x3 products, from
+// the pixels under the patch, and adds it in the epilogue in place of a shortcut tensor read from memory.
+struct exhip_lean_proj {
+    const int8_t* x;       // NHWC int8, h x w pixels of c_bytes bytes (a multiple of 64); output pixel (y, x) reads (y * stride, x * stride)
+    const void* wp;        // the 1x1 layer's packed weights: 64-channel slabs, 64-byte chunks (4 KiB per slab and chunk)
+    const float* scale;
+    const float* bias;     // may be NULL
+    int h, w, c_bytes, stride;
+};
+
 // Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then
 // runs the general kernel), another code on failure. Weights are the general kernel's packing for 64-channel slabs and
 // 64-byte channel chunks.
 int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
-                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw);
+                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw,
+                          const exhip_lean_proj* proj = nullptr);

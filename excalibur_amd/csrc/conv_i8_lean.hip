@@ -66,6 +66,13 @@ struct LeanParams {
     int adv_iy, adv_ix;  // (256 / 5) / IW, (256 / 5) % IW: how a thread's tile pixel advances from one staging load to the next
     float fs_out;
     int flags;
+    // projection shortcut (kernels instantiated with PROJ): a 1x1 convolution of ds_x accumulated beside the 3x3 products
+    const char* ds_x;
+    const char* ds_wp;
+    const float* ds_scale;
+    const float* ds_bias;
+    int ds_H, ds_W, ds_Cb, ds_chunks, ds_stride;
+    unsigned ds_img_bytes;
     int stagger;     // persistent launches: a group whose waves sit in hardware wave slot s starts s * stagger * 64 cycles late
     long long* dbg;  // phase timestamps (builds with -DEXHIP_STAMPS=1 only)
 };
@@ -108,14 +115,31 @@ __device__ __forceinline__ void half_swap4(v4i& a, v4i& b) {
     }
 }
 
+// Stores reach full speed with runs of 64 contiguous bytes from neighbouring lanes (measured: 32-byte runs take twice as
+// long), so two pixels in neighbouring lanes trade halves: afterwards `a` holds, in the even lane, its own a and, in the
+// odd lane, the even lane's c; `c` holds the odd lane's a and, in the odd lane, its own c. (DPP quad_perm [1, 0, 3, 2].)
+__device__ __forceinline__ int lane_neighbour(int v) { return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true); }
+__device__ __forceinline__ void pair_exchange4(v4i& a, v4i& c, bool odd) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int from_c = lane_neighbour(c[e]), from_a = lane_neighbour(a[e]);
+        const int a2 = odd ? from_c : a[e], c2 = odd ? c[e] : from_a;
+        a[e] = a2;
+        c[e] = c2;
+    }
+}
+
 // WRES: the slab's whole filter is resident (one 64-byte chunk); otherwise weight slices rotate through NWB buffers and
 // activation tiles through NAB. EPI >= 0: the epilogue's switches as compile-time constants; EPI < 0: read from p.flags.
-template <bool WRES, int NAB, int NWB, int EPI>
-__global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) void conv3x3_i8_lean_kernel(const LeanParams p) {
+// PROJ: the shortcut is a 1x1 convolution computed here (p.ds_*): its channel chunks follow the 3x3 layer's in every patch's
+// run as stages of one tap, into accumulators of their own.
+template <bool WRES, int NAB, int NWB, int EPI, bool PROJ = false>
+__global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 2 : 3) void conv3x3_i8_lean_kernel(const LeanParams p) {
+    static_assert(!(PROJ && WRES), "the projection's chunks run in the streamed form");
     constexpr int NWS = WRES ? 3 : NWB;
     constexpr int A0 = NWS * kWSlice;
     constexpr int SB0 = A0 + NAB * kActStride;
-    constexpr int SPARE0 = SB0 + kSbB;
+    constexpr int SPARE0 = SB0 + (PROJ ? 2 * kSbB : kSbB);
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     float* const lds_sb = reinterpret_cast<float*>(smem + SB0);
@@ -131,9 +155,14 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     auto now = [&]() -> long long { return kStamps && p.dbg ? (long long)clock64() : 0ll; };
     auto put = [&](int k, long long v) {
         if constexpr (kStamps)
-            if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * 4 + wave) * 16 + k] = v;
+            if (p.dbg && lane == 0) p.dbg[((size_t)blockIdx.x * 4 + wave) * 64 + k] = v;
     };
     put(0, now());
+    if constexpr (kStamps) {
+        put(16, __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | ((32 - 1) << 11)));   // HW_REG_HW_ID
+        put(17, __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | ((32 - 1) << 11)));  // HW_REG_XCC_ID
+    }
+    int n_epi = 0;
     if (p.stagger > 0) {
         // Groups that share a CU start together and would reach their MFMA runs, waits and epilogues together, the matrix
         // pipes idle in between. The hardware wave slot (HW_ID bits 3:0) counts the waves a SIMD already holds: delaying a
@@ -193,13 +222,17 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     const int img_px = p.OH * p.OW;
 
     v16i acc[2][2];
+    v16i acc_ds[2][2];  // PROJ: the projection's products
     auto clear_acc = [&]() {
 #pragma unroll
         for (int m = 0; m < 2; ++m)
 #pragma unroll
             for (int nn = 0; nn < 2; ++nn)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) acc[m][nn][e] = 0;
+                for (int e = 0; e < 16; ++e) {
+                    acc[m][nn][e] = 0;
+                    if constexpr (PROJ) acc_ds[m][nn][e] = 0;
+                }
     };
 
     // ---- patch bookkeeping (all wave-uniform) ----
@@ -211,8 +244,25 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
         ox0 = tx * p.PW;
     };
     // gather offsets of a patch's staging loads; returns what goes into the buffer view's base instead
+    const int part0 = tid - fast_div(tid, 0x33333334u) * 5;   // the 16-byte part of a pixel this thread's first slot holds
+    auto part_of = [&](int i) {
+        int part = part0 + i;
+        part -= part >= 5 ? 5 : 0;
+        part -= part >= 5 ? 5 : 0;
+        return part;
+    };
     auto set_offsets = [&](int oy0, int ox0) -> int {
         const int iy0 = oy0 - p.PT, ix0 = ox0 - p.PL;
+        if constexpr (PROJ) {
+            // two accumulator sets leave no registers for the patch-relative offsets: made from the pixel positions
+#pragma unroll
+            for (int i = 0; i < kNAL; ++i) {
+                const int gy = iy0 + (a_yx[i] & 0xFFFF), gx = ix0 + (int)((unsigned)a_yx[i] >> 16);
+                const bool in = ((unsigned)gy < (unsigned)p.H) & ((unsigned)gx < (unsigned)p.W);
+                a_off[i] = in ? (gy * p.W + gx) * p.C_b + part_of(i) * 16 : kOob;
+            }
+            return 0;
+        }
         const int tile_base = (iy0 * p.W + ix0) * p.C_b;
         const bool interior = iy0 >= 0 && ix0 >= 0 && iy0 + p.IH <= p.H && ix0 + p.IW <= p.W;
         if (interior) {
@@ -234,15 +284,38 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     const int w_voff = tid * 16;
     const char* const wkt = p.wp + (size_t)kt * p.n_chunks * (3 * kWSlice);  // this slab's slices, in (chunk, filter row) order
     const int w_run_b = p.n_chunks * 3 * kWSlice;
+    const int n_tot = p.n_chunks + (PROJ ? p.ds_chunks : 0);   // chunks of a patch's run: the 3x3 layer's, then the projection's
     int w_off = 0;                                  // next slice to request
-    int w_left = my_tiles * p.n_chunks * 3;         // slices of the whole run not requested yet
+    int w_left = my_tiles * n_tot * 3;              // slices of the whole run not requested yet
+    // PROJ: behind the 3x3 layer's slices a patch's run takes three per projection chunk, to keep every stage's requests
+    // alike: the chunk's one tap (4 KiB of the 1x1 layer's packed weights, slab kt) and two empty ones
+    const char* const wkt_ds = PROJ ? p.ds_wp + (size_t)kt * p.ds_chunks * 4096 : nullptr;
+    int w_ds = -1;                                  // >= 0: the next slice is number w_ds of the projection's
     auto request_w = [&](unsigned dst) {
-        const __amdgpu_buffer_rsrc_t wr = uniform_view(wkt + w_off, w_left > 0 ? kWSlice : 0);
+        const char* src = wkt + w_off;
+        int range = kWSlice;
+        if constexpr (PROJ) {
+            if (w_ds >= 0) {
+                const int dc = w_ds / 3;
+                src = wkt_ds + dc * 4096;
+                range = w_ds == dc * 3 ? 4096 : 0;
+            }
+        }
+        const __amdgpu_buffer_rsrc_t wr = uniform_view(src, w_left > 0 ? range : 0);
 #pragma unroll
         for (int i = 0; i < 3; ++i) async_load16(wr, w_voff, i * 4096, dst + wave_slot + i * 4096);
         --w_left;
+        if constexpr (PROJ) {
+            if (w_ds >= 0) {
+                if (++w_ds == p.ds_chunks * 3) w_ds = -1;
+                return;
+            }
+        }
         w_off += kWSlice;
-        if (w_off == w_run_b) w_off = 0;
+        if (w_off == w_run_b) {
+            w_off = 0;
+            if constexpr (PROJ) w_ds = 0;
+        }
     };
     auto request_a = [&](const char* img, int base, int cc, bool valid, unsigned dst) {
         const int off = base + cc * 64;
@@ -252,6 +325,23 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
             unsigned d = dst + wave_slot + i * 4096;
             if (i == kNAL - 1) d = wave == 3 ? lds0 + SPARE0 : d;  // the KiB past the buffer
             async_load16(xr, a_off[i], 0, d);
+        }
+    };
+    // PROJ: chunk dc of the projection's input under the patch at (oy0, ox0) of image n, in the 3x3 layer's tile geometry
+    // (tile pixel (y, x) is the pixel under output (oy0 - PT + y, ox0 - PL + x)): the tap reads where the 3x3 layer's
+    // centre tap does
+    auto request_ds = [&](int n, int oy0, int ox0, int dc, unsigned dst) {
+        const int off0 = dc * 64;
+        const __amdgpu_buffer_rsrc_t xr = uniform_view(p.ds_x + (size_t)n * p.ds_img_bytes + off0, (int)p.ds_img_bytes - off0);
+        const int y0 = (oy0 - p.PT) * p.ds_stride, x0 = (ox0 - p.PL) * p.ds_stride;
+#pragma unroll
+        for (int i = 0; i < kNAL; ++i) {
+            unsigned d = dst + wave_slot + i * 4096;
+            if (i == kNAL - 1) d = wave == 3 ? lds0 + SPARE0 : d;
+            const int part = part_of(i);
+            const int gy = y0 + (a_yx[i] & 0xFFFF) * p.ds_stride, gx = x0 + (int)((unsigned)a_yx[i] >> 16) * p.ds_stride;
+            const bool in = (a_yx[i] >= 0) & ((unsigned)gy < (unsigned)p.ds_H) & ((unsigned)gx < (unsigned)p.ds_W);
+            async_load16(xr, in ? (gy * p.ds_W + gx) * p.ds_Cb + part * 16 : kOob, 0, d);
         }
     };
 
@@ -289,6 +379,22 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
             }
         }
     };
+    // PROJ: a projection chunk's two k-steps, on the pixels the 3x3 layer's centre tap reads
+    auto mfma_ds = [&](const char* wrow, const char* a0c, const char* a1c) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            af[s][0] = lds_read16(wrow + s * 2048);
+            af[s][1] = lds_read16(wrow + s * 2048 + 1024);
+            bf[s][0] = lds_read16(a0c + s * 32);
+            bf[s][1] = lds_read16(a1c + s * 32);
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int nn = 0; nn < 2; ++nn) acc_ds[m][nn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[s][m], bf[s][nn], acc_ds[m][nn], 0, 0, 0);
+    };
     constexpr std::integral_constant<int, 1> one_row{};
     constexpr std::integral_constant<int, 3> three_rows{};
 
@@ -302,11 +408,19 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     auto epilogue = [&](int n, int oy0, int ox0) {
         const bool full = oy0 + p.PH <= p.OH && ox0 + p.PW <= p.OW;
         const unsigned obase = ((unsigned)n * (unsigned)img_px + (unsigned)(oy0 * p.OW + ox0)) * (unsigned)p.K + (unsigned)(kt * 64);
-        unsigned eoff[2], noff[2];
+        unsigned eoff[2], noff[2], feven[2], fodd[2];
+        const bool odd_lane = lane & 1;
 #pragma unroll
         for (int nn = 0; nn < 2; ++nn) {
             const bool valid = full ? o_y[nn] < 0x4000 : ((oy0 + o_y[nn] < p.OH) & (ox0 + o_x[nn] < p.OW));
             eoff[nn] = valid ? obase + (unsigned)o_rel[nn] : kOobElem;
+            if (has_f) {
+                // float32 rows leave in 64-byte runs that a lane pair and its neighbour pair form: the even pixel's
+                // runs in one store, the odd pixel's in the next
+                const unsigned other = (unsigned)lane_neighbour((int)eoff[nn]);
+                feven[nn] = (odd_lane ? other : eoff[nn]) * 4u + (odd_lane ? 32u : 0u) + hh * 16;
+                fodd[nn] = (odd_lane ? eoff[nn] : other) * 4u + (odd_lane ? 32u : 0u) + hh * 16;
+            }
             if (has_nchw) {
                 const unsigned e = ((unsigned)n * (unsigned)p.K + (unsigned)(kt * 64 + hh * 16)) * (unsigned)img_px +
                                    (unsigned)((oy0 + o_y[nn]) * p.OW + ox0 + o_x[nn]);
@@ -363,8 +477,15 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
                     v4f v;
+                    if constexpr (PROJ) {  // read where used: the arrays above would not fit beside two accumulator sets
+                        const v4f sc = *reinterpret_cast<const v4f*>(lds_sb + m * 32 + hh * 16 + e4 * 4);
+                        const v4f bi = *reinterpret_cast<const v4f*>(lds_sb + 64 + m * 32 + hh * 16 + e4 * 4);
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e4][e], b4[e4][e]);
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], sc[e], bi[e]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaf((float)acc[m][nn][e4 * 4 + e], s4[e4][e], b4[e4][e]);
+                    }
                     if (act_relu) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
@@ -373,6 +494,13 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                         const v4f rv = __builtin_bit_cast(v4f, r4[e4]);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] += rv[e];
+                    }
+                    if constexpr (PROJ) {
+                        // the value the 1x1 layer would have stored (no activation), added as the shortcut
+                        const v4f sd = *reinterpret_cast<const v4f*>(lds_sb + 128 + m * 32 + hh * 16 + e4 * 4);
+                        const v4f bd = *reinterpret_cast<const v4f*>(lds_sb + 192 + m * 32 + hh * 16 + e4 * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += __builtin_fmaf((float)acc_ds[m][nn][e4 * 4 + e], sd[e], bd[e]);
                     }
                     if (post_relu) {
 #pragma unroll
@@ -403,11 +531,15 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                     }
                 }
                 if (has_f) {
+                    // o4[0], o4[2]: channels 0-7 and 8-15 of the block's 32; o4[1], o4[3]: 16-23 and 24-31
                     half_swap4(o4[0], o4[1]);
                     half_swap4(o4[2], o4[3]);
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        __builtin_amdgcn_raw_buffer_store_b128(o4[j], rf, (int)(eoff[nn] * 4u + hh * 16 + m * 128 + piece(j)), 0, 0);
+                    pair_exchange4(o4[0], o4[2], odd_lane);
+                    pair_exchange4(o4[1], o4[3], odd_lane);
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[0], rf, (int)(feven[nn] + m * 128), 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[1], rf, (int)(feven[nn] + m * 128 + 64), 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[2], rf, (int)(fodd[nn] + m * 128), 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[3], rf, (int)(fodd[nn] + m * 128 + 64), 0, 0);
                 }
                 if (has_q) __builtin_amdgcn_raw_buffer_store_b128(q4, rq, (int)(eoff[nn] + hh * 16 + m * 32), 0, 0);
             }
@@ -426,6 +558,9 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
     if (tid < 128) {
         const int ch = kt * 64 + (tid & 63);
         lds_sb[tid] = tid < 64 ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
+    } else if (PROJ) {
+        const int ch = kt * 64 + (tid & 63);
+        lds_sb[tid] = tid < 192 ? p.ds_scale[ch] : (p.ds_bias ? p.ds_bias[ch] : 0.f);
     }
     clear_acc();
 
@@ -455,7 +590,9 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                 request_a(img, base, 0, true, lds0 + A0);
             }
             { const long long t = now(); t_gap += t - t_mark; t_mark = t; }
+            if (kStamps && n_epi < 20) put(18 + 2 * n_epi, (long long)clock64());
             epilogue(n, oy0, ox0);
+            if (kStamps && n_epi < 20) { put(19 + 2 * n_epi, (long long)clock64()); ++n_epi; }
             { const long long t = now(); t_epi += t - t_mark; t_mark = t; }
             if (!has_next) break;
             clear_acc();
@@ -484,8 +621,9 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
         int nn_ = n, ny = oy0, nx = ox0;
         for (int done = 0;;) {
             const bool has_next = done + 1 < my_tiles;
-            for (int cc = 0; cc < p.n_chunks; ++cc) {
-                const bool last_cc = cc + 1 == p.n_chunks;
+            for (int cc = 0; cc < n_tot; ++cc) {
+                const bool last_cc = cc + 1 == n_tot;
+                const bool proj_cc = PROJ && cc >= p.n_chunks;   // a chunk of the projection: one tap, in the first stage
                 // what the next chunk's tile request asks for: the next chunk of this patch, or the next patch's first
                 auto request_next_a = [&](unsigned dst) {
                     if (last_cc) {
@@ -496,8 +634,19 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                             base = set_offsets(ny, nx);
                         }
                         request_a(img, base, 0, has_next, dst);
+                    } else if (PROJ && cc + 1 >= p.n_chunks) {
+                        request_ds(n, oy0, ox0, cc + 1 - p.n_chunks, dst);
                     } else {
                         request_a(img, base, cc + 1, true, dst);
+                    }
+                };
+                // one stage: a filter row of a 3x3 chunk, or (first stage only) the tap of a projection chunk
+                auto stage = [&](int r, const char* w, const char* a0r, const char* a1r, auto&& requests) {
+                    if (!proj_cc) {
+                        mfma_rows(one_row, w, a0r, a1r, requests);
+                    } else {
+                        if (r == 0) mfma_ds(w, a0r + row_b + kPixB, a1r + row_b + kPixB);
+                        requests();
                     }
                 };
                 const char* const ab = smem + A0 + (NAB == 2 ? abuf * kActStride : 0);
@@ -505,7 +654,7 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                 const char* const a1 = ab + boff[1];
                 const unsigned a_other = lds0 + A0 + (NAB == 2 ? (1 - abuf) * kActStride : 0);
                 if constexpr (NWB == 3) {
-                    mfma_rows(one_row, smem + lane * 16, a0, a1, [&]() {
+                    stage(0, smem + lane * 16, a0, a1, [&]() {
                         request_w(lds0 + 2 * kWSlice);
                         if constexpr (NAB == 2) request_next_a(a_other);
                     });
@@ -514,20 +663,20 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                     { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
                     { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
-                    mfma_rows(one_row, smem + kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0); });
+                    stage(1, smem + kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0); });
                     { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait1>();
                     { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
                     { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
-                    mfma_rows(one_row, smem + 2 * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b, [&]() { request_w(lds0 + kWSlice); });
+                    stage(2, smem + 2 * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b, [&]() { request_w(lds0 + kWSlice); });
                     { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait2>();
                     { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
                     { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                 } else {
-                    mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0, a1, [&]() {
+                    stage(0, smem + wbuf * kWSlice + lane * 16, a0, a1, [&]() {
                         request_w(lds0 + (1 - wbuf) * kWSlice);
                         if constexpr (NAB == 2) request_next_a(a_other);
                     });
@@ -537,15 +686,15 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                     __syncthreads();
                     { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                     wbuf = 1 - wbuf;
-                    mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
+                    stage(1, smem + wbuf * kWSlice + lane * 16, a0 + row_b, a1 + row_b, [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
                     { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait1>();
                     { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
                     __syncthreads();
                     { const long long t = now(); t_bar += t - t_mark; t_mark = t; }
                     wbuf = 1 - wbuf;
-                    mfma_rows(one_row, smem + wbuf * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b,
-                              [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
+                    stage(2, smem + wbuf * kWSlice + lane * 16, a0 + 2 * row_b, a1 + 2 * row_b,
+                          [&]() { request_w(lds0 + (1 - wbuf) * kWSlice); });
                     { const long long t = now(); t_mfma += t - t_mark; t_mark = t; }
                     wait_vmcnt<kWait2>();
                     { const long long t = now(); t_wait += t - t_mark; t_mark = t; }
@@ -566,7 +715,9 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3) ? 2 : 3) v
                     { const long long t = now(); t_gap += t - t_mark; t_mark = t; }
                 }
             }
+            if (kStamps && n_epi < 20) put(18 + 2 * n_epi, (long long)clock64());
             epilogue(n, oy0, ox0);
+            if (kStamps && n_epi < 20) { put(19 + 2 * n_epi, (long long)clock64()); ++n_epi; }
             { const long long t = now(); t_epi += t - t_mark; t_mark = t; }
             if (!has_next) break;
             ++done;
@@ -1044,11 +1195,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 std::mutex g_attr_mutex;
 
-template <bool WRES, int NAB, int NWB, int EPI>
+template <bool WRES, int NAB, int NWB, int EPI, bool PROJ = false>
 int launch(exhip_ctx* ctx, const LeanParams& p, int grid) {
-    constexpr int lds = ((WRES ? 3 : NWB) * kWSlice) + NAB * kActStride + kSbB + kSpareB;
+    constexpr int lds = ((WRES ? 3 : NWB) * kWSlice) + NAB * kActStride + (PROJ ? 2 * kSbB : kSbB) + kSpareB;
     static unsigned long long attr_set = 0;
-    auto kernel = conv3x3_i8_lean_kernel<WRES, NAB, NWB, EPI>;
+    auto kernel = conv3x3_i8_lean_kernel<WRES, NAB, NWB, EPI, PROJ>;
     {
         std::lock_guard<std::mutex> lock(g_attr_mutex);
         const unsigned long long bit = 1ull << (ctx->device & 63);
@@ -1108,10 +1259,25 @@ extern "C" void exhip_dev_lean_stamps(void* device_buffer) { g_lean_dbg = (long 
 #endif
 
 int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
-                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw) {
+                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw,
+                          const exhip_lean_proj* proj) {
     int mode = g_exhip_options.lean;
     if (mode == 0) return EXHIP_ERR_UNSUPPORTED;
+    if (proj) {
+        // the projection's chunks ride along the persistent streamed form; the shortcut is computed, not read
+        if (residual || y_nchw || !y_f || !y_q || !g.post_relu || g.act != 0 || !(g.fs_out > 0.f)) return EXHIP_ERR_UNSUPPORTED;
+        if (!proj->x || !proj->wp || !proj->scale || proj->c_bytes % 64 != 0 || proj->c_bytes <= 0 || (proj->stride != 1 && proj->stride != 2) ||
+            (proj->h - 1) / proj->stride + 1 != g.oh || (proj->w - 1) / proj->stride + 1 != g.ow || g.oh != g.h || g.ow != g.w ||
+            proj->h >= 0x4000 || proj->w >= 0x4000 || (long long)proj->h * proj->w * proj->c_bytes >= 0x7FFFFF00ll)
+            return EXHIP_ERR_UNSUPPORTED;
+    }
     int cfg = g_exhip_options.lean_cfg;  // 0: one tile buffer, two slice buffers; 1: two and two; 2: one and three
+    if (proj) {
+        // two groups per CU (two accumulator sets); as with a shortcut tensor, two tile buffers up to 256 channels,
+        // three slice buffers beyond
+        if (mode != 1 || cfg == 0) cfg = g.c_bytes / 64 <= 4 ? 1 : 2;
+        mode = 1;
+    }
     if (mode == 4) {
         // The form that measured fastest per layer class on the ResNet-18-shaped stack at 32 x 640 x 640: without a shortcut
         // the resident filter (64 channels) or one group per patch with three groups per CU; with a shortcut, whose float32
@@ -1148,6 +1314,11 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
     p.fs_out = g.fs_out;
     p.dbg = g_lean_dbg;
     p.stagger = g_exhip_options.lean_stagger;
+    if (proj) {
+        p.ds_x = (const char*)proj->x; p.ds_wp = (const char*)proj->wp; p.ds_scale = proj->scale; p.ds_bias = proj->bias;
+        p.ds_H = proj->h; p.ds_W = proj->w; p.ds_Cb = proj->c_bytes; p.ds_chunks = proj->c_bytes / 64; p.ds_stride = proj->stride;
+        p.ds_img_bytes = (unsigned)((size_t)proj->h * proj->w * proj->c_bytes);
+    }
     const bool q_nonneg = g.fs_out > 0.f && (g.post_relu || (g.act == 1 && !residual));
     p.flags = (residual ? E_RES : 0) | (y_f ? E_F : 0) | (y_q ? E_Q : 0) | (y_nchw ? E_NCHW : 0) | (g.act == 1 ? E_ACT : 0) |
               (g.post_relu ? E_POST : 0) | (q_nonneg ? E_QNN : 0);
@@ -1166,7 +1337,7 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
         return launch_ws_epi<false>(ctx, p, (int)G);
     }
     // groups: as many as stay resident (persistent), or one per patch and slab (mode 2)
-    const bool wres = p.n_chunks == 1 && g_exhip_options.lean_wres != 0;
+    const bool wres = p.n_chunks == 1 && g_exhip_options.lean_wres != 0 && !proj;
     const int per_cu = wres ? 2 : (cfg == 0 ? 3 : 2);
     const long long total = n_ptiles * g.ktiles;
     long long G = total;
@@ -1180,6 +1351,12 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
     if (g_exhip_options.debug_plan)
         fprintf(stderr, "  lean: %s cfg %d, %lld groups for %lld tiles, flags %d\n", wres ? "resident filter" : "streamed filter", cfg, G, total,
                 p.flags);
+    if (proj) {
+        constexpr int epi = E_F | E_Q | E_POST | E_QNN;
+        if (p.flags != epi) return EXHIP_ERR_UNSUPPORTED;
+        if (cfg == 1) return launch<false, 2, 2, epi, true>(ctx, p, (int)G);
+        return launch<false, 1, 3, epi, true>(ctx, p, (int)G);
+    }
     if (wres) return launch_epi<true, 1, 2>(ctx, p, (int)G);
     if (cfg == 1) return launch_epi<false, 2, 2>(ctx, p, (int)G);
     if (cfg == 2) return launch_epi<false, 1, 3>(ctx, p, (int)G);

@@ -1580,7 +1580,7 @@ void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3
 }
 
 template <int DT>
-int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolSpec* pool = nullptr) {
+int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolSpec* pool = nullptr, const exhip_lean_proj* proj = nullptr) {
     EXHIP_REQUIRE(ctx, "conv: NULL ctx");
     Plan pl;
     int rc = make_plan(d, DT, &pl, pool);
@@ -1676,9 +1676,10 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             g.tiles_x = pl.tiles_x; g.tiles_y = pl.tiles_y; g.ktiles = pl.ktiles;
             g.act = d->act; g.post_relu = d->post_relu; g.fs_out = d->fs_out;
             rc = exhip_conv3x3_i8_lean(ctx, g, reinterpret_cast<const int8_t*>(p.x), p.wp, p.scale, p.bias, reinterpret_cast<const float*>(p.residual),
-                                       reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc), reinterpret_cast<float*>(p.y_nchw));
-            if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
+                                       reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc), reinterpret_cast<float*>(p.y_nchw), proj);
+            if (rc != EXHIP_ERR_UNSUPPORTED || proj) return rc;
         }
+        if (proj) return EXHIP_ERR_UNSUPPORTED;  // only the lean kernel computes a projection beside its own products
         if (fused) {
             p.epi_mode = 1;
             p.epi_f = p.residual || p.y_nhwc;
@@ -1768,6 +1769,36 @@ extern "C" int exhip_conv2d_i8(exhip_ctx* ctx, const exhip_conv_desc* d, const i
     p.x = (const char*)x; p.wp = (const char*)wp; p.scale = scale; p.bias = bias; p.residual = residual;
     p.y_q = y_i8; p.y_nhwc = y_f32_nhwc; p.y_nchw = y_f32_nchw; p.acc_nchw = acc_nchw;
     return run_conv<EXHIP_I8>(ctx, d, p);
+}
+
+// A residual block's second convolution with the block's projection shortcut computed in the same kernel: what
+// exhip_conv2d_i8 would do for the 1x1 layer (float32 result, no activation) and then for the 3x3 layer with that result
+// as `residual`, without the float32 tensor between them. EXHIP_ERR_UNSUPPORTED (and nothing launched) outside the
+// shapes the lean kernel takes; the caller then issues the two calls.
+extern "C" int exhip_conv2d_i8_projection(exhip_ctx* ctx, const exhip_conv_desc* d, const int8_t* x, const void* wp, const float* scale,
+                                          const float* bias, const exhip_conv_desc* d_proj, const int8_t* x_proj, const void* wp_proj,
+                                          const float* scale_proj, const float* bias_proj, int8_t* y_i8, float* y_f32_nhwc) {
+    EXHIP_REQUIRE(d && d_proj && scale && scale_proj && x_proj && wp_proj, "exhip_conv2d_i8_projection: NULL argument");
+    EXHIP_REQUIRE(y_i8 && y_f32_nhwc, "exhip_conv2d_i8_projection: both outputs are required");
+    if (d->kh != 3 || d->kw != 3 || d->sh != 1 || d->sw != 1 || d->act != 0 || !d->post_relu || d->post_op || !(d->fs_out > 0.f) ||
+        d->k % 64 != 0 || d->k_stride != d->k)
+        return EXHIP_ERR_UNSUPPORTED;
+    if (d_proj->kh != 1 || d_proj->kw != 1 || d_proj->sh != d_proj->sw || (d_proj->sh != 1 && d_proj->sh != 2) || d_proj->pt || d_proj->pb ||
+        d_proj->pl || d_proj->pr || d_proj->act != 0 || d_proj->post_relu || d_proj->post_op || d_proj->k != d->k || d_proj->n != d->n ||
+        d_proj->c_stride % 64 != 0 || d_proj->c_stride != d_proj->c)
+        return EXHIP_ERR_UNSUPPORTED;
+    // the 1x1 layer's packed weights must be the 64-channel-slab, 64-byte-chunk form: 4 KiB per slab and chunk
+    Plan pp;
+    int rc = make_plan(d_proj, EXHIP_I8, &pp);
+    if (rc) return rc;
+    if (pp.packed || pp.TM != 64 || pp.chunk_b != 64 || pp.KWe != 1 || pp.KS != 2 || pp.n_chunks != d_proj->c_stride / 64) return EXHIP_ERR_UNSUPPORTED;
+    exhip_lean_proj proj = {};
+    proj.x = x_proj; proj.wp = wp_proj; proj.scale = scale_proj; proj.bias = bias_proj;
+    proj.h = d_proj->h; proj.w = d_proj->w; proj.c_bytes = d_proj->c_stride; proj.stride = d_proj->sh;
+    ConvParams p = {};
+    p.x = (const char*)x; p.wp = (const char*)wp; p.scale = scale; p.bias = bias;
+    p.y_q = y_i8; p.y_nhwc = y_f32_nhwc;
+    return run_conv<EXHIP_I8>(ctx, d, p, nullptr, &proj);
 }
 
 extern "C" int exhip_conv2d_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_desc* d, int pool_pt, int pool_pl, int pool_oh,

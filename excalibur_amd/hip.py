@@ -233,6 +233,15 @@ class Ctx:
         _check(rc)
         return True
 
+    def conv2d_i8_projection(self, d, x, wp, scale, bias, d_proj, x_proj, wp_proj, scale_proj, bias_proj, y_i8, y_f32_nhwc):
+        """Returns False when the library leaves the pair to two exhip_conv2d_i8 calls."""
+        rc = lib().exhip_conv2d_i8_projection(self.h, ctypes.byref(d), x.ptr, wp.ptr, scale.ptr, _ptr(bias), ctypes.byref(d_proj),
+                                              x_proj.ptr, wp_proj.ptr, scale_proj.ptr, _ptr(bias_proj), y_i8.ptr, y_f32_nhwc.ptr)
+        if rc == 10002:
+            return False
+        _check(rc)
+        return True
+
     def conv2d_f16(self, d, x, wp, bias=None, residual=None, y_f16_nhwc=None, y_f16_nchw=None, y_f32_nchw=None):
         _check(lib().exhip_conv2d_f16(self.h, ctypes.byref(d), x.ptr, wp.ptr, _ptr(bias), _ptr(residual), _ptr(y_f16_nhwc),
                                       _ptr(y_f16_nchw), _ptr(y_f32_nchw)))

@@ -625,6 +625,22 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
             });
             plan->first_conv_launch = 1;
         }
+        // A block's projection shortcut (a 1x1 convolution without activation whose result only the block's sum reads) is
+        // held back until the convolution that absorbs the sum is planned: exhip_conv2d_i8_projection computes it in that
+        // convolution's kernel and its float32 tensor never exists. Where the library declines, the projection is
+        // launched on its own right before that convolution.
+        struct pending_projection {
+            exhip_conv_desc d;
+            const int8_t* x;
+            const void* wp;
+            const float *scale, *bias;
+            size_t elems;
+        };
+        std::map<int, pending_projection> pending;  // by the value the projection produces
+        auto launch_projection = [&](int value, const pending_projection& pp) {
+            float* yf = static_cast<float*>(vals[value].f32 = alloc(pp.elems * sizeof(float)));
+            plan->launches.push_back([=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &pp.d, pp.x, pp.wp, pp.scale, pp.bias, nullptr, nullptr, yf, nullptr, nullptr)); });
+        };
         for (const node& nd : nodes) {
             const value_info in = vals[nd.in_value];
             value_info& out = vals[nd.out_value];
@@ -641,12 +657,37 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                 out.n = in.n; out.c = c->output_channel_; out.h = oh; out.w = ow; out.cs = ks;
                 const size_t elems = static_cast<size_t>(out.n) * oh * ow * ks;
                 const bool pooled_node = nd.pool_op >= 0;  // its output tensors have the pooled size: allocated below
+                if (!pooled_node && nd.res_value < 0 && !nd.post_relu && d.kh == 1 && d.kw == 1 && d.act == 0 && !is_output[nd.out_value] &&
+                    out.need_f32 && !out.need_i8 && consumers[nd.out_value].size() == 1 && kind[consumers[nd.out_value][0]] == 'a') {
+                    const void* wp = c->pin_packed_weights(EXHIP_I8, d);
+                    plan->pinned.emplace_back([c, wp]() { c->unpin_packed_weights(wp); });
+                    pending[nd.out_value] = {d, static_cast<const int8_t*>(in.i8), wp, c->scale_gpu(), c->bias_gpu(), elems};
+                    continue;
+                }
                 if (out.need_i8 && !pooled_node) out.i8 = alloc(elems);
                 if (out.need_f32 && !pooled_node) out.f32 = alloc(elems * sizeof(float));
                 float** nchw = nullptr;
                 if (is_output[nd.out_value] && !pooled_node) nchw = out.nchw = plan->new_result({out.n, out.c, oh, ow}, dev);
                 const float* res = nullptr;
-                if (nd.res_value >= 0) {
+                bool with_projection = false;
+                pending_projection proj{};
+                if (nd.res_value >= 0 && pending.count(nd.res_value)) {
+                    proj = pending[nd.res_value];
+                    pending.erase(nd.res_value);
+                    const value_info& r = vals[nd.res_value];
+                    with_projection = !pooled_node && out.i8 && out.f32 && !nchw && r.n == out.n && r.h == oh && r.w == ow && r.cs == ks;
+                    if (with_projection) {
+                        const void* wp_main = c->pin_packed_weights(EXHIP_I8, d);
+                        const int rc = exhip_conv2d_i8_projection(ctx, &d, static_cast<const int8_t*>(in.i8), wp_main, c->scale_gpu(), c->bias_gpu(),
+                                                                  &proj.d, proj.x, proj.wp, proj.scale, proj.bias, static_cast<int8_t*>(out.i8),
+                                                                  static_cast<float*>(out.f32));  // trial launch
+                        c->unpin_packed_weights(wp_main);
+                        if (rc == EXHIP_ERR_UNSUPPORTED) with_projection = false;
+                        else EXHIP_FATAL(rc);
+                    }
+                    if (!with_projection) launch_projection(nd.res_value, proj);
+                }
+                if (nd.res_value >= 0 && !with_projection) {
                     const value_info& r = vals[nd.res_value];
                     if (!r.f32 || r.n != out.n || r.h != oh || r.w != ow || r.cs != ks) return give_up();
                     res = static_cast<const float*>(r.f32);
@@ -719,6 +760,12 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                 int8_t* yq = static_cast<int8_t*>(out.i8);
                 float* yf = static_cast<float*>(out.f32);
                 if (!yq && !yf && !nchw) yf = static_cast<float*>(out.f32 = alloc(elems * sizeof(float)));  // dead value: still computed
+                if (with_projection) {
+                    plan->launches.push_back([=]() {
+                        EXHIP_FATAL(exhip_conv2d_i8_projection(ctx, &d, x, wp, scale, bias, &proj.d, proj.x, proj.wp, proj.scale, proj.bias, yq, yf));
+                    });
+                    continue;
+                }
                 plan->launches.push_back(
                     [=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, res, yq, yf, nchw ? *nchw : nullptr, nullptr)); });
             } else {
@@ -743,6 +790,7 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
                 }
             }
         }
+        for (const auto& kv : pending) launch_projection(kv.first, kv.second);  // never claimed: a sum this plan did not absorb
         // several output names may be Split copies of one value: they share its tensor, as in the per-layer executor
         for (const std::string& o : output_names_) {
             const value_info& v = vals[root(blob_index_[o])];

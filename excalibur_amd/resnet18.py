@@ -136,10 +136,11 @@ class FusedRunner:
     float32_to_int8(x * fs) of the very float the CPU path would have produced.
     """
 
-    def __init__(self, ctx, net, n, h, w, profile=False, fuse_pool=True):
+    def __init__(self, ctx, net, n, h, w, profile=False, fuse_pool=True, fuse_projection=True):
         from . import hip
         self.ctx, self.net, self.n, self.h, self.w = ctx, net, n, h, w
         self.fuse_pool = fuse_pool  # stem convolution and max pool as one launch
+        self.fuse_projection = fuse_projection  # a block's projection shortcut inside its second convolution's launch
         self.hip = hip
         self.steps = []       # (label, kind, callable)
         self.conv_gop = {}    # label -> algorithmic GOP per launch
@@ -166,6 +167,36 @@ class FusedRunner:
         self.steps.append((layer.name, "conv", lambda: ctx.conv2d_i8(d, x_i8, wp, scale_d, bias_d, residual, y_i8, y_f32,
                                                                       y_nchw, None)))
         return y_i8, y_f32, y_nchw, oh, ow, ks
+
+    def _scales(self, layer):
+        ws, fs = layer.ws, layer.fs
+        with np.errstate(divide="ignore"):
+            scale = np.where(np.abs(ws.astype(np.float64)) <= 1e-6, np.float32(0),
+                             np.float32(1.0) / (ws * fs).astype(np.float32)).astype(np.float32)
+        return self.ctx.array(scale), self.ctx.array(layer.bias)
+
+    def _conv_projection(self, layer, x_i8, hin, win, cs_in, proj, xp_i8, hp, wp_, cs_p, fs_out):
+        """A block's second convolution with the block's projection shortcut computed in the same launch (sum and ReLU
+        included): int8 and float32 NHWC results, or None where the library leaves the pair to two launches."""
+        ctx, hip = self.ctx, self.hip
+        ks = hip.pad_to(layer.k, 32)
+        d = ctx.conv_desc(self.n, layer.c, hin, win, layer.k, layer.kernel, layer.stride, layer.pad, layer.act, cs_in, ks, 1, float(fs_out))
+        dp = ctx.conv_desc(self.n, proj.c, hp, wp_, proj.k, proj.kernel, proj.stride, proj.pad, proj.act, cs_p, ks, 0, 0.0)
+        oh, ow = ctx.conv_out_hw(d)
+        if ks != layer.k or cs_p != proj.c or ctx.conv_out_hw(dp) != (oh, ow):
+            return None
+        w_main, w_proj = ctx.pack_conv_weights(d, hip.I8, layer.w_i8), ctx.pack_conv_weights(dp, hip.I8, proj.w_i8)
+        scale_d, bias_d = self._scales(layer)
+        scale_p, bias_p = self._scales(proj)
+        y_i8 = ctx.empty((self.n, oh, ow, ks), np.int8)
+        y_f32 = ctx.empty((self.n, oh, ow, ks), np.float32)
+        if not ctx.conv2d_i8_projection(d, x_i8, w_main, scale_d, bias_d, dp, xp_i8, w_proj, scale_p, bias_p, y_i8, y_f32):
+            return None
+        self.conv_gop[layer.name] = (2.0 * self.n * oh * ow * layer.k * layer.c * layer.kernel * layer.kernel +
+                                     2.0 * self.n * oh * ow * proj.k * proj.c) / 1e9
+        self.steps.append((layer.name, "conv", lambda: ctx.conv2d_i8_projection(d, x_i8, w_main, scale_d, bias_d, dp, xp_i8, w_proj,
+                                                                                  scale_p, bias_p, y_i8, y_f32)))
+        return y_i8, y_f32, None, oh, ow, ks
 
     def _conv_maxpool(self, layer, x_i8, hin, win, cs_in, fs_out):
         """Convolution and the 3x3 stride-2 pad-1 max pool behind it as one launch: pooled f32 and int8 NHWC."""
@@ -256,13 +287,19 @@ class FusedRunner:
             if ds is not None:
                 assert ds.fs == c1.fs, "both consumers of a tensor share its activation scale"
             a_i8, _, _, oh, ow, ks = self._conv(c1, cur_i8, hh, ww, cs, None, 0, c2.fs, False, False)
-            if ds is not None:
-                _, short, _, _, _, _ = self._conv(ds, cur_i8, hh, ww, cs, None, 0, None, True, False)
-            else:
-                short = cur_f32
             # the float32 copy is the next block's shortcut: not needed when that block has a downsample convolution
             want_f32 = not last and net.blocks[bi + 1][2] is None
-            o_i8, o_f32, o_nchw, oh, ow, ks = self._conv(c2, a_i8, oh, ow, ks, short, 1, nxt_fs, want_f32, last)
+            fused = None
+            if ds is not None and want_f32 and self.fuse_projection:
+                fused = self._conv_projection(c2, a_i8, oh, ow, ks, ds, cur_i8, hh, ww, cs, nxt_fs)
+            if fused is not None:
+                o_i8, o_f32, o_nchw, oh, ow, ks = fused
+            else:
+                if ds is not None:
+                    _, short, _, _, _, _ = self._conv(ds, cur_i8, hh, ww, cs, None, 0, None, True, False)
+                else:
+                    short = cur_f32
+                o_i8, o_f32, o_nchw, oh, ow, ks = self._conv(c2, a_i8, oh, ow, ks, short, 1, nxt_fs, want_f32, last)
             cur_i8, cur_f32, hh, ww, cs = o_i8, o_f32, oh, ow, ks
             if last:
                 self.out = o_nchw

@@ -149,6 +149,20 @@ int exhip_conv2d_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_conv_desc* d, int p
                                  int pool_ow, const int8_t* x_nhwc, const void* w_packed, const float* scale,
                                  const float* bias, int8_t* y_i8_nhwc, float* y_f32_nhwc);
 
+/* A residual block's closing layers in one kernel: the 1x1 projection of the block's input (d_proj: kernel 1, stride 1 or
+ * 2, no padding, no activation; operation_convolution::forward_cpu_i8, src/Excalibur/operation_convolution.cpp:373-408),
+ * the 3x3 stride-1 convolution d of the block's inner tensor, their sum (BinaryOp ADD, src/Excalibur/operation_binaryop.cpp)
+ * and the ReLU behind it (d->post_relu), which the reference runs as four layers (src/Excalibur/pipeline.cpp:326-392).
+ * Values are those of exhip_conv2d_i8 for the projection (float32 result) followed by exhip_conv2d_i8 for d with that
+ * result as residual_nhwc; the projection's float32 tensor is never stored. Both outputs are required: y_i8_nhwc
+ * (requantized with d->fs_out > 0) and y_f32_nhwc. w_packed / w_packed_proj are exhip_conv_pack_weights' outputs for d /
+ * d_proj. EXHIP_ERR_UNSUPPORTED, with nothing launched, for shapes outside the kernel's (channel strides not multiples
+ * of 64, other activations, launches too small to fill the chip): the caller then issues the two calls. */
+int exhip_conv2d_i8_projection(exhip_ctx* ctx, const exhip_conv_desc* d, const int8_t* x_nhwc, const void* w_packed,
+                               const float* scale, const float* bias, const exhip_conv_desc* d_proj, const int8_t* x_proj_nhwc,
+                               const void* w_packed_proj, const float* scale_proj, const float* bias_proj, int8_t* y_i8_nhwc,
+                               float* y_f32_nhwc);
+
 /* The stem of an int8 network in one kernel: quantize_float32_to_int8 of the float32 NCHW input with the per-tensor scale
  * fs_in (src/Excalibur/operation_general_conv.cpp:584-720), the first convolution (operation_convolution::forward_cpu_i8,
  * src/Excalibur/operation_convolution.cpp:373-408) and MAX pooling 3x3 stride 2 (src/Excalibur/operation_pooling.cpp:145-159)
