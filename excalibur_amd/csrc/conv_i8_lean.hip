@@ -206,17 +206,22 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
         }
     }
     // the lane's two pixels (one per 32-pixel column block of its wave): fragment offset in a tile, position in the patch
-    int boff[2], o_rel[2], o_y[2], o_x[2];
-#pragma unroll
-    for (int nn = 0; nn < 2; ++nn) {
+    // (its position in the output is worked out again in every epilogue: a dozen instructions instead of six registers
+    // held through the MFMA stages)
+    int boff[2];
+    auto patch_pixel = [&](int nn, int& py, int& px) -> bool {
         int pp = (wave * 2 + nn) * 32 + (lane & 31);
         const bool ok = pp < p.PH * p.PW;
         pp = ok ? pp : 0;
-        const int py = fast_div(pp, p.magic_pw), px = pp - py * p.PW;
+        py = fast_div(pp, p.magic_pw);
+        px = pp - py * p.PW;
+        return ok;
+    };
+#pragma unroll
+    for (int nn = 0; nn < 2; ++nn) {
+        int py, px;
+        patch_pixel(nn, py, px);
         boff[nn] = py * (p.IW * kPixB) + px * kPixB + hh * 16;
-        o_rel[nn] = (py * p.OW + px) * p.K;
-        o_y[nn] = ok ? py : 0x4000;  // a row past any image
-        o_x[nn] = px;
     }
     const int row_b = p.IW * kPixB;
     const int img_px = p.OH * p.OW;
@@ -412,8 +417,10 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
         const bool odd_lane = lane & 1;
 #pragma unroll
         for (int nn = 0; nn < 2; ++nn) {
-            const bool valid = full ? o_y[nn] < 0x4000 : ((oy0 + o_y[nn] < p.OH) & (ox0 + o_x[nn] < p.OW));
-            eoff[nn] = valid ? obase + (unsigned)o_rel[nn] : kOobElem;
+            int py, px;
+            const bool in_patch = patch_pixel(nn, py, px);
+            const bool valid = in_patch & (full | ((oy0 + py < p.OH) & (ox0 + px < p.OW)));
+            eoff[nn] = valid ? obase + (unsigned)((py * p.OW + px) * p.K) : kOobElem;
             if (has_f) {
                 // float32 rows leave in 64-byte runs that a lane pair and its neighbour pair form: the even pixel's
                 // runs in one store, the odd pixel's in the next
@@ -423,7 +430,7 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
             }
             if (has_nchw) {
                 const unsigned e = ((unsigned)n * (unsigned)p.K + (unsigned)(kt * 64 + hh * 16)) * (unsigned)img_px +
-                                   (unsigned)((oy0 + o_y[nn]) * p.OW + ox0 + o_x[nn]);
+                                   (unsigned)((oy0 + py) * p.OW + ox0 + px);
                 noff[nn] = valid ? e * 4u : (unsigned)kOob;
             }
         }
@@ -448,6 +455,9 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
             }
 #pragma unroll
             for (int nn = 0; nn < 2; ++nn) {
+                // two accumulator sets fill the register file: keep the scheduler from starting a block's reads and
+                // conversions before the block in front of it is out
+                if constexpr (PROJ) __builtin_amdgcn_sched_barrier(0);
                 v4i q4;
                 if (q_only) {
                     // int8 output only, ReLU last: q = trunc(max(v, 0) * fs + 0.5) capped at 127. With fs > 0 the maximum
@@ -536,10 +546,14 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
                     half_swap4(o4[2], o4[3]);
                     pair_exchange4(o4[0], o4[2], odd_lane);
                     pair_exchange4(o4[1], o4[3], odd_lane);
+#ifndef DBG_NO_FSTORE
                     __builtin_amdgcn_raw_buffer_store_b128(o4[0], rf, (int)(feven[nn] + m * 128), 0, 0);
                     __builtin_amdgcn_raw_buffer_store_b128(o4[1], rf, (int)(feven[nn] + m * 128 + 64), 0, 0);
                     __builtin_amdgcn_raw_buffer_store_b128(o4[2], rf, (int)(fodd[nn] + m * 128), 0, 0);
                     __builtin_amdgcn_raw_buffer_store_b128(o4[3], rf, (int)(fodd[nn] + m * 128 + 64), 0, 0);
+#else
+                    if (o4[0][0] == 0x12345 && o4[1][1] == 0x777 && o4[2][2] == 0x999 && o4[3][3] == 0x111) __builtin_amdgcn_raw_buffer_store_b128(o4[0], rf, (int)(feven[nn] + m * 128), 0, 0);
+#endif
                 }
                 if (has_q) __builtin_amdgcn_raw_buffer_store_b128(q4, rq, (int)(eoff[nn] + hh * 16 + m * 32), 0, 0);
             }
@@ -1273,9 +1287,9 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
     }
     int cfg = g_exhip_options.lean_cfg;  // 0: one tile buffer, two slice buffers; 1: two and two; 2: one and three
     if (proj) {
-        // two groups per CU (two accumulator sets); as with a shortcut tensor, two tile buffers up to 256 channels,
-        // three slice buffers beyond
-        if (mode != 1 || cfg == 0) cfg = g.c_bytes / 64 <= 4 ? 1 : 2;
+        // two groups per CU (two accumulator sets fill the register file; what does not fit is reloaded where the one tile
+        // buffer's refill is waited for anyway, which is why this form measured faster than two tile buffers)
+        if (mode != 1 || cfg == 0) cfg = 2;
         mode = 1;
     }
     if (mode == 4) {
