@@ -87,15 +87,15 @@ def measured_traffic(n, hw):
     """HBM bytes per conv launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE, scaled by a
     plain copy kernel). The counters cannot be read inside this process, so the figure comes from the profile file, which
     names the workload and the kernel sources it was taken with: None for another workload or other sources."""
-    path = os.path.join(ROOT, "profiles", "conv_igemm_resnet18_int8_n32_640_hbm_traffic.txt")
+    path = os.path.join(ROOT, "profiles", "int8_conv_resnet18_n32_640_hbm_traffic.txt")
     if (n, hw) != (32, 640) or not os.path.exists(path):
         return None
     text = open(path).read()
     if f"kernel sources {csrc_digest()}" not in text:
         return None
     for line in text.splitlines():
-        if line.startswith("conv_igemm_kernel HBM traffic per forward"):
-            return {"value": float(line.split("=")[-1].split("MB")[0]), "unit": "MB per launch (mean of 20 launches)"}
+        if line.startswith("HBM traffic per forward"):
+            return {"value": float(line.split("=")[-1].split("MB")[0]), "unit": "MB per launch (mean over the launches of a step)"}
     return None
 
 
@@ -443,7 +443,7 @@ def main():
                                                  f"conv_igemm_kernel: {n_conv} launches for the 20 convolutions)",
                      "achieved": round(achieved_tops, 1), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(achieved_tops / PEAK_INT8_TOPS, 4), "traffic": measured_traffic(n, hw),
-                     "algorithmic_gop_per_step": round(conv_gop, 1), "avg_launch_ms": round(conv_ms / n_conv, 4),
+                     "algorithmic_gop_per_step": round(conv_gop, 1), "launches_per_step": n_conv, "avg_launch_ms": round(conv_ms / n_conv, 4),
                      "timed_region": {"achieved": round(conv_gop / ms_per_step, 1), "frac": round(conv_gop / ms_per_step / PEAK_INT8_TOPS, 4),
                                       "note": "algorithmic GOP of a step over the wall time per step of the timed region (one forward in "
                                               "flight, host-side launch gaps included)"},
