@@ -1301,6 +1301,8 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
         if (!residual) {
             mode = chunks == 1 ? 1 : (chunks <= 4 ? 2 : 1);
             cfg = chunks <= 4 ? 0 : 2;
+        } else if (chunks == 1 && !y_f && !y_nchw) {
+            mode = 1;  // 64 channels, int8 result only (the block in front of a projection): the resident filter, 75 against 79 us
         } else {
             if (chunks <= 2) return EXHIP_ERR_UNSUPPORTED;
             mode = 1;
