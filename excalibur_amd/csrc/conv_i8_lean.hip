@@ -182,6 +182,51 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
     const int GP = G / p.ktiles;
     const int my_tiles = __builtin_amdgcn_readfirstlane((p.n_ptiles - pj + GP - 1) / GP);
 
+    // ---- staging requests of weight slices ----
+    const unsigned wave_slot = (unsigned)wave * 1024u;
+    const int w_voff = tid * 16;
+    const char* const wkt = p.wp + (size_t)kt * p.n_chunks * (3 * kWSlice);  // this slab's slices, in (chunk, filter row) order
+    const int w_run_b = p.n_chunks * 3 * kWSlice;
+    const int n_tot = p.n_chunks + (PROJ ? p.ds_chunks : 0);   // chunks of a patch's run: the 3x3 layer's, then the projection's
+    int w_off = 0;                                  // next slice to request
+    int w_left = my_tiles * n_tot * 3;              // slices of the whole run not requested yet
+    // PROJ: behind the 3x3 layer's slices a patch's run takes three per projection chunk, to keep every stage's requests
+    // alike: the chunk's one tap (4 KiB of the 1x1 layer's packed weights, slab kt) and two empty ones
+    const char* const wkt_ds = PROJ ? p.ds_wp + (size_t)kt * p.ds_chunks * 4096 : nullptr;
+    int w_ds = -1;                                  // >= 0: the next slice is number w_ds of the projection's
+    auto request_w = [&](unsigned dst) {
+        const char* src = wkt + w_off;
+        int range = kWSlice;
+        if constexpr (PROJ) {
+            if (w_ds >= 0) {
+                const int dc = w_ds / 3;
+                src = wkt_ds + dc * 4096;
+                range = w_ds == dc * 3 ? 4096 : 0;
+            }
+        }
+        const __amdgpu_buffer_rsrc_t wr = uniform_view(src, w_left > 0 ? range : 0);
+#pragma unroll
+        for (int i = 0; i < 3; ++i) async_load16(wr, w_voff, i * 4096, dst + wave_slot + i * 4096);
+        --w_left;
+        if constexpr (PROJ) {
+            if (w_ds >= 0) {
+                if (++w_ds == p.ds_chunks * 3) w_ds = -1;
+                return;
+            }
+        }
+        w_off += kWSlice;
+        if (w_off == w_run_b) {
+            w_off = 0;
+            if constexpr (PROJ) w_ds = 0;
+        }
+    };
+    // the first slices go out before anything else: their latency covers the set-up below
+    if constexpr (WRES) {
+        for (int r = 0; r < 3; ++r) request_w(lds0 + r * kWSlice);
+    } else {
+        request_w(lds0);
+    }
+
     // ---- lane constants ----
     // staging: slot v = tid + 256 * i of a tile is 16 bytes of pixel v / 5, part v % 5 (part 4 is the padding)
     int a_rel[kNAL], a_yx[kNAL], a_off[kNAL];
@@ -284,44 +329,7 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
         return 0;
     };
 
-    // ---- staging requests ----
-    const unsigned wave_slot = (unsigned)wave * 1024u;
-    const int w_voff = tid * 16;
-    const char* const wkt = p.wp + (size_t)kt * p.n_chunks * (3 * kWSlice);  // this slab's slices, in (chunk, filter row) order
-    const int w_run_b = p.n_chunks * 3 * kWSlice;
-    const int n_tot = p.n_chunks + (PROJ ? p.ds_chunks : 0);   // chunks of a patch's run: the 3x3 layer's, then the projection's
-    int w_off = 0;                                  // next slice to request
-    int w_left = my_tiles * n_tot * 3;              // slices of the whole run not requested yet
-    // PROJ: behind the 3x3 layer's slices a patch's run takes three per projection chunk, to keep every stage's requests
-    // alike: the chunk's one tap (4 KiB of the 1x1 layer's packed weights, slab kt) and two empty ones
-    const char* const wkt_ds = PROJ ? p.ds_wp + (size_t)kt * p.ds_chunks * 4096 : nullptr;
-    int w_ds = -1;                                  // >= 0: the next slice is number w_ds of the projection's
-    auto request_w = [&](unsigned dst) {
-        const char* src = wkt + w_off;
-        int range = kWSlice;
-        if constexpr (PROJ) {
-            if (w_ds >= 0) {
-                const int dc = w_ds / 3;
-                src = wkt_ds + dc * 4096;
-                range = w_ds == dc * 3 ? 4096 : 0;
-            }
-        }
-        const __amdgpu_buffer_rsrc_t wr = uniform_view(src, w_left > 0 ? range : 0);
-#pragma unroll
-        for (int i = 0; i < 3; ++i) async_load16(wr, w_voff, i * 4096, dst + wave_slot + i * 4096);
-        --w_left;
-        if constexpr (PROJ) {
-            if (w_ds >= 0) {
-                if (++w_ds == p.ds_chunks * 3) w_ds = -1;
-                return;
-            }
-        }
-        w_off += kWSlice;
-        if (w_off == w_run_b) {
-            w_off = 0;
-            if constexpr (PROJ) w_ds = 0;
-        }
-    };
+    // ---- staging requests of tiles (the weight requests stand above the lane constants) ----
     auto request_a = [&](const char* img, int base, int cc, bool valid, unsigned dst) {
         const int off = base + cc * 64;
         const __amdgpu_buffer_rsrc_t xr = uniform_view(img + off, valid ? (int)p.img_bytes - off : 0);
@@ -580,7 +588,6 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
 
     if constexpr (WRES) {
         request_a(img, base, 0, true, lds0 + A0);
-        for (int r = 0; r < 3; ++r) request_w(lds0 + r * kWSlice);
         put(1, now());
         wait_vmcnt<0>();
         __syncthreads();
@@ -623,7 +630,6 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
         constexpr int kWait1 = NWB == 3 ? 3 + (NAB == 2 ? kNAL : 0) : 0;
         constexpr int kWait2 = NWB == 3 ? 3 : 0;
         request_a(img, base, 0, true, lds0 + A0);
-        request_w(lds0);
         if constexpr (NWB == 3) request_w(lds0 + kWSlice);
         put(1, now());
         wait_vmcnt<(NWB == 3 ? 3 : 0)>();
