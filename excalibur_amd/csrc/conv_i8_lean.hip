@@ -1300,9 +1300,8 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
     }
     if (mode == 4) {
         // The form that measured fastest per layer class on the ResNet-18-shaped stack at 32 x 640 x 640: without a shortcut
-        // the resident filter (64 channels) or one group per patch with three groups per CU; with a shortcut, whose float32
-        // traffic is the larger part of the launch, the general kernel up to 128 channels (its three groups per CU keep
-        // more of it in flight) and persistent groups with deeper buffers beyond.
+        // the resident filter (64 channels) or one group per patch with three groups per CU, persistent groups with three
+        // slice buffers from 512 channels on; with a shortcut see below.
         const int chunks = g.c_bytes / 64;
         if (!residual) {
             mode = chunks == 1 ? 1 : (chunks <= 4 ? 2 : 1);
@@ -1310,9 +1309,12 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
         } else if (chunks == 1 && !y_f && !y_nchw) {
             mode = 1;  // 64 channels, int8 result only (the block in front of a projection): the resident filter, 75 against 79 us
         } else {
-            if (chunks <= 2) return EXHIP_ERR_UNSUPPORTED;
+            // float32 result next to the shortcut and at most 128 channels: the general kernel's three groups per CU keep
+            // more of that traffic in flight. Otherwise one tile buffer and three slice buffers (128 channels, int8 result
+            // only: 50 against 56 us in the general kernel; 256 channels: 38 against 39 us with two tile buffers).
+            if (chunks <= 2 && (y_f || y_nchw || chunks == 1)) return EXHIP_ERR_UNSUPPORTED;
             mode = 1;
-            cfg = chunks <= 4 ? 1 : 2;
+            cfg = 2;
         }
     }
     const long long n_ptiles = (long long)g.n * g.tiles_y * g.tiles_x;
