@@ -74,6 +74,22 @@ struct exhip_options {
 extern exhip_options g_exhip_options;
 
 // ---- device helpers shared by the kernels ----
+typedef int exhip_v4i __attribute__((ext_vector_type(4)));
+// Stores reach full speed with runs of 64 contiguous bytes from neighbouring lanes (measured: 32-byte runs take twice as
+// long), so two pixels in neighbouring lanes trade halves: afterwards `a` holds, in the even lane, its own a and, in the
+// odd lane, the even lane's c; `c` holds the odd lane's a and, in the odd lane, its own c. (DPP quad_perm [1, 0, 3, 2].)
+__device__ __forceinline__ int lane_neighbour(int v) { return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true); }
+__device__ __forceinline__ void pair_exchange4(exhip_v4i& a, exhip_v4i& c, bool odd) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int from_c = lane_neighbour(c[e]), from_a = lane_neighbour(a[e]);
+        const int a2 = odd ? from_c : a[e], c2 = odd ? c[e] : from_a;
+        a[e] = a2;
+        c[e] = c2;
+    }
+}
+
+
 // float32_to_int8 of the reference (src/Primitives/simd_types.cpp:140-152): add +-0.5, saturate, truncate.
 __device__ __forceinline__ int exhip_q8(float v) {
     float t = v >= 0.f ? v + 0.5f : v - 0.5f;

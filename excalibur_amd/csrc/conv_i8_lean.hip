@@ -115,20 +115,6 @@ __device__ __forceinline__ void half_swap4(v4i& a, v4i& b) {
     }
 }
 
-// Stores reach full speed with runs of 64 contiguous bytes from neighbouring lanes (measured: 32-byte runs take twice as
-// long), so two pixels in neighbouring lanes trade halves: afterwards `a` holds, in the even lane, its own a and, in the
-// odd lane, the even lane's c; `c` holds the odd lane's a and, in the odd lane, its own c. (DPP quad_perm [1, 0, 3, 2].)
-__device__ __forceinline__ int lane_neighbour(int v) { return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true); }
-__device__ __forceinline__ void pair_exchange4(v4i& a, v4i& c, bool odd) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const int from_c = lane_neighbour(c[e]), from_a = lane_neighbour(a[e]);
-        const int a2 = odd ? from_c : a[e], c2 = odd ? c[e] : from_a;
-        a[e] = a2;
-        c[e] = c2;
-    }
-}
-
 // WRES: the slab's whole filter is resident (one 64-byte chunk); otherwise weight slices rotate through NWB buffers and
 // activation tiles through NAB. EPI >= 0: the epilogue's switches as compile-time constants; EPI < 0: read from p.flags.
 // PROJ: the shortcut is a 1x1 convolution computed here (p.ds_*): its channel chunks follow the 3x3 layer's in every patch's

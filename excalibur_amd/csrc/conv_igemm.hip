@@ -1203,9 +1203,23 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                             const uint32_t lo = exhip_f2h(v[2 * e]), hi = exhip_f2h(v[2 * e + 1]);
                             o[e >> 2][e & 3] = (int)(lo | (hi << 16));
                         }
-                        v4i* y = reinterpret_cast<v4i*>(reinterpret_cast<uint16_t*>(p.y_q) + pix * p.kstride + ch0);
-                        y[0] = o[0];
-                        y[1] = o[1];
+                        char* const yb = reinterpret_cast<char*>(p.y_q) + ch0 * 2;
+                        if (__builtin_amdgcn_ballot_w64(true) == ~0ull && (size_t)p.N * img_px < (1u << 31)) {
+                            // the whole wave stores: a lane's 32 bytes and its neighbour's trade halves, so that four
+                            // lanes (p, p + 1 and the same two of the other half-wave) write 64 contiguous bytes of one
+                            // pixel per instruction instead of four 16-byte pieces of two
+                            const bool odd = lane & 1;
+                            pair_exchange4(o[0], o[1], odd);
+                            const unsigned mine = (unsigned)pix, other = (unsigned)lane_neighbour((int)mine);
+                            const size_t even_pix = odd ? other : mine, odd_pix = odd ? mine : other;
+                            const int sub = odd ? 16 : 0;
+                            *reinterpret_cast<v4i*>(yb + even_pix * p.kstride * 2 + sub) = o[0];
+                            *reinterpret_cast<v4i*>(yb + odd_pix * p.kstride * 2 + sub) = o[1];
+                        } else {
+                            v4i* y = reinterpret_cast<v4i*>(yb + pix * p.kstride * 2);
+                            y[0] = o[0];
+                            y[1] = o[1];
+                        }
                     }
                 } else {
                     if (p.y_nhwc) {
