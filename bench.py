@@ -284,6 +284,8 @@ def main():
     ap.add_argument("--no-memory-bound", action="store_true", help="skip the memory-bound kernels' block of the line")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="set a library option (exhip_set_option) before the network is planned; may be repeated")
+    ap.add_argument("--exhip-lib", default=None, metavar="PATH",
+                    help="load this build of libexhip.so instead of the one in the tree (comparing kernel builds in one session)")
     ap.add_argument("--per-layer", action="store_true", help="print per-launch timings to stderr")
     ap.add_argument("--networks", action="store_true",
                     help="time the other configurations' whole topologies (MobileNet- and YOLOv5s-shaped, f32 / f16 / int8) "
@@ -295,6 +297,10 @@ def main():
         print("bench.py: this build runs on one GPU; the batch shards trivially across GPUs but no multi-GPU path "
               "is part of it (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
+
+    if args.exhip_lib:
+        from excalibur_amd import hip as _hip
+        _hip.LIB_PATH = os.path.abspath(args.exhip_lib)
 
     if args.bandwidth:
         print(json.dumps({"metric": "achieved HBM GB/s of the memory-bound kernels", "peak_GB/s": PEAK_HBM_GBS,

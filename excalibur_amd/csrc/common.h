@@ -73,6 +73,11 @@ struct exhip_options {
 };
 extern exhip_options g_exhip_options;
 
+// Cache policy bits of the float32 result stores of the int8 kernels (the aux operand of the raw buffer store builtins).
+#ifndef EXHIP_F32_STORE_AUX
+#define EXHIP_F32_STORE_AUX 0
+#endif
+
 // ---- device helpers shared by the kernels ----
 typedef int exhip_v4i __attribute__((ext_vector_type(4)));
 // Stores reach full speed with runs of 64 contiguous bytes from neighbouring lanes (measured: 32-byte runs take twice as

@@ -540,14 +540,10 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
                     half_swap4(o4[2], o4[3]);
                     pair_exchange4(o4[0], o4[2], odd_lane);
                     pair_exchange4(o4[1], o4[3], odd_lane);
-#ifndef DBG_NO_FSTORE
-                    __builtin_amdgcn_raw_buffer_store_b128(o4[0], rf, (int)(feven[nn] + m * 128), 0, 0);
-                    __builtin_amdgcn_raw_buffer_store_b128(o4[1], rf, (int)(feven[nn] + m * 128 + 64), 0, 0);
-                    __builtin_amdgcn_raw_buffer_store_b128(o4[2], rf, (int)(fodd[nn] + m * 128), 0, 0);
-                    __builtin_amdgcn_raw_buffer_store_b128(o4[3], rf, (int)(fodd[nn] + m * 128 + 64), 0, 0);
-#else
-                    if (o4[0][0] == 0x12345 && o4[1][1] == 0x777 && o4[2][2] == 0x999 && o4[3][3] == 0x111) __builtin_amdgcn_raw_buffer_store_b128(o4[0], rf, (int)(feven[nn] + m * 128), 0, 0);
-#endif
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[0], rf, (int)(feven[nn] + m * 128), 0, EXHIP_F32_STORE_AUX);
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[1], rf, (int)(feven[nn] + m * 128 + 64), 0, EXHIP_F32_STORE_AUX);
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[2], rf, (int)(fodd[nn] + m * 128), 0, EXHIP_F32_STORE_AUX);
+                    __builtin_amdgcn_raw_buffer_store_b128(o4[3], rf, (int)(fodd[nn] + m * 128 + 64), 0, EXHIP_F32_STORE_AUX);
                 }
                 if (has_q) __builtin_amdgcn_raw_buffer_store_b128(q4, rq, (int)(eoff[nn] + hh * 16 + m * 32), 0, 0);
             }

@@ -965,7 +965,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 for (int it = 0; it < 8; ++it) {
                     const int idx = it * 64 + lane, tp = idx >> 4, part = idx & 15;
                     __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const v4i*>(tile_f + tp * kEpiRowF + part * 16), rf,
-                                                           (int)((table[tp] + part * 4) * 4u), 0, 0);
+                                                           (int)((table[tp] + part * 4) * 4u), 0, EXHIP_F32_STORE_AUX);
                 }
             }
             if (has_q) {

@@ -292,7 +292,7 @@ __global__ __launch_bounds__(256, 3) void stem_conv_pool_kernel(const StemParams
                 }
                 const bool ok = ((it_yx[k] & 0xFFFF) < lim_y) & ((int)((unsigned)it_yx[k] >> 16) < lim_x);
                 const unsigned off = ok ? tile_elem + (unsigned)it_rel[k] : kOobElem;
-                if (has_f) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, best), rf, (int)(off * 4u), 0, 0);
+                if (has_f) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, best), rf, (int)(off * 4u), 0, EXHIP_F32_STORE_AUX);
                 if (has_q) {
                     int b[4], packed;
                     if (p.q_nonneg) {
