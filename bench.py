@@ -359,7 +359,14 @@ def main():
             q.sync()
         return time.perf_counter() - t0
 
+    # The timed pipeline brackets the convolution launches of every forward with a HIP event pair of its own (a ring of
+    # 32 pairs, read after the loop's closing synchronisation): the roofline's launch durations are taken in the steps
+    # that `value` counts, events' own cost included in both.
+    pipe.time_fused_span(-2)
     one_elapsed = timed(pipes[:1], args.steps, args.warmup)
+    spans = pipe.recent_spans(min(args.steps, 32))
+    _, n_conv = pipe.last_span()
+    pipe.time_fused_span(-1)
     assert pipe.fused, "the int8 ResNet-18 topology did not take the fused plan"
     # `value` is the rate with one forward in flight, the regime the roofline block and the profiles describe; the rate
     # with `in_flight` forwards queued on streams of their own is reported beside it (config.in_flight_N).
@@ -387,22 +394,10 @@ def main():
     ctx.sync()
 
     # The dominant kernel's launches of one forward, timed with one HIP event pair on the library's stream: from in
-    # front of the first convolution to behind the last (the 20 launches follow each other without anything else
-    # between them). The interval holds the launches and the queue's hand-over between them, as the sum of a kernel
-    # trace's durations does; one pair per forward keeps the events' own cost below 1 %.
-    # Taken on the timed path itself: the pipeline records the two events around the convolution launches of its fused
-    # plan (an input quantizer in front of them, where the stem kernel does not quantize its own input, stays outside).
-    # Each sample is the last of four forwards queued back to back (the event pair is recorded anew by every forward), so
-    # the launches it brackets run as they do in the timed loop: behind a busy queue, not behind a host synchronisation.
-    reps = max(3, min(args.steps, 10))
-    pipe.time_fused_span(-2)
-    spans = []
-    for _ in range(reps):
-        for _ in range(4):
-            pipe.run()
-        span_ms, n_conv = pipe.last_span()
-        spans.append(span_ms)
-    pipe.time_fused_span(-1)
+    # front of the first convolution to behind the last (the launches follow each other without anything else between
+    # them; an input quantizer in front of them, where the stem kernel does not quantize its own input, stays outside).
+    # The interval holds the launches and the queue's hand-over between them, as the sum of a kernel trace's durations
+    # does. The samples are those of the timed region's last steps (above).
     assert n_conv == len(run.conv_gop), f"the fused plan's span holds {n_conv} launches, expected {len(run.conv_gop)} convolutions"
     conv_ms = float(np.mean(spans))
     conv_gop = sum(run.conv_gop.values())
@@ -423,6 +418,7 @@ def main():
         ctx.sync()
         event_overhead_ms = float(np.median([e0.elapsed_ms(e1) for e0, e1 in pairs]))
         acc = {}
+        reps = max(3, min(args.steps, 10))
         for _ in range(reps):
             for label, kind, ms in run.forward_timed():
                 a = acc.setdefault(label, [kind, 0.0])
@@ -453,8 +449,8 @@ def main():
                      "timed_region": {"achieved": round(conv_gop / ms_per_step, 1), "frac": round(conv_gop / ms_per_step / PEAK_INT8_TOPS, 4),
                                       "note": "algorithmic GOP of a step over the wall time per step of the timed region (one forward in "
                                               "flight, host-side launch gaps included)"},
-                     "timing": f"HIP events around the {n_conv} consecutive launches of a forward of the timed pipeline, the last of four "
-                               f"forwards queued back to back on one stream (steady state, nothing else in flight), mean of {reps} samples"},
+                     "timing": f"HIP events around the {n_conv} consecutive launches of a forward, recorded by the timed pipeline in "
+                               f"the steps of the timed region (one forward in flight), mean of its last {len(spans)} steps"},
     }
     if not args.no_memory_bound:
         every = bandwidth_table(iters=10, quiet=True, ctx=ctx)

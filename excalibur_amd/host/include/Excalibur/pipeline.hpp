@@ -48,8 +48,12 @@ public:
     // of its launch number first_launch (0 is the input quantizer, unless the stem kernel quantizes its own input; -2 stands
     // for the first convolution's launch, whichever number it has) and one behind its last launch;
     // last_span(&launches) waits for them and returns the milliseconds between the two and the launches in between.
+    // The event pairs come from a ring of 32: recent_spans(ms, capacity) waits for the device and fills in the spans of
+    // the latest forwards since time_fused_span was called (oldest first, at most 32 and at most capacity), so that
+    // forwards queued back to back are read without a synchronisation between them; it returns how many it wrote.
     void time_fused_span(int first_launch);
     float last_span(int* launches);
+    int recent_spans(float* ms, int capacity);
 
     // Stream slots (no counterpart in the reference, whose pipelines are synchronous): a pipeline does its device work on
     // the HIP stream of the slot its constructing thread was in (memory::set_stream_slot; 0 unless set), so pipelines made

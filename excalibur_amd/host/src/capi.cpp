@@ -109,6 +109,10 @@ extern "C" float exc_pipeline_last_span(exc_pipeline* p, int* launches) {
     return p->f32 ? p->f32->last_span(launches) : 0.f;
 }
 
+extern "C" int exc_pipeline_recent_spans(exc_pipeline* p, float* ms, int capacity) {
+    return p->f32 ? p->f32->recent_spans(ms, capacity) : 0;
+}
+
 extern "C" int exc_pipeline_set_input(exc_pipeline* p, const void* input, const int shape[4]) {
     glasssix::memory::stream_scope scope(p->slot);  // the input's device block belongs to the pipeline's slot
     if (p->dtype == 0) set_input(p->in32, p->device, input, shape);

@@ -63,7 +63,12 @@ public:
     impl() : device_(-1) {}  // the reference's default-constructed pipeline (pipeline.cpp:575-577): no layers; forward is fatal
 
     // the plan lets go of the operators' packed weights: it goes first, while the operators still exist
-    ~impl() { plan_.reset(); }
+    ~impl() {
+        plan_.reset();
+        for (auto& pair : span_ev_)
+            for (void* ev : pair)
+                if (ev) exhip_event_destroy(ev);
+    }
 
     impl(const std::vector<std::string>& lines, std::string_view model_file, int device) : device_(device) {
         if (device >= 0) memory::device_context(device);  // opens the device, fatal if it is not an MI355X
@@ -331,8 +336,12 @@ public:
     bool graphs_ = false;
     bool last_fused_ = false;
     double last_ms_ = 0;
-    int span_first_ = -1, span_launches_ = 0;  // time_fused_span / last_span
-    void* span_ev_[2] = {nullptr, nullptr};
+    // time_fused_span / last_span / recent_spans: timed forwards take their event pair from a ring, so that a run of
+    // forwards queued back to back can be read after one synchronisation at its end
+    static constexpr int kSpanRing = 32;
+    int span_first_ = -1, span_launches_ = 0;
+    long long span_count_ = 0;  // timed forwards since time_fused_span was last called
+    void* span_ev_[kSpanRing][2] = {};
     int device() const { return device_; }
     const int slot_ = memory::stream_slot();  // the stream slot the constructing thread was in: all device work goes there
 
@@ -816,9 +825,10 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
     const int n_launches = static_cast<int>(plan_->launches.size());
     const int span_first = span_first_ == -2 ? plan_->first_conv_launch : span_first_;  // -2: from the first convolution on
     const bool timed = span_first >= 0 && span_first < n_launches;
-    if (timed && !span_ev_[0]) {
-        EXHIP_FATAL(exhip_event_create(&span_ev_[0]));
-        EXHIP_FATAL(exhip_event_create(&span_ev_[1]));
+    void** const span_ev = span_ev_[span_count_ % kSpanRing];
+    if (timed && !span_ev[0]) {
+        EXHIP_FATAL(exhip_event_create(&span_ev[0]));
+        EXHIP_FATAL(exhip_event_create(&span_ev[1]));
     }
     // the graph form: launch 0 eagerly, the rest as one replay (a timed span must start at launch 0 or 1 to use it)
     bool use_graph = graphs_ && n_launches > 2 && plan_->forwards >= 1 && (!timed || span_first <= 1);
@@ -835,23 +845,24 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
             EXHIP_FATAL(exhip_graph_end(ctx, &plan_->graph));
             plan_->graph_slots = slots;
         }
-        if (timed && span_first == 0) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+        if (timed && span_first == 0) EXHIP_FATAL(exhip_event_record(ctx, span_ev[0]));
         plan_->launches[0]();
-        if (timed && span_first == 1) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+        if (timed && span_first == 1) EXHIP_FATAL(exhip_event_record(ctx, span_ev[0]));
         EXHIP_FATAL(exhip_graph_launch(ctx, plan_->graph));
-        if (timed) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[1]));
+        if (timed) EXHIP_FATAL(exhip_event_record(ctx, span_ev[1]));
         span_launches_ = timed ? n_launches - span_first : 0;
     } else if (timed) {
         for (int i = 0; i < n_launches; ++i) {
-            if (i == span_first) EXHIP_FATAL(exhip_event_record(ctx, span_ev_[0]));
+            if (i == span_first) EXHIP_FATAL(exhip_event_record(ctx, span_ev[0]));
             plan_->launches[i]();
         }
-        EXHIP_FATAL(exhip_event_record(ctx, span_ev_[1]));
+        EXHIP_FATAL(exhip_event_record(ctx, span_ev[1]));
         span_launches_ = n_launches - span_first;
     } else {
         for (auto& launch : plan_->launches) launch();
         span_launches_ = 0;
     }
+    if (timed) ++span_count_;
     ++plan_->forwards;
     last_fused_ = true;
     for (auto& r : plan_->outputs) {
@@ -928,16 +939,28 @@ template <typename Dtype>
 void pipeline<Dtype>::set_graphs(bool on) { impl_->graphs_ = on; }
 
 template <typename Dtype>
-void pipeline<Dtype>::time_fused_span(int first_launch) { impl_->span_first_ = first_launch; }
+void pipeline<Dtype>::time_fused_span(int first_launch) {
+    impl_->span_first_ = first_launch;
+    impl_->span_count_ = 0;
+}
 
 template <typename Dtype>
 float pipeline<Dtype>::last_span(int* launches) {
     if (launches) *launches = impl_->span_launches_;
-    if (!impl_->span_launches_) return 0.f;
-    EXHIP_FATAL(exhip_sync(memory::device_context(impl_->device(), impl_->slot_)));
     float ms = 0.f;
-    EXHIP_FATAL(exhip_event_elapsed_ms(impl_->span_ev_[0], impl_->span_ev_[1], &ms));
-    return ms;
+    return recent_spans(&ms, 1) ? ms : 0.f;
+}
+template <typename Dtype>
+int pipeline<Dtype>::recent_spans(float* ms, int capacity) {
+    if (!impl_->span_launches_ || capacity <= 0) return 0;
+    EXHIP_FATAL(exhip_sync(memory::device_context(impl_->device(), impl_->slot_)));
+    const long long have = std::min<long long>(impl_->span_count_, impl::kSpanRing);
+    const int n = static_cast<int>(std::min<long long>(have, capacity));
+    for (int i = 0; i < n; ++i) {  // oldest of the n first
+        void** const ev = impl_->span_ev_[(impl_->span_count_ - n + i) % impl::kSpanRing];
+        EXHIP_FATAL(exhip_event_elapsed_ms(ev[0], ev[1], &ms[i]));
+    }
+    return n;
 }
 template <typename Dtype>
 double pipeline<Dtype>::last_forward_ms() const { return impl_->last_ms_; }

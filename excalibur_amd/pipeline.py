@@ -43,6 +43,8 @@ def lib():
         L.exc_pipeline_time_fused_span.argtypes = [ctypes.c_void_p, ctypes.c_int]
         L.exc_pipeline_last_span.restype = ctypes.c_float
         L.exc_pipeline_last_span.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int)]
+        L.exc_pipeline_recent_spans.restype = ctypes.c_int
+        L.exc_pipeline_recent_spans.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_float), ctypes.c_int]
         L.exc_registered_operations.restype = ctypes.c_size_t
         L.exc_registered_operations.argtypes = [ctypes.c_int, ctypes.c_char_p, ctypes.c_size_t]
         _lib = L
@@ -140,6 +142,13 @@ class Pipeline:
         n = ctypes.c_int(0)
         ms = lib().exc_pipeline_last_span(self.h, ctypes.byref(n))
         return float(ms), n.value
+
+    def recent_spans(self, capacity=32):
+        """Milliseconds between the events of the latest fused forwards since time_fused_span (oldest first, at most 32);
+        waits for the device once, so forwards queued back to back are read without a synchronisation between them."""
+        buf = (ctypes.c_float * capacity)()
+        n = lib().exc_pipeline_recent_spans(self.h, buf, capacity)
+        return [float(buf[i]) for i in range(n)]
 
     @property
     def fused(self):

@@ -55,9 +55,13 @@ long exc_pipeline_get(exc_pipeline* p, const char* name, void* out, long capacit
  * (0 = the input quantizer, or the stem when its kernel quantizes the input itself; -2 = the first convolution's launch,
  * whichever number it has) and one behind its last launch; -1 switches that off. exc_pipeline_last_span waits for
  * the device and returns the milliseconds between the two events of the last forward and, in *launches, how many
- * launches lay between them (0 and 0.0 if the last forward was not a fused one). */
+ * launches lay between them (0 and 0.0 if the last forward was not a fused one). The event pairs come from a ring of
+ * 32: exc_pipeline_recent_spans waits for the device once and writes the spans of the latest forwards since
+ * exc_pipeline_time_fused_span was called (oldest first, at most 32 and at most `capacity`), so that forwards queued
+ * back to back are read without a synchronisation between them; it returns how many it wrote. */
 void exc_pipeline_time_fused_span(exc_pipeline* p, int first_launch);
 float exc_pipeline_last_span(exc_pipeline* p, int* launches);
+int exc_pipeline_recent_spans(exc_pipeline* p, float* ms, int capacity);
 /* Test and development switches, process-wide (nothing is read from the environment): "f16_nchw_only" = 1 keeps every
  * blob of pipeline<unsigned short> NCHW instead of NHWC between layers; any other name goes to exhip_set_option.
  * Returns 0, or an error code for an unknown name. */

@@ -87,6 +87,13 @@ def test_resnet18_topology_through_the_pipeline(fusion):
         ms, launches = p.last_span()
         assert (launches, ms > 0) == ((20, True) if fusion else (0, False))
         assert np.array_equal(p.get(net.output), want)
+        # forwards queued back to back are read after one synchronisation, oldest first, from a ring of 32 event pairs
+        for _ in range(3):
+            p.run()
+        recent = p.recent_spans()
+        assert len(recent) == (4 if fusion else 0) and all(v > 0 for v in recent)
+        assert not fusion or recent[-1] == p.last_span()[0]
+        assert len(p.recent_spans(2)) == (2 if fusion else 0)
         p.time_fused_span(-1)
         p.forward(x)
         assert p.last_span() == (0.0, 0)
