@@ -64,6 +64,8 @@ I8_SHAPES = [
     (209, 2, 32, 17, 17, 40, 5, 1, 2),      # 5x5
     (210, 1, 16, 30, 30, 24, 7, 2, 3),      # 7x7 with 16 channels (generic form)
     (211, 2, 96, 24, 24, 160, 3, 2, (0, 1, 0, 1)),  # asymmetric padding
+    (212, 1, 32, 256, 8, 64, 1, 1, 0),      # 1x1 on a 256-row map: the planner's patch is one pixel wide
+    (213, 1, 32, 40, 1, 64, 3, 1, 1),       # an image one pixel wide
 ]
 
 
