@@ -27,6 +27,7 @@
 
 #include "common.h"
 #include "conv_i8_lean.h"
+#include "conv_pw.h"
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
@@ -134,8 +135,9 @@ __device__ __forceinline__ void mma(typename Acc<DT>::type& acc, const v4i& a, c
     }
 }
 
-// n / d for n < 2^16 with magic = ceil(2^32 / d): one multiply-high instead of an emulated division
-__device__ __forceinline__ int fast_div(int n, unsigned magic) { return (int)__umulhi((unsigned)n, magic); }
+// n / d for n < 2^16 with magic = ceil(2^32 / d) as a 32-bit word: one multiply-high instead of an emulated division;
+// d == 1 arrives as 0 (2^32 does not fit the word)
+__device__ __forceinline__ int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
 
 __device__ __forceinline__ v4i lds_read16(const char* p) { return *reinterpret_cast<const v4i*>(p); }
 
@@ -1700,6 +1702,21 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             p.q_nonneg = d->fs_out > 0.f && (d->post_relu || (d->act == 1 && !p.residual));
             if (pl.packed) return launch_variant<DT, true, 1>(ctx, pl, p, (int)grid);
             return launch_variant<DT, false, 1>(ctx, pl, p, (int)grid);
+        }
+    }
+    if constexpr (DT == EXHIP_F16) {
+        if (!pl.packed && !pool && d->kh == 1 && d->kw == 1 && d->sh == 1 && d->sw == 1 && !d->pt && !d->pb && !d->pl && !d->pr && p.y_q &&
+            !p.y_nchw_h && !p.y_nchw) {
+            // a pointwise layer with only the NHWC result: the kernel without staging takes it with the same packed weights;
+            // EXHIP_ERR_UNSUPPORTED leaves it to this one
+            exhip_pw_geom g = {};
+            g.pixels = (long long)d->n * d->h * d->w; g.c_bytes = p.cstride_b; g.k = d->k; g.k_stride = d->k_stride;
+            g.slab_blocks = pl.TM / 32; g.slabs = pl.ktiles;
+            g.act = d->act; g.post_relu = d->post_relu; g.post_op = d->post_op; g.post_slope_shared = d->post_slope_shared;
+            g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope;
+            rc = exhip_conv1x1_f16_pw(ctx, g, reinterpret_cast<const uint16_t*>(p.x), p.wp, p.bias, reinterpret_cast<const uint16_t*>(p.residual),
+                                      reinterpret_cast<uint16_t*>(p.y_q));
+            if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
         }
     }
     if (pl.packed) return launch_variant<DT, true, 0>(ctx, pl, p, (int)grid);

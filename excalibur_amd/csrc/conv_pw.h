@@ -1,0 +1,20 @@
+// The 1x1 stride-1 fp16 convolution (a pointwise layer: a matrix product over the flattened pixels) as a kernel without
+// LDS staging and without barriers (conv_pw.hip). conv_igemm.hip plans the layer and hands the launch over when the
+// geometry fits; the weights are the general kernel's packing.
+#pragma once
+#include "common.h"
+
+struct exhip_pw_geom {
+    long long pixels;           // N * H * W: rows of the NHWC input and output
+    int c_bytes;                // bytes per input pixel (channel stride * 2), a multiple of 32
+    int k, k_stride;            // output channels and the output's channel stride, in elements
+    int slab_blocks, slabs;     // the packing: 32-channel blocks per slab (2 or 4) and slabs
+    int act, post_relu, post_op, post_slope_shared;
+    float post_alpha, post_beta;
+    const float* post_slope;
+};
+
+// Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then
+// runs the general kernel), another code on failure. Semantics as exhip_conv2d_f16 with only the NHWC half output.
+int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t* x, const void* wp, const float* bias,
+                         const uint16_t* residual, uint16_t* y);

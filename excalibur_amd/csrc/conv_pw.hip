@@ -1,0 +1,306 @@
+// conv1x1_f16_pw_kernel: the pointwise (1x1, stride 1, no padding) fp16 convolution, y[pixel][k] = sum_c x[pixel][c] * w[k][c].
+//
+// A pointwise layer of a detection or mobile network moves a few tens of MB for a few GFLOP: what it costs is the
+// length of one group's chain from launch to last store, and the memory system's rate. So nothing is staged: a wave
+// owns 32 * NT pixels x 32 * MT output channels and fetches its MFMA operands straight into registers, 16 bytes per
+// lane and k-step -- the weight fragments in the general kernel's packing (one contiguous KiB per 32-channel block and
+// k-step), the pixel fragments from the NHWC rows themselves (lane = pixel, the two half-waves the two 16-byte halves
+// of a 32-byte k-step). No LDS, no barrier, no tile geometry: the pixels of all images form one list. The four waves of
+// a group are neighbours in (pixel tile, channel group) order with the channel group running fastest, so the waves that
+// read the same pixels sit on one CU; the pixel rows come from HBM once and from the caches after that.
+//
+// Arithmetic and roundings are the general kernel's (conv_igemm.hip, general epilogue): float32 accumulation in
+// v_mfma_f32_32x32x16_f16, bias, activation, the optional shortcut added to the value rounded to half, ReLU / the
+// activation layer behind the convolution applied to the rounded half, one final rounding.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+
+#include "conv_pw.h"
+
+namespace {
+
+typedef exhip_v4i v4i;
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer: out-of-range loads return 0
+constexpr int kOutOfRange = 0x7ffff000;       // a lane offset beyond every view
+
+struct PwParams {
+    const char* x;
+    const char* wp;
+    const float* bias;
+    const uint16_t* residual;
+    uint16_t* y;
+    const float* post_slope;
+    unsigned pixels, x_bytes, w_bytes;
+    unsigned items, ch_groups;   // waves with work; 32 * MT channel groups per pixel tile
+    int xs_b;                    // bytes per input pixel
+    int n_ksteps;                // 32-byte k-steps per pixel
+    int mts;                     // 32-channel blocks per packed slab
+    int K, kstride;
+    int act, post_relu, post_op, post_slope_shared;
+    float post_alpha, post_beta;
+};
+
+__device__ __forceinline__ float fast_activation(float v, int act) {
+    if (act == 1) return (0.f > v) ? 0.f : v;
+    if (act == 3) { const float d = (0.f > v) ? 0.f : v; return d <= 6.f ? d : 0.f; }
+    return v;
+}
+__device__ __noinline__ float slow_activation(float v, int act) { return exhip_act(v, act); }
+
+template <int OP>
+__device__ __forceinline__ void post_activation_op(float (&v)[16], float alpha, float beta) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = unary_value<OP>(exhip_h2f(exhip_f2h(v[e])), alpha, beta);
+}
+
+// The bias values of a lane's 16 channels per 32-channel block (zeros beyond K).
+template <int MT>
+__device__ __forceinline__ void load_bias(const PwParams& p, int kb0, int lane, float (&bi)[MT][16]) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int ch0 = (kb0 + m) * 32 + (lane >> 5) * 16;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) bi[m][e] = (p.bias && ch0 + e < p.K) ? p.bias[ch0 + e] : 0.f;
+    }
+}
+
+// Epilogue of one wave tile: a lane holds 16 consecutive channels of its pixel per 32-channel block.
+template <int MT, int NT>
+__device__ __forceinline__ void pw_epilogue(const PwParams& p, const v16f (&acc)[MT][NT], const unsigned (&pix)[NT], int kb0, int lane,
+                                            const float (&bi)[MT][16]) {
+    const bool odd = lane & 1;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int ch0 = (kb0 + m) * 32 + (lane >> 5) * 16;
+        if (ch0 >= p.kstride && ch0 >= p.K) continue;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const bool valid = pix[n] < p.pixels;
+            float v[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) v[e] = acc[m][n][e] + bi[m][e];
+            if (p.act >= 4) {
+#pragma unroll 1
+                for (int e = 0; e < 16; ++e) v[e] = slow_activation(v[e], p.act);
+            } else if (p.act) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = fast_activation(v[e], p.act);
+            }
+            if (p.residual && valid) {
+                // the add layer behind this one reads the stored (rounded) half
+                const uint16_t* r = p.residual + (size_t)pix[n] * p.kstride + ch0;
+                if (ch0 + 16 <= p.K) {
+                    const v4i r0 = reinterpret_cast<const v4i*>(r)[0], r1 = reinterpret_cast<const v4i*>(r)[1];
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int word = e < 8 ? r0[e >> 1] : r1[(e - 8) >> 1];
+                        v[e] = exhip_h2f(exhip_f2h(v[e])) + exhip_h2f((uint16_t)(((uint32_t)word >> ((e & 1) * 16)) & 0xffff));
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        if (ch0 + e < p.K) v[e] = exhip_h2f(exhip_f2h(v[e])) + exhip_h2f(r[e]);
+                }
+            }
+            if (p.post_relu) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    v[e] = exhip_h2f(exhip_f2h(v[e]));
+                    v[e] = (0.f > v[e]) ? 0.f : v[e];
+                }
+            }
+            if (p.post_op == EXHIP_POST_PRELU) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float t = exhip_h2f(exhip_f2h(v[e]));
+                    const float slope = p.post_slope[p.post_slope_shared || ch0 + e >= p.K ? 0 : ch0 + e];
+                    v[e] = t >= 0.f ? t : slope * t;
+                }
+            } else if (p.post_op) {
+                switch (p.post_op - 1) {
+                case EXHIP_UNARY_HARDSWISH: post_activation_op<0>(v, p.post_alpha, p.post_beta); break;
+                case EXHIP_UNARY_LEAKYRELU: post_activation_op<1>(v, p.post_alpha, p.post_beta); break;
+                case EXHIP_UNARY_HARDSIGMOID: post_activation_op<3>(v, p.post_alpha, p.post_beta); break;
+                default: post_activation_op<4>(v, p.post_alpha, p.post_beta); break;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
+            v4i o[2];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t lo = exhip_f2h(v[2 * e]), hi = exhip_f2h(v[2 * e + 1]);
+                o[e >> 2][e & 3] = (int)(lo | (hi << 16));
+            }
+            char* const yb = reinterpret_cast<char*>(p.y) + ch0 * 2;
+            if (ch0 + 16 <= p.kstride) {
+                if (__builtin_amdgcn_ballot_w64(valid) == ~0ull) {
+                    // the whole wave stores: a lane's 32 bytes and its neighbour's trade halves, so that four lanes (p,
+                    // p + 1 and the same two of the other half-wave) write 64 contiguous bytes of one pixel per instruction
+                    pair_exchange4(o[0], o[1], odd);
+                    const unsigned mine = pix[n], other = (unsigned)lane_neighbour((int)mine);
+                    const size_t even_pix = odd ? other : mine, odd_pix = odd ? mine : other;
+                    const int sub = odd ? 16 : 0;
+                    *reinterpret_cast<v4i*>(yb + even_pix * p.kstride * 2 + sub) = o[0];
+                    *reinterpret_cast<v4i*>(yb + odd_pix * p.kstride * 2 + sub) = o[1];
+                } else if (valid) {
+                    v4i* y = reinterpret_cast<v4i*>(yb + (size_t)pix[n] * p.kstride * 2);
+                    y[0] = o[0];
+                    y[1] = o[1];
+                }
+            } else if (valid) {
+                uint16_t* y = reinterpret_cast<uint16_t*>(yb + (size_t)pix[n] * p.kstride * 2);
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    if (ch0 + e < p.kstride) y[e] = (uint16_t)(((uint32_t)o[e >> 3][(e >> 1) & 3] >> ((e & 1) * 16)) & 0xffff);
+            }
+            // one 32 x 32 block at a time: interleaving the blocks buys nothing (they do not depend on each other's loads)
+            // and costs the registers of their temporaries
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int MT, int NT>
+__global__ __launch_bounds__(256, 2) void conv1x1_f16_pw_kernel(const PwParams p) {
+    constexpr int U = MT + NT > 4 ? 2 : 4;  // k-steps fetched per request round; two rounds are in flight
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // workgroup ids are dealt round-robin to the 8 XCDs: give each XCD one contiguous run of items, so that the channel
+    // groups of a pixel tile (and the weights' re-reads) share that XCD's L2
+    unsigned bid = blockIdx.x;
+    {
+        const unsigned per = gridDim.x >> 3;
+        if (bid < (per << 3)) bid = (bid & 7) * per + (bid >> 3);
+    }
+    const unsigned item = __builtin_amdgcn_readfirstlane(bid * 4 + wave);
+    if (item >= p.items) return;  // wave-uniform; the kernel has no barrier
+    const unsigned tile = __builtin_amdgcn_readfirstlane(item / p.ch_groups);
+    const int kb0 = __builtin_amdgcn_readfirstlane((int)(item - tile * p.ch_groups) * MT);  // first 32-channel block
+
+    const __amdgpu_buffer_rsrc_t xr = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(p.x), 0, (int)p.x_bytes, kRsrcWord3);
+    const __amdgpu_buffer_rsrc_t wr = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(p.wp), 0, (int)p.w_bytes, kRsrcWord3);
+
+    // pixel fragments: lane = pixel (lane & 31), 16-byte half (lane >> 5) of each 32-byte k-step
+    unsigned pix[NT];
+    int xoff[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+        pix[nt] = (tile * NT + nt) * 32 + (lane & 31);
+        xoff[nt] = pix[nt] < p.pixels ? (int)(pix[nt] * (unsigned)p.xs_b) + (lane >> 5) * 16 : kOutOfRange;
+    }
+    // weight fragments: block kb of slab kb / mts lies at ((slab * n_ksteps + ks) * mts + kb % mts) KiB; the MT blocks
+    // of a wave are neighbours in one slab (mts is a multiple of MT)
+    const int w_step = p.mts * 1024;
+    const int w_base = __builtin_amdgcn_readfirstlane(((kb0 / p.mts) * p.n_ksteps * p.mts + kb0 % p.mts) * 1024);
+    const int woff = lane * 16;
+
+    v16f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[m][n][e] = 0.f;
+
+    v4i a[2][U][MT], b[2][U][NT];
+    const int nks = p.n_ksteps;
+    auto request = [&](auto buf_c, int ks0) {
+        constexpr int buf = decltype(buf_c)::value;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (ks0 + u < nks) {
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+                    a[buf][u][m] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, woff + m * 1024, w_base + (ks0 + u) * w_step, 0));
+#pragma unroll
+                for (int n = 0; n < NT; ++n)
+                    b[buf][u][n] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(xr, xoff[n], (ks0 + u) * 32, 0));
+            }
+        }
+    };
+    auto compute = [&](auto buf_c, int ks0) {
+        constexpr int buf = decltype(buf_c)::value;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (ks0 + u < nks) {
+#pragma unroll
+                for (int m = 0; m < MT; ++m)
+#pragma unroll
+                    for (int n = 0; n < NT; ++n)
+                        acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a[buf][u][m]), __builtin_bit_cast(v8h, b[buf][u][n]),
+                                                                           acc[m][n], 0, 0, 0);
+            }
+        }
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    request(B0{}, 0);
+    for (int ks0 = 0; ks0 < nks; ks0 += 2 * U) {
+        request(B1{}, ks0 + U);
+        compute(B0{}, ks0);
+        request(B0{}, ks0 + 2 * U);
+        compute(B1{}, ks0 + U);
+    }
+
+    float bi[MT][16];
+    load_bias<MT>(p, kb0, lane, bi);
+    pw_epilogue<MT, NT>(p, acc, pix, kb0, lane, bi);
+}
+
+template <int MT, int NT>
+int launch(exhip_ctx* ctx, PwParams& p, int kblocks) {
+    const long long tiles = ((long long)p.pixels + 32 * NT - 1) / (32 * NT);
+    p.ch_groups = (unsigned)((kblocks + MT - 1) / MT);
+    const long long items = tiles * p.ch_groups;
+    if (items >= (1ll << 31)) return EXHIP_ERR_UNSUPPORTED;
+    p.items = (unsigned)items;
+    const unsigned grid = (unsigned)((items + 3) / 4);
+    hipLaunchKernelGGL((conv1x1_f16_pw_kernel<MT, NT>), dim3(grid), dim3(256), 0, ctx->stream, p);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+}  // namespace
+
+int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t* x, const void* wp, const float* bias,
+                         const uint16_t* residual, uint16_t* y) {
+    if (g_exhip_options.pw == 0) return EXHIP_ERR_UNSUPPORTED;
+    // Measured against the general kernel on the pointwise layers of a detection and a mobile network (16 and 64 images):
+    // this form wins where a launch is short, twice as fast on 20 x 20 maps, and for a lone 32-channel block (which the
+    // general kernel pads to a 64-channel slab); from about 2 GFLOP on, the general kernel's staged tiles re-read less
+    // and win. Option pw = 2 takes every layer the kernel can (tests).
+    const int blocks_needed = (std::max(g.k, g.k_stride) + 31) / 32;
+    const double flop = 2.0 * (double)g.pixels * (g.c_bytes / 2) * g.k;
+    if (g_exhip_options.pw != 2 && blocks_needed > 1 && (flop > 2.0e9 || g.pixels > 32768)) return EXHIP_ERR_UNSUPPORTED;
+    if (g.pixels <= 0 || g.c_bytes <= 0 || g.c_bytes % 32 != 0 || (g.slab_blocks != 2 && g.slab_blocks != 4) || g.k_stride % 8 != 0)
+        return EXHIP_ERR_UNSUPPORTED;
+    // lane offsets are 32-bit: the input tensor and the packed weights must stay below the out-of-range sentinel
+    const long long x_bytes = g.pixels * g.c_bytes;
+    const long long n_ksteps = g.c_bytes / 32;
+    const long long w_bytes = (long long)g.slabs * n_ksteps * g.slab_blocks * 1024;
+    if (x_bytes >= kOutOfRange || w_bytes >= kOutOfRange || g.pixels * 2 * g.k_stride >= (1ll << 40)) return EXHIP_ERR_UNSUPPORTED;
+    if (g.post_op && g.post_op != EXHIP_POST_PRELU && (g.post_op < 1 || g.post_op > 1 + EXHIP_UNARY_CLIP || g.post_op == 1 + EXHIP_UNARY_SIGMOID))
+        return EXHIP_ERR_UNSUPPORTED;
+    PwParams p = {};
+    p.x = reinterpret_cast<const char*>(x); p.wp = reinterpret_cast<const char*>(wp); p.bias = bias; p.residual = residual; p.y = y;
+    p.post_slope = g.post_slope;
+    p.pixels = (unsigned)g.pixels; p.x_bytes = (unsigned)x_bytes; p.w_bytes = (unsigned)w_bytes;
+    p.xs_b = g.c_bytes; p.n_ksteps = (int)n_ksteps; p.mts = g.slab_blocks;
+    p.K = g.k; p.kstride = g.k_stride;
+    p.act = g.act; p.post_relu = g.post_relu; p.post_op = g.post_op; p.post_slope_shared = g.post_slope_shared;
+    p.post_alpha = g.post_alpha; p.post_beta = g.post_beta;
+    // every packed block that holds a channel below max(k, k_stride): pad channels of the output are written as zeros
+    const int kblocks = std::min(g.slabs * g.slab_blocks, (std::max(g.k, g.k_stride) + 31) / 32);
+    // 64 x 64 per wave unless that leaves SIMDs without a wave: then 64 channels x 32 pixels; a lone 32-channel block
+    // takes 128 pixels per wave
+    if (kblocks == 1) return launch<1, 4>(ctx, p, kblocks);
+    const long long waves64 = ((g.pixels + 63) / 64) * ((kblocks + 1) / 2);
+    if (waves64 < 2048) return launch<2, 1>(ctx, p, kblocks);
+    return launch<2, 2>(ctx, p, kblocks);
+}

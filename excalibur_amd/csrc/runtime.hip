@@ -32,6 +32,7 @@ extern "C" int exhip_set_option(const char* name, int value) {
     else if (!strcmp(name, "share_gpu")) o.share_gpu = value;
     else if (!strcmp(name, "lean")) o.lean = value;
     else if (!strcmp(name, "lean_cfg")) o.lean_cfg = value;
+    else if (!strcmp(name, "pw")) o.pw = value;
     else if (!strcmp(name, "lean_groups")) o.lean_groups = value;
     else if (!strcmp(name, "lean_wres")) o.lean_wres = value;
     else if (!strcmp(name, "stem")) o.stem = value;

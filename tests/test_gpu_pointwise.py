@@ -1,0 +1,98 @@
+"""The pointwise (1x1 stride-1) fp16 kernel without staging (conv_pw.hip) against the general kernel, whose roundings
+it repeats (same packed weights, same order of the float32 sums: bit for bit), and against the CPU oracle at 2e-3."""
+import numpy as np
+import pytest
+
+from excalibur_amd import hip
+from oracle import port
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = hip.Ctx(0)
+    yield c
+    c.close()
+
+
+@pytest.fixture
+def options():
+    changed = []
+
+    def set_(name, value):
+        hip.set_option(name, value)
+        changed.append(name)
+    yield set_
+    defaults = dict(pw=1, force_splits=0)
+    for name in changed:
+        hip.set_option(name, defaults[name])
+
+
+def operands(seed, n, c, h, w, k, c_stride, k_stride, shortcut):
+    r = np.random.default_rng(seed)
+    x = np.zeros((n, h, w, c_stride), np.float16)
+    x[..., :c] = r.uniform(-1, 1, (n, h, w, c)).astype(np.float16)
+    wt = r.normal(0, 0.08, (k, c, 1, 1)).astype(np.float16)
+    bias = r.normal(0, 0.1, k).astype(np.float32)
+    res = r.uniform(-1, 1, (n, h, w, k_stride)).astype(np.float16) if shortcut else None
+    return x, wt, bias, res
+
+
+def run(ctx, n, c, h, w, k, x, wt, bias, res, c_stride, k_stride, act=0, post_relu=0, post_op=None, alpha=0.0, beta=0.0):
+    d = ctx.conv_desc(n, c, h, w, k, 1, 1, 0, act, c_stride, k_stride, post_relu, 0.0, post_op, alpha, beta)
+    xd = ctx.array(x.view(np.uint16))
+    wp = ctx.pack_conv_weights(d, hip.F16, wt.view(np.uint16))
+    bd = ctx.array(bias) if bias is not None else None
+    rd = ctx.array(res.view(np.uint16)) if res is not None else None
+    y = ctx.array(np.full((n, h, w, k_stride), 0x7e00, np.uint16))   # NaN bits: what the kernel leaves alone shows
+    ctx.conv2d_f16(d, xd, wp, bd, rd, y, None, None)
+    ctx.sync()
+    return y.download()
+
+
+SHAPES = [
+    # seed, n, c, h, w, k, c_stride, k_stride, shortcut, act, post_relu, post_op
+    (700, 2, 32, 56, 56, 64, 32, 64, False, 0, 0, None),            # MobileNet pointwise
+    (701, 1, 128, 40, 40, 255, 128, 256, False, 0, 0, None),        # detection head: ragged channels, one pad channel
+    (702, 1, 64, 33, 31, 64, 64, 64, True, 0, 1, None),             # 1023 pixels: a ragged last tile; shortcut + ReLU
+    (703, 3, 16, 9, 7, 32, 16, 32, False, 1, 0, None),              # one k-step, one 32-channel block (128 pixels per wave)
+    (704, 1, 48, 20, 20, 96, 48, 96, False, 0, 0, "hardswish"),     # three k-steps, three blocks in two slabs
+    (705, 1, 512, 20, 20, 256, 512, 256, False, 0, 0, "hardswish"),  # 32 k-steps: the request ring turns four times
+    (706, 1, 1024, 10, 10, 512, 1024, 512, False, 0, 0, "leakyrelu"),
+    (707, 2, 32, 256, 256, 32, 32, 32, False, 0, 0, "hardswish"),    # 131 072 pixels
+    (708, 2, 64, 200, 200, 64, 64, 64, True, 0, 0, None),            # 64 x 64 per wave, shortcut without ReLU
+    (709, 1, 40, 12, 12, 24, 48, 32, False, 3, 0, None),             # channel strides beyond the channel counts
+    (710, 1, 256, 40, 40, 128, 256, 128, False, 0, 0, "clip"),
+    (711, 1, 64, 17, 5, 128, 64, 128, False, 4, 0, None),            # sigmoid: the out-of-line activation
+]
+
+
+@pytest.mark.parametrize("args", SHAPES, ids=[f"s{a[0]}" for a in SHAPES])
+def test_pointwise_kernel_repeats_the_general_kernel_bit_for_bit(ctx, options, args):
+    seed, n, c, h, w, k, cs, ks, shortcut, act, post_relu, post_op = args
+    x, wt, bias, res = operands(seed, n, c, h, w, k, cs, ks, shortcut)
+    alpha, beta = {"hardswish": (1 / 6, 0.5), "leakyrelu": (0.1, 0.0), "clip": (-0.25, 0.5), None: (0.0, 0.0)}[post_op]
+    options("force_splits", 1)   # a small launch of the general kernel would split its sum, which changes its order
+    options("pw", 0)
+    want = run(ctx, n, c, h, w, k, x, wt, bias, res, cs, ks, act, post_relu, post_op, alpha, beta)
+    options("pw", 2)             # every layer the kernel can take, not only those it is faster on
+    got = run(ctx, n, c, h, w, k, x, wt, bias, res, cs, ks, act, post_relu, post_op, alpha, beta)
+    assert not np.any(want[..., :k] == 0x7e00)
+    assert np.array_equal(got, want), f"{np.count_nonzero(got != want)} of {want.size} halves differ"
+
+
+@pytest.mark.parametrize("args", [(720, 2, 32, 56, 56, 64), (721, 1, 128, 40, 40, 255), (722, 1, 512, 20, 20, 256), (723, 1, 64, 33, 31, 32)],
+                         ids=["s720", "s721", "s722", "s723"])
+def test_pointwise_kernel_within_2e3_of_the_oracle(ctx, options, args):
+    seed, n, c, h, w, k = args
+    options("pw", 2)
+    case = cases.conv_f32_case(seed, n, c, h, w, k, 1, 1, 0)
+    x16 = case["x"].astype(np.float16)
+    want = port.float2half(cases.oracle_eval(dict(case, x=x16.astype(np.float32)))).view(np.float16).astype(np.float32)
+    ks = hip.pad_to(k, 16)
+    got = run(ctx, n, c, h, w, k, np.ascontiguousarray(x16.transpose(0, 2, 3, 1)), case["wt"].astype(np.float16), case["bias"], None, c, ks,
+              act=case["act"])
+    got = got[..., :k].view(np.float16).astype(np.float32).transpose(0, 3, 1, 2)
+    assert cases.check_value(got, want, 2e-3) == 0
