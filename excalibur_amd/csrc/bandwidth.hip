@@ -1431,6 +1431,48 @@ __global__ __launch_bounds__(kBlock) void focus_x8_kernel(const float* __restric
     *reinterpret_cast<v4f*>(dst + (size_t)(g + 2) * C * OH * OW) = odd;
 }
 
+// The same on half storage (values are only moved): sixteen neighbouring inputs of a row per thread, 16 bytes to each
+// of the two output planes; rows of any other length take one output per thread.
+__global__ __launch_bounds__(kBlock) void focus_f16_x16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int C, int H, int W,
+                                                               size_t total16) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total16) return;
+    const int W16 = W / 16, OH = H / 2, OW = W / 2;
+    const int q = (int)(i % W16);
+    size_t t = i / W16;
+    const int iy = (int)(t % (2 * OH));
+    t /= 2 * OH;
+    const int c = (int)(t % C);
+    const size_t n = t / C;
+    const v4i* src = reinterpret_cast<const v4i*>(x + ((n * C + c) * H + iy) * W + 16 * q);
+    const v4i a = src[0], b = src[1];
+    v4i even, odd;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const unsigned lo = (unsigned)(e < 2 ? a[2 * e] : b[2 * e - 4]), hi = (unsigned)(e < 2 ? a[2 * e + 1] : b[2 * e - 3]);
+        even[e] = (int)((lo & 0xffffu) | (hi << 16));
+        odd[e] = (int)((lo >> 16) | (hi & 0xffff0000u));
+    }
+    const int g = iy & 1;
+    uint16_t* dst = y + ((n * 4 * C + c) * OH + iy / 2) * OW + 8 * q;
+    *reinterpret_cast<v4i*>(dst + (size_t)g * C * OH * OW) = even;
+    *reinterpret_cast<v4i*>(dst + (size_t)(g + 2) * C * OH * OW) = odd;
+}
+__global__ __launch_bounds__(kBlock) void focus_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y, int C, int H, int W,
+                                                           size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int OH = H / 2, OW = W / 2;
+    const int ox = (int)(i % OW);
+    size_t t = i / OW;
+    const int oy = (int)(t % OH);
+    t /= OH;
+    const int p = (int)(t % (4 * C));
+    const size_t n = t / (4 * C);
+    const int g = p / C, c = p % C;
+    y[i] = x[((n * C + c) * H + 2 * oy + g % 2) * W + 2 * ox + g / 2];
+}
+
 // Softmax over the channels of every (image, position) of an NCHW tensor: a thread owns one position and walks the
 // channels three times (maximum, exponentials and their sum, quotient); neighbouring threads read neighbouring
 // positions, so every access is coalesced.
@@ -1457,13 +1499,14 @@ __global__ __launch_bounds__(kBlock) void softmax_channels_kernel(const float* _
 }
 
 // Rows and columns of every plane change places, through a 32 x 32 LDS tile so that both sides are coalesced.
-__global__ __launch_bounds__(kBlock) void transpose_hw_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W) {
-    __shared__ float tile[32][33];
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_hw_kernel(const T* __restrict__ x, T* __restrict__ y, int H, int W) {
+    __shared__ T tile[32][33];
     const size_t plane = blockIdx.z;
     const int x0 = blockIdx.x * 32, y0 = blockIdx.y * 32;
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
-    const float* in = x + plane * H * W;
-    float* out = y + plane * H * W;
+    const T* in = x + plane * H * W;
+    T* out = y + plane * H * W;
 #pragma unroll
     for (int r = ty; r < 32; r += 8)
         if (y0 + r < H && x0 + tx < W) tile[r][tx] = in[(size_t)(y0 + r) * W + x0 + tx];
@@ -2487,11 +2530,35 @@ extern "C" int exhip_softmax_channels_f32(exhip_ctx* ctx, const float* x, float*
     return 0;
 }
 
+extern "C" int exhip_focus_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w) {
+    REQ_CTX("exhip_focus_f16");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && h > 1 && w > 1, "exhip_focus_f16: bad argument");
+    if (w % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)y % 16 == 0) {
+        const size_t total16 = (size_t)n * c * (h / 2 * 2) * (w / 16);
+        hipLaunchKernelGGL(focus_f16_x16_kernel, dim3(blocks_for(total16)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total16);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
+    const size_t total = (size_t)n * 4 * c * (h / 2) * (w / 2);
+    hipLaunchKernelGGL(focus_f16_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_transpose_hw_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int planes, int h, int w) {
+    REQ_CTX("exhip_transpose_hw_f16");
+    EXHIP_REQUIRE(x && y && planes > 0 && h > 0 && w > 0, "exhip_transpose_hw_f16: bad argument");
+    EXHIP_REQUIRE(planes <= 65535 && (h + 31) / 32 <= 65535, "exhip_transpose_hw_f16: more than 65535 planes or row tiles");
+    hipLaunchKernelGGL(transpose_hw_kernel<uint16_t>, dim3((w + 31) / 32, (h + 31) / 32, planes), dim3(kBlock), 0, ctx->stream, x, y, h, w);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" int exhip_transpose_hw_f32(exhip_ctx* ctx, const float* x, float* y, int planes, int h, int w) {
     REQ_CTX("exhip_transpose_hw_f32");
     EXHIP_REQUIRE(x && y && planes > 0 && h > 0 && w > 0, "exhip_transpose_hw_f32: bad argument");
     EXHIP_REQUIRE(planes <= 65535 && (h + 31) / 32 <= 65535, "exhip_transpose_hw_f32: more than 65535 planes or row tiles");
-    hipLaunchKernelGGL(transpose_hw_kernel, dim3((w + 31) / 32, (h + 31) / 32, planes), dim3(kBlock), 0, ctx->stream, x, y, h, w);
+    hipLaunchKernelGGL(transpose_hw_kernel<float>, dim3((w + 31) / 32, (h + 31) / 32, planes), dim3(kBlock), 0, ctx->stream, x, y, h, w);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

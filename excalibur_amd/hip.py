@@ -425,6 +425,12 @@ class Ctx:
         _check(lib().exhip_focus_f32(self.h, x.ptr, y.ptr, n, c, h, w))
         return y
 
+    def focus_f16(self, x):
+        n, c, h, w = x.shape
+        y = self.empty((n, 4 * c, h // 2, w // 2), np.uint16)
+        _check(lib().exhip_focus_f16(self.h, x.ptr, y.ptr, n, c, h, w))
+        return y
+
     def binaryop_f32(self, op, mode, large, small):
         """op 0 ADD / 1 SUB / 2 MUL / 3 DIV; mode 0 equal shapes, 1 per image, 2 per (image, channel), 3 per (image, pixel)."""
         n, c, h, w = large.shape
@@ -442,6 +448,12 @@ class Ctx:
         n, c, h, w = x.shape
         y = self.empty((n, c, w, h), np.float32)
         _check(lib().exhip_transpose_hw_f32(self.h, x.ptr, y.ptr, n * c, h, w))
+        return y
+
+    def transpose_hw_f16(self, x):
+        n, c, h, w = x.shape
+        y = self.empty((n, c, w, h), np.uint16)
+        _check(lib().exhip_transpose_hw_f16(self.h, x.ptr, y.ptr, n * c, h, w))
         return y
 
     def deconv2d_f32(self, x, w, bias, stride, pad):

@@ -370,6 +370,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 
 // src/Excalibur/operation_reshape.cpp:8-131: keys 0 / 1 / 2 = new width / height / channels (-233 when absent: that
@@ -386,6 +387,8 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
+    std::vector<int> new_shape(const std::vector<int>& old_shape, int count) const;
 };
 
 // src/Excalibur/operation_flatten.cpp:11-113: key 0 = axis (default 1); a copy with shape [n][1][h'][w'].
@@ -429,6 +432,7 @@ public:
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
+    void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };
 
 // src/Excalibur/operation_deconvolution.cpp:11-171: the convolution's keys; float32 weights [C][K][kh][kw]; group 1.

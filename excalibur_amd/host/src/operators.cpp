@@ -1490,6 +1490,16 @@ void operation_yolov5focus<Dtype>::forward_gpu_f32(const tensor_list<float>& bot
     EXHIP_FATAL(exhip_focus_f32(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num(), b->channels(), b->height(), b->width()));
 }
 
+// The fp16 pipeline's form: the layer only moves values, so it moves the halves (NCHW, as the float layer).
+template <typename Dtype>
+void operation_yolov5focus<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const half_ptr b = as_nchw(this->ctx(), bottoms[0], this->params_.device_);
+    tops[0] = new_tensor<unsigned short>({b->num(), b->channels() * 4, b->height() / 2, b->width() / 2}, this->params_.device_);
+    EXHIP_FATAL(exhip_focus_f16(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num(), b->channels(), b->height(), b->width()));
+}
+
 template <typename Dtype>
 operation_reshape<Dtype>::operation_reshape(const operation_param& param) : operation<Dtype>(param) {
     for (const layer_attr& a : parse_attrs(param.specific_params_)) {
@@ -1504,12 +1514,8 @@ operation_reshape<Dtype>::operation_reshape(const operation_param& param) : oper
 }
 
 template <typename Dtype>
-void operation_reshape<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
-    CHECK_EQ(bottoms.size(), 1);
-    CHECK_EQ(tops.size(), 1);
-    if (bottoms[0]->order() != memory::NCHW) NOT_IMPLEMENTED;
-    std::vector<int> shape = bottoms[0]->data_shape();
-    const int count = static_cast<int>(bottoms[0]->count());
+std::vector<int> operation_reshape<Dtype>::new_shape(const std::vector<int>& old_shape, int count) const {
+    std::vector<int> shape = old_shape;
     if (n_ > 0) shape[0] = n_;
     if (c_ > 0) shape[1] = c_;
     if (h_ > 0) shape[2] = h_;
@@ -1527,8 +1533,27 @@ void operation_reshape<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms
     if (h_ < 0) derive(2);
     if (w_ < 0) derive(3);
     CHECK_EQ(shape[0] * shape[1] * shape[2] * shape[3], count);
-    bottoms[0]->reshape(shape);
+    return shape;
+}
+
+template <typename Dtype>
+void operation_reshape<Dtype>::forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    if (bottoms[0]->order() != memory::NCHW) NOT_IMPLEMENTED;
+    bottoms[0]->reshape(new_shape(bottoms[0]->data_shape(), static_cast<int>(bottoms[0]->count())));
     tops[0] = bottoms[0];
+}
+
+// The fp16 pipeline's form: the NCHW blob itself takes the new shape, as in the float layer; an NHWC blob is brought
+// into NCHW order first (a new tensor, which then takes the shape).
+template <typename Dtype>
+void operation_reshape<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const half_ptr b = as_nchw(this->ctx(), bottoms[0], this->params_.device_);
+    b->reshape(new_shape(b->data_shape(), static_cast<int>(b->count())));
+    tops[0] = b;
 }
 
 template <typename Dtype>
@@ -1608,6 +1633,22 @@ void operation_transpose<Dtype>::forward_gpu_f32(const tensor_list<float>& botto
     } else if (perms_[0] == 1 && perms_[1] == 0 && perms_[2] == 2) {
         tops[0] = new_tensor<float>({b->num(), b->channels(), b->width(), b->height()}, this->params_.device_);
         EXHIP_FATAL(exhip_transpose_hw_f32(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num() * b->channels(),
+                                           b->height(), b->width()));
+    } else {
+        NOT_IMPLEMENTED << " Transpose order " << perms_[0] << "," << perms_[1] << "," << perms_[2];
+    }
+}
+
+template <typename Dtype>
+void operation_transpose<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) {
+    CHECK_EQ(bottoms.size(), 1);
+    CHECK_EQ(tops.size(), 1);
+    const half_ptr b = as_nchw(this->ctx(), bottoms[0], this->params_.device_);
+    if (perms_[0] == 0 && perms_[1] == 1 && perms_[2] == 2) {
+        tops[0] = b;
+    } else if (perms_[0] == 1 && perms_[1] == 0 && perms_[2] == 2) {
+        tops[0] = new_tensor<unsigned short>({b->num(), b->channels(), b->width(), b->height()}, this->params_.device_);
+        EXHIP_FATAL(exhip_transpose_hw_f16(this->ctx(), b->gpu_data(), tops[0]->mutable_gpu_data(), b->num() * b->channels(),
                                            b->height(), b->width()));
     } else {
         NOT_IMPLEMENTED << " Transpose order " << perms_[0] << "," << perms_[1] << "," << perms_[2];

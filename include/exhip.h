@@ -306,6 +306,9 @@ int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y, int n, in
 /* operation_yolov5focus::forward_cpu_f32 (operation_yolov5focus.cpp:17-50), for every image of the batch
  * (the reference fills image 0 only). y: [n][4c][h/2][w/2]. */
 int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w);
+/* The same on half storage: the reference's fp16 layer converts, runs the float layer and converts back
+ * (include/Excalibur/operation.hpp:204-266), which for a layer that only moves values is the move itself. */
+int exhip_focus_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w);
 
 /* operation_softmax::forward_cpu_f32, NCHW branch (src/Excalibur/operation_softmax.cpp:36-96): softmax over the channels of
  * every (image, position); x, y [n][c][hw]. */
@@ -313,6 +316,7 @@ int exhip_softmax_channels_f32(exhip_ctx* ctx, const float* x, float* y, int n, 
 /* operation_transpose::forward_cpu_f32, order (1, 0, 2) (src/Excalibur/operation_transpose.cpp:51-70): rows and columns of
  * each of `planes` planes change places, y[p][i][j] = x[p][j][i]; x [planes][h][w], y [planes][w][h]. */
 int exhip_transpose_hw_f32(exhip_ctx* ctx, const float* x, float* y, int planes, int h, int w);
+int exhip_transpose_hw_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int planes, int h, int w);  /* on half storage */
 
 /* operation_deconvolution::forward_cpu_f32 (src/Excalibur/operation_deconvolution.cpp:80-171), group 1, dilation 1:
  * x NCHW, w [c][k][kh][kw], y [n][k][(h-1)*sh + kh - pt - pb][(w-1)*sw + kw - pl - pr] = scatter of W^T x (+ bias). */

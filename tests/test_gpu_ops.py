@@ -380,6 +380,19 @@ def test_pool_nhwc_f16(ctx):
     assert np.array_equal(got, port.pool2d(x16.astype(np.float32), port.POOL_MAX, 3, 2, 1))
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 64, 96), (1, 3, 10, 14), (2, 5, 7, 9), (1, 1, 32, 16)], ids=str)
+def test_focus_and_transpose_on_half_storage_move_the_halves(ctx, shape):
+    """The fp16 pipeline's Focus and Transpose layers only move values: the halves land where the float layers put the
+    floats (rows of 16 take the vector kernel, others one element per thread; odd sizes drop their last row / column)."""
+    x = np.random.default_rng(385).integers(0, 1 << 16, shape).astype(np.uint16)
+    n, c, h, w = shape
+    want = np.concatenate([x[:, :, (g % 2):(h // 2) * 2:2, (g // 2):(w // 2) * 2:2] for g in range(4)], axis=1)
+    assert np.array_equal(ctx.focus_f16(ctx.array(x)).download(), want)
+    xf = x.astype(np.float32)
+    assert np.array_equal(ctx.focus_f32(ctx.array(xf)).download(), want.astype(np.float32))   # the float layer agrees on the order
+    assert np.array_equal(ctx.transpose_hw_f16(ctx.array(x)).download(), x.transpose(0, 1, 3, 2))
+
+
 def _half(a):
     """Round-to-nearest-even to half storage, widened again (what a tensor of the fp16 path holds)."""
     return a.astype(np.float16)
