@@ -1313,6 +1313,37 @@ __global__ __launch_bounds__(kBlock) void concat_nhwc_f16_kernel(ConcatNhwcArgs 
     reinterpret_cast<v4i*>(y)[i] = *reinterpret_cast<const v4i*>(a.src[k] + pix * ck + (c - a.first[k]));
 }
 
+// Concat (or a single blob) with the BatchNorm layer and the activation layer behind it applied on the way: the values are
+// those the layers produce one after the other (each stores halves, so the value is rounded to half between them).
+// UOP: -1 no activation, else unary_value's operation. p0 == nullptr: no BatchNorm.
+template <int UOP>
+__global__ __launch_bounds__(kBlock) void concat_affine_unary_nhwc_f16_kernel(ConcatNhwcArgs a, uint16_t* __restrict__ y, size_t total8,
+                                                                              const float* __restrict__ p0, const float* __restrict__ p1,
+                                                                              float alpha, float beta) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total8) return;
+    const int vecs = a.first[a.n_inputs] / 8;
+    const int vi = (int)(i % vecs);
+    const size_t pix = i / vecs;
+    const int c = vi * 8;
+    int k = 0;
+#pragma unroll
+    for (int j = 1; j < 8; ++j)
+        if (j < a.n_inputs && c >= a.first[j]) k = j;
+    const int ck = a.first[k + 1] - a.first[k];
+    v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(a.src[k] + pix * ck + (c - a.first[k]))), v8f);
+    if (p0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = channel_value<1>(v[e], p0[c + e], p1[c + e]);
+        if constexpr (UOP >= 0) v = __builtin_convertvector(__builtin_convertvector(v, v8h), v8f);
+    }
+    if constexpr (UOP >= 0) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = unary_value<UOP>(v[e], alpha, beta);
+    }
+    reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
+}
+
 // Nearest-neighbour resize of an NHWC half blob (channels a multiple of 8), the index rule of the NCHW kernel below.
 __global__ __launch_bounds__(kBlock) void interp_nearest_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                                          int H, int W, int C8, int OH, int OW, float hs, float ws,
@@ -2256,6 +2287,40 @@ extern "C" int exhip_concat_channels_nhwc_f16(exhip_ctx* ctx, const uint16_t* co
     EXHIP_REQUIRE((reinterpret_cast<uintptr_t>(y) & 15) == 0, "exhip_concat_channels_nhwc_f16: output must be 16-byte aligned");
     const size_t total8 = pixels * (size_t)(total / 8);
     hipLaunchKernelGGL(concat_nhwc_f16_kernel, dim3(blocks_for(total8)), dim3(kBlock), 0, ctx->stream, a, y, total8);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_concat_batchnorm_unary_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs, const int* channels, int n_inputs,
+                                                     size_t pixels, const float* bn_a, const float* bn_b, int unary_op, float alpha,
+                                                     float beta, uint16_t* y) {
+    REQ_CTX("exhip_concat_batchnorm_unary_nhwc_f16");
+    EXHIP_REQUIRE(inputs && channels && y && n_inputs >= 1 && n_inputs <= 8 && pixels > 0, "exhip_concat_batchnorm_unary_nhwc_f16: bad argument");
+    EXHIP_REQUIRE((bn_a == nullptr) == (bn_b == nullptr), "exhip_concat_batchnorm_unary_nhwc_f16: BatchNorm needs both parameter arrays");
+    ConcatNhwcArgs a = {};
+    a.n_inputs = n_inputs;
+    int total = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        EXHIP_REQUIRE(inputs[i] && channels[i] > 0 && channels[i] % 8 == 0 && (reinterpret_cast<uintptr_t>(inputs[i]) & 15) == 0,
+                      "exhip_concat_batchnorm_unary_nhwc_f16: input %d needs a multiple of 8 channels and 16-byte alignment", i);
+        a.src[i] = inputs[i];
+        a.first[i] = total;
+        total += channels[i];
+    }
+    a.first[n_inputs] = total;
+    EXHIP_REQUIRE((reinterpret_cast<uintptr_t>(y) & 15) == 0, "exhip_concat_batchnorm_unary_nhwc_f16: output must be 16-byte aligned");
+    const size_t total8 = pixels * (size_t)(total / 8);
+    const dim3 grid(blocks_for(total8)), block(kBlock);
+#define EXHIP_CAU(UOP) hipLaunchKernelGGL((concat_affine_unary_nhwc_f16_kernel<UOP>), grid, block, 0, ctx->stream, a, y, total8, bn_a, bn_b, alpha, beta)
+    switch (unary_op) {
+    case -1: EXHIP_CAU(-1); break;
+    case EXHIP_UNARY_HARDSWISH: EXHIP_CAU(0); break;
+    case EXHIP_UNARY_LEAKYRELU: EXHIP_CAU(1); break;
+    case EXHIP_UNARY_HARDSIGMOID: EXHIP_CAU(3); break;
+    case EXHIP_UNARY_CLIP: EXHIP_CAU(4); break;
+    default: exhip_set_error("exhip_concat_batchnorm_unary_nhwc_f16: activation %d is not one this kernel applies", unary_op); return EXHIP_ERR_ARG;
+    }
+#undef EXHIP_CAU
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -405,6 +405,22 @@ class Ctx:
                                                 int(shared)))
         return y
 
+    def concat_nhwc_f16(self, inputs, bn=None, unary=None, alpha=0.0, beta=0.0):
+        """Concat of NHWC half blobs along the channels; with bn=(a, b) and / or unary= the BatchNorm and activation layers
+        behind it in the same kernel (exhip_concat_batchnorm_unary_nhwc_f16), else the plain exhip_concat_channels_nhwc_f16."""
+        n, h, w, _ = inputs[0].shape
+        ptrs = (ctypes.c_void_p * len(inputs))(*[a.ptr.value for a in inputs])
+        ch = (ctypes.c_int * len(inputs))(*[a.shape[3] for a in inputs])
+        y = self.empty((n, h, w, sum(a.shape[3] for a in inputs)), np.uint16)
+        if bn is None and unary is None:
+            _check(lib().exhip_concat_channels_nhwc_f16(self.h, ptrs, ch, len(inputs), ctypes.c_size_t(n * h * w), y.ptr))
+        else:
+            _check(lib().exhip_concat_batchnorm_unary_nhwc_f16(self.h, ptrs, ch, len(inputs), ctypes.c_size_t(n * h * w),
+                                                               _ptr(bn[0] if bn else None), _ptr(bn[1] if bn else None),
+                                                               -1 if unary is None else self.UNARY[unary], ctypes.c_float(float(alpha)),
+                                                               ctypes.c_float(float(beta)), y.ptr))
+        return y
+
     def concat_channels_f32(self, inputs):
         n, _, h, w = inputs[0].shape
         ptrs = (ctypes.c_void_p * len(inputs))(*[a.ptr.value for a in inputs])

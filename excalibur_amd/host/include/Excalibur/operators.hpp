@@ -303,8 +303,16 @@ public:
     int channels_ = 0;
     float eps_ = 0.f;
     std::shared_ptr<memory::tensor<float>> a_, b_;
+    // fp16 pipeline: the activation layer on the next line (an EXHIP_UNARY_* operation other than the sigmoid) runs in this
+    // layer's kernel when the blob is NHWC; post_used() says whether it did.
+    void set_post_unary(int op, float alpha, float beta) { post_unary_ = op; post_alpha_ = alpha; post_beta_ = beta; post_used_ = false; }
+    void clear_post() { post_unary_ = -1; post_used_ = false; }
+    bool post_used() const { return post_used_; }
 
 protected:
+    int post_unary_ = -1;
+    float post_alpha_ = 0.f, post_beta_ = 0.f;
+    bool post_used_ = false;
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
     void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
     void fold();
@@ -336,8 +344,19 @@ public:
     explicit operation_concat(const operation_param& param);
     const char* type() const override { return this->params_.type_.c_str(); }
     int axis_ = 0;
+    // fp16 pipeline: the BatchNorm layer on the next line (its device-resident a / b; null = none) and the activation layer
+    // behind that (-1 = none) run in this layer's kernel when every blob is NHWC; post_used() says whether they did.
+    void set_post(const float* bn_a, const float* bn_b, int unary_op, float alpha, float beta) {
+        post_bn_a_ = bn_a; post_bn_b_ = bn_b; post_unary_ = unary_op; post_alpha_ = alpha; post_beta_ = beta; post_set_ = true; post_used_ = false;
+    }
+    void clear_post() { post_set_ = false; post_used_ = false; post_bn_a_ = post_bn_b_ = nullptr; post_unary_ = -1; }
+    bool post_used() const { return post_used_; }
 
 protected:
+    const float *post_bn_a_ = nullptr, *post_bn_b_ = nullptr;
+    int post_unary_ = -1;
+    float post_alpha_ = 0.f, post_beta_ = 0.f;
+    bool post_set_ = false, post_used_ = false;
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
     void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
 };

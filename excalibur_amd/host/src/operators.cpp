@@ -1287,9 +1287,17 @@ void operation_batchnorm<Dtype>::forward_gpu_f16(const tensor_list<unsigned shor
         CHECK_EQ(b->channels(), channels_);
         tops[i] = std::make_shared<tensor<unsigned short>>(b->data_shape(), this->params_.device_, b->order());
         if (b->order() == memory::NHWC) {
-            EXHIP_FATAL(exhip_channelwise_nhwc_f16(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(),
-                                                   static_cast<size_t>(b->num()) * b->height() * b->width(), b->channels(),
-                                                   a_->gpu_data(), b_->gpu_data(), 0));
+            const size_t pixels = static_cast<size_t>(b->num()) * b->height() * b->width();
+            if (post_unary_ >= 0 && bottoms.size() == 1 && b->channels() % 8 == 0) {
+                const unsigned short* src = b->gpu_data();
+                const int ch = b->channels();
+                EXHIP_FATAL(exhip_concat_batchnorm_unary_nhwc_f16(this->ctx(), &src, &ch, 1, pixels, a_->gpu_data(), b_->gpu_data(), post_unary_,
+                                                                  post_alpha_, post_beta_, tops[i]->mutable_gpu_data()));
+                post_used_ = true;
+                continue;
+            }
+            EXHIP_FATAL(exhip_channelwise_nhwc_f16(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(), pixels,
+                                                   b->channels(), a_->gpu_data(), b_->gpu_data(), 0));
             continue;
         }
         EXHIP_FATAL(exhip_channelwise_f16(this->ctx(), EXHIP_CHANNEL_BATCHNORM, b->gpu_data(), tops[i]->mutable_gpu_data(), b->num(),
@@ -1424,8 +1432,16 @@ void operation_concat<Dtype>::forward_gpu_f16(const tensor_list<unsigned short>&
     }
     const auto& b0 = in[0];
     tops[0] = new_tensor<unsigned short>({b0->num(), b0->height(), b0->width(), total}, dev, memory::NHWC);
-    EXHIP_FATAL(exhip_concat_channels_nhwc_f16(this->ctx(), ptrs.data(), channels.data(), static_cast<int>(ptrs.size()),
-                                               static_cast<size_t>(b0->num()) * b0->height() * b0->width(), tops[0]->mutable_gpu_data()));
+    const size_t pixels = static_cast<size_t>(b0->num()) * b0->height() * b0->width();
+    if (post_set_) {
+        EXHIP_FATAL(exhip_concat_batchnorm_unary_nhwc_f16(this->ctx(), ptrs.data(), channels.data(), static_cast<int>(ptrs.size()), pixels,
+                                                          post_bn_a_, post_bn_b_, post_unary_, post_alpha_, post_beta_,
+                                                          tops[0]->mutable_gpu_data()));
+        post_used_ = true;
+        return;
+    }
+    EXHIP_FATAL(exhip_concat_channels_nhwc_f16(this->ctx(), ptrs.data(), channels.data(), static_cast<int>(ptrs.size()), pixels,
+                                               tops[0]->mutable_gpu_data()));
 }
 
 template <typename Dtype>

@@ -182,6 +182,7 @@ public:
         }
         find_quantized_links();
         find_sum_pairs();
+        find_glue_chains();
     }
 
     // fp16 pipeline: a convolution whose only reader is the two-input sum on the next line (Eltwise SUM with unit
@@ -209,6 +210,53 @@ public:
                 if (!plain_sum || readers[mid] != 1 || op_outputs_[i + 1][0] == mid) continue;
                 if (std::find(output_names_.begin(), output_names_.end(), blob_names_[mid]) != output_names_.end()) continue;
                 sum_other_[i] = a == mid ? b : a;
+            }
+        }
+    }
+
+    // fp16 pipeline: a Concat whose only reader is the BatchNorm layer on the next line, and a BatchNorm (behind a Concat or
+    // not) whose only reader is the activation layer on the next line, run those layers in their own kernel: the blobs
+    // between them are never stored. Whether the kernel takes the NHWC path is known when the blobs are there, so the
+    // layer reports it and the absorbed layers run if it could not.
+    void find_glue_chains() {
+        chain_.assign(operations_.size(), glue_chain{});
+        if constexpr (std::is_same_v<Dtype, unsigned short>) {
+            std::vector<int> readers(blob_names_.size(), 0);
+            for (const auto& in : op_inputs_)
+                for (int b : in) ++readers[b];
+            // layer j (one input, one output) is the only reader of layer i's blob, which nobody asks for by name
+            auto follows = [&](size_t i, size_t j) {
+                if (j >= operations_.size() || op_outputs_[i].size() != 1 || op_inputs_[j].size() != 1 || op_outputs_[j].size() != 1) return false;
+                const int mid = op_outputs_[i][0];
+                if (op_inputs_[j][0] != mid) return false;
+                const bool in_place = op_outputs_[j][0] == mid;
+                const bool is_result = std::find(output_names_.begin(), output_names_.end(), blob_names_[mid]) != output_names_.end();
+                return in_place || (readers[mid] == 1 && !is_result);
+            };
+            auto activation = [&](size_t j) -> operation_unary<Dtype>* {
+                auto* u = j < operations_.size() ? dynamic_cast<operation_unary<Dtype>*>(operations_[j].get()) : nullptr;
+                return u && u->op_ != EXHIP_UNARY_SIGMOID ? u : nullptr;
+            };
+            for (size_t i = 0; i + 1 < operations_.size(); ++i) {
+                glue_chain g;
+                size_t last = i;
+                if (dynamic_cast<operation_concat<Dtype>*>(operations_[i].get())) {
+                    if (!follows(i, i + 1)) continue;
+                    if (dynamic_cast<operation_batchnorm<Dtype>*>(operations_[i + 1].get())) {
+                        g.bn = static_cast<int>(i + 1);
+                        last = i + 1;
+                    }
+                } else if (!dynamic_cast<operation_batchnorm<Dtype>*>(operations_[i].get())) {
+                    continue;
+                }
+                if (follows(last, last + 1) && activation(last + 1)) {
+                    g.unary = static_cast<int>(last + 1);
+                    last = last + 1;
+                }
+                if (last == i) continue;
+                g.last = static_cast<int>(last);
+                chain_[i] = g;
+                i = last;  // the absorbed layers start no chain of their own
             }
         }
     }
@@ -376,6 +424,35 @@ private:
                     continue;
                 }
             }
+            if constexpr (std::is_same_v<Dtype, unsigned short>) {
+                if (fusion_ && chain_[i].last > static_cast<int>(i)) {
+                    const glue_chain& g = chain_[i];
+                    auto* bn = g.bn >= 0 ? static_cast<operation_batchnorm<Dtype>*>(operations_[g.bn].get()) : nullptr;
+                    auto* un = g.unary >= 0 ? static_cast<operation_unary<Dtype>*>(operations_[g.unary].get()) : nullptr;
+                    bool used = false;
+                    if (auto* cat = dynamic_cast<operation_concat<Dtype>*>(operations_[i].get())) {
+                        cat->set_post(bn ? bn->a_->gpu_data() : nullptr, bn ? bn->b_->gpu_data() : nullptr, un ? un->op_ : -1,
+                                      un ? un->alpha_ : 0.f, un ? un->beta_ : 0.f);
+                        cat->forward_gpu(in, out);
+                        used = cat->post_used();
+                        cat->clear_post();
+                    } else {
+                        auto* first = static_cast<operation_batchnorm<Dtype>*>(operations_[i].get());
+                        first->set_post_unary(un->op_, un->alpha_, un->beta_);
+                        first->forward_gpu(in, out);
+                        used = first->post_used();
+                        first->clear_post();
+                    }
+                    if (used) {
+                        for (int j = static_cast<int>(i); j < g.last; ++j) featmaps_[op_outputs_[j][0]] = nullptr;
+                        featmaps_[op_outputs_[g.last][0]] = out[0];
+                        i = static_cast<size_t>(g.last);  // the absorbed layers have run
+                    } else {
+                        featmaps_[op_outputs_[i][0]] = out[0];
+                    }
+                    continue;
+                }
+            }
             if (fusion_ && (pair_[i].on || link_[i].on)) {
                 auto* conv = static_cast<operation_convolution<Dtype>*>(operations_[i].get());
                 if (pair_[i].on && pair_[i].prelu)
@@ -438,6 +515,10 @@ private:
         int stride = 0;
     };
     std::vector<int> sum_other_;         // per layer: the other operand's blob of the sum layer this convolution absorbs, or -1
+    struct glue_chain {
+        int bn = -1, unary = -1, last = -1;  // layer numbers of the absorbed BatchNorm / activation, and of the last absorbed layer
+    };
+    std::vector<glue_chain> chain_;      // per layer (fp16 pipeline): the layers behind a Concat or BatchNorm that run in its kernel
     std::vector<quantized_link> link_;   // per layer: an int8 convolution that writes its readers' int8 input
     int weights_mem_cost_ = 0;
 };

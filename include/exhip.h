@@ -288,6 +288,14 @@ int exhip_channelwise_nhwc_f16(exhip_ctx* ctx, int op, const uint16_t* x, uint16
  * detection topologies (operation_pooling.cpp:145-159), as a row pass into tmp (same size as x) and a column pass. */
 int exhip_concat_channels_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs, const int* channels, int n_inputs,
                                    size_t pixels, uint16_t* y);
+/* exhip_concat_channels_nhwc_f16 with the layers a detection topology puts behind its Concat applied on the way:
+ * BatchNorm (operation_batchnorm.cpp:122-156; bn_a / bn_b as exhip_channelwise_*'s p0 / p1 for the concatenated
+ * channels, both NULL = none) and then an activation layer (unary_op = EXHIP_UNARY_HARDSWISH / LEAKYRELU / HARDSIGMOID /
+ * CLIP, -1 = none). The results are those of the separate layers, each of which stores halves: the value is rounded
+ * to half after the BatchNorm step when an activation follows. n_inputs = 1: the two layers on one blob. */
+int exhip_concat_batchnorm_unary_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs, const int* channels, int n_inputs,
+                                          size_t pixels, const float* bn_a, const float* bn_b, int unary_op, float alpha,
+                                          float beta, uint16_t* y);
 int exhip_interp_nearest_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int oh, int ow);
 int exhip_maxpool_same_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* tmp, uint16_t* y, int n, int c, int h, int w, int k);
 /* exhip_maxpool_same_nhwc_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight

@@ -393,6 +393,27 @@ def test_focus_and_transpose_on_half_storage_move_the_halves(ctx, shape):
     assert np.array_equal(ctx.transpose_hw_f16(ctx.array(x)).download(), x.transpose(0, 1, 3, 2))
 
 
+@pytest.mark.parametrize("unary,alpha,beta", [("leakyrelu", 0.1, 0.0), ("hardswish", 1 / 6, 0.5), (None, 0.0, 0.0), ("clip", -0.5, 0.75)])
+@pytest.mark.parametrize("channels,with_bn", [((32, 32), True), ((64, 8, 24), True), ((16,), True), ((40, 24), False)], ids=str)
+def test_concat_batchnorm_activation_in_one_kernel_equals_the_separate_layers(ctx, channels, with_bn, unary, alpha, beta):
+    """Concat -> BatchNorm -> activation of the fp16 pipeline in one kernel against the three layers' own entry points
+    (each of which stores halves), on NHWC half blobs; one input = BatchNorm -> activation alone."""
+    r = np.random.default_rng(386)
+    n, h, w = 2, 9, 13
+    blobs = [ctx.array(r.normal(0, 2, (n, h, w, c)).astype(np.float16).view(np.uint16)) for c in channels]
+    total = sum(channels)
+    a = ctx.array(r.normal(0, 0.5, total).astype(np.float32))
+    b = ctx.array(r.uniform(0.5, 2, total).astype(np.float32))
+    want = ctx.concat_nhwc_f16(blobs) if len(blobs) > 1 else blobs[0]
+    if with_bn:
+        want = ctx.channelwise_nhwc_f16("batchnorm", want, a, b)
+    if unary:
+        want = ctx.unary_f16(unary, want, alpha, beta)
+    got = ctx.concat_nhwc_f16(blobs, (a, b) if with_bn else None, unary, alpha, beta)
+    ctx.sync()
+    assert np.array_equal(got.download(), want.download())
+
+
 def _half(a):
     """Round-to-nearest-even to half storage, widened again (what a tensor of the fp16 path holds)."""
     return a.astype(np.float16)
