@@ -90,6 +90,7 @@ struct ConvParams {
     int tiles_x, tiles_y, ktiles;
     int act, post_relu;
     int post_op;              // 0, or 1 + EXHIP_UNARY_*: the activation layer behind the convolution (general epilogue)
+    int residual_last;        // the shortcut is added behind post_relu / post_op (general epilogue)
     float post_alpha, post_beta;
     const float* post_slope;  // post_op == EXHIP_POST_PRELU: slopes per output channel (one for all if post_slope_shared)
     int post_slope_shared;
@@ -1138,7 +1139,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
 #pragma unroll
                     for (int e = 0; e < 16; ++e) v[e] = fast_activation(v[e], p.act);
                 }
-                if (p.residual) {
+                auto add_shortcut = [&]() {
                     if constexpr (DT == EXHIP_F16) {
                         // the add layer behind this one reads the stored (rounded) half
                         const uint16_t* r = reinterpret_cast<const uint16_t*>(p.residual) + pix * p.kstride + ch0;
@@ -1160,7 +1161,8 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                         for (int e = 0; e < 16; ++e)
                             if (ch0 + e < p.K) v[e] += r[e];
                     }
-                }
+                };
+                if (p.residual && !p.residual_last) add_shortcut();
                 if (p.post_relu) {
                     // a ReLU layer reads what this layer stored: in the fp16 pipeline the rounded half (a tiny negative
                     // value is -0 there and stays -0)
@@ -1181,6 +1183,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 } else if (p.post_op) {
                     post_activation<DT>(v, p.post_op - 1, p.post_alpha, p.post_beta);
                 }
+                if (p.residual && p.residual_last) add_shortcut();
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
                     if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
@@ -1604,7 +1607,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     if constexpr (DT == EXHIP_I8) {
         if (!pool) {
             const long long elems = (long long)d->n * pl.OH * pl.OW * d->k;
-            const bool fused = !p.acc_nchw && !d->post_op && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
+            const bool fused = !p.acc_nchw && !d->post_op && !d->residual_last && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
                                elems * 4 < 0xFFFFF000ll && elems < (long long)kEpiInvalid;
             const int epi_wave_b = !fused ? 0 : ((p.residual || p.y_nhwc) ? kEpiWaveBytes : 32 * kEpiRowQ + 128);
             rebuffer(pl, d, epi_wave_b, fused && pl.KWe == 3);
@@ -1628,6 +1631,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     p.tiles_x = pl.tiles_x; p.tiles_y = pl.tiles_y; p.ktiles = pl.ktiles;
     p.act = d->act; p.post_relu = d->post_relu; p.fs_out = d->fs_out; p.b_align = pl.b_align;
     p.post_op = d->post_op; p.post_alpha = d->post_alpha; p.post_beta = d->post_beta;
+    p.residual_last = d->residual_last && p.residual;
     p.post_slope = d->post_slope; p.post_slope_shared = d->post_slope_shared;
     EXHIP_REQUIRE((d->post_op >= 0 && d->post_op <= 1 + EXHIP_UNARY_CLIP && d->post_op != 1 + EXHIP_UNARY_SIGMOID) ||
                       (d->post_op == EXHIP_POST_PRELU && d->post_slope),
@@ -1681,7 +1685,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         }
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
-        const bool fused = !p.acc_nchw && !d->post_op && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
+        const bool fused = !p.acc_nchw && !d->post_op && !d->residual_last && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
                            out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
         if (fused && !pl.packed && p.splits == 1 && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
             p.cstride_b % 64 == 0) {
@@ -1713,7 +1717,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             g.pixels = (long long)d->n * d->h * d->w; g.c_bytes = p.cstride_b; g.k = d->k; g.k_stride = d->k_stride;
             g.slab_blocks = pl.TM / 32; g.slabs = pl.ktiles;
             g.act = d->act; g.post_relu = d->post_relu; g.post_op = d->post_op; g.post_slope_shared = d->post_slope_shared;
-            g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope;
+            g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope; g.residual_last = d->residual_last;
             rc = exhip_conv1x1_f16_pw(ctx, g, reinterpret_cast<const uint16_t*>(p.x), p.wp, p.bias, reinterpret_cast<const uint16_t*>(p.residual),
                                       reinterpret_cast<uint16_t*>(p.y_q));
             if (rc != EXHIP_ERR_UNSUPPORTED) return rc;

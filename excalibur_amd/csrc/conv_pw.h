@@ -10,6 +10,7 @@ struct exhip_pw_geom {
     int k, k_stride;            // output channels and the output's channel stride, in elements
     int slab_blocks, slabs;     // the packing: 32-channel blocks per slab (2 or 4) and slabs
     int act, post_relu, post_op, post_slope_shared;
+    int residual_last;          // the shortcut is added behind post_relu / post_op
     float post_alpha, post_beta;
     const float* post_slope;
 };

@@ -41,7 +41,7 @@ struct PwParams {
     int n_ksteps;                // 32-byte k-steps per pixel
     int mts;                     // 32-channel blocks per packed slab
     int K, kstride;
-    int act, post_relu, post_op, post_slope_shared;
+    int act, post_relu, post_op, post_slope_shared, residual_last;
     float post_alpha, post_beta;
 };
 
@@ -91,7 +91,7 @@ __device__ __forceinline__ void pw_epilogue(const PwParams& p, const v16f (&acc)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) v[e] = fast_activation(v[e], p.act);
             }
-            if (p.residual && valid) {
+            auto add_shortcut = [&]() {
                 // the add layer behind this one reads the stored (rounded) half
                 const uint16_t* r = p.residual + (size_t)pix[n] * p.kstride + ch0;
                 if (ch0 + 16 <= p.K) {
@@ -106,7 +106,8 @@ __device__ __forceinline__ void pw_epilogue(const PwParams& p, const v16f (&acc)
                     for (int e = 0; e < 16; ++e)
                         if (ch0 + e < p.K) v[e] = exhip_h2f(exhip_f2h(v[e])) + exhip_h2f(r[e]);
                 }
-            }
+            };
+            if (p.residual && valid && !p.residual_last) add_shortcut();
             if (p.post_relu) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
@@ -129,6 +130,7 @@ __device__ __forceinline__ void pw_epilogue(const PwParams& p, const v16f (&acc)
                 default: post_activation_op<4>(v, p.post_alpha, p.post_beta); break;
                 }
             }
+            if (p.residual && valid && p.residual_last) add_shortcut();
 #pragma unroll
             for (int e = 0; e < 16; ++e)
                 if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
@@ -293,7 +295,7 @@ int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t*
     p.pixels = (unsigned)g.pixels; p.x_bytes = (unsigned)x_bytes; p.w_bytes = (unsigned)w_bytes;
     p.xs_b = g.c_bytes; p.n_ksteps = (int)n_ksteps; p.mts = g.slab_blocks;
     p.K = g.k; p.kstride = g.k_stride;
-    p.act = g.act; p.post_relu = g.post_relu; p.post_op = g.post_op; p.post_slope_shared = g.post_slope_shared;
+    p.act = g.act; p.post_relu = g.post_relu; p.post_op = g.post_op; p.post_slope_shared = g.post_slope_shared; p.residual_last = g.residual_last && residual;
     p.post_alpha = g.post_alpha; p.post_beta = g.post_beta;
     // every packed block that holds a channel below max(k, k_stride): pad channels of the output are written as zeros
     const int kblocks = std::min(g.slabs * g.slab_blocks, (std::max(g.k, g.k_stride) + 31) / 32);

@@ -24,7 +24,7 @@ class ConvDesc(ctypes.Structure):
                 ("n", "c", "h", "w", "k", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr", "act", "c_stride", "k_stride",
                  "post_relu")] + [("fs_out", ctypes.c_float), ("post_op", ctypes.c_int), ("post_alpha", ctypes.c_float),
                                   ("post_beta", ctypes.c_float), ("post_slope", ctypes.c_void_p),
-                                  ("post_slope_shared", ctypes.c_int)]
+                                  ("post_slope_shared", ctypes.c_int), ("residual_last", ctypes.c_int)]
 
 
 _lib = None
@@ -190,13 +190,13 @@ class Ctx:
     # ---- convolution ----
     @staticmethod
     def conv_desc(n, c, h, w, k, kernel, stride=1, pad=0, act=0, c_stride=None, k_stride=None, post_relu=0, fs_out=0.0,
-                  post_op=None, post_alpha=0.0, post_beta=0.0):
+                  post_op=None, post_alpha=0.0, post_beta=0.0, residual_last=0):
         kh, kw = (kernel, kernel) if np.isscalar(kernel) else kernel
         sh, sw = (stride, stride) if np.isscalar(stride) else stride
         pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
         return ConvDesc(n, c, h, w, k, kh, kw, sh, sw, pt, pb, pl, pr, act, c_stride if c_stride else c,
                         k_stride if k_stride else k, post_relu, fs_out, 0 if post_op is None else 1 + Ctx.UNARY[post_op],
-                        post_alpha, post_beta)
+                        post_alpha, post_beta, None, 0, residual_last)
 
     @staticmethod
     def conv_out_hw(d):

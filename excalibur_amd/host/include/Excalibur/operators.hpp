@@ -66,11 +66,14 @@ public:
     void clear_post() {
         post_op_ = 0; post_alpha_ = post_beta_ = 0.f; post_relu_ = false;
         post_slope_ = nullptr; post_slope_shared_ = false;
-        post_sum_.reset(); post_sum_used_ = false;
+        post_sum_.reset(); post_sum_used_ = false; post_sum_last_ = false;
     }
-    // fp16 layers: the other operand of the two-input sum layer behind this one. The next forward adds it in the
-    // kernel's epilogue if it can (NHWC result, an NHWC operand of the result's shape) and says so in post_sum_used().
-    void set_post_sum(const std::shared_ptr<memory::tensor<unsigned short>>& other) { post_sum_ = other; post_sum_used_ = false; }
+    // fp16 layers: the other operand of the two-input sum layer behind this one, or (behind_activation) behind the
+    // activation layer set with set_post_activation / set_post_prelu. The next forward adds it in the kernel's epilogue
+    // if it can (NHWC result, an NHWC operand of the result's shape) and says so in post_sum_used().
+    void set_post_sum(const std::shared_ptr<memory::tensor<unsigned short>>& other, bool behind_activation = false) {
+        post_sum_ = other; post_sum_used_ = false; post_sum_last_ = behind_activation;
+    }
     bool post_sum_used() const { return post_sum_used_; }
     // int8 layers on the MFMA kernel. The next forward calls also write the int8 NHWC form of the output that a reader
     // quantizing with `fs` into `stride` channels per pixel would make of it (attached to the top blob as its
@@ -91,7 +94,7 @@ protected:
     const float* post_slope_ = nullptr;
     bool post_slope_shared_ = false;
     std::shared_ptr<memory::tensor<unsigned short>> post_sum_;
-    bool post_sum_used_ = false;
+    bool post_sum_used_ = false, post_sum_last_ = false;
     float q_out_fs_ = 0.f;
     int q_out_stride_ = 0;
     bool q_out_only_ = false;

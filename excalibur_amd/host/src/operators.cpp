@@ -553,9 +553,10 @@ void operation_convolution<Dtype>::forward_gpu_f16(const tensor_list<unsigned sh
                        : new_tensor<unsigned short>({n, this->output_channel_, oh, ow}, dev);
     unsigned short* y = tops[0]->mutable_gpu_data();
     const unsigned short* residual = nullptr;
-    if (post_sum_ && out_nhwc && post_sum_->order() == memory::NHWC && post_sum_->data_shape() == tops[0]->data_shape() && !post_op_ &&
-        !post_relu_) {
+    if (post_sum_ && out_nhwc && post_sum_->order() == memory::NHWC && post_sum_->data_shape() == tops[0]->data_shape() &&
+        (post_sum_last_ || (!post_op_ && !post_relu_))) {
         residual = post_sum_->gpu_data();
+        d.residual_last = post_sum_last_ ? 1 : 0;
         post_sum_used_ = true;
     }
     EXHIP_FATAL(exhip_conv2d_f16(this->ctx(), &d, x->gpu_data(), packed_weights(EXHIP_F16, d), bias_gpu(), residual,

@@ -189,6 +189,8 @@ public:
     // coefficients, BinaryOp ADD of two blobs: the residual add of a bottleneck block) adds the other operand in its
     // epilogue, to its own result rounded to half as the sum layer would read it. Whether it can is known only when the
     // blobs are there (both NHWC, same shape), so the convolution reports it and the sum layer runs if it could not.
+    // The sum may also stand behind the activation layer that already runs in the convolution's epilogue (convolution ->
+    // HardSwish -> add, the bottleneck of the detection topologies): the epilogue then adds behind the activation.
     void find_sum_pairs() {
         sum_other_.assign(operations_.size(), -1);
         if constexpr (std::is_same_v<Dtype, unsigned short>) {
@@ -197,17 +199,22 @@ public:
                 for (int b : in) ++readers[b];
             for (size_t i = 0; i + 1 < operations_.size(); ++i) {
                 auto* conv = dynamic_cast<operation_convolution<Dtype>*>(operations_[i].get());
-                if (!conv || dynamic_cast<operation_convolutiondepthwise<Dtype>*>(conv) || pair_[i].on) continue;
-                if (op_outputs_[i].size() != 1 || op_inputs_[i + 1].size() != 2 || op_outputs_[i + 1].size() != 1) continue;
-                const int mid = op_outputs_[i][0];
-                const int a = op_inputs_[i + 1][0], b = op_inputs_[i + 1][1];
-                if ((a == mid) == (b == mid)) continue;  // exactly one operand is the convolution's blob
+                if (!conv || dynamic_cast<operation_convolutiondepthwise<Dtype>*>(conv)) continue;
+                // the layer whose top the sum reads: the convolution, or the activation layer that runs in its epilogue
+                const size_t last = pair_[i].on ? i + 1 : i;
+                if (last + 1 >= operations_.size()) continue;
+                if (op_outputs_[last].size() != 1 || op_inputs_[last + 1].size() != 2 || op_outputs_[last + 1].size() != 1) continue;
+                const int mid = op_outputs_[last][0];
+                const int a = op_inputs_[last + 1][0], b = op_inputs_[last + 1][1];
+                if ((a == mid) == (b == mid)) continue;  // exactly one operand is the blob
                 bool plain_sum = false;
-                if (auto* e = dynamic_cast<operation_eltwise<Dtype>*>(operations_[i + 1].get()))
+                if (auto* e = dynamic_cast<operation_eltwise<Dtype>*>(operations_[last + 1].get()))
                     plain_sum = e->type_ == 1 && e->coeffs_.size() == 2 && e->coeffs_[0] == 1.f && e->coeffs_[1] == 1.f;
-                else if (auto* bo = dynamic_cast<operation_binaryop<Dtype>*>(operations_[i + 1].get()))
+                else if (auto* bo = dynamic_cast<operation_binaryop<Dtype>*>(operations_[last + 1].get()))
                     plain_sum = bo->op_type_ == 0 && !bo->with_scalar_;
-                if (!plain_sum || readers[mid] != 1 || op_outputs_[i + 1][0] == mid) continue;
+                // an activation writing over its input reads the blob as well
+                const int own_readers = pair_[i].on && op_outputs_[i][0] == mid ? 2 : 1;
+                if (!plain_sum || readers[mid] != own_readers || op_outputs_[last + 1][0] == mid) continue;
                 if (std::find(output_names_.begin(), output_names_.end(), blob_names_[mid]) != output_names_.end()) continue;
                 sum_other_[i] = a == mid ? b : a;
             }
@@ -410,17 +417,20 @@ private:
             if constexpr (std::is_same_v<Dtype, unsigned short>) {
                 if (fusion_ && sum_other_[i] >= 0 && featmaps_[sum_other_[i]]) {
                     auto* conv = static_cast<operation_convolution<Dtype>*>(operations_[i].get());
-                    conv->set_post_sum(featmaps_[sum_other_[i]]);
+                    const bool paired = pair_[i].on;  // the activation layer between the convolution and the sum
+                    if (paired && pair_[i].prelu)
+                        conv->set_post_prelu(pair_[i].prelu->weights_f32()[0]->gpu_data(), pair_[i].prelu->share_channel_);
+                    else if (paired)
+                        conv->set_post_activation(pair_[i].post_op, pair_[i].alpha, pair_[i].beta, pair_[i].relu);
+                    conv->set_post_sum(featmaps_[sum_other_[i]], paired);
                     conv->forward_gpu(in, out);
                     const bool summed = conv->post_sum_used();
                     conv->clear_post();
-                    if (summed) {
-                        featmaps_[op_outputs_[i][0]] = nullptr;
-                        featmaps_[op_outputs_[i + 1][0]] = out[0];
-                        ++i;  // the sum layer has run
-                    } else {
-                        featmaps_[op_outputs_[i][0]] = out[0];
-                    }
+                    size_t done = i;  // the last layer whose work the launch did
+                    if (paired) featmaps_[op_outputs_[done++][0]] = nullptr;
+                    if (summed) featmaps_[op_outputs_[done++][0]] = nullptr;
+                    featmaps_[op_outputs_[done][0]] = out[0];
+                    i = done;
                     continue;
                 }
             }

@@ -113,6 +113,8 @@ typedef struct exhip_conv_desc {
                                  * (operation_prelu.cpp:57-124), v >= 0 ? v : slope * v with these device-resident
                                  * slopes, one per output channel, or one for all if post_slope_shared */
     int post_slope_shared;
+    int residual_last;          /* 1: the shortcut is added behind post_relu / post_op instead of in front of them (a sum
+                                 * layer behind the activation layer that follows the convolution; general epilogue only) */
 } exhip_conv_desc;
 #define EXHIP_POST_PRELU 16
 

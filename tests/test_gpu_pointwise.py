@@ -40,8 +40,9 @@ def operands(seed, n, c, h, w, k, c_stride, k_stride, shortcut):
     return x, wt, bias, res
 
 
-def run(ctx, n, c, h, w, k, x, wt, bias, res, c_stride, k_stride, act=0, post_relu=0, post_op=None, alpha=0.0, beta=0.0):
-    d = ctx.conv_desc(n, c, h, w, k, 1, 1, 0, act, c_stride, k_stride, post_relu, 0.0, post_op, alpha, beta)
+def run(ctx, n, c, h, w, k, x, wt, bias, res, c_stride, k_stride, act=0, post_relu=0, post_op=None, alpha=0.0, beta=0.0, residual_last=0,
+        kernel=1):
+    d = ctx.conv_desc(n, c, h, w, k, kernel, 1, kernel // 2, act, c_stride, k_stride, post_relu, 0.0, post_op, alpha, beta, residual_last)
     xd = ctx.array(x.view(np.uint16))
     wp = ctx.pack_conv_weights(d, hip.F16, wt.view(np.uint16))
     bd = ctx.array(bias) if bias is not None else None
@@ -96,3 +97,24 @@ def test_pointwise_kernel_within_2e3_of_the_oracle(ctx, options, args):
               act=case["act"])
     got = got[..., :k].view(np.float16).astype(np.float32).transpose(0, 3, 1, 2)
     assert cases.check_value(got, want, 2e-3) == 0
+
+
+@pytest.mark.parametrize("kernel,pw", [(1, 0), (1, 2), (3, 0)], ids=["general-1x1", "pointwise", "general-3x3"])
+def test_shortcut_behind_the_activation_equals_the_sum_layer(ctx, options, kernel, pw):
+    """convolution -> HardSwish -> add in one launch (residual_last) == the launch without the shortcut, then the sum layer
+    on the stored halves."""
+    n, c, h, w, k = 2, 64, 20, 24, 64
+    r = np.random.default_rng(730 + kernel)
+    x = r.uniform(-1, 1, (n, h, w, c)).astype(np.float16)
+    wt = r.normal(0, 0.08, (k, c, kernel, kernel)).astype(np.float16)
+    bias = r.normal(0, 0.1, k).astype(np.float32)
+    res = r.uniform(-1, 1, (n, h, w, k)).astype(np.float16)
+    options("pw", pw)
+    plain = run(ctx, n, c, h, w, k, x, wt, bias, None, c, k, post_op="hardswish", alpha=1 / 6, beta=0.5, kernel=kernel)
+    want = ctx.add_f16(ctx.array(plain), ctx.array(res.view(np.uint16))).download()
+    assert np.array_equal(want, (plain.view(np.float16).astype(np.float32) + res.astype(np.float32)).astype(np.float16).view(np.uint16))
+    got = run(ctx, n, c, h, w, k, x, wt, bias, res, c, k, post_op="hardswish", alpha=1 / 6, beta=0.5, residual_last=1, kernel=kernel)
+    assert np.array_equal(got, want), f"{np.count_nonzero(got != want)} of {want.size} halves differ"
+    # in front of the activation (the default) the shortcut gives other values
+    front = run(ctx, n, c, h, w, k, x, wt, bias, res, c, k, post_op="hardswish", alpha=1 / 6, beta=0.5, kernel=kernel)
+    assert not np.array_equal(front, want)
