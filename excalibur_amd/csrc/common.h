@@ -70,6 +70,8 @@ struct exhip_options {
     int lean_stagger = 0;    // experiment: start delay per hardware wave slot, in units of 64 cycles
     int stem = 1;            // the stem (quantizer + first convolution + max pooling) as one kernel where the entry point offers it
     int lean_groups = 0;     // at most this many groups per 64-channel slab (tests: a few groups that walk many patches each)
+    int lean_f16 = 1;        // 3x3 stride-1 fp16 layers with an NHWC result on the lean kernel: 0 never, 1 the form per layer class, 2 one group per
+                             // patch, 3 persistent groups with three slice buffers, 4 persistent groups with two
     int pw = 1;              // 1x1 stride-1 fp16 layers with an NHWC result: 1 the pointwise kernel where it measured faster, 2 wherever it can run, 0 never
 };
 extern exhip_options g_exhip_options;

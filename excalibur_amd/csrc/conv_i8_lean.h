@@ -29,3 +29,12 @@ struct exhip_lean_proj {
 int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
                           const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw,
                           const exhip_lean_proj* proj = nullptr);
+
+// The fp16 3x3 stride-1 layer on the same kernel: half operands and result, the general kernel's fp16 epilogue.
+struct exhip_lean_f16_epilogue {
+    int post_op;              // 0, or 1 + EXHIP_UNARY_*: the activation layer behind the convolution
+    float post_alpha, post_beta;
+    int residual_last;        // the shortcut is added behind post_relu / post_op
+};
+int exhip_conv3x3_f16_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const exhip_lean_f16_epilogue& e, const uint16_t* x, const void* wp,
+                           const float* bias, const uint16_t* residual, uint16_t* y);

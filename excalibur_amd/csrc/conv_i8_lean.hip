@@ -26,6 +26,8 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 namespace {
 
@@ -46,7 +48,10 @@ constexpr unsigned kOobElem = 0x3FFFFF00u;    // an element offset whose byte of
 constexpr bool kStamps = EXHIP_STAMPS != 0;
 long long* g_lean_dbg = nullptr;
 
-enum { E_RES = 1, E_F = 2, E_Q = 4, E_NCHW = 8, E_ACT = 16, E_POST = 32, E_QNN = 64 };
+// E_HALF: the fp16 layer -- half operands (v_mfma_f32_32x32x16_f16 on the same bytes: a 64-byte chunk is 32 channels),
+// float accumulators, the general kernel's fp16 epilogue with a half NHWC result (its switches are read from the
+// parameters: E_RES / E_ACT / E_POST and post_op, residual_last).
+enum { E_RES = 1, E_F = 2, E_Q = 4, E_NCHW = 8, E_ACT = 16, E_POST = 32, E_QNN = 64, E_HALF = 128 };
 
 struct LeanParams {
     const char* x;
@@ -73,6 +78,9 @@ struct LeanParams {
     const float* ds_bias;
     int ds_H, ds_W, ds_Cb, ds_chunks, ds_stride;
     unsigned ds_img_bytes;
+    // fp16 layers (E_HALF): the activation layer behind the convolution and where the shortcut is added
+    int post_op, residual_last;
+    float post_alpha, post_beta;
     int stagger;     // persistent launches: a group whose waves sit in hardware wave slot s starts s * stagger * 64 cycles late
     long long* dbg;  // phase timestamps (builds with -DEXHIP_STAMPS=1 only)
 };
@@ -130,7 +138,10 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
     const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
     float* const lds_sb = reinterpret_cast<float*>(smem + SB0);
 
-    const int flags = EPI >= 0 ? EPI : p.flags;
+    constexpr bool F16 = EPI >= 0 && (EPI & E_HALF) != 0;
+    static_assert(!(F16 && PROJ), "the projection form is int8");
+    using acc_t = std::conditional_t<F16, v16f, v16i>;
+    const int flags = F16 ? p.flags : (EPI >= 0 ? EPI : p.flags);
     const bool has_res = flags & E_RES, has_f = flags & E_F, has_q = flags & E_Q, has_nchw = flags & E_NCHW;
     const bool act_relu = flags & E_ACT, post_relu = flags & E_POST, q_nonneg = flags & E_QNN;
     const bool q_only = q_nonneg && has_q && !has_res && !has_f && !has_nchw;
@@ -257,8 +268,8 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
     const int row_b = p.IW * kPixB;
     const int img_px = p.OH * p.OW;
 
-    v16i acc[2][2];
-    v16i acc_ds[2][2];  // PROJ: the projection's products
+    acc_t acc[2][2];
+    acc_t acc_ds[2][2];  // PROJ: the projection's products
     auto clear_acc = [&]() {
 #pragma unroll
         for (int m = 0; m < 2; ++m)
@@ -350,7 +361,13 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
 #pragma unroll
         for (int m = 0; m < 2; ++m)
 #pragma unroll
-            for (int nn = 0; nn < 2; ++nn) acc[m][nn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][m], bf[buf][nn], acc[m][nn], 0, 0, 0);
+            for (int nn = 0; nn < 2; ++nn) {
+                if constexpr (F16)
+                    acc[m][nn] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, af[buf][m]), __builtin_bit_cast(v8h, bf[buf][nn]),
+                                                                        acc[m][nn], 0, 0, 0);
+                else
+                    acc[m][nn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[buf][m], bf[buf][nn], acc[m][nn], 0, 0, 0);
+            }
     };
     auto fetch = [&](int buf, const char* wrow, const char* a0, const char* a1, int s) {
         af[buf][0] = lds_read16(wrow + s * 2048);
@@ -392,7 +409,8 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
 #pragma unroll
             for (int m = 0; m < 2; ++m)
 #pragma unroll
-                for (int nn = 0; nn < 2; ++nn) acc_ds[m][nn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[s][m], bf[s][nn], acc_ds[m][nn], 0, 0, 0);
+                for (int nn = 0; nn < 2; ++nn)
+                    if constexpr (!F16) acc_ds[m][nn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[s][m], bf[s][nn], acc_ds[m][nn], 0, 0, 0);
     };
     constexpr std::integral_constant<int, 1> one_row{};
     constexpr std::integral_constant<int, 3> three_rows{};
@@ -407,6 +425,89 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
     auto epilogue = [&](int n, int oy0, int ox0) {
         const bool full = oy0 + p.PH <= p.OH && ox0 + p.PW <= p.OW;
         const unsigned obase = ((unsigned)n * (unsigned)img_px + (unsigned)(oy0 * p.OW + ox0)) * (unsigned)p.K + (unsigned)(kt * 64);
+        if constexpr (F16) {
+            // The general kernel's fp16 epilogue (conv_igemm.hip) on 16 consecutive channels of a pixel per block: bias,
+            // ReLU, the shortcut added to the value rounded to half (in front of or behind the activation layer), the
+            // activation layer on the rounded half, one rounding; 64-byte runs from lanes (p, p + 1) of both half-waves.
+            // Every wave issues the same eight stores and, with a shortcut, eight loads, whatever its pixels: what lies
+            // outside the image goes to an offset the buffer view drops.
+            const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(p.y_q, 0, (int)(p.out_elems * 2u), kRsrcWord3);
+            const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.residual), 0, (int)(p.out_elems * 2u), kRsrcWord3);
+            const bool odd = lane & 1;
+#pragma unroll
+            for (int nn = 0; nn < 2; ++nn) {
+                int py, px;
+                const bool in_patch = patch_pixel(nn, py, px);
+                const bool valid = in_patch & (full | ((oy0 + py < p.OH) & (ox0 + px < p.OW)));
+                const unsigned mine = valid ? (obase + (unsigned)((py * p.OW + px) * p.K)) * 2u : (unsigned)kOob;
+                const unsigned other = (unsigned)lane_neighbour((int)mine);
+                const unsigned even_b = odd ? other : mine, odd_b = odd ? mine : other;
+#pragma unroll
+                for (int m = 0; m < 2; ++m) {
+                    const int cb = (m * 32 + hh * 16) * 2;  // byte offset of the lane's 16 channels in the pixel's slab
+                    v4i r0 = {0, 0, 0, 0}, r1 = {0, 0, 0, 0};
+                    if (has_res) {
+                        r0 = __builtin_amdgcn_raw_buffer_load_b128(rh, (int)mine + cb, 0, 0);
+                        r1 = __builtin_amdgcn_raw_buffer_load_b128(rh, (int)mine + cb + 16, 0, 0);
+                    }
+                    float v[16];
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) v[e] = acc[m][nn][e] + lds_sb[64 + m * 32 + hh * 16 + e];
+                    if (act_relu) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) v[e] = (0.f > v[e]) ? 0.f : v[e];
+                    }
+                    auto add_shortcut = [&]() {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            const int word = e < 8 ? r0[e >> 1] : r1[(e - 8) >> 1];
+                            v[e] = exhip_h2f(exhip_f2h(v[e])) + exhip_h2f((uint16_t)(((uint32_t)word >> ((e & 1) * 16)) & 0xffff));
+                        }
+                    };
+                    if (has_res && !p.residual_last) add_shortcut();
+                    if (post_relu) {
+#pragma unroll
+                        for (int e = 0; e < 16; ++e) {
+                            v[e] = exhip_h2f(exhip_f2h(v[e]));
+                            v[e] = (0.f > v[e]) ? 0.f : v[e];
+                        }
+                    }
+                    if (p.post_op) {
+                        const float al = p.post_alpha, be = p.post_beta;
+                        switch (p.post_op - 1) {
+                        case EXHIP_UNARY_HARDSWISH:
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) v[e] = unary_value<0>(exhip_h2f(exhip_f2h(v[e])), al, be);
+                            break;
+                        case EXHIP_UNARY_LEAKYRELU:
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) v[e] = unary_value<1>(exhip_h2f(exhip_f2h(v[e])), al, be);
+                            break;
+                        case EXHIP_UNARY_HARDSIGMOID:
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) v[e] = unary_value<3>(exhip_h2f(exhip_f2h(v[e])), al, be);
+                            break;
+                        default:
+#pragma unroll
+                            for (int e = 0; e < 16; ++e) v[e] = unary_value<4>(exhip_h2f(exhip_f2h(v[e])), al, be);
+                            break;
+                        }
+                    }
+                    if (has_res && p.residual_last) add_shortcut();
+                    v4i o0, o1;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const uint32_t lo = exhip_f2h(v[2 * e]), hi = exhip_f2h(v[2 * e + 1]);
+                        if (e < 4) o0[e] = (int)(lo | (hi << 16));
+                        else o1[e - 4] = (int)(lo | (hi << 16));
+                    }
+                    pair_exchange4(o0, o1, odd);
+                    __builtin_amdgcn_raw_buffer_store_b128(o0, ry, (int)even_b + cb + (odd ? 16 : 0), 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(o1, ry, (int)odd_b + cb + (odd ? 16 : 0), 0, 0);
+                }
+            }
+            return;
+        }
         unsigned eoff[2], noff[2], feven[2], fodd[2];
         const bool odd_lane = lane & 1;
 #pragma unroll
@@ -550,7 +651,7 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
         }
     };
     // stores an epilogue issues (they stand behind the next tile's request in the wave's memory queue)
-    constexpr int kEpiStores = EPI < 0 ? 64 : ((EPI & E_F) ? 16 : 0) + ((EPI & E_Q) ? 4 : 0) + ((EPI & E_NCHW) ? 64 : 0);
+    constexpr int kEpiStores = EPI < 0 ? 64 : F16 ? 8 : ((EPI & E_F) ? 16 : 0) + ((EPI & E_Q) ? 4 : 0) + ((EPI & E_NCHW) ? 64 : 0);
     constexpr int kWaitBehindEpi = EPI < 0 ? 0 : (kEpiStores < 60 ? kEpiStores : 60);
 
     // ---- the run ----
@@ -561,7 +662,7 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
     int base = set_offsets(oy0, ox0);
     if (tid < 128) {
         const int ch = kt * 64 + (tid & 63);
-        lds_sb[tid] = tid < 64 ? p.scale[ch] : (p.bias ? p.bias[ch] : 0.f);
+        lds_sb[tid] = tid < 64 ? (F16 ? 1.f : p.scale[ch]) : (p.bias ? p.bias[ch] : 0.f);
     } else if (PROJ) {
         const int ch = kt * 64 + (tid & 63);
         lds_sb[tid] = tid < 192 ? p.ds_scale[ch] : (p.ds_bias ? p.ds_bias[ch] : 0.f);
@@ -1367,4 +1468,57 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
     if (cfg == 1) return launch_epi<false, 2, 2>(ctx, p, (int)G);
     if (cfg == 2) return launch_epi<false, 1, 3>(ctx, p, (int)G);
     return launch_epi<false, 1, 2>(ctx, p, (int)G);
+}
+
+// The fp16 layer on the same kernel (E_HALF): half NHWC in, the general kernel's packed weights (64-channel slabs,
+// 64-byte chunks = 32 channels), half NHWC out. Returns EXHIP_ERR_UNSUPPORTED outside what the kernel takes.
+int exhip_conv3x3_f16_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const exhip_lean_f16_epilogue& e, const uint16_t* x, const void* wp,
+                           const float* bias, const uint16_t* residual, uint16_t* y) {
+    if (g_exhip_options.lean == 0 || g_exhip_options.lean_f16 == 0) return EXHIP_ERR_UNSUPPORTED;
+    const long long n_ptiles = (long long)g.n * g.tiles_y * g.tiles_x;
+    const long long out_elems = (long long)g.n * g.oh * g.ow * g.k;
+    if (g.c_bytes % 64 != 0 || g.k % 64 != 0 || g.ph * g.pw > 256 || g.ih * g.iw * kPixB + 16 > kActStride || n_ptiles >= 65536 ||
+        g.h >= 0x4000 || g.w >= 0x4000 || g.ih >= 0x4000 || g.iw >= 0x4000 || g.ph >= 0x4000 || out_elems * 2 >= 0x7FFFF000ll ||
+        (long long)g.h * g.w * g.c_bytes >= 0x7FFFFF00ll || g.act > 1 || g.ktiles != g.k / 64)
+        return EXHIP_ERR_UNSUPPORTED;
+    if (e.post_op && (e.post_op < 1 || e.post_op > 1 + EXHIP_UNARY_CLIP || e.post_op == 1 + EXHIP_UNARY_SIGMOID)) return EXHIP_ERR_UNSUPPORTED;
+    LeanParams p = {};
+    p.x = (const char*)x; p.wp = (const char*)wp; p.bias = bias; p.residual = reinterpret_cast<const float*>(residual);
+    p.y_q = reinterpret_cast<int8_t*>(y);
+    p.H = g.h; p.W = g.w; p.K = g.k; p.OH = g.oh; p.OW = g.ow; p.PT = g.pt; p.PL = g.pl;
+    p.C_b = g.c_bytes; p.n_chunks = g.c_bytes / 64;
+    p.PH = g.ph; p.PW = g.pw; p.IH = g.ih; p.IW = g.iw;
+    p.tiles_x = g.tiles_x; p.tiles_xy = g.tiles_x * g.tiles_y; p.ktiles = g.ktiles; p.n_ptiles = (int)n_ptiles;
+    p.img_bytes = (unsigned)((size_t)g.h * g.w * g.c_bytes);
+    p.out_elems = (unsigned)out_elems;
+    auto magic = [](int d) { return (unsigned)(((1ull << 32) + d - 1) / d); };
+    p.magic_iw = magic(g.iw); p.magic_pw = magic(g.pw); p.magic_tx = magic(g.tiles_x); p.magic_txy = magic(p.tiles_xy);
+    p.adv_iy = 51 / g.iw; p.adv_ix = 51 % g.iw;
+    p.dbg = g_lean_dbg;
+    p.post_op = e.post_op; p.post_alpha = e.post_alpha; p.post_beta = e.post_beta; p.residual_last = residual && e.residual_last;
+    p.flags = E_HALF | (residual ? E_RES : 0) | (g.act == 1 ? E_ACT : 0) | (g.post_relu ? E_POST : 0);
+    // the forms as for the int8 layers without a shortcut: the resident filter for one chunk, one group per patch up to
+    // four chunks, persistent groups with three slice buffers beyond; lean_f16 = 2 / 3 / 4 pin the second / third / a
+    // persistent two-slice form (tests)
+    const int pin = g_exhip_options.lean_f16;
+    const bool wres = p.n_chunks == 1 && g_exhip_options.lean_wres != 0 && pin == 1;
+    const bool one_shot = pin == 2 || (pin == 1 && !wres && p.n_chunks <= 4);
+    const bool three_slices = pin == 3 || (pin == 1 && !wres && !one_shot);
+    const int per_cu = wres || three_slices ? 2 : 3;
+    const long long total = n_ptiles * g.ktiles;
+    long long G = total;
+    if (!one_shot && total > per_cu * 256ll) {
+        const long long unit = 8ll * g.ktiles;  // the XCD mapping and the slab of a group need whole units
+        G = per_cu * 256ll / unit * unit;
+        if (G <= 0) G = g.ktiles;
+    }
+    if (g_exhip_options.lean_groups > 0 && G > (long long)g_exhip_options.lean_groups * g.ktiles)
+        G = (long long)g_exhip_options.lean_groups * g.ktiles;
+    if (g_exhip_options.debug_plan)
+        fprintf(stderr, "  lean fp16: %s, %lld groups for %lld tiles, flags %d\n",
+                wres ? "resident filter" : one_shot ? "one group per patch" : three_slices ? "persistent, three slices" : "persistent, two slices", G,
+                total, p.flags);
+    if (wres) return launch<true, 1, 2, E_HALF>(ctx, p, (int)G);
+    if (three_slices) return launch<false, 1, 3, E_HALF>(ctx, p, (int)G);
+    return launch<false, 1, 2, E_HALF>(ctx, p, (int)G);
 }

@@ -1654,6 +1654,28 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     EXHIP_REQUIRE((long long)d->n * pl.OH * pl.OW < (1ll << 31), "conv: more than 2^31 output pixels");
     const long long tiles = (long long)d->n * pl.tiles_y * pl.tiles_x * pl.ktiles;
     EXHIP_REQUIRE(tiles > 0 && tiles < (1ll << 31), "conv: grid too large");
+    if constexpr (DT == EXHIP_F16) {
+        // 3x3 stride-1 layers with only the NHWC result: the lean kernel takes them with the same packed weights, also where
+        // this kernel would split the reduction of a small launch (measured faster down to 25 tiles; below 16 tiles the
+        // split keeps more CUs busy). EXHIP_ERR_UNSUPPORTED leaves the layer to this kernel.
+        const int min_chunks_ = (3 + pl.n_rg - 1) / pl.n_rg;
+        const bool would_split = g_exhip_options.force_splits != 1 && pl.n_chunks / min_chunks_ >= 2 && kCUs / tiles >= 2;
+        if ((tiles >= 16 || !would_split) && g_exhip_options.force_splits <= 1) {
+            if (!pl.packed && !pool && d->kh == 3 && d->kw == 3 && d->sh == 1 && d->sw == 1 && pl.variant == 0 && pl.chunk_b == 64 &&
+                pl.RS == 1 && p.cstride_b % 64 == 0 && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 && p.y_q && !p.y_nchw_h && !p.y_nchw &&
+                d->post_op != EXHIP_POST_PRELU) {
+                exhip_lean_geom g = {};
+                g.n = d->n; g.h = d->h; g.w = d->w; g.c_bytes = p.cstride_b; g.k = d->k; g.oh = pl.OH; g.ow = pl.OW;
+                g.pt = d->pt; g.pl = d->pl; g.ph = pl.PH; g.pw = pl.PW; g.ih = pl.IH; g.iw = pl.IW;
+                g.tiles_x = pl.tiles_x; g.tiles_y = pl.tiles_y; g.ktiles = pl.ktiles;
+                g.act = d->act; g.post_relu = d->post_relu;
+                const exhip_lean_f16_epilogue e = {d->post_op, d->post_alpha, d->post_beta, d->residual_last};
+                rc = exhip_conv3x3_f16_lean(ctx, g, e, reinterpret_cast<const uint16_t*>(p.x), p.wp, p.bias, reinterpret_cast<const uint16_t*>(p.residual),
+                                            reinterpret_cast<uint16_t*>(p.y_q));
+                if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
+            }
+        }
+    }
     // A launch with too few tiles for the chip's 256 CUs (one image, deep layers) walks its whole reduction on a handful
     // of groups, one stage after the other. Such a launch splits each tile's channel chunks over several groups (at least
     // three stages each, which the loop's prologue counts on), up to about two groups per CU; the parts are added in a
