@@ -26,6 +26,8 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0  # MI355X dense int8 MFMA
 PEAK_HBM_GBS = 8000.0
+PEAK_F16_TFLOPS = 2500.0  # dense fp16 MFMA
+PEAK_F32_TFLOPS = 157.3   # fp32 MFMA
 
 
 def cpu_baseline(net, hw, budget_s=10.0):
@@ -126,8 +128,13 @@ def network_table(iters=10):
         p.sync()
         ms = (time.perf_counter() - t0) / iters * 1e3
         p.close()
+        from excalibur_amd import topologies
+        gop = topologies.algorithmic_gop(net.topology(), x.shape[1:]) * x.shape[0]   # of the whole batch
+        peak = {"f32": PEAK_F32_TFLOPS, "f16": PEAK_F16_TFLOPS, "int8": PEAK_INT8_TOPS}[dtype]
         rows.append({"network": label, "dtype": dtype, "layers": len(net.lines), "ms": round(ms, 3),
-                     "images/s": round(x.shape[0] / ms * 1e3, 1)})
+                     "images/s": round(x.shape[0] / ms * 1e3, 1), "algorithmic_gop": round(gop, 1),
+                     "achieved": round(gop / ms, 1), "peak": peak, "unit": "TOP/s" if dtype == "int8" else "TFLOP/s",
+                     "frac": round(gop / ms / peak, 4)})
         print(f"{label:72s} {dtype:5s} {ms:7.2f} ms {x.shape[0] / ms * 1e3:9.0f} images/s", file=sys.stderr, flush=True)
 
     face = MobileFaceNetF32(hw=112, width=64, blocks=((2, 64, 2), (1, 64, 2), (1, 64, 2), (2, 128, 4), (1, 128, 2), (1, 128, 2),
@@ -166,6 +173,51 @@ def network_table(iters=10):
     for dt, int8 in (("f32", False), ("f16", False), ("int8", True)):
         text, _ = topologies.yolov5s_simp(640, int8=int8)
         run("yolov5s_simp topology (3 heads x 255 channels), 16x3x640x640", Seeded(text, 5), x, dt, "f32" if int8 else dt)
+    return rows
+
+
+def layer_table(ctx, iters=30):
+    """Single layers of the small configurations through the C ABI, NHWC operands resident: cfg1 (float32 3x3, one image)
+    and cfg2 (int8 3x3 and 1x1 at 8 x 128 x 80 x 80, int8 NHWC result). HIP events around `iters` back-to-back launches."""
+    from excalibur_amd import hip
+    rng = np.random.default_rng(1)
+    rows = []
+
+    def timed(fn):
+        for _ in range(5):
+            fn()
+        ctx.sync()
+        e0, e1 = hip.Event(), hip.Event()
+        e0.record(ctx)
+        for _ in range(iters):
+            fn()
+        e1.record(ctx)
+        ctx.sync()
+        return e0.elapsed_ms(e1) / iters
+
+    def row(label, dtype, gop, ms):
+        peak = {"f32": PEAK_F32_TFLOPS, "f16": PEAK_F16_TFLOPS, "int8": PEAK_INT8_TOPS}[dtype]
+        rows.append({"layer": label, "dtype": dtype, "us": round(ms * 1e3, 1), "algorithmic_gop": round(gop, 3),
+                     "achieved": round(gop / ms, 1), "peak": peak, "unit": "TOP/s" if dtype == "int8" else "TFLOP/s",
+                     "frac": round(gop / ms / peak, 4)})
+
+    n, c, hw, k = 1, 64, 56, 64   # cfg1
+    d = ctx.conv_desc(n, c, hw, hw, k, 3, 1, 1, 1, c, k)
+    x = ctx.array(rng.uniform(-1, 1, (n, hw, hw, c)).astype(np.float32))
+    wp = ctx.pack_conv_weights(d, hip.F32, rng.normal(0, 0.05, (k, c, 3, 3)).astype(np.float32))
+    b = ctx.array(rng.normal(0, 0.01, k).astype(np.float32))
+    y = ctx.empty((n, k, hw, hw), np.float32)
+    row("cfg1 3x3 1x64x56x56 -> 64", "f32", 2.0 * n * hw * hw * c * k * 9 / 1e9, timed(lambda: ctx.conv2d_f32(d, x, wp, b, None, None, y)))
+    n, c, hw = 8, 128, 80         # cfg2
+    xq = ctx.array(rng.integers(-127, 128, (n, hw, hw, c)).astype(np.int8))
+    for kernel, k in ((3, 128), (3, 256), (1, 128), (1, 256)):
+        d = ctx.conv_desc(n, c, hw, hw, k, kernel, 1, kernel // 2, 1, c, k, 0, 16.0)
+        wp = ctx.pack_conv_weights(d, hip.I8, rng.integers(-127, 128, (k, c, kernel, kernel)).astype(np.int8))
+        scale = ctx.array(rng.uniform(1e-4, 1e-2, k).astype(np.float32))
+        b = ctx.array(rng.normal(0, 1, k).astype(np.float32))
+        yq = ctx.empty((n, hw, hw, k), np.int8)
+        row(f"cfg2 {kernel}x{kernel} 8x128x80x80 -> {k}", "int8", 2.0 * n * hw * hw * c * k * kernel * kernel / 1e9,
+            timed(lambda: ctx.conv2d_i8(d, xq, wp, scale, b, None, yq)))
     return rows
 
 
@@ -282,6 +334,7 @@ def main():
                     help="set the planner option share_gpu: one more group per CU wherever a single activation tile buffer allows "
                          "it (3 %% faster with two forwards in flight, 2 %% slower with one; off by default)")
     ap.add_argument("--no-memory-bound", action="store_true", help="skip the memory-bound kernels' block of the line")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the other configurations' block of the line")
     ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
                     help="set a library option (exhip_set_option) before the network is planned; may be repeated")
     ap.add_argument("--exhip-lib", default=None, metavar="PATH",
@@ -463,6 +516,12 @@ def main():
                                 "launch_bound": [f'{r["kernel"]} ({r["MB"]} MB, {r["us"]} us per launch)' for r in every if r.get("launch_bound")],
                                 "timing": "HIP events around 10 back-to-back launches of each memory-bound kernel of the path, "
                                           "algorithmic bytes over the 8 TB/s peak (python bench.py --bandwidth prints every row)"}
+    if not args.no_other_configs:
+        # the other configurations: single layers of cfg1 / cfg2 and the whole generated topologies of cfg3 / cfg5 through
+        # the per-layer executor (python bench.py --networks prints the latter as a table)
+        line["other_configs"] = {"layers": layer_table(ctx), "networks": network_table(iters=5),
+                                 "note": "networks: wall time per forward of the per-layer executor, algorithmic GOP of the batch "
+                                         "(convolutions and inner products) over it, against the dense MFMA peak of the dtype"}
     if not args.no_cpu_baseline:
         one, many = cpu_baseline(net, hw)
         line["cpu_baseline"] = one

@@ -267,3 +267,68 @@ SHIPPED = {
     "mobile_unicorn.phai": mobile_unicorn,
     "unicorn_light_806204_m1x3x2+120k_universial_noised_usefulpart_int8.phai": unicorn_light_int8,
 }
+
+
+def algorithmic_gop(text, input_chw):
+    """2 x multiply-accumulates of the Convolution / ConvolutionDepthWise / Deconvolution / InnerProduct layers of a
+    topology for one image of shape (c, h, w), in GOP: 2 * OH * OW * K * (C / groups) * kh * kw per convolution
+    (src/Excalibur/operation_convolution.cpp:270-271 for the output size), 2 * K * C * H * W per InnerProduct. Shapes
+    follow the layers' parameters; layers that keep their input's shape need no entry here."""
+    shapes = {}
+    gop = 0.0
+    for line in text.splitlines()[2:]:
+        t = line.split()
+        if not t:
+            continue
+        typ, nb, nt = t[0], int(t[2]), int(t[3])
+        bots, tops = t[4:4 + nb], t[4 + nb:4 + nb + nt]
+        kv = dict(x.split("=", 1) for x in t[4 + nb + nt:] if "=" in x)
+        geti = lambda k, d=0: int(float(kv.get(str(k), d)))
+        if typ == "Input":
+            shapes[tops[0]] = tuple(input_chw)
+            continue
+        if not bots or bots[0] not in shapes:
+            for tp in tops:
+                shapes[tp] = tuple(input_chw)   # a topology that starts at its first layer
+            if typ not in ("Convolution", "ConvolutionDepthWise", "InnerProduct"):
+                continue
+            shapes.setdefault(bots[0] if bots else tops[0], tuple(input_chw))
+        c, h, w = shapes[bots[0]]
+        if typ in ("Convolution", "ConvolutionDepthWise"):
+            k, kw, kh = geti(0), geti(1), geti(11, geti(1))
+            sw, sh = geti(3, 1), geti(13, geti(3, 1))
+            pl = geti(4)
+            pr, pt, pb = geti(15, pl), geti(14, pl), geti(16, pl)
+            groups = max(1, geti(7, 1))
+            oh, ow = (h + pt + pb - kh) // sh + 1, (w + pl + pr - kw) // sw + 1
+            gop += 2.0 * oh * ow * k * (c // groups) * kh * kw / 1e9
+            shapes[tops[0]] = (k, oh, ow)
+        elif typ == "InnerProduct":
+            k = geti(0)
+            gop += 2.0 * k * c * h * w / 1e9
+            shapes[tops[0]] = (k, 1, 1)
+        elif typ == "Pooling":
+            if geti(4):
+                shapes[tops[0]] = (c, 1, 1)
+            else:
+                kw, kh = geti(1), geti(11, geti(1))
+                sw, sh = geti(2, 1), geti(12, geti(2, 1))
+                pl = geti(3)
+                pr, pt, pb = geti(14, pl), geti(13, pl), geti(15, pl)
+                ceil_mode = geti(5, 1) == 0
+                def size(n, k_, s_, a, b):
+                    v = n + a + b - k_
+                    return (-(-v // s_) if ceil_mode else v // s_) + 1
+                shapes[tops[0]] = (c, size(h, kh, sh, pt, pb), size(w, kw, sw, pl, pr))
+        elif typ == "YoloV5Focus":
+            shapes[tops[0]] = (4 * c, h // 2, w // 2)
+        elif typ == "Interp":
+            ws_, hs_ = float(kv.get("1", 1.0)), float(kv.get("2", 1.0))
+            ow, oh = geti(3), geti(4)
+            shapes[tops[0]] = (c, oh if oh > 0 else int(h * hs_), ow if ow > 0 else int(w * ws_))
+        elif typ == "Concat":
+            shapes[tops[0]] = (sum(shapes[b][0] for b in bots), h, w)
+        else:   # Split, activations, BatchNorm, Eltwise, BinaryOp, Reshape, Transpose ...: the input's shape (no MACs behind them)
+            for tp in tops:
+                shapes[tp] = (c, h, w)
+    return gop
