@@ -32,3 +32,16 @@ def test_detector_topologies_scale_with_the_input(size):
     assert len(outs) == 3
     text, outs = topologies.det_db_resnet18(size)
     assert f"0={size} 1={size}" in text and outs == ["output"]
+
+
+def test_algorithmic_gop_counts_the_benchmark_stack_as_the_survey_does():
+    """14.80 GMAC per 640 x 640 image for the ResNet-18-shaped stack (473.75 GMAC per batch of 32), and a depthwise
+    layer counts C / groups input channels per output."""
+    from excalibur_amd.resnet18 import ResNet18Int8
+    gop = topologies.algorithmic_gop(ResNet18Int8(seed=1, calib_hw=32).topology(), (3, 640, 640))
+    assert abs(gop * 32 - 947.5) < 0.5
+    text = "glsv1 t\n2 2\nConvolution c 1 1 x y 0=8 1=3 11=3 3=1 13=1 4=1 14=1 15=1 16=1 5=0 6=72 7=1\n" \
+           "ConvolutionDepthWise d 1 1 y z 0=8 1=3 11=3 3=2 13=2 4=1 14=1 15=1 16=1 5=0 6=72 7=8\n"
+    dense = 2 * 10 * 12 * 8 * 4 * 9 / 1e9
+    depthwise = 2 * 5 * 6 * 8 * 1 * 9 / 1e9
+    assert abs(topologies.algorithmic_gop(text, (4, 10, 12)) - (dense + depthwise)) < 1e-12
