@@ -628,3 +628,91 @@ def test_int8_convolutions_hand_their_readers_int8_tensors():
         assert all(np.count_nonzero(got[True][b]) > got[True][b].size // 4 for b in outputs)
     finally:
         os.unlink(path)
+
+
+def _fp16_joins_net(seed):
+    """The joins of the fp16 executor beyond the activation pairs: Focus / Reshape / Transpose on halves, the sum behind
+    convolution -> activation, Concat -> BatchNorm -> activation chains and their shorter forms, and the cases that
+    must stay separate layers (a second reader in the middle of a chain, a sigmoid)."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(seed)
+    lines, blobs = ["Input data 0 1 data 0=32 1=32 2=3 3=0,0,0 4=1.0", "YoloV5Focus focus 1 1 data f0"], []
+
+    def conv(bottom, top, cin, k, kernel, stride=1):
+        w = r.normal(0, np.sqrt(2.0 / (cin * kernel * kernel)), (k, cin, kernel, kernel)).astype(np.float32)
+        b = r.normal(0, 0.5, (k,)).astype(np.float32)
+        lines.append(mf.conv_line("Convolution", top + "_l", bottom, top, k, kernel, stride, kernel // 2, True, w.size, 1))
+        blobs.append(mf.conv_blob_f32(w, b))
+
+    def batchnorm(bottom, top, c):
+        lines.append(f"BatchNorm {top}_l 1 1 {bottom} {top} 0={c}")
+        blobs.append(mf.floats_blob(r.uniform(0.5, 1.5, c), r.normal(0, 0.3, c), r.uniform(0.3, 2.0, c), r.normal(0, 0.2, c)))
+
+    hs = "0=1.666667e-01 1=5.000000e-01"
+    conv("f0", "c1", 12, 32, 3)
+    lines.append(f"HardSwish hs1 1 1 c1 a1 {hs}")
+    lines.append("Split sp1 1 3 a1 a1a a1b a1c")
+    conv("a1a", "c2", 32, 32, 1)                       # pointwise kernel, activation, then the sum behind the activation
+    lines.append(f"HardSwish hs2 1 1 c2 a2 {hs}")
+    conv("a2", "c3", 32, 32, 3)                        # 3x3: the lean kernel's fp16 form with the sum behind the activation
+    lines.append(f"HardSwish hs3 1 1 c3 a3 {hs}")
+    lines.append("BinaryOp add3 2 1 a1b a3 s3 0=0")
+    conv("s3", "c4", 32, 32, 1)                        # no bias-less form needed: Concat -> BatchNorm -> LeakyRelu
+    conv("a1c", "c5", 32, 32, 1)
+    lines.append("Concat cat6 2 1 c4 c5 k6 0=-1")
+    batchnorm("k6", "b6", 64)
+    lines.append("LeakyRelu lk6 1 1 b6 a6 0=1.000000e-01")
+    lines.append("Split sp6 1 3 a6 a6a a6b a6c")
+    conv("a6a", "c7", 64, 32, 3, 2)
+    lines.append("Interp up7 1 1 c7 u7 0=1 1=2.000000e+00 2=2.000000e+00")
+    lines.append("Concat cat8 2 1 u7 a6b k8 0=-1")      # Concat -> BatchNorm, no activation behind it
+    batchnorm("k8", "b8", 96)
+    conv("b8", "c9", 96, 64, 1)
+    batchnorm("c9", "b9", 64)                          # BatchNorm -> HardSwish without a Concat
+    lines.append(f"HardSwish hs9 1 1 b9 a9 {hs}")
+    lines.append("Concat cat10 2 1 a9 a6c k10 0=-1")    # Concat whose BatchNorm output has a second reader: the chain ends at the BatchNorm
+    batchnorm("k10", "b10", 128)
+    lines.append("Split sp10 1 2 b10 b10a b10b")
+    lines.append("LeakyRelu lk10 1 1 b10a a10 0=1.000000e-01")
+    lines.append("Eltwise sum11 2 1 a10 b10b s11 0=1")
+    batchnorm("s11", "b11", 128)                       # BatchNorm -> Sigmoid: the sigmoid stays a layer
+    lines.append("Sigmoid sg11 1 1 b11 a11")
+    conv("a11", "c12", 128, 21, 1)                     # a detection head: 21 channels, Reshape and Transpose on halves
+    lines.append("Reshape rs12 1 1 c12 r12 0=256 1=7 2=3")
+    lines.append("Transpose tp12 1 1 r12 t12 0=1,0,2")
+    middle = ["f0", "a1", "a2", "s3", "a6", "b8", "a9", "b10", "a10", "s11", "a11"]
+    gone = ["c2", "c3", "a3", "k6", "b6", "k8", "b9", "k10"]
+    return lines, blobs, ["t12"], middle, gone
+
+
+def test_fp16_executor_joins_equal_the_separate_layers():
+    """fusion on against fusion off in pipeline<unsigned short>, bit for bit, on a network with every join of the fp16
+    executor; the blobs inside a join are not stored and come from a per-layer rerun when asked for."""
+    from excalibur_amd import modelfile as mf
+    lines, blobs, outputs, middle, gone = _fp16_joins_net(31)
+    x = np.random.default_rng(32).normal(0, 1.0, (2, 3, 32, 32)).astype(np.float16).view(np.uint16)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        mf.write_model(path, blobs)
+        got = {}
+        for fusion in (False, True):
+            p = xp.Pipeline(mf.topology(lines, "joins"), path, 0, "f16", fusion=fusion)
+            p.forward(x)
+            if fusion:
+                for b in gone:
+                    assert not p.stored(b), b
+                for b in middle:
+                    assert p.stored(b), b
+            else:
+                assert all(p.stored(b) for b in middle + gone)
+            got[fusion] = {b: p.get(b) for b in outputs + middle + gone}
+            p.close()
+        for b in got[True]:
+            assert got[False][b].shape == got[True][b].shape, b
+            assert np.array_equal(got[False][b], got[True][b]), b
+        out = got[True]["t12"].view(np.float16).astype(np.float32)
+        assert out.shape == (2, 3, 256, 7)
+        assert np.isfinite(out).all() and np.count_nonzero(out) > out.size // 2
+    finally:
+        os.unlink(path)
