@@ -146,6 +146,32 @@ __global__ __launch_bounds__(kBlock) void quantize_nchw_to_nhwc4_x4_kernel(const
     y[(size_t)n * HW4 + p] = make_int4((int)w[0], (int)w[1], (int)w[2], (int)w[3]);
 }
 
+// Half NCHW planes of an image with at most four channels -> NHWC pixels of four halves (the packed first-layer form of
+// the fp16 convolution; absent channels are zero). Eight pixels per thread: one 16-byte load per plane, four 16-byte
+// stores (HW a multiple of 8, 16-byte aligned tensors).
+__global__ __launch_bounds__(kBlock) void nchw_f16_to_nhwc4_x8_kernel(const uint16_t* __restrict__ x, v4i* __restrict__ y, int C, int HW8) {
+    const int n = blockIdx.y;
+    const int p = blockIdx.x * kBlock + threadIdx.x;
+    if (p >= HW8) return;
+    v4i plane[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        if (c < C) plane[c] = reinterpret_cast<const v4i*>(x + ((size_t)n * C + c) * HW8 * 8)[p];
+    auto half_of = [](const v4i& v, int i) { return ((unsigned)v[i >> 1] >> ((i & 1) * 16)) & 0xffffu; };
+    v4i* dst = y + ((size_t)n * HW8 + p) * 4;   // eight pixels x 8 bytes = four 16-byte vectors
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        v4i o;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int px = 2 * q + e;
+            o[2 * e] = (int)(half_of(plane[0], px) | (half_of(plane[1], px) << 16));
+            o[2 * e + 1] = (int)(half_of(plane[2], px) | (half_of(plane[3], px) << 16));
+        }
+        dst[q] = o;
+    }
+}
+
 // NHWC -> NCHW (graph outputs; small). MODE 0: f32->f32, 1: f16->f32, 2: f16->f16
 template <int MODE, typename Tin, typename Tout>
 __global__ __launch_bounds__(kBlock) void nhwc_to_nchw_kernel(const Tin* __restrict__ x, Tout* __restrict__ y, int C, int HW,
@@ -1762,6 +1788,14 @@ extern "C" int exhip_nchw_f32_to_nhwc_f16(exhip_ctx* ctx, const float* x, int n,
 }
 extern "C" int exhip_nchw_f16_to_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, int n, int c, int h, int w, int cs, uint16_t* y) {
     REQ_CTX("exhip_nchw_f16_to_nhwc_f16");
+    if (cs == 4 && c >= 1 && c <= 4 && x && y && n > 0 && n <= 65535 && h > 0 && w > 0 && ((size_t)h * w) % 8 == 0 && (uintptr_t)x % 16 == 0 &&
+        (uintptr_t)y % 16 == 0) {
+        const int hw8 = (int)((size_t)h * w / 8);
+        hipLaunchKernelGGL(nchw_f16_to_nhwc4_x8_kernel, dim3(blocks_for((size_t)hw8), n), dim3(kBlock), 0, ctx->stream, x,
+                           reinterpret_cast<v4i*>(y), c, hw8);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
     return launch_to_nhwc<3>(ctx, x, y, n, c, h, w, cs, 0.f, nullptr);
 }
 

@@ -414,6 +414,16 @@ def test_concat_batchnorm_activation_in_one_kernel_equals_the_separate_layers(ct
     assert np.array_equal(got.download(), want.download())
 
 
+@pytest.mark.parametrize("shape", [(2, 3, 8, 16), (3, 1, 4, 6), (1, 4, 16, 16), (2, 2, 5, 7), (2, 3, 3, 8)], ids=str)
+def test_half_planes_to_four_channel_pixels(ctx, shape):
+    """Half NCHW -> NHWC with four-half pixels (the packed first-layer form of the fp16 convolution): planes of a multiple
+    of eight pixels take the eight-pixels-per-thread kernel, the others the general one; absent channels are zero."""
+    x = np.random.default_rng(387).integers(1, 1 << 16, shape).astype(np.uint16)
+    got = ctx.nchw_to_nhwc(ctx.array(x), 4, "f16").download()
+    assert np.array_equal(got[..., :shape[1]], x.transpose(0, 2, 3, 1))
+    assert not got[..., shape[1]:].any()
+
+
 def _half(a):
     """Round-to-nearest-even to half storage, widened again (what a tensor of the fp16 path holds)."""
     return a.astype(np.float16)
