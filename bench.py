@@ -315,6 +315,29 @@ def bandwidth_table(iters=20, quiet=False, ctx=None):
     gfy = ctx.empty((32, 512, 1, 1), np.float32)
     bw("global average pool f32 NCHW, 32x512x20x20", gf.size * 4 + gfy.size * 4,
        lambda: L.exhip_pool2d_nchw_f32(ctx.h, gf.ptr, gfy.ptr, 32, 512, 20, 20, 1, 1, 1, 20, 20, 1, 1, 0, 0, 0, 0, 0))
+    # the detection topology's glue on halves, and the layers that so far had correctness-grade kernels only
+    fx = ctx.array(rng.integers(0, 1 << 15, (16, 3, 640, 640)).astype(np.uint16))
+    fy = ctx.empty((16, 12, 320, 320), np.uint16)
+    bw("Focus f16, 16x3x640x640", fx.size * 4, lambda: L.exhip_focus_f16(ctx.h, fx.ptr, fy.ptr, 16, 3, 640, 640))
+    ix = ctx.array(rng.integers(0, 1 << 15, (64, 3, 224, 224)).astype(np.uint16))
+    iy = ctx.empty((64, 224, 224, 4), np.uint16)
+    bw("layout NCHW f16 (3 channels) -> NHWC f16 pixels of 4, 64x3x224x224", ix.size * 2 + iy.size * 2,
+       lambda: L.exhip_nchw_f16_to_nhwc_f16(ctx.h, ix.ptr, 64, 3, 224, 224, 4, iy.ptr))
+    hptrs, hchs = (ctypes.c_void_p * 2)(xh.ptr, yh.ptr), (ctypes.c_int * 2)(c, c)
+    bigh = ctx.empty((n, h, w, 2 * c), np.uint16)
+    pa, pb = ctx.array(rng.normal(0, 1, 2 * c).astype(np.float32)), ctx.array(rng.uniform(0.5, 2, 2 * c).astype(np.float32))
+    bw("Concat -> BatchNorm -> LeakyReLU f16 NHWC, 2 x 64 channels", cnt * 8,
+       lambda: L.exhip_concat_batchnorm_unary_nhwc_f16(ctx.h, hptrs, hchs, 2, sz(n * h * w), pa.ptr, pb.ptr, 1, cf(0.1), cf(0.0), bigh.ptr))
+    tp, th_, tw_ = 48, 85, 6400            # a detection head: 16 images x 3 anchors, 85 values x 80 x 80 positions
+    tx = ctx.array(rng.normal(0, 1, (tp, th_, tw_)).astype(np.float32))
+    ty = ctx.empty((tp, tw_, th_), np.float32)
+    bw("Transpose rows / columns f32, 48 planes of 85 x 6400", tx.size * 8, lambda: L.exhip_transpose_hw_f32(ctx.h, tx.ptr, ty.ptr, tp, th_, tw_))
+    txh = ctx.array(rng.integers(0, 1 << 15, (tp, th_, tw_)).astype(np.uint16))
+    tyh = ctx.empty((tp, tw_, th_), np.uint16)
+    bw("Transpose rows / columns f16, 48 planes of 85 x 6400", txh.size * 4, lambda: L.exhip_transpose_hw_f16(ctx.h, txh.ptr, tyh.ptr, tp, th_, tw_))
+    sx = ctx.array(rng.normal(0, 1, (16, 21, 320, 320)).astype(np.float32))
+    sy = ctx.empty((16, 21, 320, 320), np.float32)
+    bw("Softmax over 21 channels f32, 16x21x320x320", sx.size * 8, lambda: L.exhip_softmax_channels_f32(ctx.h, sx.ptr, sy.ptr, 16, 21, 320 * 320))
     if own_ctx:
         ctx.close()
     return rows

@@ -1359,8 +1359,14 @@ __global__ __launch_bounds__(kBlock) void concat_affine_unary_nhwc_f16_kernel(Co
     const int ck = a.first[k + 1] - a.first[k];
     v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(a.src[k] + pix * ck + (c - a.first[k]))), v8f);
     if (p0) {
+        // eight consecutive parameters of each array: 16-byte aligned where the arrays are (device allocations)
+        const v4f a0 = *reinterpret_cast<const v4f*>(p0 + c), a1 = *reinterpret_cast<const v4f*>(p0 + c + 4);
+        const v4f b0 = *reinterpret_cast<const v4f*>(p1 + c), b1 = *reinterpret_cast<const v4f*>(p1 + c + 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = channel_value<1>(v[e], p0[c + e], p1[c + e]);
+        for (int e = 0; e < 4; ++e) {
+            v[e] = channel_value<1>(v[e], a0[e], b0[e]);
+            v[e + 4] = channel_value<1>(v[e + 4], a1[e], b1[e]);
+        }
         if constexpr (UOP >= 0) v = __builtin_convertvector(__builtin_convertvector(v, v8h), v8f);
     }
     if constexpr (UOP >= 0) {
@@ -1553,6 +1559,37 @@ __global__ __launch_bounds__(kBlock) void softmax_channels_kernel(const float* _
         sum += e;
     }
     for (int j = 0; j < C; ++j) out[(size_t)j * HW] = out[(size_t)j * HW] / sum;
+}
+
+// The same for at most CMAX channels: a position's values stay in registers between the three walks, so every value
+// is read once and written once (same operations in the same order: same results).
+template <int CMAX>
+__global__ __launch_bounds__(kBlock) void softmax_channels_reg_kernel(const float* __restrict__ x, float* __restrict__ y, int C, int HW,
+                                                                      size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const size_t img = i / HW;
+    const int k = (int)(i - img * HW);
+    const float* in = x + img * C * HW + k;
+    float* out = y + img * C * HW + k;
+    float v[CMAX];
+#pragma unroll
+    for (int j = 0; j < CMAX; ++j) v[j] = j < C ? in[(size_t)j * HW] : 0.f;
+    float m = v[0];
+#pragma unroll
+    for (int j = 1; j < CMAX; ++j)
+        if (j < C) m = m < v[j] ? v[j] : m;
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < CMAX; ++j) {
+        if (j < C) {
+            v[j] = expf(v[j] - m);
+            sum += v[j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CMAX; ++j)
+        if (j < C) out[(size_t)j * HW] = v[j] / sum;
 }
 
 // Rows and columns of every plane change places, through a 32 x 32 LDS tile so that both sides are coalesced.
@@ -2343,6 +2380,8 @@ extern "C" int exhip_concat_batchnorm_unary_nhwc_f16(exhip_ctx* ctx, const uint1
     }
     a.first[n_inputs] = total;
     EXHIP_REQUIRE((reinterpret_cast<uintptr_t>(y) & 15) == 0, "exhip_concat_batchnorm_unary_nhwc_f16: output must be 16-byte aligned");
+    EXHIP_REQUIRE(!bn_a || ((reinterpret_cast<uintptr_t>(bn_a) | reinterpret_cast<uintptr_t>(bn_b)) & 15) == 0,
+                  "exhip_concat_batchnorm_unary_nhwc_f16: BatchNorm parameters must be 16-byte aligned");
     const size_t total8 = pixels * (size_t)(total / 8);
     const dim3 grid(blocks_for(total8)), block(kBlock);
 #define EXHIP_CAU(UOP) hipLaunchKernelGGL((concat_affine_unary_nhwc_f16_kernel<UOP>), grid, block, 0, ctx->stream, a, y, total8, bn_a, bn_b, alpha, beta)
@@ -2624,7 +2663,8 @@ extern "C" int exhip_softmax_channels_f32(exhip_ctx* ctx, const float* x, float*
     REQ_CTX("exhip_softmax_channels_f32");
     EXHIP_REQUIRE(x && y && n > 0 && c > 0 && hw > 0, "exhip_softmax_channels_f32: bad argument");
     const size_t total = (size_t)n * hw;
-    hipLaunchKernelGGL(softmax_channels_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, hw, total);
+    if (c <= 32) hipLaunchKernelGGL(softmax_channels_reg_kernel<32>, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, hw, total);
+    else hipLaunchKernelGGL(softmax_channels_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, hw, total);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
