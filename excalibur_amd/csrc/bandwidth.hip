@@ -1376,6 +1376,53 @@ __global__ __launch_bounds__(kBlock) void concat_affine_unary_nhwc_f16_kernel(Co
     reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
 }
 
+// The float32 NHWC form of the kernel above for the int8 executor: channel blocks of up to eight float32 NHWC tensors
+// (each with its own channel stride) are laid side by side, then BatchNorm and the activation layer as the float32
+// layers compute them (no rounding between them), and the result leaves as a float32 NHWC tensor and / or as the int8
+// tensor the convolutions that read it would make of it (q8(v * fs)). A thread moves four channels of one pixel.
+struct ConcatNhwcF32Args {
+    const float* src[8];
+    int first[9];   // first[n_inputs] = total channels
+    int stride[8];  // channel stride of each input, in elements
+    int n_inputs;
+};
+template <int UOP>
+__global__ __launch_bounds__(kBlock) void concat_affine_unary_nhwc_f32_kernel(ConcatNhwcF32Args a, float* __restrict__ y_f,
+                                                                              int8_t* __restrict__ y_q, int out_stride, float fs,
+                                                                              size_t total4, const float* __restrict__ p0,
+                                                                              const float* __restrict__ p1, float alpha, float beta) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total4) return;
+    const int vecs = out_stride / 4;
+    const int vi = (int)(i % vecs);
+    const size_t pix = i / vecs;
+    const int c = vi * 4;
+    v4f v = {0.f, 0.f, 0.f, 0.f};
+    if (c < a.first[a.n_inputs]) {  // pad channels of the output hold zeros
+        int k = 0;
+#pragma unroll
+        for (int j = 1; j < 8; ++j)
+            if (j < a.n_inputs && c >= a.first[j]) k = j;
+        v = *reinterpret_cast<const v4f*>(a.src[k] + pix * a.stride[k] + (c - a.first[k]));
+        if (p0) {
+            const v4f a0 = *reinterpret_cast<const v4f*>(p0 + c), b0 = *reinterpret_cast<const v4f*>(p1 + c);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = channel_value<1>(v[e], a0[e], b0[e]);
+        }
+        if constexpr (UOP >= 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = unary_value<UOP>(v[e], alpha, beta);
+        }
+    }
+    if (y_f) *reinterpret_cast<v4f*>(y_f + pix * out_stride + c) = v;
+    if (y_q) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(v[e] * fs) & 0xff) << (8 * e);
+        *reinterpret_cast<uint32_t*>(y_q + pix * out_stride + c) = w;
+    }
+}
+
 // Nearest-neighbour resize of an NHWC half blob (channels a multiple of 8), the index rule of the NCHW kernel below.
 __global__ __launch_bounds__(kBlock) void interp_nearest_nhwc_f16_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ y,
                                                                          int H, int W, int C8, int OH, int OW, float hs, float ws,
@@ -2394,6 +2441,49 @@ extern "C" int exhip_concat_batchnorm_unary_nhwc_f16(exhip_ctx* ctx, const uint1
     default: exhip_set_error("exhip_concat_batchnorm_unary_nhwc_f16: activation %d is not one this kernel applies", unary_op); return EXHIP_ERR_ARG;
     }
 #undef EXHIP_CAU
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_concat_batchnorm_unary_nhwc_f32(exhip_ctx* ctx, const float* const* inputs, const int* channels, const int* strides,
+                                                     int n_inputs, size_t pixels, const float* bn_a, const float* bn_b, int unary_op,
+                                                     float alpha, float beta, int out_stride, float* y_f32, int8_t* y_i8, float fs_out) {
+    REQ_CTX("exhip_concat_batchnorm_unary_nhwc_f32");
+    EXHIP_REQUIRE(inputs && channels && strides && (y_f32 || y_i8) && n_inputs >= 1 && n_inputs <= 8 && pixels > 0,
+                  "exhip_concat_batchnorm_unary_nhwc_f32: bad argument");
+    EXHIP_REQUIRE((bn_a == nullptr) == (bn_b == nullptr), "exhip_concat_batchnorm_unary_nhwc_f32: BatchNorm needs both parameter arrays");
+    ConcatNhwcF32Args a = {};
+    a.n_inputs = n_inputs;
+    int total = 0;
+    for (int i = 0; i < n_inputs; ++i) {
+        EXHIP_REQUIRE(inputs[i] && channels[i] > 0 && channels[i] % 4 == 0 && strides[i] >= channels[i] && strides[i] % 4 == 0 &&
+                          (reinterpret_cast<uintptr_t>(inputs[i]) & 15) == 0,
+                      "exhip_concat_batchnorm_unary_nhwc_f32: input %d needs channels and a stride that are multiples of 4 and 16-byte alignment", i);
+        a.src[i] = inputs[i];
+        a.first[i] = total;
+        a.stride[i] = strides[i];
+        total += channels[i];
+    }
+    a.first[n_inputs] = total;
+    EXHIP_REQUIRE(out_stride >= total && out_stride % 4 == 0, "exhip_concat_batchnorm_unary_nhwc_f32: output stride %d for %d channels", out_stride, total);
+    EXHIP_REQUIRE(!y_f32 || (reinterpret_cast<uintptr_t>(y_f32) & 15) == 0, "exhip_concat_batchnorm_unary_nhwc_f32: float output must be 16-byte aligned");
+    EXHIP_REQUIRE(!y_i8 || (reinterpret_cast<uintptr_t>(y_i8) & 3) == 0, "exhip_concat_batchnorm_unary_nhwc_f32: int8 output must be 4-byte aligned");
+    EXHIP_REQUIRE(!bn_a || ((reinterpret_cast<uintptr_t>(bn_a) | reinterpret_cast<uintptr_t>(bn_b)) & 15) == 0,
+                  "exhip_concat_batchnorm_unary_nhwc_f32: BatchNorm parameters must be 16-byte aligned");
+    const size_t total4 = pixels * (size_t)(out_stride / 4);
+    const dim3 grid(blocks_for(total4)), block(kBlock);
+#define EXHIP_CAU32(UOP)                                                                                                              \
+    hipLaunchKernelGGL((concat_affine_unary_nhwc_f32_kernel<UOP>), grid, block, 0, ctx->stream, a, y_f32, y_i8, out_stride, fs_out, total4, \
+                       bn_a, bn_b, alpha, beta)
+    switch (unary_op) {
+    case -1: EXHIP_CAU32(-1); break;
+    case EXHIP_UNARY_HARDSWISH: EXHIP_CAU32(0); break;
+    case EXHIP_UNARY_LEAKYRELU: EXHIP_CAU32(1); break;
+    case EXHIP_UNARY_HARDSIGMOID: EXHIP_CAU32(3); break;
+    case EXHIP_UNARY_CLIP: EXHIP_CAU32(4); break;
+    default: exhip_set_error("exhip_concat_batchnorm_unary_nhwc_f32: activation %d is not one this kernel applies", unary_op); return EXHIP_ERR_ARG;
+    }
+#undef EXHIP_CAU32
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -242,6 +242,19 @@ __device__ __forceinline__ void post_activation(float (&v)[16], int op, float al
     }
 }
 
+// The same on four float32 values (the fused int8 epilogue works on vectors of four channels).
+__device__ __forceinline__ void post_activation4(v4f& v, int op, float alpha, float beta) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        switch (op) {
+        case EXHIP_UNARY_HARDSWISH: v[e] = unary_value<0>(v[e], alpha, beta); break;
+        case EXHIP_UNARY_LEAKYRELU: v[e] = unary_value<1>(v[e], alpha, beta); break;
+        case EXHIP_UNARY_HARDSIGMOID: v[e] = unary_value<3>(v[e], alpha, beta); break;
+        default: v[e] = unary_value<4>(v[e], alpha, beta); break;
+        }
+    }
+}
+
 // KWE x KSC: the k-steps of one filter row (taps x 32-byte channel steps) when known at compile time, which
 // turns every LDS fragment address of a row into an immediate offset; KWE == 0 keeps them as run-time values.
 // LOWREG: held to 128 registers (a few spills) so that two 512-thread groups can share a CU.
@@ -925,13 +938,20 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                     // ReLU as a maximum with 0, no ReLU as a maximum with -inf: one instruction either way
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], act_floor);
-                    if (has_res) {
-                        const v4f rv = *reinterpret_cast<const v4f*>(tf + e4 * 16);
+                    v4f rv = {0.f, 0.f, 0.f, 0.f};
+                    if (has_res) rv = *reinterpret_cast<const v4f*>(tf + e4 * 16);
+                    if (has_res && !p.residual_last) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] += rv[e];
                     }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], post_floor);
+                    // the activation layer behind the convolution, and the sum layer behind that one
+                    if (p.post_op) post_activation4(v, p.post_op - 1, p.post_alpha, p.post_beta);
+                    if (has_res && p.residual_last) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[e] += rv[e];
+                    }
                     if (has_f) *reinterpret_cast<v4f*>(tf + e4 * 16) = v;
                     if (has_nchw) {
                         // the reference's boundary layout, straight from the registers: lanes run along pixels, so
@@ -1598,6 +1618,13 @@ void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3
     }
 }
 
+// The fused int8 epilogue takes: int8 / float32 NHWC tensors (and the NCHW float32 one), whole 64-channel slabs, plain or
+// ReLU activation, the activation layers of the general epilogue other than PReLU, the shortcut on either side of them.
+inline bool fused_epilogue_ok(const exhip_conv_desc* d, const ConvParams& p, long long out_elems) {
+    return !p.acc_nchw && d->post_op != EXHIP_POST_PRELU && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 && out_elems * 4 < 0xFFFFF000ll &&
+           out_elems < (long long)kEpiInvalid;
+}
+
 template <int DT>
 int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolSpec* pool = nullptr, const exhip_lean_proj* proj = nullptr) {
     EXHIP_REQUIRE(ctx, "conv: NULL ctx");
@@ -1607,8 +1634,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
     if constexpr (DT == EXHIP_I8) {
         if (!pool) {
             const long long elems = (long long)d->n * pl.OH * pl.OW * d->k;
-            const bool fused = !p.acc_nchw && !d->post_op && !d->residual_last && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
-                               elems * 4 < 0xFFFFF000ll && elems < (long long)kEpiInvalid;
+            const bool fused = fused_epilogue_ok(d, p, elems);
             const int epi_wave_b = !fused ? 0 : ((p.residual || p.y_nhwc) ? kEpiWaveBytes : 32 * kEpiRowQ + 128);
             rebuffer(pl, d, epi_wave_b, fused && pl.KWe == 3);
         }
@@ -1707,9 +1733,8 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         }
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
-        const bool fused = !p.acc_nchw && !d->post_op && !d->residual_last && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 &&
-                           out_elems * 4 < 0xFFFFF000ll && out_elems < (long long)kEpiInvalid;
-        if (fused && !pl.packed && p.splits == 1 && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
+        const bool fused = fused_epilogue_ok(d, p, out_elems);
+        if (fused && !d->post_op && !d->residual_last && !pl.packed && p.splits == 1 && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
             p.cstride_b % 64 == 0) {
             // the lean kernel takes these layers with the same packed weights; EXHIP_ERR_UNSUPPORTED leaves them to this one
             exhip_lean_geom g = {};
@@ -1725,7 +1750,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         if (fused) {
             p.epi_mode = 1;
             p.epi_f = p.residual || p.y_nhwc;
-            p.q_nonneg = d->fs_out > 0.f && (d->post_relu || (d->act == 1 && !p.residual));
+            p.q_nonneg = d->fs_out > 0.f && !d->post_op && ((d->post_relu && !p.residual_last) || (d->act == 1 && !p.residual));
             if (pl.packed) return launch_variant<DT, true, 1>(ctx, pl, p, (int)grid);
             return launch_variant<DT, false, 1>(ctx, pl, p, (int)grid);
         }

@@ -405,6 +405,23 @@ class Ctx:
                                                 int(shared)))
         return y
 
+    def concat_nhwc_f32(self, inputs, channels, out_stride, bn=None, unary=None, alpha=0.0, beta=0.0, want_f32=True, fs_out=None):
+        """Channel blocks of float32 NHWC blobs (inputs[i] has channels[i] channels at a stride of its last dimension) side by
+        side, BatchNorm bn=(a, b) and the activation `unary` behind them, as float32 NHWC and / or int8 NHWC q8(v * fs_out)
+        (exhip_concat_batchnorm_unary_nhwc_f32). Returns (float32 or None, int8 or None)."""
+        n, h, w, _ = inputs[0].shape
+        ptrs = (ctypes.c_void_p * len(inputs))(*[a.ptr.value for a in inputs])
+        ch = (ctypes.c_int * len(inputs))(*channels)
+        st = (ctypes.c_int * len(inputs))(*[a.shape[3] for a in inputs])
+        y_f = self.empty((n, h, w, out_stride), np.float32) if want_f32 else None
+        y_q = self.empty((n, h, w, out_stride), np.int8) if fs_out is not None else None
+        _check(lib().exhip_concat_batchnorm_unary_nhwc_f32(self.h, ptrs, ch, st, len(inputs), ctypes.c_size_t(n * h * w),
+                                                           _ptr(bn[0] if bn else None), _ptr(bn[1] if bn else None),
+                                                           -1 if unary is None else self.UNARY[unary], ctypes.c_float(float(alpha)),
+                                                           ctypes.c_float(float(beta)), int(out_stride), _ptr(y_f), _ptr(y_q),
+                                                           ctypes.c_float(float(fs_out or 0.0))))
+        return y_f, y_q
+
     def concat_nhwc_f16(self, inputs, bn=None, unary=None, alpha=0.0, beta=0.0):
         """Concat of NHWC half blobs along the channels; with bn=(a, b) and / or unary= the BatchNorm and activation layers
         behind it in the same kernel (exhip_concat_batchnorm_unary_nhwc_f16), else the plain exhip_concat_channels_nhwc_f16."""

@@ -496,6 +496,8 @@ private:
 
     // ---------------------------------------------------------------- fused int8 executor
     bool try_fused(const tensor_ptr& input, blob_map* results);
+    bool build_block_plan(const tensor_ptr& input, const std::vector<int>& shape);  // residual networks: Convolution / max Pooling / Split / add / ReLU
+    bool build_graph_plan(const tensor_ptr& input, const std::vector<int>& shape);  // + activation layers, Concat, BatchNorm, Interp, Focus
     struct fused_plan;
     std::shared_ptr<fused_plan> plan_;
     bool fused_unsupported_ = false;
@@ -542,12 +544,18 @@ struct pipeline<Dtype>::impl::fused_plan {
     // Results: the launches write through `slot` into `t`, which forward() hands out. A result the caller still holds
     // when the next forward starts is left to the caller: the plan then writes into a new tensor.
     struct result {
-        std::string name;
+        std::string name;         // the network outputs it is, one per line (empty: only a tail layer reads it)
+        std::vector<int> blobs;   // blob ids a tail layer reads it by
         std::shared_ptr<tensor<float>> t;
         std::vector<int> shape;
         float* slot = nullptr;
     };
     std::deque<result> outputs;  // stable addresses: the launches keep pointers to the slots
+    // Layers in front of the first convolution that work on the caller's NCHW tensor (Input, YoloV5Focus) and layers
+    // behind the last one that only rearrange a result (Reshape, Transpose) run as in the per-layer executor, before
+    // and after the launches; input_ptr is then the last front layer's blob.
+    std::vector<int> front_ops, tail_ops;
+    std::shared_ptr<tensor<float>> front_blob;
     const float* input_ptr = nullptr;
     int first_conv_launch = 1;  // 1: launch 0 is the input quantizer; 0: the stem kernel quantizes its own input
     // Launches 1 .. end (everything behind the input quantizer, which alone reads the caller's input pointer) recorded as
@@ -577,14 +585,21 @@ template <>
 bool pipeline<double>::impl::try_fused(const tensor_ptr&, blob_map*) { return false; }
 
 template <>
-bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results) {
-    if (!fusion_ || fused_unsupported_) return false;
-    const std::vector<int> shape = input->data_shape();
-    if (!plan_ || plan_->in_shape != shape) {
-        // ---- classify layers; anything outside the fusable set selects the per-layer executor ----
+bool pipeline<unsigned short>::impl::build_block_plan(const tensor_ptr&, const std::vector<int>&) { return false; }
+template <>
+bool pipeline<double>::impl::build_block_plan(const tensor_ptr&, const std::vector<int>&) { return false; }
+template <>
+bool pipeline<unsigned short>::impl::build_graph_plan(const tensor_ptr&, const std::vector<int>&) { return false; }
+template <>
+bool pipeline<double>::impl::build_graph_plan(const tensor_ptr&, const std::vector<int>&) { return false; }
+
+template <>
+bool pipeline<float>::impl::build_block_plan(const tensor_ptr& input, const std::vector<int>& shape) {
+    {
+        // ---- classify layers; anything outside the fusable set leaves the network to the other planner ----
         using conv_t = operation_convolution<float>;
         const int n_ops = static_cast<int>(operations_.size());
-        auto give_up = [&]() { fused_unsupported_ = true; plan_.reset(); return false; };
+        auto give_up = [&]() { plan_.reset(); return false; };
         if (input->order() != memory::NCHW) return give_up();
         std::vector<int> alias(blob_names_.size());
         for (size_t b = 0; b < alias.size(); ++b) alias[b] = static_cast<int>(b);
@@ -900,7 +915,465 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
         }
         plan_ = plan;
     }
-    plan_->input_ptr = input->gpu_data();
+    return true;
+}
+
+// The planner for int8 networks beyond residual blocks (the detection topologies): every tensor between layers is kept
+// in the form its readers take it in -- int8 NHWC at the readers' feature-map scale, float32 NHWC where a sum, a
+// BatchNorm or a pooling layer reads it, float32 NCHW where it leaves the network -- and the layers between convolutions
+// run on those forms:
+//   * Convolution [-> activation layer] [-> add] [-> ReLU] is one launch (the general epilogue applies them in that
+//     order, the sum in front of or behind the activation as the layers stand);
+//   * Concat [-> BatchNorm] [-> activation] is one launch that also writes the int8 tensor its readers' quantizers would
+//     make of the result; a Concat read by int8 convolutions only concatenates int8 tensors (the quantizer works
+//     value by value, so it commutes with layers that only move or select values: Concat, nearest Interp, max pooling);
+//   * Input and YoloV5Focus in front of the first convolution and Reshape / Transpose behind the last run as layers.
+// Values are those of the per-layer executor. Anything else in the topology returns false (the per-layer executor runs).
+template <>
+bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std::vector<int>& shape) {
+    // EXCALIBUR_PLAN_DEBUG=1 in the environment names the check that left a network to the per-layer executor
+    auto refuse = [&](int check) {
+        if (std::getenv("EXCALIBUR_PLAN_DEBUG")) LOG(INFO) << name_ << ": int8 graph plan not used (check " << check << ")";
+        return false;
+    };
+    using conv_t = operation_convolution<float>;
+    const int n_ops = static_cast<int>(operations_.size());
+    const int n_blobs = static_cast<int>(blob_names_.size());
+    if (input->order() != memory::NCHW || shape.size() != 4 || input_names_.size() != 1) return refuse(1);
+
+    // ---- classify; blobs must be written once (a layer writing over its input is left to the per-layer executor) ----
+    std::vector<int> alias(n_blobs), producer(n_blobs, -1);
+    for (int b = 0; b < n_blobs; ++b) alias[b] = b;
+    std::vector<char> kind(n_ops, 0);  // c conv, u activation, r relu, s split, a add, k concat, b batchnorm, i interp, p max pool, n input, f focus, t tail
+    for (int i = 0; i < n_ops; ++i) {
+        operation<float>* op = operations_[i].get();
+        for (int o : op_outputs_[i]) {
+            if (producer[o] >= 0 || o == blob_index_[input_names_[0]]) return refuse(2);
+            producer[o] = i;
+        }
+        if (dynamic_cast<operation_convolutiondepthwise<float>*>(op)) return refuse(3);
+        if (auto* c = dynamic_cast<conv_t*>(op)) {
+            if (!c->param().int8_quantization_ || c->group_ != 1 || c->stride_h_ != c->stride_w_ || c->dilation_h_ != 1 || c->dilation_w_ != 1 ||
+                c->activation_type_ > 1 || c->weights_i8().empty() || op_inputs_[i].size() != 1 || op_outputs_[i].size() != 1)
+                return refuse(4);
+            kind[i] = 'c';
+        } else if (auto* u = dynamic_cast<operation_unary<float>*>(op)) {
+            if (u->op_ == EXHIP_UNARY_SIGMOID) return refuse(5);
+            kind[i] = 'u';
+        } else if (dynamic_cast<operation_relu<float>*>(op)) {
+            kind[i] = 'r';
+        } else if (dynamic_cast<operation_split<float>*>(op)) {
+            kind[i] = 's';
+            for (int o : op_outputs_[i]) alias[o] = alias[op_inputs_[i][0]];
+        } else if (auto* b = dynamic_cast<operation_binaryop<float>*>(op)) {
+            if (b->op_type_ != 0 || b->with_scalar_ || op_inputs_[i].size() != 2) return refuse(6);
+            kind[i] = 'a';
+        } else if (auto* k = dynamic_cast<operation_concat<float>*>(op)) {
+            if (k->axis_ + 2 != 1 || op_inputs_[i].size() > 8) return refuse(7);
+            kind[i] = 'k';
+        } else if (dynamic_cast<operation_batchnorm<float>*>(op)) {
+            kind[i] = 'b';
+        } else if (auto* ip = dynamic_cast<operation_interp<float>*>(op)) {
+            if (ip->resize_type_ != 1 || ip->align_corner_ != 0) return refuse(8);
+            kind[i] = 'i';
+        } else if (auto* p = dynamic_cast<operation_pooling<float>*>(op)) {
+            if (p->type_ != 0 || p->global_pooling_) return refuse(9);
+            kind[i] = 'p';
+        } else if (dynamic_cast<operation_input<float>*>(op)) {
+            kind[i] = 'n';
+        } else if (dynamic_cast<operation_yolov5focus<float>*>(op)) {
+            kind[i] = 'f';
+        } else if (dynamic_cast<operation_reshape<float>*>(op) || dynamic_cast<operation_transpose<float>*>(op)) {
+            kind[i] = 't';
+        } else {
+            return refuse(10);
+        }
+        if (kind[i] != 's' && kind[i] != 'a' && kind[i] != 'k' && (op_inputs_[i].size() != 1 || op_outputs_[i].size() != 1)) return refuse(11);
+        if (op_outputs_[i].size() != 1 && kind[i] != 's') return refuse(12);
+    }
+    auto root = [&](int b) { return alias[b]; };
+    std::vector<std::vector<int>> consumers(n_blobs);
+    for (int i = 0; i < n_ops; ++i)
+        if (kind[i] != 's')
+            for (int b : op_inputs_[i]) consumers[root(b)].push_back(i);
+    std::vector<char> is_output(n_blobs, 0);
+    for (const std::string& o : output_names_) is_output[root(blob_index_[o])] = 1;
+    const int in_value = root(blob_index_[input_names_[0]]);
+
+    // ---- the layers in front (a chain from the input, each blob read once until the convolutions) and behind ----
+    auto plan = std::make_shared<fused_plan>();
+    plan->in_shape = shape;
+    std::vector<char> where(n_blobs, 0);  // 0 a value of the plan, 1 an NCHW blob of the front chain, 2 a blob of the tail
+    where[in_value] = 1;
+    int front_value = in_value;
+    std::vector<int> front_shape = shape;
+    for (int i = 0; i < n_ops; ++i) {
+        if (kind[i] != 'n' && kind[i] != 'f') continue;
+        if (root(op_inputs_[i][0]) != front_value || consumers[front_value].size() != 1 || is_output[front_value]) return refuse(13);
+        plan->front_ops.push_back(i);
+        front_value = root(op_outputs_[i][0]);
+        where[front_value] = 1;
+        if (kind[i] == 'f') front_shape = {front_shape[0], front_shape[1] * 4, front_shape[2] / 2, front_shape[3] / 2};
+    }
+    if (is_output[front_value] || consumers[front_value].empty()) return refuse(14);
+    for (int c : consumers[front_value])
+        if (kind[c] != 'c') return refuse(15);
+    for (int i = 0; i < n_ops; ++i) {
+        if (kind[i] != 't') continue;
+        plan->tail_ops.push_back(i);
+        where[root(op_outputs_[i][0])] = 2;
+    }
+    for (int i = 0; i < n_ops; ++i)  // nothing but the tail reads the tail
+        if (kind[i] != 't' && kind[i] != 's')
+            for (int b : op_inputs_[i])
+                if (where[root(b)] == 2) return refuse(16);
+
+    // ---- nodes ----
+    struct node {
+        char kind;  // c convolution, g glue (Concat / BatchNorm / activation), i interp, p max pool
+        int op, at;
+        std::vector<int> in;
+        int res = -1, out = -1;
+        int unary = -1, bn = -1;  // layer numbers of the absorbed activation / BatchNorm
+        bool post_relu = false, residual_last = false, as_f32 = true;
+    };
+    std::vector<node> nodes;
+    std::vector<char> absorbed(n_ops, 0);
+    auto sole = [&](int v, char want) -> int {  // the single reader of v if it is an unclaimed layer of kind `want`
+        if (is_output[v] || consumers[v].size() != 1) return -1;
+        const int c = consumers[v][0];
+        return (kind[c] == want && !absorbed[c]) ? c : -1;
+    };
+    for (int i = 0; i < n_ops; ++i) {
+        if (absorbed[i] || kind[i] == 's' || kind[i] == 'n' || kind[i] == 'f' || kind[i] == 't') continue;
+        node nd;
+        nd.kind = kind[i] == 'c' ? 'c' : kind[i] == 'i' ? 'i' : kind[i] == 'p' ? 'p' : 'g';
+        nd.op = nd.at = i;
+        for (int b : op_inputs_[i]) nd.in.push_back(root(b));
+        nd.out = root(op_outputs_[i][0]);
+        auto absorb = [&](int layer) {
+            absorbed[layer] = 1;
+            nd.at = layer;
+            nd.out = root(op_outputs_[layer][0]);
+        };
+        if (kind[i] == 'c') {
+            int act = sole(nd.out, 'u');
+            if (act >= 0) {
+                nd.unary = act;
+                absorb(act);
+            } else if ((act = sole(nd.out, 'r')) >= 0) {
+                nd.post_relu = true;
+                absorb(act);
+            }
+            const int sum = sole(nd.out, 'a');
+            if (sum >= 0) {
+                const int x = root(op_inputs_[sum][0]), y = root(op_inputs_[sum][1]);
+                nd.res = x == nd.out ? y : x;
+                if (nd.res == nd.out) return refuse(17);
+                nd.residual_last = act >= 0;
+                absorb(sum);
+                if (act < 0) {  // the activation behind the sum
+                    int behind = sole(nd.out, 'r');
+                    if (behind >= 0) {
+                        nd.post_relu = true;
+                        absorb(behind);
+                    } else if ((behind = sole(nd.out, 'u')) >= 0) {
+                        nd.unary = behind;
+                        absorb(behind);
+                    }
+                }
+            }
+        } else if (kind[i] == 'k' || kind[i] == 'b' || kind[i] == 'u') {
+            if (kind[i] == 'b') nd.bn = i;
+            if (kind[i] == 'u') nd.unary = i;
+            if (kind[i] == 'k') {
+                const int bn = sole(nd.out, 'b');
+                if (bn >= 0) {
+                    nd.bn = bn;
+                    absorb(bn);
+                }
+            }
+            if (kind[i] != 'u') {
+                const int act = sole(nd.out, 'u');
+                if (act >= 0) {
+                    nd.unary = act;
+                    absorb(act);
+                }
+            }
+        } else if (kind[i] == 'a' || kind[i] == 'r') {
+            return refuse(18);  // a sum or ReLU no convolution's epilogue takes
+        }
+        nodes.push_back(nd);
+    }
+    std::stable_sort(nodes.begin(), nodes.end(), [](const node& a, const node& b) { return a.at < b.at; });
+
+    // ---- what each value must exist as: readers first ----
+    struct value_info {
+        bool need_f32 = false, need_i8 = false, need_nchw = false;
+        float fs = 0.f;
+        int n = 0, c = 0, h = 0, w = 0, cs = 0;
+        void *f32 = nullptr, *i8 = nullptr;
+        float** nchw = nullptr;
+    };
+    std::vector<value_info> vals(n_blobs);
+    for (int b = 0; b < n_blobs; ++b)
+        if (is_output[b] && where[b] == 0) vals[b].need_nchw = true;
+    for (int t : plan->tail_ops)
+        for (int b : op_inputs_[t])
+            if (where[root(b)] == 0) vals[root(b)].need_nchw = true;
+    auto want_i8 = [&](int v, float fs) {
+        if (!(fs > 0.f) || (vals[v].need_i8 && vals[v].fs != fs)) return refuse(19);  // one int8 form per tensor
+        vals[v].need_i8 = true;
+        vals[v].fs = fs;
+        return true;
+    };
+    // channel counts are known from the layers alone; an int8 Concat needs inputs without pad channels
+    vals[front_value].c = front_shape[1];
+    for (const node& nd : nodes) {
+        int c = 0;
+        if (nd.kind == 'c') c = static_cast<conv_t*>(operations_[nd.op].get())->output_channel_;
+        else if (nd.kind == 'g') for (int v : nd.in) c += vals[v].c;
+        else c = vals[nd.in[0]].c;
+        vals[nd.out].c = c;
+    }
+    for (auto it = nodes.rbegin(); it != nodes.rend(); ++it) {
+        node& nd = *it;
+        const value_info out = vals[nd.out];
+        if (where[nd.out] != 0) return refuse(20);
+        if (nd.kind == 'c') {
+            auto* c = static_cast<conv_t*>(operations_[nd.op].get());
+            if (!want_i8(nd.in[0], c->featmap_scale())) return refuse(21);
+            if (nd.res >= 0) {
+                if (where[nd.res] != 0) return refuse(22);
+                vals[nd.res].need_f32 = true;
+            }
+            continue;
+        }
+        if (!out.need_i8 && !out.need_f32 && !out.need_nchw) return refuse(23);  // nobody reads it
+        for (int v : nd.in)
+            if (where[v] != 0) return refuse(24);
+        if (nd.kind == 'g') {
+            nd.as_f32 = nd.bn >= 0 || nd.unary >= 0 || out.need_f32 || out.need_nchw;
+            for (int v : nd.in)
+                if (vals[v].c % 32 != 0) nd.as_f32 = true;
+            for (int v : nd.in) {
+                if (nd.as_f32) vals[v].need_f32 = true;
+                else if (!want_i8(v, out.fs)) return refuse(25);
+            }
+        } else if (nd.kind == 'i') {
+            if (out.need_i8 && !want_i8(nd.in[0], out.fs)) return refuse(26);
+            if (out.need_f32 || out.need_nchw) vals[nd.in[0]].need_f32 = true;
+        } else {
+            vals[nd.in[0]].need_f32 = true;
+        }
+    }
+
+    // ---- shapes, buffers, launches ----
+    exhip_ctx* ctx = memory::device_context(device_);
+    const int dev = device_;
+    auto alloc = [&](size_t bytes) {
+        plan->buffers.emplace_back(dev, bytes);
+        return plan->buffers.back().ptr;
+    };
+    auto blobs_of = [&](int value) {  // the names a tail layer may read the value by
+        std::vector<int> ids;
+        for (int b = 0; b < n_blobs; ++b)
+            if (root(b) == value) ids.push_back(b);
+        return ids;
+    };
+    auto nchw_result = [&](value_info& v, int value) {
+        v.nchw = plan->new_result({v.n, v.c, v.h, v.w}, dev);
+        plan->outputs.back().blobs = blobs_of(value);
+        return v.nchw;
+    };
+    {
+        value_info& v = vals[front_value];
+        if (!v.need_i8 || v.need_f32 || v.need_nchw) return refuse(27);
+        v.n = front_shape[0]; v.c = front_shape[1]; v.h = front_shape[2]; v.w = front_shape[3];
+        int kw_first = 0;
+        for (int c : consumers[front_value]) kw_first = std::max(kw_first, static_cast<conv_t*>(operations_[c].get())->kernel_size_w_);
+        v.cs = (v.c <= 4 && kw_first <= 8) ? 4 : pad_to(v.c, 32);
+        v.i8 = alloc(static_cast<size_t>(v.n) * v.h * v.w * v.cs);
+        int8_t* q = static_cast<int8_t*>(v.i8);
+        const value_info vi = v;
+        fused_plan* pl = plan.get();
+        plan->launches.push_back(
+            [=]() { EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(ctx, pl->input_ptr, vi.n, vi.c, vi.h, vi.w, vi.fs, nullptr, vi.cs, q)); });
+        plan->first_conv_launch = 1;
+    }
+    // a value that leaves as NCHW from a layer other than a convolution: converted from its float32 NHWC form
+    auto nchw_from_f32 = [&](value_info& v, int value) {
+        if (!v.need_nchw) return;
+        float** slot = nchw_result(v, value);
+        const value_info o = v;
+        plan->launches.push_back(
+            [=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, static_cast<const float*>(o.f32), o.n, o.c, o.h, o.w, o.cs, *slot)); });
+    };
+    for (const node& nd : nodes) {
+        const value_info in = vals[nd.in[0]];
+        value_info& out = vals[nd.out];
+        if (in.n == 0) return refuse(28);
+        if (nd.kind == 'c') {
+            auto* c = static_cast<conv_t*>(operations_[nd.op].get());
+            if (in.c != c->input_channels() || !in.i8) return refuse(29);
+            const int ks = pad_to(c->output_channel_, 32);
+            exhip_conv_desc d = c->describe(in.n, in.h, in.w, in.cs, ks);
+            d.post_relu = nd.post_relu ? 1 : 0;
+            d.residual_last = nd.residual_last ? 1 : 0;
+            if (nd.unary >= 0) {
+                auto* u = static_cast<operation_unary<float>*>(operations_[nd.unary].get());
+                d.post_op = 1 + u->op_; d.post_alpha = u->alpha_; d.post_beta = u->beta_;
+            }
+            d.fs_out = out.need_i8 ? out.fs : 0.f;
+            int oh, ow;
+            EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
+            out.n = in.n; out.c = c->output_channel_; out.h = oh; out.w = ow; out.cs = ks;
+            const size_t elems = static_cast<size_t>(out.n) * oh * ow * ks;
+            if (out.need_i8) out.i8 = alloc(elems);
+            if (out.need_f32 || (!out.need_i8 && !out.need_nchw)) out.f32 = alloc(elems * sizeof(float));
+            float** nchw = out.need_nchw ? nchw_result(out, nd.out) : nullptr;
+            const float* res = nullptr;
+            if (nd.res >= 0) {
+                const value_info& r = vals[nd.res];
+                if (!r.f32 || r.n != out.n || r.h != oh || r.w != ow || r.cs != ks || r.c != out.c) return refuse(30);
+                res = static_cast<const float*>(r.f32);
+            }
+            const void* wp = c->pin_packed_weights(EXHIP_I8, d);  // the launch keeps this pointer
+            plan->pinned.emplace_back([c, wp]() { c->unpin_packed_weights(wp); });
+            const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
+            const int8_t* x = static_cast<const int8_t*>(in.i8);
+            int8_t* yq = static_cast<int8_t*>(out.i8);
+            float* yf = static_cast<float*>(out.f32);
+            plan->launches.push_back(
+                [=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, res, yq, yf, nchw ? *nchw : nullptr, nullptr)); });
+        } else if (nd.kind == 'g') {
+            int total = 0;
+            std::vector<const void*> ptrs;
+            std::vector<int> channels, strides;
+            for (int v : nd.in) {
+                const value_info& s = vals[v];
+                if (s.n != in.n || s.h != in.h || s.w != in.w || s.c % 4 != 0) return refuse(31);
+                if (nd.as_f32 ? !s.f32 : (!s.i8 || s.cs != s.c || s.c % 16 != 0)) return refuse(32);
+                ptrs.push_back(nd.as_f32 ? s.f32 : s.i8);
+                channels.push_back(s.c);
+                strides.push_back(s.cs);
+                total += s.c;
+            }
+            out.n = in.n; out.c = total; out.h = in.h; out.w = in.w; out.cs = pad_to(total, 32);
+            const size_t pixels = static_cast<size_t>(out.n) * out.h * out.w;
+            const size_t elems = pixels * out.cs;
+            if (out.need_i8) out.i8 = alloc(elems);
+            const int n_in = static_cast<int>(ptrs.size());
+            if (nd.as_f32) {
+                if (out.need_f32 || out.need_nchw) out.f32 = alloc(elems * sizeof(float));
+                const float *bn_a = nullptr, *bn_b = nullptr;
+                if (nd.bn >= 0) {
+                    auto* bn = static_cast<operation_batchnorm<float>*>(operations_[nd.bn].get());
+                    if (bn->channels_ != total || !bn->a_ || !bn->b_) return refuse(33);
+                    bn_a = bn->a_->gpu_data();
+                    bn_b = bn->b_->gpu_data();
+                }
+                int uop = -1;
+                float alpha = 0.f, beta = 0.f;
+                if (nd.unary >= 0) {
+                    auto* u = static_cast<operation_unary<float>*>(operations_[nd.unary].get());
+                    uop = u->op_; alpha = u->alpha_; beta = u->beta_;
+                }
+                const value_info o = out;
+                plan->launches.push_back([=]() {
+                    EXHIP_FATAL(exhip_concat_batchnorm_unary_nhwc_f32(ctx, reinterpret_cast<const float* const*>(ptrs.data()), channels.data(),
+                                                                      strides.data(), n_in, pixels, bn_a, bn_b, uop, alpha, beta, o.cs,
+                                                                      static_cast<float*>(o.f32), static_cast<int8_t*>(o.i8), o.fs));
+                });
+                nchw_from_f32(out, nd.out);
+            } else {
+                if (out.cs != total) return refuse(34);
+                std::vector<int> pairs;  // the byte tensors as tensors of two-byte elements
+                for (int ch : channels) pairs.push_back(ch / 2);
+                uint16_t* y = static_cast<uint16_t*>(out.i8);
+                plan->launches.push_back([=]() {
+                    EXHIP_FATAL(exhip_concat_channels_nhwc_f16(ctx, reinterpret_cast<const uint16_t* const*>(ptrs.data()), pairs.data(), n_in, pixels, y));
+                });
+            }
+        } else if (nd.kind == 'i') {
+            auto* ip = static_cast<operation_interp<float>*>(operations_[nd.op].get());
+            int oh = ip->output_height_, ow = ip->output_width_;
+            if (oh == 0 || ow == 0) {
+                oh = static_cast<int>(in.h * ip->height_scale_);
+                ow = static_cast<int>(in.w * ip->width_scale_);
+            }
+            if (oh <= 0 || ow <= 0) return refuse(35);
+            out.n = in.n; out.c = in.c; out.h = oh; out.w = ow; out.cs = in.cs;
+            const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
+            if (out.need_i8) {
+                if (!in.i8 || in.cs % 16 != 0) return refuse(36);
+                out.i8 = alloc(elems);
+                const uint16_t* x = static_cast<const uint16_t*>(in.i8);
+                uint16_t* y = static_cast<uint16_t*>(out.i8);
+                plan->launches.push_back([=]() { EXHIP_FATAL(exhip_interp_nearest_nhwc_f16(ctx, x, y, in.n, in.cs / 2, in.h, in.w, oh, ow)); });
+            }
+            if (out.need_f32 || out.need_nchw) {
+                if (!in.f32 || in.cs % 4 != 0) return refuse(37);
+                out.f32 = alloc(elems * sizeof(float));
+                const uint16_t* x = static_cast<const uint16_t*>(in.f32);
+                uint16_t* y = static_cast<uint16_t*>(out.f32);
+                plan->launches.push_back([=]() { EXHIP_FATAL(exhip_interp_nearest_nhwc_f16(ctx, x, y, in.n, in.cs * 2, in.h, in.w, oh, ow)); });
+                nchw_from_f32(out, nd.out);
+            }
+        } else {
+            auto* p = static_cast<operation_pooling<float>*>(operations_[nd.op].get());
+            if (!in.f32) return refuse(38);
+            int kh, kw, sh, sw, pt, pb, pl, pr, oh, ow;
+            p->geometry(in.h, in.w, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &oh, &ow);
+            out.n = in.n; out.c = in.c; out.h = oh; out.w = ow; out.cs = in.cs;
+            const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
+            if (out.need_i8) out.i8 = alloc(elems);
+            if (out.need_f32 || out.need_nchw) out.f32 = alloc(elems * sizeof(float));
+            const float* x = static_cast<const float*>(in.f32);
+            float* yf = static_cast<float*>(out.f32);
+            int8_t* yq = static_cast<int8_t*>(out.i8);
+            const float fs = out.fs;
+            plan->launches.push_back([=]() {
+                EXHIP_FATAL(exhip_maxpool2d_nhwc_f32(ctx, x, yf, yq, fs, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl));
+            });
+            nchw_from_f32(out, nd.out);
+        }
+    }
+    // the network's outputs: results of the plan by name (Split copies share their tensor), the rest comes from the tail
+    for (const std::string& o : output_names_) {
+        const int v = root(blob_index_[o]);
+        if (where[v] == 2) continue;
+        if (where[v] != 0 || !vals[v].nchw) return refuse(39);
+        for (auto& r : plan->outputs)
+            if (&r.slot == vals[v].nchw) r.name += (r.name.empty() ? "" : "\n") + o;
+    }
+    plan_ = plan;
+    return true;
+}
+
+template <>
+bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results) {
+    if (!fusion_ || fused_unsupported_) return false;
+    const std::vector<int> shape = input->data_shape();
+    if (!plan_ || plan_->in_shape != shape) {
+        plan_.reset();
+        if (!build_block_plan(input, shape) && !build_graph_plan(input, shape)) {
+            fused_unsupported_ = true;  // the per-layer executor from now on
+            plan_.reset();
+            return false;
+        }
+    }
+    // layers in front of the first convolution that work on the caller's NCHW tensor
+    {
+        tensor_ptr blob = input;
+        for (int op : plan_->front_ops) {
+            std::vector<tensor_ptr> in{blob}, out(1);
+            operations_[op]->forward_gpu(in, out);
+            blob = out[0];
+        }
+        plan_->front_blob = blob;
+        plan_->input_ptr = blob->gpu_data();
+    }
     last_input_ = input;
     last_input_writes_ = input->writes();
     all_blobs_stored_ = false;
@@ -910,6 +1383,8 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
         if (r.t.use_count() > 1) {  // a result of an earlier forward is still held outside: it stays the caller's
             r.t = std::make_shared<tensor<float>>(r.shape, device_);
             r.slot = r.t->mutable_gpu_data();
+        } else if (r.t->data_shape() != r.shape) {
+            r.t->reshape(r.shape);  // a Reshape layer behind it gave the tensor another shape in the last forward
         }
     }
     exhip_ctx* const ctx = memory::device_context(device_);
@@ -958,11 +1433,23 @@ bool pipeline<float>::impl::try_fused(const tensor_ptr& input, blob_map* results
     last_fused_ = true;
     for (auto& r : plan_->outputs) {
         r.t->mutable_gpu_data();  // the kernels just wrote it: the device copy is the newest
+        for (int b : r.blobs) featmaps_[b] = r.t;
+        if (r.name.empty()) continue;
         for (const std::string& name : split_string(r.name, "\n")) {
             (*results)[name] = r.t;
             featmaps_[blob_index_[name]] = r.t;
         }
     }
+    // layers that only rearrange a result
+    for (int op : plan_->tail_ops) {
+        std::vector<tensor_ptr> in, out(op_outputs_[op].size());
+        for (int b : op_inputs_[op]) in.push_back(featmaps_[b]);
+        operations_[op]->forward_gpu(in, out);
+        for (size_t j = 0; j < out.size(); ++j) featmaps_[op_outputs_[op][j]] = out[j];
+    }
+    if (!plan_->tail_ops.empty())
+        for (const std::string& o : output_names_)
+            if (!results->count(o)) (*results)[o] = featmaps_[blob_index_[o]];
     return true;
 }
 

@@ -110,14 +110,14 @@ typedef struct exhip_conv_desc {
     float fs_out;               /* scale of the optional int8 output: q = sat8(trunc(v*fs_out +- 0.5)) */
     int post_op;                /* 0, or 1 + EXHIP_UNARY_*: the activation layer behind the convolution, applied to the
                                  * value the convolution layer would have stored (rounded to half first in the fp16
-                                 * kernel) by the general epilogue; not available with the fused int8 outputs */
+                                 * kernel); with exhip_conv2d_i8_projection and exhip_conv2d_i8_maxpool3x3s2 it must be 0 */
     float post_alpha, post_beta; /* that layer's parameters (operation_hardswish.cpp:32-63, operation_leakyrelu.cpp:31-58) */
     const float* post_slope;    /* post_op == EXHIP_POST_PRELU: the PReLU layer behind the convolution
                                  * (operation_prelu.cpp:57-124), v >= 0 ? v : slope * v with these device-resident
                                  * slopes, one per output channel, or one for all if post_slope_shared */
     int post_slope_shared;
     int residual_last;          /* 1: the shortcut is added behind post_relu / post_op instead of in front of them (a sum
-                                 * layer behind the activation layer that follows the convolution; general epilogue only) */
+                                 * layer behind the activation layer that follows the convolution) */
 } exhip_conv_desc;
 #define EXHIP_POST_PRELU 16
 
@@ -301,6 +301,15 @@ int exhip_concat_channels_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs
 int exhip_concat_batchnorm_unary_nhwc_f16(exhip_ctx* ctx, const uint16_t* const* inputs, const int* channels, int n_inputs,
                                           size_t pixels, const float* bn_a, const float* bn_b, int unary_op, float alpha,
                                           float beta, uint16_t* y);
+/* The same layers on float32 NHWC blobs (operation_concat.cpp:31-103, operation_batchnorm.cpp:122-156 and the activation
+ * layers' forward_cpu_f32), for an int8 network's executor: input i has channels[i] channels (multiples of 4) at a
+ * channel stride of strides[i] elements; the result has out_stride elements per pixel (pad channels zero) and is
+ * written as float32 (y_f32) and / or as the int8 tensor an int8 convolution's quantizer
+ * (operation_general_conv.cpp:584-720) would make of it, q8(v * fs_out) (y_i8); either may be NULL. Without BatchNorm
+ * and activation and with one input it is that quantizer on an NHWC blob. */
+int exhip_concat_batchnorm_unary_nhwc_f32(exhip_ctx* ctx, const float* const* inputs, const int* channels, const int* strides,
+                                          int n_inputs, size_t pixels, const float* bn_a, const float* bn_b, int unary_op,
+                                          float alpha, float beta, int out_stride, float* y_f32, int8_t* y_i8, float fs_out);
 int exhip_interp_nearest_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int oh, int ow);
 int exhip_maxpool_same_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* tmp, uint16_t* y, int n, int c, int h, int w, int k);
 /* exhip_maxpool_same_nhwc_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight

@@ -21,13 +21,14 @@ def in_stride(c, dtype, kw):
     return hip.pad_to(c * es, 32) // es
 
 
-def conv_i8(ctx, case, fs_out=None, residual=None, post_relu=0, want=("nchw", "acc")):
+def conv_i8(ctx, case, fs_out=None, residual=None, post_relu=0, want=("nchw", "acc"), post_op=None, post_alpha=0.0, post_beta=0.0,
+            residual_last=0):
     n, c, h, w = case["x"].shape
     k = case["k"]
     cs = in_stride(c, hip.I8, case["kw"])
     ks = hip.pad_to(k, 32)
     d = ctx.conv_desc(n, c, h, w, k, (case["kh"], case["kw"]), case["stride"], case["pad"], case["act"], cs, ks,
-                      post_relu, float(fs_out or 0.0))
+                      post_relu, float(fs_out or 0.0), post_op, post_alpha, post_beta, residual_last)
     oh, ow = ctx.conv_out_hw(d)
     xq = ctx.quantize_nchw_to_nhwc_i8(ctx.array(case["x"]), case["fs"], cs)
     wp = ctx.pack_conv_weights(d, hip.I8, case["wt"])

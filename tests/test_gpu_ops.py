@@ -690,3 +690,83 @@ def test_conv_split_reduction_float_within_tolerance(ctx, splits):
     h = gpueval.conv_f16(ctx, case, x16.view(np.uint16))
     assert cases.check_value(h.view(np.float16).astype(np.float32), want, 2e-3) == 0
     assert np.array_equal(h, gpueval.conv_f16(ctx, case, x16.view(np.uint16)))
+
+
+@pytest.mark.parametrize("channels,strides,out_stride,with_bn,unary,alpha,beta", [
+    ((32, 32), (32, 32), 64, True, "leakyrelu", 0.1, 0.0),        # the detection block: Concat -> BatchNorm -> LeakyRelu
+    ((64, 32, 32), (64, 64, 32), 128, True, None, 0.0, 0.0),      # an input whose stride holds pad channels
+    ((24, 8), (32, 8), 32, False, "hardswish", 1 / 6, 0.5),
+    ((20,), (32,), 32, False, None, 0.0, 0.0),                    # one input: the quantizer on an NHWC blob, pad channels zero
+    ((16,), (16,), 32, True, "clip", -0.5, 1.5),
+], ids=["cat-bn-leaky", "cat-bn", "cat-hardswish", "quantizer", "bn-clip"])
+def test_concat_batchnorm_activation_float32_nhwc_with_int8_copy(ctx, channels, strides, out_stride, with_bn, unary, alpha, beta):
+    """The int8 executor's glue kernel against the float32 layers' own kernels (Concat as a copy, BatchNorm and the
+    activation on NCHW) and the oracle's quantizer: the float32 NHWC result and the int8 copy q8(v * fs), pad channels zero."""
+    r = np.random.default_rng(390)
+    n, h, w = 2, 7, 9
+    arrays = []
+    for c, st in zip(channels, strides):
+        a = r.normal(0, 2, (n, h, w, st)).astype(np.float32)
+        a[..., c:] = np.nan    # pad channels of an input are never read
+        arrays.append(a)
+    total = sum(channels)
+    pa = r.normal(0, 0.5, total).astype(np.float32)
+    pb = r.uniform(0.5, 2, total).astype(np.float32)
+    want = np.ascontiguousarray(np.concatenate([a[..., :c] for a, c in zip(arrays, channels)], axis=3).transpose(0, 3, 1, 2))
+    dev = ctx.array(want)
+    if with_bn:
+        dev = ctx.channelwise_f32("batchnorm", dev, ctx.array(pa), ctx.array(pb))
+    if unary:
+        dev = ctx.unary_f32(unary, dev, alpha, beta)
+    ctx.sync()
+    want = dev.download()
+    fs = np.float32(9.3)
+    for want_f32 in (True, False):
+        y_f, y_q = ctx.concat_nhwc_f32([ctx.array(a) for a in arrays], channels, out_stride, (ctx.array(pa), ctx.array(pb)) if with_bn else None,
+                                       unary, alpha, beta, want_f32=want_f32, fs_out=fs)
+        ctx.sync()
+        if want_f32:
+            got = y_f.download()
+            assert np.array_equal(got[..., :total].view(np.uint32), want.transpose(0, 2, 3, 1).view(np.uint32))
+            assert not got[..., total:].any()
+        q = y_q.download()
+        assert np.array_equal(q[..., :total], port.quantize(want, fs).transpose(0, 2, 3, 1))
+        assert not q[..., total:].any()
+
+
+_POST_LAYERS = {
+    "hardswish": (1 / 6, 0.5, lambda v: port.hardswish(v, 1 / 6, 0.5)),
+    "leakyrelu": (0.1, 0.0, lambda v: port.leakyrelu(v, 0.1)),
+    "hardsigmoid": (0.2, 0.5, lambda v: port.hardsigmoid(v, 0.2, 0.5)),
+    "clip": (-0.75, 1.25, lambda v: port.clip(v, -0.75, 1.25)),
+}
+
+
+@pytest.mark.parametrize("shortcut", ["none", "front", "behind"])
+@pytest.mark.parametrize("post_op", list(_POST_LAYERS))
+@pytest.mark.parametrize("k,kernel", [(64, 3), (128, 1), (48, 3)], ids=["k64-3x3", "k128-1x1", "k48-3x3"])
+def test_conv_int8_activation_layer_and_sum_in_the_epilogue(ctx, k, kernel, post_op, shortcut):
+    """int8 convolution -> activation layer [-> sum], or -> sum -> activation layer, in one launch against the oracle's
+    layers one after the other: float32 NHWC / NCHW results and the requantized int8 copy, bit for bit. 64 / 128 output
+    channels take the epilogue with the per-wave tiles, 48 the general one."""
+    case = cases.conv_i8_case(640 + k, 2, 32, 11, 13, k, kernel, 1, kernel // 2, act=0)
+    y = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], 0, cases.geom_of(case))
+    res = np.random.default_rng(641).uniform(-2, 2, y.shape).astype(np.float32)
+    alpha, beta, layer = _POST_LAYERS[post_op]
+    want = y
+    if shortcut == "front":
+        want = port.binaryop_add(want, res)
+    want = layer(want)
+    if shortcut == "behind":
+        want = port.binaryop_add(want, res)
+    fs_out = np.float32(11.7)
+    ks = (k + 31) // 32 * 32
+    res_nhwc = None
+    if shortcut != "none":
+        res_nhwc = np.zeros(y.shape[:1] + y.shape[2:] + (ks,), np.float32)
+        res_nhwc[..., :k] = res.transpose(0, 2, 3, 1)
+    got = gpueval.conv_i8(ctx, case, fs_out=fs_out, residual=res_nhwc, want=("nhwc", "nchw"), post_op=post_op, post_alpha=alpha,
+                          post_beta=beta, residual_last=1 if shortcut == "behind" else 0)
+    assert np.array_equal(got["nchw"].view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(got["nhwc"][..., :k].view(np.uint32), want.transpose(0, 2, 3, 1).view(np.uint32))
+    assert np.array_equal(got["i8"][..., :k], port.quantize(want, fs_out).transpose(0, 2, 3, 1))

@@ -548,7 +548,8 @@ def test_activation_layer_in_the_convolution_epilogue_equals_two_layers(kind):
 def test_yolov5_shaped_int8_topology_matches_the_reference_fixture(fusion):
     """The detector topology with int8 convolutions through pipeline<float>: each convolution quantizes its float input,
     accumulates in int32 and dequantizes with fmaf, every other layer is float, so the outputs equal the compiled
-    reference's bit for bit, with the HardSwish layers in the convolutions' epilogues (fusion) and as layers."""
+    reference's bit for bit, layer by layer and through the int8 graph plan (fusion: int8 / float32 NHWC tensors between
+    the layers, activation layers and sums in the convolutions' epilogues, Concat -> BatchNorm -> LeakyRelu in one kernel)."""
     from excalibur_amd.yolo import YoloV5ShapedF32
     net = YoloV5ShapedF32(int8=True, outputs=8)
     z = np.load(os.path.join(GOLDEN, "net_yolov5_shaped_int8.npz"))
@@ -559,7 +560,7 @@ def test_yolov5_shaped_int8_topology_matches_the_reference_fixture(fusion):
         net.write_model(path)
         p = xp.Pipeline(net.topology(), path, 0, fusion=fusion)
         p.forward(x)
-        assert not p.fused
+        assert p.fused == fusion   # with fusion the int8 graph plan takes the network
         for i, name in enumerate(net.outputs):
             got = p.get(name)
             assert got.shape == z[f"expected{i}"].shape
@@ -714,5 +715,109 @@ def test_fp16_executor_joins_equal_the_separate_layers():
         out = got[True]["t12"].view(np.float16).astype(np.float32)
         assert out.shape == (2, 3, 256, 7)
         assert np.isfinite(out).all() and np.count_nonzero(out) > out.size // 2
+    finally:
+        os.unlink(path)
+
+
+def _int8_graph_net(seed, head_channels=21):
+    """An int8 detection-shaped network with every join of the int8 graph plan: Input + Focus in front; convolution ->
+    HardSwish; the sum behind convolution -> HardSwish (a bottleneck) and convolution -> add -> ReLU; Concat -> BatchNorm
+    -> LeakyRelu read by a convolution; a 5 / 9 pooling pyramid whose Concat is read by a convolution only (int8
+    Concat); Interp -> Concat; a Concat that leaves the network; heads of 21 channels with Reshape and Transpose."""
+    from excalibur_amd import modelfile as mf
+    r = np.random.default_rng(seed)
+    lines, blobs = ["Input data 0 1 data 0=64 1=64 2=3 3=10.0,20.0,30.0 4=0.0039215", "YoloV5Focus focus 1 1 data f0"], []
+
+    def conv(bottom, top, cin, k, kernel, stride=1, scale=8.0, bias=True):
+        w = r.normal(0, np.sqrt(2.0 / (cin * kernel * kernel)), (k, cin, kernel, kernel)).astype(np.float32)
+        b = r.normal(0, 0.3, (k,)).astype(np.float32)
+        ws = (np.float32(127.0) / np.abs(w).reshape(k, -1).max(axis=1)).astype(np.float32)
+        wq = np.clip(np.rint(w * ws[:, None, None, None]), -127, 127).astype(np.int8)
+        lines.append(mf.conv_line("Convolution", top + "_l", bottom, top, k, kernel, stride, kernel // 2, bias, w.size, 1, int8=True))
+        blobs.append(mf.conv_blob_i8(wq, b if bias else None, ws, np.float32(scale)))
+
+    def batchnorm(bottom, top, c):
+        lines.append(f"BatchNorm {top}_l 1 1 {bottom} {top} 0={c}")
+        blobs.append(mf.floats_blob(r.uniform(0.5, 1.5, c), r.normal(0, 0.3, c), r.uniform(0.3, 2.0, c), r.normal(0, 0.2, c)))
+
+    hs = "0=1.666667e-01 1=5.000000e-01"
+    conv("f0", "c1", 12, 32, 3, scale=60.0)
+    lines.append(f"HardSwish hs1 1 1 c1 a1 {hs}")
+    conv("a1", "c2", 32, 64, 3, 2, scale=20.0)
+    lines.append(f"HardSwish hs2 1 1 c2 a2 {hs}")
+    lines.append("Split sp2 1 2 a2 a2a a2b")
+    conv("a2a", "c3", 64, 32, 1, scale=12.0)           # the block's first 1x1, read by the bottleneck and by its sum
+    lines.append(f"HardSwish hs3 1 1 c3 a3 {hs}")
+    lines.append("Split sp3 1 2 a3 a3a a3b")
+    conv("a3a", "c4", 32, 32, 1, scale=14.0)
+    lines.append(f"HardSwish hs4 1 1 c4 a4 {hs}")
+    conv("a4", "c5", 32, 32, 3, scale=15.0)
+    lines.append(f"HardSwish hs5 1 1 c5 a5 {hs}")
+    lines.append("BinaryOp add5 2 1 a3b a5 s5 0=0")     # the sum behind the activation
+    lines.append("Split sp5 1 2 s5 s5a s5b")
+    conv("s5a", "c6", 32, 32, 3, scale=9.0)            # a second block in the ResNet order: convolution -> add -> ReLU
+    lines.append("BinaryOp add6 2 1 c6 s5b s6 0=0")
+    lines.append("ReLU relu6 1 1 s6 a6")
+    conv("a6", "c7", 32, 32, 1, scale=11.0, bias=False)   # the two plain convolutions in front of Concat -> BatchNorm -> LeakyRelu
+    conv("a2b", "c8", 64, 32, 1, scale=12.0, bias=False)
+    lines.append("Concat cat9 2 1 c7 c8 k9 0=-1")
+    batchnorm("k9", "b9", 64)
+    lines.append("LeakyRelu lk9 1 1 b9 a9 0=1.000000e-01")
+    conv("a9", "c10", 64, 64, 1, scale=10.0)
+    lines.append(f"HardSwish hs10 1 1 c10 a10 {hs}")
+    lines.append("Split sp10 1 2 a10 a10a a10b")
+    conv("a10a", "c11", 64, 128, 3, 2, scale=10.0)
+    lines.append(f"HardSwish hs11 1 1 c11 a11 {hs}")
+    conv("a11", "c12", 128, 64, 1, scale=13.0)          # the pooling pyramid
+    lines.append(f"HardSwish hs12 1 1 c12 a12 {hs}")
+    lines.append("Split sp12 1 3 a12 a12a a12b a12c")
+    lines.append(mf.pool_line("p5", "a12b", "q5", 0, kernel=5, stride=1, pad=2))
+    lines.append(mf.pool_line("p9", "a12c", "q9", 0, kernel=9, stride=1, pad=4))
+    lines.append("Concat cat13 3 1 a12a q5 q9 k13 0=-1")
+    conv("k13", "c14", 192, 64, 1, scale=16.0)
+    lines.append(f"HardSwish hs14 1 1 c14 a14 {hs}")
+    lines.append("Split sp14 1 2 a14 a14a a14b")
+    lines.append("Interp up15 1 1 a14a u15 0=1 1=2.000000e+00 2=2.000000e+00")
+    lines.append("Concat cat16 2 1 u15 a10b k16 0=-1")  # Interp -> Concat read by two convolutions and kept as an output
+    lines.append("Split sp16 1 3 k16 k16a k16b k16c")
+    conv("k16a", "c17", 128, head_channels, 1, scale=18.0)
+    lines.append(f"Reshape rs17 1 1 c17 r17 0=256 1={head_channels // 3} 2=3")
+    lines.append("Transpose tp17 1 1 r17 t17 0=1,0,2")
+    conv("k16b", "c18", 128, 32, 3, scale=18.0)
+    lines.append(f"HardSwish hs18 1 1 c18 a18 {hs}")
+    conv("a14b", "c19", 64, head_channels, 1, scale=17.0)
+    lines.append(f"Reshape rs19 1 1 c19 r19 0=64 1={head_channels // 3} 2=3")
+    lines.append("Transpose tp19 1 1 r19 t19 0=1,0,2")
+    return lines, blobs, ["t17", "a18", "t19", "k16c"]
+
+
+def test_int8_graph_plan_equals_the_per_layer_executor():
+    """The int8 executor for networks beyond residual blocks (activation layers, sums behind them, Concat / BatchNorm /
+    Interp / pooling pyramids, Focus in front, Reshape / Transpose behind) against the per-layer executor with fusion
+    off: bit for bit on every output, on a second forward, and on an input of another size (the plan is rebuilt)."""
+    from excalibur_amd import modelfile as mf
+    lines, blobs, outputs = _int8_graph_net(61)
+    with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+        path = f.name
+    try:
+        mf.write_model(path, blobs)
+        plain = xp.Pipeline(mf.topology(lines, "graph"), path, 0, fusion=False)
+        fused = xp.Pipeline(mf.topology(lines, "graph"), path, 0, fusion=True)
+        for seed, n in ((62, 2), (63, 3), (62, 2)):
+            x = np.random.default_rng(seed).uniform(0, 255, (n, 3, 64, 64)).astype(np.float32)
+            plain.forward(x)
+            assert not plain.fused
+            fused.forward(x)
+            assert fused.fused
+            for b in outputs:
+                want, got = plain.get(b), fused.get(b)
+                assert want.shape == got.shape, b
+                assert np.array_equal(want.view(np.uint32), got.view(np.uint32)), (b, seed)
+                assert np.isfinite(got).all() and np.count_nonzero(got) > got.size // 4, b
+            # a blob inside the plan comes from a per-layer rerun of the same input
+            assert not fused.stored("a5")
+            assert np.array_equal(fused.get("s5"), plain.get("s5"))
+        plain.close()
+        fused.close()
     finally:
         os.unlink(path)
