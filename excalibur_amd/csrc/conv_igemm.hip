@@ -1731,6 +1731,20 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             if (pl.packed) return launch_shape<DT, 2, 1, 4, true, 2>(ctx, pl, p, (int)grid);
             return launch_shape<DT, 2, 1, 4, false, 2>(ctx, pl, p, (int)grid);
         }
+        if (!pl.packed && !proj && d->kh == 1 && d->kw == 1 && d->sh == 1 && d->sw == 1 && !d->pt && !d->pb && !d->pl && !d->pr && !p.acc_nchw &&
+            !p.y_nchw && (p.y_q || p.y_nhwc)) {
+            // a pointwise layer with NHWC results only: the kernel without staging takes it with the same packed weights;
+            // EXHIP_ERR_UNSUPPORTED leaves it to this one
+            exhip_pw_geom g = {};
+            g.pixels = (long long)d->n * d->h * d->w; g.c_bytes = p.cstride_b; g.k = d->k; g.k_stride = d->k_stride;
+            g.slab_blocks = pl.TM / 32; g.slabs = pl.ktiles;
+            g.act = d->act; g.post_relu = d->post_relu; g.post_op = d->post_op; g.post_slope_shared = d->post_slope_shared;
+            g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope; g.residual_last = d->residual_last;
+            g.fs_out = d->fs_out;
+            rc = exhip_conv1x1_i8_pw(ctx, g, reinterpret_cast<const int8_t*>(p.x), p.wp, p.scale, p.bias, reinterpret_cast<const float*>(p.residual),
+                                     reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc));
+            if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
+        }
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = fused_epilogue_ok(d, p, out_elems);

@@ -1,21 +1,25 @@
-// The 1x1 stride-1 fp16 convolution (a pointwise layer: a matrix product over the flattened pixels) as a kernel without
-// LDS staging and without barriers (conv_pw.hip). conv_igemm.hip plans the layer and hands the launch over when the
+// The 1x1 stride-1 fp16 / int8 convolution (a pointwise layer: a matrix product over the flattened pixels) as a kernel
+// without LDS staging and without barriers (conv_pw.hip). conv_igemm.hip plans the layer and hands the launch over when the
 // geometry fits; the weights are the general kernel's packing.
 #pragma once
 #include "common.h"
 
 struct exhip_pw_geom {
     long long pixels;           // N * H * W: rows of the NHWC input and output
-    int c_bytes;                // bytes per input pixel (channel stride * 2), a multiple of 32
+    int c_bytes;                // bytes per input pixel (channel stride * element size), a multiple of 32
     int k, k_stride;            // output channels and the output's channel stride, in elements
     int slab_blocks, slabs;     // the packing: 32-channel blocks per slab (2 or 4) and slabs
     int act, post_relu, post_op, post_slope_shared;
     int residual_last;          // the shortcut is added behind post_relu / post_op
     float post_alpha, post_beta;
     const float* post_slope;
+    float fs_out;               // int8 layers: the scale of the requantized int8 result
 };
 
 // Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then
 // runs the general kernel), another code on failure. Semantics as exhip_conv2d_f16 with only the NHWC half output.
 int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t* x, const void* wp, const float* bias,
                          const uint16_t* residual, uint16_t* y);
+// The int8 layer: semantics as exhip_conv2d_i8 with the NHWC results only (y_i8 and / or y_f32; k_stride a multiple of 16).
+int exhip_conv1x1_i8_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const int8_t* x, const void* wp, const float* scale, const float* bias,
+                        const float* residual, int8_t* y_i8, float* y_f32);

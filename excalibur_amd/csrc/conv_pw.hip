@@ -12,10 +12,16 @@
 // Arithmetic and roundings are the general kernel's (conv_igemm.hip, general epilogue): float32 accumulation in
 // v_mfma_f32_32x32x16_f16, bias, activation, the optional shortcut added to the value rounded to half, ReLU / the
 // activation layer behind the convolution applied to the rounded half, one final rounding.
+//
+// The int8 layer (DT == EXHIP_I8) is the same kernel on the same byte geometry -- a 32-byte k-step is 32 int8 channels,
+// v_mfma_i32_32x32x32_i8 on the same 16-byte fragments -- with the int8 epilogue of the general kernel: dequantization
+// fmaf((float)acc, scale, bias), activation, float32 shortcut, ReLU / activation layer, float32 NHWC and / or
+// requantized int8 NHWC results.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
 #include <cstdint>
+#include <type_traits>
 
 #include "conv_pw.h"
 
@@ -23,6 +29,8 @@ namespace {
 
 typedef exhip_v4i v4i;
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer: out-of-range loads return 0
@@ -35,6 +43,12 @@ struct PwParams {
     const uint16_t* residual;
     uint16_t* y;
     const float* post_slope;
+    // int8 layers: dequantization scales, float32 shortcut, float32 and int8 results
+    const float* scale;
+    const float* residual_f;
+    float* y_f;
+    int8_t* y_q;
+    float fs_out;
     unsigned pixels, x_bytes, w_bytes;
     unsigned items, ch_groups;   // waves with work; 32 * MT channel groups per pixel tile
     int xs_b;                    // bytes per input pixel
@@ -169,8 +183,117 @@ __device__ __forceinline__ void pw_epilogue(const PwParams& p, const v16f (&acc)
     }
 }
 
+// The int8 layer's epilogue: the general kernel's, value by value.
 template <int MT, int NT>
-__global__ __launch_bounds__(256, 2) void conv1x1_f16_pw_kernel(const PwParams p) {
+__device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&acc)[MT][NT], const unsigned (&pix)[NT], int kb0, int lane) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int ch0 = (kb0 + m) * 32 + (lane >> 5) * 16;
+        if (ch0 >= p.kstride && ch0 >= p.K) continue;
+        float sc[16], bi[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            sc[e] = ch0 + e < p.K ? p.scale[ch0 + e] : 0.f;
+            bi[e] = (p.bias && ch0 + e < p.K) ? p.bias[ch0 + e] : 0.f;
+        }
+        const bool vec_ok = ch0 + 16 <= p.kstride;
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const bool valid = pix[n] < p.pixels;
+            const size_t at = (size_t)pix[n] * p.kstride + ch0;
+            float v[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) v[e] = __builtin_fmaf((float)acc[m][n][e], sc[e], bi[e]);
+            if (p.act >= 4) {
+#pragma unroll 1
+                for (int e = 0; e < 16; ++e) v[e] = slow_activation(v[e], p.act);
+            } else if (p.act) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = fast_activation(v[e], p.act);
+            }
+            float r[16];
+            if (p.residual_f) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) r[e] = 0.f;
+                if (valid && ch0 + 16 <= p.K) {
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const v4f t = *reinterpret_cast<const v4f*>(p.residual_f + at + e4 * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) r[e4 * 4 + e] = t[e];
+                    }
+                } else if (valid) {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        if (ch0 + e < p.K) r[e] = p.residual_f[at + e];
+                }
+            }
+            if (p.residual_f && !p.residual_last) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    if (ch0 + e < p.K) v[e] += r[e];
+            }
+            if (p.post_relu) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = (0.f > v[e]) ? 0.f : v[e];
+            }
+            if (p.post_op == EXHIP_POST_PRELU) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float slope = p.post_slope[p.post_slope_shared || ch0 + e >= p.K ? 0 : ch0 + e];
+                    v[e] = v[e] >= 0.f ? v[e] : slope * v[e];
+                }
+            } else if (p.post_op) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    switch (p.post_op - 1) {
+                    case EXHIP_UNARY_HARDSWISH: v[e] = unary_value<0>(v[e], p.post_alpha, p.post_beta); break;
+                    case EXHIP_UNARY_LEAKYRELU: v[e] = unary_value<1>(v[e], p.post_alpha, p.post_beta); break;
+                    case EXHIP_UNARY_HARDSIGMOID: v[e] = unary_value<3>(v[e], p.post_alpha, p.post_beta); break;
+                    default: v[e] = unary_value<4>(v[e], p.post_alpha, p.post_beta); break;
+                    }
+                }
+            }
+            if (p.residual_f && p.residual_last) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e)
+                    if (ch0 + e < p.K) v[e] += r[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
+            if (p.y_f && valid) {
+                float* y = p.y_f + at;
+                if (vec_ok) {
+#pragma unroll
+                    for (int e4 = 0; e4 < 4; ++e4) {
+                        const v4f o = {v[e4 * 4], v[e4 * 4 + 1], v[e4 * 4 + 2], v[e4 * 4 + 3]};
+                        *reinterpret_cast<v4f*>(y + e4 * 4) = o;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e)
+                        if (ch0 + e < p.kstride) y[e] = v[e];
+                }
+            }
+            if (p.y_q && valid && vec_ok) {
+                v4i o;
+#pragma unroll
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(v[e4 * 4 + e] * p.fs_out) & 0xff) << (8 * e);
+                    o[e4] = (int)w;
+                }
+                *reinterpret_cast<v4i*>(p.y_q + at) = o;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+template <int DT, int MT, int NT>
+__global__ __launch_bounds__(256, 2) void conv1x1_pw_kernel(const PwParams p) {
     constexpr int U = MT + NT > 4 ? 2 : 4;  // k-steps fetched per request round; two rounds are in flight
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // workgroup ids are dealt round-robin to the 8 XCDs: give each XCD one contiguous run of items, so that the channel
@@ -202,13 +325,14 @@ __global__ __launch_bounds__(256, 2) void conv1x1_f16_pw_kernel(const PwParams p
     const int w_base = __builtin_amdgcn_readfirstlane(((kb0 / p.mts) * p.n_ksteps * p.mts + kb0 % p.mts) * 1024);
     const int woff = lane * 16;
 
-    v16f acc[MT][NT];
+    typedef typename std::conditional<DT == EXHIP_I8, v16i, v16f>::type acc_t;
+    acc_t acc[MT][NT];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
         for (int n = 0; n < NT; ++n)
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[m][n][e] = 0.f;
+            for (int e = 0; e < 16; ++e) acc[m][n][e] = 0;
 
     v4i a[2][U][MT], b[2][U][NT];
     const int nks = p.n_ksteps;
@@ -234,9 +358,13 @@ __global__ __launch_bounds__(256, 2) void conv1x1_f16_pw_kernel(const PwParams p
 #pragma unroll
                 for (int m = 0; m < MT; ++m)
 #pragma unroll
-                    for (int n = 0; n < NT; ++n)
-                        acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a[buf][u][m]), __builtin_bit_cast(v8h, b[buf][u][n]),
-                                                                           acc[m][n], 0, 0, 0);
+                    for (int n = 0; n < NT; ++n) {
+                        if constexpr (DT == EXHIP_I8)
+                            acc[m][n] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[buf][u][m], b[buf][u][n], acc[m][n], 0, 0, 0);
+                        else
+                            acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a[buf][u][m]), __builtin_bit_cast(v8h, b[buf][u][n]),
+                                                                               acc[m][n], 0, 0, 0);
+                    }
             }
         }
     };
@@ -250,12 +378,16 @@ __global__ __launch_bounds__(256, 2) void conv1x1_f16_pw_kernel(const PwParams p
         compute(B1{}, ks0 + U);
     }
 
-    float bi[MT][16];
-    load_bias<MT>(p, kb0, lane, bi);
-    pw_epilogue<MT, NT>(p, acc, pix, kb0, lane, bi);
+    if constexpr (DT == EXHIP_I8) {
+        pw_epilogue_i8<MT, NT>(p, acc, pix, kb0, lane);
+    } else {
+        float bi[MT][16];
+        load_bias<MT>(p, kb0, lane, bi);
+        pw_epilogue<MT, NT>(p, acc, pix, kb0, lane, bi);
+    }
 }
 
-template <int MT, int NT>
+template <int DT, int MT, int NT>
 int launch(exhip_ctx* ctx, PwParams& p, int kblocks) {
     const long long tiles = ((long long)p.pixels + 32 * NT - 1) / (32 * NT);
     p.ch_groups = (unsigned)((kblocks + MT - 1) / MT);
@@ -263,22 +395,25 @@ int launch(exhip_ctx* ctx, PwParams& p, int kblocks) {
     if (items >= (1ll << 31)) return EXHIP_ERR_UNSUPPORTED;
     p.items = (unsigned)items;
     const unsigned grid = (unsigned)((items + 3) / 4);
-    hipLaunchKernelGGL((conv1x1_f16_pw_kernel<MT, NT>), dim3(grid), dim3(256), 0, ctx->stream, p);
+    hipLaunchKernelGGL((conv1x1_pw_kernel<DT, MT, NT>), dim3(grid), dim3(256), 0, ctx->stream, p);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
 
 }  // namespace
 
-int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t* x, const void* wp, const float* bias,
-                         const uint16_t* residual, uint16_t* y) {
+namespace {
+
+// Geometry checks and the wave tile, shared by the two data types. `es`: bytes per input element.
+template <int DT>
+int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has_residual) {
     if (g_exhip_options.pw == 0) return EXHIP_ERR_UNSUPPORTED;
     // Measured against the general kernel on the pointwise layers of a detection and a mobile network (16 and 64 images):
     // this form wins where a launch is short, twice as fast on 20 x 20 maps, and for a lone 32-channel block (which the
     // general kernel pads to a 64-channel slab); from about 2 GFLOP on, the general kernel's staged tiles re-read less
     // and win. Option pw = 2 takes every layer the kernel can (tests).
     const int blocks_needed = (std::max(g.k, g.k_stride) + 31) / 32;
-    const double flop = 2.0 * (double)g.pixels * (g.c_bytes / 2) * g.k;
+    const double flop = 2.0 * (double)g.pixels * (g.c_bytes / es) * g.k;
     if (g_exhip_options.pw != 2 && blocks_needed > 1 && (flop > 2.0e9 || g.pixels > 32768)) return EXHIP_ERR_UNSUPPORTED;
     if (g.pixels <= 0 || g.c_bytes <= 0 || g.c_bytes % 32 != 0 || (g.slab_blocks != 2 && g.slab_blocks != 4) || g.k_stride % 8 != 0)
         return EXHIP_ERR_UNSUPPORTED;
@@ -286,23 +421,40 @@ int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t*
     const long long x_bytes = g.pixels * g.c_bytes;
     const long long n_ksteps = g.c_bytes / 32;
     const long long w_bytes = (long long)g.slabs * n_ksteps * g.slab_blocks * 1024;
-    if (x_bytes >= kOutOfRange || w_bytes >= kOutOfRange || g.pixels * 2 * g.k_stride >= (1ll << 40)) return EXHIP_ERR_UNSUPPORTED;
+    if (x_bytes >= kOutOfRange || w_bytes >= kOutOfRange || g.pixels * 4 * g.k_stride >= (1ll << 40)) return EXHIP_ERR_UNSUPPORTED;
     if (g.post_op && g.post_op != EXHIP_POST_PRELU && (g.post_op < 1 || g.post_op > 1 + EXHIP_UNARY_CLIP || g.post_op == 1 + EXHIP_UNARY_SIGMOID))
         return EXHIP_ERR_UNSUPPORTED;
-    PwParams p = {};
-    p.x = reinterpret_cast<const char*>(x); p.wp = reinterpret_cast<const char*>(wp); p.bias = bias; p.residual = residual; p.y = y;
     p.post_slope = g.post_slope;
     p.pixels = (unsigned)g.pixels; p.x_bytes = (unsigned)x_bytes; p.w_bytes = (unsigned)w_bytes;
     p.xs_b = g.c_bytes; p.n_ksteps = (int)n_ksteps; p.mts = g.slab_blocks;
     p.K = g.k; p.kstride = g.k_stride;
-    p.act = g.act; p.post_relu = g.post_relu; p.post_op = g.post_op; p.post_slope_shared = g.post_slope_shared; p.residual_last = g.residual_last && residual;
+    p.act = g.act; p.post_relu = g.post_relu; p.post_op = g.post_op; p.post_slope_shared = g.post_slope_shared;
+    p.residual_last = g.residual_last && has_residual;
     p.post_alpha = g.post_alpha; p.post_beta = g.post_beta;
     // every packed block that holds a channel below max(k, k_stride): pad channels of the output are written as zeros
     const int kblocks = std::min(g.slabs * g.slab_blocks, (std::max(g.k, g.k_stride) + 31) / 32);
     // 64 x 64 per wave unless that leaves SIMDs without a wave: then 64 channels x 32 pixels; a lone 32-channel block
     // takes 128 pixels per wave
-    if (kblocks == 1) return launch<1, 4>(ctx, p, kblocks);
+    if (kblocks == 1) return launch<DT, 1, 4>(ctx, p, kblocks);
     const long long waves64 = ((g.pixels + 63) / 64) * ((kblocks + 1) / 2);
-    if (waves64 < 2048) return launch<2, 1>(ctx, p, kblocks);
-    return launch<2, 2>(ctx, p, kblocks);
+    if (waves64 < 2048) return launch<DT, 2, 1>(ctx, p, kblocks);
+    return launch<DT, 2, 2>(ctx, p, kblocks);
+}
+
+}  // namespace
+
+int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t* x, const void* wp, const float* bias,
+                         const uint16_t* residual, uint16_t* y) {
+    PwParams p = {};
+    p.x = reinterpret_cast<const char*>(x); p.wp = reinterpret_cast<const char*>(wp); p.bias = bias; p.residual = residual; p.y = y;
+    return run_pw<EXHIP_F16>(ctx, g, p, 2, residual != nullptr);
+}
+
+int exhip_conv1x1_i8_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const int8_t* x, const void* wp, const float* scale, const float* bias,
+                        const float* residual, int8_t* y_i8, float* y_f32) {
+    if (!scale || (!y_i8 && !y_f32) || g.k_stride % 16 != 0) return EXHIP_ERR_UNSUPPORTED;
+    PwParams p = {};
+    p.x = reinterpret_cast<const char*>(x); p.wp = reinterpret_cast<const char*>(wp); p.bias = bias; p.scale = scale;
+    p.residual_f = residual; p.y_f = y_f32; p.y_q = y_i8; p.fs_out = g.fs_out;
+    return run_pw<EXHIP_I8>(ctx, g, p, 1, residual != nullptr);
 }

@@ -118,3 +118,63 @@ def test_shortcut_behind_the_activation_equals_the_sum_layer(ctx, options, kerne
     # in front of the activation (the default) the shortcut gives other values
     front = run(ctx, n, c, h, w, k, x, wt, bias, res, c, k, post_op="hardswish", alpha=1 / 6, beta=0.5, kernel=kernel)
     assert not np.array_equal(front, want)
+
+
+I8_SHAPES = [
+    # seed, n, c, h, w, k, shortcut (0 none, 1 in front of the activation, 2 behind it), act, post_relu, post_op
+    (740, 2, 32, 56, 56, 64, 0, 0, 0, None),
+    (741, 1, 128, 40, 40, 255, 0, 0, 0, None),              # ragged channels: the last block's stores are guarded
+    (742, 1, 64, 33, 31, 64, 1, 0, 1, None),                # a ragged last tile; shortcut + ReLU
+    (743, 3, 16, 9, 7, 32, 0, 1, 0, None),                  # one k-step (16 of its 32 bytes are pad), one 32-channel block
+    (744, 1, 48, 20, 20, 96, 2, 0, 0, "hardswish"),         # the sum behind the activation layer
+    (745, 1, 512, 20, 20, 256, 0, 0, 0, "hardswish"),       # 16 k-steps: the request ring turns twice
+    (746, 2, 32, 128, 128, 32, 0, 0, 0, "leakyrelu"),       # 32 768 pixels, a lone 32-channel block
+    (747, 2, 64, 100, 100, 64, 1, 0, 0, "clip"),
+    (748, 1, 40, 12, 12, 24, 0, 3, 0, None),
+    (749, 1, 64, 17, 5, 128, 0, 4, 0, "hardsigmoid"),       # sigmoid: the out-of-line activation
+]
+I8_PARAMS = {"hardswish": (1 / 6, 0.5), "leakyrelu": (0.1, 0.0), "clip": (-0.25, 0.5), "hardsigmoid": (0.2, 0.5), None: (0.0, 0.0)}
+
+
+@pytest.mark.parametrize("outputs", ["both", "int8", "float32"])
+@pytest.mark.parametrize("args", I8_SHAPES, ids=[f"s{a[0]}" for a in I8_SHAPES])
+def test_int8_pointwise_kernel_repeats_the_general_kernel_bit_for_bit(ctx, options, args, outputs):
+    """The int8 form of the kernel (same byte geometry, v_mfma_i32_32x32x32_i8, the general kernel's int8 epilogue) against
+    the general kernel on the same packed weights: float32 NHWC and requantized int8 NHWC results. The general kernel's
+    results are pinned against the oracle in tests/test_gpu_ops.py."""
+    from tests import gpueval
+    seed, n, c, h, w, k, shortcut, act, post_relu, post_op = args
+    case = cases.conv_i8_case(seed, n, c, h, w, k, 1, 1, 0, act=act)
+    ks = hip.pad_to(k, 32)
+    res = np.random.default_rng(seed + 50).uniform(-2, 2, (n, h, w, ks)).astype(np.float32) if shortcut else None
+    alpha, beta = I8_PARAMS[post_op]
+    want_list = ("nhwc",) if outputs != "int8" else ()
+    fs_out = None if outputs == "float32" else np.float32(9.7)
+    kw = dict(fs_out=fs_out, residual=res, post_relu=post_relu, want=want_list, post_op=post_op, post_alpha=alpha, post_beta=beta,
+              residual_last=1 if shortcut == 2 else 0)
+    options("force_splits", 1)
+    options("pw", 0)
+    want = gpueval.conv_i8(ctx, case, **kw)
+    options("pw", 2)
+    got = gpueval.conv_i8(ctx, case, **kw)
+    for name in ("nhwc", "i8"):
+        if name in want:
+            a, b = want[name][..., :k], got[name][..., :k]
+            assert np.array_equal(a.view(np.uint32) if name == "nhwc" else a, b.view(np.uint32) if name == "nhwc" else b), \
+                f"{name}: {np.count_nonzero(a != b)} of {a.size} differ"
+            assert act == 3 or np.count_nonzero(b) > b.size // 8   # activation 3 zeroes what lies above 6
+            if k < ks:
+                assert not got[name][..., k:].any()     # pad channels are written as zeros
+
+
+@pytest.mark.parametrize("args", [(760, 2, 32, 28, 28, 64), (761, 1, 128, 20, 20, 255), (762, 1, 256, 10, 10, 96)], ids=["s760", "s761", "s762"])
+def test_int8_pointwise_kernel_equals_the_oracle(ctx, options, args):
+    seed, n, c, h, w, k = args
+    options("pw", 2)
+    from tests import gpueval
+    case = cases.conv_i8_case(seed, n, c, h, w, k, 1, 1, 0)
+    want = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], case["act"], cases.geom_of(case))
+    fs_out = np.float32(7.3)
+    got = gpueval.conv_i8(ctx, case, fs_out=fs_out, want=("nhwc",))
+    assert np.array_equal(got["nhwc"][..., :k].view(np.uint32), want.transpose(0, 2, 3, 1).view(np.uint32))
+    assert np.array_equal(got["i8"][..., :k], port.quantize(want, fs_out).transpose(0, 2, 3, 1))
