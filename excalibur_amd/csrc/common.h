@@ -97,6 +97,21 @@ __device__ __forceinline__ void pair_exchange4(exhip_v4i& a, exhip_v4i& c, bool 
     }
 }
 
+// v_permlane32_swap: the upper half-wave of `a` changes places with the lower half-wave of `b`.
+__device__ __forceinline__ void half_swap(int& a, int& b) {
+    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)a, (unsigned)b, false, false);
+    a = (int)r[0];
+    b = (int)r[1];
+}
+__device__ __forceinline__ void half_swap4(exhip_v4i& a, exhip_v4i& b) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        int x = a[e], y = b[e];
+        half_swap(x, y);
+        a[e] = x;
+        b[e] = y;
+    }
+}
 
 // float32_to_int8 of the reference (src/Primitives/simd_types.cpp:140-152): add +-0.5, saturate, truncate.
 __device__ __forceinline__ int exhip_q8(float v) {

@@ -107,22 +107,6 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t uniform_view(const char* base,
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() { __asm__ volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-// v_permlane32_swap: the upper half-wave of `a` changes places with the lower half-wave of `b`.
-__device__ __forceinline__ void half_swap(int& a, int& b) {
-    const auto r = __builtin_amdgcn_permlane32_swap((unsigned)a, (unsigned)b, false, false);
-    a = (int)r[0];
-    b = (int)r[1];
-}
-__device__ __forceinline__ void half_swap4(v4i& a, v4i& b) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        int x = a[e], y = b[e];
-        half_swap(x, y);
-        a[e] = x;
-        b[e] = y;
-    }
-}
-
 // WRES: the slab's whole filter is resident (one 64-byte chunk); otherwise weight slices rotate through NWB buffers and
 // activation tiles through NAB. EPI >= 0: the epilogue's switches as compile-time constants; EPI < 0: read from p.flags.
 // PROJ: the shortcut is a 1x1 convolution computed here (p.ds_*): its channel chunks follow the 3x3 layer's in every patch's

@@ -1036,6 +1036,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         int res = -1, out = -1;
         int unary = -1, bn = -1;  // layer numbers of the absorbed activation / BatchNorm
         bool post_relu = false, residual_last = false, as_f32 = true;
+        int cascade = -1, cascade_k = 0;  // max pool: the value of a smaller pool of the same input to pool again, and with which window
     };
     std::vector<node> nodes;
     std::vector<char> absorbed(n_ops, 0);
@@ -1164,7 +1165,30 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             if (out.need_i8 && !want_i8(nd.in[0], out.fs)) return refuse(26);
             if (out.need_f32 || out.need_nchw) vals[nd.in[0]].need_f32 = true;
         } else {
-            vals[nd.in[0]].need_f32 = true;
+            // A pyramid of stride-1 "same" max pools over one tensor (windows 5 / 9 / 13): the maximum over a window of k is
+            // the maximum over a window of k - k' + 1 of the maxima over windows of k' (taps outside the image count in
+            // neither), so each pool reads the next smaller one's result with a 5-wide window instead of 81 or 169 taps.
+            auto same_window = [&](const node& q) {
+                auto* p = static_cast<operation_pooling<float>*>(operations_[q.op].get());
+                const int k = p->kernel_size_w_;
+                const bool same = k == p->kernel_size_h_ && (k & 1) && p->stride_w_ == 1 && p->stride_h_ == 1 && p->pad_left_ == k / 2 &&
+                                  p->pad_right_ == k / 2 && p->pad_top_ == k / 2 && p->pad_bottom_ == k / 2;
+                return same ? k : 0;
+            };
+            const int k = same_window(nd);
+            int best = 0;
+            if (k > 0)
+                for (const node& q : nodes) {
+                    if (q.kind != 'p' || q.op == nd.op || q.at > nd.at || q.in[0] != nd.in[0]) continue;
+                    const int kq = same_window(q);
+                    if (kq > best && kq < k) {
+                        best = kq;
+                        nd.cascade = q.out;
+                        nd.cascade_k = k - kq + 1;
+                    }
+                }
+            if (nd.cascade >= 0) vals[nd.cascade].need_f32 = true;
+            else vals[nd.in[0]].need_f32 = true;
         }
     }
 
@@ -1322,14 +1346,22 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             }
         } else {
             auto* p = static_cast<operation_pooling<float>*>(operations_[nd.op].get());
-            if (!in.f32) return refuse(38);
             int kh, kw, sh, sw, pt, pb, pl, pr, oh, ow;
             p->geometry(in.h, in.w, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &oh, &ow);
+            const void* source = in.f32;
+            if (nd.cascade >= 0) {  // the smaller pool's result, pooled again (same size as the input: stride 1, "same" padding)
+                const value_info& q = vals[nd.cascade];
+                if (q.n != in.n || q.h != in.h || q.w != in.w || q.cs != in.cs || oh != in.h || ow != in.w) return refuse(40);
+                source = q.f32;
+                kh = kw = nd.cascade_k;
+                pt = pl = nd.cascade_k / 2;
+            }
+            if (!source) return refuse(38);
             out.n = in.n; out.c = in.c; out.h = oh; out.w = ow; out.cs = in.cs;
             const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
             if (out.need_i8) out.i8 = alloc(elems);
             if (out.need_f32 || out.need_nchw) out.f32 = alloc(elems * sizeof(float));
-            const float* x = static_cast<const float*>(in.f32);
+            const float* x = static_cast<const float*>(source);
             float* yf = static_cast<float*>(out.f32);
             int8_t* yq = static_cast<int8_t*>(out.i8);
             const float fs = out.fs;
