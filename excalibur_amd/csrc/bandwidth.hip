@@ -1497,6 +1497,57 @@ __global__ __launch_bounds__(kBlock) void focus_kernel(const float* __restrict__
     y[i] = x[((n * C + c) * H + 2 * oy + g % 2) * W + 2 * ox + g / 2];
 }
 
+// The front of an int8 detection network in one pass: the Input layer's (x - mean[c]) * scale[c], YoloV5Focus (above) and
+// the first convolution's quantizer q8(v * fs), from the float32 NCHW image to int8 NHWC pixels of 32 bytes (4 C channels,
+// the rest zero). A thread makes one output pixel from two neighbouring columns of two rows of each plane.
+struct FrontArgs {
+    float mean[4], scale[4];
+};
+template <int C>
+__global__ __launch_bounds__(kBlock) void input_focus_quantize_kernel(const float* __restrict__ x, int8_t* __restrict__ y, int H, int W,
+                                                                      FrontArgs a, float fs, size_t total) {
+    static_assert(4 * C <= 16, "one 16-byte vector of channels");
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int OH = H / 2, OW = W / 2;
+    const int ox = (int)(i % OW);
+    size_t t = i / OW;
+    const int oy = (int)(t % OH);
+    const size_t n = t / OH;
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const float* src = x + ((n * C + c) * H + 2 * oy + r) * W + 2 * ox;
+            const float v0 = src[0], v1 = src[1];
+            // channel g * C + c holds row parity g % 2 and column parity g / 2
+            const int p0 = r * C + c, p1 = (r + 2) * C + c;
+            const int q0 = exhip_q8(((v0 - a.mean[c]) * a.scale[c]) * fs), q1 = exhip_q8(((v1 - a.mean[c]) * a.scale[c]) * fs);
+            w[p0 >> 2] |= (uint32_t)(q0 & 0xff) << (8 * (p0 & 3));
+            w[p1 >> 2] |= (uint32_t)(q1 & 0xff) << (8 * (p1 & 3));
+        }
+    }
+    v4i* dst = reinterpret_cast<v4i*>(y + i * 32);
+    dst[0] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    dst[1] = v4i{0, 0, 0, 0};
+}
+
+// A detection head's Reshape + Transpose on the convolution's float32 NHWC result: y[n][g][pixel][j] = x[n][pixel][g * J + j]
+// (G groups of J channels: the anchors and their values). One value per thread; reads and writes run along j.
+__global__ __launch_bounds__(kBlock) void nhwc_f32_to_grouped_kernel(const float* __restrict__ x, float* __restrict__ y, int HW, int G, int J,
+                                                                     int stride, size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int j = (int)(i % J);
+    size_t t = i / J;
+    const int pix = (int)(t % HW);
+    t /= HW;
+    const int g = (int)(t % G);
+    const size_t n = t / G;
+    y[i] = x[(n * HW + pix) * stride + g * J + j];
+}
+
 // Four neighbouring outputs of a row per thread (output rows a multiple of four long): one 16-byte store
 __global__ __launch_bounds__(kBlock) void interp_nearest_x4_kernel(const float* __restrict__ x, float* __restrict__ y, int H, int W,
                                                                    int OH, int OW4, float hs, float ws, size_t total4) {
@@ -2706,6 +2757,30 @@ extern "C" int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, 
     }
     const size_t total = (size_t)n * 4 * c * (h / 2) * (w / 2);
     hipLaunchKernelGGL(focus_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, c, h, w, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_input_focus_quantize_nchw_f32_to_nhwc_i8(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, const float* means,
+                                                              const float* scales, float fs, int c_stride, int8_t* y) {
+    REQ_CTX("exhip_input_focus_quantize_nchw_f32_to_nhwc_i8");
+    EXHIP_REQUIRE(x && y && means && scales && n > 0 && h > 1 && w > 1, "exhip_input_focus_quantize_nchw_f32_to_nhwc_i8: bad argument");
+    if (c != 3 || c_stride != 32 || (h & 1) || (w & 1) || (reinterpret_cast<uintptr_t>(y) & 15) != 0) return EXHIP_ERR_UNSUPPORTED;
+    FrontArgs a = {};
+    for (int i = 0; i < c; ++i) { a.mean[i] = means[i]; a.scale[i] = scales[i]; }
+    const size_t total = (size_t)n * (h / 2) * (w / 2);
+    hipLaunchKernelGGL(input_focus_quantize_kernel<3>, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, a, fs, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_nhwc_f32_to_grouped_f32(exhip_ctx* ctx, const float* x, int n, int hw, int groups, int per_group, int c_stride, float* y) {
+    REQ_CTX("exhip_nhwc_f32_to_grouped_f32");
+    EXHIP_REQUIRE(x && y && n > 0 && hw > 0 && groups > 0 && per_group > 0 && c_stride >= groups * per_group,
+                  "exhip_nhwc_f32_to_grouped_f32: bad argument");
+    const size_t total = (size_t)n * groups * hw * per_group;
+    hipLaunchKernelGGL(nhwc_f32_to_grouped_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, hw, groups, per_group, c_stride,
+                       total);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -406,11 +406,12 @@ public:
     explicit operation_reshape(const operation_param& param);
     const char* type() const override { return this->params_.type_.c_str(); }
     int n_ = 0, c_ = -233, h_ = -233, w_ = -233, permute_ = 0;
+    // the shape the layer gives a tensor of `old_shape` with `count` elements
+    std::vector<int> new_shape(const std::vector<int>& old_shape, int count) const;
 
 protected:
     void forward_gpu_f32(const tensor_list<float>& bottoms, tensor_list<float>& tops) override;
     void forward_gpu_f16(const tensor_list<unsigned short>& bottoms, tensor_list<unsigned short>& tops) override;
-    std::vector<int> new_shape(const std::vector<int>& old_shape, int count) const;
 };
 
 // src/Excalibur/operation_flatten.cpp:11-113: key 0 = axis (default 1); a copy with shape [n][1][h'][w'].

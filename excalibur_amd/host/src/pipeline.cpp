@@ -12,6 +12,7 @@
 //    (+ shortcut add + ReLU) and writing what its consumers read. Same values as the per-layer executor.
 #include "../include/Excalibur/pipeline.hpp"
 
+#include <array>
 #include <type_traits>
 #include <chrono>
 #include <cmath>
@@ -1018,15 +1019,6 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     if (is_output[front_value] || consumers[front_value].empty()) return refuse(14);
     for (int c : consumers[front_value])
         if (kind[c] != 'c') return refuse(15);
-    for (int i = 0; i < n_ops; ++i) {
-        if (kind[i] != 't') continue;
-        plan->tail_ops.push_back(i);
-        where[root(op_outputs_[i][0])] = 2;
-    }
-    for (int i = 0; i < n_ops; ++i)  // nothing but the tail reads the tail
-        if (kind[i] != 't' && kind[i] != 's')
-            for (int b : op_inputs_[i])
-                if (where[root(b)] == 2) return refuse(16);
 
     // ---- nodes ----
     struct node {
@@ -1037,6 +1029,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         int unary = -1, bn = -1;  // layer numbers of the absorbed activation / BatchNorm
         bool post_relu = false, residual_last = false, as_f32 = true;
         int cascade = -1, cascade_k = 0;  // max pool: the value of a smaller pool of the same input to pool again, and with which window
+        int head_reshape = -1;            // convolution: the Reshape layer of a detection head (Reshape -> Transpose) it absorbs
     };
     std::vector<node> nodes;
     std::vector<char> absorbed(n_ops, 0);
@@ -1066,7 +1059,18 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                 nd.post_relu = true;
                 absorb(act);
             }
-            const int sum = sole(nd.out, 'a');
+            // a detection head: convolution -> Reshape (channels into groups) -> Transpose of the last two axes
+            const int rs = act < 0 ? sole(nd.out, 't') : -1;
+            if (rs >= 0 && dynamic_cast<operation_reshape<float>*>(operations_[rs].get())) {
+                const int tp = sole(root(op_outputs_[rs][0]), 't');
+                auto* transpose = tp >= 0 ? dynamic_cast<operation_transpose<float>*>(operations_[tp].get()) : nullptr;
+                if (transpose && transpose->perms_.size() == 3 && transpose->perms_[0] == 1 && transpose->perms_[1] == 0 && transpose->perms_[2] == 2) {
+                    nd.head_reshape = rs;
+                    absorb(rs);
+                    absorb(tp);
+                }
+            }
+            const int sum = nd.head_reshape < 0 ? sole(nd.out, 'a') : -1;
             if (sum >= 0) {
                 const int x = root(op_inputs_[sum][0]), y = root(op_inputs_[sum][1]);
                 nd.res = x == nd.out ? y : x;
@@ -1107,6 +1111,15 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         nodes.push_back(nd);
     }
     std::stable_sort(nodes.begin(), nodes.end(), [](const node& a, const node& b) { return a.at < b.at; });
+    for (int i = 0; i < n_ops; ++i) {
+        if (kind[i] != 't' || absorbed[i]) continue;
+        plan->tail_ops.push_back(i);
+        where[root(op_outputs_[i][0])] = 2;
+    }
+    for (int i = 0; i < n_ops; ++i)  // nothing but the tail reads the tail
+        if (kind[i] != 't' && kind[i] != 's')
+            for (int b : op_inputs_[i])
+                if (where[root(b)] == 2) return refuse(16);
 
     // ---- what each value must exist as: readers first ----
     struct value_info {
@@ -1221,8 +1234,32 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         int8_t* q = static_cast<int8_t*>(v.i8);
         const value_info vi = v;
         fused_plan* pl = plan.get();
-        plan->launches.push_back(
-            [=]() { EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(ctx, pl->input_ptr, vi.n, vi.c, vi.h, vi.w, vi.fs, nullptr, vi.cs, q)); });
+        // Input -> YoloV5Focus -> quantizer as one kernel where the library has it; else the two layers run as layers
+        bool one_kernel = false;
+        if (plan->front_ops.size() == 2 && kind[plan->front_ops[0]] == 'n' && kind[plan->front_ops[1]] == 'f') {
+            auto* in_op = static_cast<operation_input<float>*>(operations_[plan->front_ops[0]].get());
+            const int ch = shape[1];
+            if ((ch == 1 || ch == 3) && static_cast<int>(in_op->means_.size()) == ch && static_cast<int>(in_op->vars_.size()) >= ch) {
+                std::array<float, 4> means{}, scales{};
+                for (int c = 0; c < ch; ++c) { means[c] = in_op->means_[c]; scales[c] = in_op->vars_[c]; }
+                const int n0 = shape[0], h0 = shape[2], w0 = shape[3];
+                const int rc = exhip_input_focus_quantize_nchw_f32_to_nhwc_i8(ctx, input->gpu_data(), n0, ch, h0, w0, means.data(), scales.data(),
+                                                                              vi.fs, vi.cs, q);  // trial launch
+                if (rc == 0) {
+                    one_kernel = true;
+                    plan->front_ops.clear();
+                    plan->launches.push_back([=]() {
+                        EXHIP_FATAL(exhip_input_focus_quantize_nchw_f32_to_nhwc_i8(ctx, pl->input_ptr, n0, ch, h0, w0, means.data(), scales.data(), vi.fs,
+                                                                                    vi.cs, q));
+                    });
+                } else if (rc != EXHIP_ERR_UNSUPPORTED) {
+                    EXHIP_FATAL(rc);
+                }
+            }
+        }
+        if (!one_kernel)
+            plan->launches.push_back(
+                [=]() { EXHIP_FATAL(exhip_quantize_nchw_f32_to_nhwc_i8(ctx, pl->input_ptr, vi.n, vi.c, vi.h, vi.w, vi.fs, nullptr, vi.cs, q)); });
         plan->first_conv_launch = 1;
     }
     // a value that leaves as NCHW from a layer other than a convolution: converted from its float32 NHWC form
@@ -1253,6 +1290,27 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
             out.n = in.n; out.c = c->output_channel_; out.h = oh; out.w = ow; out.cs = ks;
             const size_t elems = static_cast<size_t>(out.n) * oh * ow * ks;
+            if (nd.head_reshape >= 0) {
+                // [n, K, oh, ow] -> Reshape [n, G, J, oh * ow] -> Transpose [n, G, oh * ow, J]: the convolution writes float32
+                // NHWC and one kernel regroups the channels of every pixel
+                auto* rs = static_cast<operation_reshape<float>*>(operations_[nd.head_reshape].get());
+                const std::vector<int> to = rs->new_shape({in.n, c->output_channel_, oh, ow}, in.n * c->output_channel_ * oh * ow);
+                if (to.size() != 4 || to[0] != in.n || to[1] * to[2] != c->output_channel_ || to[3] != oh * ow) return refuse(41);
+                if (out.need_i8 || out.need_f32 || !out.need_nchw || nd.res >= 0) return refuse(42);
+                const int groups = to[1], per_group = to[2], hw = oh * ow, n0 = in.n;
+                out.n = in.n; out.c = groups; out.h = hw; out.w = per_group; out.cs = 0;
+                float* mid = static_cast<float*>(alloc(elems * sizeof(float)));
+                float** slot = nchw_result(out, nd.out);
+                const void* wp = c->pin_packed_weights(EXHIP_I8, d);
+                plan->pinned.emplace_back([c, wp]() { c->unpin_packed_weights(wp); });
+                const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
+                const int8_t* x = static_cast<const int8_t*>(in.i8);
+                plan->launches.push_back([=]() {
+                    EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, nullptr, nullptr, mid, nullptr, nullptr));
+                    EXHIP_FATAL(exhip_nhwc_f32_to_grouped_f32(ctx, mid, n0, hw, groups, per_group, ks, *slot));
+                });
+                continue;
+            }
             if (out.need_i8) out.i8 = alloc(elems);
             if (out.need_f32 || (!out.need_i8 && !out.need_nchw)) out.f32 = alloc(elems * sizeof(float));
             float** nchw = out.need_nchw ? nchw_result(out, nd.out) : nullptr;

@@ -328,6 +328,16 @@ int exhip_interp_nearest_f32(exhip_ctx* ctx, const float* x, float* y, int n, in
 /* operation_yolov5focus::forward_cpu_f32 (operation_yolov5focus.cpp:17-50), for every image of the batch
  * (the reference fills image 0 only). y: [n][4c][h/2][w/2]. */
 int exhip_focus_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c, int h, int w);
+/* The front of an int8 detection network in one pass: the Input layer (src/Excalibur/operation_input.cpp:10-151, host
+ * arrays means[c] / scales[c]: (x - mean) * scale), YoloV5Focus (operation_yolov5focus.cpp:12-50) and the first
+ * convolution's quantizer (operation_general_conv.cpp:584-720, q8(v * fs)), float32 NCHW -> int8 NHWC. Takes c == 3,
+ * c_stride == 32 and even h, w; EXHIP_ERR_UNSUPPORTED otherwise (the caller then runs the three layers). */
+int exhip_input_focus_quantize_nchw_f32_to_nhwc_i8(exhip_ctx* ctx, const float* x, int n, int c, int h, int w, const float* means,
+                                                   const float* scales, float fs, int c_stride, int8_t* y);
+/* A detection head's Reshape (operation_reshape.cpp:8-131) to groups x per_group x pixels followed by the Transpose of the
+ * last two axes (operation_transpose.cpp), on the convolution's float32 NHWC result:
+ * y[n][g][pixel][j] = x[n][pixel][g * per_group + j]. */
+int exhip_nhwc_f32_to_grouped_f32(exhip_ctx* ctx, const float* x, int n, int hw, int groups, int per_group, int c_stride, float* y);
 /* The same on half storage: the reference's fp16 layer converts, runs the float layer and converts back
  * (include/Excalibur/operation.hpp:204-266), which for a layer that only moves values is the move itself. */
 int exhip_focus_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w);
