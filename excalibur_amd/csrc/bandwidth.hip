@@ -1534,18 +1534,34 @@ __global__ __launch_bounds__(kBlock) void input_focus_quantize_kernel(const floa
 }
 
 // A detection head's Reshape + Transpose on the convolution's float32 NHWC result: y[n][g][pixel][j] = x[n][pixel][g * J + j]
-// (G groups of J channels: the anchors and their values). One value per thread; reads and writes run along j.
-__global__ __launch_bounds__(kBlock) void nhwc_f32_to_grouped_kernel(const float* __restrict__ x, float* __restrict__ y, int HW, int G, int J,
-                                                                     int stride, size_t total) {
-    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= total) return;
-    const int j = (int)(i % J);
-    size_t t = i / J;
-    const int pix = (int)(t % HW);
-    t /= HW;
-    const int g = (int)(t % G);
-    const size_t n = t / G;
-    y[i] = x[(n * HW + pix) * stride + g * J + j];
+// (G groups of J channels: the anchors and their values). blockIdx.y = n * G + g; one value per thread, reads and writes
+// run along j; 32-bit index arithmetic with one division.
+__global__ __launch_bounds__(kBlock) void nhwc_f32_to_grouped_kernel(const float* __restrict__ x, float* __restrict__ y, unsigned HW, unsigned G,
+                                                                     unsigned J, unsigned stride, unsigned per_plane) {
+    const unsigned i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= per_plane) return;
+    const unsigned plane = blockIdx.y, n = plane / G, g = plane - n * G;
+    const unsigned pix = i / J, j = i - pix * J;
+    y[(size_t)plane * per_plane + i] = x[((size_t)n * HW + pix) * stride + g * J + j];
+}
+// The same, four consecutive results per thread (planes a multiple of four values long): one 16-byte store
+__global__ __launch_bounds__(kBlock) void nhwc_f32_to_grouped_x4_kernel(const float* __restrict__ x, float* __restrict__ y, unsigned HW, unsigned G,
+                                                                        unsigned J, unsigned stride, unsigned per_plane4) {
+    const unsigned i4 = blockIdx.x * kBlock + threadIdx.x;
+    if (i4 >= per_plane4) return;
+    const unsigned plane = blockIdx.y, n = plane / G, g = plane - n * G;
+    unsigned pix = (i4 * 4) / J, j = i4 * 4 - pix * J;
+    const float* src = x + ((size_t)n * HW + pix) * stride + g * J;
+    v4f o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        o[e] = src[j];
+        if (++j == J) {  // on to the next pixel
+            j = 0;
+            src += stride;
+        }
+    }
+    reinterpret_cast<v4f*>(y + (size_t)plane * per_plane4 * 4)[i4] = o;
 }
 
 // Four neighbouring outputs of a row per thread (output rows a multiple of four long): one 16-byte store
@@ -2778,9 +2794,14 @@ extern "C" int exhip_nhwc_f32_to_grouped_f32(exhip_ctx* ctx, const float* x, int
     REQ_CTX("exhip_nhwc_f32_to_grouped_f32");
     EXHIP_REQUIRE(x && y && n > 0 && hw > 0 && groups > 0 && per_group > 0 && c_stride >= groups * per_group,
                   "exhip_nhwc_f32_to_grouped_f32: bad argument");
-    const size_t total = (size_t)n * groups * hw * per_group;
-    hipLaunchKernelGGL(nhwc_f32_to_grouped_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, hw, groups, per_group, c_stride,
-                       total);
+    const long long per_plane = (long long)hw * per_group, planes = (long long)n * groups;
+    EXHIP_REQUIRE(per_plane < (1ll << 31) && planes <= 65535, "exhip_nhwc_f32_to_grouped_f32: tensor too large");
+    if (per_plane % 4 == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0)
+        hipLaunchKernelGGL(nhwc_f32_to_grouped_x4_kernel, dim3((unsigned)((per_plane / 4 + kBlock - 1) / kBlock), (unsigned)planes), dim3(kBlock), 0,
+                           ctx->stream, x, y, (unsigned)hw, (unsigned)groups, (unsigned)per_group, (unsigned)c_stride, (unsigned)(per_plane / 4));
+    else
+        hipLaunchKernelGGL(nhwc_f32_to_grouped_kernel, dim3((unsigned)((per_plane + kBlock - 1) / kBlock), (unsigned)planes), dim3(kBlock), 0,
+                           ctx->stream, x, y, (unsigned)hw, (unsigned)groups, (unsigned)per_group, (unsigned)c_stride, (unsigned)per_plane);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -435,9 +435,13 @@ int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has
     // general kernel pads to a 64-channel slab); from about 2 GFLOP on, the general kernel's staged tiles re-read less
     // and win. Option pw = 2 takes every layer the kernel can (tests).
     const int blocks_needed = (std::max(g.k, g.k_stride) + 31) / 32;
-    // The int8 layers of the same networks: this form wins on every layer of at most 32 768 pixels (up to 6.7 GOP measured).
+    // The int8 layers of the same networks: this form wins on every layer of at most 32 768 pixels (up to 6.7 GOP measured)
+    // and, up to 131 072 pixels, on layers of at most 64 input channels and on those with only a float32 result (its
+    // 64-byte store runs against the general epilogue's 16-byte pieces: 41 against 60 us on a 128 -> 255 head at 16 x 80 x 80).
     const double flop = 2.0 * (double)g.pixels * (g.c_bytes / es) * g.k;
-    if (g_exhip_options.pw != 2 && blocks_needed > 1 && (flop > (DT == EXHIP_I8 ? 8.0e9 : 2.0e9) || g.pixels > 32768)) return EXHIP_ERR_UNSUPPORTED;
+    bool take = blocks_needed == 1 || (flop <= (DT == EXHIP_I8 ? 8.0e9 : 2.0e9) && g.pixels <= 32768);
+    if (DT == EXHIP_I8 && g.pixels <= 131072 && (g.c_bytes <= 64 || (p.y_f && !p.y_q))) take = true;
+    if (g_exhip_options.pw != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
     if (g.pixels <= 0 || g.c_bytes <= 0 || g.c_bytes % 32 != 0 || (g.slab_blocks != 2 && g.slab_blocks != 4) || g.k_stride % 8 != 0)
         return EXHIP_ERR_UNSUPPORTED;
     // lane offsets are 32-bit: the input tensor and the packed weights must stay below the out-of-range sentinel
