@@ -102,9 +102,10 @@ def measured_traffic(n, hw):
 
 
 def network_table(iters=10):
-    """The generated topologies of the other configurations through pipeline<float> / pipeline<unsigned short> layer by
-    layer (every output blob allocated per forward, as in the reference), input resident on the device: wall time per
-    forward over `iters` forwards, device drained before and after. Returns [{"network", "dtype", "ms", "images/s"}]."""
+    """The generated topologies of the other configurations through pipeline<float> / pipeline<unsigned short> (float32 and
+    fp16: layer by layer with the executor's joins; int8: the int8 graph plan where it takes the network, which the row's
+    "executor" says), input resident on the device: wall time per forward over `iters` forwards, device drained before and
+    after. Returns [{"network", "dtype", "executor", "ms", "images/s", ...}]."""
     import tempfile
     from excalibur_amd import pipeline as xp
     from excalibur_amd.mobilenet import CFG3, MobileFaceNetF32
@@ -127,11 +128,12 @@ def network_table(iters=10):
             p.run()
         p.sync()
         ms = (time.perf_counter() - t0) / iters * 1e3
+        executor = "int8 graph plan" if p.fused else "per-layer"
         p.close()
         from excalibur_amd import topologies
         gop = topologies.algorithmic_gop(net.topology(), x.shape[1:]) * x.shape[0]   # of the whole batch
         peak = {"f32": PEAK_F32_TFLOPS, "f16": PEAK_F16_TFLOPS, "int8": PEAK_INT8_TOPS}[dtype]
-        rows.append({"network": label, "dtype": dtype, "layers": len(net.lines), "ms": round(ms, 3),
+        rows.append({"network": label, "dtype": dtype, "layers": len(net.lines), "executor": executor, "ms": round(ms, 3),
                      "images/s": round(x.shape[0] / ms * 1e3, 1), "algorithmic_gop": round(gop, 1),
                      "achieved": round(gop / ms, 1), "peak": peak, "unit": "TOP/s" if dtype == "int8" else "TFLOP/s",
                      "frac": round(gop / ms / peak, 4)})
@@ -365,7 +367,7 @@ def main():
     ap.add_argument("--per-layer", action="store_true", help="print per-launch timings to stderr")
     ap.add_argument("--networks", action="store_true",
                     help="time the other configurations' whole topologies (MobileNet- and YOLOv5s-shaped, f32 / f16 / int8) "
-                         "through the per-layer executor instead of the headline benchmark")
+                         "through the pipeline (per-layer executor; int8 graph plan) instead of the headline benchmark")
     ap.add_argument("--bandwidth", action="store_true",
                     help="instead of the network: time the memory-bound kernels of the path and print their GB/s")
     args = ap.parse_args()
@@ -383,7 +385,7 @@ def main():
                           "kernels": bandwidth_table()}))
         return
     if args.networks:
-        print(json.dumps({"metric": "forward time of the generated topologies through the per-layer executor",
+        print(json.dumps({"metric": "forward time of the generated topologies through the pipeline (executor per row)",
                           "networks": network_table()}))
         return
 
@@ -543,7 +545,7 @@ def main():
         # the other configurations: single layers of cfg1 / cfg2 and the whole generated topologies of cfg3 / cfg5 through
         # the per-layer executor (python bench.py --networks prints the latter as a table)
         line["other_configs"] = {"layers": layer_table(ctx), "networks": network_table(iters=5),
-                                 "note": "networks: wall time per forward of the per-layer executor, algorithmic GOP of the batch "
+                                 "note": "networks: wall time per forward of the executor the row names, algorithmic GOP of the batch "
                                          "(convolutions and inner products) over it, against the dense MFMA peak of the dtype"}
     if not args.no_cpu_baseline:
         one, many = cpu_baseline(net, hw)
