@@ -23,18 +23,21 @@ struct exhip_lean_proj {
     int h, w, c_bytes, stride;
 };
 
-// Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then
-// runs the general kernel), another code on failure. Weights are the general kernel's packing for 64-channel slabs and
-// 64-byte channel chunks.
-int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
-                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw,
-                          const exhip_lean_proj* proj = nullptr);
-
-// The fp16 3x3 stride-1 layer on the same kernel: half operands and result, the general kernel's fp16 epilogue.
+// The layers behind the convolution that the epilogue applies (both data types): an activation layer, and a sum layer
+// behind it instead of in front of it.
 struct exhip_lean_f16_epilogue {
     int post_op;              // 0, or 1 + EXHIP_UNARY_*: the activation layer behind the convolution
     float post_alpha, post_beta;
     int residual_last;        // the shortcut is added behind post_relu / post_op
 };
+
+// Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then
+// runs the general kernel), another code on failure. Weights are the general kernel's packing for 64-channel slabs and
+// 64-byte channel chunks. `post` (may be NULL): not together with a projection.
+int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
+                          const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw,
+                          const exhip_lean_proj* proj = nullptr, const exhip_lean_f16_epilogue* post = nullptr);
+
+// The fp16 3x3 stride-1 layer on the same kernel: half operands and result, the general kernel's fp16 epilogue.
 int exhip_conv3x3_f16_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const exhip_lean_f16_epilogue& e, const uint16_t* x, const void* wp,
                            const float* bias, const uint16_t* residual, uint16_t* y);

@@ -579,7 +579,10 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
                     }
-                    if (has_res) {
+                    // the instantiation with run-time flags also takes the activation layer behind the convolution and the sum
+                    // layer behind that one (a detection network's bottleneck)
+                    const bool res_last = EPI < 0 && p.residual_last;
+                    if (has_res && !res_last) {
                         const v4f rv = __builtin_bit_cast(v4f, r4[e4]);
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] += rv[e];
@@ -594,6 +597,24 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
                     if (post_relu) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) v[e] = __builtin_fmaxf(v[e], 0.f);
+                    }
+                    if constexpr (EPI < 0) {
+                        if (p.post_op) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                switch (p.post_op - 1) {
+                                case EXHIP_UNARY_HARDSWISH: v[e] = unary_value<0>(v[e], p.post_alpha, p.post_beta); break;
+                                case EXHIP_UNARY_LEAKYRELU: v[e] = unary_value<1>(v[e], p.post_alpha, p.post_beta); break;
+                                case EXHIP_UNARY_HARDSIGMOID: v[e] = unary_value<3>(v[e], p.post_alpha, p.post_beta); break;
+                                default: v[e] = unary_value<4>(v[e], p.post_alpha, p.post_beta); break;
+                                }
+                            }
+                        }
+                        if (has_res && res_last) {
+                            const v4f rv = __builtin_bit_cast(v4f, r4[e4]);
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) v[e] += rv[e];
+                        }
                     }
                     o4[e4] = __builtin_bit_cast(v4i, v);
                     if (has_nchw) {
@@ -1302,6 +1323,7 @@ int launch(exhip_ctx* ctx, const LeanParams& p, int grid) {
 
 template <bool WRES, int NAB, int NWB>
 int launch_epi(exhip_ctx* ctx, const LeanParams& p, int grid) {
+    if (p.post_op || p.residual_last) return launch<WRES, NAB, NWB, -1>(ctx, p, grid);  // only the run-time-flag form applies them
     switch (p.flags) {
     case E_Q | E_ACT | E_QNN: return launch<WRES, NAB, NWB, (E_Q | E_ACT | E_QNN)>(ctx, p, grid);
     case E_RES | E_F | E_Q | E_POST | E_QNN: return launch<WRES, NAB, NWB, (E_RES | E_F | E_Q | E_POST | E_QNN)>(ctx, p, grid);
@@ -1347,9 +1369,13 @@ extern "C" void exhip_dev_lean_stamps(void* device_buffer) { g_lean_dbg = (long 
 
 int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t* x, const void* wp, const float* scale,
                           const float* bias, const float* residual, int8_t* y_q, float* y_f, float* y_nchw,
-                          const exhip_lean_proj* proj) {
+                          const exhip_lean_proj* proj, const exhip_lean_f16_epilogue* post) {
     int mode = g_exhip_options.lean;
     if (mode == 0) return EXHIP_ERR_UNSUPPORTED;
+    const bool with_post = post && (post->post_op || (post->residual_last && residual));
+    if (with_post && (proj || mode == 3)) return EXHIP_ERR_UNSUPPORTED;
+    if (post && post->post_op && (post->post_op < 1 || post->post_op > 1 + EXHIP_UNARY_CLIP || post->post_op == 1 + EXHIP_UNARY_SIGMOID))
+        return EXHIP_ERR_UNSUPPORTED;
     if (proj) {
         // the projection's chunks ride along the persistent streamed form; the shortcut is computed, not read
         if (residual || y_nchw || !y_f || !y_q || !g.post_relu || g.act != 0 || !(g.fs_out > 0.f)) return EXHIP_ERR_UNSUPPORTED;
@@ -1379,7 +1405,10 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
             // float32 result next to the shortcut and at most 128 channels: the general kernel's three groups per CU keep
             // more of that traffic in flight. Otherwise one tile buffer and three slice buffers (128 channels, int8 result
             // only: 50 against 56 us in the general kernel; 256 channels: 38 against 39 us with two tile buffers).
-            if (chunks <= 2 && (y_f || y_nchw || chunks == 1)) return EXHIP_ERR_UNSUPPORTED;
+            // On small maps (a detection network's 64-channel bottlenecks at 16 x 80 x 80: 27 against 34 us) the resident filter
+            // wins with a float32 result as well.
+            const bool small_map = chunks == 1 && (long long)g.n * g.oh * g.ow <= 262144;
+            if (!small_map && chunks <= 2 && (y_f || y_nchw || chunks == 1)) return EXHIP_ERR_UNSUPPORTED;
             mode = 1;
             cfg = 2;
         }
@@ -1410,7 +1439,11 @@ int exhip_conv3x3_i8_lean(exhip_ctx* ctx, const exhip_lean_geom& g, const int8_t
         p.ds_H = proj->h; p.ds_W = proj->w; p.ds_Cb = proj->c_bytes; p.ds_chunks = proj->c_bytes / 64; p.ds_stride = proj->stride;
         p.ds_img_bytes = (unsigned)((size_t)proj->h * proj->w * proj->c_bytes);
     }
-    const bool q_nonneg = g.fs_out > 0.f && (g.post_relu || (g.act == 1 && !residual));
+    if (with_post) {
+        p.post_op = post->post_op; p.post_alpha = post->post_alpha; p.post_beta = post->post_beta;
+        p.residual_last = residual && post->residual_last;
+    }
+    const bool q_nonneg = g.fs_out > 0.f && !with_post && (g.post_relu || (g.act == 1 && !residual));
     p.flags = (residual ? E_RES : 0) | (y_f ? E_F : 0) | (y_q ? E_Q : 0) | (y_nchw ? E_NCHW : 0) | (g.act == 1 ? E_ACT : 0) |
               (g.post_relu ? E_POST : 0) | (q_nonneg ? E_QNN : 0);
 

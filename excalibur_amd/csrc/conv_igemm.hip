@@ -1748,7 +1748,7 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = fused_epilogue_ok(d, p, out_elems);
-        if (fused && !d->post_op && !d->residual_last && !pl.packed && p.splits == 1 && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
+        if (fused && (!proj || (!d->post_op && !d->residual_last)) && !pl.packed && p.splits == 1 && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
             p.cstride_b % 64 == 0) {
             // the lean kernel takes these layers with the same packed weights; EXHIP_ERR_UNSUPPORTED leaves them to this one
             exhip_lean_geom g = {};
@@ -1756,8 +1756,10 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             g.pt = d->pt; g.pl = d->pl; g.ph = pl.PH; g.pw = pl.PW; g.ih = pl.IH; g.iw = pl.IW;
             g.tiles_x = pl.tiles_x; g.tiles_y = pl.tiles_y; g.ktiles = pl.ktiles;
             g.act = d->act; g.post_relu = d->post_relu; g.fs_out = d->fs_out;
+            const exhip_lean_f16_epilogue post = {d->post_op, d->post_alpha, d->post_beta, d->residual_last};
             rc = exhip_conv3x3_i8_lean(ctx, g, reinterpret_cast<const int8_t*>(p.x), p.wp, p.scale, p.bias, reinterpret_cast<const float*>(p.residual),
-                                       reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc), reinterpret_cast<float*>(p.y_nchw), proj);
+                                       reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc), reinterpret_cast<float*>(p.y_nchw), proj,
+                                       &post);
             if (rc != EXHIP_ERR_UNSUPPORTED || proj) return rc;
         }
         if (proj) return EXHIP_ERR_UNSUPPORTED;  // only the lean kernel computes a projection beside its own products
