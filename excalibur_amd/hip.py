@@ -464,6 +464,28 @@ class Ctx:
         _check(lib().exhip_focus_f16(self.h, x.ptr, y.ptr, n, c, h, w))
         return y
 
+    def input_focus_quantize(self, x, means, scales, fs, c_stride=32):
+        """Input layer, YoloV5Focus and the int8 quantizer in one pass (exhip_input_focus_quantize_nchw_f32_to_nhwc_i8): float32
+        NCHW -> int8 NHWC [n, h / 2, w / 2, c_stride]. Returns None where the library leaves the shape to the three layers."""
+        n, c, h, w = x.shape
+        y = self.empty((n, h // 2, w // 2, c_stride), np.int8)
+        m = (ctypes.c_float * len(means))(*[float(v) for v in means])
+        sc = (ctypes.c_float * len(scales))(*[float(v) for v in scales])
+        rc = lib().exhip_input_focus_quantize_nchw_f32_to_nhwc_i8(self.h, x.ptr, n, c, h, w, m, sc, ctypes.c_float(float(fs)), int(c_stride), y.ptr)
+        if rc == 10002:
+            return None
+        _check(rc)
+        return y
+
+    def nhwc_to_grouped_f32(self, x, channels, groups):
+        """[n, h, w, stride] float32 with `channels` = groups * per_group real channels -> [n, groups, h * w, per_group]
+        (exhip_nhwc_f32_to_grouped_f32): a detection head's Reshape + Transpose on the NHWC result."""
+        n, h, w, stride = x.shape
+        per_group = channels // groups
+        y = self.empty((n, groups, h * w, per_group), np.float32)
+        _check(lib().exhip_nhwc_f32_to_grouped_f32(self.h, x.ptr, n, h * w, int(groups), int(per_group), int(stride), y.ptr))
+        return y
+
     def binaryop_f32(self, op, mode, large, small):
         """op 0 ADD / 1 SUB / 2 MUL / 3 DIV; mode 0 equal shapes, 1 per image, 2 per (image, channel), 3 per (image, pixel)."""
         n, c, h, w = large.shape

@@ -777,3 +777,36 @@ def test_conv_int8_activation_layer_and_sum_in_the_epilogue(ctx, c, k, kernel, p
                           post_beta=beta, residual_last=1 if shortcut == "behind" else 0)
     assert np.array_equal(got["nhwc"][..., :k].view(np.uint32), want.transpose(0, 2, 3, 1).view(np.uint32))
     assert np.array_equal(got["i8"][..., :k], port.quantize(want, fs_out).transpose(0, 2, 3, 1))
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 16, 24), (1, 3, 6, 10), (3, 3, 32, 32)], ids=str)
+def test_input_focus_quantizer_in_one_pass(ctx, shape):
+    """The front of an int8 detection network (Input layer, YoloV5Focus, the first convolution's quantizer) in one kernel
+    against the oracle's three layers; int8 NHWC pixels of 32 bytes, 12 of them channels."""
+    r = np.random.default_rng(395)
+    x = r.uniform(0, 255, shape).astype(np.float32)
+    means, scales, fs = [10.0, 20.5, 30.25], [0.0039215, 0.004, 0.0038], np.float32(113.0)
+    want = port.quantize(port.focus(port.input_layer(x, means, scales)), fs).transpose(0, 2, 3, 1)
+    got = ctx.input_focus_quantize(ctx.array(x), means, scales, fs)
+    assert got is not None
+    got = got.download()
+    assert np.array_equal(got[..., :12], want)
+    assert not got[..., 12:].any()
+    assert np.count_nonzero(want) > want.size // 2
+    # shapes the kernel does not take are refused, not mangled
+    assert ctx.input_focus_quantize(ctx.array(x[:, :, :-1]), means, scales, fs) is None
+    assert ctx.input_focus_quantize(ctx.array(x), means, scales, fs, c_stride=64) is None
+
+
+@pytest.mark.parametrize("n,h,w,groups,per_group,stride", [(2, 8, 8, 3, 85, 256), (1, 5, 3, 3, 7, 32), (3, 4, 4, 1, 16, 16)], ids=str)
+def test_detection_head_regrouping(ctx, n, h, w, groups, per_group, stride):
+    """Reshape [n, G * J, h, w] -> [n, G, J, h * w] and Transpose of the last two axes, from the float32 NHWC tensor: the
+    oracle's transpose of the reshaped NCHW tensor."""
+    r = np.random.default_rng(396)
+    k = groups * per_group
+    nhwc = r.normal(0, 1, (n, h, w, stride)).astype(np.float32)
+    nchw = np.ascontiguousarray(nhwc[..., :k].transpose(0, 3, 1, 2))
+    want = port.transpose_hw(nchw.reshape(n, groups, per_group, h * w))
+    got = ctx.nhwc_to_grouped_f32(ctx.array(nhwc), k, groups).download()
+    assert got.shape == want.shape
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

@@ -821,3 +821,40 @@ def test_int8_graph_plan_equals_the_per_layer_executor():
         fused.close()
     finally:
         os.unlink(path)
+
+
+def test_int8_graph_plan_leaves_what_it_cannot_take_to_the_per_layer_executor():
+    """Two readers of one tensor with different feature-map scales (the plan keeps one int8 form per tensor) and a
+    sigmoid layer (not an activation the epilogues apply): both networks run layer by layer, with the same results as
+    with fusion off."""
+    from excalibur_amd import modelfile as mf
+    for change in ("scale", "sigmoid"):
+        lines, blobs, outputs = _int8_graph_net(64)
+        if change == "scale":
+            # c8 is the 8th convolution: it reads a2 next to c3, whose scale stays 12
+            at = [i for i, l in enumerate(lines) if l.startswith("Convolution c8_l ")][0]
+            n_conv = sum(1 for l in lines[:at] if l.startswith("Convolution "))
+            n_blob = sum(1 for l in lines[:at] if l.startswith(("Convolution ", "BatchNorm ")))
+            assert n_conv == 7
+            raw = bytearray(blobs[n_blob])
+            raw[-4:] = np.float32(13.0).tobytes()     # the blob ends with the feature-map scale
+            blobs[n_blob] = bytes(raw)
+        else:
+            at = [i for i, l in enumerate(lines) if l.startswith("HardSwish hs18 ")][0]
+            lines[at] = "Sigmoid hs18 1 1 c18 a18"
+        with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
+            path = f.name
+        try:
+            mf.write_model(path, blobs)
+            x = np.random.default_rng(65).uniform(0, 255, (2, 3, 64, 64)).astype(np.float32)
+            got = {}
+            for fusion in (False, True):
+                p = xp.Pipeline(mf.topology(lines, "graph"), path, 0, fusion=fusion)
+                p.forward(x)
+                assert not p.fused, change
+                got[fusion] = {b: p.get(b) for b in outputs}
+                p.close()
+            for b in outputs:
+                assert np.array_equal(got[False][b].view(np.uint32), got[True][b].view(np.uint32)), (change, b)
+        finally:
+            os.unlink(path)
