@@ -340,6 +340,21 @@ def bandwidth_table(iters=20, quiet=False, ctx=None):
     sx = ctx.array(rng.normal(0, 1, (16, 21, 320, 320)).astype(np.float32))
     sy = ctx.empty((16, 21, 320, 320), np.float32)
     bw("Softmax over 21 channels f32, 16x21x320x320", sx.size * 8, lambda: L.exhip_softmax_channels_f32(ctx.h, sx.ptr, sy.ptr, 16, 21, 320 * 320))
+    # the int8 graph plan's glue: the fused front, Concat -> BatchNorm -> LeakyReLU on float32 NHWC with the int8 copy, a head's regrouping
+    gx = ctx.array(rng.uniform(0, 255, (16, 3, 640, 640)).astype(np.float32))
+    gq = ctx.empty((16, 320, 320, 32), np.int8)
+    gm, gs = (cf * 3)(0.0, 0.0, 0.0), (cf * 3)(0.0039215, 0.0039215, 0.0039215)
+    bw("Input + Focus + int8 quantizer, 16x3x640x640 -> 16x320x320x32", gx.size * 4 + gq.size,
+       lambda: L.exhip_input_focus_quantize_nchw_f32_to_nhwc_i8(ctx.h, gx.ptr, 16, 3, 640, 640, gm, gs, cf(60.0), 32, gq.ptr))
+    fptrs, fchs = (ctypes.c_void_p * 2)(xf.ptr, yf.ptr), (ctypes.c_int * 2)(c, c)
+    bigq = ctx.empty((n, h, w, 2 * c), np.int8)
+    bw("Concat -> BatchNorm -> LeakyReLU f32 NHWC -> int8, 2 x 64 channels", cnt * 8 + cnt * 2,
+       lambda: L.exhip_concat_batchnorm_unary_nhwc_f32(ctx.h, fptrs, fchs, fchs, 2, sz(n * h * w), pa.ptr, pb.ptr, 1, cf(0.1), cf(0.0), 2 * c,
+                                                       None, bigq.ptr, cf(8.0)))
+    hx = ctx.array(rng.normal(0, 1, (16, 80, 80, 256)).astype(np.float32))
+    hy = ctx.empty((16, 3, 6400, 85), np.float32)
+    bw("Head regrouping f32 NHWC 16x80x80x(3x85) -> 16x3x6400x85", hy.size * 8,
+       lambda: L.exhip_nhwc_f32_to_grouped_f32(ctx.h, hx.ptr, 16, 6400, 3, 85, 256, hy.ptr))
     if own_ctx:
         ctx.close()
     return rows

@@ -1342,38 +1342,52 @@ __global__ __launch_bounds__(kBlock) void concat_nhwc_f16_kernel(ConcatNhwcArgs 
 // Concat (or a single blob) with the BatchNorm layer and the activation layer behind it applied on the way: the values are
 // those the layers produce one after the other (each stores halves, so the value is rounded to half between them).
 // UOP: -1 no activation, else unary_value's operation. p0 == nullptr: no BatchNorm.
-template <int UOP>
-__global__ __launch_bounds__(kBlock) void concat_affine_unary_nhwc_f16_kernel(ConcatNhwcArgs a, uint16_t* __restrict__ y, size_t total8,
+// V: 16-byte vectors (eight channels) per thread.
+template <int UOP, int V>
+__global__ __launch_bounds__(kBlock) void concat_affine_unary_nhwc_f16_kernel(ConcatNhwcArgs a, uint16_t* __restrict__ y, size_t total,
                                                                               const float* __restrict__ p0, const float* __restrict__ p1,
                                                                               float alpha, float beta) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= total8) return;
-    const int vecs = a.first[a.n_inputs] / 8;
-    const int vi = (int)(i % vecs);
-    const size_t pix = i / vecs;
-    const int c = vi * 8;
+    if (i >= total) return;
+    const int channels = a.first[a.n_inputs];
+    const int per_pixel = channels / (8 * V);
+    int part;
+    size_t pix;
+    if (total <= 0xFFFFFFFFull) {  // 32-bit division where it will do
+        const unsigned p32 = (unsigned)i / (unsigned)per_pixel;
+        part = (int)((unsigned)i - p32 * (unsigned)per_pixel);
+        pix = p32;
+    } else {
+        part = (int)(i % per_pixel);
+        pix = i / per_pixel;
+    }
+    const int c = part * 8 * V;
     int k = 0;
-#pragma unroll
-    for (int j = 1; j < 8; ++j)
-        if (j < a.n_inputs && c >= a.first[j]) k = j;
+    for (int j = 1; j < a.n_inputs; ++j)
+        if (c >= a.first[j]) k = j;
     const int ck = a.first[k + 1] - a.first[k];
-    v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, *reinterpret_cast<const v4i*>(a.src[k] + pix * ck + (c - a.first[k]))), v8f);
-    if (p0) {
-        // eight consecutive parameters of each array: 16-byte aligned where the arrays are (device allocations)
-        const v4f a0 = *reinterpret_cast<const v4f*>(p0 + c), a1 = *reinterpret_cast<const v4f*>(p0 + c + 4);
-        const v4f b0 = *reinterpret_cast<const v4f*>(p1 + c), b1 = *reinterpret_cast<const v4f*>(p1 + c + 4);
+    const v4i* src = reinterpret_cast<const v4i*>(a.src[k] + pix * ck + (c - a.first[k]));
+    v4i* dst = reinterpret_cast<v4i*>(y + pix * channels + c);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            v[e] = channel_value<1>(v[e], a0[e], b0[e]);
-            v[e + 4] = channel_value<1>(v[e + 4], a1[e], b1[e]);
+    for (int u = 0; u < V; ++u) {
+        v8f v = __builtin_convertvector(__builtin_bit_cast(v8h, src[u]), v8f);
+        if (p0) {
+            // eight consecutive parameters of each array: 16-byte aligned where the arrays are (device allocations)
+            const v4f a0 = *reinterpret_cast<const v4f*>(p0 + c + 8 * u), a1 = *reinterpret_cast<const v4f*>(p0 + c + 8 * u + 4);
+            const v4f b0 = *reinterpret_cast<const v4f*>(p1 + c + 8 * u), b1 = *reinterpret_cast<const v4f*>(p1 + c + 8 * u + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                v[e] = channel_value<1>(v[e], a0[e], b0[e]);
+                v[e + 4] = channel_value<1>(v[e + 4], a1[e], b1[e]);
+            }
+            if constexpr (UOP >= 0) v = __builtin_convertvector(__builtin_convertvector(v, v8h), v8f);
         }
-        if constexpr (UOP >= 0) v = __builtin_convertvector(__builtin_convertvector(v, v8h), v8f);
-    }
-    if constexpr (UOP >= 0) {
+        if constexpr (UOP >= 0) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = unary_value<UOP>(v[e], alpha, beta);
+            for (int e = 0; e < 8; ++e) v[e] = unary_value<UOP>(v[e], alpha, beta);
+        }
+        dst[u] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
     }
-    reinterpret_cast<v4i*>(y)[i] = __builtin_bit_cast(v4i, __builtin_convertvector(v, v8h));
 }
 
 // The float32 NHWC form of the kernel above for the int8 executor: channel blocks of up to eight float32 NHWC tensors
@@ -1386,40 +1400,67 @@ struct ConcatNhwcF32Args {
     int stride[8];  // channel stride of each input, in elements
     int n_inputs;
 };
-template <int UOP>
+// V: vectors of four channels per thread. V == 4 (every input's channel count and the output stride multiples of 16): the
+// thread's index arithmetic and input selection are shared by 16 channels and the int8 result leaves as one 16-byte store
+// -- the kernel is bound by its vector instructions, not by memory.
+template <int UOP, int V>
 __global__ __launch_bounds__(kBlock) void concat_affine_unary_nhwc_f32_kernel(ConcatNhwcF32Args a, float* __restrict__ y_f,
                                                                               int8_t* __restrict__ y_q, int out_stride, float fs,
-                                                                              size_t total4, const float* __restrict__ p0,
+                                                                              size_t total, const float* __restrict__ p0,
                                                                               const float* __restrict__ p1, float alpha, float beta) {
     const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= total4) return;
-    const int vecs = out_stride / 4;
-    const int vi = (int)(i % vecs);
-    const size_t pix = i / vecs;
-    const int c = vi * 4;
-    v4f v = {0.f, 0.f, 0.f, 0.f};
+    if (i >= total) return;
+    const int per_pixel = out_stride / (4 * V);
+    int part;
+    size_t pix;
+    if (total <= 0xFFFFFFFFull) {  // 32-bit division where it will do
+        const unsigned p32 = (unsigned)i / (unsigned)per_pixel;
+        part = (int)((unsigned)i - p32 * (unsigned)per_pixel);
+        pix = p32;
+    } else {
+        part = (int)(i % per_pixel);
+        pix = i / per_pixel;
+    }
+    const int c = part * 4 * V;
+    v4f v[V];
+#pragma unroll
+    for (int u = 0; u < V; ++u) v[u] = v4f{0.f, 0.f, 0.f, 0.f};
     if (c < a.first[a.n_inputs]) {  // pad channels of the output hold zeros
         int k = 0;
+        for (int j = 1; j < a.n_inputs; ++j)
+            if (c >= a.first[j]) k = j;
+        const float* src = a.src[k] + pix * a.stride[k] + (c - a.first[k]);
 #pragma unroll
-        for (int j = 1; j < 8; ++j)
-            if (j < a.n_inputs && c >= a.first[j]) k = j;
-        v = *reinterpret_cast<const v4f*>(a.src[k] + pix * a.stride[k] + (c - a.first[k]));
+        for (int u = 0; u < V; ++u) v[u] = reinterpret_cast<const v4f*>(src)[u];
         if (p0) {
-            const v4f a0 = *reinterpret_cast<const v4f*>(p0 + c), b0 = *reinterpret_cast<const v4f*>(p1 + c);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = channel_value<1>(v[e], a0[e], b0[e]);
+            for (int u = 0; u < V; ++u) {
+                const v4f a0 = *reinterpret_cast<const v4f*>(p0 + c + 4 * u), b0 = *reinterpret_cast<const v4f*>(p1 + c + 4 * u);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[u][e] = channel_value<1>(v[u][e], a0[e], b0[e]);
+            }
         }
         if constexpr (UOP >= 0) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = unary_value<UOP>(v[e], alpha, beta);
+            for (int u = 0; u < V; ++u)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[u][e] = unary_value<UOP>(v[u][e], alpha, beta);
         }
     }
-    if (y_f) *reinterpret_cast<v4f*>(y_f + pix * out_stride + c) = v;
-    if (y_q) {
-        uint32_t w = 0;
+    if (y_f) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w |= (uint32_t)(exhip_q8(v[e] * fs) & 0xff) << (8 * e);
-        *reinterpret_cast<uint32_t*>(y_q + pix * out_stride + c) = w;
+        for (int u = 0; u < V; ++u) reinterpret_cast<v4f*>(y_f + pix * out_stride + c)[u] = v[u];
+    }
+    if (y_q) {
+        uint32_t w[V];
+#pragma unroll
+        for (int u = 0; u < V; ++u) {
+            w[u] = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[u] |= (uint32_t)(exhip_q8(v[u][e] * fs) & 0xff) << (8 * e);
+        }
+        if constexpr (V == 4) *reinterpret_cast<v4i*>(y_q + pix * out_stride + c) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+        else *reinterpret_cast<uint32_t*>(y_q + pix * out_stride + c) = w[0];
     }
 }
 
@@ -2496,9 +2537,10 @@ extern "C" int exhip_concat_batchnorm_unary_nhwc_f16(exhip_ctx* ctx, const uint1
     EXHIP_REQUIRE((reinterpret_cast<uintptr_t>(y) & 15) == 0, "exhip_concat_batchnorm_unary_nhwc_f16: output must be 16-byte aligned");
     EXHIP_REQUIRE(!bn_a || ((reinterpret_cast<uintptr_t>(bn_a) | reinterpret_cast<uintptr_t>(bn_b)) & 15) == 0,
                   "exhip_concat_batchnorm_unary_nhwc_f16: BatchNorm parameters must be 16-byte aligned");
-    const size_t total8 = pixels * (size_t)(total / 8);
-    const dim3 grid(blocks_for(total8)), block(kBlock);
-#define EXHIP_CAU(UOP) hipLaunchKernelGGL((concat_affine_unary_nhwc_f16_kernel<UOP>), grid, block, 0, ctx->stream, a, y, total8, bn_a, bn_b, alpha, beta)
+    // one vector per thread: two (the float32 kernel's gain) measured slower on halves, 104 against 90 us at 2 x 32x64x160x160
+    const size_t threads = pixels * (size_t)(total / 8);
+    const dim3 grid(blocks_for(threads)), block(kBlock);
+#define EXHIP_CAU(UOP) hipLaunchKernelGGL((concat_affine_unary_nhwc_f16_kernel<UOP, 1>), grid, block, 0, ctx->stream, a, y, threads, bn_a, bn_b, alpha, beta)
     switch (unary_op) {
     case -1: EXHIP_CAU(-1); break;
     case EXHIP_UNARY_HARDSWISH: EXHIP_CAU(0); break;
@@ -2537,11 +2579,19 @@ extern "C" int exhip_concat_batchnorm_unary_nhwc_f32(exhip_ctx* ctx, const float
     EXHIP_REQUIRE(!y_i8 || (reinterpret_cast<uintptr_t>(y_i8) & 3) == 0, "exhip_concat_batchnorm_unary_nhwc_f32: int8 output must be 4-byte aligned");
     EXHIP_REQUIRE(!bn_a || ((reinterpret_cast<uintptr_t>(bn_a) | reinterpret_cast<uintptr_t>(bn_b)) & 15) == 0,
                   "exhip_concat_batchnorm_unary_nhwc_f32: BatchNorm parameters must be 16-byte aligned");
-    const size_t total4 = pixels * (size_t)(out_stride / 4);
-    const dim3 grid(blocks_for(total4)), block(kBlock);
-#define EXHIP_CAU32(UOP)                                                                                                              \
-    hipLaunchKernelGGL((concat_affine_unary_nhwc_f32_kernel<UOP>), grid, block, 0, ctx->stream, a, y_f32, y_i8, out_stride, fs_out, total4, \
-                       bn_a, bn_b, alpha, beta)
+    bool wide = out_stride % 16 == 0 && (!y_i8 || (reinterpret_cast<uintptr_t>(y_i8) & 15) == 0);
+    for (int i = 0; i < n_inputs; ++i) wide = wide && channels[i] % 16 == 0;
+    const size_t threads = pixels * (size_t)(out_stride / (wide ? 16 : 4));
+    const dim3 grid(blocks_for(threads)), block(kBlock);
+#define EXHIP_CAU32(UOP)                                                                                                                      \
+    do {                                                                                                                                      \
+        if (wide)                                                                                                                             \
+            hipLaunchKernelGGL((concat_affine_unary_nhwc_f32_kernel<UOP, 4>), grid, block, 0, ctx->stream, a, y_f32, y_i8, out_stride, fs_out, \
+                               threads, bn_a, bn_b, alpha, beta);                                                                              \
+        else                                                                                                                                  \
+            hipLaunchKernelGGL((concat_affine_unary_nhwc_f32_kernel<UOP, 1>), grid, block, 0, ctx->stream, a, y_f32, y_i8, out_stride, fs_out, \
+                               threads, bn_a, bn_b, alpha, beta);                                                                              \
+    } while (0)
     switch (unary_op) {
     case -1: EXHIP_CAU32(-1); break;
     case EXHIP_UNARY_HARDSWISH: EXHIP_CAU32(0); break;
