@@ -817,6 +817,17 @@ def test_int8_graph_plan_equals_the_per_layer_executor():
             # a blob inside the plan comes from a per-layer rerun of the same input
             assert not fused.stored("a5")
             assert np.array_equal(fused.get("s5"), plain.get("s5"))
+        # the plan's launches replayed as one HIP graph (the front kernel stays eager, the tail layers run behind the replay):
+        # every replay against the eager results, with other work and synchronisations between the replays
+        replay = xp.Pipeline(mf.topology(lines, "graph"), path, 0, fusion=True)
+        replay.set_graphs(True)
+        for seed in (62, 66, 62, 67):
+            x = np.random.default_rng(seed).uniform(0, 255, (2, 3, 64, 64)).astype(np.float32)
+            fused.forward(x)
+            replay.forward(x)
+            for b in outputs:
+                assert np.array_equal(fused.get(b).view(np.uint32), replay.get(b).view(np.uint32)), (b, seed)
+        replay.close()
         plain.close()
         fused.close()
     finally:
