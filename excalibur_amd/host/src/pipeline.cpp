@@ -1128,6 +1128,14 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         int n = 0, c = 0, h = 0, w = 0, cs = 0;
         void *f32 = nullptr, *i8 = nullptr;
         float** nchw = nullptr;
+        // readers with other feature-map scales than `fs`: their int8 forms are made from the float32 form by a quantizer launch
+        std::vector<std::pair<float, void*>> more_i8;
+        const void* int8_at(float scale) const {
+            if (i8 && fs == scale) return i8;
+            for (const auto& m : more_i8)
+                if (m.first == scale) return m.second;
+            return nullptr;
+        }
     };
     std::vector<value_info> vals(n_blobs);
     for (int b = 0; b < n_blobs; ++b)
@@ -1136,9 +1144,19 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         for (int b : op_inputs_[t])
             if (where[root(b)] == 0) vals[root(b)].need_nchw = true;
     auto want_i8 = [&](int v, float fs) {
-        if (!(fs > 0.f) || (vals[v].need_i8 && vals[v].fs != fs)) return refuse(19);  // one int8 form per tensor
-        vals[v].need_i8 = true;
-        vals[v].fs = fs;
+        if (!(fs > 0.f)) return refuse(19);
+        value_info& val = vals[v];
+        if (!val.need_i8) {
+            val.need_i8 = true;
+            val.fs = fs;
+        } else if (val.fs != fs) {
+            // a second scale: that form comes from the float32 form (the network's input has none: layer by layer then)
+            if (where[v] != 0) return refuse(43);
+            bool known = false;
+            for (const auto& m : val.more_i8) known = known || m.first == fs;
+            if (!known) val.more_i8.emplace_back(fs, nullptr);
+            val.need_f32 = true;
+        }
         return true;
     };
     // channel counts are known from the layers alone; an int8 Concat needs inputs without pad channels
@@ -1270,13 +1288,32 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         plan->launches.push_back(
             [=]() { EXHIP_FATAL(exhip_nhwc_f32_to_nchw_f32(ctx, static_cast<const float*>(o.f32), o.n, o.c, o.h, o.w, o.cs, *slot)); });
     };
+    // the int8 forms of a value at its readers' other scales: the quantizer on the float32 NHWC form
+    auto more_forms = [&](value_info& v) {
+        if (v.more_i8.empty()) return true;
+        if (!v.f32 || v.c % 4 != 0 || v.cs % 4 != 0) return false;
+        const size_t pixels = static_cast<size_t>(v.n) * v.h * v.w;
+        for (auto& m : v.more_i8) {
+            m.second = alloc(pixels * v.cs);
+            const float* src = static_cast<const float*>(v.f32);
+            int8_t* dst = static_cast<int8_t*>(m.second);
+            const int ch = v.c, stride = v.cs;
+            const float scale = m.first;
+            plan->launches.push_back([=]() {
+                EXHIP_FATAL(exhip_concat_batchnorm_unary_nhwc_f32(ctx, &src, &ch, &stride, 1, pixels, nullptr, nullptr, -1, 0.f, 0.f, stride, nullptr, dst,
+                                                                  scale));
+            });
+        }
+        return true;
+    };
     for (const node& nd : nodes) {
         const value_info in = vals[nd.in[0]];
         value_info& out = vals[nd.out];
         if (in.n == 0) return refuse(28);
         if (nd.kind == 'c') {
             auto* c = static_cast<conv_t*>(operations_[nd.op].get());
-            if (in.c != c->input_channels() || !in.i8) return refuse(29);
+            const int8_t* x = static_cast<const int8_t*>(in.int8_at(c->featmap_scale()));
+            if (in.c != c->input_channels() || !x) return refuse(29);
             const int ks = pad_to(c->output_channel_, 32);
             exhip_conv_desc d = c->describe(in.n, in.h, in.w, in.cs, ks);
             d.post_relu = nd.post_relu ? 1 : 0;
@@ -1304,7 +1341,6 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                 const void* wp = c->pin_packed_weights(EXHIP_I8, d);
                 plan->pinned.emplace_back([c, wp]() { c->unpin_packed_weights(wp); });
                 const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
-                const int8_t* x = static_cast<const int8_t*>(in.i8);
                 plan->launches.push_back([=]() {
                     EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, nullptr, nullptr, mid, nullptr, nullptr));
                     EXHIP_FATAL(exhip_nhwc_f32_to_grouped_f32(ctx, mid, n0, hw, groups, per_group, ks, *slot));
@@ -1323,7 +1359,6 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             const void* wp = c->pin_packed_weights(EXHIP_I8, d);  // the launch keeps this pointer
             plan->pinned.emplace_back([c, wp]() { c->unpin_packed_weights(wp); });
             const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
-            const int8_t* x = static_cast<const int8_t*>(in.i8);
             int8_t* yq = static_cast<int8_t*>(out.i8);
             float* yf = static_cast<float*>(out.f32);
             plan->launches.push_back(
@@ -1335,8 +1370,9 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             for (int v : nd.in) {
                 const value_info& s = vals[v];
                 if (s.n != in.n || s.h != in.h || s.w != in.w || s.c % 4 != 0) return refuse(31);
-                if (nd.as_f32 ? !s.f32 : (!s.i8 || s.cs != s.c || s.c % 16 != 0)) return refuse(32);
-                ptrs.push_back(nd.as_f32 ? s.f32 : s.i8);
+                const void* form = nd.as_f32 ? s.f32 : s.int8_at(out.fs);
+                if (!form || (!nd.as_f32 && (s.cs != s.c || s.c % 16 != 0))) return refuse(32);
+                ptrs.push_back(form);
                 channels.push_back(s.c);
                 strides.push_back(s.cs);
                 total += s.c;
@@ -1388,9 +1424,9 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             out.n = in.n; out.c = in.c; out.h = oh; out.w = ow; out.cs = in.cs;
             const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
             if (out.need_i8) {
-                if (!in.i8 || in.cs % 16 != 0) return refuse(36);
+                const uint16_t* x = static_cast<const uint16_t*>(in.int8_at(out.fs));
+                if (!x || in.cs % 16 != 0) return refuse(36);
                 out.i8 = alloc(elems);
-                const uint16_t* x = static_cast<const uint16_t*>(in.i8);
                 uint16_t* y = static_cast<uint16_t*>(out.i8);
                 plan->launches.push_back([=]() { EXHIP_FATAL(exhip_interp_nearest_nhwc_f16(ctx, x, y, in.n, in.cs / 2, in.h, in.w, oh, ow)); });
             }
@@ -1428,6 +1464,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             });
             nchw_from_f32(out, nd.out);
         }
+        if (!more_forms(out)) return refuse(44);
     }
     // the network's outputs: results of the plan by name (Split copies share their tensor), the rest comes from the tail
     for (const std::string& o : output_names_) {

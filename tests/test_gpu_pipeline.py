@@ -834,10 +834,10 @@ def test_int8_graph_plan_equals_the_per_layer_executor():
         os.unlink(path)
 
 
-def test_int8_graph_plan_leaves_what_it_cannot_take_to_the_per_layer_executor():
-    """Two readers of one tensor with different feature-map scales (the plan keeps one int8 form per tensor) and a
-    sigmoid layer (not an activation the epilogues apply): both networks run layer by layer, with the same results as
-    with fusion off."""
+def test_int8_graph_plan_second_scale_and_refusal():
+    """Two readers of one tensor with different feature-map scales: the plan makes the second int8 form from the float32
+    form with a quantizer launch and still takes the network. A sigmoid layer (not an activation the epilogues apply)
+    leaves the network to the per-layer executor. Same results as with fusion off either way."""
     from excalibur_amd import modelfile as mf
     for change in ("scale", "sigmoid"):
         lines, blobs, outputs = _int8_graph_net(64)
@@ -862,7 +862,7 @@ def test_int8_graph_plan_leaves_what_it_cannot_take_to_the_per_layer_executor():
             for fusion in (False, True):
                 p = xp.Pipeline(mf.topology(lines, "graph"), path, 0, fusion=fusion)
                 p.forward(x)
-                assert not p.fused, change
+                assert p.fused == (fusion and change == "scale"), change
                 got[fusion] = {b: p.get(b) for b in outputs}
                 p.close()
             for b in outputs:
