@@ -175,6 +175,11 @@ def network_table(iters=10):
     for dt, int8 in (("f32", False), ("f16", False), ("int8", True)):
         text, _ = topologies.yolov5s_simp(640, int8=int8)
         run("yolov5s_simp topology (3 heads x 255 channels), 16x3x640x640", Seeded(text, 5), x, dt, "f32" if int8 else dt)
+    # the int8 network Excalibur ships: a residual network with Eltwise sums, ReLU layers and a depthwise tail
+    light = topologies.unicorn_light_int8()
+    light = light[0] if isinstance(light, tuple) else light
+    x = r.uniform(0, 255, (64, 3, 128, 128)).astype(np.float32)
+    run("unicorn_light_int8 topology, 64x3x128x128", Seeded(light, 6), x, "int8", "f32")
     return rows
 
 

@@ -952,45 +952,43 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             if (producer[o] >= 0 || o == blob_index_[input_names_[0]]) return refuse(2);
             producer[o] = i;
         }
-        if (dynamic_cast<operation_convolutiondepthwise<float>*>(op)) return refuse(3);
-        if (auto* c = dynamic_cast<conv_t*>(op)) {
-            if (!c->param().int8_quantization_ || c->group_ != 1 || c->stride_h_ != c->stride_w_ || c->dilation_h_ != 1 || c->dilation_w_ != 1 ||
-                c->activation_type_ > 1 || c->weights_i8().empty() || op_inputs_[i].size() != 1 || op_outputs_[i].size() != 1)
-                return refuse(4);
-            kind[i] = 'c';
+        // A layer the plan has no launch for is a tail layer ('t'): it runs as a layer behind the launches, on the NCHW results
+        // of the plan. That is right where such layers end a network (a depthwise or float convolution, a sigmoid, an inner
+        // product, Reshape / Transpose); one in the middle, whose result a planned layer reads, makes the plan refuse below.
+        kind[i] = 't';
+        if (dynamic_cast<operation_convolutiondepthwise<float>*>(op)) {
+        } else if (auto* c = dynamic_cast<conv_t*>(op)) {
+            if (c->param().int8_quantization_ && c->group_ == 1 && c->stride_h_ == c->stride_w_ && c->dilation_h_ == 1 && c->dilation_w_ == 1 &&
+                c->activation_type_ <= 1 && !c->weights_i8().empty() && op_inputs_[i].size() == 1 && op_outputs_[i].size() == 1)
+                kind[i] = 'c';
         } else if (auto* u = dynamic_cast<operation_unary<float>*>(op)) {
-            if (u->op_ == EXHIP_UNARY_SIGMOID) return refuse(5);
-            kind[i] = 'u';
+            if (u->op_ != EXHIP_UNARY_SIGMOID) kind[i] = 'u';
         } else if (dynamic_cast<operation_relu<float>*>(op)) {
             kind[i] = 'r';
         } else if (dynamic_cast<operation_split<float>*>(op)) {
             kind[i] = 's';
             for (int o : op_outputs_[i]) alias[o] = alias[op_inputs_[i][0]];
         } else if (auto* b = dynamic_cast<operation_binaryop<float>*>(op)) {
-            if (b->op_type_ != 0 || b->with_scalar_ || op_inputs_[i].size() != 2) return refuse(6);
-            kind[i] = 'a';
+            if (b->op_type_ == 0 && !b->with_scalar_ && op_inputs_[i].size() == 2) kind[i] = 'a';
+        } else if (auto* e = dynamic_cast<operation_eltwise<float>*>(op)) {
+            // a two-input SUM with unit coefficients is the same sum (x * 1 is exact, fused or not)
+            if (e->type_ == 1 && op_inputs_[i].size() == 2 && e->coeffs_.size() == 2 && e->coeffs_[0] == 1.f && e->coeffs_[1] == 1.f) kind[i] = 'a';
         } else if (auto* k = dynamic_cast<operation_concat<float>*>(op)) {
-            if (k->axis_ + 2 != 1 || op_inputs_[i].size() > 8) return refuse(7);
-            kind[i] = 'k';
+            if (k->axis_ + 2 == 1 && op_inputs_[i].size() <= 8) kind[i] = 'k';
         } else if (dynamic_cast<operation_batchnorm<float>*>(op)) {
             kind[i] = 'b';
         } else if (auto* ip = dynamic_cast<operation_interp<float>*>(op)) {
-            if (ip->resize_type_ != 1 || ip->align_corner_ != 0) return refuse(8);
-            kind[i] = 'i';
+            if (ip->resize_type_ == 1 && ip->align_corner_ == 0) kind[i] = 'i';
         } else if (auto* p = dynamic_cast<operation_pooling<float>*>(op)) {
-            if (p->type_ != 0 || p->global_pooling_) return refuse(9);
-            kind[i] = 'p';
+            if (p->type_ == 0 && !p->global_pooling_) kind[i] = 'p';
         } else if (dynamic_cast<operation_input<float>*>(op)) {
             kind[i] = 'n';
         } else if (dynamic_cast<operation_yolov5focus<float>*>(op)) {
             kind[i] = 'f';
-        } else if (dynamic_cast<operation_reshape<float>*>(op) || dynamic_cast<operation_transpose<float>*>(op)) {
-            kind[i] = 't';
-        } else {
-            return refuse(10);
         }
-        if (kind[i] != 's' && kind[i] != 'a' && kind[i] != 'k' && (op_inputs_[i].size() != 1 || op_outputs_[i].size() != 1)) return refuse(11);
-        if (op_outputs_[i].size() != 1 && kind[i] != 's') return refuse(12);
+        if (kind[i] != 's' && kind[i] != 'a' && kind[i] != 'k' && kind[i] != 't' && (op_inputs_[i].size() != 1 || op_outputs_[i].size() != 1))
+            return refuse(11);
+        if (op_outputs_[i].size() != 1 && kind[i] != 's' && kind[i] != 't') return refuse(12);
     }
     auto root = [&](int b) { return alias[b]; };
     std::vector<std::vector<int>> consumers(n_blobs);
@@ -1112,10 +1110,17 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     }
     std::stable_sort(nodes.begin(), nodes.end(), [](const node& a, const node& b) { return a.at < b.at; });
     for (int i = 0; i < n_ops; ++i) {
-        if (kind[i] != 't' || absorbed[i]) continue;
-        plan->tail_ops.push_back(i);
-        where[root(op_outputs_[i][0])] = 2;
+        if (absorbed[i]) continue;
+        if (kind[i] == 't') {
+            for (int b : op_inputs_[i])
+                if (where[root(b)] == 1) return refuse(45);  // the front chain's blobs are not kept
+            plan->tail_ops.push_back(i);
+            for (int o : op_outputs_[i]) where[root(o)] = 2;
+        } else if (kind[i] == 's' && where[root(op_inputs_[i][0])] == 2) {
+            plan->tail_ops.push_back(i);  // a Split of a tail blob runs as a layer too: its tops are blobs the tail reads by name
+        }
     }
+    if (plan->tail_ops.size() == static_cast<size_t>(n_ops)) return refuse(46);  // nothing left to plan
     for (int i = 0; i < n_ops; ++i)  // nothing but the tail reads the tail
         if (kind[i] != 't' && kind[i] != 's')
             for (int b : op_inputs_[i])

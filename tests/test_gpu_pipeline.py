@@ -106,8 +106,9 @@ def test_resnet18_topology_through_the_pipeline(fusion):
         os.unlink(path)
 
 
-def test_mixed_topology_falls_back_to_per_layer():
-    """conv(int8) -> global average pool -> inner product: not a fusable chain; runs layer by layer."""
+def test_mixed_topology_plans_the_convolution_and_runs_the_rest_as_layers():
+    """conv(int8) -> global average pool -> inner product: the int8 graph plan takes the convolution and runs the two
+    layers behind it as layers on its NCHW result; with fusion off everything runs layer by layer. Same values."""
     from excalibur_amd import modelfile as mf
     r = np.random.default_rng(31)
     c = cases.conv_i8_case(32, 2, 16, 12, 12, 32, 3, 1, 1)
@@ -120,15 +121,19 @@ def test_mixed_topology_falls_back_to_per_layer():
         f.write(mf.conv_blob_i8(c["wt"], c["bias"], c["ws"], c["fs"]) + mf.fc_blob_f32(wfc, bfc))
         path = f.name
     try:
-        p = xp.Pipeline(mf.topology(lines), path, 0)
-        p.forward(c["x"])
-        assert not p.fused
         a = cases.oracle_eval(c)
         b = port.pool2d(a, port.POOL_AVE, global_pool=True)
         want = port.innerproduct(b, wfc, bfc)
-        assert np.array_equal(p.get("a"), a)
-        assert cases.check_value(p.get("out"), want, 1e-4) == 0
-        p.close()
+        outs = {}
+        for fusion in (True, False):
+            p = xp.Pipeline(mf.topology(lines), path, 0, fusion=fusion)
+            p.forward(c["x"])
+            assert p.fused == fusion
+            assert np.array_equal(p.get("a"), a)
+            outs[fusion] = p.get("out")
+            assert cases.check_value(outs[fusion], want, 1e-4) == 0
+            p.close()
+        assert np.array_equal(outs[True], outs[False])
     finally:
         os.unlink(path)
 
@@ -596,12 +601,15 @@ def test_int8_convolutions_hand_their_readers_int8_tensors():
     conv("a2y", "c4", 24, 32, 3, 1, 50.0)
     lines.append("Split sp3 1 2 c3 c3x c3y")                 # c3: an int8 reader and a float reader
     conv("c3x", "c5", 32, 32, 1, 1, 20.0)
-    lines.append("Eltwise sum 2 1 c3y c4 s 0=1")             # c4: float reader only
+    lines.append("Split sp4 1 2 c4 c4a c4b")
+    lines.append("Eltwise sum 2 1 c3y c4a s 0=1")            # c4: float readers only
+    lines.append("Sigmoid sg4 1 1 c4b g4")                   # a sigmoid in the middle: no int8 plan takes this network,
+    conv("g4", "c9", 32, 16, 1, 1, 90.0)                     # so the per-layer executor's own joins are what runs
     conv("s", "c6", 32, 64, 3, 1, 25.0)
     lines.append("Split sp6 1 2 c6 c6x c6y")                 # c6: two int8 readers with different scales
     conv("c6x", "c7", 64, 16, 1, 1, 35.0)
     conv("c6y", "c8", 64, 16, 1, 1, 45.0)
-    outputs = ["c5", "c7", "c8"]
+    outputs = ["c5", "c7", "c8", "c9"]
     x = np.random.default_rng(52).normal(0, 1.0, (2, 3, 24, 24)).astype(np.float32)
     with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
         path = f.name
@@ -836,10 +844,11 @@ def test_int8_graph_plan_equals_the_per_layer_executor():
 
 def test_int8_graph_plan_second_scale_and_refusal():
     """Two readers of one tensor with different feature-map scales: the plan makes the second int8 form from the float32
-    form with a quantizer launch and still takes the network. A sigmoid layer (not an activation the epilogues apply)
-    leaves the network to the per-layer executor. Same results as with fusion off either way."""
+    form with a quantizer launch and still takes the network. A sigmoid layer (not an activation the epilogues apply) at
+    the end of a branch runs as a layer behind the plan's launches; in the middle, where a convolution reads its result, it
+    leaves the network to the per-layer executor. Same results as with fusion off in every case."""
     from excalibur_amd import modelfile as mf
-    for change in ("scale", "sigmoid"):
+    for change in ("scale", "sigmoid at the end", "sigmoid in the middle"):
         lines, blobs, outputs = _int8_graph_net(64)
         if change == "scale":
             # c8 is the 8th convolution: it reads a2 next to c3, whose scale stays 12
@@ -850,9 +859,12 @@ def test_int8_graph_plan_second_scale_and_refusal():
             raw = bytearray(blobs[n_blob])
             raw[-4:] = np.float32(13.0).tobytes()     # the blob ends with the feature-map scale
             blobs[n_blob] = bytes(raw)
-        else:
+        elif change == "sigmoid at the end":
             at = [i for i, l in enumerate(lines) if l.startswith("HardSwish hs18 ")][0]
             lines[at] = "Sigmoid hs18 1 1 c18 a18"
+        else:
+            at = [i for i, l in enumerate(lines) if l.startswith("HardSwish hs10 ")][0]
+            lines[at] = "Sigmoid hs10 1 1 c10 a10"
         with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
             path = f.name
         try:
@@ -862,7 +874,7 @@ def test_int8_graph_plan_second_scale_and_refusal():
             for fusion in (False, True):
                 p = xp.Pipeline(mf.topology(lines, "graph"), path, 0, fusion=fusion)
                 p.forward(x)
-                assert p.fused == (fusion and change == "scale"), change
+                assert p.fused == (fusion and change != "sigmoid in the middle"), change
                 got[fusion] = {b: p.get(b) for b in outputs}
                 p.close()
             for b in outputs:
