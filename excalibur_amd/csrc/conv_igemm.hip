@@ -1748,7 +1748,8 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = fused_epilogue_ok(d, p, out_elems);
-        if (fused && (!proj || (!d->post_op && !d->residual_last)) && !pl.packed && p.splits == 1 && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
+        // (also where this kernel would split the reduction of a small launch, down to 16 tiles: as for the fp16 layers above)
+        if (fused && (!proj || (!d->post_op && !d->residual_last)) && !pl.packed && (p.splits == 1 || (tiles >= 16 && g_exhip_options.force_splits <= 1)) && d->kh == 3 && d->kw == 3 && d->sh == 1 && pl.variant == 0 && pl.chunk_b == 64 && pl.RS == 1 &&
             p.cstride_b % 64 == 0) {
             // the lean kernel takes these layers with the same packed weights; EXHIP_ERR_UNSUPPORTED leaves them to this one
             exhip_lean_geom g = {};
