@@ -400,6 +400,11 @@ def main():
         from excalibur_amd import hip as _hip
         _hip.LIB_PATH = os.path.abspath(args.exhip_lib)
 
+    if args.option:   # library options hold for every mode of this script
+        from excalibur_amd import pipeline as _xp
+        for item in args.option:
+            name, _, value = item.partition("=")
+            _xp.set_option(name, int(value))
     if args.bandwidth:
         print(json.dumps({"metric": "achieved HBM GB/s of the memory-bound kernels", "peak_GB/s": PEAK_HBM_GBS,
                           "kernels": bandwidth_table()}))
@@ -432,9 +437,6 @@ def main():
     in_flight = max(1, min(args.in_flight, 8))
     if args.shared_gpu_plans:
         xp.set_option("share_gpu", 1)
-    for item in args.option:
-        name, _, value = item.partition("=")
-        xp.set_option(name, int(value))
     pipes = []
     for k in range(in_flight):
         xp.set_stream_slot(k)

@@ -430,17 +430,19 @@ namespace {
 template <int DT>
 int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has_residual) {
     if (g_exhip_options.pw == 0) return EXHIP_ERR_UNSUPPORTED;
-    // Measured against the general kernel on the pointwise layers of a detection and a mobile network (16 and 64 images):
-    // this form wins where a launch is short, twice as fast on 20 x 20 maps, and for a lone 32-channel block (which the
-    // general kernel pads to a 64-channel slab); from about 2 GFLOP on, the general kernel's staged tiles re-read less
-    // and win. Option pw = 2 takes every layer the kernel can (tests).
+    // Measured per layer against the general kernel inside a detection and two mobile networks (16 and 64 images, kernel
+    // traces): this form wins where a launch is short -- every layer of at most 32 768 pixels up to about 7 GFLOP (twice
+    // as fast on 20 x 20 maps) --, for a lone 32-channel block (which the general kernel pads to a 64-channel slab), and on
+    // larger maps while the input is narrow: fp16 up to 64 input channels (64 -> 64 at 16 x 160 x 160: 42 against 49 us)
+    // and 128 -> 64 at 80 x 80; int8 up to 64 channels at 131 072 pixels, and layers with only a float32 result (its
+    // 64-byte store runs against the general epilogue's 16-byte pieces: 41 against 60 us on a 128 -> 255 head at
+    // 16 x 80 x 80). Beyond that the general kernel's staged tiles re-read less and win (128 -> 128 at 80 x 80).
+    // Option pw = 2 takes every layer the kernel can (tests), 0 none.
     const int blocks_needed = (std::max(g.k, g.k_stride) + 31) / 32;
-    // The int8 layers of the same networks: this form wins on every layer of at most 32 768 pixels (up to 6.7 GOP measured)
-    // and, up to 131 072 pixels, on layers of at most 64 input channels and on those with only a float32 result (its
-    // 64-byte store runs against the general epilogue's 16-byte pieces: 41 against 60 us on a 128 -> 255 head at 16 x 80 x 80).
     const double flop = 2.0 * (double)g.pixels * (g.c_bytes / es) * g.k;
-    bool take = blocks_needed == 1 || (flop <= (DT == EXHIP_I8 ? 8.0e9 : 2.0e9) && g.pixels <= 32768);
+    bool take = blocks_needed == 1 || (flop <= 8.0e9 && g.pixels <= 32768);
     if (DT == EXHIP_I8 && g.pixels <= 131072 && (g.c_bytes <= 64 || (p.y_f && !p.y_q))) take = true;
+    if (DT == EXHIP_F16 && ((g.c_bytes <= 128 && g.pixels <= 524288) || (g.c_bytes <= 256 && g.k <= 64 && g.pixels <= 131072))) take = true;
     if (g_exhip_options.pw != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
     if (g.pixels <= 0 || g.c_bytes <= 0 || g.c_bytes % 32 != 0 || (g.slab_blocks != 2 && g.slab_blocks != 4) || g.k_stride % 8 != 0)
         return EXHIP_ERR_UNSUPPORTED;
