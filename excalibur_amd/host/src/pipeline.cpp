@@ -932,15 +932,16 @@ bool pipeline<float>::impl::build_block_plan(const tensor_ptr& input, const std:
 // Values are those of the per-layer executor. Anything else in the topology returns false (the per-layer executor runs).
 template <>
 bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std::vector<int>& shape) {
-    // EXCALIBUR_PLAN_DEBUG=1 in the environment names the check that left a network to the per-layer executor
-    auto refuse = [&](int check) {
-        if (std::getenv("EXCALIBUR_PLAN_DEBUG")) LOG(INFO) << name_ << ": int8 graph plan not used (check " << check << ")";
+    // EXCALIBUR_PLAN_DEBUG=1 in the environment names the check (by its line in this file) that left a network to the
+    // per-layer executor
+    auto refuse = [&](int line) {
+        if (std::getenv("EXCALIBUR_PLAN_DEBUG")) LOG(INFO) << name_ << ": int8 graph plan not used (the check at pipeline.cpp:" << line << ")";
         return false;
     };
     using conv_t = operation_convolution<float>;
     const int n_ops = static_cast<int>(operations_.size());
     const int n_blobs = static_cast<int>(blob_names_.size());
-    if (input->order() != memory::NCHW || shape.size() != 4 || input_names_.size() != 1) return refuse(1);
+    if (input->order() != memory::NCHW || shape.size() != 4 || input_names_.size() != 1) return refuse(__LINE__);
 
     // ---- classify; blobs must be written once (a layer writing over its input is left to the per-layer executor) ----
     std::vector<int> alias(n_blobs), producer(n_blobs, -1);
@@ -949,7 +950,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     for (int i = 0; i < n_ops; ++i) {
         operation<float>* op = operations_[i].get();
         for (int o : op_outputs_[i]) {
-            if (producer[o] >= 0 || o == blob_index_[input_names_[0]]) return refuse(2);
+            if (producer[o] >= 0 || o == blob_index_[input_names_[0]]) return refuse(__LINE__);
             producer[o] = i;
         }
         // A layer the plan has no launch for is a tail layer ('t'): it runs as a layer behind the launches, on the NCHW results
@@ -987,8 +988,8 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             kind[i] = 'f';
         }
         if (kind[i] != 's' && kind[i] != 'a' && kind[i] != 'k' && kind[i] != 't' && (op_inputs_[i].size() != 1 || op_outputs_[i].size() != 1))
-            return refuse(11);
-        if (op_outputs_[i].size() != 1 && kind[i] != 's' && kind[i] != 't') return refuse(12);
+            return refuse(__LINE__);
+        if (op_outputs_[i].size() != 1 && kind[i] != 's' && kind[i] != 't') return refuse(__LINE__);
     }
     auto root = [&](int b) { return alias[b]; };
     std::vector<std::vector<int>> consumers(n_blobs);
@@ -1008,15 +1009,15 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     std::vector<int> front_shape = shape;
     for (int i = 0; i < n_ops; ++i) {
         if (kind[i] != 'n' && kind[i] != 'f') continue;
-        if (root(op_inputs_[i][0]) != front_value || consumers[front_value].size() != 1 || is_output[front_value]) return refuse(13);
+        if (root(op_inputs_[i][0]) != front_value || consumers[front_value].size() != 1 || is_output[front_value]) return refuse(__LINE__);
         plan->front_ops.push_back(i);
         front_value = root(op_outputs_[i][0]);
         where[front_value] = 1;
         if (kind[i] == 'f') front_shape = {front_shape[0], front_shape[1] * 4, front_shape[2] / 2, front_shape[3] / 2};
     }
-    if (is_output[front_value] || consumers[front_value].empty()) return refuse(14);
+    if (is_output[front_value] || consumers[front_value].empty()) return refuse(__LINE__);
     for (int c : consumers[front_value])
-        if (kind[c] != 'c') return refuse(15);
+        if (kind[c] != 'c') return refuse(__LINE__);
 
     // ---- nodes ----
     struct node {
@@ -1072,7 +1073,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             if (sum >= 0) {
                 const int x = root(op_inputs_[sum][0]), y = root(op_inputs_[sum][1]);
                 nd.res = x == nd.out ? y : x;
-                if (nd.res == nd.out) return refuse(17);
+                if (nd.res == nd.out) return refuse(__LINE__);
                 nd.residual_last = act >= 0;
                 absorb(sum);
                 if (act < 0) {  // the activation behind the sum
@@ -1104,7 +1105,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                 }
             }
         } else if (kind[i] == 'a' || kind[i] == 'r') {
-            return refuse(18);  // a sum or ReLU no convolution's epilogue takes
+            return refuse(__LINE__);  // a sum or ReLU no convolution's epilogue takes
         }
         nodes.push_back(nd);
     }
@@ -1113,18 +1114,18 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         if (absorbed[i]) continue;
         if (kind[i] == 't') {
             for (int b : op_inputs_[i])
-                if (where[root(b)] == 1) return refuse(45);  // the front chain's blobs are not kept
+                if (where[root(b)] == 1) return refuse(__LINE__);  // the front chain's blobs are not kept
             plan->tail_ops.push_back(i);
             for (int o : op_outputs_[i]) where[root(o)] = 2;
         } else if (kind[i] == 's' && where[root(op_inputs_[i][0])] == 2) {
             plan->tail_ops.push_back(i);  // a Split of a tail blob runs as a layer too: its tops are blobs the tail reads by name
         }
     }
-    if (plan->tail_ops.size() == static_cast<size_t>(n_ops)) return refuse(46);  // nothing left to plan
+    if (plan->tail_ops.size() == static_cast<size_t>(n_ops)) return refuse(__LINE__);  // nothing left to plan
     for (int i = 0; i < n_ops; ++i)  // nothing but the tail reads the tail
         if (kind[i] != 't' && kind[i] != 's')
             for (int b : op_inputs_[i])
-                if (where[root(b)] == 2) return refuse(16);
+                if (where[root(b)] == 2) return refuse(__LINE__);
 
     // ---- what each value must exist as: readers first ----
     struct value_info {
@@ -1149,14 +1150,14 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         for (int b : op_inputs_[t])
             if (where[root(b)] == 0) vals[root(b)].need_nchw = true;
     auto want_i8 = [&](int v, float fs) {
-        if (!(fs > 0.f)) return refuse(19);
+        if (!(fs > 0.f)) return refuse(__LINE__);
         value_info& val = vals[v];
         if (!val.need_i8) {
             val.need_i8 = true;
             val.fs = fs;
         } else if (val.fs != fs) {
             // a second scale: that form comes from the float32 form (the network's input has none: layer by layer then)
-            if (where[v] != 0) return refuse(43);
+            if (where[v] != 0) return refuse(__LINE__);
             bool known = false;
             for (const auto& m : val.more_i8) known = known || m.first == fs;
             if (!known) val.more_i8.emplace_back(fs, nullptr);
@@ -1176,29 +1177,29 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     for (auto it = nodes.rbegin(); it != nodes.rend(); ++it) {
         node& nd = *it;
         const value_info out = vals[nd.out];
-        if (where[nd.out] != 0) return refuse(20);
+        if (where[nd.out] != 0) return refuse(__LINE__);
         if (nd.kind == 'c') {
             auto* c = static_cast<conv_t*>(operations_[nd.op].get());
-            if (!want_i8(nd.in[0], c->featmap_scale())) return refuse(21);
+            if (!want_i8(nd.in[0], c->featmap_scale())) return refuse(__LINE__);
             if (nd.res >= 0) {
-                if (where[nd.res] != 0) return refuse(22);
+                if (where[nd.res] != 0) return refuse(__LINE__);
                 vals[nd.res].need_f32 = true;
             }
             continue;
         }
-        if (!out.need_i8 && !out.need_f32 && !out.need_nchw) return refuse(23);  // nobody reads it
+        if (!out.need_i8 && !out.need_f32 && !out.need_nchw) return refuse(__LINE__);  // nobody reads it
         for (int v : nd.in)
-            if (where[v] != 0) return refuse(24);
+            if (where[v] != 0) return refuse(__LINE__);
         if (nd.kind == 'g') {
             nd.as_f32 = nd.bn >= 0 || nd.unary >= 0 || out.need_f32 || out.need_nchw;
             for (int v : nd.in)
                 if (vals[v].c % 32 != 0) nd.as_f32 = true;
             for (int v : nd.in) {
                 if (nd.as_f32) vals[v].need_f32 = true;
-                else if (!want_i8(v, out.fs)) return refuse(25);
+                else if (!want_i8(v, out.fs)) return refuse(__LINE__);
             }
         } else if (nd.kind == 'i') {
-            if (out.need_i8 && !want_i8(nd.in[0], out.fs)) return refuse(26);
+            if (out.need_i8 && !want_i8(nd.in[0], out.fs)) return refuse(__LINE__);
             if (out.need_f32 || out.need_nchw) vals[nd.in[0]].need_f32 = true;
         } else {
             // A pyramid of stride-1 "same" max pools over one tensor (windows 5 / 9 / 13): the maximum over a window of k is
@@ -1248,7 +1249,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     };
     {
         value_info& v = vals[front_value];
-        if (!v.need_i8 || v.need_f32 || v.need_nchw) return refuse(27);
+        if (!v.need_i8 || v.need_f32 || v.need_nchw) return refuse(__LINE__);
         v.n = front_shape[0]; v.c = front_shape[1]; v.h = front_shape[2]; v.w = front_shape[3];
         int kw_first = 0;
         for (int c : consumers[front_value]) kw_first = std::max(kw_first, static_cast<conv_t*>(operations_[c].get())->kernel_size_w_);
@@ -1314,11 +1315,11 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     for (const node& nd : nodes) {
         const value_info in = vals[nd.in[0]];
         value_info& out = vals[nd.out];
-        if (in.n == 0) return refuse(28);
+        if (in.n == 0) return refuse(__LINE__);
         if (nd.kind == 'c') {
             auto* c = static_cast<conv_t*>(operations_[nd.op].get());
             const int8_t* x = static_cast<const int8_t*>(in.int8_at(c->featmap_scale()));
-            if (in.c != c->input_channels() || !x) return refuse(29);
+            if (in.c != c->input_channels() || !x) return refuse(__LINE__);
             const int ks = pad_to(c->output_channel_, 32);
             exhip_conv_desc d = c->describe(in.n, in.h, in.w, in.cs, ks);
             d.post_relu = nd.post_relu ? 1 : 0;
@@ -1337,8 +1338,8 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                 // NHWC and one kernel regroups the channels of every pixel
                 auto* rs = static_cast<operation_reshape<float>*>(operations_[nd.head_reshape].get());
                 const std::vector<int> to = rs->new_shape({in.n, c->output_channel_, oh, ow}, in.n * c->output_channel_ * oh * ow);
-                if (to.size() != 4 || to[0] != in.n || to[1] * to[2] != c->output_channel_ || to[3] != oh * ow) return refuse(41);
-                if (out.need_i8 || out.need_f32 || !out.need_nchw || nd.res >= 0) return refuse(42);
+                if (to.size() != 4 || to[0] != in.n || to[1] * to[2] != c->output_channel_ || to[3] != oh * ow) return refuse(__LINE__);
+                if (out.need_i8 || out.need_f32 || !out.need_nchw || nd.res >= 0) return refuse(__LINE__);
                 const int groups = to[1], per_group = to[2], hw = oh * ow, n0 = in.n;
                 out.n = in.n; out.c = groups; out.h = hw; out.w = per_group; out.cs = 0;
                 float* mid = static_cast<float*>(alloc(elems * sizeof(float)));
@@ -1358,7 +1359,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             const float* res = nullptr;
             if (nd.res >= 0) {
                 const value_info& r = vals[nd.res];
-                if (!r.f32 || r.n != out.n || r.h != oh || r.w != ow || r.cs != ks || r.c != out.c) return refuse(30);
+                if (!r.f32 || r.n != out.n || r.h != oh || r.w != ow || r.cs != ks || r.c != out.c) return refuse(__LINE__);
                 res = static_cast<const float*>(r.f32);
             }
             const void* wp = c->pin_packed_weights(EXHIP_I8, d);  // the launch keeps this pointer
@@ -1374,9 +1375,9 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             std::vector<int> channels, strides;
             for (int v : nd.in) {
                 const value_info& s = vals[v];
-                if (s.n != in.n || s.h != in.h || s.w != in.w || s.c % 4 != 0) return refuse(31);
+                if (s.n != in.n || s.h != in.h || s.w != in.w || s.c % 4 != 0) return refuse(__LINE__);
                 const void* form = nd.as_f32 ? s.f32 : s.int8_at(out.fs);
-                if (!form || (!nd.as_f32 && (s.cs != s.c || s.c % 16 != 0))) return refuse(32);
+                if (!form || (!nd.as_f32 && (s.cs != s.c || s.c % 16 != 0))) return refuse(__LINE__);
                 ptrs.push_back(form);
                 channels.push_back(s.c);
                 strides.push_back(s.cs);
@@ -1392,7 +1393,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                 const float *bn_a = nullptr, *bn_b = nullptr;
                 if (nd.bn >= 0) {
                     auto* bn = static_cast<operation_batchnorm<float>*>(operations_[nd.bn].get());
-                    if (bn->channels_ != total || !bn->a_ || !bn->b_) return refuse(33);
+                    if (bn->channels_ != total || !bn->a_ || !bn->b_) return refuse(__LINE__);
                     bn_a = bn->a_->gpu_data();
                     bn_b = bn->b_->gpu_data();
                 }
@@ -1410,7 +1411,7 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                 });
                 nchw_from_f32(out, nd.out);
             } else {
-                if (out.cs != total) return refuse(34);
+                if (out.cs != total) return refuse(__LINE__);
                 std::vector<int> pairs;  // the byte tensors as tensors of two-byte elements
                 for (int ch : channels) pairs.push_back(ch / 2);
                 uint16_t* y = static_cast<uint16_t*>(out.i8);
@@ -1425,18 +1426,18 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                 oh = static_cast<int>(in.h * ip->height_scale_);
                 ow = static_cast<int>(in.w * ip->width_scale_);
             }
-            if (oh <= 0 || ow <= 0) return refuse(35);
+            if (oh <= 0 || ow <= 0) return refuse(__LINE__);
             out.n = in.n; out.c = in.c; out.h = oh; out.w = ow; out.cs = in.cs;
             const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
             if (out.need_i8) {
                 const uint16_t* x = static_cast<const uint16_t*>(in.int8_at(out.fs));
-                if (!x || in.cs % 16 != 0) return refuse(36);
+                if (!x || in.cs % 16 != 0) return refuse(__LINE__);
                 out.i8 = alloc(elems);
                 uint16_t* y = static_cast<uint16_t*>(out.i8);
                 plan->launches.push_back([=]() { EXHIP_FATAL(exhip_interp_nearest_nhwc_f16(ctx, x, y, in.n, in.cs / 2, in.h, in.w, oh, ow)); });
             }
             if (out.need_f32 || out.need_nchw) {
-                if (!in.f32 || in.cs % 4 != 0) return refuse(37);
+                if (!in.f32 || in.cs % 4 != 0) return refuse(__LINE__);
                 out.f32 = alloc(elems * sizeof(float));
                 const uint16_t* x = static_cast<const uint16_t*>(in.f32);
                 uint16_t* y = static_cast<uint16_t*>(out.f32);
@@ -1450,12 +1451,12 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             const void* source = in.f32;
             if (nd.cascade >= 0) {  // the smaller pool's result, pooled again (same size as the input: stride 1, "same" padding)
                 const value_info& q = vals[nd.cascade];
-                if (q.n != in.n || q.h != in.h || q.w != in.w || q.cs != in.cs || oh != in.h || ow != in.w) return refuse(40);
+                if (q.n != in.n || q.h != in.h || q.w != in.w || q.cs != in.cs || oh != in.h || ow != in.w) return refuse(__LINE__);
                 source = q.f32;
                 kh = kw = nd.cascade_k;
                 pt = pl = nd.cascade_k / 2;
             }
-            if (!source) return refuse(38);
+            if (!source) return refuse(__LINE__);
             out.n = in.n; out.c = in.c; out.h = oh; out.w = ow; out.cs = in.cs;
             const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
             if (out.need_i8) out.i8 = alloc(elems);
@@ -1469,13 +1470,13 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             });
             nchw_from_f32(out, nd.out);
         }
-        if (!more_forms(out)) return refuse(44);
+        if (!more_forms(out)) return refuse(__LINE__);
     }
     // the network's outputs: results of the plan by name (Split copies share their tensor), the rest comes from the tail
     for (const std::string& o : output_names_) {
         const int v = root(blob_index_[o]);
         if (where[v] == 2) continue;
-        if (where[v] != 0 || !vals[v].nchw) return refuse(39);
+        if (where[v] != 0 || !vals[v].nchw) return refuse(__LINE__);
         for (auto& r : plan->outputs)
             if (&r.slot == vals[v].nchw) r.name += (r.name.empty() ? "" : "\n") + o;
     }
