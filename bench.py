@@ -101,7 +101,7 @@ def measured_traffic(n, hw):
     return None
 
 
-def network_table(iters=10):
+def network_table(iters=10, only=None):
     """The generated topologies of the other configurations through pipeline<float> / pipeline<unsigned short> (float32 and
     fp16: layer by layer with the executor's joins; int8: the int8 graph plan where it takes the network, which the row's
     "executor" says), input resident on the device: wall time per forward over `iters` forwards, device drained before and
@@ -114,6 +114,8 @@ def network_table(iters=10):
     rows = []
 
     def run(label, net, x, dtype, pipe_dtype):
+        if only and only not in f"{label} {dtype}":   # --only: a substring of "<network label> <dtype>"
+            return
         with tempfile.NamedTemporaryFile(suffix=".racy", delete=False) as f:
             path = f.name
         net.write_model(path)
@@ -388,6 +390,8 @@ def main():
     ap.add_argument("--networks", action="store_true",
                     help="time the other configurations' whole topologies (MobileNet- and YOLOv5s-shaped, f32 / f16 / int8) "
                          "through the pipeline (per-layer executor; int8 graph plan) instead of the headline benchmark")
+    ap.add_argument("--only", default=None, metavar="TEXT",
+                    help="with --networks: only the rows whose '<network label> <dtype>' contains TEXT (e.g. 'yolov5s_simp topology (3 heads x 255 channels), 16x3x640x640 int8')")
     ap.add_argument("--bandwidth", action="store_true",
                     help="instead of the network: time the memory-bound kernels of the path and print their GB/s")
     args = ap.parse_args()
@@ -411,7 +415,7 @@ def main():
         return
     if args.networks:
         print(json.dumps({"metric": "forward time of the generated topologies through the pipeline (executor per row)",
-                          "networks": network_table()}))
+                          "networks": network_table(only=args.only)}))
         return
 
     import tempfile
