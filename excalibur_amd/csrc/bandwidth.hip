@@ -814,6 +814,41 @@ __global__ __launch_bounds__(kBlock) void maxpool_nhwc_f32_kernel(const float* _
     }
 }
 
+// The same pooling on an int8 NHWC tensor (the int8 executor: the quantizer is monotone, so the maximum of the quantized
+// values is the quantized maximum). 16 channels per thread; the running maxima stay unpacked over the window.
+__global__ __launch_bounds__(kBlock) void maxpool_nhwc_i8_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y, int H, int W, int cs,
+                                                                 int OH, int OW, int kh, int kw, int sh, int sw, int pt, int pl,
+                                                                 size_t total) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const int groups = cs / 16;
+    const int g = (int)(i % groups);
+    size_t pix = i / groups;
+    const int ox = (int)(pix % OW);
+    pix /= OW;
+    const int oy = (int)(pix % OH);
+    const size_t n = pix / OH;
+    const int hs = max(oy * sh - pt, 0), wsx = max(ox * sw - pl, 0);
+    const int he = min(oy * sh - pt + kh, H), we = min(ox * sw - pl + kw, W);
+    int m[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) m[e] = -128;
+    for (int a = hs; a < he; ++a)
+        for (int b = wsx; b < we; ++b) {
+            const v4i t = *reinterpret_cast<const v4i*>(x + ((n * H + a) * W + b) * cs + g * 16);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int v = (t[e >> 2] << (24 - 8 * (e & 3))) >> 24;  // byte e, sign-extended
+                m[e] = m[e] < v ? v : m[e];
+            }
+        }
+    v4i o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        o[q] = (m[4 * q] & 0xff) | ((m[4 * q + 1] & 0xff) << 8) | ((m[4 * q + 2] & 0xff) << 16) | (m[4 * q + 3] << 24);
+    *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 16) = o;
+}
+
 // 3x3 stride-2 max pooling on NHWC float32, a 2 x 2 block of output pixels per thread (four channels each): the four
 // windows share a row and a column, so 25 loads instead of 36, all in flight at once. Taps outside the image count as
 // -FLT_MAX, the clipped window of the general kernel. Optional requantized int8 copy as there.
@@ -2280,6 +2315,22 @@ extern "C" int exhip_maxpool2d_nhwc_f32(exhip_ctx* ctx, const float* x, float* y
     const size_t total = (size_t)n * oh * ow * (cs / 4);
     hipLaunchKernelGGL(maxpool_nhwc_f32_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, y_i8, fs_out, h, w,
                        cs, oh, ow, kh, kw, sh, sw, pt, pl, total);
+    EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_maxpool2d_nhwc_i8(exhip_ctx* ctx, const int8_t* x, int8_t* y, int n, int c, int h, int w, int cs, int oh, int ow,
+                                       int kh, int kw, int sh, int sw, int pt, int pl) {
+    REQ_CTX("exhip_maxpool2d_nhwc_i8");
+    EXHIP_REQUIRE(x && y && n > 0 && c > 0 && cs >= c && cs % 16 == 0 && h > 0 && w > 0 && oh > 0 && ow > 0 && kh > 0 && kw > 0 && sh > 0 && sw > 0 &&
+                      pt >= 0 && pl >= 0 && pt < kh && pl < kw,
+                  "exhip_maxpool2d_nhwc_i8: bad argument");
+    EXHIP_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0, "exhip_maxpool2d_nhwc_i8: tensors must be 16-byte aligned");
+    // every window holds at least one pixel of the image
+    EXHIP_REQUIRE((oh - 1) * sh - pt < h && (ow - 1) * sw - pl < w, "exhip_maxpool2d_nhwc_i8: output %dx%d does not fit input %dx%d", oh, ow, h, w);
+    const size_t total = (size_t)n * oh * ow * (cs / 16);
+    hipLaunchKernelGGL(maxpool_nhwc_i8_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, cs, oh, ow, kh, kw, sh, sw, pt, pl,
+                       total);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }

@@ -464,6 +464,14 @@ class Ctx:
         _check(lib().exhip_focus_f16(self.h, x.ptr, y.ptr, n, c, h, w))
         return y
 
+    def maxpool2d_nhwc_i8(self, x, c, kernel, stride, pad, oh, ow):
+        """MAX pooling on an int8 NHWC tensor [n, h, w, c_stride] (exhip_maxpool2d_nhwc_i8); pad = (top, left)."""
+        n, h, w, cs = x.shape
+        y = self.empty((n, oh, ow, cs), np.int8)
+        _check(lib().exhip_maxpool2d_nhwc_i8(self.h, x.ptr, y.ptr, n, int(c), h, w, cs, int(oh), int(ow), int(kernel), int(kernel), int(stride),
+                                             int(stride), int(pad[0]), int(pad[1])))
+        return y
+
     def input_focus_quantize(self, x, means, scales, fs, c_stride=32):
         """Input layer, YoloV5Focus and the int8 quantizer in one pass (exhip_input_focus_quantize_nchw_f32_to_nhwc_i8): float32
         NCHW -> int8 NHWC [n, h / 2, w / 2, c_stride]. Returns None where the library leaves the shape to the three layers."""

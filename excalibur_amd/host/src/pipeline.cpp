@@ -1224,8 +1224,11 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
                         nd.cascade_k = k - kq + 1;
                     }
                 }
-            if (nd.cascade >= 0) vals[nd.cascade].need_f32 = true;
-            else vals[nd.in[0]].need_f32 = true;
+            // read by int8 convolutions only (at one scale): the pool runs on the int8 tensor, the quantizer being monotone
+            nd.as_f32 = out.need_f32 || out.need_nchw || !out.need_i8 || !out.more_i8.empty();
+            const int source = nd.cascade >= 0 ? nd.cascade : nd.in[0];
+            if (nd.as_f32) vals[source].need_f32 = true;
+            else if (!want_i8(source, out.fs)) return refuse(__LINE__);
         }
     }
 
@@ -1448,11 +1451,11 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             auto* p = static_cast<operation_pooling<float>*>(operations_[nd.op].get());
             int kh, kw, sh, sw, pt, pb, pl, pr, oh, ow;
             p->geometry(in.h, in.w, &kh, &kw, &sh, &sw, &pt, &pb, &pl, &pr, &oh, &ow);
-            const void* source = in.f32;
+            const void* source = nd.as_f32 ? in.f32 : in.int8_at(out.fs);
             if (nd.cascade >= 0) {  // the smaller pool's result, pooled again (same size as the input: stride 1, "same" padding)
                 const value_info& q = vals[nd.cascade];
                 if (q.n != in.n || q.h != in.h || q.w != in.w || q.cs != in.cs || oh != in.h || ow != in.w) return refuse(__LINE__);
-                source = q.f32;
+                source = nd.as_f32 ? q.f32 : q.int8_at(out.fs);
                 kh = kw = nd.cascade_k;
                 pt = pl = nd.cascade_k / 2;
             }
@@ -1461,14 +1464,21 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             const size_t elems = static_cast<size_t>(out.n) * oh * ow * out.cs;
             if (out.need_i8) out.i8 = alloc(elems);
             if (out.need_f32 || out.need_nchw) out.f32 = alloc(elems * sizeof(float));
-            const float* x = static_cast<const float*>(source);
-            float* yf = static_cast<float*>(out.f32);
             int8_t* yq = static_cast<int8_t*>(out.i8);
-            const float fs = out.fs;
-            plan->launches.push_back([=]() {
-                EXHIP_FATAL(exhip_maxpool2d_nhwc_f32(ctx, x, yf, yq, fs, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl));
-            });
-            nchw_from_f32(out, nd.out);
+            if (!nd.as_f32) {
+                if (in.cs % 16 != 0 || pt >= kh || pl >= kw) return refuse(__LINE__);
+                const int8_t* xq = static_cast<const int8_t*>(source);
+                plan->launches.push_back(
+                    [=]() { EXHIP_FATAL(exhip_maxpool2d_nhwc_i8(ctx, xq, yq, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl)); });
+            } else {
+                const float* x = static_cast<const float*>(source);
+                float* yf = static_cast<float*>(out.f32);
+                const float fs = out.fs;
+                plan->launches.push_back([=]() {
+                    EXHIP_FATAL(exhip_maxpool2d_nhwc_f32(ctx, x, yf, yq, fs, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl));
+                });
+                nchw_from_f32(out, nd.out);
+            }
         }
         if (!more_forms(out)) return refuse(__LINE__);
     }

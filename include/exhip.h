@@ -233,6 +233,10 @@ int exhip_pool2d_nchw_f32(exhip_ctx* ctx, const float* x, float* y, int n, int c
 int exhip_maxpool2d_nhwc_f32(exhip_ctx* ctx, const float* x, float* y, int8_t* y_i8, float fs_out, int n, int c,
                              int h, int w, int c_stride, int oh, int ow, int kh, int kw, int sh, int sw, int pt,
                              int pl);
+/* The same MAX pooling (operation_pooling.cpp:145-159) on an int8 NHWC tensor, c_stride a multiple of 16: what the layer's
+ * float result would quantize to, since max commutes with the monotone quantizer (taps outside the image do not count). */
+int exhip_maxpool2d_nhwc_i8(exhip_ctx* ctx, const int8_t* x, int8_t* y, int n, int c, int h, int w, int c_stride, int oh, int ow,
+                            int kh, int kw, int sh, int sw, int pt, int pl);
 int exhip_pool2d_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int c_stride,
                           int oh, int ow, int type, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr,
                           int count_include_pad);

@@ -810,3 +810,24 @@ def test_detection_head_regrouping(ctx, n, h, w, groups, per_group, stride):
     got = ctx.nhwc_to_grouped_f32(ctx.array(nhwc), k, groups).download()
     assert got.shape == want.shape
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("kernel,stride,pad,h,w", [(2, 2, 0, 12, 14), (3, 2, 1, 13, 9), (5, 1, 2, 10, 10), (13, 1, 6, 8, 7), (2, 2, 0, 7, 9)], ids=str)
+def test_max_pooling_on_int8_nhwc(ctx, kernel, stride, pad, h, w):
+    """MAX pooling on an int8 NHWC tensor against the oracle's pooling of the same values as floats (the quantizer is
+    monotone: pooling the quantized tensor gives the quantized pooled tensor); clipped windows, ragged sizes, pad channels
+    carried along."""
+    r = np.random.default_rng(397)
+    n, c, cs = 2, 24, 32
+    x = r.integers(-128, 128, (n, h, w, cs)).astype(np.int8)
+    want = port.pool2d(np.ascontiguousarray(x[..., :c].transpose(0, 3, 1, 2)).astype(np.float32), port.POOL_MAX, kernel, stride, pad)
+    oh, ow = want.shape[2:]
+    got = ctx.maxpool2d_nhwc_i8(ctx.array(x), c, kernel, stride, (pad, pad), oh, ow).download()
+    assert np.array_equal(got[..., :c].astype(np.float32), want.transpose(0, 2, 3, 1))
+    # and through the quantizer: q8(max(v) * fs) == max(q8(v * fs))
+    v = r.normal(0, 3, (n, c, h, w)).astype(np.float32)
+    fs = np.float32(21.0)
+    q = np.zeros((n, h, w, cs), np.int8)
+    q[..., :c] = port.quantize(v, fs).transpose(0, 2, 3, 1)
+    got = ctx.maxpool2d_nhwc_i8(ctx.array(q), c, kernel, stride, (pad, pad), oh, ow).download()
+    assert np.array_equal(got[..., :c], port.quantize(port.pool2d(v, port.POOL_MAX, kernel, stride, pad), fs).transpose(0, 2, 3, 1))
