@@ -877,6 +877,9 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
         const bool has_nchw = p.y_nchw != nullptr;
         const __amdgpu_buffer_rsrc_t rn = __builtin_amdgcn_make_buffer_rsrc(p.y_nchw, 0, (int)(bytes_q * 4u), kRsrcWord3);
         const int nt_run = chb < p.K ? NT : 0;  // a wave whose slab lies past the last channel has nothing to write
+        // K a multiple of 32 only: the last slab holds 32 channels. Its rows in the tiles keep the 64-channel layout; the
+        // pieces of a row past the last channel are not stored (they would land in the next pixel's row).
+        const int live_ch = p.K - chb;
         const float act_floor = p.act == 1 ? 0.f : -__builtin_inff(), post_floor = p.post_relu ? 0.f : -__builtin_inff();
         const bool q_only = p.q_nonneg && has_q && !has_res && !has_f && !has_nchw;
 #pragma unroll
@@ -906,6 +909,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
             if (nn == 0) stamp(6);
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
+                if (m * 32 >= live_ch) continue;  // wave-uniform: the slab's second block has no channel
                 const int ch0 = chb + m * 32 + hh * 16;
                 char* const tf = tile_f + px_l * kEpiRowF + (m * 32 + hh * 16) * 4;
                 v4i q4;
@@ -988,7 +992,8 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 for (int it = 0; it < 8; ++it) {
                     const int idx = it * 64 + lane, tp = idx >> 4, part = idx & 15;
                     __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const v4i*>(tile_f + tp * kEpiRowF + part * 16), rf,
-                                                           (int)((table[tp] + part * 4) * 4u), 0, EXHIP_F32_STORE_AUX);
+                                                           (int)(((part * 4 < live_ch ? table[tp] : kEpiInvalid) + part * 4) * 4u), 0,
+                                                           EXHIP_F32_STORE_AUX);
                 }
             }
             if (has_q) {
@@ -996,7 +1001,7 @@ __global__ __launch_bounds__(64 * WM * WN, (MT * NT > 4 ? 1 : (LOWREG ? 4 : 2)))
                 for (int it = 0; it < 2; ++it) {
                     const int idx = it * 64 + lane, tp = idx >> 2, part = idx & 3;
                     __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const v4i*>(tile_q + tp * kEpiRowQ + part * 16), rq,
-                                                           (int)(table[tp] + part * 16), 0, 0);
+                                                           (int)((part * 16 < live_ch ? table[tp] : kEpiInvalid) + part * 16), 0, 0);
                 }
             }
             wave_sync();  // the tiles and the table are rewritten by the next column block
@@ -1618,10 +1623,10 @@ void rebuffer(Plan& pl, const exhip_conv_desc* d, int epi_wave_b, bool fused_3x3
     }
 }
 
-// The fused int8 epilogue takes: int8 / float32 NHWC tensors (and the NCHW float32 one), whole 64-channel slabs, plain or
+// The fused int8 epilogue takes: int8 / float32 NHWC tensors (and the NCHW float32 one), whole 32-channel blocks, plain or
 // ReLU activation, the activation layers of the general epilogue other than PReLU, the shortcut on either side of them.
 inline bool fused_epilogue_ok(const exhip_conv_desc* d, const ConvParams& p, long long out_elems) {
-    return !p.acc_nchw && d->post_op != EXHIP_POST_PRELU && d->k % 64 == 0 && d->k_stride == d->k && d->act <= 1 && out_elems * 4 < 0xFFFFF000ll &&
+    return !p.acc_nchw && d->post_op != EXHIP_POST_PRELU && d->k % 32 == 0 && d->k_stride == d->k && d->act <= 1 && out_elems * 4 < 0xFFFFF000ll &&
            out_elems < (long long)kEpiInvalid;
 }
 

@@ -744,13 +744,14 @@ _POST_LAYERS = {
 
 @pytest.mark.parametrize("shortcut", ["none", "front", "behind"])
 @pytest.mark.parametrize("post_op", list(_POST_LAYERS))
-@pytest.mark.parametrize("c,k,kernel", [(32, 64, 3), (32, 128, 1), (32, 48, 3), (64, 64, 3), (128, 128, 3)],
-                         ids=["k64-3x3", "k128-1x1", "k48-3x3", "c64-k64-3x3", "c128-k128-3x3"])
+@pytest.mark.parametrize("c,k,kernel", [(32, 64, 3), (32, 128, 1), (32, 48, 3), (64, 64, 3), (128, 128, 3), (32, 32, 3), (64, 96, 3), (16, 160, 3)],
+                         ids=["k64-3x3", "k128-1x1", "k48-3x3", "c64-k64-3x3", "c128-k128-3x3", "k32-3x3", "k96-3x3", "k160-3x3"])
 def test_conv_int8_activation_layer_and_sum_in_the_epilogue(ctx, c, k, kernel, post_op, shortcut):
     """int8 convolution -> activation layer [-> sum], or -> sum -> activation layer, in one launch against the oracle's
-    layers one after the other: float32 NHWC / NCHW results and the requantized int8 copy, bit for bit. 64 / 128 output
-    channels take the epilogue with the per-wave tiles, 48 the general one; with 64 / 128 input channels and without the
-    NCHW result the 3x3 layers run in the lean kernel (checked in a second launch)."""
+    layers one after the other: float32 NHWC / NCHW results and the requantized int8 copy, bit for bit. Output channel
+    counts that are multiples of 32 take the epilogue with the per-wave tiles (32, 96 and 160: the last 64-channel slab is
+    half empty), 48 the general one; with 64 / 128 input channels and without the NCHW result the 3x3 layers run in the lean
+    kernel (checked in a second launch)."""
     case = cases.conv_i8_case(640 + k + c, 2, c, 11, 13, k, kernel, 1, kernel // 2, act=0)
     y = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], 0, cases.geom_of(case))
     res = np.random.default_rng(641).uniform(-2, 2, y.shape).astype(np.float32)
