@@ -600,14 +600,15 @@ __global__ __launch_bounds__(kThreads, (WRES || NAB == 2 || NWB == 3 || PROJ) ? 
                     }
                     if constexpr (EPI < 0) {
                         if (p.post_op) {
+                            auto apply = [&](auto op) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                switch (p.post_op - 1) {
-                                case EXHIP_UNARY_HARDSWISH: v[e] = unary_value<0>(v[e], p.post_alpha, p.post_beta); break;
-                                case EXHIP_UNARY_LEAKYRELU: v[e] = unary_value<1>(v[e], p.post_alpha, p.post_beta); break;
-                                case EXHIP_UNARY_HARDSIGMOID: v[e] = unary_value<3>(v[e], p.post_alpha, p.post_beta); break;
-                                default: v[e] = unary_value<4>(v[e], p.post_alpha, p.post_beta); break;
-                                }
+                                for (int e = 0; e < 4; ++e) v[e] = unary_value<decltype(op)::value>(v[e], p.post_alpha, p.post_beta);
+                            };
+                            switch (p.post_op - 1) {  // one switch per vector, not per value
+                            case EXHIP_UNARY_HARDSWISH: apply(std::integral_constant<int, 0>{}); break;
+                            case EXHIP_UNARY_LEAKYRELU: apply(std::integral_constant<int, 1>{}); break;
+                            case EXHIP_UNARY_HARDSIGMOID: apply(std::integral_constant<int, 3>{}); break;
+                            default: apply(std::integral_constant<int, 4>{}); break;
                             }
                         }
                         if (has_res && res_last) {

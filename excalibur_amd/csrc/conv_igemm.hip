@@ -243,15 +243,18 @@ __device__ __forceinline__ void post_activation(float (&v)[16], int op, float al
 }
 
 // The same on four float32 values (the fused int8 epilogue works on vectors of four channels).
-__device__ __forceinline__ void post_activation4(v4f& v, int op, float alpha, float beta) {
+template <int OP>
+__device__ __forceinline__ void post_activation4_op(v4f& v, float alpha, float beta) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        switch (op) {
-        case EXHIP_UNARY_HARDSWISH: v[e] = unary_value<0>(v[e], alpha, beta); break;
-        case EXHIP_UNARY_LEAKYRELU: v[e] = unary_value<1>(v[e], alpha, beta); break;
-        case EXHIP_UNARY_HARDSIGMOID: v[e] = unary_value<3>(v[e], alpha, beta); break;
-        default: v[e] = unary_value<4>(v[e], alpha, beta); break;
-        }
+    for (int e = 0; e < 4; ++e) v[e] = unary_value<OP>(v[e], alpha, beta);
+}
+// one switch per vector: a switch per value is a chain of wave-uniform branches around every operation
+__device__ __forceinline__ void post_activation4(v4f& v, int op, float alpha, float beta) {
+    switch (op) {
+    case EXHIP_UNARY_HARDSWISH: post_activation4_op<0>(v, alpha, beta); break;
+    case EXHIP_UNARY_LEAKYRELU: post_activation4_op<1>(v, alpha, beta); break;
+    case EXHIP_UNARY_HARDSIGMOID: post_activation4_op<3>(v, alpha, beta); break;
+    default: post_activation4_op<4>(v, alpha, beta); break;
     }
 }
 
@@ -1633,6 +1636,8 @@ inline bool fused_epilogue_ok(const exhip_conv_desc* d, const ConvParams& p, lon
 template <int DT>
 int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolSpec* pool = nullptr, const exhip_lean_proj* proj = nullptr) {
     EXHIP_REQUIRE(ctx, "conv: NULL ctx");
+    // a BatchNorm in the epilogue and writes limited to the layer's own channels: int8 pointwise layers only (below)
+    if ((d->post_bn_a || d->post_bn_b || d->exact_k) && (DT != EXHIP_I8 || pool || proj)) return EXHIP_ERR_UNSUPPORTED;
     Plan pl;
     int rc = make_plan(d, DT, &pl, pool);
     if (rc) return rc;
@@ -1746,10 +1751,12 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             g.act = d->act; g.post_relu = d->post_relu; g.post_op = d->post_op; g.post_slope_shared = d->post_slope_shared;
             g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope; g.residual_last = d->residual_last;
             g.fs_out = d->fs_out;
+            g.post_bn_a = d->post_bn_a; g.post_bn_b = d->post_bn_b; g.exact_k = d->exact_k;
             rc = exhip_conv1x1_i8_pw(ctx, g, reinterpret_cast<const int8_t*>(p.x), p.wp, p.scale, p.bias, reinterpret_cast<const float*>(p.residual),
                                      reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc));
             if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
         }
+        if (d->post_bn_a || d->post_bn_b || d->exact_k) return EXHIP_ERR_UNSUPPORTED;  // only the pointwise kernel has these
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = fused_epilogue_ok(d, p, out_elems);

@@ -14,6 +14,12 @@ struct exhip_pw_geom {
     float post_alpha, post_beta;
     const float* post_slope;
     float fs_out;               // int8 layers: the scale of the requantized int8 result
+    // int8 layers: a BatchNorm layer in front of post_op (device arrays of k floats, both or neither), and whether only
+    // channels [0, k) are written (the results point into a wider tensor; k a multiple of 32). Either makes the kernel
+    // take the layer whatever its size.
+    const float* post_bn_a;
+    const float* post_bn_b;
+    int exact_k;
 };
 
 // Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then

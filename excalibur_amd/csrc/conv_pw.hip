@@ -49,6 +49,9 @@ struct PwParams {
     float* y_f;
     int8_t* y_q;
     float fs_out;
+    const float* post_bn_a;   // BatchNorm in front of post_op: fmaf(post_bn_b[ch], v, post_bn_a[ch])
+    const float* post_bn_b;
+    int exact;                // channels [0, K) only: blocks past K are not written (the results lie inside a wider tensor)
     unsigned pixels, x_bytes, w_bytes;
     unsigned items, ch_groups;   // waves with work; 32 * MT channel groups per pixel tile
     int xs_b;                    // bytes per input pixel
@@ -189,7 +192,7 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int ch0 = (kb0 + m) * 32 + (lane >> 5) * 16;
-        if (ch0 >= p.kstride && ch0 >= p.K) continue;
+        if (ch0 >= p.K && (p.exact || ch0 >= p.kstride)) continue;
         float sc[16], bi[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
@@ -197,6 +200,12 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
             bi[e] = (p.bias && ch0 + e < p.K) ? p.bias[ch0 + e] : 0.f;
         }
         const bool vec_ok = ch0 + 16 <= p.kstride;
+        float bna[16], bnb[16];  // the BatchNorm's parameters of these channels (identity beyond K)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            bna[e] = (p.post_bn_a && ch0 + e < p.K) ? p.post_bn_a[ch0 + e] : 0.f;
+            bnb[e] = (p.post_bn_a && ch0 + e < p.K) ? p.post_bn_b[ch0 + e] : 1.f;
+        }
 #pragma unroll
         for (int n = 0; n < NT; ++n) {
             const bool valid = pix[n] < p.pixels;
@@ -237,6 +246,10 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
 #pragma unroll
                 for (int e = 0; e < 16; ++e) v[e] = (0.f > v[e]) ? 0.f : v[e];
             }
+            if (p.post_bn_a) {  // the BatchNorm layer between this layer (through a Concat) and its activation layer
+#pragma unroll
+                for (int e = 0; e < 16; ++e) v[e] = __builtin_fmaf(bnb[e], v[e], bna[e]);
+            }
             if (p.post_op == EXHIP_POST_PRELU) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
@@ -244,14 +257,15 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
                     v[e] = v[e] >= 0.f ? v[e] : slope * v[e];
                 }
             } else if (p.post_op) {
+                auto apply = [&](auto op) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    switch (p.post_op - 1) {
-                    case EXHIP_UNARY_HARDSWISH: v[e] = unary_value<0>(v[e], p.post_alpha, p.post_beta); break;
-                    case EXHIP_UNARY_LEAKYRELU: v[e] = unary_value<1>(v[e], p.post_alpha, p.post_beta); break;
-                    case EXHIP_UNARY_HARDSIGMOID: v[e] = unary_value<3>(v[e], p.post_alpha, p.post_beta); break;
-                    default: v[e] = unary_value<4>(v[e], p.post_alpha, p.post_beta); break;
-                    }
+                    for (int e = 0; e < 16; ++e) v[e] = unary_value<decltype(op)::value>(v[e], p.post_alpha, p.post_beta);
+                };
+                switch (p.post_op - 1) {
+                case EXHIP_UNARY_HARDSWISH: apply(std::integral_constant<int, 0>{}); break;
+                case EXHIP_UNARY_LEAKYRELU: apply(std::integral_constant<int, 1>{}); break;
+                case EXHIP_UNARY_HARDSIGMOID: apply(std::integral_constant<int, 3>{}); break;
+                default: apply(std::integral_constant<int, 4>{}); break;
                 }
             }
             if (p.residual_f && p.residual_last) {
@@ -438,9 +452,12 @@ int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has
     // 64-byte store runs against the general epilogue's 16-byte pieces: 41 against 60 us on a 128 -> 255 head at
     // 16 x 80 x 80). Beyond that the general kernel's staged tiles re-read less and win (128 -> 128 at 80 x 80).
     // Option pw = 2 takes every layer the kernel can (tests), 0 none.
-    const int blocks_needed = (std::max(g.k, g.k_stride) + 31) / 32;
+    const bool joined = g.post_bn_a || g.exact_k;  // only this kernel has those: it takes the layer whatever its size
+    if (joined && (DT != EXHIP_I8 || (g.post_bn_a == nullptr) != (g.post_bn_b == nullptr) || (g.exact_k && g.k % 32 != 0))) return EXHIP_ERR_UNSUPPORTED;
+    const int out_channels = g.exact_k ? g.k : std::max(g.k, g.k_stride);  // channels this launch writes
+    const int blocks_needed = (out_channels + 31) / 32;
     const double flop = 2.0 * (double)g.pixels * (g.c_bytes / es) * g.k;
-    bool take = blocks_needed == 1 || (flop <= 8.0e9 && g.pixels <= 32768);
+    bool take = joined || blocks_needed == 1 || (flop <= 8.0e9 && g.pixels <= 32768);
     if (DT == EXHIP_I8 && g.pixels <= 131072 && (g.c_bytes <= 64 || (p.y_f && !p.y_q))) take = true;
     if (DT == EXHIP_F16 && ((g.c_bytes <= 128 && g.pixels <= 524288) || (g.c_bytes <= 256 && g.k <= 64 && g.pixels <= 131072))) take = true;
     if (g_exhip_options.pw != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
@@ -461,7 +478,8 @@ int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has
     p.residual_last = g.residual_last && has_residual;
     p.post_alpha = g.post_alpha; p.post_beta = g.post_beta;
     // every packed block that holds a channel below max(k, k_stride): pad channels of the output are written as zeros
-    const int kblocks = std::min(g.slabs * g.slab_blocks, (std::max(g.k, g.k_stride) + 31) / 32);
+    // (exact_k: only the blocks of the k channels themselves)
+    const int kblocks = std::min(g.slabs * g.slab_blocks, (out_channels + 31) / 32);
     // 64 x 64 per wave unless that leaves SIMDs without a wave: then 64 channels x 32 pixels; a lone 32-channel block
     // takes 128 pixels per wave
     if (kblocks == 1) return launch<DT, 1, 4>(ctx, p, kblocks);
@@ -485,5 +503,6 @@ int exhip_conv1x1_i8_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const int8_t* x,
     PwParams p = {};
     p.x = reinterpret_cast<const char*>(x); p.wp = reinterpret_cast<const char*>(wp); p.bias = bias; p.scale = scale;
     p.residual_f = residual; p.y_f = y_f32; p.y_q = y_i8; p.fs_out = g.fs_out;
+    p.post_bn_a = g.post_bn_a; p.post_bn_b = g.post_bn_b; p.exact = g.exact_k;
     return run_pw<EXHIP_I8>(ctx, g, p, 1, residual != nullptr);
 }

@@ -346,7 +346,7 @@ extern "C" int exhip_stem_f32_conv_i8_maxpool3x3s2(exhip_ctx* ctx, const exhip_c
     EXHIP_REQUIRE(y_i8 || y_f32_nhwc, "exhip_stem_f32_conv_i8_maxpool3x3s2: no output requested");
     if (!g_exhip_options.stem || !scales_nonnegative) return EXHIP_ERR_UNSUPPORTED;
     if (d->c < 3 || d->c > 4 || d->c_stride != 4 || d->kw > 8 || d->sh != 2 || d->sw != 2 || d->k % 64 != 0 || d->k_stride != d->k ||
-        d->act > 1 || d->post_relu || d->post_op || pool_pt < 0 || pool_pt > 1 || pool_pl < 0 || pool_pl > 1 ||
+        d->act > 1 || d->post_relu || d->post_op || d->post_bn_a || d->post_bn_b || d->exact_k || pool_pt < 0 || pool_pt > 1 || pool_pl < 0 || pool_pl > 1 ||
         !(d->kh == 7 || d->kh == 5 || d->kh == 3))
         return EXHIP_ERR_UNSUPPORTED;
     int oh = 0, ow = 0;

@@ -24,7 +24,8 @@ class ConvDesc(ctypes.Structure):
                 ("n", "c", "h", "w", "k", "kh", "kw", "sh", "sw", "pt", "pb", "pl", "pr", "act", "c_stride", "k_stride",
                  "post_relu")] + [("fs_out", ctypes.c_float), ("post_op", ctypes.c_int), ("post_alpha", ctypes.c_float),
                                   ("post_beta", ctypes.c_float), ("post_slope", ctypes.c_void_p),
-                                  ("post_slope_shared", ctypes.c_int), ("residual_last", ctypes.c_int)]
+                                  ("post_slope_shared", ctypes.c_int), ("residual_last", ctypes.c_int),
+                                  ("post_bn_a", ctypes.c_void_p), ("post_bn_b", ctypes.c_void_p), ("exact_k", ctypes.c_int)]
 
 
 _lib = None
@@ -93,6 +94,16 @@ class DevArray:
         if self.ptr:
             _check(lib().exhip_free(self.ctx.h, self.ptr))
             self.ptr = None
+
+    def at(self, offset_bytes):
+        """Something with a .ptr that many bytes into the allocation (an operand that starts inside a larger tensor)."""
+        assert 0 <= offset_bytes < self.nbytes
+        return _Inside(ctypes.c_void_p(self.ptr.value + int(offset_bytes)))
+
+
+class _Inside:
+    def __init__(self, ptr):
+        self.ptr = ptr
 
 
 class Event:
@@ -190,13 +201,14 @@ class Ctx:
     # ---- convolution ----
     @staticmethod
     def conv_desc(n, c, h, w, k, kernel, stride=1, pad=0, act=0, c_stride=None, k_stride=None, post_relu=0, fs_out=0.0,
-                  post_op=None, post_alpha=0.0, post_beta=0.0, residual_last=0):
+                  post_op=None, post_alpha=0.0, post_beta=0.0, residual_last=0, post_bn=None, exact_k=0):
         kh, kw = (kernel, kernel) if np.isscalar(kernel) else kernel
         sh, sw = (stride, stride) if np.isscalar(stride) else stride
         pt, pb, pl, pr = (pad,) * 4 if np.isscalar(pad) else pad
         return ConvDesc(n, c, h, w, k, kh, kw, sh, sw, pt, pb, pl, pr, act, c_stride if c_stride else c,
                         k_stride if k_stride else k, post_relu, fs_out, 0 if post_op is None else 1 + Ctx.UNARY[post_op],
-                        post_alpha, post_beta, None, 0, residual_last)
+                        post_alpha, post_beta, None, 0, residual_last, post_bn[0].ptr if post_bn else None,
+                        post_bn[1].ptr if post_bn else None, int(exact_k))
 
     @staticmethod
     def conv_out_hw(d):

@@ -1029,6 +1029,12 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         bool post_relu = false, residual_last = false, as_f32 = true;
         int cascade = -1, cascade_k = 0;  // max pool: the value of a smaller pool of the same input to pool again, and with which window
         int head_reshape = -1;            // convolution: the Reshape layer of a detection head (Reshape -> Transpose) it absorbs
+        // A Concat [-> BatchNorm] [-> activation] whose inputs are plain 1x1 convolutions read by nothing else and whose result
+        // only int8 convolutions read: each producer applies its channels' BatchNorm and the activation in its own
+        // epilogue and writes its int8 slice of the joined tensor (`joined`; the producers carry `into` = the Concat's
+        // node and their first channel there), so the join costs no launch and no float32 tensor.
+        bool joined = false;
+        int into = -1, into_offset = 0;
     };
     std::vector<node> nodes;
     std::vector<char> absorbed(n_ops, 0);
@@ -1174,6 +1180,8 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         else c = vals[nd.in[0]].c;
         vals[nd.out].c = c;
     }
+    std::vector<int> node_of(n_blobs, -1);  // the node that produces a value
+    for (size_t i = 0; i < nodes.size(); ++i) node_of[nodes[i].out] = static_cast<int>(i);
     for (auto it = nodes.rbegin(); it != nodes.rend(); ++it) {
         node& nd = *it;
         const value_info out = vals[nd.out];
@@ -1191,6 +1199,31 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
         for (int v : nd.in)
             if (where[v] != 0) return refuse(__LINE__);
         if (nd.kind == 'g') {
+            if (kind[nd.op] == 'k' && out.need_i8 && !out.need_f32 && !out.need_nchw && out.more_i8.empty() && vals[nd.out].c % 32 == 0) {
+                bool ok = true;
+                for (int v : nd.in) {
+                    const int pn = node_of[v];
+                    ok = ok && pn >= 0 && !is_output[v] && consumers[v].size() == 1 && vals[v].c % 32 == 0;
+                    if (!ok) break;
+                    const node& pr = nodes[pn];
+                    auto* c = pr.kind == 'c' ? static_cast<conv_t*>(operations_[pr.op].get()) : nullptr;
+                    ok = c && pr.unary < 0 && !pr.post_relu && pr.res < 0 && pr.head_reshape < 0 && pr.into < 0 && c->kernel_size_h_ == 1 &&
+                         c->kernel_size_w_ == 1 && c->stride_h_ == 1 && c->stride_w_ == 1 && c->pad_top_ == 0 && c->pad_bottom_ == 0 &&
+                         c->pad_left_ == 0 && c->pad_right_ == 0;
+                }
+                if (nd.unary >= 0 && static_cast<operation_unary<float>*>(operations_[nd.unary].get())->op_ == EXHIP_UNARY_SIGMOID) ok = false;
+                if (ok) {
+                    nd.joined = true;
+                    int offset = 0;
+                    const int self = static_cast<int>(&nd - nodes.data());
+                    for (int v : nd.in) {
+                        nodes[node_of[v]].into = self;
+                        nodes[node_of[v]].into_offset = offset;
+                        offset += vals[v].c;
+                    }
+                    continue;
+                }
+            }
             nd.as_f32 = nd.bn >= 0 || nd.unary >= 0 || out.need_f32 || out.need_nchw;
             for (int v : nd.in)
                 if (vals[v].c % 32 != 0) nd.as_f32 = true;
@@ -1336,6 +1369,41 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             EXHIP_FATAL(exhip_conv_out_hw(&d, &oh, &ow));
             out.n = in.n; out.c = c->output_channel_; out.h = oh; out.w = ow; out.cs = ks;
             const size_t elems = static_cast<size_t>(out.n) * oh * ow * ks;
+            if (nd.into >= 0) {
+                // a producer of a joined Concat: BatchNorm and activation of its channels in its own epilogue, its int8 slice
+                // written into the joined tensor
+                const node& jn = nodes[nd.into];
+                value_info& jo = vals[jn.out];
+                const int total = jo.c;
+                if (!jo.i8) {
+                    jo.n = in.n; jo.h = oh; jo.w = ow; jo.cs = total;
+                    jo.i8 = alloc(static_cast<size_t>(in.n) * oh * ow * total);
+                } else if (jo.n != in.n || jo.h != oh || jo.w != ow) {
+                    return refuse(__LINE__);
+                }
+                d.k_stride = total;
+                d.exact_k = 1;
+                d.fs_out = jo.fs;
+                if (jn.bn >= 0) {
+                    auto* bn = static_cast<operation_batchnorm<float>*>(operations_[jn.bn].get());
+                    if (bn->channels_ != total || !bn->a_ || !bn->b_) return refuse(__LINE__);
+                    d.post_bn_a = bn->a_->gpu_data() + nd.into_offset;
+                    d.post_bn_b = bn->b_->gpu_data() + nd.into_offset;
+                }
+                if (jn.unary >= 0) {
+                    auto* u = static_cast<operation_unary<float>*>(operations_[jn.unary].get());
+                    d.post_op = 1 + u->op_; d.post_alpha = u->alpha_; d.post_beta = u->beta_;
+                }
+                const void* wp = c->pin_packed_weights(EXHIP_I8, d);
+                plan->pinned.emplace_back([c, wp]() { c->unpin_packed_weights(wp); });
+                const float *scale = c->scale_gpu(), *bias = c->bias_gpu();
+                int8_t* yq = static_cast<int8_t*>(jo.i8) + nd.into_offset;
+                const int rc = exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, nullptr, yq, nullptr, nullptr, nullptr);  // trial launch
+                if (rc == EXHIP_ERR_UNSUPPORTED) return refuse(__LINE__);
+                EXHIP_FATAL(rc);
+                plan->launches.push_back([=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, nullptr, yq, nullptr, nullptr, nullptr)); });
+                continue;
+            }
             if (nd.head_reshape >= 0) {
                 // [n, K, oh, ow] -> Reshape [n, G, J, oh * ow] -> Transpose [n, G, oh * ow, J]: the convolution writes float32
                 // NHWC and one kernel regroups the channels of every pixel
@@ -1372,6 +1440,9 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             float* yf = static_cast<float*>(out.f32);
             plan->launches.push_back(
                 [=]() { EXHIP_FATAL(exhip_conv2d_i8(ctx, &d, x, wp, scale, bias, res, yq, yf, nchw ? *nchw : nullptr, nullptr)); });
+        } else if (nd.kind == 'g' && nd.joined) {
+            if (!out.i8 || out.n != in.n || out.h != in.h || out.w != in.w) return refuse(__LINE__);  // its producers wrote it
+            continue;
         } else if (nd.kind == 'g') {
             int total = 0;
             std::vector<const void*> ptrs;

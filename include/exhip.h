@@ -118,6 +118,15 @@ typedef struct exhip_conv_desc {
     int post_slope_shared;
     int residual_last;          /* 1: the shortcut is added behind post_relu / post_op instead of in front of them (a sum
                                  * layer behind the activation layer that follows the convolution) */
+    /* exhip_conv2d_i8, 1x1 stride-1 layers with NHWC results only: the BatchNorm layer (operation_batchnorm.cpp:122-156)
+     * that follows the layer through a Concat, applied in front of post_op: v = fmaf(post_bn_b[k], v, post_bn_a[k]) with
+     * device arrays of k floats (the layer's a / b for this convolution's channels); both NULL = none */
+    const float* post_bn_a;
+    const float* post_bn_b;
+    int exact_k;                /* the same layers: 1 = write channels [0, k) only (k a multiple of 32), no zeros into the
+                                 * pad channels up to k_stride: the outputs point into a wider tensor that other layers
+                                 * fill beside this one (a Concat's buffer). EXHIP_ERR_UNSUPPORTED where the kernel that
+                                 * has these two features cannot take the layer */
 } exhip_conv_desc;
 #define EXHIP_POST_PRELU 16
 

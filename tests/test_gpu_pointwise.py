@@ -178,3 +178,65 @@ def test_int8_pointwise_kernel_equals_the_oracle(ctx, options, args):
     got = gpueval.conv_i8(ctx, case, fs_out=fs_out, want=("nhwc",))
     assert np.array_equal(got["nhwc"][..., :k].view(np.uint32), want.transpose(0, 2, 3, 1).view(np.uint32))
     assert np.array_equal(got["i8"][..., :k], port.quantize(want, fs_out).transpose(0, 2, 3, 1))
+
+
+@pytest.mark.parametrize("unary", [None, "leakyrelu", "hardswish"])
+@pytest.mark.parametrize("splits", [(32, 64), (64, 32, 32), (96,)], ids=["32+64", "64+32+32", "96"])
+def test_int8_pointwise_layers_write_their_slices_of_a_concat_with_its_batchnorm_and_activation(ctx, options, splits, unary):
+    """Concat -> BatchNorm -> activation over 1x1 int8 layers, done by the layers themselves: each launch carries its slice
+    of the BatchNorm coefficients (post_bn_a / post_bn_b), the activation (post_op), the Concat's channel count as output
+    stride and exact_k = 1, and writes channels [offset, offset + k) of the int8 tensor only. Against the oracle's
+    convolution and quantizer around the float32 layers' own BatchNorm and activation kernels; what a launch does not own
+    (the other layers' slices, pad channels of the stride) keeps the fill value."""
+    r = np.random.default_rng(905)
+    n, c, h, w = 2, 64, 9, 11
+    total = sum(splits)
+    stride = total + 32            # a stride wider than the Concat: those channels belong to nobody
+    pa = r.normal(0, 0.5, total).astype(np.float32)
+    pb = r.uniform(0.5, 2, total).astype(np.float32)
+    alpha, beta = I8_PARAMS[unary]
+    fs_out = np.float32(11.5)
+    bn = (ctx.array(pa), ctx.array(pb))
+    y = ctx.array(np.full((n, h, w, stride), 77, np.int8))
+    parts, offset = [], 0
+    for i, k in enumerate(splits):
+        case = cases.conv_i8_case(906 + i, n, c, h, w, k, 1, 1, 0, act=0, out_scale=0.02)
+        parts.append(port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], 0, cases.geom_of(case)))
+        d = ctx.conv_desc(n, c, h, w, k, 1, 1, 0, 0, 64, stride, 0, float(fs_out), unary, alpha, beta, 0,
+                          (bn[0].at(4 * offset), bn[1].at(4 * offset)), 1)
+        xq = ctx.quantize_nchw_to_nhwc_i8(ctx.array(case["x"]), case["fs"], 64)
+        wp = ctx.pack_conv_weights(d, hip.I8, case["wt"])
+        from tests.gpueval import dequant_scales
+        ctx.conv2d_i8(d, xq, wp, ctx.array(dequant_scales(case["ws"], case["fs"], k)), ctx.array(case["bias"]), None, y.at(offset))
+        ctx.sync()
+        got = y.download()
+        assert (got[..., offset + k:] == 77).all()      # nothing behind the slice is touched
+        offset += k
+    dev = ctx.channelwise_f32("batchnorm", ctx.array(np.ascontiguousarray(np.concatenate(parts, axis=1))), *bn)
+    if unary:
+        dev = ctx.unary_f32(unary, dev, alpha, beta)
+    ctx.sync()
+    want = port.quantize(dev.download(), fs_out).transpose(0, 2, 3, 1)
+    assert np.array_equal(got[..., :total], want), f"{np.count_nonzero(got[..., :total] != want)} of {want.size} differ"
+    assert np.count_nonzero(want) > want.size // 2
+
+
+def test_batchnorm_and_exact_channels_are_refused_outside_the_int8_pointwise_kernel(ctx):
+    """The two descriptor fields exist for 1x1 int8 layers only: every other layer answers EXHIP_ERR_UNSUPPORTED."""
+    n, c, h, w, k = 1, 64, 8, 8, 64
+    case = cases.conv_i8_case(930, n, c, h, w, k, 3, 1, 1, act=0)
+    bn = (ctx.array(np.zeros(k, np.float32)), ctx.array(np.ones(k, np.float32)))
+    xq = ctx.quantize_nchw_to_nhwc_i8(ctx.array(case["x"]), case["fs"], 64)
+    from tests.gpueval import dequant_scales
+    scale = ctx.array(dequant_scales(case["ws"], case["fs"], k))
+    y = ctx.empty((n, h, w, k), np.int8)
+    for kwargs in (dict(post_bn=bn), dict(exact_k=1)):
+        d = ctx.conv_desc(n, c, h, w, k, 3, 1, 1, 0, 64, k, 0, 5.0, **kwargs)
+        wp = ctx.pack_conv_weights(d, hip.I8, case["wt"])
+        with pytest.raises(hip.ExhipError):
+            ctx.conv2d_i8(d, xq, wp, scale, None, None, y)
+    d = ctx.conv_desc(n, c, h, w, 48, 1, 1, 0, 0, 64, 64, 0, 5.0, exact_k=1)     # exact_k needs whole 32-channel blocks
+    case1 = cases.conv_i8_case(931, n, c, h, w, 48, 1, 1, 0, act=0)
+    wp = ctx.pack_conv_weights(d, hip.I8, case1["wt"])
+    with pytest.raises(hip.ExhipError):
+        ctx.conv2d_i8(d, xq, wp, ctx.array(dequant_scales(case1["ws"], case1["fs"], 48)), None, None, y)
