@@ -72,6 +72,8 @@ struct exhip_options {
     int lean_groups = 0;     // at most this many groups per 64-channel slab (tests: a few groups that walk many patches each)
     int lean_f16 = 1;        // 3x3 stride-1 fp16 layers with an NHWC result on the lean kernel: 0 never, 1 the form per layer class, 2 one group per
                              // patch, 3 persistent groups with three slice buffers, 4 persistent groups with two
+    int direct = 1;          // layers with a filter, a stride or padding and NHWC results on the pointwise kernel's tapped form: 1 where it measured
+                             // faster, 2 wherever it can run, 0 never
     int pw = 1;              // 1x1 stride-1 fp16 layers with an NHWC result: 1 the pointwise kernel where it measured faster, 2 wherever it can run, 0 never
 };
 extern exhip_options g_exhip_options;
@@ -114,11 +116,14 @@ __device__ __forceinline__ void half_swap4(exhip_v4i& a, exhip_v4i& b) {
 }
 
 // float32_to_int8 of the reference (src/Primitives/simd_types.cpp:140-152): add +-0.5, saturate, truncate.
+// Here: the +-0.5 by the value's sign bit, one conversion that truncates toward zero and saturates at the int32 range
+// (NaN -> 0), and the saturation to [-128, 127] on the integer -- for every float the value of add, saturate, truncate
+// (a sum beyond +-128 truncates to an integer beyond it, and -0.0 - 0.5 truncates to 0 like 0.0 + 0.5).
 __device__ __forceinline__ int exhip_q8(float v) {
-    float t = v >= 0.f ? v + 0.5f : v - 0.5f;
-    t = t > 127.f ? 127.f : t;
-    t = t < -128.f ? -128.f : t;
-    return (int)t;  // v_cvt_i32_f32 truncates toward zero
+    int i;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(i) : "v"(v + __builtin_copysignf(0.5f, v)));
+    i = i > 127 ? 127 : i;
+    return i < -128 ? -128 : i;
 }
 
 // suffix_activation_cpu_f32 of the reference (src/Excalibur/operation_general_conv.cpp:127-272).
@@ -140,18 +145,14 @@ __device__ __forceinline__ uint16_t exhip_f2h(float f) { return __builtin_bit_ca
 template <int OP>
 __device__ __forceinline__ float unary_value(float x, float alpha, float beta) {
     if constexpr (OP == 0) {
-        float t = __builtin_fmaf(x, alpha, beta);
-        t = t > 0.f ? t : 0.f;
-        t = t < 1.f ? t : 1.f;
-        return t * x;
+        // clamp to [0, 1] as one median: NaN gives 0 as the two selects do (and the product below is NaN either way)
+        return __builtin_amdgcn_fmed3f(__builtin_fmaf(x, alpha, beta), 0.f, 1.f) * x;
     } else if constexpr (OP == 1) {
         return x < 0.f ? alpha * x : x;
     } else if constexpr (OP == 2) {
         return (float)(1. / (1. + exp(-(double)x)));
     } else if constexpr (OP == 3) {
-        float t = __builtin_fmaf(alpha, x, beta);
-        t = 1.f < t ? 1.f : t;
-        return 0.f < t ? t : 0.f;
+        return __builtin_amdgcn_fmed3f(__builtin_fmaf(alpha, x, beta), 0.f, 1.f);  // NaN -> 0 as with the two selects
     } else {
         const float t = beta < x ? beta : x;  // clip to [alpha, beta]
         return alpha < t ? t : alpha;

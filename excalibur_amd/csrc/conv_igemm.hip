@@ -1757,6 +1757,19 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
         }
         if (d->post_bn_a || d->post_bn_b || d->exact_k) return EXHIP_ERR_UNSUPPORTED;  // only the pointwise kernel has these
+        if (!pl.packed && !proj && !p.acc_nchw && !p.y_nchw && (p.y_q || p.y_nhwc) && pl.KWe == d->kw) {
+            // a layer with a filter on that kernel's tapped form, where it takes the layer
+            exhip_pw_geom g = {};
+            g.pixels = (long long)d->n * pl.OH * pl.OW; g.c_bytes = p.cstride_b; g.k = d->k; g.k_stride = d->k_stride;
+            g.slab_blocks = pl.TM / 32; g.slabs = pl.ktiles;
+            g.act = d->act; g.post_relu = d->post_relu; g.post_op = d->post_op; g.post_slope_shared = d->post_slope_shared;
+            g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope; g.residual_last = d->residual_last;
+            g.fs_out = d->fs_out;
+            const exhip_pw_taps t = {d->n, d->h, d->w, pl.OH, pl.OW, d->kh, d->kw, d->sh, d->pt, d->pl, pl.n_chunks, pl.chunk_b};
+            rc = exhip_conv1x1_i8_pw(ctx, g, reinterpret_cast<const int8_t*>(p.x), p.wp, p.scale, p.bias, reinterpret_cast<const float*>(p.residual),
+                                     reinterpret_cast<int8_t*>(p.y_q), reinterpret_cast<float*>(p.y_nhwc), &t);
+            if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
+        }
         // the fused epilogue: int8 / float32 NHWC tensors only, whole 64-channel slabs, plain or ReLU activation
         const long long out_elems = (long long)d->n * pl.OH * pl.OW * d->k;
         const bool fused = fused_epilogue_ok(d, p, out_elems);
@@ -1796,6 +1809,17 @@ int run_conv(exhip_ctx* ctx, const exhip_conv_desc* d, ConvParams p, const PoolS
             g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope; g.residual_last = d->residual_last;
             rc = exhip_conv1x1_f16_pw(ctx, g, reinterpret_cast<const uint16_t*>(p.x), p.wp, p.bias, reinterpret_cast<const uint16_t*>(p.residual),
                                       reinterpret_cast<uint16_t*>(p.y_q));
+            if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
+        } else if (!pl.packed && !pool && p.y_q && !p.y_nchw_h && !p.y_nchw && pl.KWe == d->kw) {
+            // a layer with a filter on that kernel's tapped form, where it takes the layer
+            exhip_pw_geom g = {};
+            g.pixels = (long long)d->n * pl.OH * pl.OW; g.c_bytes = p.cstride_b; g.k = d->k; g.k_stride = d->k_stride;
+            g.slab_blocks = pl.TM / 32; g.slabs = pl.ktiles;
+            g.act = d->act; g.post_relu = d->post_relu; g.post_op = d->post_op; g.post_slope_shared = d->post_slope_shared;
+            g.post_alpha = d->post_alpha; g.post_beta = d->post_beta; g.post_slope = d->post_slope; g.residual_last = d->residual_last;
+            const exhip_pw_taps t = {d->n, d->h, d->w, pl.OH, pl.OW, d->kh, d->kw, d->sh, d->pt, d->pl, pl.n_chunks, pl.chunk_b};
+            rc = exhip_conv1x1_f16_pw(ctx, g, reinterpret_cast<const uint16_t*>(p.x), p.wp, p.bias, reinterpret_cast<const uint16_t*>(p.residual),
+                                      reinterpret_cast<uint16_t*>(p.y_q), &t);
             if (rc != EXHIP_ERR_UNSUPPORTED) return rc;
         }
     }

@@ -22,10 +22,19 @@ struct exhip_pw_geom {
     int exact_k;
 };
 
+// A layer with a filter, a stride or padding on the same kernel (`taps` below; NULL: the pointwise layer). The wave's
+// pixel fragments then come from the filter's taps around each output pixel -- still straight from the NHWC rows into
+// registers, a tap outside the image reading zeros -- in the order of the packing's k-steps. g.pixels counts output pixels.
+struct exhip_pw_taps {
+    int n, in_h, in_w, out_h, out_w;   // images, input and output maps
+    int kh, kw, stride, pad_t, pad_l;  // at most 32 taps
+    int n_chunks, chunk_b;             // the packing: channel chunks of chunk_b bytes (a multiple of 32), n_chunks * chunk_b bytes per pixel
+};
+
 // Returns 0 when launched, EXHIP_ERR_UNSUPPORTED when the geometry is outside what the kernel takes (the caller then
 // runs the general kernel), another code on failure. Semantics as exhip_conv2d_f16 with only the NHWC half output.
 int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t* x, const void* wp, const float* bias,
-                         const uint16_t* residual, uint16_t* y);
+                         const uint16_t* residual, uint16_t* y, const exhip_pw_taps* taps = nullptr);
 // The int8 layer: semantics as exhip_conv2d_i8 with the NHWC results only (y_i8 and / or y_f32; k_stride a multiple of 16).
 int exhip_conv1x1_i8_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const int8_t* x, const void* wp, const float* scale, const float* bias,
-                        const float* residual, int8_t* y_i8, float* y_f32);
+                        const float* residual, int8_t* y_i8, float* y_f32, const exhip_pw_taps* taps = nullptr);

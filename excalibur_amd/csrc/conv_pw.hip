@@ -35,6 +35,8 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr unsigned kRsrcWord3 = 0x00020000u;  // raw buffer: out-of-range loads return 0
 constexpr int kOutOfRange = 0x7ffff000;       // a lane offset beyond every view
+constexpr int kMaxDirectSteps = 40;           // k-steps of a layer with a filter (taps x 32-byte steps per pixel)
+constexpr int kTapShift = 27;                 // a step's table entry: byte offset below, tap number above
 
 struct PwParams {
     const char* x;
@@ -60,6 +62,10 @@ struct PwParams {
     int K, kstride;
     int act, post_relu, post_op, post_slope_shared, residual_last;
     float post_alpha, post_beta;
+    // the form with a filter (TAPS): output pixel (img, oy, ox) reads input pixel (oy * stride - pt + r, ox * stride - pl + q)
+    // for k-step s of tap r * kw + q, that many bytes behind its top-left input pixel
+    int in_h, in_w, out_h, out_w, stride, pad_t, pad_l, kh, kw;
+    int step[kMaxDirectSteps];   // offset | tap << kTapShift
 };
 
 __device__ __forceinline__ float fast_activation(float v, int act) {
@@ -193,18 +199,21 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
     for (int m = 0; m < MT; ++m) {
         const int ch0 = (kb0 + m) * 32 + (lane >> 5) * 16;
         if (ch0 >= p.K && (p.exact || ch0 >= p.kstride)) continue;
+        // FULL: every channel of the block exists (wave-uniform), and the per-value tests against K fall away
+        auto block = [&](auto full_c) {
+        constexpr bool FULL = decltype(full_c)::value;
         float sc[16], bi[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            sc[e] = ch0 + e < p.K ? p.scale[ch0 + e] : 0.f;
-            bi[e] = (p.bias && ch0 + e < p.K) ? p.bias[ch0 + e] : 0.f;
+            sc[e] = (FULL || ch0 + e < p.K) ? p.scale[ch0 + e] : 0.f;
+            bi[e] = (p.bias && (FULL || ch0 + e < p.K)) ? p.bias[ch0 + e] : 0.f;
         }
         const bool vec_ok = ch0 + 16 <= p.kstride;
         float bna[16], bnb[16];  // the BatchNorm's parameters of these channels (identity beyond K)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            bna[e] = (p.post_bn_a && ch0 + e < p.K) ? p.post_bn_a[ch0 + e] : 0.f;
-            bnb[e] = (p.post_bn_a && ch0 + e < p.K) ? p.post_bn_b[ch0 + e] : 1.f;
+            bna[e] = (p.post_bn_a && (FULL || ch0 + e < p.K)) ? p.post_bn_a[ch0 + e] : 0.f;
+            bnb[e] = (p.post_bn_a && (FULL || ch0 + e < p.K)) ? p.post_bn_b[ch0 + e] : 1.f;
         }
 #pragma unroll
         for (int n = 0; n < NT; ++n) {
@@ -224,7 +233,7 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
             if (p.residual_f) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) r[e] = 0.f;
-                if (valid && ch0 + 16 <= p.K) {
+                if (valid && (FULL || ch0 + 16 <= p.K)) {
 #pragma unroll
                     for (int e4 = 0; e4 < 4; ++e4) {
                         const v4f t = *reinterpret_cast<const v4f*>(p.residual_f + at + e4 * 4);
@@ -240,7 +249,7 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
             if (p.residual_f && !p.residual_last) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
-                    if (ch0 + e < p.K) v[e] += r[e];
+                    if (FULL || ch0 + e < p.K) v[e] += r[e];
             }
             if (p.post_relu) {
 #pragma unroll
@@ -253,7 +262,7 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
             if (p.post_op == EXHIP_POST_PRELU) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const float slope = p.post_slope[p.post_slope_shared || ch0 + e >= p.K ? 0 : ch0 + e];
+                    const float slope = p.post_slope[p.post_slope_shared || (!FULL && ch0 + e >= p.K) ? 0 : ch0 + e];
                     v[e] = v[e] >= 0.f ? v[e] : slope * v[e];
                 }
             } else if (p.post_op) {
@@ -271,11 +280,11 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
             if (p.residual_f && p.residual_last) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e)
-                    if (ch0 + e < p.K) v[e] += r[e];
+                    if (FULL || ch0 + e < p.K) v[e] += r[e];
             }
 #pragma unroll
             for (int e = 0; e < 16; ++e)
-                if (ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
+                if (!FULL && ch0 + e >= p.K) v[e] = 0.f;  // pad channels hold zeros
             if (p.y_f && (kb0 + m) * 32 + 32 <= p.kstride && __builtin_amdgcn_ballot_w64(valid) == ~0ull) {
                 // the whole wave stores a whole 32-channel block: the two half-waves trade 16-byte pieces and neighbouring
                 // lanes trade pixels, so that four lanes (p, p + 1 and the same two of the other half-wave) write 64
@@ -325,10 +334,13 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        };
+        if ((kb0 + m) * 32 + 32 <= p.K) block(std::true_type{});
+        else block(std::false_type{});
     }
 }
 
-template <int DT, int MT, int NT>
+template <int DT, int MT, int NT, bool TAPS>
 __global__ __launch_bounds__(256, 2) void conv1x1_pw_kernel(const PwParams p) {
     constexpr int U = MT + NT > 4 ? 2 : 4;  // k-steps fetched per request round; two rounds are in flight
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -350,10 +362,28 @@ __global__ __launch_bounds__(256, 2) void conv1x1_pw_kernel(const PwParams p) {
     // pixel fragments: lane = pixel (lane & 31), 16-byte half (lane >> 5) of each 32-byte k-step
     unsigned pix[NT];
     int xoff[NT];
+    unsigned taps_in[NT];  // TAPS: bit r * kw + q set where that tap of the pixel lies inside the image
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         pix[nt] = (tile * NT + nt) * 32 + (lane & 31);
-        xoff[nt] = pix[nt] < p.pixels ? (int)(pix[nt] * (unsigned)p.xs_b) + (lane >> 5) * 16 : kOutOfRange;
+        if constexpr (TAPS) {
+            // the filter's top-left input pixel; its offset may lie in front of the tensor (padding), the taps inside the
+            // image never do, and 32-bit wrap-around of the sum gives their offsets
+            const unsigned per_image = (unsigned)(p.out_h * p.out_w);
+            const unsigned img = pix[nt] / per_image, rem = pix[nt] - img * per_image;
+            const int oy = (int)(rem / (unsigned)p.out_w), ox = (int)(rem - (unsigned)oy * (unsigned)p.out_w);
+            const int iy = oy * p.stride - p.pad_t, ix = ox * p.stride - p.pad_l;
+            xoff[nt] = (((int)img * p.in_h + iy) * p.in_w + ix) * p.xs_b + (lane >> 5) * 16;
+            unsigned m = 0;
+            if (pix[nt] < p.pixels) {
+                for (int r = 0; r < p.kh; ++r)
+                    for (int q = 0; q < p.kw; ++q)
+                        if ((unsigned)(iy + r) < (unsigned)p.in_h && (unsigned)(ix + q) < (unsigned)p.in_w) m |= 1u << (r * p.kw + q);
+            }
+            taps_in[nt] = m;
+        } else {
+            xoff[nt] = pix[nt] < p.pixels ? (int)(pix[nt] * (unsigned)p.xs_b) + (lane >> 5) * 16 : kOutOfRange;
+        }
     }
     // weight fragments: block kb of slab kb / mts lies at ((slab * n_ksteps + ks) * mts + kb % mts) KiB; the MT blocks
     // of a wave are neighbours in one slab (mts is a multiple of MT)
@@ -380,9 +410,18 @@ __global__ __launch_bounds__(256, 2) void conv1x1_pw_kernel(const PwParams p) {
 #pragma unroll
                 for (int m = 0; m < MT; ++m)
                     a[buf][u][m] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(wr, woff + m * 1024, w_base + (ks0 + u) * w_step, 0));
+                if constexpr (TAPS) {
+                    const int entry = p.step[ks0 + u];
+                    const int off = entry & ((1 << kTapShift) - 1);
+                    const unsigned bit = 1u << ((unsigned)entry >> kTapShift);
 #pragma unroll
-                for (int n = 0; n < NT; ++n)
-                    b[buf][u][n] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(xr, xoff[n], (ks0 + u) * 32, 0));
+                    for (int n = 0; n < NT; ++n)
+                        b[buf][u][n] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(xr, (taps_in[n] & bit) ? xoff[n] + off : kOutOfRange, 0, 0));
+                } else {
+#pragma unroll
+                    for (int n = 0; n < NT; ++n)
+                        b[buf][u][n] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(xr, xoff[n], (ks0 + u) * 32, 0));
+                }
             }
         }
     };
@@ -423,7 +462,7 @@ __global__ __launch_bounds__(256, 2) void conv1x1_pw_kernel(const PwParams p) {
     }
 }
 
-template <int DT, int MT, int NT>
+template <int DT, int MT, int NT, bool TAPS = false>
 int launch(exhip_ctx* ctx, PwParams& p, int kblocks) {
     const long long tiles = ((long long)p.pixels + 32 * NT - 1) / (32 * NT);
     p.ch_groups = (unsigned)((kblocks + MT - 1) / MT);
@@ -431,7 +470,7 @@ int launch(exhip_ctx* ctx, PwParams& p, int kblocks) {
     if (items >= (1ll << 31)) return EXHIP_ERR_UNSUPPORTED;
     p.items = (unsigned)items;
     const unsigned grid = (unsigned)((items + 3) / 4);
-    hipLaunchKernelGGL((conv1x1_pw_kernel<DT, MT, NT>), dim3(grid), dim3(256), 0, ctx->stream, p);
+    hipLaunchKernelGGL((conv1x1_pw_kernel<DT, MT, NT, TAPS>), dim3(grid), dim3(256), 0, ctx->stream, p);
     EXHIP_LAUNCH_CHECK();
     return 0;
 }
@@ -440,10 +479,58 @@ int launch(exhip_ctx* ctx, PwParams& p, int kblocks) {
 
 namespace {
 
+// A layer with a filter, a stride or padding on the same kernel: g.pixels counts output pixels, the k-steps walk the
+// packing's order (channel chunk, filter row, tap, 32-byte step).
+template <int DT>
+int run_taps(exhip_ctx* ctx, const exhip_pw_geom& g, const exhip_pw_taps& t, PwParams& p, bool has_residual) {
+    if (g_exhip_options.direct == 0) return EXHIP_ERR_UNSUPPORTED;
+    if (g.post_bn_a || g.post_bn_b || g.exact_k) return EXHIP_ERR_UNSUPPORTED;
+    const long long n_ksteps = (long long)t.n_chunks * t.kh * t.kw * (t.chunk_b / 32);
+    if (g.pixels <= 0 || g.c_bytes <= 0 || g.c_bytes % 32 != 0 || t.chunk_b % 32 != 0 || t.n_chunks * t.chunk_b != g.c_bytes ||
+        (g.slab_blocks != 2 && g.slab_blocks != 4) || g.k_stride % 8 != 0 || n_ksteps > kMaxDirectSteps || t.kh * t.kw > (1 << (32 - kTapShift)) || t.stride < 1 || t.pad_t < 0 || t.pad_l < 0)
+        return EXHIP_ERR_UNSUPPORTED;
+    const long long x_bytes = (long long)t.n * t.in_h * t.in_w * g.c_bytes;
+    const long long w_bytes = (long long)g.slabs * n_ksteps * g.slab_blocks * 1024;
+    const long long reach = ((long long)(t.kh - 1) * t.in_w + t.kw) * g.c_bytes;   // the furthest step behind a pixel's top-left tap
+    if (x_bytes >= kOutOfRange || w_bytes >= kOutOfRange || reach >= (1ll << kTapShift) || g.pixels != (long long)t.n * t.out_h * t.out_w ||
+        g.pixels * 4 * g.k_stride >= (1ll << 40) || g.pixels >= (1ll << 31))
+        return EXHIP_ERR_UNSUPPORTED;
+    if (g.post_op && g.post_op != EXHIP_POST_PRELU && (g.post_op < 1 || g.post_op > 1 + EXHIP_UNARY_CLIP || g.post_op == 1 + EXHIP_UNARY_SIGMOID))
+        return EXHIP_ERR_UNSUPPORTED;
+    const int kblocks = std::min(g.slabs * g.slab_blocks, (std::max(g.k, g.k_stride) + 31) / 32);
+    // Measured inside two detection networks at 16 x 3 x 640 x 640 and two mobile networks: the fp16 layers the lean
+    // kernel leaves (stride 2, 12 or 32 input channels, ragged output channels) are faster here as a whole (0.88 -> 0.85 ms
+    // and 1.83 -> 1.81 ms per forward of the detection networks); of the int8 layers only a few deep ones are (3x3
+    // stride 2 from 40 x 40: 29 -> 23 us) while the wide first layers lose (12 -> 32 channels at 320 x 320: 81 -> 94 us),
+    // so int8 layers stay with the staged kernels unless the option asks.
+    const bool take = DT == EXHIP_F16;
+    if (g_exhip_options.direct != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
+    p.post_slope = g.post_slope;
+    p.pixels = (unsigned)g.pixels; p.x_bytes = (unsigned)x_bytes; p.w_bytes = (unsigned)w_bytes;
+    p.xs_b = g.c_bytes; p.n_ksteps = (int)n_ksteps; p.mts = g.slab_blocks;
+    p.K = g.k; p.kstride = g.k_stride;
+    p.act = g.act; p.post_relu = g.post_relu; p.post_op = g.post_op; p.post_slope_shared = g.post_slope_shared;
+    p.residual_last = g.residual_last && has_residual;
+    p.post_alpha = g.post_alpha; p.post_beta = g.post_beta;
+    p.in_h = t.in_h; p.in_w = t.in_w; p.out_h = t.out_h; p.out_w = t.out_w; p.stride = t.stride; p.pad_t = t.pad_t; p.pad_l = t.pad_l;
+    p.kh = t.kh; p.kw = t.kw;
+    int s = 0;
+    for (int cc = 0; cc < t.n_chunks; ++cc)
+        for (int r = 0; r < t.kh; ++r)
+            for (int q = 0; q < t.kw; ++q)
+                for (int j = 0; j < t.chunk_b / 32; ++j)
+                    p.step[s++] = ((r * t.in_w + q) * g.c_bytes + cc * t.chunk_b + j * 32) | (int)((unsigned)(r * t.kw + q) << kTapShift);
+    if (kblocks == 1) return launch<DT, 1, 4, true>(ctx, p, kblocks);
+    const long long waves64 = ((g.pixels + 63) / 64) * ((kblocks + 1) / 2);
+    if (waves64 < 2048) return launch<DT, 2, 1, true>(ctx, p, kblocks);
+    return launch<DT, 2, 2, true>(ctx, p, kblocks);
+}
+
 // Geometry checks and the wave tile, shared by the two data types. `es`: bytes per input element.
 template <int DT>
-int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has_residual) {
+int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has_residual, const exhip_pw_taps* t = nullptr) {
     if (g_exhip_options.pw == 0) return EXHIP_ERR_UNSUPPORTED;
+    if (t) return run_taps<DT>(ctx, g, *t, p, has_residual);
     // Measured per layer against the general kernel inside a detection and two mobile networks (16 and 64 images, kernel
     // traces): this form wins where a launch is short -- every layer of at most 32 768 pixels up to about 7 GFLOP (twice
     // as fast on 20 x 20 maps) --, for a lone 32-channel block (which the general kernel pads to a 64-channel slab), and on
@@ -491,18 +578,18 @@ int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has
 }  // namespace
 
 int exhip_conv1x1_f16_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const uint16_t* x, const void* wp, const float* bias,
-                         const uint16_t* residual, uint16_t* y) {
+                         const uint16_t* residual, uint16_t* y, const exhip_pw_taps* taps) {
     PwParams p = {};
     p.x = reinterpret_cast<const char*>(x); p.wp = reinterpret_cast<const char*>(wp); p.bias = bias; p.residual = residual; p.y = y;
-    return run_pw<EXHIP_F16>(ctx, g, p, 2, residual != nullptr);
+    return run_pw<EXHIP_F16>(ctx, g, p, 2, residual != nullptr, taps);
 }
 
 int exhip_conv1x1_i8_pw(exhip_ctx* ctx, const exhip_pw_geom& g, const int8_t* x, const void* wp, const float* scale, const float* bias,
-                        const float* residual, int8_t* y_i8, float* y_f32) {
+                        const float* residual, int8_t* y_i8, float* y_f32, const exhip_pw_taps* taps) {
     if (!scale || (!y_i8 && !y_f32) || g.k_stride % 16 != 0) return EXHIP_ERR_UNSUPPORTED;
     PwParams p = {};
     p.x = reinterpret_cast<const char*>(x); p.wp = reinterpret_cast<const char*>(wp); p.bias = bias; p.scale = scale;
     p.residual_f = residual; p.y_f = y_f32; p.y_q = y_i8; p.fs_out = g.fs_out;
     p.post_bn_a = g.post_bn_a; p.post_bn_b = g.post_bn_b; p.exact = g.exact_k;
-    return run_pw<EXHIP_I8>(ctx, g, p, 1, residual != nullptr);
+    return run_pw<EXHIP_I8>(ctx, g, p, 1, residual != nullptr, taps);
 }

@@ -832,3 +832,31 @@ def test_max_pooling_on_int8_nhwc(ctx, kernel, stride, pad, h, w):
     q[..., :c] = port.quantize(v, fs).transpose(0, 2, 3, 1)
     got = ctx.maxpool2d_nhwc_i8(ctx.array(q), c, kernel, stride, (pad, pad), oh, ow).download()
     assert np.array_equal(got[..., :c], port.quantize(port.pool2d(v, port.POOL_MAX, kernel, stride, pad), fs).transpose(0, 2, 3, 1))
+
+
+def test_quantizer_and_clamped_activations_at_the_edges_of_their_ranges(ctx):
+    """float32_to_int8 and the activations that clamp (HardSwish, HardSigmoid) on the values where their selects turn:
+    zeros of both signs, denormals, the halves around every rounding step near the saturation points, values beyond the
+    int32 range and infinities -- against the oracle, bit for bit. (NaN is left out: the reference's conversion of it is
+    undefined behaviour.)"""
+    edge = [0.0, -0.0, 1e-45, -1e-45, 1e-39, -1e-39, 0.49999997, 0.5, 0.50000006, -0.49999997, -0.5, -0.50000006, 1.4999999, 1.5, -1.5,
+            126.49999, 126.5, 127.0, 127.49999, 127.5, 128.0, 128.5, 1000.0, -127.5, -128.0, -128.49999, -128.5, -129.0, -1000.0,
+            2147483520.0, 2147483648.0, -2147483648.0, 4294967296.0, 3e38, -3e38, np.inf, -np.inf,
+            -3.0, -2.9999998, -3.0000002, 3.0, 2.9999998, 3.0000002, -2.5, 2.5, 6.0, -6.0]
+    r = np.random.default_rng(77)
+    x = np.concatenate([np.array(edge, np.float32), r.uniform(-140, 140, 4096).astype(np.float32),
+                        (r.integers(-130, 131, 2048) + r.choice([-0.5, 0.5], 2048)).astype(np.float32)]).astype(np.float32)
+    x = np.ascontiguousarray(x.reshape(1, 1, 1, -1))
+    for fs in (1.0, 0.37, 3.0):
+        q = ctx.quantize_nchw_to_nhwc_i8(ctx.array(x), fs, 32)
+        ctx.sync()
+        assert np.array_equal(q.download()[0, 0, :, 0], port.quantize(x, np.float32(fs))[0, 0, 0])
+    for name, fn, a, b in (("hardswish", port.hardswish, 1 / 6, 0.5), ("hardsigmoid", port.hardsigmoid, 0.2, 0.5),
+                           ("hardswish", port.hardswish, 0.5, -0.25)):
+        y = ctx.unary_f32(name, ctx.array(x), a, b)
+        ctx.sync()
+        want = fn(x, a, b)
+        got = y.download()
+        ok = ~np.isnan(want)     # inf * 0 is NaN on both sides; payloads are not compared
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32)), name

@@ -25,7 +25,7 @@ def options():
         hip.set_option(name, value)
         changed.append(name)
     yield set_
-    defaults = dict(pw=1, force_splits=0)
+    defaults = dict(pw=1, force_splits=0, direct=1, lean=4, lean_f16=1)
     for name in changed:
         hip.set_option(name, defaults[name])
 
@@ -240,3 +240,115 @@ def test_batchnorm_and_exact_channels_are_refused_outside_the_int8_pointwise_ker
     wp = ctx.pack_conv_weights(d, hip.I8, case1["wt"])
     with pytest.raises(hip.ExhipError):
         ctx.conv2d_i8(d, xq, wp, ctx.array(dequant_scales(case1["ws"], case1["fs"], 48)), None, None, y)
+
+
+TAP_SHAPES = [
+    # seed, n, c, h, w, k, kernel, stride, pad, shortcut (0 none, 1 in front, 2 behind), act, post_relu, post_op
+    (800, 2, 12, 40, 36, 32, 3, 1, 1, 0, 0, 0, "hardswish"),       # a first layer behind Focus: 12 channels in a 32-byte pixel
+    (801, 2, 32, 41, 37, 64, 3, 2, 1, 0, 0, 0, "hardswish"),       # stride 2 on odd sizes
+    (802, 1, 64, 20, 20, 128, 3, 2, 1, 0, 1, 0, None),
+    (803, 2, 32, 17, 19, 32, 3, 1, 1, 2, 0, 0, "leakyrelu"),       # a bottleneck's 3x3 with the sum behind the activation
+    (804, 1, 64, 14, 14, 96, 3, 1, 1, 1, 0, 1, None),              # shortcut + ReLU; 96 channels: a half-empty second group
+    (805, 1, 16, 13, 11, 40, 5, 1, 2, 0, 1, 0, None),              # 25 taps, ragged channels
+    (806, 3, 64, 16, 16, 64, 1, 2, 0, 0, 0, 0, None),              # a projection shortcut: 1x1 stride 2
+    (807, 1, 32, 9, 30, 64, (3, 1), 1, (1, 1, 0, 0), 0, 1, 0, None),   # 3x1 filter
+    (808, 1, 128, 12, 12, 64, 3, 1, 0, 0, 0, 0, "clip"),           # no padding: the output is smaller than the input
+    (809, 2, 48, 10, 10, 32, 2, 2, 0, 0, 0, 0, None),              # 2x2 stride 2 (a 64-byte pixel with 16 pad bytes)
+]
+
+
+@pytest.mark.parametrize("outputs", ["both", "int8", "float32"])
+@pytest.mark.parametrize("args", TAP_SHAPES, ids=[f"s{a[0]}" for a in TAP_SHAPES])
+def test_int8_layers_with_a_filter_on_the_kernel_without_staging_repeat_the_general_kernel(ctx, options, args, outputs):
+    """The tapped form of the kernel (pixel fragments fetched from the filter's taps around each output pixel, zeros
+    outside the image) against the general and lean kernels on the same packed weights, bit for bit; those are pinned
+    against the oracle in tests/test_gpu_ops.py."""
+    from tests import gpueval
+    seed, n, c, h, w, k, kernel, stride, pad, shortcut, act, post_relu, post_op = args
+    case = cases.conv_i8_case(seed, n, c, h, w, k, kernel, stride, pad, act=act)
+    ks = hip.pad_to(k, 32)
+    oh, ow = port.out_hw(cases.geom_of(case))
+    res = np.random.default_rng(seed + 50).uniform(-2, 2, (n, oh, ow, ks)).astype(np.float32) if shortcut else None
+    alpha, beta = I8_PARAMS[post_op]
+    want_list = ("nhwc",) if outputs != "int8" else ()
+    fs_out = None if outputs == "float32" else np.float32(9.7)
+    kw = dict(fs_out=fs_out, residual=res, post_relu=post_relu, want=want_list, post_op=post_op, post_alpha=alpha, post_beta=beta,
+              residual_last=1 if shortcut == 2 else 0)
+    options("force_splits", 1)
+    options("direct", 0)
+    want = gpueval.conv_i8(ctx, case, **kw)
+    options("direct", 2)
+    got = gpueval.conv_i8(ctx, case, **kw)
+    for name in ("nhwc", "i8"):
+        if name in want:
+            a, b = want[name][..., :k], got[name][..., :k]
+            assert a.shape == (n, oh, ow, k)
+            assert np.array_equal(a.view(np.uint32) if name == "nhwc" else a, b.view(np.uint32) if name == "nhwc" else b), \
+                f"{name}: {np.count_nonzero(a != b)} of {a.size} differ"
+            assert np.count_nonzero(b) > b.size // 8
+            if k < ks:
+                assert not got[name][..., k:].any()
+
+
+def test_int8_tapped_form_equals_the_oracle(ctx, options):
+    from tests import gpueval
+    options("direct", 2)
+    for seed, n, c, h, w, k, kernel, stride, pad in [(820, 2, 12, 24, 20, 32, 3, 1, 1), (821, 1, 32, 23, 25, 64, 3, 2, 1), (822, 1, 64, 9, 9, 255, 3, 1, 1)]:
+        case = cases.conv_i8_case(seed, n, c, h, w, k, kernel, stride, pad)
+        want = port.conv2d_i8(case["x"], case["wt"], case["bias"], case["ws"], case["fs"], case["act"], cases.geom_of(case))
+        fs_out = np.float32(7.3)
+        got = gpueval.conv_i8(ctx, case, fs_out=fs_out, want=("nhwc",))
+        assert np.array_equal(got["nhwc"][..., :k].view(np.uint32), want.transpose(0, 2, 3, 1).view(np.uint32))
+        assert np.array_equal(got["i8"][..., :k], port.quantize(want, fs_out).transpose(0, 2, 3, 1))
+
+
+F16_TAP_SHAPES = [
+    # seed, n, c, h, w, k, kernel, stride, pad, shortcut, act, post_relu, post_op
+    (840, 2, 12, 40, 36, 32, 3, 1, 1, False, 0, 0, "hardswish"),
+    (841, 2, 32, 41, 37, 64, 3, 2, 1, False, 0, 0, "hardswish"),
+    (842, 1, 64, 20, 20, 128, 3, 2, 1, False, 1, 0, None),
+    (843, 2, 32, 17, 19, 32, 3, 1, 1, True, 0, 1, None),
+    (844, 1, 16, 13, 11, 40, 5, 1, 2, False, 1, 0, None),
+    (845, 3, 64, 16, 16, 64, 1, 2, 0, False, 0, 0, None),
+]
+
+
+@pytest.mark.parametrize("args", F16_TAP_SHAPES, ids=[f"s{a[0]}" for a in F16_TAP_SHAPES])
+def test_fp16_layers_with_a_filter_on_the_kernel_without_staging(ctx, options, args):
+    """fp16: against the general kernel (the k-steps run in the same order: bit for bit) and against the oracle on the
+    half-rounded operands at 2e-3."""
+    seed, n, c, h, w, k, kernel, stride, pad, shortcut, act, post_relu, post_op = args
+    r = np.random.default_rng(seed)
+    cs, ks = hip.pad_to(c, 16), hip.pad_to(k, 16)
+    x = np.zeros((n, h, w, cs), np.float16)
+    x[..., :c] = r.uniform(-1, 1, (n, h, w, c)).astype(np.float16)
+    wt = r.normal(0, 0.08, (k, c, kernel, kernel)).astype(np.float16)
+    bias = r.normal(0, 0.1, k).astype(np.float32)
+    g = port.geom((n, c, h, w), k, kernel, kernel, stride, pad)
+    oh, ow = port.out_hw(g)
+    res = r.uniform(-1, 1, (n, oh, ow, ks)).astype(np.float16) if shortcut else None
+    alpha, beta = I8_PARAMS[post_op]
+
+    def launch():
+        d = ctx.conv_desc(n, c, h, w, k, kernel, stride, pad, act, cs, ks, post_relu, 0.0, post_op, alpha, beta, 0)
+        wp = ctx.pack_conv_weights(d, hip.F16, wt.view(np.uint16))
+        y = ctx.array(np.full((n, oh, ow, ks), 0x7e00, np.uint16))
+        ctx.conv2d_f16(d, ctx.array(x.view(np.uint16)), wp, ctx.array(bias), ctx.array(res.view(np.uint16)) if shortcut else None, y, None, None)
+        ctx.sync()
+        return y.download()
+
+    options("force_splits", 1)
+    options("lean_f16", 0)
+    options("direct", 0)
+    want = launch()
+    options("direct", 2)
+    got = launch()
+    assert np.array_equal(want, got), f"{np.count_nonzero(want != got)} of {want.size} differ"
+    ref = port.conv2d_f32(x[..., :c].astype(np.float32).transpose(0, 3, 1, 2), wt.astype(np.float32), bias, act, g)
+    if shortcut:
+        ref = ref + res[..., :k].astype(np.float32).transpose(0, 3, 1, 2)
+    if post_relu:
+        ref = np.maximum(ref, 0)
+    if post_op:
+        ref = port.hardswish(ref, alpha, beta)
+    assert cases.check_value(got[..., :k].view(np.float16).astype(np.float32), ref.transpose(0, 2, 3, 1), 2e-3) == 0
