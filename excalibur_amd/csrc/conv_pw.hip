@@ -335,8 +335,13 @@ __device__ __forceinline__ void pw_epilogue_i8(const PwParams& p, const v16i (&a
             __builtin_amdgcn_sched_barrier(0);
         }
         };
-        if ((kb0 + m) * 32 + 32 <= p.K) block(std::true_type{});
-        else block(std::false_type{});
+        // (the 64 x 64 tile keeps the one general form: with both its epilogue no longer fits the register file)
+        if constexpr (MT + NT < 4 || MT == 1) {
+            if ((kb0 + m) * 32 + 32 <= p.K) block(std::true_type{});
+            else block(std::false_type{});
+        } else {
+            block(std::false_type{});
+        }
     }
 }
 
