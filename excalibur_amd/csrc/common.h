@@ -74,6 +74,7 @@ struct exhip_options {
                              // patch, 3 persistent groups with three slice buffers, 4 persistent groups with two
     int direct = 1;          // layers with a filter, a stride or padding and NHWC results on the pointwise kernel's tapped form: 1 where it measured
                              // faster, 2 wherever it can run, 0 never
+    int pw_tile = 0;         // that kernel's wave tile for more than 32 output channels: 0 = 32 pixels x 64 channels, 2 = 64 x 64 from 2048 waves on
     int pw = 1;              // 1x1 stride-1 fp16 layers with an NHWC result: 1 the pointwise kernel where it measured faster, 2 wherever it can run, 0 never
 };
 extern exhip_options g_exhip_options;

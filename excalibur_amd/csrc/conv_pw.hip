@@ -484,6 +484,13 @@ int launch(exhip_ctx* ctx, PwParams& p, int kblocks) {
 
 namespace {
 
+// Layers of more than 32 output channels take the 32-pixel x 64-channel wave tile whatever their size: half the registers of
+// the 64 x 64 tile, so more waves hide each other's loads and epilogues. Measured on whole forwards against "64 x 64 from
+// 2048 waves on" (option pw_tile = 2): int8 64 -> 64 at 16 x 160 x 160 41 -> 30 us, a detection network's int8 forward
+// 1.44 -> 1.35 ms, its fp16 forward 1.81 -> 1.79 ms, two mobile networks' fp16 forwards 0.435 -> 0.42 and 0.82 -> 0.805 ms.
+template <int DT>
+bool small_tile() { return g_exhip_options.pw_tile != 2; }
+
 // A layer with a filter, a stride or padding on the same kernel: g.pixels counts output pixels, the k-steps walk the
 // packing's order (channel chunk, filter row, tap, 32-byte step).
 template <int DT>
@@ -508,7 +515,7 @@ int run_taps(exhip_ctx* ctx, const exhip_pw_geom& g, const exhip_pw_taps& t, PwP
     // and 1.83 -> 1.81 ms per forward of the detection networks); of the int8 layers only a few deep ones are (3x3
     // stride 2 from 40 x 40: 29 -> 23 us) while the wide first layers lose (12 -> 32 channels at 320 x 320: 81 -> 94 us),
     // so int8 layers stay with the staged kernels unless the option asks.
-    const bool take = DT == EXHIP_F16;
+    const bool take = DT == EXHIP_F16 || g.c_bytes == 32 || (g.pixels <= 32768 && kblocks <= 4) || g.pixels <= 6400;
     if (g_exhip_options.direct != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
     p.post_slope = g.post_slope;
     p.pixels = (unsigned)g.pixels; p.x_bytes = (unsigned)x_bytes; p.w_bytes = (unsigned)w_bytes;
@@ -527,7 +534,7 @@ int run_taps(exhip_ctx* ctx, const exhip_pw_geom& g, const exhip_pw_taps& t, PwP
                     p.step[s++] = ((r * t.in_w + q) * g.c_bytes + cc * t.chunk_b + j * 32) | (int)((unsigned)(r * t.kw + q) << kTapShift);
     if (kblocks == 1) return launch<DT, 1, 4, true>(ctx, p, kblocks);
     const long long waves64 = ((g.pixels + 63) / 64) * ((kblocks + 1) / 2);
-    if (waves64 < 2048) return launch<DT, 2, 1, true>(ctx, p, kblocks);
+    if (waves64 < 2048 || small_tile<DT>()) return launch<DT, 2, 1, true>(ctx, p, kblocks);
     return launch<DT, 2, 2, true>(ctx, p, kblocks);
 }
 
@@ -551,6 +558,8 @@ int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has
     const double flop = 2.0 * (double)g.pixels * (g.c_bytes / es) * g.k;
     bool take = joined || blocks_needed == 1 || (flop <= 8.0e9 && g.pixels <= 32768);
     if (DT == EXHIP_I8 && g.pixels <= 131072 && (g.c_bytes <= 64 || (p.y_f && !p.y_q))) take = true;
+    if (DT == EXHIP_I8 && g_exhip_options.pw_tile != 2 && g.c_bytes <= 512) take = true;  // with the small tile: every layer measured
+    if (DT == EXHIP_F16 && g_exhip_options.pw_tile != 2) take = true;  // with the small tile: every layer measured
     if (DT == EXHIP_F16 && ((g.c_bytes <= 128 && g.pixels <= 524288) || (g.c_bytes <= 256 && g.k <= 64 && g.pixels <= 131072))) take = true;
     if (g_exhip_options.pw != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
     if (g.pixels <= 0 || g.c_bytes <= 0 || g.c_bytes % 32 != 0 || (g.slab_blocks != 2 && g.slab_blocks != 4) || g.k_stride % 8 != 0)
@@ -576,7 +585,7 @@ int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has
     // takes 128 pixels per wave
     if (kblocks == 1) return launch<DT, 1, 4>(ctx, p, kblocks);
     const long long waves64 = ((g.pixels + 63) / 64) * ((kblocks + 1) / 2);
-    if (waves64 < 2048) return launch<DT, 2, 1>(ctx, p, kblocks);
+    if (waves64 < 2048 || small_tile<DT>()) return launch<DT, 2, 1>(ctx, p, kblocks);
     return launch<DT, 2, 2>(ctx, p, kblocks);
 }
 

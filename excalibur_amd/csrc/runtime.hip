@@ -34,6 +34,7 @@ extern "C" int exhip_set_option(const char* name, int value) {
     else if (!strcmp(name, "lean_cfg")) o.lean_cfg = value;
     else if (!strcmp(name, "pw")) o.pw = value;
     else if (!strcmp(name, "direct")) o.direct = value;
+    else if (!strcmp(name, "pw_tile")) o.pw_tile = value;
     else if (!strcmp(name, "lean_f16")) o.lean_f16 = value;
     else if (!strcmp(name, "lean_groups")) o.lean_groups = value;
     else if (!strcmp(name, "lean_wres")) o.lean_wres = value;

@@ -25,7 +25,7 @@ def options():
         hip.set_option(name, value)
         changed.append(name)
     yield set_
-    defaults = dict(pw=1, force_splits=0, direct=1, lean=4, lean_f16=1)
+    defaults = dict(pw=1, force_splits=0, direct=1, lean=4, lean_f16=1, pw_tile=0)
     for name in changed:
         hip.set_option(name, defaults[name])
 
@@ -352,3 +352,28 @@ def test_fp16_layers_with_a_filter_on_the_kernel_without_staging(ctx, options, a
     if post_op:
         ref = port.hardswish(ref, alpha, beta)
     assert cases.check_value(got[..., :k].view(np.float16).astype(np.float32), ref.transpose(0, 2, 3, 1), 2e-3) == 0
+
+
+def test_the_two_wave_tiles_give_the_same_results(ctx, options):
+    """Layers of more than 32 output channels run on 32-pixel x 64-channel wave tiles; option pw_tile = 2 brings back the
+    64 x 64 tile for launches of 2048 waves and more. Same k-step order, same epilogue: int8 and fp16 results bit for bit,
+    pointwise and with a filter."""
+    from tests import gpueval
+    options("pw", 2)
+    options("direct", 2)
+    options("lean_f16", 0)
+    options("force_splits", 1)
+    for kernel, stride, pad, h in ((1, 1, 0, 128), (3, 2, 1, 256)):
+        case = cases.conv_i8_case(950 + kernel, 2, 32, h, h, 256, kernel, stride, pad, act=0, out_scale=0.05)
+        res = {}
+        for tile in (0, 2):
+            options("pw_tile", tile)
+            res[tile] = gpueval.conv_i8(ctx, case, fs_out=np.float32(3.1), want=("nhwc",), post_op="hardswish", post_alpha=1 / 6, post_beta=0.5)
+        assert np.array_equal(res[0]["nhwc"].view(np.uint32), res[2]["nhwc"].view(np.uint32))
+        assert np.array_equal(res[0]["i8"], res[2]["i8"]) and np.count_nonzero(res[0]["i8"]) > res[0]["i8"].size // 4
+    x, wt, bias, _ = operands(955, 2, 64, 128, 128, 256, 64, 256, False)
+    out = {}
+    for tile in (0, 2):
+        options("pw_tile", tile)
+        out[tile] = run(ctx, 2, 64, 128, 128, 256, x, wt, bias, None, 64, 256, post_op="hardswish", alpha=1 / 6, beta=0.5)
+    assert np.array_equal(out[0], out[2]) and np.count_nonzero(out[0]) > out[0].size // 2
