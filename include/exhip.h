@@ -52,8 +52,10 @@ const char* exhip_last_error(void);
  * planner that launches of several streams overlap on the GPU (it then prefers one more group per CU over fewer rounds
  * of a launch: measured 3 % faster with two forwards in flight, 2 % slower alone; off unless set).
  * "lean" / "lean_cfg" / "lean_wres" / "lean_groups" / "lean_f16" choose the form of the lean 3x3 kernel for int8 / fp16
- * layers (0 = the general kernel), "pw" the pointwise fp16 kernel (1 where it measured faster, 2 wherever it can run,
- * 0 never), "stem" the one-kernel stem: every form computes the same values.
+ * layers (0 = the general kernel), "pw" the fp16 / int8 kernel without staging for pointwise layers and "direct" its
+ * form for layers with a filter (1 where it measured faster, 2 wherever it can run, 0 never), "pw_tile" that kernel's wave
+ * tile (0 = 32 pixels x 64 channels, 2 = 64 x 64 for large launches), "stem" the one-kernel stem: every form computes
+ * the same values.
  * Process-wide; packed weights depend on the first three, so set them before packing. */
 int exhip_set_option(const char* name, int value);
 int exhip_device_name(exhip_ctx* ctx, char* buf, size_t len);
