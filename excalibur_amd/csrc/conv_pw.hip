@@ -515,7 +515,9 @@ int run_taps(exhip_ctx* ctx, const exhip_pw_geom& g, const exhip_pw_taps& t, PwP
     // and 1.83 -> 1.81 ms per forward of the detection networks); of the int8 layers only a few deep ones are (3x3
     // stride 2 from 40 x 40: 29 -> 23 us) while the wide first layers lose (12 -> 32 channels at 320 x 320: 81 -> 94 us),
     // so int8 layers stay with the staged kernels unless the option asks.
-    const bool take = DT == EXHIP_F16 || g.c_bytes == 32 || (g.pixels <= 32768 && kblocks <= 4) || g.pixels <= 6400;
+    // A lone 32-channel block (its 128-pixel tile with the tap bookkeeping fills the register file) never wins: 12 -> 32
+    // at 16 x 320 x 320 78 against 80 us, 16 -> 32 stride 2 at 224 x 224 11.5 against 9 us in either data type.
+    const bool take = kblocks > 1 && (DT == EXHIP_F16 || g.c_bytes == 32 || (g.pixels <= 32768 && kblocks <= 4) || g.pixels <= 6400);
     if (g_exhip_options.direct != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
     p.post_slope = g.post_slope;
     p.pixels = (unsigned)g.pixels; p.x_bytes = (unsigned)x_bytes; p.w_bytes = (unsigned)w_bytes;
@@ -559,7 +561,11 @@ int run_pw(exhip_ctx* ctx, const exhip_pw_geom& g, PwParams& p, int es, bool has
     bool take = joined || blocks_needed == 1 || (flop <= 8.0e9 && g.pixels <= 32768);
     if (DT == EXHIP_I8 && g.pixels <= 131072 && (g.c_bytes <= 64 || (p.y_f && !p.y_q))) take = true;
     if (DT == EXHIP_I8 && g_exhip_options.pw_tile != 2 && g.c_bytes <= 512) take = true;  // with the small tile: every layer measured
-    if (DT == EXHIP_F16 && g_exhip_options.pw_tile != 2) take = true;  // with the small tile: every layer measured
+    // With the small tile: every fp16 layer. Launched thirty times alone, long reductions on large maps lose a little
+    // (256 -> 256 at 64 x 28 x 28: 33 against 32 us, 512 -> 512 at 16 x 40 x 40: 49 against 46 us); inside the networks,
+    // between other layers, taking them too is what measured faster (same box, two runs each: a detection network 1.752
+    // -> 1.738 ms, another 0.820 -> 0.805 ms, a depthwise / pointwise network 0.772 -> 0.761 ms), and the networks decide.
+    if (DT == EXHIP_F16 && g_exhip_options.pw_tile != 2) take = true;
     if (DT == EXHIP_F16 && ((g.c_bytes <= 128 && g.pixels <= 524288) || (g.c_bytes <= 256 && g.k <= 64 && g.pixels <= 131072))) take = true;
     if (g_exhip_options.pw != 2 && !take) return EXHIP_ERR_UNSUPPORTED;
     if (g.pixels <= 0 || g.c_bytes <= 0 || g.c_bytes % 32 != 0 || (g.slab_blocks != 2 && g.slab_blocks != 4) || g.k_stride % 8 != 0)
