@@ -849,6 +849,68 @@ __global__ __launch_bounds__(kBlock) void maxpool_nhwc_i8_kernel(const int8_t* _
     *reinterpret_cast<v4i*>(y + ((n * OH + oy) * OW + ox) * cs + g * 16) = o;
 }
 
+// A pyramid of stride-1 "same" max pools on an int8 NHWC tensor in one launch: y1 = pool_k(x), y2 = pool_k(y1), y3 = pool_k(y2)
+// (windows k, 2k - 1, 3k - 2 over x: 5 / 9 / 13). One group per image and 16-channel slab keeps the slab's map in LDS as
+// int16 pairs (v_pk_max_i16 takes two channels per instruction) and pools it separably, rows then columns, level after
+// level; taps outside the image count in no maximum. kPyrPixels bounds the map (two buffers of 32 bytes per pixel).
+constexpr int kPyrPixels = 960;
+typedef short v2s __attribute__((ext_vector_type(2)));
+struct PyrPixel { v2s c[8]; };  // 16 channels
+__global__ __launch_bounds__(kBlock) void maxpool_pyramid_nhwc_i8_kernel(const int8_t* __restrict__ x, int8_t* __restrict__ y1, int8_t* __restrict__ y2,
+                                                                        int8_t* __restrict__ y3, int H, int W, int cs, int k) {
+    __shared__ PyrPixel buf[2][kPyrPixels];
+    const int slab = blockIdx.x, n = blockIdx.y, px = H * W, r = k / 2;
+    const size_t base = (size_t)n * px * cs + (size_t)slab * 16;
+    for (int i = threadIdx.x; i < px; i += kBlock) {
+        const v4i t = *reinterpret_cast<const v4i*>(x + base + (size_t)i * cs);
+        PyrPixel o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int w = t[e >> 1] >> ((e & 1) * 16);                       // bytes 2e, 2e + 1 in the low half
+            o.c[e] = v2s{(short)((w << 24) >> 24), (short)((w << 16) >> 24)};  // sign-extended
+        }
+        buf[0][i] = o;
+    }
+    __syncthreads();
+    int8_t* const outs[3] = {y1, y2, y3};
+#pragma unroll 1
+    for (int level = 0; level < 3; ++level) {
+        int8_t* const y = outs[level];
+        if (!y) break;  // uniform
+        // rows: buf[0] -> buf[1]
+        for (int i = threadIdx.x; i < px; i += kBlock) {
+            const int yy = i / W, xx = i - yy * W;
+            const int lo = xx - r < 0 ? 0 : xx - r, hi = xx + r >= W ? W - 1 : xx + r;
+            PyrPixel m = buf[0][yy * W + lo];
+            for (int b = lo + 1; b <= hi; ++b) {
+                const PyrPixel t = buf[0][yy * W + b];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) m.c[e] = __builtin_elementwise_max(m.c[e], t.c[e]);
+            }
+            buf[1][i] = m;
+        }
+        __syncthreads();
+        // columns: buf[1] -> buf[0] (the level's result, the next level's input) and out
+        for (int i = threadIdx.x; i < px; i += kBlock) {
+            const int yy = i / W, xx = i - yy * W;
+            const int lo = yy - r < 0 ? 0 : yy - r, hi = yy + r >= H ? H - 1 : yy + r;
+            PyrPixel m = buf[1][lo * W + xx];
+            for (int a = lo + 1; a <= hi; ++a) {
+                const PyrPixel t = buf[1][a * W + xx];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) m.c[e] = __builtin_elementwise_max(m.c[e], t.c[e]);
+            }
+            buf[0][i] = m;
+            v4i o;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                o[q] = (m.c[2 * q][0] & 0xff) | ((m.c[2 * q][1] & 0xff) << 8) | ((m.c[2 * q + 1][0] & 0xff) << 16) | ((int)m.c[2 * q + 1][1] << 24);
+            *reinterpret_cast<v4i*>(y + base + (size_t)i * cs) = o;
+        }
+        __syncthreads();
+    }
+}
+
 // 3x3 stride-2 max pooling on NHWC float32, a 2 x 2 block of output pixels per thread (four channels each): the four
 // windows share a row and a column, so 25 loads instead of 36, all in flight at once. Taps outside the image count as
 // -FLT_MAX, the clipped window of the general kernel. Optional requantized int8 copy as there.
@@ -2332,6 +2394,28 @@ extern "C" int exhip_maxpool2d_nhwc_i8(exhip_ctx* ctx, const int8_t* x, int8_t* 
     hipLaunchKernelGGL(maxpool_nhwc_i8_kernel, dim3(blocks_for(total)), dim3(kBlock), 0, ctx->stream, x, y, h, w, cs, oh, ow, kh, kw, sh, sw, pt, pl,
                        total);
     EXHIP_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int exhip_maxpool_same_pyramid_nhwc_i8(exhip_ctx* ctx, const int8_t* x, int8_t* y1, int8_t* y2, int8_t* y3, int n, int c, int h, int w,
+                                                  int cs, int k) {
+    REQ_CTX("exhip_maxpool_same_pyramid_nhwc_i8");
+    EXHIP_REQUIRE(x && y1 && (y2 || !y3) && n > 0 && c > 0 && cs >= c && cs % 16 == 0 && h > 0 && w > 0 && k > 0 && (k & 1), "exhip_maxpool_same_pyramid_nhwc_i8: bad argument");
+    EXHIP_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y1) | reinterpret_cast<uintptr_t>(y2) | reinterpret_cast<uintptr_t>(y3)) & 15) == 0,
+                  "exhip_maxpool_same_pyramid_nhwc_i8: tensors must be 16-byte aligned");
+    if ((long long)h * w <= kPyrPixels && n <= 65535) {
+        hipLaunchKernelGGL(maxpool_pyramid_nhwc_i8_kernel, dim3((unsigned)(cs / 16), (unsigned)n), dim3(kBlock), 0, ctx->stream, x, y1, y2, y3, h, w, cs, k);
+        EXHIP_LAUNCH_CHECK();
+        return 0;
+    }
+    // a map that does not fit the group's LDS: level by level through the window kernel
+    const int8_t* src = x;
+    int8_t* const outs[3] = {y1, y2, y3};
+    for (int level = 0; level < 3 && outs[level]; ++level) {
+        const int rc = exhip_maxpool2d_nhwc_i8(ctx, src, outs[level], n, c, h, w, cs, h, w, k, k, 1, 1, k / 2, k / 2);
+        if (rc) return rc;
+        src = outs[level];
+    }
     return 0;
 }
 

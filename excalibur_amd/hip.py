@@ -484,6 +484,15 @@ class Ctx:
                                              int(stride), int(pad[0]), int(pad[1])))
         return y
 
+
+    def maxpool_same_pyramid_nhwc_i8(self, x, c, k, levels=3):
+        """Stride-1 "same" max pools of window k applied `levels` times to an int8 NHWC tensor, every level's result returned
+        (exhip_maxpool_same_pyramid_nhwc_i8)."""
+        n, h, w, cs = x.shape
+        ys = [self.empty((n, h, w, cs), np.int8) for _ in range(levels)]
+        ptrs = [y.ptr for y in ys] + [None] * (3 - levels)
+        _check(lib().exhip_maxpool_same_pyramid_nhwc_i8(self.h, x.ptr, ptrs[0], ptrs[1], ptrs[2], n, int(c), h, w, cs, int(k)))
+        return ys
     def input_focus_quantize(self, x, means, scales, fs, c_stride=32):
         """Input layer, YoloV5Focus and the int8 quantizer in one pass (exhip_input_focus_quantize_nchw_f32_to_nhwc_i8): float32
         NCHW -> int8 NHWC [n, h / 2, w / 2, c_stride]. Returns None where the library leaves the shape to the three layers."""

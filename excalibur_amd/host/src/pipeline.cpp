@@ -1266,6 +1266,12 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
     }
 
     // ---- shapes, buffers, launches ----
+    struct {  // the int8 pooling pyramid whose launch is the plan's last one
+        const int8_t* x = nullptr;
+        int8_t* y[3] = {nullptr, nullptr, nullptr};
+        int levels = 0, k = 0, n = 0, h = 0, w = 0, cs = 0;
+        size_t launch = 0;
+    } pyramid;
     exhip_ctx* ctx = memory::device_context(device_);
     const int dev = device_;
     auto alloc = [&](size_t bytes) {
@@ -1539,8 +1545,27 @@ bool pipeline<float>::impl::build_graph_plan(const tensor_ptr& input, const std:
             if (!nd.as_f32) {
                 if (in.cs % 16 != 0 || pt >= kh || pl >= kw) return refuse(__LINE__);
                 const int8_t* xq = static_cast<const int8_t*>(source);
-                plan->launches.push_back(
-                    [=]() { EXHIP_FATAL(exhip_maxpool2d_nhwc_i8(ctx, xq, yq, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl)); });
+                // A pool that pools the result of the pool launched just before it with the same window (the 5 / 9 / 13
+                // pyramid as 5, 5 of 5, 5 of that) joins that launch: one kernel keeps the map in LDS for all levels.
+                const bool same = kh == kw && (kh & 1) && sh == 1 && sw == 1 && pt == kh / 2 && pl == kh / 2 && oh == in.h && ow == in.w;
+                if (same && nd.cascade >= 0 && pyramid.levels > 0 && pyramid.levels < 3 && pyramid.launch + 1 == plan->launches.size() &&
+                    xq == pyramid.y[pyramid.levels - 1] && kh == pyramid.k && in.n == pyramid.n && in.h == pyramid.h && in.w == pyramid.w &&
+                    in.cs == pyramid.cs) {
+                    pyramid.y[pyramid.levels++] = yq;
+                    const auto py = pyramid;
+                    const int c = in.c;
+                    plan->launches.back() = [=]() {
+                        EXHIP_FATAL(exhip_maxpool_same_pyramid_nhwc_i8(ctx, py.x, py.y[0], py.y[1], py.y[2], py.n, c, py.h, py.w, py.cs, py.k));
+                    };
+                } else {
+                    plan->launches.push_back(
+                        [=]() { EXHIP_FATAL(exhip_maxpool2d_nhwc_i8(ctx, xq, yq, in.n, in.c, in.h, in.w, in.cs, oh, ow, kh, kw, sh, sw, pt, pl)); });
+                    pyramid = {};
+                    if (same) {
+                        pyramid.x = xq; pyramid.y[0] = yq; pyramid.levels = 1; pyramid.launch = plan->launches.size() - 1;
+                        pyramid.k = kh; pyramid.n = in.n; pyramid.h = in.h; pyramid.w = in.w; pyramid.cs = in.cs;
+                    }
+                }
             } else {
                 const float* x = static_cast<const float*>(source);
                 float* yf = static_cast<float*>(out.f32);

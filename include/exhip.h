@@ -248,6 +248,12 @@ int exhip_maxpool2d_nhwc_f32(exhip_ctx* ctx, const float* x, float* y, int8_t* y
  * float result would quantize to, since max commutes with the monotone quantizer (taps outside the image do not count). */
 int exhip_maxpool2d_nhwc_i8(exhip_ctx* ctx, const int8_t* x, int8_t* y, int n, int c, int h, int w, int c_stride, int oh, int ow,
                             int kh, int kw, int sh, int sw, int pt, int pl);
+/* The pooling pyramid of a detection network's SPP block (models/yolov5s_simp.phai: three Pooling layers, windows 5 / 9 / 13,
+ * stride 1, "same" padding, over one tensor) on the int8 tensor in one launch: y1 = pool_k(x), y2 = pool_k(y1),
+ * y3 = pool_k(y2), which are the maxima over windows k, 2k - 1 and 3k - 2 of x (operation_pooling.cpp:145-159: taps outside
+ * the image count in no maximum). y3, or y2 and y3, may be NULL. k odd; tensors [n][h][w][cs], cs a multiple of 16. */
+int exhip_maxpool_same_pyramid_nhwc_i8(exhip_ctx* ctx, const int8_t* x, int8_t* y1, int8_t* y2, int8_t* y3, int n, int c, int h, int w,
+                                       int cs, int k);
 int exhip_pool2d_nhwc_f16(exhip_ctx* ctx, const uint16_t* x, uint16_t* y, int n, int c, int h, int w, int c_stride,
                           int oh, int ow, int type, int kh, int kw, int sh, int sw, int pt, int pb, int pl, int pr,
                           int count_include_pad);

@@ -860,3 +860,21 @@ def test_quantizer_and_clamped_activations_at_the_edges_of_their_ranges(ctx):
         ok = ~np.isnan(want)     # inf * 0 is NaN on both sides; payloads are not compared
         assert np.array_equal(np.isnan(got), np.isnan(want))
         assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32)), name
+
+
+@pytest.mark.parametrize("shape,k,levels", [((2, 20, 20, 64), 5, 3), ((1, 7, 11, 32), 5, 3), ((3, 30, 32, 16), 3, 2), ((1, 1, 9, 16), 5, 1),
+                                            ((1, 40, 40, 32), 5, 3)],
+                         ids=["spp-20x20", "ragged-7x11", "k3-two-levels", "one-row", "40x40-level-by-level"])
+def test_int8_pooling_pyramid_in_one_launch(ctx, shape, k, levels):
+    """y1 = pool_k(x), y2 = pool_k(y1), y3 = pool_k(y2) on an int8 NHWC tensor in one launch, against the oracle's MAX pooling
+    of x with windows k, 2k - 1, 3k - 2 (stride 1, "same" padding): the SPP block's three Pooling layers. The 40 x 40 map does
+    not fit a group's LDS and goes level by level through the window kernel."""
+    n, h, w, c = shape
+    x = np.random.default_rng(1200 + h).integers(-128, 128, shape).astype(np.int8)
+    ys = ctx.maxpool_same_pyramid_nhwc_i8(ctx.array(x), c, k, levels)
+    ctx.sync()
+    xf = np.ascontiguousarray(x.astype(np.float32).transpose(0, 3, 1, 2))
+    for level, y in enumerate(ys):
+        win = (level + 1) * (k - 1) + 1
+        want = port.pool2d(xf, 0, win, 1, win // 2).transpose(0, 2, 3, 1)
+        assert np.array_equal(y.download().astype(np.float32), want), f"level {level + 1}"
